@@ -1,0 +1,156 @@
+"""``approx_ops`` -- the native operator module of the LUT-based approximate-multiplier GEMM, for MI355X.
+
+Drop-in for the reference's compiled extension of the same name (module name:
+``setup.py:37``; the three registered functions: ``self_ops/src/op_register.cpp:16-19``).  The
+functions take the same tensors in the same order, require the same devices / dtypes / contiguity /
+shapes as the reference's ``CHECK_INPUT`` and ``TORCH_CHECK`` lines and raise ``RuntimeError`` when they
+are violated; outputs are caller-allocated and overwritten.  Behind them sits ``libamr_lutgemm.so``
+(HIP kernels for gfx950) reached through its C ABI with ctypes -- torch is used for device memory
+and streams only.
+
+Differences from the reference, all on the safe side:
+  * the bit-width is taken from the table length at run time (the reference bakes it in at compile
+    time, ``self_ops/src/approx_mult.h:12``);
+  * kernels run on torch's current stream of the tensors' device, under a device guard
+    (reference: legacy default stream, bare ``cudaSetDevice``, ``approx_gemm_forward.cu:256,287``);
+  * a failed launch raises instead of printing (``approx_gemm_forward.cu:304-306``).
+
+There is no CPU implementation: importing this module without the built library raises ImportError.
+"""
+import ctypes
+import os
+
+import torch
+
+_PKG_DIR = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+_LIB_PATH = os.path.join(_PKG_DIR, "libamr_lutgemm.so")
+
+if not os.path.exists(_LIB_PATH):
+    raise ImportError(
+        f"{_LIB_PATH} is missing: build the HIP library first (python {os.path.join(_PKG_DIR, 'build.py')}); "
+        "approx_ops has no CPU fallback")
+_lib = ctypes.CDLL(_LIB_PATH)
+
+_vp, _i, _i64, _sz = ctypes.c_void_p, ctypes.c_int, ctypes.c_int64, ctypes.c_size_t
+_lib.amr_last_error.restype = ctypes.c_char_p
+_lib.amr_target_arch.restype = ctypes.c_char_p
+_lib.amr_lut_gemm_forward.argtypes = [_vp, _vp, _vp, _vp, _i64, _i, _i, _i, _vp]
+_lib.amr_lut_gemm_backward.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i, _i, _i, _vp, _sz, _vp]
+_lib.amr_lut_gemm_backward_workspace_bytes.argtypes = [_i, _i, _i]
+_lib.amr_lut_gemm_backward_workspace_bytes.restype = _sz
+_lib.amr_acc_gemm_forward_fp32.argtypes = [_vp, _vp, _vp, _i, _i, _i, _vp]
+_lib.amr_bits_from_lut_elems.argtypes = [_i64]
+_lib.amr_lut_geometry.argtypes = [_i, ctypes.POINTER(_i), ctypes.POINTER(_i), ctypes.POINTER(_i64)]
+_lib.amr_lds_gather_probe.argtypes = [_i, _i, _i, ctypes.POINTER(ctypes.c_float), ctypes.POINTER(ctypes.c_double), _vp]
+
+LIBRARY_PATH = _LIB_PATH
+
+
+def _check_input(x, dtype, name):
+    # same three conditions, same order and wording as CHECK_INPUT (self_ops/src/cuda_helper.h:64-68)
+    if not (isinstance(x, torch.Tensor) and x.device.type == "cuda"):
+        raise RuntimeError(f"{name} must be a CUDAtensor")
+    if not x.is_contiguous():
+        raise RuntimeError(f"{name} must be contiguous")
+    if x.dtype != dtype:
+        raise RuntimeError(f"{name} must be of type {dtype}")
+
+
+def _check(cond, msg):
+    if not cond:
+        raise RuntimeError(msg)
+
+
+def _raise_for(rc, what):
+    if rc != 0:
+        raise RuntimeError(f"{what} failed ({rc}): {_lib.amr_last_error().decode()}")
+
+
+def _lut_len_check(lut, name):
+    _check(lut.dim() == 1 and _lib.amr_bits_from_lut_elems(lut.size(0)) > 0,
+           f"{name} size should be 1024, 5120, 17408 or 66306 (4-, 6-, 7-, 8-bit padded table), got {tuple(lut.shape)}; "
+           "please check the value of QUANTIZATION_BIT")
+
+
+def _stream_ptr(device):
+    return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+
+
+def approx_gemm_forward(a_tensor, b_tensor, c_tensor, lut_appmult_tensor):
+    """c[m,n] = sum_k lut[a[m,k]][b[k,n]]; a u8 [M,K], b u8 [K,N], c u32 [M,N] (out), lut u16 padded table.
+    Contract of approx_gemm_forward_gpu (self_ops/src/approx_gemm_forward.cu:241-259)."""
+    _check_input(a_tensor, torch.uint8, "a_tensor")
+    _check_input(b_tensor, torch.uint8, "b_tensor")
+    _check_input(c_tensor, torch.uint32, "c_tensor")
+    _check_input(lut_appmult_tensor, torch.uint16, "lut_appmult_tensor")
+    _check(a_tensor.dim() == 2 and b_tensor.dim() == 2 and c_tensor.dim() == 2, "a, b and c must be 2-D")
+    M, K = a_tensor.shape
+    N = b_tensor.size(1)
+    _check(K == b_tensor.size(0), f"b_tensor's shape should be {K} x {N}")
+    _check(M == c_tensor.size(0) and N == c_tensor.size(1), f"c_tensor's shape should be {M} x {N}")
+    _lut_len_check(lut_appmult_tensor, "lut_appmult_tensor")
+    dev = a_tensor.device
+    _check(dev == b_tensor.device and dev == c_tensor.device and dev == lut_appmult_tensor.device, "device id not match")
+    with torch.cuda.device(dev):
+        rc = _lib.amr_lut_gemm_forward(a_tensor.data_ptr(), b_tensor.data_ptr(), c_tensor.data_ptr(),
+                                       lut_appmult_tensor.data_ptr(), lut_appmult_tensor.size(0), M, K, N, _stream_ptr(dev))
+    _raise_for(rc, "approx_gemm_forward")
+
+
+def acc_gemm_forward_fp32(a_tensor, b_tensor, c_tensor):
+    """c = a @ b in fp32; contract of acc_gemm_forward_fp32_gpu (self_ops/src/approx_gemm_forward.cu:500-520)."""
+    _check_input(a_tensor, torch.float32, "a_tensor")
+    _check_input(b_tensor, torch.float32, "b_tensor")
+    _check_input(c_tensor, torch.float32, "c_tensor")
+    _check(a_tensor.dim() == 2 and b_tensor.dim() == 2 and c_tensor.dim() == 2, "a, b and c must be 2-D")
+    M, K = a_tensor.shape
+    N = b_tensor.size(1)
+    _check(K == b_tensor.size(0), f"b_tensor's shape should be {K} x {N}")
+    _check(M == c_tensor.size(0) and N == c_tensor.size(1), f"c_tensor's shape should be {M} x {N}")
+    dev = a_tensor.device
+    _check(dev == b_tensor.device and dev == c_tensor.device, "device id not match")
+    with torch.cuda.device(dev):
+        rc = _lib.amr_acc_gemm_forward_fp32(a_tensor.data_ptr(), b_tensor.data_ptr(), c_tensor.data_ptr(), M, K, N, _stream_ptr(dev))
+    _raise_for(rc, "acc_gemm_forward_fp32")
+
+
+def approx_gemm_backward(gc_tensor, a_tensor, b_tensor, ga_tensor, gb_tensor, lut_grad_a_tensor, lut_grad_b_tensor):
+    """ga[m,k] = 1/16 sum_n gc[m,n]*lutA[a][b], gb[k,n] = 1/16 sum_m lutB[a][b]*gc[m,n]; outputs overwritten.
+    Contract of approx_gemm_backward_gpu (self_ops/src/approx_gemm_backward.cu:506-529)."""
+    _check_input(gc_tensor, torch.float32, "gc_tensor")
+    _check_input(a_tensor, torch.uint8, "a_tensor")
+    _check_input(b_tensor, torch.uint8, "b_tensor")
+    _check_input(ga_tensor, torch.float32, "ga_tensor")
+    _check_input(gb_tensor, torch.float32, "gb_tensor")
+    _check_input(lut_grad_a_tensor, torch.int16, "lut_grad_a_tensor")
+    _check_input(lut_grad_b_tensor, torch.int16, "lut_grad_b_tensor")
+    _check(all(t.dim() == 2 for t in (gc_tensor, a_tensor, b_tensor, ga_tensor, gb_tensor)), "gc, a, b, ga and gb must be 2-D")
+    M, K = a_tensor.shape
+    N = b_tensor.size(1)
+    _check(gc_tensor.size(0) == M and gc_tensor.size(1) == N, f"gc_tensor's shape should be {M} x {N}")
+    _check(K == b_tensor.size(0), f"b_tensor's shape should be {K} x {N}")
+    _check(ga_tensor.size(0) == M and ga_tensor.size(1) == K, f"ga_tensor's shape should be {M} x {K}")
+    _check(gb_tensor.size(0) == K and gb_tensor.size(1) == N, f"gb_tensor's shape should be {K} x {N}")
+    _lut_len_check(lut_grad_a_tensor, "lut_grad_a_tensor")
+    _lut_len_check(lut_grad_b_tensor, "lut_grad_b_tensor")
+    _check(lut_grad_a_tensor.size(0) == lut_grad_b_tensor.size(0), "the two gradient tables must have the same length")
+    dev = gc_tensor.device
+    _check(all(t.device == dev for t in (a_tensor, b_tensor, ga_tensor, gb_tensor, lut_grad_a_tensor, lut_grad_b_tensor)),
+           "All tensors should be on the same device")
+    with torch.cuda.device(dev):
+        need = _lib.amr_lut_gemm_backward_workspace_bytes(M, K, N)
+        ws = torch.empty(need, dtype=torch.uint8, device=dev) if need else None
+        rc = _lib.amr_lut_gemm_backward(gc_tensor.data_ptr(), a_tensor.data_ptr(), b_tensor.data_ptr(),
+                                        ga_tensor.data_ptr(), gb_tensor.data_ptr(), lut_grad_a_tensor.data_ptr(),
+                                        lut_grad_b_tensor.data_ptr(), lut_grad_a_tensor.size(0), M, K, N,
+                                        ws.data_ptr() if ws is not None else None, need, _stream_ptr(dev))
+    _raise_for(rc, "approx_gemm_backward")
+
+
+def lds_gather_probe(pattern=0, waves_per_cu=16, iters=4000):
+    """Measured LDS gather rate (gathers per second) of the current device; see amr_lds_gather_probe."""
+    ms, n = ctypes.c_float(0), ctypes.c_double(0)
+    rc = _lib.amr_lds_gather_probe(pattern, waves_per_cu, iters, ctypes.byref(ms), ctypes.byref(n),
+                                   _stream_ptr(torch.device("cuda", torch.cuda.current_device())))
+    _raise_for(rc, "lds_gather_probe")
+    return n.value / (ms.value * 1e-3)

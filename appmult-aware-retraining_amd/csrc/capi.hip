@@ -1,0 +1,204 @@
+// extern "C" entry points of libamr_lutgemm.so (declared in include/amr_lutgemm.h): argument checks,
+// bit-width dispatch from the table length, per-device caches, launches on the caller's stream.
+#include "../../include/amr_lutgemm.h"
+
+#include <mutex>
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include "amr_common.h"
+
+namespace amr {
+hipError_t launch_fwd(const uint8_t* A, const uint8_t* B, uint32_t* C, const uint16_t* lut, const LutGeom& g, int M,
+                      int K, int N, int n_cu, hipStream_t stream);
+size_t gradB_workspace_bytes(int M, int K, int N, int n_cu, int* splits_out);
+hipError_t launch_gradB(const float* gC, const uint8_t* A, const uint8_t* B, float* gB, const int16_t* lut,
+                        const LutGeom& g, int M, int K, int N, float scale, void* workspace, int splits,
+                        hipStream_t stream);
+hipError_t launch_gradA(const float* gC, const uint8_t* A, const uint8_t* B, float* gA, const int16_t* lut,
+                        const LutGeom& g, int M, int K, int N, float scale, int n_cu, hipStream_t stream);
+hipError_t launch_accgemm(const float* A, const float* B, float* C, int M, int K, int N, hipStream_t stream);
+hipError_t run_lds_probe(int pattern, int waves_per_cu, int iters, int n_cu, float* ms_out, double* gathers_out,
+                         hipStream_t stream);
+}  // namespace amr
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+int hip_fail(hipError_t e, const char* where) {
+    snprintf(g_err, sizeof(g_err), "%s: %s", where, hipGetErrorString(e));
+    return (int)e;
+}
+
+constexpr int kMaxDevices = 64;
+struct DeviceState {
+    int n_cu = 0;
+    void* ws = nullptr;
+    size_t ws_bytes = 0;
+};
+DeviceState g_dev[kMaxDevices];
+std::mutex g_mu;
+
+// Number of compute units of the current device (cached).
+int current_device_cus(int* dev_out) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return -1;
+    std::lock_guard<std::mutex> lk(g_mu);
+    if (g_dev[dev].n_cu == 0) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) return -1;
+        g_dev[dev].n_cu = n;
+    }
+    if (dev_out) *dev_out = dev;
+    return g_dev[dev].n_cu;
+}
+
+// Library-owned scratch for callers that pass no workspace: grown on demand, kept until exit.
+void* internal_workspace(int dev, size_t bytes, hipError_t* err) {
+    std::lock_guard<std::mutex> lk(g_mu);
+    DeviceState& d = g_dev[dev];
+    *err = hipSuccess;
+    if (d.ws_bytes >= bytes) return d.ws;
+    if (d.ws) {
+        (void)hipDeviceSynchronize();
+        (void)hipFree(d.ws);
+        d.ws = nullptr;
+        d.ws_bytes = 0;
+    }
+    size_t want = bytes + bytes / 4;
+    *err = hipMalloc(&d.ws, want);
+    if (*err != hipSuccess) { d.ws = nullptr; return nullptr; }
+    d.ws_bytes = want;
+    return d.ws;
+}
+
+}  // namespace
+
+extern "C" {
+
+int amr_version(void) { return 100; }
+const char* amr_target_arch(void) { return "gfx950"; }
+const char* amr_last_error(void) { return g_err; }
+
+int amr_lut_geometry(int bits, int* rows, int* cols, int64_t* elem_num) {
+    amr::LutGeom g;
+    if (!amr::lut_geom_from_bits(bits, &g)) return fail(AMR_ELUTLEN, "quantization_bit = %d is not supported", bits);
+    if (rows) *rows = g.rows;
+    if (cols) *cols = g.cols;
+    if (elem_num) *elem_num = g.elems;
+    return AMR_OK;
+}
+
+int amr_bits_from_lut_elems(int64_t lut_elems) {
+    amr::LutGeom g;
+    if (!amr::lut_geom_from_elems(lut_elems, &g))
+        return fail(AMR_ELUTLEN, "table length %lld matches no supported bit-width (1024, 5120, 17408, 66306)", (long long)lut_elems);
+    return g.bits;
+}
+
+int amr_lut_gemm_forward(const uint8_t* A, const uint8_t* B, uint32_t* C, const uint16_t* lut, int64_t lut_elems,
+                         int M, int K, int N, void* stream) {
+    if (M < 0 || K < 0 || N < 0) return fail(AMR_EINVAL, "negative dimension M=%d K=%d N=%d", M, K, N);
+    amr::LutGeom g;
+    if (!amr::lut_geom_from_elems(lut_elems, &g))
+        return fail(AMR_ELUTLEN, "lut size should be one of 1024/5120/17408/66306, got %lld", (long long)lut_elems);
+    if (M == 0 || N == 0) return AMR_OK;
+    if (!C || !lut || (K > 0 && (!A || !B))) return fail(AMR_EINVAL, "null pointer argument");
+    if ((uintptr_t)lut & 3) return fail(AMR_EINVAL, "lut must be 4-byte aligned");
+    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    if (K == 0) {
+        hipError_t e = hipMemsetAsync(C, 0, (size_t)M * N * sizeof(uint32_t), s);
+        return e == hipSuccess ? AMR_OK : hip_fail(e, "hipMemsetAsync");
+    }
+    const int n_cu = current_device_cus(nullptr);
+    if (n_cu <= 0) return fail(AMR_EINVAL, "no HIP device available");
+    hipError_t e = amr::launch_fwd(A, B, C, lut, g, M, K, N, n_cu, s);
+    return e == hipSuccess ? AMR_OK : hip_fail(e, "forward launch");
+}
+
+size_t amr_lut_gemm_backward_workspace_bytes(int M, int K, int N) {
+    if (M <= 0 || K <= 0 || N <= 0) return 0;
+    const int n_cu = current_device_cus(nullptr);
+    // Without a device (e.g. a host-only query) size for the largest supported split count.
+    return amr::gradB_workspace_bytes(M, K, N, n_cu > 0 ? n_cu : 256, nullptr);
+}
+
+int amr_lut_gemm_backward(const float* gC, const uint8_t* A, const uint8_t* B, float* gA, float* gB,
+                          const int16_t* lut_grad_a, const int16_t* lut_grad_b, int64_t lut_elems, int M, int K,
+                          int N, void* workspace, size_t workspace_bytes, void* stream) {
+    if (M < 0 || K < 0 || N < 0) return fail(AMR_EINVAL, "negative dimension M=%d K=%d N=%d", M, K, N);
+    amr::LutGeom g;
+    if (!amr::lut_geom_from_elems(lut_elems, &g))
+        return fail(AMR_ELUTLEN, "lut size should be one of 1024/5120/17408/66306, got %lld", (long long)lut_elems);
+    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    const float scale = 1.0f / 16.0f;  // FACTOR, self_ops/src/approx_mult.h:41
+    if (gA && !lut_grad_a) return fail(AMR_EINVAL, "lut_grad_a is null");
+    if (gB && !lut_grad_b) return fail(AMR_EINVAL, "lut_grad_b is null");
+    if (((uintptr_t)lut_grad_a & 3) || ((uintptr_t)lut_grad_b & 3)) return fail(AMR_EINVAL, "gradient tables must be 4-byte aligned");
+    // Degenerate reductions: an empty sum is zero.
+    if (M == 0 || K == 0 || N == 0) {
+        hipError_t e = hipSuccess;
+        if (gA && (size_t)M * K) e = hipMemsetAsync(gA, 0, (size_t)M * K * sizeof(float), s);
+        if (e == hipSuccess && gB && (size_t)K * N) e = hipMemsetAsync(gB, 0, (size_t)K * N * sizeof(float), s);
+        return e == hipSuccess ? AMR_OK : hip_fail(e, "hipMemsetAsync");
+    }
+    if (!gC || !A || !B) return fail(AMR_EINVAL, "null pointer argument");
+    int dev = 0;
+    const int n_cu = current_device_cus(&dev);
+    if (n_cu <= 0) return fail(AMR_EINVAL, "no HIP device available");
+    hipError_t e;
+    if (gA) {
+        e = amr::launch_gradA(gC, A, B, gA, lut_grad_a, g, M, K, N, scale, n_cu, s);
+        if (e != hipSuccess) return hip_fail(e, "gradA launch");
+    }
+    if (gB) {
+        int splits = 1;
+        const size_t need = amr::gradB_workspace_bytes(M, K, N, n_cu, &splits);
+        void* ws = workspace;
+        if (need > 0) {
+            if (ws) {
+                if (workspace_bytes < need) return fail(AMR_EWORKSPACE, "workspace of %zu bytes is smaller than the %zu required", workspace_bytes, need);
+                if ((uintptr_t)ws & 255) return fail(AMR_EINVAL, "workspace must be 256-byte aligned");
+            } else {
+                ws = internal_workspace(dev, need, &e);
+                if (!ws) return hip_fail(e, "workspace hipMalloc");
+            }
+        }
+        e = amr::launch_gradB(gC, A, B, gB, lut_grad_b, g, M, K, N, scale, ws, splits, s);
+        if (e != hipSuccess) return hip_fail(e, "gradB launch");
+    }
+    return AMR_OK;
+}
+
+int amr_acc_gemm_forward_fp32(const float* A, const float* B, float* C, int M, int K, int N, void* stream) {
+    if (M < 0 || K < 0 || N < 0) return fail(AMR_EINVAL, "negative dimension M=%d K=%d N=%d", M, K, N);
+    if (M == 0 || N == 0) return AMR_OK;
+    if (!C || (K > 0 && (!A || !B))) return fail(AMR_EINVAL, "null pointer argument");
+    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    if (K == 0) {
+        hipError_t e = hipMemsetAsync(C, 0, (size_t)M * N * sizeof(float), s);
+        return e == hipSuccess ? AMR_OK : hip_fail(e, "hipMemsetAsync");
+    }
+    hipError_t e = amr::launch_accgemm(A, B, C, M, K, N, s);
+    return e == hipSuccess ? AMR_OK : hip_fail(e, "accgemm launch");
+}
+
+int amr_lds_gather_probe(int pattern, int waves_per_cu, int iters, float* ms_out, double* gathers_out, void* stream) {
+    if (pattern < 0 || pattern > 1 || iters <= 0) return fail(AMR_EINVAL, "bad probe arguments");
+    const int n_cu = current_device_cus(nullptr);
+    if (n_cu <= 0) return fail(AMR_EINVAL, "no HIP device available");
+    hipError_t e = amr::run_lds_probe(pattern, waves_per_cu, iters, n_cu, ms_out, gathers_out, reinterpret_cast<hipStream_t>(stream));
+    return e == hipSuccess ? AMR_OK : hip_fail(e, "lds probe");
+}
+
+}  // extern "C"

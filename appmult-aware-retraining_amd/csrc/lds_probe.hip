@@ -1,0 +1,63 @@
+// LDS gather-rate probe: calibrates the denominator of the LDS-gather roofline on the device at hand.
+// Every wave issues rounds of 8 independent ds_read_u16 and waits for them; with `waves_per_cu` waves
+// resident on each CU the LDS pipe is the only limiter, so gathers / time is the sustained
+// conflict-free (pattern 0) or 2-way-conflicted uniform-row (pattern 1) gather rate.
+#include "amr_common.h"
+
+namespace amr {
+
+__global__ __launch_bounds__(1024) void lds_probe_kernel(int pattern, int iters, uint32_t* __restrict__ sink) {
+    __shared__ uint32_t lds[8192];
+    for (int i = threadIdx.x; i < 8192; i += blockDim.x) lds[i] = (uint32_t)i * 2654435761u;
+    __syncthreads();
+    const int lane = threadIdx.x & 63;
+    uint32_t addr[4];
+    uint32_t h = (uint32_t)(lane * 747796405u + 2891336453u);
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+        h = h * 1664525u + 1013904223u;
+        // pattern 0: lane*2 (64 consecutive u16, conflict-free); pattern 1: random u16 inside a 256-byte row
+        addr[s] = (pattern == 0 ? (uint32_t)(lane * 2) : ((h >> 10) % 128u) * 2u) + s * 1024;
+    }
+    uint32_t acc = 0;
+    for (int it = 0; it < iters; ++it) {
+        uint32_t r0, r1, r2, r3, r4, r5, r6, r7;
+        asm volatile(
+            "ds_read_u16 %0, %8\n ds_read_u16 %1, %9\n ds_read_u16 %2, %10\n ds_read_u16 %3, %11\n"
+            "ds_read_u16 %4, %8 offset:4096\n ds_read_u16 %5, %9 offset:4096\n ds_read_u16 %6, %10 offset:4096\n"
+            "ds_read_u16 %7, %11 offset:4096\n s_waitcnt lgkmcnt(0)\n"
+            : "=&v"(r0), "=&v"(r1), "=&v"(r2), "=&v"(r3), "=&v"(r4), "=&v"(r5), "=&v"(r6), "=&v"(r7)
+            : "v"(addr[0]), "v"(addr[1]), "v"(addr[2]), "v"(addr[3])
+            : "memory");
+        acc += r0 + r1 + r2 + r3 + r4 + r5 + r6 + r7;
+    }
+    if (acc == 0x12345678u) sink[0] = acc;  // keeps the reads alive; practically never taken
+}
+
+hipError_t run_lds_probe(int pattern, int waves_per_cu, int iters, int n_cu, float* ms_out, double* gathers_out,
+                         hipStream_t stream) {
+    if (waves_per_cu < 1) waves_per_cu = 1;
+    if (waves_per_cu > 16) waves_per_cu = 16;
+    uint32_t* sink = nullptr;
+    hipError_t e = hipMalloc(&sink, 4);
+    if (e != hipSuccess) return e;
+    hipEvent_t e0, e1;
+    (void)hipEventCreate(&e0);
+    (void)hipEventCreate(&e1);
+    hipLaunchKernelGGL(lds_probe_kernel, dim3(n_cu), dim3(64 * waves_per_cu), 0, stream, pattern, 16, sink);  // warm-up
+    (void)hipEventRecord(e0, stream);
+    hipLaunchKernelGGL(lds_probe_kernel, dim3(n_cu), dim3(64 * waves_per_cu), 0, stream, pattern, iters, sink);
+    (void)hipEventRecord(e1, stream);
+    e = hipEventSynchronize(e1);
+    if (e == hipSuccess) e = hipGetLastError();
+    float ms = 0.f;
+    if (e == hipSuccess) e = hipEventElapsedTime(&ms, e0, e1);
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    (void)hipFree(sink);
+    if (ms_out) *ms_out = ms;
+    if (gathers_out) *gathers_out = (double)n_cu * waves_per_cu * (double)iters * 8.0 * 64.0;
+    return e;
+}
+
+}  // namespace amr

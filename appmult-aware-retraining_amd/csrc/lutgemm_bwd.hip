@@ -1,0 +1,280 @@
+// Backward LUT-GEMM kernels for gfx950.
+//
+//   gA[m,k] = scale * sum_n gC[m,n] * (float)Gx[A[m,k]][B[k,n]]     (lutgemm_gradA_kernel)
+//   gB[k,n] = scale * sum_m (float)Gy[A[m,k]][B[k,n]] * gC[m,n]     (lutgemm_gradB_kernel)
+//
+// They replace ApproxGemmBackwardKernelForGA / ...ForGB
+// (self_ops/src/approx_gemm_backward.cu:21-258 and :269-492); scale is the reference's
+// FACTOR = 1/16 (self_ops/src/approx_mult.h:41) applied once per output, which is exact in fp32.
+//
+// Both kernels use the same "uniform-row gather" as the forward kernel: one operand code is
+// wave-uniform per gather, so the 64 lanes read inside one 256-byte (7-bit) table row and bank
+// conflicts are at most 2-way for any data.
+//   gradB: lanes own columns n (their code b is fixed per k), the uniform operand is a = A[m,k];
+//          each wave owns KT values of k, keeps KT fp32 accumulators per lane and walks down a
+//          chunk of rows m.  The M reduction is split over blockIdx.z; partial sums go to a
+//          workspace and are added in a fixed order by reduce_partials_kernel (deterministic).
+//   gradA: lanes own rows m (their code a is fixed per k), the uniform operand is b = B[k,n]; the
+//          table is transposed while it is staged into LDS so that the uniform code again selects
+//          the row.  Each lane keeps RM x KT accumulators and walks along n; no cross-lane
+//          reduction is needed.
+#include "amr_common.h"
+
+namespace amr {
+
+// ------------------------------------------------------------------------------------------ gradB
+template <int KT, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void lutgemm_gradB_kernel(
+    const float* __restrict__ gC, const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
+    float* __restrict__ out, const uint32_t* __restrict__ lut32, int lut_dwords, int row_bytes, int M, int K, int N,
+    int m_chunk, float scale) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    {
+        uint32_t* s32 = reinterpret_cast<uint32_t*>(smem);
+        for (int i = threadIdx.x; i < lut_dwords; i += WAVES * 64) s32[i] = lut32[i];
+    }
+    __syncthreads();
+
+    const int wave = uniform(threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    const int k0 = (blockIdx.y * WAVES + wave) * KT;
+    if (k0 >= K) return;
+    const int n = blockIdx.x * 64 + lane;
+    const int nc = min(n, N - 1);
+    const int mb = blockIdx.z * m_chunk;
+    const int me = min(M, mb + m_chunk);
+
+    constexpr int DW = KT / 4;        // code dwords per row in this k tile
+    constexpr int RPL = 64 / DW;      // rows covered by one loader instruction
+    // Loader lane -> (row lane / DW, dword lane % DW).  A k tile that sticks out of K is clamped to the
+    // last full dword-aligned position inside the row; its surplus accumulators are never stored.
+    const int ldw = lane % DW;
+    const int lrow = lane / DW;
+
+    uint32_t boff[KT];
+#pragma unroll
+    for (int kk = 0; kk < KT; ++kk) boff[kk] = 2u * (uint32_t)B[(size_t)min(k0 + kk, K - 1) * N + nc];
+    float acc[KT];
+#pragma unroll
+    for (int kk = 0; kk < KT; ++kk) acc[kk] = 0.f;
+
+    for (int m = mb; m < me; m += RPL) {
+        const int r = min(m + lrow, me - 1);
+        const uint32_t a4 = load_codes4_clamped(A + (size_t)r * K, k0 + 4 * ldw, K);
+        float g[RPL];
+#pragma unroll
+        for (int i = 0; i < RPL; ++i) g[i] = (m + i < me) ? gC[(size_t)(m + i) * N + nc] : 0.f;
+#pragma unroll
+        for (int i = 0; i < RPL; ++i) {
+            float t[KT];
+#pragma unroll
+            for (int d = 0; d < DW; ++d) {
+                const uint32_t aw = __builtin_amdgcn_readlane(a4, i * DW + d);
+#pragma unroll
+                for (int kk = 0; kk < 4; ++kk) {
+                    const uint32_t ro = ((aw >> (8 * kk)) & 0xffu) * (uint32_t)row_bytes;
+                    t[4 * d + kk] = (float)*reinterpret_cast<const int16_t*>(smem + ro + boff[4 * d + kk]);
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int kk = 0; kk < KT; ++kk) acc[kk] = __builtin_fmaf(t[kk], g[i], acc[kk]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+    if (n < N) {
+        float* o = out + (size_t)blockIdx.z * K * N;
+#pragma unroll
+        for (int kk = 0; kk < KT; ++kk)
+            if (k0 + kk < K) o[(size_t)(k0 + kk) * N + n] = acc[kk] * scale;
+    }
+}
+
+// out[i] = sum_s partial[s][i], s ascending (fixed order -> deterministic).
+__global__ void reduce_partials_kernel(const float* __restrict__ partial, float* __restrict__ out, size_t count, int splits) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= count) return;
+    float s = partial[i];
+    for (int p = 1; p < splits; ++p) s += partial[(size_t)p * count + i];
+    out[i] = s;
+}
+
+// ------------------------------------------------------------------------------------------ gradA
+template <int KT, int RM, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void lutgemm_gradA_kernel(
+    const float* __restrict__ gC, const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
+    float* __restrict__ gA, const uint16_t* __restrict__ lut, int rows, int cols, int M, int K, int N, float scale) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    // Transposed staging: entry (a,b) of the row-major table goes to T[b][a], T row stride = cols
+    // entries (cols is even, so T rows stay dword aligned).  T needs cols rows of `rows` entries.
+    {
+        uint16_t* t16 = reinterpret_cast<uint16_t*>(smem);
+        const int total = rows * cols;
+        for (int i = threadIdx.x; i < total; i += WAVES * 64) {
+            const int a = i / cols;
+            const int b = i - a * cols;
+            t16[b * cols + a] = lut[i];
+        }
+    }
+    __syncthreads();
+    const int trow_bytes = cols * 2;
+
+    const int wave = uniform(threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    const int k0 = blockIdx.x * KT;
+    const int m0 = (blockIdx.y * WAVES + wave) * (64 * RM);
+    if (m0 >= M) return;
+
+    int mr[RM];
+    uint32_t aoff[RM][KT];
+    float acc[RM][KT];
+#pragma unroll
+    for (int r = 0; r < RM; ++r) {
+        mr[r] = min(m0 + lane + 64 * r, M - 1);
+        const uint8_t* arow = A + (size_t)mr[r] * K;
+#pragma unroll
+        for (int d = 0; d < KT / 4; ++d) {
+            const uint32_t a4 = load_codes4_clamped(arow, k0 + 4 * d, K);
+#pragma unroll
+            for (int kk = 0; kk < 4; ++kk) {
+                aoff[r][4 * d + kk] = 2u * ((a4 >> (8 * kk)) & 0xffu);
+                acc[r][4 * d + kk] = 0.f;
+            }
+        }
+    }
+    // Loader lane kk (< KT) carries four B codes of row k0+kk; rows beyond K are clamped (never stored).
+    const uint8_t* brow = B + (size_t)min(k0 + (lane % KT), K - 1) * N;
+
+    for (int n = 0; n < N; n += 4) {
+        const uint32_t b4 = load_codes4_clamped(brow, n, N);
+        float g[RM][4];
+#pragma unroll
+        for (int r = 0; r < RM; ++r)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) g[r][j] = (n + j < N) ? gC[(size_t)mr[r] * N + n + j] : 0.f;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            float t[RM][KT];
+#pragma unroll
+            for (int kk = 0; kk < KT; ++kk) {
+                const uint32_t bw = __builtin_amdgcn_readlane(b4, kk);
+                const uint32_t ro = ((bw >> (8 * j)) & 0xffu) * (uint32_t)trow_bytes;
+#pragma unroll
+                for (int r = 0; r < RM; ++r)
+                    t[r][kk] = (float)*reinterpret_cast<const int16_t*>(smem + ro + aoff[r][kk]);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int r = 0; r < RM; ++r)
+#pragma unroll
+                for (int kk = 0; kk < KT; ++kk) acc[r][kk] = __builtin_fmaf(g[r][j], t[r][kk], acc[r][kk]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < RM; ++r) {
+        const int m = m0 + lane + 64 * r;
+        if (m < M) {
+#pragma unroll
+            for (int kk = 0; kk < KT; ++kk)
+                if (k0 + kk < K) gA[(size_t)m * K + k0 + kk] = acc[r][kk] * scale;
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------ host
+static hipError_t set_lds_attr(const void* f) {
+    return hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+}
+
+size_t gradB_workspace_bytes(int M, int K, int N, int n_cu, int* splits_out) {
+    // Split M so that the launch has about 4 workgroups (of 4 waves) per CU and every split keeps
+    // at least 256 rows.
+    constexpr int KT = 16;
+    const long wg_per_split = (long)((N + 63) / 64) * (((K + KT - 1) / KT + 3) / 4);
+    long splits = (4L * n_cu + wg_per_split - 1) / wg_per_split;
+    const long max_by_rows = M / 256 > 0 ? M / 256 : 1;
+    if (splits > max_by_rows) splits = max_by_rows;
+    if (splits > 256) splits = 256;
+    if (splits < 1) splits = 1;
+    if (splits_out) *splits_out = (int)splits;
+    return splits > 1 ? (size_t)splits * K * N * sizeof(float) : 0;
+}
+
+hipError_t launch_gradB(const float* gC, const uint8_t* A, const uint8_t* B, float* gB, const int16_t* lut,
+                        const LutGeom& g, int M, int K, int N, float scale, void* workspace, int splits,
+                        hipStream_t stream) {
+    constexpr int KT = 16;
+    const int lut_dwords = g.rows * g.cols / 2;
+    const size_t lds = (size_t)lut_dwords * 4;
+    const bool big = g.bits == 8;
+    int m_chunk = (M + splits - 1) / splits;
+    m_chunk = (m_chunk + 15) & ~15;
+    const int zs = (M + m_chunk - 1) / m_chunk;
+    float* out = zs > 1 ? reinterpret_cast<float*>(workspace) : gB;
+    const int ktiles = (K + KT - 1) / KT;
+    hipError_t e;
+    if (big) {
+        auto kern = lutgemm_gradB_kernel<KT, 16>;
+        static bool done = false;
+        if (!done) { e = set_lds_attr(reinterpret_cast<const void*>(kern)); if (e != hipSuccess) return e; done = true; }
+        dim3 grid((N + 63) / 64, (ktiles + 15) / 16, zs);
+        hipLaunchKernelGGL(kern, grid, dim3(1024), lds, stream, gC, A, B, out, reinterpret_cast<const uint32_t*>(lut),
+                           lut_dwords, g.cols * 2, M, K, N, m_chunk, scale);
+    } else {
+        auto kern = lutgemm_gradB_kernel<KT, 4>;
+        static bool done = false;
+        if (!done) { e = set_lds_attr(reinterpret_cast<const void*>(kern)); if (e != hipSuccess) return e; done = true; }
+        dim3 grid((N + 63) / 64, (ktiles + 3) / 4, zs);
+        hipLaunchKernelGGL(kern, grid, dim3(256), lds, stream, gC, A, B, out, reinterpret_cast<const uint32_t*>(lut),
+                           lut_dwords, g.cols * 2, M, K, N, m_chunk, scale);
+    }
+    e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    if (zs > 1) {
+        const size_t count = (size_t)K * N;
+        hipLaunchKernelGGL(reduce_partials_kernel, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, stream,
+                           reinterpret_cast<const float*>(workspace), gB, count, zs);
+        e = hipGetLastError();
+    }
+    return e;
+}
+
+hipError_t launch_gradA(const float* gC, const uint8_t* A, const uint8_t* B, float* gA, const int16_t* lut,
+                        const LutGeom& g, int M, int K, int N, float scale, int n_cu, hipStream_t stream) {
+    constexpr int KT = 16;
+    const size_t lds = (size_t)g.cols * g.cols * 2;
+    const bool big = g.bits == 8;
+    hipError_t e;
+    const int ktiles = (K + KT - 1) / KT;
+    if (big) {
+        auto kern = lutgemm_gradA_kernel<KT, 1, 16>;
+        static bool done = false;
+        if (!done) { e = set_lds_attr(reinterpret_cast<const void*>(kern)); if (e != hipSuccess) return e; done = true; }
+        dim3 grid(ktiles, (M + 1023) / 1024);
+        hipLaunchKernelGGL(kern, grid, dim3(1024), lds, stream, gC, A, B, gA, reinterpret_cast<const uint16_t*>(lut), g.rows,
+                           g.cols, M, K, N, scale);
+    } else {
+        // Two rows per lane amortise the scalar work per gather; fall back to one when that would
+        // leave CUs idle.
+        const long wg2 = (long)ktiles * ((M + 511) / 512);
+        if (wg2 >= 2L * n_cu) {
+            auto kern = lutgemm_gradA_kernel<KT, 2, 4>;
+            static bool done = false;
+            if (!done) { e = set_lds_attr(reinterpret_cast<const void*>(kern)); if (e != hipSuccess) return e; done = true; }
+            dim3 grid(ktiles, (M + 511) / 512);
+            hipLaunchKernelGGL(kern, grid, dim3(256), lds, stream, gC, A, B, gA, reinterpret_cast<const uint16_t*>(lut),
+                               g.rows, g.cols, M, K, N, scale);
+        } else {
+            auto kern = lutgemm_gradA_kernel<KT, 1, 4>;
+            static bool done = false;
+            if (!done) { e = set_lds_attr(reinterpret_cast<const void*>(kern)); if (e != hipSuccess) return e; done = true; }
+            dim3 grid(ktiles, (M + 255) / 256);
+            hipLaunchKernelGGL(kern, grid, dim3(256), lds, stream, gC, A, B, gA, reinterpret_cast<const uint16_t*>(lut),
+                               g.rows, g.cols, M, K, N, scale);
+        }
+    }
+    return hipGetLastError();
+}
+
+}  // namespace amr

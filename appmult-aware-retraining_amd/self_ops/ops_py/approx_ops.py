@@ -1,0 +1,192 @@
+"""Autograd operators over the native LUT-GEMM (host-side mirror of ``self_ops/ops_py/approx_ops.py``).
+
+Public names, argument meaning and error behaviour follow the reference module; the work is done by
+the ``approx_ops`` native module (HIP, gfx950).  The three look-up tables live in module globals with
+the reference's names (``lut_appmult``, ``lut_grad_a``, ``lut_grad_b``; reference ``approx_ops.py:13-15``).
+"""
+import gzip
+
+import numpy as np
+import torch
+import torch.nn.functional as F
+from torch.autograd import Function
+
+import approx_ops  # native module: approx_gemm_forward / acc_gemm_forward_fp32 / approx_gemm_backward
+
+lut_appmult = None   # uint16 padded table of the approximate products
+lut_grad_a = None    # int16 padded table, 16 x d(product)/d(first operand)
+lut_grad_b = None    # int16 padded table, 16 x d(product)/d(second operand)
+
+_SECTION_HEADERS = (
+    ("LUT for approximate multiplier:", 0),
+    ("LUT for the gradient of the approximate multiplier w.r.t. the first operand:", 1),
+    ("LUT for the gradient of the approximate multiplier w.r.t. the second operand:", 2),
+)
+_TAIL = {7: 638, 8: 0, 4: 718, 6: 830}
+
+
+def lut_geometry(quantization_bit):
+    """(rows, cols, elem_num) of the padded table (reference ``approx_ops.py:21-41``)."""
+    if quantization_bit not in _TAIL:
+        raise NotImplementedError(f'quantization_bit = {quantization_bit} is not supported')
+    maxval = 2 ** quantization_bit - 1
+    rows, cols = maxval + 2, maxval + 3
+    return rows, cols, rows * cols + _TAIL[quantization_bit]
+
+
+def read_lut_file(file_name, quantization_bit):
+    """Parse a table file into three padded 1-D NumPy arrays (uint16, int16, int16).
+
+    Same acceptance rules as the reference's line-by-line state machine (``approx_ops.py:54-79``):
+    everything before the first section header is ignored, a header switches the section, every
+    other line must be ``a b value``; entries the file does not mention stay 0.  The sections are
+    parsed in bulk instead of one device write per entry.  ``.gz`` files are accepted as well.
+    """
+    rows, cols, elems = lut_geometry(quantization_bit)
+    opener = gzip.open if str(file_name).endswith(".gz") else open
+    with opener(file_name, "rt") as f:
+        lines = f.readlines()
+    marks = []  # (line index, section id)
+    for i, line in enumerate(lines):
+        if line[:3] == "LUT":
+            for header, sec in _SECTION_HEADERS:
+                if line.startswith(header):
+                    marks.append((i, sec))
+                    break
+    tables = [np.zeros(elems, np.uint16), np.zeros(elems, np.int16), np.zeros(elems, np.int16)]
+    for j, (start, sec) in enumerate(marks):
+        stop = marks[j + 1][0] if j + 1 < len(marks) else len(lines)
+        body = lines[start + 1:stop]
+        if not body:
+            continue
+        vals = np.array(" ".join(body).split(), dtype=np.int64)
+        if vals.size != 3 * len(body):
+            raise ValueError(f"{file_name}: every table line must hold three integers 'a b value'")
+        vals = vals.reshape(-1, 3)
+        idx = vals[:, 0] * cols + vals[:, 1]
+        if idx.size and (idx.min() < 0 or idx.max() >= elems):
+            raise IndexError(f"{file_name}: operand outside the {quantization_bit}-bit table")
+        tables[sec][idx] = vals[:, 2].astype(tables[sec].dtype)
+    return tables
+
+
+def set_lookup_tables(device, appmult, grad_a, grad_b):
+    """Install padded tables given as arrays/tensors (uint16, int16, int16); one copy per table."""
+    global lut_appmult, lut_grad_a, lut_grad_b
+    lut_appmult = torch.as_tensor(np.ascontiguousarray(appmult, np.uint16)).to(device)
+    lut_grad_a = torch.as_tensor(np.ascontiguousarray(grad_a, np.int16)).to(device)
+    lut_grad_b = torch.as_tensor(np.ascontiguousarray(grad_b, np.int16)).to(device)
+
+
+def init_lookup_tables(device, file_name, quantization_bit):
+    """Load the forward and gradient tables of an approximate multiplier onto ``device``
+    (reference ``approx_ops.py:18-79``)."""
+    lut_geometry(quantization_bit)  # raises NotImplementedError first, like the reference
+    print(f'Initializing lookup tables from {file_name}...')
+    fwd, ga, gb = read_lut_file(file_name, quantization_bit)
+    set_lookup_tables(device, fwd, ga, gb)
+
+
+def _codes(x):
+    return x.to(torch.uint8).contiguous()
+
+
+def _lut_forward(a_codes, b_codes):
+    M, N = a_codes.shape[0], b_codes.shape[1]
+    c = torch.empty((M, N), dtype=torch.uint32, device=a_codes.device)
+    approx_ops.approx_gemm_forward(a_codes, b_codes, c, lut_appmult)
+    return c.to(torch.float32)
+
+
+class AccGemm(Function):
+    """Accurate fp32 GEMM through the native kernel (reference ``approx_ops.py:89-145``)."""
+
+    @staticmethod
+    def forward(ctx, a, b):
+        a_c, b_c = a.contiguous().to(torch.float32), b.contiguous().to(torch.float32)
+        c = torch.empty((a_c.shape[0], b_c.shape[1]), dtype=torch.float32, device=a_c.device)
+        approx_ops.acc_gemm_forward_fp32(a_c, b_c, c)
+        ctx.save_for_backward(a_c, b_c)
+        return c
+
+    @staticmethod
+    def backward(ctx, g_c):
+        assert g_c.dtype == torch.float32
+        a_c, b_c = ctx.saved_tensors
+        return torch.matmul(g_c, b_c.t()), torch.matmul(a_c.t(), g_c)
+
+
+acc_gemm_op = AccGemm.apply
+
+
+class ApproxGemm(Function):
+    """LUT GEMM with LUT gradients (reference ``approx_ops.py:148-205``).
+
+    ``a`` [M,K] and ``b`` [K,N] hold integer codes (any dtype convertible to uint8, any strides);
+    returns fp32 [M,N]."""
+
+    @staticmethod
+    def forward(ctx, a, b):
+        a_c, b_c = _codes(a), _codes(b)
+        ctx.save_for_backward(a_c, b_c)
+        return _lut_forward(a_c, b_c)
+
+    @staticmethod
+    def backward(ctx, g_c):
+        assert g_c.dtype == torch.float32
+        a_c, b_c = ctx.saved_tensors
+        g_a = torch.empty(a_c.shape, dtype=torch.float32, device=g_c.device)
+        g_b = torch.empty(b_c.shape, dtype=torch.float32, device=g_c.device)
+        approx_ops.approx_gemm_backward(g_c.contiguous(), a_c, b_c, g_a, g_b, lut_grad_a, lut_grad_b)
+        return g_a, g_b
+
+
+approx_gemm_op = ApproxGemm.apply
+
+
+class ApproxGemmBaseline(Function):
+    """LUT GEMM forward, straight-through (dense) gradients on the original operands
+    (reference ``approx_ops.py:210-262``)."""
+
+    @staticmethod
+    def forward(ctx, a, b):
+        ctx.save_for_backward(a, b)
+        return _lut_forward(_codes(a), _codes(b))
+
+    @staticmethod
+    def backward(ctx, g_c):
+        assert g_c.dtype == torch.float32
+        a, b = ctx.saved_tensors
+        g = g_c.contiguous()
+        return torch.matmul(g, b.t().contiguous()), torch.matmul(a.t().contiguous(), g)
+
+
+approx_gemm_baseline_op = ApproxGemmBaseline.apply
+
+
+def _conv2d_by_gemm(gemm, input, weight, bias, stride, padding, dilation, groups):
+    # reference: approx_ops.py:545-571.  Only element 0 of the tuples is used; padding pixels hold
+    # code 0 (not the zero-point); K index order is c*kh*kw + i*kw + j.
+    assert bias is None, 'bias is not supported in approximate convolution'
+    assert groups == 1, 'groups is not supported in approximate convolution'
+    s, p, d = stride[0], padding[0], dilation[0]
+    batch, cin, h, w = input.shape
+    cout, _, kh, kw = weight.shape
+    oh = (h + 2 * p - d * (kh - 1) - 1) // s + 1
+    ow = (w + 2 * p - d * (kw - 1) - 1) // s + 1
+    cols = F.unfold(F.pad(input, (p, p, p, p), mode='constant', value=0), kernel_size=(kh, kw), dilation=(d, d), stride=(s, s))
+    lhs = cols.transpose(1, 2).reshape(-1, cin * kh * kw)      # [batch*oh*ow, cin*kh*kw]
+    rhs = weight.view(cout, -1).t()                            # [cin*kh*kw, cout]
+    out = gemm(lhs, rhs)                                       # [batch*oh*ow, cout]
+    return out.view(batch, oh * ow, cout).transpose(1, 2).view(batch, cout, oh, ow)
+
+
+def approx_conv2d_op(input, weight, bias, stride, padding, dilation, groups):
+    """conv2d as im2col + LUT GEMM with LUT gradients (reference ``approx_ops.py:530-573``).
+    ``input`` [B,C,H,W] and ``weight`` [O,C,kh,kw] hold integer codes; returns fp32 [B,O,oh,ow]."""
+    return _conv2d_by_gemm(approx_gemm_op, input, weight, bias, stride, padding, dilation, groups)
+
+
+def approx_conv2d_baseline_op(input, weight, bias, stride, padding, dilation, groups):
+    """Same forward, straight-through gradients (reference ``approx_ops.py:576-619``)."""
+    return _conv2d_by_gemm(approx_gemm_baseline_op, input, weight, bias, stride, padding, dilation, groups)

@@ -1,0 +1,100 @@
+/*
+ * amr_lutgemm.h -- C ABI of the MI355X (gfx950) LUT-based approximate-multiplier GEMM.
+ *
+ * Shared library: libamr_lutgemm.so.  Plain pointers and sizes only; every pointer is a DEVICE
+ * pointer on the current HIP device unless stated otherwise; `stream` is a hipStream_t passed as
+ * void* (NULL = the default stream).  All launches are asynchronous on `stream`.
+ *
+ * Return value: 0 on success, a negative AMR_E* code on a rejected argument, or a positive
+ * hipError_t value when the HIP runtime reported a failure.  amr_last_error() returns a
+ * thread-local human readable message for the last non-zero return.
+ *
+ * Table layout ("padded table"), as the reference defines it
+ * (self_ops/src/approx_mult.h:12-40, self_ops/ops_py/approx_ops.py:21-41,70-77):
+ *   bits b in {4, 6, 7, 8};  rows = 2^b + 1, cols = 2^b + 2;
+ *   entry (a, b) at a * cols + b;  total length rows * cols + tail, tail = 718 / 830 / 638 / 0;
+ *   everything outside [0,2^b) x [0,2^b) is zero, so the code value 2^b is a "masked" operand
+ *   that contributes 0 (self_ops/src/approx_mult.h:40).
+ * The bit-width is derived from the table length at run time (1024 -> 4, 5120 -> 6, 17408 -> 7,
+ * 66306 -> 8); the reference fixes it with a compile-time macro instead (approx_mult.h:12).
+ * Operand codes above 2^b are a precondition violation exactly as in the reference
+ * (approx_gemm_forward.cu:200 reads out of bounds); they are not checked on the device.
+ */
+#ifndef AMR_LUTGEMM_H
+#define AMR_LUTGEMM_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define AMR_OK 0
+#define AMR_EINVAL (-1)    /* null pointer, negative size, misaligned table pointer            */
+#define AMR_ELUTLEN (-2)   /* table length matches no supported bit-width                      */
+#define AMR_EWORKSPACE (-3)/* caller workspace too small                                       */
+#define AMR_EUNSUPPORTED (-4)
+
+/* Library version (major*10000 + minor*100 + patch) and the gfx target it was built for. */
+int amr_version(void);
+const char *amr_target_arch(void);
+const char *amr_last_error(void);
+
+/* Geometry helpers (host only, no device work).
+ * Mirrors self_ops/ops_py/approx_ops.py:21-41.  Return AMR_ELUTLEN for unsupported values. */
+int amr_lut_geometry(int bits, int *rows, int *cols, int64_t *elem_num);
+int amr_bits_from_lut_elems(int64_t lut_elems);
+
+/*
+ * Forward:  C[m,n] = sum_{k<K} lut[A[m,k] * cols + B[k,n]]   (uint32 wrap-around accumulate)
+ * Replaces approx_gemm_forward_gpu (self_ops/src/approx_gemm_forward.cu:241-314), which is what
+ * the pybind function approx_ops.approx_gemm_forward binds (self_ops/src/op_register.cpp:17).
+ *   A   [M,K] uint8 row-major      B [K,N] uint8 row-major      C [M,N] uint32 row-major (overwritten)
+ *   lut padded table, uint16, length lut_elems, 4-byte aligned.
+ * M, K or N equal to 0 is accepted (K == 0 zero-fills C).
+ */
+int amr_lut_gemm_forward(const uint8_t *A, const uint8_t *B, uint32_t *C, const uint16_t *lut,
+                         int64_t lut_elems, int M, int K, int N, void *stream);
+
+/*
+ * Backward (both gradients, as the reference always produces both):
+ *   gA[m,k] = (1/16) * sum_{n<N} gC[m,n] * (float)lut_grad_a[A[m,k] * cols + B[k,n]]
+ *   gB[k,n] = (1/16) * sum_{m<M} (float)lut_grad_b[A[m,k] * cols + B[k,n]] * gC[m,n]
+ * Replaces approx_gemm_backward_gpu (self_ops/src/approx_gemm_backward.cu:506-624), bound as
+ * approx_ops.approx_gemm_backward (self_ops/src/op_register.cpp:19).  fp32 accumulation; the
+ * summation order differs from the reference's sequential order (results agree to fp32
+ * summation-order tolerance and are deterministic run to run).
+ *   gC [M,N] fp32   A [M,K] uint8   B [K,N] uint8   gA [M,K] fp32 (overwritten)   gB [K,N] fp32 (overwritten)
+ *   lut_grad_a / lut_grad_b: padded tables, int16 (slope x 16), length lut_elems, 4-byte aligned.
+ * gA or gB may be NULL to skip that gradient (extension; the reference computes both).
+ * workspace: device scratch for the split-M partial sums of gB, at least
+ *   amr_lut_gemm_backward_workspace_bytes(M,K,N) bytes, 256-byte aligned; or NULL, in which case the
+ *   library keeps a per-device buffer that it grows with hipMalloc when needed (not stream-safe
+ *   across concurrent streams; pass a workspace for that).
+ */
+size_t amr_lut_gemm_backward_workspace_bytes(int M, int K, int N);
+int amr_lut_gemm_backward(const float *gC, const uint8_t *A, const uint8_t *B, float *gA, float *gB,
+                          const int16_t *lut_grad_a, const int16_t *lut_grad_b, int64_t lut_elems,
+                          int M, int K, int N, void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * Accurate fp32 GEMM  C = A . B  (row-major), kept for API parity only.
+ * Replaces acc_gemm_forward_fp32_gpu (self_ops/src/approx_gemm_forward.cu:494-571), bound as
+ * approx_ops.acc_gemm_forward_fp32 (self_ops/src/op_register.cpp:18).
+ */
+int amr_acc_gemm_forward_fp32(const float *A, const float *B, float *C, int M, int K, int N, void *stream);
+
+/*
+ * LDS gather-rate probe used to calibrate the roofline denominator.  Runs `iters` rounds of 8
+ * ds_read_u16 per wave with conflict-free (pattern 0) or uniform-random-in-a-256-byte-row
+ * (pattern 1) addresses on every CU and writes the kernel time in milliseconds to *ms_out (host
+ * pointer; the call synchronises the stream).  gathers = waves_per_cu * n_cu * iters * 8 * 64.
+ * No counterpart in the reference.
+ */
+int amr_lds_gather_probe(int pattern, int waves_per_cu, int iters, float *ms_out, double *gathers_out, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* AMR_LUTGEMM_H */

@@ -1,0 +1,124 @@
+"""GPU tests of the Python operator layer (approx_ops module + self_ops autograd Functions), written
+the way a user of the reference would call them."""
+import os
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ops(golden_dir):
+    import self_ops
+    from self_ops.ops_py import approx_ops as P
+    P.init_lookup_tables(torch.device("cuda"), os.path.join(golden_dir, "lut7_resub_63_bp8.txt.gz"), 7)
+    return self_ops, P
+
+
+def test_native_module_checks_dtype_shape_contiguity(ops):
+    import approx_ops
+    print("native checks", flush=True)
+    d = "cuda"
+    a = torch.zeros(4, 6, dtype=torch.uint8, device=d)
+    b = torch.zeros(6, 8, dtype=torch.uint8, device=d)
+    c = torch.zeros(4, 8, dtype=torch.uint32, device=d)
+    lut = torch.zeros(17408, dtype=torch.uint16, device=d)
+    approx_ops.approx_gemm_forward(a, b, c, lut)
+    with pytest.raises(RuntimeError, match="b_tensor must be contiguous"):
+        approx_ops.approx_gemm_forward(a, torch.zeros(8, 6, dtype=torch.uint8, device=d).t(), c, lut)
+    with pytest.raises(RuntimeError, match="a_tensor must be of type"):
+        approx_ops.approx_gemm_forward(a.float(), b, c, lut)
+    with pytest.raises(RuntimeError, match="c_tensor's shape should be 4 x 8"):
+        approx_ops.approx_gemm_forward(a, b, torch.zeros(4, 9, dtype=torch.uint32, device=d), lut)
+    with pytest.raises(RuntimeError, match="b_tensor's shape should be"):
+        approx_ops.approx_gemm_forward(a, torch.zeros(5, 8, dtype=torch.uint8, device=d), c, lut)
+    with pytest.raises(RuntimeError, match="QUANTIZATION_BIT"):
+        approx_ops.approx_gemm_forward(a, b, c, lut[:17000].contiguous())
+    with pytest.raises(RuntimeError, match="lut_appmult_tensor must be a CUDAtensor"):
+        approx_ops.approx_gemm_forward(a, b, c, lut.cpu())
+
+
+def test_gemm_op_forward_and_backward_against_oracle(ops, oracle, golden_dir):
+    self_ops, P = ops
+    print("gemm op", flush=True)
+    fwd, ga, gb = oracle.parse_lut_file(os.path.join(golden_dir, "lut7_resub_63_bp8.txt.gz"), 7)
+    rng = np.random.default_rng(0)
+    A = rng.integers(0, 128, (200, 72)).astype(np.uint8)
+    B = rng.integers(0, 128, (72, 48)).astype(np.uint8)
+    a = torch.tensor(A, dtype=torch.float32, device="cuda", requires_grad=True)
+    bt = torch.tensor(B.T.copy(), dtype=torch.float32, device="cuda", requires_grad=True)   # weight arrives as a .t() view
+    out = self_ops.approx_gemm_op(a, bt.t())
+    assert out.dtype == torch.float32
+    assert (out.detach().cpu().numpy() == oracle.forward_np(A, B, fwd).astype(np.float32)).all()
+    g = torch.randn(200, 48, device="cuda")
+    out.backward(g)
+    a64, b64 = oracle.backward_np(g.cpu().numpy(), A, B, ga, gb)
+    np.testing.assert_allclose(a.grad.cpu().numpy(), a64, rtol=0, atol=1e-5 * np.abs(a64).max())
+    np.testing.assert_allclose(bt.grad.cpu().numpy().T, b64, rtol=0, atol=1e-5 * np.abs(b64).max())
+
+
+def test_baseline_op_uses_dense_ste_gradients(ops):
+    self_ops, P = ops
+    print("baseline op", flush=True)
+    a = torch.randint(0, 128, (50, 30), device="cuda").float().requires_grad_()
+    b = torch.randint(0, 128, (30, 20), device="cuda").float().requires_grad_()
+    out = self_ops.approx_gemm_baseline_op(a, b)
+    ref = self_ops.approx_gemm_op(a.detach(), b.detach())
+    assert torch.equal(out, ref)
+    g = torch.randn(50, 20, device="cuda")
+    out.backward(g)
+    torch.testing.assert_close(a.grad, g @ b.detach().t())
+    torch.testing.assert_close(b.grad, a.detach().t() @ g)
+
+
+@pytest.mark.parametrize("stride,padding,dilation,k", [(1, 1, 1, 3), (2, 1, 1, 3), (1, 0, 1, 1), (2, 0, 1, 1), (1, 2, 2, 3)])
+def test_conv_op_equals_conv2d_with_exact_multiplier(ops, oracle, stride, padding, dilation, k):
+    self_ops, P = ops
+    print("conv op", stride, padding, dilation, k, flush=True)
+    keep = (P.lut_appmult, P.lut_grad_a, P.lut_grad_b)
+    try:
+        n = np.arange(128)
+        Sx, Sy = oracle.ste_tables16(7)
+        P.set_lookup_tables("cuda", oracle.pack_table(n[:, None] * n[None, :], 7, np.uint16),
+                            oracle.pack_table(Sx, 7, np.int16), oracle.pack_table(Sy, 7, np.int16))
+        x = torch.randint(0, 128, (3, 5, 10, 10), device="cuda").float().requires_grad_()
+        w = torch.randint(0, 128, (7, 5, k, k), device="cuda").float().requires_grad_()
+        args = dict(bias=None, stride=(stride, stride), padding=(padding, padding), dilation=(dilation, dilation), groups=1)
+        y = self_ops.approx_conv2d_op(x, w, **args)
+        x2, w2 = x.detach().clone().requires_grad_(), w.detach().clone().requires_grad_()
+        y2 = F.conv2d(x2, w2, **args)
+        assert torch.equal(y, y2)                                    # integers < 2^24: exact in fp32
+        g = torch.randint(-2, 3, y.shape, device="cuda").float()
+        y.backward(g)
+        y2.backward(g)
+        assert torch.equal(x.grad, x2.grad) and torch.equal(w.grad, w2.grad)
+        yb = self_ops.approx_conv2d_baseline_op(x.detach(), w.detach(), **args)
+        assert torch.equal(yb, y2.detach())
+    finally:
+        P.lut_appmult, P.lut_grad_a, P.lut_grad_b = keep
+
+
+def test_conv_op_against_oracle_with_shipped_table(ops, oracle, golden_dir):
+    self_ops, P = ops
+    print("conv oracle", flush=True)
+    fwd, _, _ = oracle.parse_lut_file(os.path.join(golden_dir, "lut7_resub_63_bp8.txt.gz"), 7)
+    rng = np.random.default_rng(3)
+    x = rng.integers(0, 128, (2, 4, 8, 8)).astype(np.uint8)
+    w = rng.integers(0, 128, (6, 4, 3, 3)).astype(np.uint8)
+    y = self_ops.approx_conv2d_op(torch.tensor(x, device="cuda").float(), torch.tensor(w, device="cuda").float(), None,
+                                  (1, 1), (1, 1), (1, 1), 1)
+    want = oracle.conv2d_lut_np(x, w, fwd, 1, 1, 1)     # padding pixels are code 0 and LUT[0][w] != 0 for this table
+    assert (y.cpu().numpy() == want.astype(np.float32)).all()
+
+
+def test_acc_gemm_op(ops):
+    self_ops, P = ops
+    a = torch.randn(70, 40, device="cuda", requires_grad=True)
+    b = torch.randn(40, 30, device="cuda", requires_grad=True)
+    y = P.acc_gemm_op(a, b)
+    torch.testing.assert_close(y, a @ b, rtol=1e-4, atol=1e-4)
+    y.sum().backward()
+    torch.testing.assert_close(a.grad, torch.ones(70, 30, device="cuda") @ b.detach().t())

@@ -1,0 +1,261 @@
+"""GPU parity tests (run on the MI355X box with -m gpu): the HIP path, called through the C ABI of
+libamr_lutgemm.so, against the CPU oracle on the same seeded inputs.
+
+Bars: forward bit-exact (uint32); backward within 1e-5 of the float64 sums, relative to the sum of
+term magnitudes per output (fp32 summation-order tolerance) and norm-wise relative to the largest
+output; STE tables with small-integer gC are bit-exact.
+"""
+import ctypes
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from conftest import PKG
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-5
+
+
+@pytest.fixture(scope="module")
+def lib():
+    assert torch.cuda.is_available(), "gpu tests need a device"
+    L = ctypes.CDLL(os.path.join(PKG, "libamr_lutgemm.so"))
+    vp, i64, i, sz = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_size_t
+    L.amr_last_error.restype = ctypes.c_char_p
+    L.amr_lut_gemm_forward.argtypes = [vp, vp, vp, vp, i64, i, i, i, vp]
+    L.amr_lut_gemm_backward.argtypes = [vp, vp, vp, vp, vp, vp, vp, i64, i, i, i, vp, sz, vp]
+    L.amr_lut_gemm_backward_workspace_bytes.argtypes = [i, i, i]
+    L.amr_lut_gemm_backward_workspace_bytes.restype = sz
+    L.amr_acc_gemm_forward_fp32.argtypes = [vp, vp, vp, i, i, i, vp]
+    return L
+
+
+def dev(x):
+    return torch.from_numpy(np.ascontiguousarray(x)).cuda()
+
+
+def gpu_forward(lib, A, B, flat_u16):
+    M, K = A.shape
+    N = B.shape[1]
+    a, b, l = dev(A), dev(B), dev(flat_u16)
+    c = torch.full((M, N), 0xDEADBEEF, dtype=torch.int64, device="cuda").to(torch.int32)  # poison: op must overwrite
+    rc = lib.amr_lut_gemm_forward(a.data_ptr(), b.data_ptr(), c.data_ptr(), l.data_ptr(), l.numel(), M, K, N, None)
+    assert rc == 0, lib.amr_last_error()
+    torch.cuda.synchronize()
+    return c.cpu().numpy().view(np.uint32)
+
+
+def gpu_backward(lib, g, A, B, la, lb, own_workspace=True):
+    M, K = A.shape
+    N = B.shape[1]
+    gd, a, b, ta, tb = dev(g), dev(A), dev(B), dev(la), dev(lb)
+    ga = torch.full((M, K), float("nan"), device="cuda")
+    gb = torch.full((K, N), float("nan"), device="cuda")
+    need = lib.amr_lut_gemm_backward_workspace_bytes(M, K, N)
+    ws = torch.empty(max(need, 1), dtype=torch.uint8, device="cuda") if own_workspace else None
+    rc = lib.amr_lut_gemm_backward(gd.data_ptr(), a.data_ptr(), b.data_ptr(), ga.data_ptr(), gb.data_ptr(), ta.data_ptr(),
+                                   tb.data_ptr(), ta.numel(), M, K, N, ws.data_ptr() if ws is not None else None,
+                                   need if ws is not None else 0, None)
+    assert rc == 0, lib.amr_last_error()
+    torch.cuda.synchronize()
+    return ga.cpu().numpy(), gb.cpu().numpy()
+
+
+def rand_case(seed, M, K, N, bits):
+    rng = np.random.default_rng(seed)
+    n = 1 << bits
+    A = rng.integers(0, n, (M, K)).astype(np.uint8)
+    B = rng.integers(0, n, (K, N)).astype(np.uint8)
+    T = rng.integers(0, 65536, (n, n))
+    return rng, A, B, T
+
+
+FWD_SHAPES = [(1, 1, 1), (3, 5, 7), (9, 27, 10), (64, 64, 64), (33, 130, 65), (128, 576, 64), (257, 100, 129),
+              (100, 64, 300), (40, 1152, 128), (1000, 27, 64), (70, 2304, 256), (17, 9, 513)]
+
+
+@pytest.mark.parametrize("bits", [7, 8, 6, 4])
+@pytest.mark.parametrize("shape", FWD_SHAPES)
+def test_forward_bit_exact_random_tables(lib, oracle, bits, shape):
+    print("forward", bits, shape, flush=True)
+    _, A, B, T = rand_case(hash((bits, shape)) % 2**32, *shape, bits)
+    flat = oracle.pack_table(T, bits, np.uint16)
+    assert (gpu_forward(lib, A, B, flat) == oracle.forward_c(A, B, flat, bits)).all()
+
+
+def test_forward_config1_bit_exact_and_exact_multiplier(lib, oracle):
+    print("forward config1", flush=True)
+    A, B, T, _ = oracle.synth_gemm(4096, 576, 64, bits=7, err=64, seed=0)
+    flat = oracle.pack_table(T, 7, np.uint16)
+    got = gpu_forward(lib, A, B, flat)
+    assert (got == oracle.forward_c(A, B, flat, 7)).all()
+    exact = oracle.pack_table(np.arange(128)[:, None] * np.arange(128)[None, :], 7, np.uint16)
+    assert (gpu_forward(lib, A, B, exact) == (A.astype(np.int64) @ B.astype(np.int64)).astype(np.uint32)).all()
+
+
+def test_forward_masked_code_and_unaligned_views(lib, oracle):
+    print("forward masked/unaligned", flush=True)
+    _, A, B, T = rand_case(77, 50, 37, 70, 7)
+    A[:, 3] = 128
+    B[5, :] = 128
+    flat = oracle.pack_table(T, 7, np.uint16)
+    want = oracle.forward_c(A, B, flat, 7)
+    assert (gpu_forward(lib, A, B, flat) == want).all()
+    # operand pointers at odd byte addresses (a slice of a larger buffer)
+    buf_a = torch.zeros(A.size + 3, dtype=torch.uint8, device="cuda")
+    buf_b = torch.zeros(B.size + 1, dtype=torch.uint8, device="cuda")
+    buf_a[3:] = dev(A).flatten()
+    buf_b[1:] = dev(B).flatten()
+    l = dev(flat)
+    c = torch.zeros(want.shape, dtype=torch.int32, device="cuda")
+    rc = lib.amr_lut_gemm_forward(buf_a.data_ptr() + 3, buf_b.data_ptr() + 1, c.data_ptr(), l.data_ptr(), l.numel(), 50, 37, 70, None)
+    assert rc == 0
+    assert (c.cpu().numpy().view(np.uint32) == want).all()
+
+
+def test_forward_golden_shipped_tables(lib, oracle, golden_dir):
+    print("forward golden", flush=True)
+    fwd, _, _ = oracle.parse_lut_file(os.path.join(golden_dir, "lut7_resub_63_bp8.txt.gz"), 7)
+    _, A, B, _ = rand_case(5, 300, 200, 96, 7)
+    flat = oracle.pack_table(fwd, 7, np.uint16)
+    assert (gpu_forward(lib, A, B, flat) == oracle.forward_np(A, B, fwd)).all()
+    z = np.load(os.path.join(golden_dir, "lut8_resub_183.npz"))
+    _, A, B, _ = rand_case(6, 200, 150, 80, 8)
+    flat = oracle.pack_table(z["fwd"], 8, np.uint16)
+    assert (gpu_forward(lib, A, B, flat) == oracle.forward_np(A, B, z["fwd"])).all()
+
+
+def test_forward_wraparound_and_k_zero(lib, oracle):
+    print("forward wrap", flush=True)
+    A = np.full((3, 70000), 255, np.uint8)
+    B = np.full((70000, 5), 255, np.uint8)
+    flat = oracle.pack_table(np.full((256, 256), 65535), 8, np.uint16)
+    assert (gpu_forward(lib, A, B, flat) == (70000 * 65535) % 2**32).all()
+    assert (gpu_forward(lib, np.zeros((4, 0), np.uint8), np.zeros((0, 6), np.uint8), flat) == 0).all()
+
+
+def check_backward(oracle, got, g, A, B, la, lb, bits):
+    gA, gB = got
+    a64, b64, absA, absB = oracle.backward_c_f64(g, A, B, la, lb, bits, want_abs=True)
+    assert np.isfinite(gA).all() and np.isfinite(gB).all()
+    for x, r, ab in ((gA, a64, absA), (gB, b64, absB)):
+        err = np.abs(x - r)
+        assert np.max(err / np.maximum(ab, 1e-30)) < TOL          # relative to sum of |terms|
+        assert np.max(err) <= TOL * np.max(np.abs(r)) + 1e-30      # norm-wise relative
+
+
+BWD_SHAPES = [(1, 1, 1), (3, 5, 7), (9, 27, 10), (64, 64, 64), (33, 130, 65), (600, 96, 64), (257, 100, 129),
+              (1100, 27, 64), (300, 288, 256), (70, 50, 513)]
+
+
+@pytest.mark.parametrize("bits", [7, 8, 6])
+@pytest.mark.parametrize("shape", BWD_SHAPES)
+def test_backward_within_tolerance_random_tables(lib, oracle, bits, shape):
+    print("backward", bits, shape, flush=True)
+    rng, A, B, _ = rand_case(hash((bits, shape, "b")) % 2**32, *shape, bits)
+    n = 1 << bits
+    la = oracle.pack_table(rng.integers(-32768, 32768, (n, n)), bits, np.int16)
+    lb = oracle.pack_table(rng.integers(-32768, 32768, (n, n)), bits, np.int16)
+    g = rng.standard_normal((shape[0], shape[2])).astype(np.float32)
+    check_backward(oracle, gpu_backward(lib, g, A, B, la, lb), g, A, B, la, lb, bits)
+
+
+def test_backward_config2_difference_tables_and_ste(lib, oracle):
+    print("backward config2", flush=True)
+    A, B, T, g = oracle.synth_gemm(4096, 576, 64, bits=7, err=64, seed=0)
+    Gx, Gy = oracle.gen_bp_lut(T, 8)
+    la, lb = oracle.pack_table(Gx, 7, np.int16), oracle.pack_table(Gy, 7, np.int16)
+    check_backward(oracle, gpu_backward(lib, g, A, B, la, lb), g, A, B, la, lb, 7)
+    check_backward(oracle, gpu_backward(lib, g, A, B, la, lb, own_workspace=False), g, A, B, la, lb, 7)
+    # STE tables + small integer gC: every partial sum is exact in fp32 -> bit-exact dense matmuls
+    Sx, Sy = oracle.ste_tables16(7)
+    gi = np.random.default_rng(1).integers(-4, 5, g.shape).astype(np.float32)
+    gA, gB = gpu_backward(lib, gi, A, B, oracle.pack_table(Sx, 7, np.int16), oracle.pack_table(Sy, 7, np.int16))
+    assert (gA == gi.astype(np.int64) @ B.astype(np.int64).T).all()
+    assert (gB == A.astype(np.int64).T @ gi.astype(np.int64)).all()
+
+
+def test_backward_golden_shipped_tables(lib, oracle, golden_dir):
+    print("backward golden", flush=True)
+    _, ga, gb = oracle.parse_lut_file(os.path.join(golden_dir, "lut7_evo_081_bp16.txt.gz"), 7)
+    rng, A, B, _ = rand_case(8, 500, 144, 128, 7)
+    g = rng.standard_normal((500, 128)).astype(np.float32)
+    la, lb = oracle.pack_table(ga, 7, np.int16), oracle.pack_table(gb, 7, np.int16)
+    check_backward(oracle, gpu_backward(lib, g, A, B, la, lb), g, A, B, la, lb, 7)
+    z = np.load(os.path.join(golden_dir, "lut8_resub_183.npz"))
+    rng, A, B, _ = rand_case(9, 300, 100, 70, 8)
+    g = rng.standard_normal((300, 70)).astype(np.float32)
+    la, lb = oracle.pack_table(z["grad_a"], 8, np.int16), oracle.pack_table(z["grad_b"], 8, np.int16)
+    check_backward(oracle, gpu_backward(lib, g, A, B, la, lb), g, A, B, la, lb, 8)
+
+
+def test_backward_deterministic_and_skippable_outputs(lib, oracle):
+    print("backward determinism", flush=True)
+    rng, A, B, _ = rand_case(10, 3000, 64, 64, 7)
+    la = oracle.pack_table(rng.integers(-3000, 3000, (128, 128)), 7, np.int16)
+    g = rng.standard_normal((3000, 64)).astype(np.float32)
+    r1 = gpu_backward(lib, g, A, B, la, la)
+    r2 = gpu_backward(lib, g, A, B, la, la)
+    assert (r1[0] == r2[0]).all() and (r1[1] == r2[1]).all()
+    gd, a, b, t = dev(g), dev(A), dev(B), dev(la)
+    gb = torch.zeros(64, 64, device="cuda")
+    assert lib.amr_lut_gemm_backward(gd.data_ptr(), a.data_ptr(), b.data_ptr(), None, gb.data_ptr(), None, t.data_ptr(),
+                                     t.numel(), 3000, 64, 64, None, 0, None) == 0
+    torch.cuda.synchronize()
+    assert (gb.cpu().numpy() == r1[1]).all()
+
+
+def test_accgemm_matches_torch(lib):
+    print("accgemm", flush=True)
+    torch.manual_seed(0)
+    for (M, K, N) in [(1, 1, 1), (65, 33, 70), (256, 576, 64)]:
+        a = torch.randint(-4, 5, (M, K), device="cuda").float()
+        b = torch.randint(-4, 5, (K, N), device="cuda").float()
+        c = torch.full((M, N), float("nan"), device="cuda")
+        assert lib.amr_acc_gemm_forward_fp32(a.data_ptr(), b.data_ptr(), c.data_ptr(), M, K, N, None) == 0
+        torch.cuda.synchronize()
+        assert torch.equal(c, a @ b)
+
+
+# ---------------------------------------------------------------- full-size, size-independent properties
+def test_full_size_resnet_layer_properties(lib, oracle):
+    """conv2_x at batch 256 (M=262144, K=576, N=64): too big for the CPU oracle in seconds, so check
+    properties: exact-multiplier table == torch integer matmul; linearity in the table; row-subset
+    agreement with the oracle; STE backward == dense matmul on integer gC."""
+    print("full size", flush=True)
+    M, K, N = 262144, 576, 64
+    gen = torch.Generator(device="cuda").manual_seed(0)
+    a = torch.randint(0, 128, (M, K), dtype=torch.uint8, device="cuda", generator=gen)
+    b = torch.randint(0, 128, (K, N), dtype=torch.uint8, device="cuda", generator=gen)
+    rng = np.random.default_rng(0)
+    T1 = oracle.synth_lut(7, 64, rng)
+    Tx = np.arange(128)[:, None] * np.arange(128)[None, :]
+
+    def fwd(T):
+        l = dev(oracle.pack_table(T, 7, np.uint16))
+        c = torch.empty((M, N), dtype=torch.int32, device="cuda")
+        assert lib.amr_lut_gemm_forward(a.data_ptr(), b.data_ptr(), c.data_ptr(), l.data_ptr(), l.numel(), M, K, N, None) == 0
+        torch.cuda.synchronize()
+        return c
+
+    cx = fwd(Tx)
+    want = (a.double() @ b.double()).to(torch.int32)          # < 2^53, exact
+    assert torch.equal(cx, want)
+    c1 = fwd(T1)
+    assert torch.equal(fwd(T1 + Tx), c1 + cx)                  # linearity in the table
+    rows = np.r_[0:64, 131000:131064, M - 64:M]
+    sub = oracle.forward_c(a[rows].cpu().numpy(), b.cpu().numpy(), oracle.pack_table(T1, 7, np.uint16), 7)
+    assert (c1[rows].cpu().numpy().view(np.uint32) == sub).all()
+    # STE backward, integer gC in {-1,0,1}: sums are exact in fp32 (|gB| <= 262144*127 < 2^25 needs care -> use sparse gC)
+    g = (torch.rand((M, N), device="cuda", generator=gen) < 0.05).float() * torch.randint(-1, 2, (M, N), device="cuda", generator=gen).float()
+    Sx, Sy = oracle.ste_tables16(7)
+    ta, tb = dev(oracle.pack_table(Sx, 7, np.int16)), dev(oracle.pack_table(Sy, 7, np.int16))
+    ga = torch.empty((M, K), device="cuda")
+    gb = torch.empty((K, N), device="cuda")
+    assert lib.amr_lut_gemm_backward(g.data_ptr(), a.data_ptr(), b.data_ptr(), ga.data_ptr(), gb.data_ptr(), ta.data_ptr(),
+                                     tb.data_ptr(), ta.numel(), M, K, N, None, 0, None) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(ga.double(), g.double() @ b.double().t())
+    assert torch.equal(gb.double(), a.double().t() @ g.double())
