@@ -12,10 +12,10 @@ __global__ __launch_bounds__(1024) void lds_probe_kernel(int pattern, int iters,
     __syncthreads();
     const int lane = threadIdx.x & 63;
     uint32_t addr[4];
-    uint32_t h = (uint32_t)(lane * 747796405u + 2891336453u);
 #pragma unroll
     for (int s = 0; s < 4; ++s) {
-        h = h * 1664525u + 1013904223u;
+        uint32_t h = (uint32_t)(lane * 4 + s) + 0x9e3779b9u;   // murmur3 finaliser: a real per-lane hash
+        h ^= h >> 16; h *= 0x85ebca6bu; h ^= h >> 13; h *= 0xc2b2ae35u; h ^= h >> 16;
         // pattern 0: lane*2 (64 consecutive u16, conflict-free); pattern 1: random u16 inside a 256-byte row
         addr[s] = (pattern == 0 ? (uint32_t)(lane * 2) : ((h >> 10) % 128u) * 2u) + s * 1024;
     }

@@ -1,0 +1,237 @@
+#!/usr/bin/env python3
+"""Benchmark of the LUT-GEMM hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--layers]
+
+One "step" = forward + backward (gradA and gradB) LUT-GEMM of every conv layer and the fc layer of a
+CIFAR-style ResNet-18 at batch 256, 7-bit tables (BASELINE.json configs[2]: 21 GEMMs,
+426 564 648 960 LUT-MACs), called through the C ABI of libamr_lutgemm.so on torch's current stream.
+Operands are uniform random codes (worst case for LDS bank conflicts), the forward table is
+a*b + seeded error in [-64,64], the gradient tables are its difference-based slopes (half window 8)
+in the reference's int16 x16 encoding.  All inputs and outputs are resident in HBM before the timed
+region starts.  Prints ONE JSON line.
+
+The rate is compared with the LDS-gather roofline: one table gather per LUT-MAC,
+256 CUs x 2.4 GHz x 32 lanes/clk = 1.966e13 gathers/s (a wave64 ds_read_u16/b32 occupies the LDS pipe
+for two clocks when conflict-free; measured on this device by the probe in the library).
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+PKG = os.path.join(ROOT, "appmult-aware-retraining_amd")
+for _p in (ROOT, PKG):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+# (name, count, M, K, N) at batch 256: M = batch*oh*ow, K = cin*kh*kw, N = cout
+RESNET18_B256 = [
+    ("conv1", 1, 262144, 27, 64), ("conv2_x", 4, 262144, 576, 64),
+    ("conv3_first", 1, 65536, 576, 128), ("conv3_x", 3, 65536, 1152, 128), ("conv3_short", 1, 65536, 64, 128),
+    ("conv4_first", 1, 16384, 1152, 256), ("conv4_x", 3, 16384, 2304, 256), ("conv4_short", 1, 16384, 128, 256),
+    ("conv5_first", 1, 4096, 2304, 512), ("conv5_x", 3, 4096, 4608, 512), ("conv5_short", 1, 4096, 256, 512),
+    ("fc", 1, 256, 512, 10),
+]
+BATCH = 256
+LDS_GATHER_PEAK = 256 * 2.4e9 * 32      # gathers/s: CUs x peak clock x conflict-free lanes per clock
+HBM_PEAK = 8.0e12
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--layers", action="store_true", help="also print a per-layer table to stderr")
+    ap.add_argument("--only", default="", help="comma-separated layer names: restrict the step to them (profiling aid; the JSON line then describes that subset)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures the one-GPU hot path only: every box of this build has one GPU; run with --gpus 1")
+
+    import numpy as np
+    import torch
+
+    global RESNET18_B256
+    full = not args.only
+    if args.only:
+        keep = set(args.only.split(","))
+        RESNET18_B256 = [l for l in RESNET18_B256 if l[0] in keep]
+        assert RESNET18_B256, "no such layer"
+
+    import approx_ops  # loads libamr_lutgemm.so, fails loudly when it is missing
+    from oracle import lutgemm_oracle as O   # checker + CPU baseline only
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    lib = approx_ops._lib
+    stream = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+
+    # tables (config 1 recipe) -------------------------------------------------------------------
+    rng = np.random.default_rng(0)
+    T = O.synth_lut(7, 64, rng)
+    Gx, Gy = O.gen_bp_lut(T, 8)
+    lut = torch.from_numpy(O.pack_table(T, 7, np.uint16)).to(dev)
+    lga = torch.from_numpy(O.pack_table(Gx, 7, np.int16)).to(dev)
+    lgb = torch.from_numpy(O.pack_table(Gy, 7, np.int16)).to(dev)
+    L = lut.numel()
+
+    # operands, resident in HBM --------------------------------------------------------------------
+    gen = torch.Generator(device=dev).manual_seed(0)
+    bufs = {}
+    ws_need = 0
+    for name, cnt, M, K, N in RESNET18_B256:
+        bufs[name] = dict(
+            A=torch.randint(0, 128, (M, K), dtype=torch.uint8, device=dev, generator=gen),
+            B=torch.randint(0, 128, (K, N), dtype=torch.uint8, device=dev, generator=gen),
+            C=torch.empty((M, N), dtype=torch.int32, device=dev),
+            gC=torch.randn((M, N), dtype=torch.float32, device=dev, generator=gen),
+            gA=torch.empty((M, K), dtype=torch.float32, device=dev),
+            gB=torch.empty((K, N), dtype=torch.float32, device=dev))
+        ws_need = max(ws_need, lib.amr_lut_gemm_backward_workspace_bytes(M, K, N))
+    ws = torch.empty(max(ws_need, 256), dtype=torch.uint8, device=dev)
+
+    def fwd(name, M, K, N):
+        b = bufs[name]
+        rc = lib.amr_lut_gemm_forward(b["A"].data_ptr(), b["B"].data_ptr(), b["C"].data_ptr(), lut.data_ptr(), L, M, K, N, stream)
+        assert rc == 0, lib.amr_last_error()
+
+    def bwd(name, M, K, N, want_a=True, want_b=True):
+        b = bufs[name]
+        rc = lib.amr_lut_gemm_backward(b["gC"].data_ptr(), b["A"].data_ptr(), b["B"].data_ptr(),
+                                       b["gA"].data_ptr() if want_a else None, b["gB"].data_ptr() if want_b else None,
+                                       lga.data_ptr(), lgb.data_ptr(), L, M, K, N, ws.data_ptr(), ws.numel(), stream)
+        assert rc == 0, lib.amr_last_error()
+
+    def step():
+        for name, cnt, M, K, N in RESNET18_B256:
+            for _ in range(cnt):
+                fwd(name, M, K, N)
+        for name, cnt, M, K, N in reversed(RESNET18_B256):
+            for _ in range(cnt):
+                bwd(name, M, K, N)
+
+    macs_fwd = sum(c * M * K * N for _, c, M, K, N in RESNET18_B256)
+    assert macs_fwd == 142188216320 or not full
+    macs_step = 3 * macs_fwd
+
+    # quick parity guard on a row sample of one layer (the full parity suite is tests/ -m gpu) ---------
+    gname, _, gM, gK, gN = RESNET18_B256[-1] if not full else RESNET18_B256[4]
+    fwd(gname, gM, gK, gN)
+    torch.cuda.synchronize()
+    b = bufs[gname]
+    rows = slice(100, 164)
+    want = O.forward_c(b["A"][rows].cpu().numpy(), b["B"].cpu().numpy(), lut.cpu().numpy(), 7)
+    assert (b["C"][rows].cpu().numpy().view(np.uint32) == want).all(), "forward parity guard failed"
+
+    # timed region ------------------------------------------------------------------------------------
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ms_step = dt / args.steps * 1e3
+    rate = macs_step * args.steps / dt
+
+    # per-kernel timing with events on the launch stream -------------------------------------------------
+    def timed(fn, reps=3):
+        fn()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            fn()
+        e1.record()
+        e1.synchronize()
+        return e0.elapsed_time(e1) / reps
+
+    kernels = {"forward": 0.0, "gradA": 0.0, "gradB": 0.0}
+    per_layer = []
+    for name, cnt, M, K, N in RESNET18_B256:
+        tf = timed(lambda: fwd(name, M, K, N))
+        ta = timed(lambda: bwd(name, M, K, N, True, False))
+        tb = timed(lambda: bwd(name, M, K, N, False, True))
+        kernels["forward"] += cnt * tf
+        kernels["gradA"] += cnt * ta
+        kernels["gradB"] += cnt * tb
+        per_layer.append((name, cnt, M, K, N, tf, ta, tb))
+    dominant = max(kernels, key=kernels.get)
+    dom_ms = kernels[dominant]
+    dom_rate = macs_fwd / (dom_ms * 1e-3)         # each kernel does M*K*N gathers per GEMM
+    launches = sum(c for _, c, *_ in RESNET18_B256)
+    if args.layers:
+        print(f"{'layer':12s} cnt {'M':>7s} {'K':>5s} {'N':>4s}   fwd ms (GMAC/s)   gradA ms (GMAC/s)   gradB ms (GMAC/s)", file=sys.stderr)
+        for name, cnt, M, K, N, tf, ta, tb in per_layer:
+            w = M * K * N / 1e6
+            print(f"{name:12s} {cnt:3d} {M:7d} {K:5d} {N:4d}   {tf:7.3f} ({w/tf:7.0f})   {ta:7.3f} ({w/ta:7.0f})   {tb:7.3f} ({w/tb:7.0f})", file=sys.stderr)
+        print("kernel totals per step (ms):", {k: round(v, 3) for k, v in kernels.items()}, file=sys.stderr)
+
+    # algorithmic HBM bytes of the dominant kernel over one step
+    def hbm_bytes(kind, M, K, N):
+        if kind == "forward":
+            return M * K + K * N + 4 * M * N + 2 * L
+        if kind == "gradA":
+            return 4 * M * N + M * K + K * N + 4 * M * K + 2 * L
+        return 4 * M * N + M * K + K * N + 4 * K * N + 2 * L
+    dom_bytes = sum(c * hbm_bytes(dominant, M, K, N) for _, c, M, K, N in RESNET18_B256)
+
+    probe_free = approx_ops.lds_gather_probe(0, 16, 4000)
+    probe_row = approx_ops.lds_gather_probe(1, 16, 4000)
+
+    # single-GEMM configuration (BASELINE configs[1]: M=4096, K=576, N=64 forward+backward) ---------------
+    M1, K1, N1 = 4096, 576, 64
+    bufs["single"] = dict(A=torch.randint(0, 128, (M1, K1), dtype=torch.uint8, device=dev, generator=gen),
+                          B=torch.randint(0, 128, (K1, N1), dtype=torch.uint8, device=dev, generator=gen),
+                          C=torch.empty((M1, N1), dtype=torch.int32, device=dev),
+                          gC=torch.randn((M1, N1), dtype=torch.float32, device=dev, generator=gen),
+                          gA=torch.empty((M1, K1), dtype=torch.float32, device=dev),
+                          gB=torch.empty((K1, N1), dtype=torch.float32, device=dev))
+    t_single = timed(lambda: (fwd("single", M1, K1, N1), bwd("single", M1, K1, N1)), reps=50)
+
+    out = {
+        "metric": "LUT-MAC/s fwd+bwd (ResNet-18 conv shapes, 7-bit)",
+        "value": rate, "unit": "LUT-MAC/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "u8 codes; u16 table -> int32 sums (fwd); i16 table x f32 -> f32 sums (bwd)",
+        "data": "synthetic",
+        "config": {"workload": "resnet18_cifar_b256_7bit_lutgemm_fwd_bwd (BASELINE.json configs[2]: 20 conv + 1 fc GEMMs)" if full else "subset: " + args.only,
+                   "batch": BATCH, "lut_macs_per_step": macs_step, "codes": "uniform random", "grad_tables": "int16 x16 difference-based, half window 8"},
+        "images_per_s": BATCH * args.steps / dt,
+        "frac_of_lds_gather_roofline": rate / LDS_GATHER_PEAK,
+        "kernel_ms_per_step": {k: round(v, 4) for k, v in kernels.items()},
+        "roofline": {"bound": "lds", "kernel": dominant, "achieved": dom_rate / 1e9, "peak": LDS_GATHER_PEAK / 1e9,
+                     "unit": "Ggather/s", "frac": dom_rate / LDS_GATHER_PEAK, "traffic": None,
+                     "avg_launch_ms": dom_ms / launches,
+                     "hbm": {"achieved": dom_bytes / (dom_ms * 1e-3) / 1e9, "peak": HBM_PEAK / 1e9, "unit": "GB/s",
+                             "frac": dom_bytes / (dom_ms * 1e-3) / HBM_PEAK},
+                     "lds_probe_gathers_per_s": {"conflict_free": probe_free, "uniform_row_256B": probe_row}},
+        "single_gemm": {"workload": "M=4096 K=576 N=64 fwd+bwd (BASELINE.json configs[1])", "us": t_single * 1e3,
+                        "lut_mac_per_s": 3 * M1 * K1 * N1 / (t_single * 1e-3),
+                        "frac_of_lds_gather_roofline": 3 * M1 * K1 * N1 / (t_single * 1e-3) / LDS_GATHER_PEAK},
+    }
+
+    # CPU baseline: the C oracle (port of the reference formulation) on the host cores ----------------------
+    if not args.no_cpu:
+        A, B, Tc, g = O.synth_gemm(M1, K1, N1, bits=7, err=64, seed=0)
+        f16, a16, b16 = O.pack_table(Tc, 7, np.uint16), O.pack_table(Gx, 7, np.int16), O.pack_table(Gy, 7, np.int16)
+        O.forward_c(A, B, f16, 7)
+        reps, t0 = 0, time.perf_counter()
+        while time.perf_counter() - t0 < 10.0:
+            O.forward_c(A, B, f16, 7)
+            O.backward_c_f32(g, A, B, a16, b16, 7)
+            reps += 1
+        el = time.perf_counter() - t0
+        out["cpu_baseline"] = {"value": reps * 3 * M1 * K1 * N1 / el, "unit": "LUT-MAC/s", "cores": O.c_lib().oracle_num_threads(),
+                               "kind": "port", "sample": f"{reps} x (M=4096,K=576,N=64 forward+backward), C/OpenMP restatement of the reference loops"}
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()
