@@ -12,6 +12,9 @@
 namespace amr {
 hipError_t launch_fwd(const uint8_t* A, const uint8_t* B, uint32_t* C, const uint16_t* lut, const LutGeom& g, int M,
                       int K, int N, int n_cu, hipStream_t stream);
+size_t fwd_slab_workspace_bytes(const LutGeom& g, int M, int K, int N);
+hipError_t launch_fwd_slab(const uint8_t* A, const uint8_t* B, uint32_t* C, const uint16_t* lut, const LutGeom& g,
+                           int M, int K, int N, int n_cu, void* workspace, hipStream_t stream);
 size_t gradB_workspace_bytes(int M, int K, int N, int n_cu, int* splits_out);
 hipError_t launch_gradB(const float* gC, const uint8_t* A, const uint8_t* B, float* gB, const int16_t* lut,
                         const LutGeom& g, int M, int K, int N, float scale, void* workspace, int splits,
@@ -106,8 +109,14 @@ int amr_bits_from_lut_elems(int64_t lut_elems) {
     return g.bits;
 }
 
-int amr_lut_gemm_forward(const uint8_t* A, const uint8_t* B, uint32_t* C, const uint16_t* lut, int64_t lut_elems,
-                         int M, int K, int N, void* stream) {
+size_t amr_lut_gemm_forward_workspace_bytes(int64_t lut_elems, int M, int K, int N) {
+    amr::LutGeom g;
+    if (M <= 0 || K <= 0 || N <= 0 || !amr::lut_geom_from_elems(lut_elems, &g)) return 0;
+    return amr::fwd_slab_workspace_bytes(g, M, K, N);
+}
+
+int amr_lut_gemm_forward_ws(const uint8_t* A, const uint8_t* B, uint32_t* C, const uint16_t* lut, int64_t lut_elems,
+                            int M, int K, int N, void* workspace, size_t workspace_bytes, void* stream) {
     if (M < 0 || K < 0 || N < 0) return fail(AMR_EINVAL, "negative dimension M=%d K=%d N=%d", M, K, N);
     amr::LutGeom g;
     if (!amr::lut_geom_from_elems(lut_elems, &g))
@@ -120,10 +129,30 @@ int amr_lut_gemm_forward(const uint8_t* A, const uint8_t* B, uint32_t* C, const 
         hipError_t e = hipMemsetAsync(C, 0, (size_t)M * N * sizeof(uint32_t), s);
         return e == hipSuccess ? AMR_OK : hip_fail(e, "hipMemsetAsync");
     }
-    const int n_cu = current_device_cus(nullptr);
+    int dev = 0;
+    const int n_cu = current_device_cus(&dev);
     if (n_cu <= 0) return fail(AMR_EINVAL, "no HIP device available");
-    hipError_t e = amr::launch_fwd(A, B, C, lut, g, M, K, N, n_cu, s);
+    const size_t need = amr::fwd_slab_workspace_bytes(g, M, K, N);
+    hipError_t e;
+    if (need > 0) {
+        void* ws = workspace;
+        if (ws) {
+            if (workspace_bytes < need) return fail(AMR_EWORKSPACE, "workspace of %zu bytes is smaller than the %zu required", workspace_bytes, need);
+            if ((uintptr_t)ws & 255) return fail(AMR_EINVAL, "workspace must be 256-byte aligned");
+        } else {
+            ws = internal_workspace(dev, need, &e);
+            if (!ws) return hip_fail(e, "workspace hipMalloc");
+        }
+        e = amr::launch_fwd_slab(A, B, C, lut, g, M, K, N, n_cu, ws, s);
+    } else {
+        e = amr::launch_fwd(A, B, C, lut, g, M, K, N, n_cu, s);
+    }
     return e == hipSuccess ? AMR_OK : hip_fail(e, "forward launch");
+}
+
+int amr_lut_gemm_forward(const uint8_t* A, const uint8_t* B, uint32_t* C, const uint16_t* lut, int64_t lut_elems,
+                         int M, int K, int N, void* stream) {
+    return amr_lut_gemm_forward_ws(A, B, C, lut, lut_elems, M, K, N, nullptr, 0, stream);
 }
 
 size_t amr_lut_gemm_backward_workspace_bytes(int M, int K, int N) {

@@ -20,8 +20,9 @@ template <int R, int TN, int WAVES>
 __global__ __launch_bounds__(WAVES * 64) void lutgemm_fwd_kernel(
     const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, uint32_t* __restrict__ C,
     const uint32_t* __restrict__ lut32, int lut_dwords, int row_bytes, int M, int K, int N, int k_chunk,
-    int atomic_out) {
+    int atomic_out, const uint32_t* __restrict__ gate) {
     extern __shared__ __align__(16) unsigned char smem[];
+    if (gate != nullptr && *gate == 0u) return;   // queued as a fallback that turned out not to be needed
     {
         uint32_t* s32 = reinterpret_cast<uint32_t*>(smem);
         for (int i = threadIdx.x; i < lut_dwords; i += WAVES * 64) s32[i] = lut32[i];
@@ -124,7 +125,7 @@ __global__ __launch_bounds__(WAVES * 64) void lutgemm_fwd_kernel(
 
 template <int R, int TN, int WAVES>
 static hipError_t launch_fwd_t(const uint8_t* A, const uint8_t* B, uint32_t* C, const uint16_t* lut, const LutGeom& g,
-                               int M, int K, int N, int ksplit, hipStream_t stream) {
+                               int M, int K, int N, int ksplit, hipStream_t stream, const uint32_t* gate = nullptr) {
     const int lut_dwords = g.rows * g.cols / 2;  // rows*cols is even for every supported bit-width
     const size_t lds = (size_t)lut_dwords * 4;
     auto kern = lutgemm_fwd_kernel<R, TN, WAVES>;
@@ -142,7 +143,7 @@ static hipError_t launch_fwd_t(const uint8_t* A, const uint8_t* B, uint32_t* C, 
         if (e != hipSuccess) return e;
     }
     hipLaunchKernelGGL(kern, grid, dim3(WAVES * 64), lds, stream, A, B, C, reinterpret_cast<const uint32_t*>(lut),
-                       lut_dwords, g.cols * 2, M, K, N, k_chunk, zs > 1 ? 1 : 0);
+                       lut_dwords, g.cols * 2, M, K, N, k_chunk, zs > 1 ? 1 : 0, gate);
     return hipGetLastError();
 }
 
@@ -179,6 +180,15 @@ hipError_t launch_fwd(const uint8_t* A, const uint8_t* B, uint32_t* C, const uin
     AMR_FWD_CASE(16, 4)
 #undef AMR_FWD_CASE
     return hipErrorInvalidValue;
+}
+
+// Direct kernel queued behind the expanded-table kernel: it runs only when *gate != 0 (the operand
+// held a masked code) and then overwrites all of C, so it must not split K.
+hipError_t launch_fwd_gated(const uint8_t* A, const uint8_t* B, uint32_t* C, const uint16_t* lut, const LutGeom& g,
+                            int M, int K, int N, const uint32_t* gate, hipStream_t stream) {
+    if (N <= 64) return launch_fwd_t<32, 1, 4>(A, B, C, lut, g, M, K, N, 1, stream, gate);
+    if (N <= 128) return launch_fwd_t<32, 2, 4>(A, B, C, lut, g, M, K, N, 1, stream, gate);
+    return launch_fwd_t<16, 4, 4>(A, B, C, lut, g, M, K, N, 1, stream, gate);
 }
 
 }  // namespace amr

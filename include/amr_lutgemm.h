@@ -58,6 +58,19 @@ int amr_lut_gemm_forward(const uint8_t *A, const uint8_t *B, uint32_t *C, const 
                          int64_t lut_elems, int M, int K, int N, void *stream);
 
 /*
+ * Same operation with caller-provided scratch.  For large M and tables of at most 7 bits the forward
+ * pass first expands the table along B (E[k][a][n] = lut[a][B[k,n]]) into `workspace` and then adds
+ * rows of E; amr_lut_gemm_forward_workspace_bytes gives the size that needs (0 = no scratch used for
+ * this shape).  workspace must be 256-byte aligned; NULL makes the library use its own per-device
+ * buffer, grown with hipMalloc when needed (amr_lut_gemm_forward does exactly that).
+ * No counterpart in the reference, whose forward kernel needs no scratch.
+ */
+size_t amr_lut_gemm_forward_workspace_bytes(int64_t lut_elems, int M, int K, int N);
+int amr_lut_gemm_forward_ws(const uint8_t *A, const uint8_t *B, uint32_t *C, const uint16_t *lut,
+                            int64_t lut_elems, int M, int K, int N, void *workspace, size_t workspace_bytes,
+                            void *stream);
+
+/*
  * Backward (both gradients, as the reference always produces both):
  *   gA[m,k] = (1/16) * sum_{n<N} gC[m,n] * (float)lut_grad_a[A[m,k] * cols + B[k,n]]
  *   gB[k,n] = (1/16) * sum_{m<M} (float)lut_grad_b[A[m,k] * cols + B[k,n]] * gC[m,n]

@@ -25,6 +25,9 @@ def lib():
     vp, i64, i, sz = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_size_t
     L.amr_last_error.restype = ctypes.c_char_p
     L.amr_lut_gemm_forward.argtypes = [vp, vp, vp, vp, i64, i, i, i, vp]
+    L.amr_lut_gemm_forward_ws.argtypes = [vp, vp, vp, vp, i64, i, i, i, vp, sz, vp]
+    L.amr_lut_gemm_forward_workspace_bytes.argtypes = [i64, i, i, i]
+    L.amr_lut_gemm_forward_workspace_bytes.restype = sz
     L.amr_lut_gemm_backward.argtypes = [vp, vp, vp, vp, vp, vp, vp, i64, i, i, i, vp, sz, vp]
     L.amr_lut_gemm_backward_workspace_bytes.argtypes = [i, i, i]
     L.amr_lut_gemm_backward_workspace_bytes.restype = sz
@@ -83,6 +86,47 @@ def test_forward_bit_exact_random_tables(lib, oracle, bits, shape):
     _, A, B, T = rand_case(hash((bits, shape)) % 2**32, *shape, bits)
     flat = oracle.pack_table(T, bits, np.uint16)
     assert (gpu_forward(lib, A, B, flat) == oracle.forward_c(A, B, flat, bits)).all()
+
+
+# shapes with M >= 2048 and K >= 512 take the expanded-table forward path (tables of at most 7 bits)
+BIG_M_SHAPES = [(2048, 512, 64), (2081, 515, 65), (3000, 27, 10), (4096, 640, 300), (2500, 1153, 128), (5000, 777, 1)]
+
+
+@pytest.mark.parametrize("bits", [7, 6, 4, 8])
+@pytest.mark.parametrize("shape", BIG_M_SHAPES)
+def test_forward_bit_exact_large_m(lib, oracle, bits, shape):
+    print("forward large M", bits, shape, flush=True)
+    _, A, B, T = rand_case(hash((bits, shape, "L")) % 2**32, *shape, bits)
+    flat = oracle.pack_table(T, bits, np.uint16)
+    assert (gpu_forward(lib, A, B, flat) == oracle.forward_c(A, B, flat, bits)).all()
+
+
+def test_forward_large_m_small_table_values_masked_codes_and_own_workspace(lib, oracle):
+    print("forward large M masked / workspace", flush=True)
+    M, K, N = 2600, 530, 70
+    rng, A, B, _ = rand_case(99, M, K, N, 7)
+    T = oracle.synth_lut(7, 64, rng)                      # max < 16384: packed 16-bit partial sums
+    flat = oracle.pack_table(T, 7, np.uint16)
+    want = oracle.forward_c(A, B, flat, 7)
+    assert (gpu_forward(lib, A, B, flat) == want).all()
+    a, b, l = dev(A), dev(B), dev(flat)
+    need = lib.amr_lut_gemm_forward_workspace_bytes(l.numel(), M, K, N)
+    assert need > 0
+    ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+    c = torch.zeros((M, N), dtype=torch.int32, device="cuda")
+    assert lib.amr_lut_gemm_forward_ws(a.data_ptr(), b.data_ptr(), c.data_ptr(), l.data_ptr(), l.numel(), M, K, N, ws.data_ptr(), need, None) == 0
+    torch.cuda.synchronize()
+    assert (c.cpu().numpy().view(np.uint32) == want).all()
+    assert lib.amr_lut_gemm_forward_ws(a.data_ptr(), b.data_ptr(), c.data_ptr(), l.data_ptr(), l.numel(), M, K, N, ws.data_ptr(), need - 1, None) == -3
+    # masked code 2^b in both operands (zero contribution), rows spread over several workgroups
+    A2, B2 = A.copy(), B.copy()
+    A2[::7, 3] = 128
+    A2[1234, :] = 128
+    B2[5, ::3] = 128
+    want2 = oracle.forward_c(A2, B2, flat, 7)
+    assert (gpu_forward(lib, A2, B2, flat) == want2).all()
+    # and the next call without masked codes is clean again
+    assert (gpu_forward(lib, A, B, flat) == want).all()
 
 
 def test_forward_config1_bit_exact_and_exact_multiplier(lib, oracle):
