@@ -18,9 +18,15 @@ hipError_t launch_fwd_slab(const uint8_t* A, const uint8_t* B, uint32_t* C, cons
 size_t gradB_workspace_bytes(int M, int K, int N, int n_cu, int* splits_out);
 hipError_t launch_gradB(const float* gC, const uint8_t* A, const uint8_t* B, float* gB, const int16_t* lut,
                         const LutGeom& g, int M, int K, int N, float scale, void* workspace, int splits,
-                        hipStream_t stream);
+                        hipStream_t stream, const uint32_t* gate = nullptr);
 hipError_t launch_gradA(const float* gC, const uint8_t* A, const uint8_t* B, float* gA, const int16_t* lut,
-                        const LutGeom& g, int M, int K, int N, float scale, int n_cu, hipStream_t stream);
+                        const LutGeom& g, int M, int K, int N, float scale, int n_cu, hipStream_t stream,
+                        const uint32_t* gate = nullptr);
+bool bwd_slab_applies(const LutGeom& g, int M, int K, int N);
+int gradB_slab_splits(int M, int K, int N, int n_cu);
+hipError_t launch_gradB_slab(const float* gC, const uint8_t* A, const uint8_t* B, float* gB, const int16_t* lut,
+                             const LutGeom& g, int M, int K, int N, float scale, uint32_t* flags, float* partials,
+                             int splits, hipStream_t stream);
 hipError_t launch_accgemm(const float* A, const float* B, float* C, int M, int K, int N, hipStream_t stream);
 hipError_t run_lds_probe(int pattern, int waves_per_cu, int iters, int n_cu, float* ms_out, double* gathers_out,
                          hipStream_t stream);
@@ -155,11 +161,19 @@ int amr_lut_gemm_forward(const uint8_t* A, const uint8_t* B, uint32_t* C, const 
     return amr_lut_gemm_forward_ws(A, B, C, lut, lut_elems, M, K, N, nullptr, 0, stream);
 }
 
+// Scratch layout of the backward pass: [256 B of flags][partial sums of gB over the M splits].
+static size_t backward_partial_bytes(int M, int K, int N, int n_cu) {
+    size_t direct = amr::gradB_workspace_bytes(M, K, N, n_cu, nullptr);
+    const int s = amr::gradB_slab_splits(M, K, N, n_cu);
+    size_t slab = s > 1 ? (size_t)s * K * N * sizeof(float) : 0;
+    return direct > slab ? direct : slab;
+}
+
 size_t amr_lut_gemm_backward_workspace_bytes(int M, int K, int N) {
     if (M <= 0 || K <= 0 || N <= 0) return 0;
     const int n_cu = current_device_cus(nullptr);
-    // Without a device (e.g. a host-only query) size for the largest supported split count.
-    return amr::gradB_workspace_bytes(M, K, N, n_cu > 0 ? n_cu : 256, nullptr);
+    // Without a device (e.g. a host-only query) size for a 256-CU part.
+    return 256 + backward_partial_bytes(M, K, N, n_cu > 0 ? n_cu : 256);
 }
 
 int amr_lut_gemm_backward(const float* gC, const uint8_t* A, const uint8_t* B, float* gA, float* gB,
@@ -182,28 +196,40 @@ int amr_lut_gemm_backward(const float* gC, const uint8_t* A, const uint8_t* B, f
         return e == hipSuccess ? AMR_OK : hip_fail(e, "hipMemsetAsync");
     }
     if (!gC || !A || !B) return fail(AMR_EINVAL, "null pointer argument");
+    if (!gA && !gB) return AMR_OK;
     int dev = 0;
     const int n_cu = current_device_cus(&dev);
     if (n_cu <= 0) return fail(AMR_EINVAL, "no HIP device available");
     hipError_t e;
+    const size_t need = 256 + backward_partial_bytes(M, K, N, n_cu);
+    void* ws = workspace;
+    if (ws) {
+        if (workspace_bytes < need) return fail(AMR_EWORKSPACE, "workspace of %zu bytes is smaller than the %zu required", workspace_bytes, need);
+        if ((uintptr_t)ws & 255) return fail(AMR_EINVAL, "workspace must be 256-byte aligned");
+    } else {
+        ws = internal_workspace(dev, need, &e);
+        if (!ws) return hip_fail(e, "workspace hipMalloc");
+    }
+    uint32_t* flags = reinterpret_cast<uint32_t*>(ws);
+    float* partials = reinterpret_cast<float*>(reinterpret_cast<unsigned char*>(ws) + 256);
+    const bool slab = amr::bwd_slab_applies(g, M, K, N);
+    if (slab && gB) {
+        e = hipMemsetAsync(flags, 0, 256, s);
+        if (e != hipSuccess) return hip_fail(e, "hipMemsetAsync");
+    }
     if (gA) {
         e = amr::launch_gradA(gC, A, B, gA, lut_grad_a, g, M, K, N, scale, n_cu, s);
         if (e != hipSuccess) return hip_fail(e, "gradA launch");
     }
     if (gB) {
-        int splits = 1;
-        const size_t need = amr::gradB_workspace_bytes(M, K, N, n_cu, &splits);
-        void* ws = workspace;
-        if (need > 0) {
-            if (ws) {
-                if (workspace_bytes < need) return fail(AMR_EWORKSPACE, "workspace of %zu bytes is smaller than the %zu required", workspace_bytes, need);
-                if ((uintptr_t)ws & 255) return fail(AMR_EINVAL, "workspace must be 256-byte aligned");
-            } else {
-                ws = internal_workspace(dev, need, &e);
-                if (!ws) return hip_fail(e, "workspace hipMalloc");
-            }
+        if (slab) {
+            e = amr::launch_gradB_slab(gC, A, B, gB, lut_grad_b, g, M, K, N, scale, flags, partials,
+                                       amr::gradB_slab_splits(M, K, N, n_cu), s);
+        } else {
+            int splits = 1;
+            amr::gradB_workspace_bytes(M, K, N, n_cu, &splits);
+            e = amr::launch_gradB(gC, A, B, gB, lut_grad_b, g, M, K, N, scale, partials, splits, s);
         }
-        e = amr::launch_gradB(gC, A, B, gB, lut_grad_b, g, M, K, N, scale, ws, splits, s);
         if (e != hipSuccess) return hip_fail(e, "gradB launch");
     }
     return AMR_OK;

@@ -27,8 +27,9 @@ template <int KT, int WAVES>
 __global__ __launch_bounds__(WAVES * 64) void lutgemm_gradB_kernel(
     const float* __restrict__ gC, const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
     float* __restrict__ out, const uint32_t* __restrict__ lut32, int lut_dwords, int row_bytes, int M, int K, int N,
-    int m_chunk, float scale) {
+    int m_chunk, float scale, const uint32_t* __restrict__ gate) {
     extern __shared__ __align__(16) unsigned char smem[];
+    if (gate != nullptr && *gate == 0u) return;   // queued as a fallback that turned out not to be needed
     {
         uint32_t* s32 = reinterpret_cast<uint32_t*>(smem);
         for (int i = threadIdx.x; i < lut_dwords; i += WAVES * 64) s32[i] = lut32[i];
@@ -103,8 +104,10 @@ __global__ void reduce_partials_kernel(const float* __restrict__ partial, float*
 template <int KT, int RM, int WAVES>
 __global__ __launch_bounds__(WAVES * 64) void lutgemm_gradA_kernel(
     const float* __restrict__ gC, const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
-    float* __restrict__ gA, const uint16_t* __restrict__ lut, int rows, int cols, int M, int K, int N, float scale) {
+    float* __restrict__ gA, const uint16_t* __restrict__ lut, int rows, int cols, int M, int K, int N, float scale,
+    const uint32_t* __restrict__ gate) {
     extern __shared__ __align__(16) unsigned char smem[];
+    if (gate != nullptr && *gate == 0u) return;   // queued as a fallback that turned out not to be needed
     // Transposed staging: entry (a,b) of the row-major table goes to T[b][a], T row stride = cols
     // entries (cols is even, so T rows stay dword aligned).  T needs cols rows of `rows` entries.
     {
@@ -203,7 +206,7 @@ size_t gradB_workspace_bytes(int M, int K, int N, int n_cu, int* splits_out) {
 
 hipError_t launch_gradB(const float* gC, const uint8_t* A, const uint8_t* B, float* gB, const int16_t* lut,
                         const LutGeom& g, int M, int K, int N, float scale, void* workspace, int splits,
-                        hipStream_t stream) {
+                        hipStream_t stream, const uint32_t* gate = nullptr) {
     constexpr int KT = 16;
     const int lut_dwords = g.rows * g.cols / 2;
     const size_t lds = (size_t)lut_dwords * 4;
@@ -220,14 +223,14 @@ hipError_t launch_gradB(const float* gC, const uint8_t* A, const uint8_t* B, flo
         if (!done) { e = set_lds_attr(reinterpret_cast<const void*>(kern)); if (e != hipSuccess) return e; done = true; }
         dim3 grid((N + 63) / 64, (ktiles + 15) / 16, zs);
         hipLaunchKernelGGL(kern, grid, dim3(1024), lds, stream, gC, A, B, out, reinterpret_cast<const uint32_t*>(lut),
-                           lut_dwords, g.cols * 2, M, K, N, m_chunk, scale);
+                           lut_dwords, g.cols * 2, M, K, N, m_chunk, scale, gate);
     } else {
         auto kern = lutgemm_gradB_kernel<KT, 4>;
         static bool done = false;
         if (!done) { e = set_lds_attr(reinterpret_cast<const void*>(kern)); if (e != hipSuccess) return e; done = true; }
         dim3 grid((N + 63) / 64, (ktiles + 3) / 4, zs);
         hipLaunchKernelGGL(kern, grid, dim3(256), lds, stream, gC, A, B, out, reinterpret_cast<const uint32_t*>(lut),
-                           lut_dwords, g.cols * 2, M, K, N, m_chunk, scale);
+                           lut_dwords, g.cols * 2, M, K, N, m_chunk, scale, gate);
     }
     e = hipGetLastError();
     if (e != hipSuccess) return e;
@@ -241,7 +244,8 @@ hipError_t launch_gradB(const float* gC, const uint8_t* A, const uint8_t* B, flo
 }
 
 hipError_t launch_gradA(const float* gC, const uint8_t* A, const uint8_t* B, float* gA, const int16_t* lut,
-                        const LutGeom& g, int M, int K, int N, float scale, int n_cu, hipStream_t stream) {
+                        const LutGeom& g, int M, int K, int N, float scale, int n_cu, hipStream_t stream,
+                        const uint32_t* gate = nullptr) {
     constexpr int KT = 16;
     const size_t lds = (size_t)g.cols * g.cols * 2;
     const bool big = g.bits == 8;
@@ -253,7 +257,7 @@ hipError_t launch_gradA(const float* gC, const uint8_t* A, const uint8_t* B, flo
         if (!done) { e = set_lds_attr(reinterpret_cast<const void*>(kern)); if (e != hipSuccess) return e; done = true; }
         dim3 grid(ktiles, (M + 1023) / 1024);
         hipLaunchKernelGGL(kern, grid, dim3(1024), lds, stream, gC, A, B, gA, reinterpret_cast<const uint16_t*>(lut), g.rows,
-                           g.cols, M, K, N, scale);
+                           g.cols, M, K, N, scale, gate);
     } else {
         // Two rows per lane amortise the scalar work per gather; fall back to one when that would
         // leave CUs idle.
@@ -264,17 +268,24 @@ hipError_t launch_gradA(const float* gC, const uint8_t* A, const uint8_t* B, flo
             if (!done) { e = set_lds_attr(reinterpret_cast<const void*>(kern)); if (e != hipSuccess) return e; done = true; }
             dim3 grid(ktiles, (M + 511) / 512);
             hipLaunchKernelGGL(kern, grid, dim3(256), lds, stream, gC, A, B, gA, reinterpret_cast<const uint16_t*>(lut),
-                               g.rows, g.cols, M, K, N, scale);
+                               g.rows, g.cols, M, K, N, scale, gate);
         } else {
             auto kern = lutgemm_gradA_kernel<KT, 1, 4>;
             static bool done = false;
             if (!done) { e = set_lds_attr(reinterpret_cast<const void*>(kern)); if (e != hipSuccess) return e; done = true; }
             dim3 grid(ktiles, (M + 255) / 256);
             hipLaunchKernelGGL(kern, grid, dim3(256), lds, stream, gC, A, B, gA, reinterpret_cast<const uint16_t*>(lut),
-                               g.rows, g.cols, M, K, N, scale);
+                               g.rows, g.cols, M, K, N, scale, gate);
         }
     }
     return hipGetLastError();
+}
+
+// Direct kernel queued behind the expanded-table kernel; it runs only when *gate != 0 (an operand
+// held a masked code) and then overwrites the whole result (no M split: no scratch).
+hipError_t launch_gradB_gated(const float* gC, const uint8_t* A, const uint8_t* B, float* gB, const int16_t* lut,
+                              const LutGeom& g, int M, int K, int N, float scale, const uint32_t* gate, hipStream_t stream) {
+    return launch_gradB(gC, A, B, gB, lut, g, M, K, N, scale, nullptr, 1, stream, gate);
 }
 
 }  // namespace amr

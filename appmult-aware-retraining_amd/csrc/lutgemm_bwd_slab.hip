@@ -1,0 +1,226 @@
+// Backward LUT-GEMM, gradient of B, for large M on gfx950: "expanded-table" kernel (7-bit tables and
+// narrower).
+//
+// Same result (to fp32 summation order) as lutgemm_gradB_kernel and as the reference's
+// ApproxGemmBackwardKernelForGB (self_ops/src/approx_gemm_backward.cu:269-492).
+//
+// A workgroup owns KT values of k and one 64-column tile of B.  It first expands the gradient table
+// along its B codes into LDS as fp32,
+//       S[kk][a][c] = (float) G[a][ B[k0+kk, n0+c] ]          (a = every operand code, 256 B per row)
+// and then streams rows m of A / gC.  For one (m, k) everything a lane needs sits in ROW a = A[m,k]
+// of S, next to each other, so it is fetched with 128-bit LDS reads instead of one gather per
+// multiply-add:
+//   lane = (row slot l/16, column group l%16 of 4 columns); acc[kk][c] += gC[m,c] * S[kk][a][c];
+//   partial sums of the 4 row slots, 16 waves and M splits are added at the end.
+// Every wave-level 128-bit read touches all 64 banks exactly four times, i.e. it is conflict-free.
+// The LDS address (slab<<16 | a<<8 | lane part) is assembled from the code byte by one v_perm_b32,
+// which needs a < 128: a masked code (128 in a 7-bit operand) raises flags[1] and the direct kernel,
+// queued behind this one and gated on that flag, recomputes the result.
+// (The gradient of A has no such formulation that pays off: its reduction runs over n, so the rows of
+// gC would have to be re-read once per k tile; it stays with the direct gather kernel.)
+#include "amr_common.h"
+
+namespace amr {
+
+constexpr int kBwdSlabRows = 128;
+constexpr int kBwdSlabBytes = kBwdSlabRows * 256;   // one k: 128 codes x 64 columns x fp32 = 32 KB
+constexpr int kBwdKT = 4;                            // k per workgroup (128 KB of LDS)
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+// S[kk][a][c] for kk < KT, built by all 1024 threads straight from the table in global memory (it is
+// 33 KB and stays in the L2; the expansion is 2^b / M of the streaming work).
+__device__ __forceinline__ void build_bwd_slab(float* slab, const int16_t* __restrict__ G, int lut_cols, int n_codes,
+                                               const uint8_t* __restrict__ B, int K, int N, int k0, int n0, int kt) {
+    const int col = threadIdx.x & 63;
+    const int a0 = threadIdx.x >> 6;
+    for (int kk = 0; kk < kt; ++kk) {
+        const bool live = (k0 + kk < K) && (n0 + col < N);
+        const int b = live ? (int)B[(size_t)(k0 + kk) * N + n0 + col] : 0;
+        float* s = slab + kk * (kBwdSlabBytes / 4);
+        for (int a = a0; a < kBwdSlabRows; a += 16) {
+            float v = 0.f;
+            if (live && a < n_codes) v = (float)G[a * lut_cols + b];
+            s[a * 64 + col] = v;
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------ gradB
+// grid (n_tiles, ceil(K/KT), m_splits), 1024 threads.  out: gB itself (m_splits == 1) or the partial
+// buffer [split][K][N].
+// FAST: K % 4 == 0, N % 64 == 0 and gC 16-byte aligned, so every operand load is an unconditional
+// dword / 128-bit load (no tail handling in the streaming loop).
+template <bool FAST>
+__global__ __launch_bounds__(1024) void lutgemm_gradB_slab_kernel(
+    const float* __restrict__ gC, const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, float* __restrict__ out,
+    const int16_t* __restrict__ G, int lut_cols, int n_codes, uint32_t* __restrict__ flags, int M, int K, int N,
+    int m_chunk, float scale, int vec_ok) {
+    __shared__ __align__(16) unsigned char smem[kBwdKT * kBwdSlabBytes];
+    float* slab = reinterpret_cast<float*>(smem);
+    const int tid = threadIdx.x;
+    const int wave = uniform(tid >> 6);
+    const int lane = tid & 63;
+    const int rs = lane >> 4, cg = lane & 15;
+    const int n0 = blockIdx.x * 64;
+    const int k0 = blockIdx.y * kBwdKT;
+    const int mb = blockIdx.z * m_chunk;
+    const int me = min(M, mb + m_chunk);
+
+    build_bwd_slab(slab, G, lut_cols, n_codes, B, K, N, k0, n0, kBwdKT);
+    __syncthreads();
+
+    // address pieces: byte0 = 16*cg, byte1 = code (v_perm), byte2 = slab pair (kk>>1), +32768 for odd kk
+    const uint32_t base_lo = (uint32_t)(cg << 4), base_hi = base_lo | 0x10000u;
+    const bool k_full = FAST || (k0 + 4 <= K);
+    const bool cols_vec = FAST || (vec_ok && (n0 + 64 <= N));
+    const int ncol = n0 + 4 * cg;
+
+    float acc[kBwdKT][4];
+#pragma unroll
+    for (int kk = 0; kk < kBwdKT; ++kk)
+#pragma unroll
+        for (int c = 0; c < 4; ++c) acc[kk][c] = 0.f;
+    uint32_t seen = 0;
+
+    constexpr int RU = 2;   // row groups per wave and iteration; the next iteration's operands are prefetched
+
+    auto load_rows = [&](int g0, uint32_t (&a4)[RU], f32x4 (&gv)[RU]) {
+#pragma unroll
+        for (int u = 0; u < RU; ++u) {
+            const int m = mb + 4 * (g0 + u) + rs;
+            const bool valid = m < me;
+            const int mc = valid ? m : me - 1;
+            const uint8_t* arow = A + (size_t)mc * K;
+            uint32_t a;
+            if (FAST) a = load_u32_unaligned(arow + k0);
+            else a = k_full ? load_u32_unaligned(arow + k0) : load_codes4_clamped(arow, k0, K);
+            a4[u] = valid ? a : 0u;
+            const float* grow = gC + (size_t)mc * N;
+            f32x4 v;
+            if (FAST || cols_vec) {
+                v = *reinterpret_cast<const f32x4*>(grow + ncol);
+            } else {
+                v.x = (ncol + 0 < N) ? grow[ncol + 0] : 0.f;
+                v.y = (ncol + 1 < N) ? grow[ncol + 1] : 0.f;
+                v.z = (ncol + 2 < N) ? grow[ncol + 2] : 0.f;
+                v.w = (ncol + 3 < N) ? grow[ncol + 3] : 0.f;
+            }
+            const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
+            gv[u] = valid ? v : zero;
+        }
+    };
+
+    uint32_t a4[RU], a4n[RU];
+    f32x4 gv[RU], gvn[RU];
+    int g0 = wave * RU;
+    if (mb + 4 * g0 < me) load_rows(g0, a4, gv);
+    for (; mb + 4 * g0 < me; g0 += 16 * RU) {
+        const bool more = mb + 4 * (g0 + 16 * RU) < me;
+        if (more) load_rows(g0 + 16 * RU, a4n, gvn);
+#pragma unroll
+        for (int u = 0; u < RU; ++u) {
+            seen |= a4[u];
+            f32x4 s[kBwdKT];
+#pragma unroll
+            for (int kk = 0; kk < kBwdKT; ++kk) {
+                const uint32_t addr = __builtin_amdgcn_perm(a4[u], (kk & 2) ? base_hi : base_lo, 0x0c020400u + ((uint32_t)kk << 8));
+                s[kk] = *reinterpret_cast<const f32x4*>(smem + addr + (kk & 1) * kBwdSlabBytes);
+            }
+#pragma unroll
+            for (int kk = 0; kk < kBwdKT; ++kk) {
+                acc[kk][0] = __builtin_fmaf(gv[u].x, s[kk].x, acc[kk][0]);
+                acc[kk][1] = __builtin_fmaf(gv[u].y, s[kk].y, acc[kk][1]);
+                acc[kk][2] = __builtin_fmaf(gv[u].z, s[kk].z, acc[kk][2]);
+                acc[kk][3] = __builtin_fmaf(gv[u].w, s[kk].w, acc[kk][3]);
+            }
+        }
+        if (more) {
+#pragma unroll
+            for (int u = 0; u < RU; ++u) {
+                a4[u] = a4n[u];
+                gv[u] = gvn[u];
+            }
+        }
+    }
+    if (__builtin_amdgcn_ballot_w64((seen & 0x80808080u) != 0) != 0) {
+        if (lane == 0) atomicOr(&flags[1], 1u);
+    }
+
+    // sum the four row slots of the wave, then the 16 waves through LDS (the slabs are no longer needed)
+#pragma unroll
+    for (int kk = 0; kk < kBwdKT; ++kk)
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            float v = acc[kk][c];
+            v += __shfl_xor(v, 16);
+            v += __shfl_xor(v, 32);
+            acc[kk][c] = v;
+        }
+    __syncthreads();
+    float* red = reinterpret_cast<float*>(smem);   // [wave][kk][64]
+    if (rs == 0) {
+#pragma unroll
+        for (int kk = 0; kk < kBwdKT; ++kk)
+#pragma unroll
+            for (int c = 0; c < 4; ++c) red[(wave * kBwdKT + kk) * 64 + 4 * cg + c] = acc[kk][c];
+    }
+    __syncthreads();
+    if (tid < kBwdKT * 64) {
+        const int kk = tid >> 6, col = tid & 63;
+        float v = 0.f;
+#pragma unroll
+        for (int w = 0; w < 16; ++w) v += red[(w * kBwdKT + kk) * 64 + col];
+        if (k0 + kk < K && n0 + col < N) out[((size_t)blockIdx.z * K + k0 + kk) * N + n0 + col] = v * scale;
+    }
+}
+
+// ------------------------------------------------------------------------------------------ host
+hipError_t launch_gradB_gated(const float* gC, const uint8_t* A, const uint8_t* B, float* gB, const int16_t* lut,
+                              const LutGeom& g, int M, int K, int N, float scale, const uint32_t* gate, hipStream_t stream);
+__global__ void reduce_partials_kernel(const float* __restrict__ partial, float* __restrict__ out, size_t count, int splits);
+
+bool bwd_slab_applies(const LutGeom& g, int M, int K, int N) {
+    (void)N;
+    return g.bits <= 7 && M >= 4096 && K >= 4;
+}
+
+// M splits of the expanded-table gradB: enough workgroups to fill the device, at least 2048 rows each.
+int gradB_slab_splits(int M, int K, int N, int n_cu) {
+    const long per_split = (long)((N + 63) / 64) * ((K + kBwdKT - 1) / kBwdKT);
+    long splits = (2L * n_cu + per_split - 1) / per_split;
+    const long max_rows = M / 2048 > 0 ? M / 2048 : 1;
+    if (splits > max_rows) splits = max_rows;
+    if (splits > 64) splits = 64;
+    return splits < 1 ? 1 : (int)splits;
+}
+
+hipError_t launch_gradB_slab(const float* gC, const uint8_t* A, const uint8_t* B, float* gB, const int16_t* lut,
+                             const LutGeom& g, int M, int K, int N, float scale, uint32_t* flags, float* partials,
+                             int splits, hipStream_t stream) {
+    int m_chunk = (M + splits - 1) / splits;
+    m_chunk = (m_chunk + 255) & ~255;
+    const int zs = (M + m_chunk - 1) / m_chunk;
+    float* out = zs > 1 ? partials : gB;
+    const int vec_ok = ((N & 3) == 0) && (((uintptr_t)gC & 15) == 0);
+    dim3 grid((N + 63) / 64, (K + kBwdKT - 1) / kBwdKT, zs);
+    if (vec_ok && (K & 3) == 0 && (N & 63) == 0)
+        hipLaunchKernelGGL(lutgemm_gradB_slab_kernel<true>, grid, dim3(1024), 0, stream, gC, A, B, out, lut, g.cols, 1 << g.bits,
+                           flags, M, K, N, m_chunk, scale, vec_ok);
+    else
+        hipLaunchKernelGGL(lutgemm_gradB_slab_kernel<false>, grid, dim3(1024), 0, stream, gC, A, B, out, lut, g.cols, 1 << g.bits,
+                           flags, M, K, N, m_chunk, scale, vec_ok);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    if (zs > 1) {
+        const size_t count = (size_t)K * N;
+        hipLaunchKernelGGL(reduce_partials_kernel, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, stream, partials, gB,
+                           count, zs);
+        e = hipGetLastError();
+        if (e != hipSuccess) return e;
+    }
+    if (g.bits == 7) return launch_gradB_gated(gC, A, B, gB, lut, g, M, K, N, scale, flags + 1, stream);
+    return hipSuccess;
+}
+
+}  // namespace amr

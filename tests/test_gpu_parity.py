@@ -206,6 +206,37 @@ def test_backward_within_tolerance_random_tables(lib, oracle, bits, shape):
     check_backward(oracle, gpu_backward(lib, g, A, B, la, lb), g, A, B, la, lb, bits)
 
 
+# M >= 4096 takes the expanded-table backward kernels (tables of at most 7 bits); N > 256 needs two passes of gradA
+BWD_BIG_M_SHAPES = [(4096, 8, 64), (4100, 27, 10), (5000, 130, 65), (4096, 64, 300), (4500, 70, 129), (4096, 33, 513), (9000, 5, 200)]
+
+
+@pytest.mark.parametrize("bits", [7, 6, 8])
+@pytest.mark.parametrize("shape", BWD_BIG_M_SHAPES)
+def test_backward_within_tolerance_large_m(lib, oracle, bits, shape):
+    print("backward large M", bits, shape, flush=True)
+    rng, A, B, _ = rand_case(hash((bits, shape, "bL")) % 2**32, *shape, bits)
+    n = 1 << bits
+    la = oracle.pack_table(rng.integers(-32768, 32768, (n, n)), bits, np.int16)
+    lb = oracle.pack_table(rng.integers(-32768, 32768, (n, n)), bits, np.int16)
+    g = rng.standard_normal((shape[0], shape[2])).astype(np.float32)
+    check_backward(oracle, gpu_backward(lib, g, A, B, la, lb), g, A, B, la, lb, bits)
+
+
+def test_backward_large_m_masked_codes(lib, oracle):
+    print("backward large M masked", flush=True)
+    M, K, N = 4300, 40, 70
+    rng, A, B, _ = rand_case(123, M, K, N, 7)
+    la = oracle.pack_table(rng.integers(-3000, 3000, (128, 128)), 7, np.int16)
+    lb = oracle.pack_table(rng.integers(-3000, 3000, (128, 128)), 7, np.int16)
+    g = rng.standard_normal((M, N)).astype(np.float32)
+    A2, B2 = A.copy(), B.copy()
+    A2[::5, 7] = 128
+    A2[4000, :] = 128
+    B2[3, ::2] = 128
+    check_backward(oracle, gpu_backward(lib, g, A2, B2, la, lb), g, A2, B2, la, lb, 7)
+    check_backward(oracle, gpu_backward(lib, g, A, B, la, lb), g, A, B, la, lb, 7)
+
+
 def test_backward_config2_difference_tables_and_ste(lib, oracle):
     print("backward config2", flush=True)
     A, B, T, g = oracle.synth_gemm(4096, 576, 64, bits=7, err=64, seed=0)
