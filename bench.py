@@ -48,6 +48,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--layers", action="store_true", help="also print a per-layer table to stderr")
+    ap.add_argument("--calib", action="store_true", help="also run three plain 256 MiB device copies (reference for scaling FETCH_SIZE/WRITE_SIZE counters)")
     ap.add_argument("--only", default="", help="comma-separated layer names: restrict the step to them (profiling aid; the JSON line then describes that subset)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -128,6 +129,14 @@ def main():
     rows = slice(100, 164)
     want = O.forward_c(b["A"][rows].cpu().numpy(), b["B"].cpu().numpy(), lut.cpu().numpy(), 7)
     assert (b["C"][rows].cpu().numpy().view(np.uint32) == want).all(), "forward parity guard failed"
+
+    if args.calib:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).random_(0, 255)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     # timed region ------------------------------------------------------------------------------------
     for _ in range(args.warmup):
