@@ -101,7 +101,10 @@ __global__ void reduce_partials_kernel(const float* __restrict__ partial, float*
 }
 
 // ------------------------------------------------------------------------------------------ gradA
-template <int KT, int RM, int WAVES>
+// VEC: N % 4 == 0, K % 4 == 0 and gC / gA 16-byte aligned, so the per-lane rows of gC are read and the
+// per-lane rows of gA are written 16 bytes at a time (a lane owns a row, so every scalar access would
+// touch 64 different cache lines per instruction).
+template <int KT, int RM, int WAVES, bool VEC>
 __global__ __launch_bounds__(WAVES * 64) void lutgemm_gradA_kernel(
     const float* __restrict__ gC, const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
     float* __restrict__ gA, const uint16_t* __restrict__ lut, int rows, int cols, int M, int K, int N, float scale,
@@ -152,9 +155,16 @@ __global__ __launch_bounds__(WAVES * 64) void lutgemm_gradA_kernel(
         const uint32_t b4 = load_codes4_clamped(brow, n, N);
         float g[RM][4];
 #pragma unroll
-        for (int r = 0; r < RM; ++r)
+        for (int r = 0; r < RM; ++r) {
+            if (VEC) {
+                typedef float f32x4 __attribute__((ext_vector_type(4)));
+                const f32x4 v = *reinterpret_cast<const f32x4*>(gC + (size_t)mr[r] * N + n);
+                g[r][0] = v.x; g[r][1] = v.y; g[r][2] = v.z; g[r][3] = v.w;
+            } else {
 #pragma unroll
-            for (int j = 0; j < 4; ++j) g[r][j] = (n + j < N) ? gC[(size_t)mr[r] * N + n + j] : 0.f;
+                for (int j = 0; j < 4; ++j) g[r][j] = (n + j < N) ? gC[(size_t)mr[r] * N + n + j] : 0.f;
+            }
+        }
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             float t[RM][KT];
@@ -178,9 +188,20 @@ __global__ __launch_bounds__(WAVES * 64) void lutgemm_gradA_kernel(
     for (int r = 0; r < RM; ++r) {
         const int m = m0 + lane + 64 * r;
         if (m < M) {
+            if (VEC) {
+                typedef float f32x4 __attribute__((ext_vector_type(4)));
 #pragma unroll
-            for (int kk = 0; kk < KT; ++kk)
-                if (k0 + kk < K) gA[(size_t)m * K + k0 + kk] = acc[r][kk] * scale;
+                for (int d = 0; d < KT / 4; ++d) {
+                    if (k0 + 4 * d < K) {   // K % 4 == 0: the whole group is inside the row
+                        f32x4 v = {acc[r][4 * d] * scale, acc[r][4 * d + 1] * scale, acc[r][4 * d + 2] * scale, acc[r][4 * d + 3] * scale};
+                        *reinterpret_cast<f32x4*>(gA + (size_t)m * K + k0 + 4 * d) = v;
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int kk = 0; kk < KT; ++kk)
+                    if (k0 + kk < K) gA[(size_t)m * K + k0 + kk] = acc[r][kk] * scale;
+            }
         }
     }
 }
@@ -243,42 +264,41 @@ hipError_t launch_gradB(const float* gC, const uint8_t* A, const uint8_t* B, flo
     return e;
 }
 
+template <int KT, int RM, int WAVES, bool VEC>
+static hipError_t launch_gradA_t(const float* gC, const uint8_t* A, const uint8_t* B, float* gA, const int16_t* lut,
+                                 const LutGeom& g, int M, int K, int N, float scale, hipStream_t stream, const uint32_t* gate) {
+    auto kern = lutgemm_gradA_kernel<KT, RM, WAVES, VEC>;
+    static bool done = false;
+    if (!done) {
+        hipError_t e = set_lds_attr(reinterpret_cast<const void*>(kern));
+        if (e != hipSuccess) return e;
+        done = true;
+    }
+    const int rows_per_wg = 64 * RM * WAVES;
+    dim3 grid((K + KT - 1) / KT, (M + rows_per_wg - 1) / rows_per_wg);
+    hipLaunchKernelGGL(kern, grid, dim3(WAVES * 64), (size_t)g.cols * g.cols * 2, stream, gC, A, B, gA,
+                       reinterpret_cast<const uint16_t*>(lut), g.rows, g.cols, M, K, N, scale, gate);
+    return hipGetLastError();
+}
+
 hipError_t launch_gradA(const float* gC, const uint8_t* A, const uint8_t* B, float* gA, const int16_t* lut,
                         const LutGeom& g, int M, int K, int N, float scale, int n_cu, hipStream_t stream,
                         const uint32_t* gate = nullptr) {
     constexpr int KT = 16;
-    const size_t lds = (size_t)g.cols * g.cols * 2;
-    const bool big = g.bits == 8;
-    hipError_t e;
+    const bool vec = ((N & 3) == 0) && ((K & 3) == 0) && (((uintptr_t)gC & 15) == 0) && (((uintptr_t)gA & 15) == 0);
     const int ktiles = (K + KT - 1) / KT;
-    if (big) {
-        auto kern = lutgemm_gradA_kernel<KT, 1, 16>;
-        static bool done = false;
-        if (!done) { e = set_lds_attr(reinterpret_cast<const void*>(kern)); if (e != hipSuccess) return e; done = true; }
-        dim3 grid(ktiles, (M + 1023) / 1024);
-        hipLaunchKernelGGL(kern, grid, dim3(1024), lds, stream, gC, A, B, gA, reinterpret_cast<const uint16_t*>(lut), g.rows,
-                           g.cols, M, K, N, scale, gate);
-    } else {
-        // Two rows per lane amortise the scalar work per gather; fall back to one when that would
-        // leave CUs idle.
-        const long wg2 = (long)ktiles * ((M + 511) / 512);
-        if (wg2 >= 2L * n_cu) {
-            auto kern = lutgemm_gradA_kernel<KT, 2, 4>;
-            static bool done = false;
-            if (!done) { e = set_lds_attr(reinterpret_cast<const void*>(kern)); if (e != hipSuccess) return e; done = true; }
-            dim3 grid(ktiles, (M + 511) / 512);
-            hipLaunchKernelGGL(kern, grid, dim3(256), lds, stream, gC, A, B, gA, reinterpret_cast<const uint16_t*>(lut),
-                               g.rows, g.cols, M, K, N, scale, gate);
-        } else {
-            auto kern = lutgemm_gradA_kernel<KT, 1, 4>;
-            static bool done = false;
-            if (!done) { e = set_lds_attr(reinterpret_cast<const void*>(kern)); if (e != hipSuccess) return e; done = true; }
-            dim3 grid(ktiles, (M + 255) / 256);
-            hipLaunchKernelGGL(kern, grid, dim3(256), lds, stream, gC, A, B, gA, reinterpret_cast<const uint16_t*>(lut),
-                               g.rows, g.cols, M, K, N, scale, gate);
-        }
+    if (g.bits == 8) {
+        return vec ? launch_gradA_t<KT, 1, 16, true>(gC, A, B, gA, lut, g, M, K, N, scale, stream, gate)
+                   : launch_gradA_t<KT, 1, 16, false>(gC, A, B, gA, lut, g, M, K, N, scale, stream, gate);
     }
-    return hipGetLastError();
+    // Two rows per lane amortise the scalar work per gather; fall back to one when that would leave CUs idle.
+    const long wg2 = (long)ktiles * ((M + 511) / 512);
+    if (wg2 >= 2L * n_cu) {
+        return vec ? launch_gradA_t<KT, 2, 4, true>(gC, A, B, gA, lut, g, M, K, N, scale, stream, gate)
+                   : launch_gradA_t<KT, 2, 4, false>(gC, A, B, gA, lut, g, M, K, N, scale, stream, gate);
+    }
+    return vec ? launch_gradA_t<KT, 1, 4, true>(gC, A, B, gA, lut, g, M, K, N, scale, stream, gate)
+               : launch_gradA_t<KT, 1, 4, false>(gC, A, B, gA, lut, g, M, K, N, scale, stream, gate);
 }
 
 // Direct kernel queued behind the expanded-table kernel; it runs only when *gate != 0 (an operand
