@@ -49,8 +49,9 @@ __device__ __forceinline__ void build_bwd_slab(float* slab, const int16_t* __res
 // ------------------------------------------------------------------------------------------ gradB
 // grid (n_tiles, ceil(K/KT), m_splits), 1024 threads.  out: gB itself (m_splits == 1) or the partial
 // buffer [split][K][N].
-// FAST: K % 4 == 0, N % 64 == 0 and gC 16-byte aligned, so every operand load is an unconditional
-// dword / 128-bit load (no tail handling in the streaming loop).
+// FAST: K % 4 == 0, N % 64 == 0, M % 128 == 0, gC 16-byte aligned and M*K, 4*M*N < 2^31, so every
+// operand load is an unconditional dword / 128-bit load at a 32-bit offset (no tail handling in the
+// streaming loop).
 template <bool FAST>
 __global__ __launch_bounds__(1024) void lutgemm_gradB_slab_kernel(
     const float* __restrict__ gC, const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, float* __restrict__ out,
@@ -72,8 +73,8 @@ __global__ __launch_bounds__(1024) void lutgemm_gradB_slab_kernel(
 
     // address pieces: byte0 = 16*cg, byte1 = code (v_perm), byte2 = slab pair (kk>>1), +32768 for odd kk
     const uint32_t base_lo = (uint32_t)(cg << 4), base_hi = base_lo | 0x10000u;
-    const bool k_full = FAST || (k0 + 4 <= K);
-    const bool cols_vec = FAST || (vec_ok && (n0 + 64 <= N));
+    const bool k_full = (k0 + 4 <= K);
+    const bool cols_vec = vec_ok && (n0 + 64 <= N);
     const int ncol = n0 + 4 * cg;
 
     float acc[kBwdKT][4];
@@ -83,63 +84,85 @@ __global__ __launch_bounds__(1024) void lutgemm_gradB_slab_kernel(
         for (int c = 0; c < 4; ++c) acc[kk][c] = 0.f;
     uint32_t seen = 0;
 
-    constexpr int RU = 2;   // row groups per wave and iteration; the next iteration's operands are prefetched
+    constexpr int RU = 2;   // row groups (of 4 rows) per wave and iteration
 
-    auto load_rows = [&](int g0, uint32_t (&a4)[RU], f32x4 (&gv)[RU]) {
+    // one row group: four 128-bit slab reads (one per k) and 16 multiply-adds
+    auto consume = [&](uint32_t a, const f32x4& gvec) {
+        seen |= a;
+        f32x4 s[kBwdKT];
 #pragma unroll
-        for (int u = 0; u < RU; ++u) {
-            const int m = mb + 4 * (g0 + u) + rs;
-            const bool valid = m < me;
-            const int mc = valid ? m : me - 1;
-            const uint8_t* arow = A + (size_t)mc * K;
-            uint32_t a;
-            if (FAST) a = load_u32_unaligned(arow + k0);
-            else a = k_full ? load_u32_unaligned(arow + k0) : load_codes4_clamped(arow, k0, K);
-            a4[u] = valid ? a : 0u;
-            const float* grow = gC + (size_t)mc * N;
-            f32x4 v;
-            if (FAST || cols_vec) {
-                v = *reinterpret_cast<const f32x4*>(grow + ncol);
-            } else {
-                v.x = (ncol + 0 < N) ? grow[ncol + 0] : 0.f;
-                v.y = (ncol + 1 < N) ? grow[ncol + 1] : 0.f;
-                v.z = (ncol + 2 < N) ? grow[ncol + 2] : 0.f;
-                v.w = (ncol + 3 < N) ? grow[ncol + 3] : 0.f;
-            }
-            const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
-            gv[u] = valid ? v : zero;
+        for (int kk = 0; kk < kBwdKT; ++kk) {
+            const uint32_t addr = __builtin_amdgcn_perm(a, (kk & 2) ? base_hi : base_lo, 0x0c020400u + ((uint32_t)kk << 8));
+            s[kk] = *reinterpret_cast<const f32x4*>(smem + addr + (kk & 1) * kBwdSlabBytes);
+        }
+#pragma unroll
+        for (int kk = 0; kk < kBwdKT; ++kk) {
+            acc[kk][0] = __builtin_fmaf(gvec.x, s[kk].x, acc[kk][0]);
+            acc[kk][1] = __builtin_fmaf(gvec.y, s[kk].y, acc[kk][1]);
+            acc[kk][2] = __builtin_fmaf(gvec.z, s[kk].z, acc[kk][2]);
+            acc[kk][3] = __builtin_fmaf(gvec.w, s[kk].w, acc[kk][3]);
         }
     };
 
-    uint32_t a4[RU], a4n[RU];
-    f32x4 gv[RU], gvn[RU];
-    int g0 = wave * RU;
-    if (mb + 4 * g0 < me) load_rows(g0, a4, gv);
-    for (; mb + 4 * g0 < me; g0 += 16 * RU) {
-        const bool more = mb + 4 * (g0 + 16 * RU) < me;
-        if (more) load_rows(g0 + 16 * RU, a4n, gvn);
+    if (FAST) {
+        // Every row of the chunk exists (M % 128 == 0) and offsets fit 32 bits: the operands of a row
+        // group are one unaligned dword of codes and one 16-byte piece of gC at per-lane 32-bit offsets
+        // that advance by a wave-uniform stride.  Two register sets alternate (no copies); the loads of
+        // the next iteration are in flight while the current one is consumed.
+        const int iters = (me - mb) / (16 * RU * 4);
+        uint32_t aoff[RU], goff[RU];
 #pragma unroll
         for (int u = 0; u < RU; ++u) {
-            seen |= a4[u];
-            f32x4 s[kBwdKT];
-#pragma unroll
-            for (int kk = 0; kk < kBwdKT; ++kk) {
-                const uint32_t addr = __builtin_amdgcn_perm(a4[u], (kk & 2) ? base_hi : base_lo, 0x0c020400u + ((uint32_t)kk << 8));
-                s[kk] = *reinterpret_cast<const f32x4*>(smem + addr + (kk & 1) * kBwdSlabBytes);
-            }
-#pragma unroll
-            for (int kk = 0; kk < kBwdKT; ++kk) {
-                acc[kk][0] = __builtin_fmaf(gv[u].x, s[kk].x, acc[kk][0]);
-                acc[kk][1] = __builtin_fmaf(gv[u].y, s[kk].y, acc[kk][1]);
-                acc[kk][2] = __builtin_fmaf(gv[u].z, s[kk].z, acc[kk][2]);
-                acc[kk][3] = __builtin_fmaf(gv[u].w, s[kk].w, acc[kk][3]);
-            }
+            const uint32_t m = (uint32_t)(mb + 4 * (wave * RU + u) + rs);
+            aoff[u] = m * (uint32_t)K + (uint32_t)k0;
+            goff[u] = (m * (uint32_t)N + (uint32_t)ncol) * 4u;
         }
-        if (more) {
+        const uint32_t astep = (uint32_t)(16 * RU * 4) * (uint32_t)K;
+        const uint32_t gstep = (uint32_t)(16 * RU * 4) * (uint32_t)N * 4u;
+        const unsigned char* gbytes = reinterpret_cast<const unsigned char*>(gC);
+        uint32_t a0[RU], a1[RU];
+        f32x4 g0[RU], g1[RU];
+        auto load = [&](uint32_t (&a)[RU], f32x4 (&g)[RU]) {
 #pragma unroll
             for (int u = 0; u < RU; ++u) {
-                a4[u] = a4n[u];
-                gv[u] = gvn[u];
+                a[u] = load_u32_unaligned(A + aoff[u]);
+                g[u] = *reinterpret_cast<const f32x4*>(gbytes + goff[u]);
+                aoff[u] += astep;
+                goff[u] += gstep;
+            }
+        };
+        if (iters > 0) load(a0, g0);
+        for (int it = 0; it < iters; it += 2) {
+            if (it + 1 < iters) load(a1, g1);
+#pragma unroll
+            for (int u = 0; u < RU; ++u) consume(a0[u], g0[u]);
+            if (it + 1 < iters) {
+                if (it + 2 < iters) load(a0, g0);
+#pragma unroll
+                for (int u = 0; u < RU; ++u) consume(a1[u], g1[u]);
+            }
+        }
+    } else {
+        for (int g0 = wave * RU; mb + 4 * g0 < me; g0 += 16 * RU) {
+#pragma unroll
+            for (int u = 0; u < RU; ++u) {
+                const int m = mb + 4 * (g0 + u) + rs;
+                const bool valid = m < me;
+                const int mc = valid ? m : me - 1;
+                const uint8_t* arow = A + (size_t)mc * K;
+                const uint32_t a = k_full ? load_u32_unaligned(arow + k0) : load_codes4_clamped(arow, k0, K);
+                const float* grow = gC + (size_t)mc * N;
+                f32x4 v;
+                if (cols_vec) {
+                    v = *reinterpret_cast<const f32x4*>(grow + ncol);
+                } else {
+                    v.x = (ncol + 0 < N) ? grow[ncol + 0] : 0.f;
+                    v.y = (ncol + 1 < N) ? grow[ncol + 1] : 0.f;
+                    v.z = (ncol + 2 < N) ? grow[ncol + 2] : 0.f;
+                    v.w = (ncol + 3 < N) ? grow[ncol + 3] : 0.f;
+                }
+                const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
+                consume(valid ? a : 0u, valid ? v : zero);
             }
         }
     }
@@ -204,7 +227,8 @@ hipError_t launch_gradB_slab(const float* gC, const uint8_t* A, const uint8_t* B
     float* out = zs > 1 ? partials : gB;
     const int vec_ok = ((N & 3) == 0) && (((uintptr_t)gC & 15) == 0);
     dim3 grid((N + 63) / 64, (K + kBwdKT - 1) / kBwdKT, zs);
-    if (vec_ok && (K & 3) == 0 && (N & 63) == 0)
+    const bool small = (size_t)M * K < (1ull << 31) && (size_t)M * N * 4 < (1ull << 31);
+    if (vec_ok && small && (K & 3) == 0 && (N & 63) == 0 && (M & 127) == 0 && (m_chunk & 127) == 0)
         hipLaunchKernelGGL(lutgemm_gradB_slab_kernel<true>, grid, dim3(1024), 0, stream, gC, A, B, out, lut, g.cols, 1 << g.bits,
                            flags, M, K, N, m_chunk, scale, vec_ok);
     else
