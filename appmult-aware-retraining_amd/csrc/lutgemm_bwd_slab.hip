@@ -25,6 +25,8 @@ namespace amr {
 constexpr int kBwdSlabRows = 128;
 constexpr int kBwdSlabBytes = kBwdSlabRows * 256;   // one k: 128 codes x 64 columns x fp32 = 32 KB
 constexpr int kBwdKT = 4;                            // k per workgroup (128 KB of LDS)
+constexpr int kBwdRU = 2;                            // row groups (of 4 rows) per wave and iteration in gradB
+constexpr int kBwdRowsPerIter = 16 * kBwdRU * 4;      // rows a workgroup consumes per iteration
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
@@ -84,7 +86,7 @@ __global__ __launch_bounds__(1024) void lutgemm_gradB_slab_kernel(
         for (int c = 0; c < 4; ++c) acc[kk][c] = 0.f;
     uint32_t seen = 0;
 
-    constexpr int RU = 2;   // row groups (of 4 rows) per wave and iteration
+    constexpr int RU = kBwdRU;   // row groups (of 4 rows) per wave and iteration
 
     // one row group: four 128-bit slab reads (one per k) and 16 multiply-adds
     auto consume = [&](uint32_t a, const f32x4& gvec) {
@@ -228,7 +230,7 @@ hipError_t launch_gradB_slab(const float* gC, const uint8_t* A, const uint8_t* B
     const int vec_ok = ((N & 3) == 0) && (((uintptr_t)gC & 15) == 0);
     dim3 grid((N + 63) / 64, (K + kBwdKT - 1) / kBwdKT, zs);
     const bool small = (size_t)M * K < (1ull << 31) && (size_t)M * N * 4 < (1ull << 31);
-    if (vec_ok && small && (K & 3) == 0 && (N & 63) == 0 && (M & 127) == 0 && (m_chunk & 127) == 0)
+    if (vec_ok && small && (K & 3) == 0 && (N & 63) == 0 && (M % kBwdRowsPerIter) == 0 && (m_chunk % kBwdRowsPerIter) == 0)
         hipLaunchKernelGGL(lutgemm_gradB_slab_kernel<true>, grid, dim3(1024), 0, stream, gC, A, B, out, lut, g.cols, 1 << g.bits,
                            flags, M, K, N, m_chunk, scale, vec_ok);
     else
