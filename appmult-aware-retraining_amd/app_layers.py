@@ -1,0 +1,245 @@
+"""Quantised layers that call the LUT operators (counterpart of the reference's ``micronet+/app_layers.py``).
+
+Same class names, constructor arguments, buffers and numerics as the reference, so a model prepared
+with :func:`prepare` behaves like one prepared there:
+
+* per-layer asymmetric quantisation to unsigned codes, ``scale = max((max-min)/(2^b-1), eps)``,
+  ``zp_neg = round(min/scale)``, real value ``= (code + zp_neg) * scale`` (reference ``app_layers.py:154-160``);
+* activations are tracked by an exponential moving average of min/max (momentum 0.1), weights by the
+  running extremes (reference ``:21-53``); both only update in training mode;
+* ``ApproxConv2d`` evaluates ``s_a*s_w*(AM(X,W) + conv(X,Zw) + conv(Za,W) + conv(Za,Zw)) + bias`` where
+  ``AM`` is the LUT convolution and the three ordinary convolutions undo the zero points
+  (reference ``:175-183``); rounding uses the straight-through estimator (``:147-150``);
+* ``QuantLinear`` and the pooling layers fake-quantise and call the ordinary torch op (``:101-111``,
+  ``:188-267``).
+"""
+import copy
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+import self_ops
+
+
+# ------------------------------------------------------------------------------------------ range tracking
+class ObserverBase(nn.Module):
+    """Tracks a (min, max) pair of the tensors it sees; never takes part in autograd."""
+
+    def __init__(self, q_level):
+        super().__init__()
+        self.q_level = q_level
+        self.num_flag = 0           # 0 until the first batch has been seen (python attribute, as in the reference)
+        self.register_buffer("min_val", torch.zeros(1, dtype=torch.float32))
+        self.register_buffer("max_val", torch.zeros(1, dtype=torch.float32))
+
+    def update_range(self, min_val_cur, max_val_cur):
+        raise NotImplementedError
+
+    @torch.no_grad()
+    def forward(self, input):
+        lo, hi = torch.min(input), torch.max(input)
+        if self.num_flag == 0:
+            self.num_flag = 1
+            self.min_val, self.max_val = lo, hi
+        else:
+            self.update_range(lo, hi)
+
+
+class MinMaxObserver(ObserverBase):
+    """Running extremes."""
+
+    def __init__(self, q_level, out_channels):
+        super().__init__(q_level)
+
+    def update_range(self, min_val_cur, max_val_cur):
+        self.min_val = torch.min(min_val_cur, self.min_val)
+        self.max_val = torch.max(max_val_cur, self.max_val)
+
+
+class MovingAverageMinMaxObserver(ObserverBase):
+    """Exponential moving average of the per-batch extremes."""
+
+    def __init__(self, q_level, out_channels, momentum=0.1):
+        super().__init__(q_level)
+        self.momentum = momentum
+
+    def update_range(self, min_val_cur, max_val_cur):
+        self.min_val = (1 - self.momentum) * self.min_val + self.momentum * min_val_cur
+        self.max_val = (1 - self.momentum) * self.max_val + self.momentum * max_val_cur
+
+
+def _scale_and_zero_point(observer, quant_max, eps):
+    scale = torch.max((observer.max_val - observer.min_val) / quant_max, eps)
+    return scale, torch.round(observer.min_val / scale)
+
+
+def _to_codes(x, scale, zp_neg, quant_max):
+    """Affine map to [0, quant_max] with straight-through rounding; returns integer-valued floats."""
+    affine = x / scale - zp_neg
+    return torch.clamp(affine - affine.detach() + torch.round(affine), 0, quant_max)
+
+
+# ------------------------------------------------------------------------------------------ quantiser module
+class AsymmetricQuantizer(nn.Module):
+    """Fake quantiser used in front of the pooling layers (reference ``app_layers.py:56-74``; note that its
+    rounding happens before the clamp, unlike the layer quantisers)."""
+
+    def __init__(self, bits, observer, activation_weight_flag=False, qaft=False, union=False):
+        super().__init__()
+        self.observer = observer
+        self.register_buffer("scale", torch.ones(1, dtype=torch.float32))
+        self.register_buffer("eps", torch.tensor(torch.finfo(torch.float32).eps, dtype=torch.float32))
+        self.register_buffer("quant_max_val", torch.tensor((1 << bits) - 1, dtype=torch.float32))
+        self.register_buffer("zero_point_neg", torch.zeros(1, dtype=torch.float32))
+
+    def forward(self, input):
+        if self.training:
+            self.observer(input)
+            self.scale, self.zero_point_neg = _scale_and_zero_point(self.observer, self.quant_max_val, self.eps)
+        q = input / self.scale - self.zero_point_neg
+        q = q - q.detach() + torch.round(q)
+        return (torch.clamp(q, 0, self.quant_max_val) + self.zero_point_neg) * self.scale
+
+
+class _QuantParamsMixin:
+    """Observers, scale / zero-point buffers shared by QuantLinear and ApproxConv2d."""
+
+    def _init_quant(self, a_bits, w_bits):
+        self.activation_observer = MovingAverageMinMaxObserver(q_level="L", out_channels=None)
+        self.weight_observer = MinMaxObserver(q_level="L", out_channels=None)
+        self.eps = torch.tensor(torch.finfo(torch.float32).eps, dtype=torch.float32)
+        self.activation_quant_max = torch.tensor((1 << a_bits) - 1, dtype=torch.float32)
+        self.register_buffer("activation_scale", torch.ones(1, dtype=torch.float32))
+        self.register_buffer("activation_zp_neg", torch.zeros(1, dtype=torch.float32))
+        self.weight_quant_max = torch.tensor((1 << w_bits) - 1, dtype=torch.float32)
+        self.register_buffer("weight_scale", torch.ones(1, dtype=torch.float32))
+        self.register_buffer("weight_zp_neg", torch.zeros(1, dtype=torch.float32))
+
+    def _update_ranges(self, input):
+        if self.training:
+            self.activation_observer(input)
+            self.activation_scale, self.activation_zp_neg = _scale_and_zero_point(
+                self.activation_observer, self.activation_quant_max, self.eps)
+            self.weight_observer(self.weight)
+            self.weight_scale, self.weight_zp_neg = _scale_and_zero_point(
+                self.weight_observer, self.weight_quant_max, self.eps)
+
+
+# ------------------------------------------------------------------------------------------ layers
+class QuantLinear(nn.Linear, _QuantParamsMixin):
+    """Fake-quantised fully connected layer (exact products, reference ``app_layers.py:78-113``)."""
+
+    def __init__(self, in_features, out_features, bias=True, a_bits=8, w_bits=8):
+        super().__init__(in_features, out_features, bias)
+        self._init_quant(a_bits, w_bits)
+
+    def quantize(self, x, s, zpn, qmax):
+        return (_to_codes(x, s, zpn, qmax) + zpn) * s
+
+    def forward(self, input):
+        self._update_ranges(input)
+        input_fq = self.quantize(input, self.activation_scale, self.activation_zp_neg, self.activation_quant_max)
+        weight_fq = self.quantize(self.weight, self.weight_scale, self.weight_zp_neg, self.weight_quant_max)
+        return F.linear(input_fq, weight_fq, self.bias)
+
+
+class ApproxConv2d(nn.Conv2d, _QuantParamsMixin):
+    """Convolution whose code products come from the approximate-multiplier table
+    (reference ``app_layers.py:116-185``)."""
+
+    def __init__(self, in_channels, out_channels, kernel_size, stride=1, padding=0, dilation=1, groups=1, bias=True,
+                 padding_mode="zeros", a_bits=8, w_bits=8, use_ste_gradient=False):
+        super().__init__(in_channels, out_channels, kernel_size, stride, padding, dilation, groups, bias, padding_mode)
+        self._init_quant(a_bits, w_bits)
+        self.conv2d_op = self_ops.approx_conv2d_baseline_op if use_ste_gradient else self_ops.approx_conv2d_op
+
+    def quantize_v2(self, x, s, zpn, qmax):
+        return _to_codes(x, s, zpn, qmax)
+
+    def forward(self, input):
+        self._update_ranges(input)
+        conv_args = dict(bias=None, stride=self.stride, padding=self.padding, dilation=self.dilation, groups=self.groups)
+        x_codes = self.quantize_v2(input, self.activation_scale, self.activation_zp_neg, self.activation_quant_max)
+        w_codes = self.quantize_v2(self.weight, self.weight_scale, self.weight_zp_neg, self.weight_quant_max)
+        x_zp = torch.full_like(x_codes, self.activation_zp_neg)
+        w_zp = torch.full_like(w_codes, self.weight_zp_neg)
+        total = (self.conv2d_op(x_codes, w_codes, **conv_args)      # approximate products of the codes
+                 + F.conv2d(x_codes, w_zp, **conv_args)             # zero-point corrections, exact
+                 + F.conv2d(x_zp, w_codes, **conv_args)
+                 + F.conv2d(x_zp, w_zp, **conv_args))
+        output = self.activation_scale * self.weight_scale * total
+        if self.bias is not None:
+            output += self.bias.view(1, -1, 1, 1)
+        return output
+
+
+def _pool_quantizer(a_bits, qaft):
+    return AsymmetricQuantizer(bits=a_bits, observer=MovingAverageMinMaxObserver(q_level="L", out_channels=None),
+                               activation_weight_flag=1, qaft=qaft)
+
+
+class QuantMaxPool2d(nn.MaxPool2d):
+    def __init__(self, kernel_size, stride=None, padding=0, dilation=1, return_indices=False, ceil_mode=False, a_bits=8,
+                 q_type=0, qaft=False, ptq=False, percentile=0.9999):
+        super().__init__(kernel_size, stride, padding, dilation, return_indices, ceil_mode)
+        self.activation_quantizer = _pool_quantizer(a_bits, qaft)
+
+    def forward(self, input):
+        return F.max_pool2d(self.activation_quantizer(input), self.kernel_size, self.stride, self.padding, self.dilation,
+                            self.return_indices, self.ceil_mode)
+
+
+class QuantAvgPool2d(nn.AvgPool2d):
+    def __init__(self, kernel_size, stride=None, padding=0, ceil_mode=False, count_include_pad=True, divisor_override=None,
+                 a_bits=8, q_type=0, qaft=False, ptq=False, percentile=0.9999):
+        super().__init__(kernel_size, stride, padding, ceil_mode, count_include_pad, divisor_override)
+        self.activation_quantizer = _pool_quantizer(a_bits, qaft)
+
+    def forward(self, input):
+        return F.avg_pool2d(self.activation_quantizer(input), self.kernel_size, self.stride, self.padding, self.ceil_mode,
+                            self.count_include_pad, self.divisor_override)
+
+
+# ------------------------------------------------------------------------------------------ model rewriting
+def add_quant_op(module, a_bits=8, w_bits=8, q_type=0, q_level=0, weight_observer=0, bn_fuse=False, bn_fuse_calib=False,
+                 pretrained_model=False, qaft=False, ptq=False, percentile=0.9999, use_ste_gradient=False):
+    """Replace, in place and recursively, Linear / Conv2d / MaxPool2d / AvgPool2d children by their quantised
+    versions; parameters are shared with the replaced module (reference ``app_layers.py:285-339``)."""
+    opts = dict(a_bits=a_bits, w_bits=w_bits, q_type=q_type, q_level=q_level, weight_observer=weight_observer, bn_fuse=bn_fuse,
+                bn_fuse_calib=bn_fuse_calib, pretrained_model=pretrained_model, qaft=qaft, ptq=ptq, percentile=percentile,
+                use_ste_gradient=use_ste_gradient)
+    for name, child in module.named_children():
+        if isinstance(child, nn.Linear):
+            new = QuantLinear(child.in_features, child.out_features, bias=child.bias is not None, a_bits=a_bits, w_bits=w_bits)
+        elif isinstance(child, nn.Conv2d):
+            new = ApproxConv2d(child.in_channels, child.out_channels, child.kernel_size, stride=child.stride, padding=child.padding,
+                               dilation=child.dilation, groups=child.groups, bias=child.bias is not None,
+                               padding_mode=child.padding_mode, a_bits=a_bits, w_bits=w_bits, use_ste_gradient=use_ste_gradient)
+        elif isinstance(child, nn.MaxPool2d):
+            new = QuantMaxPool2d(child.kernel_size, stride=child.stride, padding=child.padding, a_bits=a_bits, q_type=q_type,
+                                 qaft=qaft, ptq=ptq, percentile=percentile)
+        elif isinstance(child, nn.AvgPool2d):
+            new = QuantAvgPool2d(child.kernel_size, stride=child.stride, padding=child.padding, a_bits=a_bits, q_type=q_type,
+                                 qaft=qaft, ptq=ptq, percentile=percentile)
+        else:
+            add_quant_op(child, **opts)
+            continue
+        if isinstance(child, (nn.Linear, nn.Conv2d)):
+            new.weight.data = child.weight
+            if child.bias is not None:
+                new.bias.data = child.bias
+        module._modules[name] = new
+
+
+def prepare(model, inplace=False, a_bits=8, w_bits=8, q_type=0, q_level=0, weight_observer=0, bn_fuse=False, bn_fuse_calib=False,
+            pretrained_model=False, qaft=False, ptq=False, percentile=0.9999, use_ste_gradient=False):
+    """Return ``model`` (a deep copy unless ``inplace``) with every supported layer quantised
+    (reference ``app_layers.py:342-377``)."""
+    print(f'Quantizing model with a_bits={a_bits}, w_bits={w_bits}, use_ste_gradient={use_ste_gradient}')
+    if not inplace:
+        model = copy.deepcopy(model)
+    add_quant_op(model, a_bits=a_bits, w_bits=w_bits, q_type=q_type, q_level=q_level, weight_observer=weight_observer,
+                 bn_fuse=bn_fuse, bn_fuse_calib=bn_fuse_calib, pretrained_model=pretrained_model, qaft=qaft, ptq=ptq,
+                 percentile=percentile, use_ste_gradient=use_ste_gradient)
+    return model

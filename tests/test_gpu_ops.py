@@ -123,3 +123,49 @@ def test_acc_gemm_op(ops):
     torch.testing.assert_close(y, a @ b, rtol=1e-4, atol=1e-4)
     y.sum().backward()
     torch.testing.assert_close(a.grad, torch.ones(70, 30, device="cuda") @ b.detach().t())
+
+
+def test_approx_conv_layer_equals_fake_quant_conv_with_exact_multiplier(ops, oracle):
+    """With the exact-multiplier table the four-term expression of ApproxConv2d is the convolution of
+    the fake-quantised tensors (reference app_layers.py:175-183), up to fp32 rounding."""
+    import app_layers as L
+    self_ops, P = ops
+    print("layer exact", flush=True)
+    keep = (P.lut_appmult, P.lut_grad_a, P.lut_grad_b)
+    try:
+        n = np.arange(128)
+        Sx, Sy = oracle.ste_tables16(7)
+        P.set_lookup_tables("cuda", oracle.pack_table(n[:, None] * n[None, :], 7, np.uint16),
+                            oracle.pack_table(Sx, 7, np.int16), oracle.pack_table(Sy, 7, np.int16))
+        torch.manual_seed(0)
+        layer = L.ApproxConv2d(5, 7, 3, stride=1, padding=1, bias=True, a_bits=7, w_bits=7).cuda().train()
+        x = torch.randn(4, 5, 12, 12, device="cuda", requires_grad=True)
+        y = layer(x)
+        s_a, z_a, s_w, z_w = layer.activation_scale, layer.activation_zp_neg, layer.weight_scale, layer.weight_zp_neg
+        xq = (L._to_codes(x.detach(), s_a, z_a, 127.0) + z_a) * s_a
+        wq = (L._to_codes(layer.weight.detach(), s_w, z_w, 127.0) + z_w) * s_w
+        # a padding pixel contributes 0 to each of the four terms (code 0 times anything is 0 for the exact
+        # multiplier; the zero-point convolutions are zero padded), i.e. it is a real zero
+        ref = F.conv2d(xq, wq, layer.bias, padding=1)
+        torch.testing.assert_close(y, ref, rtol=1e-4, atol=1e-4)
+        y.square().mean().backward()
+        assert x.grad is not None and layer.weight.grad is not None and torch.isfinite(layer.weight.grad).all()
+    finally:
+        P.lut_appmult, P.lut_grad_a, P.lut_grad_b = keep
+
+
+def test_synthetic_training_steps_reduce_loss(ops, golden_dir):
+    """prepare -> calibrate -> a few optimiser steps of a small quantised net on one fixed batch."""
+    import app_layers as L
+    import app_train as T
+    print("train steps", flush=True)
+    torch.manual_seed(1)
+    net = torch.nn.Sequential(torch.nn.Conv2d(3, 8, 3, padding=1, bias=False), torch.nn.BatchNorm2d(8), torch.nn.ReLU(),
+                              torch.nn.Conv2d(8, 16, 3, stride=2, padding=1, bias=False), torch.nn.BatchNorm2d(16), torch.nn.ReLU(),
+                              torch.nn.AdaptiveAvgPool2d(1), torch.nn.Flatten(), torch.nn.Linear(16, 10)).cuda()
+    net = L.prepare(net, inplace=True, a_bits=7, w_bits=7)
+    xs, ys = T.synthetic_batches(1, 64, torch.device("cuda"))
+    T.calibrate(net, xs)
+    opt = torch.optim.Adam(net.parameters(), lr=1e-2)
+    losses = [float(l) for l in T.train_steps(net, opt, xs * 12, ys * 12)]
+    assert all(np.isfinite(losses)) and losses[-1] < losses[0]
