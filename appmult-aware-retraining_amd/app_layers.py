@@ -153,21 +153,41 @@ class ApproxConv2d(nn.Conv2d, _QuantParamsMixin):
         super().__init__(in_channels, out_channels, kernel_size, stride, padding, dilation, groups, bias, padding_mode)
         self._init_quant(a_bits, w_bits)
         self.conv2d_op = self_ops.approx_conv2d_baseline_op if use_ste_gradient else self_ops.approx_conv2d_op
+        self.reference_zero_point_terms = False     # True: evaluate the three correction terms as full convolutions
 
     def quantize_v2(self, x, s, zpn, qmax):
         return _to_codes(x, s, zpn, qmax)
+
+    def _zero_point_terms(self, x_codes, w_codes, conv_args):
+        """conv(X,Zw) + conv(Za,W) + conv(Za,Zw) without the three full convolutions: a convolution with a
+        constant operand factorises, conv(X, Zw*1) = Zw * box-sum of X over channels and window (one
+        output channel), conv(Za*1, W) = Za * (response of W to an all-ones image, batch of one), and
+        conv(Za*1, Zw*1) = Za*Zw*C * (number of taps inside the image).  All quantities are integer valued,
+        so as long as they stay below 2^24 the result is bit-identical to the literal form; autograd sees
+        ordinary torch ops and yields the same gradients for the codes."""
+        z_a, z_w = self.activation_zp_neg, self.weight_zp_neg
+        _, cin, h, w = x_codes.shape
+        kh, kw = w_codes.shape[2], w_codes.shape[3]
+        ones_k = torch.ones(1, 1, kh, kw, dtype=x_codes.dtype, device=x_codes.device)
+        ones_img = torch.ones(1, 1, h, w, dtype=x_codes.dtype, device=x_codes.device)
+        x_sum = F.conv2d(x_codes.sum(dim=1, keepdim=True), ones_k, **conv_args)                 # [B,1,oh,ow]
+        w_resp = F.conv2d(ones_img.expand(1, cin, h, w), w_codes, **conv_args)                  # [1,N,oh,ow]
+        taps = F.conv2d(ones_img, ones_k, **conv_args) * float(cin)                             # [1,1,oh,ow]
+        return z_w * x_sum + z_a * w_resp + (z_a * z_w) * taps
 
     def forward(self, input):
         self._update_ranges(input)
         conv_args = dict(bias=None, stride=self.stride, padding=self.padding, dilation=self.dilation, groups=self.groups)
         x_codes = self.quantize_v2(input, self.activation_scale, self.activation_zp_neg, self.activation_quant_max)
         w_codes = self.quantize_v2(self.weight, self.weight_scale, self.weight_zp_neg, self.weight_quant_max)
-        x_zp = torch.full_like(x_codes, self.activation_zp_neg)
-        w_zp = torch.full_like(w_codes, self.weight_zp_neg)
-        total = (self.conv2d_op(x_codes, w_codes, **conv_args)      # approximate products of the codes
-                 + F.conv2d(x_codes, w_zp, **conv_args)             # zero-point corrections, exact
-                 + F.conv2d(x_zp, w_codes, **conv_args)
-                 + F.conv2d(x_zp, w_zp, **conv_args))
+        total = self.conv2d_op(x_codes, w_codes, **conv_args)       # approximate products of the codes
+        if self.reference_zero_point_terms:
+            # the reference's literal form: three full convolutions with constant operands
+            x_zp = torch.full_like(x_codes, self.activation_zp_neg)
+            w_zp = torch.full_like(w_codes, self.weight_zp_neg)
+            total = total + F.conv2d(x_codes, w_zp, **conv_args) + F.conv2d(x_zp, w_codes, **conv_args) + F.conv2d(x_zp, w_zp, **conv_args)
+        else:
+            total = total + self._zero_point_terms(x_codes, w_codes, conv_args)
         output = self.activation_scale * self.weight_scale * total
         if self.bias is not None:
             output += self.bias.view(1, -1, 1, 1)

@@ -150,6 +150,21 @@ def test_approx_conv_layer_equals_fake_quant_conv_with_exact_multiplier(ops, ora
         torch.testing.assert_close(y, ref, rtol=1e-4, atol=1e-4)
         y.square().mean().backward()
         assert x.grad is not None and layer.weight.grad is not None and torch.isfinite(layer.weight.grad).all()
+        # the factorised zero-point terms equal the reference's three full convolutions, values and gradients
+        layer.eval()                                   # freeze the observers: both forms see the same scales
+        grads = []
+        outs = []
+        for literal in (False, True):
+            x.grad = None
+            layer.weight.grad = None
+            layer.reference_zero_point_terms = literal
+            out = layer(x)
+            out.square().mean().backward()
+            outs.append(out.detach())
+            grads.append((x.grad.clone(), layer.weight.grad.clone()))
+        assert torch.equal(outs[0], outs[1])           # integer-valued terms below 2^24: bit-identical
+        torch.testing.assert_close(grads[0][0], grads[1][0], rtol=1e-5, atol=1e-6)
+        torch.testing.assert_close(grads[0][1], grads[1][1], rtol=1e-5, atol=1e-6)
     finally:
         P.lut_appmult, P.lut_grad_a, P.lut_grad_b = keep
 
