@@ -36,6 +36,8 @@ _lib.amr_last_error.restype = ctypes.c_char_p
 _lib.amr_target_arch.restype = ctypes.c_char_p
 _lib.amr_lut_gemm_forward.argtypes = [_vp, _vp, _vp, _vp, _i64, _i, _i, _i, _vp]
 _lib.amr_lut_gemm_backward.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i, _i, _i, _vp, _sz, _vp]
+_lib.amr_lut_gemm_backward_ex.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i, _i, _i, _i, _vp, _sz, _vp]
+_lib.amr_im2col_u8_f32.argtypes = [_vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp]
 _lib.amr_lut_gemm_backward_workspace_bytes.argtypes = [_i, _i, _i]
 _lib.amr_lut_gemm_backward_workspace_bytes.restype = _sz
 _lib.amr_acc_gemm_forward_fp32.argtypes = [_vp, _vp, _vp, _i, _i, _i, _vp]
@@ -114,9 +116,13 @@ def acc_gemm_forward_fp32(a_tensor, b_tensor, c_tensor):
     _raise_for(rc, "acc_gemm_forward_fp32")
 
 
-def approx_gemm_backward(gc_tensor, a_tensor, b_tensor, ga_tensor, gb_tensor, lut_grad_a_tensor, lut_grad_b_tensor):
+def approx_gemm_backward(gc_tensor, a_tensor, b_tensor, ga_tensor, gb_tensor, lut_grad_a_tensor, lut_grad_b_tensor,
+                         ga_rows_per_image=0):
     """ga[m,k] = 1/16 sum_n gc[m,n]*lutA[a][b], gb[k,n] = 1/16 sum_m lutB[a][b]*gc[m,n]; outputs overwritten.
-    Contract of approx_gemm_backward_gpu (self_ops/src/approx_gemm_backward.cu:506-529)."""
+    Contract of approx_gemm_backward_gpu (self_ops/src/approx_gemm_backward.cu:506-529).
+
+    ga_rows_per_image = L > 0 (an extension; the reference has no such argument) makes ga_tensor the image-major
+    transposed gradient of shape [M/L, K, L], the layout torch's fold takes."""
     _check_input(gc_tensor, torch.float32, "gc_tensor")
     _check_input(a_tensor, torch.uint8, "a_tensor")
     _check_input(b_tensor, torch.uint8, "b_tensor")
@@ -124,12 +130,18 @@ def approx_gemm_backward(gc_tensor, a_tensor, b_tensor, ga_tensor, gb_tensor, lu
     _check_input(gb_tensor, torch.float32, "gb_tensor")
     _check_input(lut_grad_a_tensor, torch.int16, "lut_grad_a_tensor")
     _check_input(lut_grad_b_tensor, torch.int16, "lut_grad_b_tensor")
-    _check(all(t.dim() == 2 for t in (gc_tensor, a_tensor, b_tensor, ga_tensor, gb_tensor)), "gc, a, b, ga and gb must be 2-D")
+    L = int(ga_rows_per_image)
+    _check(all(t.dim() == 2 for t in (gc_tensor, a_tensor, b_tensor, gb_tensor)), "gc, a, b and gb must be 2-D")
     M, K = a_tensor.shape
     N = b_tensor.size(1)
     _check(gc_tensor.size(0) == M and gc_tensor.size(1) == N, f"gc_tensor's shape should be {M} x {N}")
     _check(K == b_tensor.size(0), f"b_tensor's shape should be {K} x {N}")
-    _check(ga_tensor.size(0) == M and ga_tensor.size(1) == K, f"ga_tensor's shape should be {M} x {K}")
+    if L > 0:
+        _check(M % L == 0, f"ga_rows_per_image={L} must divide {M}")
+        _check(tuple(ga_tensor.shape) == (M // L, K, L), f"ga_tensor's shape should be {M // L} x {K} x {L}")
+    else:
+        _check(L == 0, "ga_rows_per_image must not be negative")
+        _check(ga_tensor.dim() == 2 and ga_tensor.size(0) == M and ga_tensor.size(1) == K, f"ga_tensor's shape should be {M} x {K}")
     _check(gb_tensor.size(0) == K and gb_tensor.size(1) == N, f"gb_tensor's shape should be {K} x {N}")
     _lut_len_check(lut_grad_a_tensor, "lut_grad_a_tensor")
     _lut_len_check(lut_grad_b_tensor, "lut_grad_b_tensor")
@@ -140,11 +152,32 @@ def approx_gemm_backward(gc_tensor, a_tensor, b_tensor, ga_tensor, gb_tensor, lu
     with torch.cuda.device(dev):
         need = _lib.amr_lut_gemm_backward_workspace_bytes(M, K, N)
         ws = torch.empty(need, dtype=torch.uint8, device=dev) if need else None
-        rc = _lib.amr_lut_gemm_backward(gc_tensor.data_ptr(), a_tensor.data_ptr(), b_tensor.data_ptr(),
-                                        ga_tensor.data_ptr(), gb_tensor.data_ptr(), lut_grad_a_tensor.data_ptr(),
-                                        lut_grad_b_tensor.data_ptr(), lut_grad_a_tensor.size(0), M, K, N,
-                                        ws.data_ptr() if ws is not None else None, need, _stream_ptr(dev))
+        rc = _lib.amr_lut_gemm_backward_ex(gc_tensor.data_ptr(), a_tensor.data_ptr(), b_tensor.data_ptr(),
+                                           ga_tensor.data_ptr(), gb_tensor.data_ptr(), lut_grad_a_tensor.data_ptr(),
+                                           lut_grad_b_tensor.data_ptr(), lut_grad_a_tensor.size(0), M, K, N, L,
+                                           ws.data_ptr() if ws is not None else None, need, _stream_ptr(dev))
     _raise_for(rc, "approx_gemm_backward")
+
+
+def im2col_codes(x_tensor, a_tensor, kernel_size, stride, padding, dilation):
+    """a[(b,oy,ox), c*kh*kw+i*kw+j] = uint8(x[b,c,oy*s-p+i*d,ox*s-p+j*d]) (0 outside the image): the operand matrix that
+    the reference builds by pad + unfold + transpose + reshape + cast (self_ops/ops_py/approx_ops.py:556-563, :161-164).
+    x is a contiguous float32 [B,C,H,W] tensor of integer codes; a is uint8 [B*oh*ow, C*kh*kw]."""
+    _check_input(x_tensor, torch.float32, "x_tensor")
+    _check_input(a_tensor, torch.uint8, "a_tensor")
+    _check(x_tensor.dim() == 4 and a_tensor.dim() == 2, "x must be 4-D and a 2-D")
+    kh, kw = kernel_size
+    Bn, C, H, W = x_tensor.shape
+    oh = (H + 2 * padding - dilation * (kh - 1) - 1) // stride + 1
+    ow = (W + 2 * padding - dilation * (kw - 1) - 1) // stride + 1
+    _check(oh > 0 and ow > 0, "empty convolution output")
+    _check(tuple(a_tensor.shape) == (Bn * oh * ow, C * kh * kw), f"a_tensor's shape should be {Bn * oh * ow} x {C * kh * kw}")
+    dev = x_tensor.device
+    _check(dev == a_tensor.device, "device id not match")
+    with torch.cuda.device(dev):
+        rc = _lib.amr_im2col_u8_f32(x_tensor.data_ptr(), a_tensor.data_ptr(), Bn, C, H, W, kh, kw, stride, padding, dilation,
+                                    _stream_ptr(dev))
+    _raise_for(rc, "im2col_codes")
 
 
 def lds_gather_probe(pattern=0, waves_per_cu=16, iters=4000):

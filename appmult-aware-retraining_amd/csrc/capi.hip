@@ -21,7 +21,9 @@ hipError_t launch_gradB(const float* gC, const uint8_t* A, const uint8_t* B, flo
                         hipStream_t stream, const uint32_t* gate = nullptr);
 hipError_t launch_gradA(const float* gC, const uint8_t* A, const uint8_t* B, float* gA, const int16_t* lut,
                         const LutGeom& g, int M, int K, int N, float scale, int n_cu, hipStream_t stream,
-                        const uint32_t* gate = nullptr);
+                        const uint32_t* gate = nullptr, int rows_per_image = 0);
+hipError_t launch_im2col_u8_f32(const float* x, uint8_t* A, int B, int C, int H, int W, int kh, int kw, int stride, int pad,
+                                int dil, int oh, int ow, hipStream_t stream);
 bool bwd_slab_applies(const LutGeom& g, int M, int K, int N);
 int gradB_slab_splits(int M, int K, int N, int n_cu);
 hipError_t launch_gradB_slab(const float* gC, const uint8_t* A, const uint8_t* B, float* gB, const int16_t* lut,
@@ -179,6 +181,15 @@ size_t amr_lut_gemm_backward_workspace_bytes(int M, int K, int N) {
 int amr_lut_gemm_backward(const float* gC, const uint8_t* A, const uint8_t* B, float* gA, float* gB,
                           const int16_t* lut_grad_a, const int16_t* lut_grad_b, int64_t lut_elems, int M, int K,
                           int N, void* workspace, size_t workspace_bytes, void* stream) {
+    return amr_lut_gemm_backward_ex(gC, A, B, gA, gB, lut_grad_a, lut_grad_b, lut_elems, M, K, N, 0, workspace,
+                                    workspace_bytes, stream);
+}
+
+int amr_lut_gemm_backward_ex(const float* gC, const uint8_t* A, const uint8_t* B, float* gA, float* gB,
+                             const int16_t* lut_grad_a, const int16_t* lut_grad_b, int64_t lut_elems, int M, int K,
+                             int N, int ga_rows_per_image, void* workspace, size_t workspace_bytes, void* stream) {
+    if (ga_rows_per_image < 0 || (ga_rows_per_image > 0 && M % ga_rows_per_image != 0))
+        return fail(AMR_EINVAL, "ga_rows_per_image=%d must divide M=%d", ga_rows_per_image, M);
     if (M < 0 || K < 0 || N < 0) return fail(AMR_EINVAL, "negative dimension M=%d K=%d N=%d", M, K, N);
     amr::LutGeom g;
     if (!amr::lut_geom_from_elems(lut_elems, &g))
@@ -218,7 +229,7 @@ int amr_lut_gemm_backward(const float* gC, const uint8_t* A, const uint8_t* B, f
         if (e != hipSuccess) return hip_fail(e, "hipMemsetAsync");
     }
     if (gA) {
-        e = amr::launch_gradA(gC, A, B, gA, lut_grad_a, g, M, K, N, scale, n_cu, s);
+        e = amr::launch_gradA(gC, A, B, gA, lut_grad_a, g, M, K, N, scale, n_cu, s, nullptr, ga_rows_per_image);
         if (e != hipSuccess) return hip_fail(e, "gradA launch");
     }
     if (gB) {
@@ -233,6 +244,20 @@ int amr_lut_gemm_backward(const float* gC, const uint8_t* A, const uint8_t* B, f
         if (e != hipSuccess) return hip_fail(e, "gradB launch");
     }
     return AMR_OK;
+}
+
+int amr_im2col_u8_f32(const float* x, uint8_t* A, int B, int C, int H, int W, int kh, int kw, int stride, int pad, int dil,
+                      void* stream) {
+    if (B < 0 || C <= 0 || H <= 0 || W <= 0 || kh <= 0 || kw <= 0 || stride <= 0 || pad < 0 || dil <= 0)
+        return fail(AMR_EINVAL, "bad convolution geometry");
+    const int oh = (H + 2 * pad - dil * (kh - 1) - 1) / stride + 1;
+    const int ow = (W + 2 * pad - dil * (kw - 1) - 1) / stride + 1;
+    if (oh <= 0 || ow <= 0) return fail(AMR_EINVAL, "empty convolution output");
+    if (B == 0) return AMR_OK;
+    if ((long)B * oh * ow >= (1L << 31)) return fail(AMR_EUNSUPPORTED, "more than 2^31 output positions");
+    if (!x || !A) return fail(AMR_EINVAL, "null pointer argument");
+    hipError_t e = amr::launch_im2col_u8_f32(x, A, B, C, H, W, kh, kw, stride, pad, dil, oh, ow, reinterpret_cast<hipStream_t>(stream));
+    return e == hipSuccess ? AMR_OK : hip_fail(e, "im2col launch");
 }
 
 int amr_acc_gemm_forward_fp32(const float* A, const float* B, float* C, int M, int K, int N, void* stream) {

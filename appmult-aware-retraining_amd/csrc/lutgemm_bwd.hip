@@ -108,7 +108,7 @@ template <int KT, int RM, int WAVES, bool VEC>
 __global__ __launch_bounds__(WAVES * 64) void lutgemm_gradA_kernel(
     const float* __restrict__ gC, const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
     float* __restrict__ gA, const uint16_t* __restrict__ lut, int rows, int cols, int M, int K, int N, float scale,
-    const uint32_t* __restrict__ gate) {
+    const uint32_t* __restrict__ gate, int rows_per_image) {
     extern __shared__ __align__(16) unsigned char smem[];
     if (gate != nullptr && *gate == 0u) return;   // queued as a fallback that turned out not to be needed
     // Transposed staging: entry (a,b) of the row-major table goes to T[b][a], T row stride = cols
@@ -187,7 +187,15 @@ __global__ __launch_bounds__(WAVES * 64) void lutgemm_gradA_kernel(
 #pragma unroll
     for (int r = 0; r < RM; ++r) {
         const int m = m0 + lane + 64 * r;
-        if (m < M) {
+        if (m < M && rows_per_image > 0) {
+            // image-major transposed output gA_T[m / L][k][m % L] (L = rows_per_image): consecutive lanes hold
+            // consecutive rows, so every store instruction writes a contiguous run (the layout col2im wants)
+            const int img = m / rows_per_image, l = m - img * rows_per_image;
+            float* o = gA + ((size_t)img * K + k0) * rows_per_image + l;
+#pragma unroll
+            for (int kk = 0; kk < KT; ++kk)
+                if (k0 + kk < K) o[(size_t)kk * rows_per_image] = acc[r][kk] * scale;
+        } else if (m < M) {
             if (VEC) {
                 typedef float f32x4 __attribute__((ext_vector_type(4)));
 #pragma unroll
@@ -266,7 +274,8 @@ hipError_t launch_gradB(const float* gC, const uint8_t* A, const uint8_t* B, flo
 
 template <int KT, int RM, int WAVES, bool VEC>
 static hipError_t launch_gradA_t(const float* gC, const uint8_t* A, const uint8_t* B, float* gA, const int16_t* lut,
-                                 const LutGeom& g, int M, int K, int N, float scale, hipStream_t stream, const uint32_t* gate) {
+                                 const LutGeom& g, int M, int K, int N, float scale, hipStream_t stream, const uint32_t* gate,
+                                 int rows_per_image) {
     auto kern = lutgemm_gradA_kernel<KT, RM, WAVES, VEC>;
     static bool done = false;
     if (!done) {
@@ -277,28 +286,28 @@ static hipError_t launch_gradA_t(const float* gC, const uint8_t* A, const uint8_
     const int rows_per_wg = 64 * RM * WAVES;
     dim3 grid((K + KT - 1) / KT, (M + rows_per_wg - 1) / rows_per_wg);
     hipLaunchKernelGGL(kern, grid, dim3(WAVES * 64), (size_t)g.cols * g.cols * 2, stream, gC, A, B, gA,
-                       reinterpret_cast<const uint16_t*>(lut), g.rows, g.cols, M, K, N, scale, gate);
+                       reinterpret_cast<const uint16_t*>(lut), g.rows, g.cols, M, K, N, scale, gate, rows_per_image);
     return hipGetLastError();
 }
 
 hipError_t launch_gradA(const float* gC, const uint8_t* A, const uint8_t* B, float* gA, const int16_t* lut,
                         const LutGeom& g, int M, int K, int N, float scale, int n_cu, hipStream_t stream,
-                        const uint32_t* gate = nullptr) {
+                        const uint32_t* gate = nullptr, int rows_per_image = 0) {
     constexpr int KT = 16;
     const bool vec = ((N & 3) == 0) && ((K & 3) == 0) && (((uintptr_t)gC & 15) == 0) && (((uintptr_t)gA & 15) == 0);
     const int ktiles = (K + KT - 1) / KT;
     if (g.bits == 8) {
-        return vec ? launch_gradA_t<KT, 1, 16, true>(gC, A, B, gA, lut, g, M, K, N, scale, stream, gate)
-                   : launch_gradA_t<KT, 1, 16, false>(gC, A, B, gA, lut, g, M, K, N, scale, stream, gate);
+        return vec ? launch_gradA_t<KT, 1, 16, true>(gC, A, B, gA, lut, g, M, K, N, scale, stream, gate, rows_per_image)
+                   : launch_gradA_t<KT, 1, 16, false>(gC, A, B, gA, lut, g, M, K, N, scale, stream, gate, rows_per_image);
     }
     // Two rows per lane amortise the scalar work per gather; fall back to one when that would leave CUs idle.
     const long wg2 = (long)ktiles * ((M + 511) / 512);
     if (wg2 >= 2L * n_cu) {
-        return vec ? launch_gradA_t<KT, 2, 4, true>(gC, A, B, gA, lut, g, M, K, N, scale, stream, gate)
-                   : launch_gradA_t<KT, 2, 4, false>(gC, A, B, gA, lut, g, M, K, N, scale, stream, gate);
+        return vec ? launch_gradA_t<KT, 2, 4, true>(gC, A, B, gA, lut, g, M, K, N, scale, stream, gate, rows_per_image)
+                   : launch_gradA_t<KT, 2, 4, false>(gC, A, B, gA, lut, g, M, K, N, scale, stream, gate, rows_per_image);
     }
-    return vec ? launch_gradA_t<KT, 1, 4, true>(gC, A, B, gA, lut, g, M, K, N, scale, stream, gate)
-               : launch_gradA_t<KT, 1, 4, false>(gC, A, B, gA, lut, g, M, K, N, scale, stream, gate);
+    return vec ? launch_gradA_t<KT, 1, 4, true>(gC, A, B, gA, lut, g, M, K, N, scale, stream, gate, rows_per_image)
+               : launch_gradA_t<KT, 1, 4, false>(gC, A, B, gA, lut, g, M, K, N, scale, stream, gate, rows_per_image);
 }
 
 // Direct kernel queued behind the expanded-table kernel; it runs only when *gate != 0 (an operand

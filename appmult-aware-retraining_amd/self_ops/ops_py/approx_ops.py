@@ -181,12 +181,112 @@ def _conv2d_by_gemm(gemm, input, weight, bias, stride, padding, dilation, groups
     return out.view(batch, oh * ow, cout).transpose(1, 2).view(batch, cout, oh, ow)
 
 
+def _conv_geometry(input, weight, stride, padding, dilation):
+    s, p, d = stride[0], padding[0], dilation[0]
+    batch, cin, h, w = input.shape
+    cout, _, kh, kw = weight.shape
+    oh = (h + 2 * p - d * (kh - 1) - 1) // s + 1
+    ow = (w + 2 * p - d * (kw - 1) - 1) // s + 1
+    return s, p, d, batch, cin, h, w, cout, kh, kw, oh, ow
+
+
+def _conv_forward_codes(input, weight, geo):
+    """uint8 operand matrices of the convolution and its LUT-GEMM result as fp32 [B,O,oh,ow] (a view of the
+    [B*oh*ow, O] product, as the reference returns it, approx_ops.py:569-571)."""
+    s, p, d, batch, cin, h, w, cout, kh, kw, oh, ow = geo
+    x = input.detach().contiguous().to(torch.float32)
+    a_c = torch.empty((batch * oh * ow, cin * kh * kw), dtype=torch.uint8, device=x.device)
+    approx_ops.im2col_codes(x, a_c, (kh, kw), s, p, d)
+    b_c = weight.detach().reshape(cout, -1).t().to(torch.uint8).contiguous()
+    out = _lut_forward(a_c, b_c)
+    return a_c, b_c, out.view(batch, oh * ow, cout).transpose(1, 2).view(batch, cout, oh, ow)
+
+
+def _conv_grad_rows(g_out, geo):
+    """[B,O,oh,ow] output gradient as the contiguous [B*oh*ow, O] matrix of the GEMM (free when the gradient
+    arrives in the strides the forward result had)."""
+    batch, cout, oh, ow = geo[3], geo[7], geo[10], geo[11]
+    return g_out.permute(0, 2, 3, 1).reshape(batch * oh * ow, cout).contiguous()
+
+
+class ApproxConv2dFn(Function):
+    """Convolution of code tensors by im2col + LUT GEMM with LUT gradients: the computation of the reference's
+    approx_conv2d_op (approx_ops.py:530-573) with the unfold / transpose / cast glue done by one uint8 im2col pass,
+    and the input gradient produced directly in the [B, C*kh*kw, oh*ow] layout that fold consumes."""
+
+    @staticmethod
+    def forward(ctx, input, weight, stride, padding, dilation):
+        geo = _conv_geometry(input, weight, stride, padding, dilation)
+        a_c, b_c, out = _conv_forward_codes(input, weight, geo)
+        ctx.save_for_backward(a_c, b_c)
+        ctx.geo = geo
+        ctx.dtypes = (input.dtype, weight.dtype)
+        return out
+
+    @staticmethod
+    def backward(ctx, g_out):
+        assert g_out.dtype == torch.float32
+        a_c, b_c = ctx.saved_tensors
+        s, p, d, batch, cin, h, w, cout, kh, kw, oh, ow = ctx.geo
+        g_c = _conv_grad_rows(g_out, ctx.geo)
+        g_a = torch.empty((batch, cin * kh * kw, oh * ow), dtype=torch.float32, device=g_c.device)
+        g_b = torch.empty(b_c.shape, dtype=torch.float32, device=g_c.device)
+        approx_ops.approx_gemm_backward(g_c, a_c, b_c, g_a, g_b, lut_grad_a, lut_grad_b, ga_rows_per_image=oh * ow)
+        g_in = F.fold(g_a, (h, w), kernel_size=(kh, kw), dilation=(d, d), padding=(p, p), stride=(s, s))
+        g_w = g_b.t().reshape(cout, cin, kh, kw)
+        return g_in.to(ctx.dtypes[0]), g_w.to(ctx.dtypes[1]), None, None, None
+
+
+class ApproxConv2dBaselineFn(Function):
+    """Same forward; straight-through gradients, i.e. those of an exact convolution of the code tensors
+    (reference approx_conv2d_baseline_op, approx_ops.py:576-619, whose dense g_c.b^T and a^T.g_c followed by
+    fold are the input and weight gradients of conv2d)."""
+
+    @staticmethod
+    def forward(ctx, input, weight, stride, padding, dilation):
+        geo = _conv_geometry(input, weight, stride, padding, dilation)
+        _, _, out = _conv_forward_codes(input, weight, geo)
+        ctx.save_for_backward(input, weight)
+        ctx.geo = geo
+        return out
+
+    @staticmethod
+    def backward(ctx, g_out):
+        assert g_out.dtype == torch.float32
+        input, weight = ctx.saved_tensors
+        s, p, d = ctx.geo[:3]
+        g = g_out.contiguous()
+        x, wt = input.to(torch.float32), weight.to(torch.float32)
+        g_in = torch.nn.grad.conv2d_input(x.shape, wt, g, stride=s, padding=p, dilation=d)
+        g_w = torch.nn.grad.conv2d_weight(x, wt.shape, g, stride=s, padding=p, dilation=d)
+        return g_in.to(input.dtype), g_w.to(weight.dtype), None, None, None
+
+
+def _check_conv_args(bias, groups):
+    assert bias is None, 'bias is not supported in approximate convolution'
+    assert groups == 1, 'groups is not supported in approximate convolution'
+
+
 def approx_conv2d_op(input, weight, bias, stride, padding, dilation, groups):
     """conv2d as im2col + LUT GEMM with LUT gradients (reference ``approx_ops.py:530-573``).
-    ``input`` [B,C,H,W] and ``weight`` [O,C,kh,kw] hold integer codes; returns fp32 [B,O,oh,ow]."""
-    return _conv2d_by_gemm(approx_gemm_op, input, weight, bias, stride, padding, dilation, groups)
+    ``input`` [B,C,H,W] and ``weight`` [O,C,kh,kw] hold integer codes; returns fp32 [B,O,oh,ow].
+    Only element 0 of the stride / padding / dilation tuples is used, padding pixels hold code 0 (not the
+    zero-point) and the K index order is c*kh*kw + i*kw + j, all as in the reference."""
+    _check_conv_args(bias, groups)
+    return ApproxConv2dFn.apply(input, weight, tuple(stride), tuple(padding), tuple(dilation))
 
 
 def approx_conv2d_baseline_op(input, weight, bias, stride, padding, dilation, groups):
     """Same forward, straight-through gradients (reference ``approx_ops.py:576-619``)."""
+    _check_conv_args(bias, groups)
+    return ApproxConv2dBaselineFn.apply(input, weight, tuple(stride), tuple(padding), tuple(dilation))
+
+
+def approx_conv2d_unfold_op(input, weight, bias, stride, padding, dilation, groups):
+    """approx_conv2d_op composed exactly as the reference composes it (pad, unfold, transpose, GEMM op); kept as the
+    cross-check of the fused path."""
+    return _conv2d_by_gemm(approx_gemm_op, input, weight, bias, stride, padding, dilation, groups)
+
+
+def approx_conv2d_baseline_unfold_op(input, weight, bias, stride, padding, dilation, groups):
     return _conv2d_by_gemm(approx_gemm_baseline_op, input, weight, bias, stride, padding, dilation, groups)

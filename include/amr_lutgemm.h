@@ -92,6 +92,27 @@ int amr_lut_gemm_backward(const float *gC, const uint8_t *A, const uint8_t *B, f
                           int M, int K, int N, void *workspace, size_t workspace_bytes, void *stream);
 
 /*
+ * Same as amr_lut_gemm_backward with a choice of layout for gA.  ga_rows_per_image = 0: row-major [M,K].
+ * ga_rows_per_image = L > 0 (L must divide M): image-major transposed gA_T[M/L][K][L], i.e. the
+ * [batch, C*kh*kw, oh*ow] layout that col2im (torch fold) consumes directly when the rows of A are
+ * the im2col windows of M/L images -- saves the transpose copy between the GEMM and the fold in the
+ * reference's conv glue (self_ops/ops_py/approx_ops.py:562-563, backward).  No counterpart in the reference.
+ */
+int amr_lut_gemm_backward_ex(const float *gC, const uint8_t *A, const uint8_t *B, float *gA, float *gB,
+                             const int16_t *lut_grad_a, const int16_t *lut_grad_b, int64_t lut_elems,
+                             int M, int K, int N, int ga_rows_per_image, void *workspace, size_t workspace_bytes,
+                             void *stream);
+
+/*
+ * im2col of operand codes: x [B,C,H,W] float32 holding integer codes 0..255 -> A [B*oh*ow, C*kh*kw] uint8,
+ * row (b,oy,ox), column c*kh*kw + i*kw + j, same stride / padding / dilation on both axes, padding
+ * positions = code 0.  One pass instead of the reference's pad + unfold + transpose + reshape + cast
+ * (self_ops/ops_py/approx_ops.py:556-563, :161-164).
+ */
+int amr_im2col_u8_f32(const float *x, uint8_t *A, int B, int C, int H, int W, int kh, int kw, int stride, int pad,
+                      int dil, void *stream);
+
+/*
  * Accurate fp32 GEMM  C = A . B  (row-major), kept for API parity only.
  * Replaces acc_gemm_forward_fp32_gpu (self_ops/src/approx_gemm_forward.cu:494-571), bound as
  * approx_ops.acc_gemm_forward_fp32 (self_ops/src/op_register.cpp:18).

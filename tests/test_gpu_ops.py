@@ -115,6 +115,114 @@ def test_conv_op_against_oracle_with_shipped_table(ops, oracle, golden_dir):
     assert (y.cpu().numpy() == want.astype(np.float32)).all()
 
 
+@pytest.mark.parametrize("shape,k,stride,padding,dilation", [
+    ((3, 5, 10, 10), 3, 1, 1, 1),      # K = 45: byte stores
+    ((2, 4, 9, 7), 3, 2, 1, 1),        # K = 36, odd image, M not a multiple of 64
+    ((2, 8, 12, 12), 1, 2, 0, 1),      # 1x1 stride-2 downsample
+    ((1, 3, 16, 16), 7, 2, 3, 1),      # stem-like 7x7
+    ((2, 6, 11, 11), 3, 1, 2, 2),      # dilation
+    ((1, 130, 6, 6), 3, 1, 1, 1),      # K = 1170 > one 512-column tile, not a multiple of 4
+    ((2, 64, 8, 8), 3, 1, 1, 1),       # K = 576: two column tiles, 32-bit stores
+])
+def test_im2col_codes_against_oracle(ops, oracle, shape, k, stride, padding, dilation):
+    import approx_ops
+    print("im2col", shape, k, stride, padding, dilation, flush=True)
+    rng = np.random.default_rng(11)
+    x = rng.integers(0, 256, shape).astype(np.uint8)
+    want, oh, ow = oracle.im2col_np(x, k, k, stride, padding, dilation)
+    a = torch.full(want.shape, 77, dtype=torch.uint8, device="cuda")
+    approx_ops.im2col_codes(torch.tensor(x, device="cuda").float(), a, (k, k), stride, padding, dilation)
+    assert (a.cpu().numpy() == want).all()
+    # the same matrix the reference's pad + unfold + transpose + reshape + cast produces
+    xt = torch.tensor(x, device="cuda").float()
+    cols = F.unfold(F.pad(xt, (padding,) * 4), kernel_size=(k, k), dilation=dilation, stride=stride)
+    assert torch.equal(a, cols.transpose(1, 2).reshape(-1, want.shape[1]).to(torch.uint8))
+
+
+def test_im2col_codes_rejects_wrong_shapes(ops):
+    import approx_ops
+    x = torch.zeros(2, 3, 8, 8, device="cuda")
+    with pytest.raises(RuntimeError, match="a_tensor's shape should be 128 x 27"):
+        approx_ops.im2col_codes(x, torch.zeros(128, 28, dtype=torch.uint8, device="cuda"), (3, 3), 1, 1, 1)
+    with pytest.raises(RuntimeError, match="x_tensor must be of type"):
+        approx_ops.im2col_codes(x.half(), torch.zeros(128, 27, dtype=torch.uint8, device="cuda"), (3, 3), 1, 1, 1)
+    with pytest.raises(RuntimeError, match="empty convolution output"):
+        approx_ops.im2col_codes(x, torch.zeros(0, 3 * 81, dtype=torch.uint8, device="cuda"), (9, 9), 1, 0, 1)
+
+
+@pytest.mark.parametrize("M,K,N,L", [(192, 40, 24, 64), (150, 33, 10, 25), (4096, 64, 64, 1024), (6, 5, 3, 1)])
+def test_backward_image_major_ga_equals_row_major(ops, oracle, golden_dir, M, K, N, L):
+    import approx_ops
+    self_ops, P = ops
+    print("gA layout", M, K, N, L, flush=True)
+    rng = np.random.default_rng(5)
+    a = torch.tensor(rng.integers(0, 128, (M, K)).astype(np.uint8), device="cuda")
+    b = torch.tensor(rng.integers(0, 128, (K, N)).astype(np.uint8), device="cuda")
+    g = torch.tensor(rng.standard_normal((M, N)).astype(np.float32), device="cuda")
+    ga, gb = torch.empty(M, K, device="cuda"), torch.empty(K, N, device="cuda")
+    approx_ops.approx_gemm_backward(g, a, b, ga, gb, P.lut_grad_a, P.lut_grad_b)
+    ga_t, gb2 = torch.full((M // L, K, L), float("nan"), device="cuda"), torch.empty(K, N, device="cuda")
+    approx_ops.approx_gemm_backward(g, a, b, ga_t, gb2, P.lut_grad_a, P.lut_grad_b, ga_rows_per_image=L)
+    assert torch.equal(ga_t, ga.view(M // L, L, K).transpose(1, 2))      # same sums, other addresses
+    assert torch.equal(gb2, gb)
+    with pytest.raises(RuntimeError, match="must divide"):
+        approx_ops.approx_gemm_backward(g, a, b, ga_t, gb2, P.lut_grad_a, P.lut_grad_b, ga_rows_per_image=M + 1)
+
+
+@pytest.mark.parametrize("shape,cout,k,stride,padding,dilation", [
+    ((4, 16, 12, 12), 24, 3, 1, 1, 1), ((3, 8, 9, 9), 5, 3, 2, 1, 1), ((2, 12, 8, 8), 16, 1, 2, 0, 1),
+    ((2, 6, 10, 10), 7, 3, 1, 2, 2), ((64, 16, 8, 8), 64, 3, 1, 1, 1)])
+def test_conv_op_matches_reference_composition(ops, oracle, golden_dir, shape, cout, k, stride, padding, dilation):
+    """The one-pass convolution against pad + unfold + transpose + GEMM op, the composition the reference uses
+    (approx_ops.py:545-571), forward and both gradients, and against the float64 oracle."""
+    self_ops, P = ops
+    print("conv fused", shape, cout, k, stride, padding, dilation, flush=True)
+    fwd, ga, gb = oracle.parse_lut_file(os.path.join(golden_dir, "lut7_resub_63_bp8.txt.gz"), 7)
+    rng = np.random.default_rng(9)
+    xn = rng.integers(0, 128, shape).astype(np.uint8)
+    wn = rng.integers(0, 128, (cout, shape[1], k, k)).astype(np.uint8)
+    args = (None, (stride, stride), (padding, padding), (dilation, dilation), 1)
+    x = torch.tensor(xn, device="cuda").float().requires_grad_()
+    w = torch.tensor(wn, device="cuda").float().requires_grad_()
+    x2, w2 = x.detach().clone().requires_grad_(), w.detach().clone().requires_grad_()
+    y = self_ops.approx_conv2d_op(x, w, *args)
+    y2 = P.approx_conv2d_unfold_op(x2, w2, *args)
+    assert torch.equal(y, y2) and y.stride() == y2.stride()
+    g = torch.randn(y.shape, device="cuda")
+    y.backward(g)
+    y2.backward(g)
+    assert torch.equal(w.grad, w2.grad)
+    # fold adds the same per-window terms in a different order than the transposed copy + fold does: not bitwise
+    torch.testing.assert_close(x.grad, x2.grad, rtol=0, atol=1e-5 * float(x2.grad.abs().max()))
+    if np.prod(shape) <= 4096:
+        cols, oh, ow = oracle.im2col_np(xn, k, k, stride, padding, dilation)
+        gc = g.permute(0, 2, 3, 1).reshape(-1, cout).cpu().numpy()
+        a64, b64 = oracle.backward_np(gc, cols, wn.reshape(cout, -1).T, ga, gb)
+        np.testing.assert_allclose(w.grad.reshape(cout, -1).t().cpu().numpy(), b64, rtol=0, atol=1e-5 * np.abs(b64).max())
+        gx = F.fold(torch.tensor(a64, dtype=torch.float64).view(shape[0], oh * ow, -1).transpose(1, 2), shape[2:], (k, k),
+                    dilation=dilation, padding=padding, stride=stride).numpy()
+        np.testing.assert_allclose(x.grad.cpu().numpy(), gx, rtol=0, atol=1e-5 * np.abs(gx).max())
+    # straight-through variant: same forward, gradients of the exact convolution of the codes
+    xb, wb = x.detach().clone().requires_grad_(), w.detach().clone().requires_grad_()
+    xb2, wb2 = x.detach().clone().requires_grad_(), w.detach().clone().requires_grad_()
+    yb = self_ops.approx_conv2d_baseline_op(xb, wb, *args)
+    yb2 = P.approx_conv2d_baseline_unfold_op(xb2, wb2, *args)
+    assert torch.equal(yb, y2)
+    yb.backward(g)
+    yb2.backward(g)
+    torch.testing.assert_close(xb.grad, xb2.grad, rtol=1e-4, atol=1e-4 * float(xb2.grad.abs().max()))
+    torch.testing.assert_close(wb.grad, wb2.grad, rtol=1e-4, atol=1e-4 * float(wb2.grad.abs().max()))
+
+
+def test_conv_op_rejects_bias_and_groups(ops):
+    self_ops, P = ops
+    x, w = torch.zeros(1, 2, 4, 4, device="cuda"), torch.zeros(2, 2, 3, 3, device="cuda")
+    with pytest.raises(AssertionError, match="bias is not supported"):
+        self_ops.approx_conv2d_op(x, w, torch.zeros(2, device="cuda"), (1, 1), (1, 1), (1, 1), 1)
+    with pytest.raises(AssertionError, match="groups is not supported"):
+        self_ops.approx_conv2d_op(x, w, None, (1, 1), (1, 1), (1, 1), 2)
+
+
 def test_acc_gemm_op(ops):
     self_ops, P = ops
     a = torch.randn(70, 40, device="cuda", requires_grad=True)
