@@ -28,7 +28,7 @@ bool bwd_slab_applies(const LutGeom& g, int M, int K, int N);
 int gradB_slab_splits(int M, int K, int N, int n_cu);
 hipError_t launch_gradB_slab(const float* gC, const uint8_t* A, const uint8_t* B, float* gB, const int16_t* lut,
                              const LutGeom& g, int M, int K, int N, float scale, uint32_t* flags, float* partials,
-                             int splits, hipStream_t stream);
+                             int n_cu, hipStream_t stream);
 hipError_t launch_accgemm(const float* A, const float* B, float* C, int M, int K, int N, hipStream_t stream);
 hipError_t run_lds_probe(int pattern, int waves_per_cu, int iters, int n_cu, float* ms_out, double* gathers_out,
                          hipStream_t stream);
@@ -234,8 +234,7 @@ int amr_lut_gemm_backward_ex(const float* gC, const uint8_t* A, const uint8_t* B
     }
     if (gB) {
         if (slab) {
-            e = amr::launch_gradB_slab(gC, A, B, gB, lut_grad_b, g, M, K, N, scale, flags, partials,
-                                       amr::gradB_slab_splits(M, K, N, n_cu), s);
+            e = amr::launch_gradB_slab(gC, A, B, gB, lut_grad_b, g, M, K, N, scale, flags, partials, n_cu, s);
         } else {
             int splits = 1;
             amr::gradB_workspace_bytes(M, K, N, n_cu, &splits);

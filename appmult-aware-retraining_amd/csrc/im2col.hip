@@ -32,15 +32,26 @@ __global__ __launch_bounds__(256) void im2col_u8_f32_kernel(const float* __restr
     const int y0 = oy * stride - pad, x0 = ox * stride - pad;
     const float* xb = x + (size_t)b * C * H * W;
     const int khw = kh * kw;
-    for (int kk = wave; kk < kc; kk += 4) {
-        const int k = kc0 + kk;              // wave-uniform: the divisions below are scalar
-        const int c = k / khw;
-        const int t = k - c * khw;
-        const int i = t / kw, j = t - i * kw;
-        const int yy = y0 + i * dil, xx = x0 + j * dil;
-        float v = 0.f;
-        if (valid && yy >= 0 && yy < H && xx >= 0 && xx < W) v = xb[((size_t)c * H + yy) * W + xx];
-        tile[lane][kk] = (uint8_t)(int)v;
+    // Each wave takes every 4th column; kU columns per trip so that kU independent loads are in flight.
+    // Out-of-image taps read a clamped (valid) address and are zeroed by a select: no divergent branch.
+    constexpr int kU = 8;
+    for (int kb = wave; kb < kc; kb += 4 * kU) {
+        float v[kU];
+        bool in[kU];
+#pragma unroll
+        for (int u = 0; u < kU; ++u) {
+            const int k = min(kc0 + kb + 4 * u, K - 1);   // wave-uniform: the divisions below are scalar
+            const int c = k / khw;
+            const int t = k - c * khw;
+            const int i = t / kw, j = t - i * kw;
+            const int yy = y0 + i * dil, xx = x0 + j * dil;
+            in[u] = valid && yy >= 0 && yy < H && xx >= 0 && xx < W;
+            const int yc = min(max(yy, 0), H - 1), xc = min(max(xx, 0), W - 1);
+            v[u] = xb[((size_t)c * H + yc) * W + xc];
+        }
+#pragma unroll
+        for (int u = 0; u < kU; ++u)
+            if (kb + 4 * u < kc) tile[lane][kb + 4 * u] = in[u] ? (uint8_t)(int)v[u] : (uint8_t)0;
     }
     __syncthreads();
     const int rows = min(64, M - m0);

@@ -36,14 +36,19 @@ __device__ __forceinline__ void build_bwd_slab(float* slab, const int16_t* __res
                                                const uint8_t* __restrict__ B, int K, int N, int k0, int n0, int kt) {
     const int col = threadIdx.x & 63;
     const int a0 = threadIdx.x >> 6;
+    // all loads of one k are issued before the first is used (the table sits in L2; a dependent
+    // load-convert-store chain would pay that latency once per entry)
     for (int kk = 0; kk < kt; ++kk) {
         const bool live = (k0 + kk < K) && (n0 + col < N);
         const int b = live ? (int)B[(size_t)(k0 + kk) * N + n0 + col] : 0;
         float* s = slab + kk * (kBwdSlabBytes / 4);
-        for (int a = a0; a < kBwdSlabRows; a += 16) {
-            float v = 0.f;
-            if (live && a < n_codes) v = (float)G[a * lut_cols + b];
-            s[a * 64 + col] = v;
+        int16_t e[kBwdSlabRows / 16];
+#pragma unroll
+        for (int i = 0; i < kBwdSlabRows / 16; ++i) e[i] = G[min(a0 + 16 * i, n_codes - 1) * lut_cols + b];
+#pragma unroll
+        for (int i = 0; i < kBwdSlabRows / 16; ++i) {
+            const int a = a0 + 16 * i;
+            s[a * 64 + col] = (live && a < n_codes) ? (float)e[i] : 0.f;
         }
     }
 }
@@ -200,6 +205,181 @@ __global__ __launch_bounds__(1024) void lutgemm_gradB_slab_kernel(
     }
 }
 
+
+// ------------------------------------------------------------------------------------------ gradB, half-precision slab
+// Same scheme with the expanded table held as IEEE half, S16[kk][a][c] = half(G[a][b] - 1024), so that
+// eight k fit the 128 KB (half the gC traffic per multiply-add: every row of gC a workgroup streams is
+// used for 8 instead of 4 values of k) and one 64-bit LDS read brings four entries.  Exact: a half holds
+// every integer of magnitude <= 2048, i.e. table entries in [-1024, 3072] (16 x the gradient of a 7-bit
+// multiplier is about 16*b <= 2032); an entry outside that range raises flags[1] like a masked code does
+// and the direct kernel recomputes.  The multiply-add takes the half straight into an fp32 fma
+// (v_fma_mix_f32), products and sums are the same fp32 values as with an fp32 table, and the offset is
+// undone at the end with the column sums of gC:  sum_m g*(G-1024) + 1024 * sum_m g.
+//
+// LDS layout: byte address = (kk>>1)*32768 + a*256 + (kk&1)*128 + 2*c: the two k of a pair share a 256 B
+// row.  Row slots 1 and 3 of a wave visit the two k of every pair in the other order than slots 0 and 2,
+// so that the 32 lanes of a half-wave always read one 128 B half-row in banks 0-31 and one in banks 32-63.
+// Requires K % 8 == 0, N % 64 == 0, row counts that are multiples of the rows per iteration, gC 16-byte
+// aligned and 32-bit offsets (the launcher checks).
+constexpr int kBwdKT16 = 8;
+constexpr float kBwdHalfOffset = 1024.f;
+
+__global__ __launch_bounds__(1024) void lutgemm_gradB_slab16_kernel(
+    const float* __restrict__ gC, const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, float* __restrict__ out,
+    const int16_t* __restrict__ G, int lut_cols, int n_codes, uint32_t* __restrict__ flags, int M, int K, int N,
+    int m_chunk, float scale) {
+    constexpr int KT = kBwdKT16;
+    __shared__ __align__(16) unsigned char smem[KT * 16384];
+    const int tid = threadIdx.x;
+    const int wave = uniform(tid >> 6);
+    const int lane = tid & 63;
+    const int rs = lane >> 4, cg = lane & 15;
+    const uint32_t swap = (uint32_t)(rs & 1);
+    const int n0 = blockIdx.x * 64;
+    const int k0 = blockIdx.y * KT;
+    const int mb = blockIdx.z * m_chunk;
+    const int me = min(M, mb + m_chunk);
+
+    {   // expansion: wave-uniform code a, lanes = columns (the gathers of a wave stay inside one table row).
+        // All loads of a step are issued before the first is used: the table sits in L2 and a dependent
+        // load-convert-store chain would pay that latency 64 times per workgroup.
+        const int col = lane;
+        bool inexact = false;
+        int bcode[KT];
+#pragma unroll
+        for (int kk = 0; kk < KT; ++kk) bcode[kk] = (int)B[(size_t)(k0 + kk) * N + n0 + col];
+#pragma unroll
+        for (int kk = 0; kk < KT; ++kk) {
+            unsigned char* s = smem + (kk >> 1) * 32768 + (kk & 1) * 128 + 2 * col;
+            int16_t e[kBwdSlabRows / 16];
+#pragma unroll
+            for (int i = 0; i < kBwdSlabRows / 16; ++i) {
+                const int a = min(wave + 16 * i, n_codes - 1);
+                e[i] = G[a * lut_cols + bcode[kk]];
+            }
+#pragma unroll
+            for (int i = 0; i < kBwdSlabRows / 16; ++i) {
+                const int a = wave + 16 * i;
+                const float v = (a < n_codes) ? (float)e[i] : 0.f;
+                const _Float16 h = (_Float16)(v - kBwdHalfOffset);
+                inexact |= ((float)h != v - kBwdHalfOffset);
+                *reinterpret_cast<_Float16*>(s + a * 256) = h;
+            }
+        }
+        if (__builtin_amdgcn_ballot_w64(inexact) != 0 && lane == 0) atomicOr(&flags[1], 1u);
+    }
+    __syncthreads();
+
+    // address pieces: byte0 = half-row (pair member) and column group, byte1 = code (v_perm), byte2 = pair >> 1
+    const uint32_t lo_even = (swap << 7) | (uint32_t)(cg << 3);          // reads 0,2,4,6
+    const uint32_t lo_odd = ((swap ^ 1u) << 7) | (uint32_t)(cg << 3);    // reads 1,3,5,7
+    uint32_t sel[4];                                                     // code byte of read j: (j & 3) ^ swap
+#pragma unroll
+    for (int j = 0; j < 4; ++j) sel[j] = 0x0c020400u + ((uint32_t)(j ^ (int)swap) << 8);
+    const int ncol = n0 + 4 * cg;
+
+    typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+    float acc[KT][4];      // acc[j]: k = k0 + (j ^ swap)
+    float gsum[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int j = 0; j < KT; ++j)
+#pragma unroll
+        for (int c = 0; c < 4; ++c) acc[j][c] = 0.f;
+    uint32_t seen = 0;
+
+    constexpr int RU = kBwdRU;
+    auto consume = [&](uint32_t alo, uint32_t ahi, const f32x4& gvec) {
+        seen |= alo | ahi;
+        const uint32_t a4[2] = {alo, ahi};
+        f16x4 s[KT];
+#pragma unroll
+        for (int j = 0; j < KT; ++j) {
+            const uint32_t base = ((j & 1) ? lo_odd : lo_even) | ((j & 4) ? 0x10000u : 0u);
+            const uint32_t addr = __builtin_amdgcn_perm(a4[j >> 2], base, sel[j & 3]);
+            s[j] = *reinterpret_cast<const f16x4*>(smem + addr + ((j >> 1) & 1) * 32768);
+        }
+#pragma unroll
+        for (int j = 0; j < KT; ++j) {
+            acc[j][0] = __builtin_fmaf(gvec.x, (float)s[j].x, acc[j][0]);
+            acc[j][1] = __builtin_fmaf(gvec.y, (float)s[j].y, acc[j][1]);
+            acc[j][2] = __builtin_fmaf(gvec.z, (float)s[j].z, acc[j][2]);
+            acc[j][3] = __builtin_fmaf(gvec.w, (float)s[j].w, acc[j][3]);
+        }
+        gsum[0] += gvec.x; gsum[1] += gvec.y; gsum[2] += gvec.z; gsum[3] += gvec.w;
+    };
+
+    {
+        const int iters = (me - mb) / (16 * RU * 4);
+        uint32_t aoff[RU], goff[RU];
+#pragma unroll
+        for (int u = 0; u < RU; ++u) {
+            const uint32_t m = (uint32_t)(mb + 4 * (wave * RU + u) + rs);
+            aoff[u] = m * (uint32_t)K + (uint32_t)k0;
+            goff[u] = (m * (uint32_t)N + (uint32_t)ncol) * 4u;
+        }
+        const uint32_t astep = (uint32_t)(16 * RU * 4) * (uint32_t)K;
+        const uint32_t gstep = (uint32_t)(16 * RU * 4) * (uint32_t)N * 4u;
+        const unsigned char* gbytes = reinterpret_cast<const unsigned char*>(gC);
+        uint32_t al0[RU], ah0[RU], al1[RU], ah1[RU];
+        f32x4 g0[RU], g1[RU];
+        auto load = [&](uint32_t (&al)[RU], uint32_t (&ah)[RU], f32x4 (&g)[RU]) {
+#pragma unroll
+            for (int u = 0; u < RU; ++u) {
+                al[u] = load_u32_unaligned(A + aoff[u]);
+                ah[u] = load_u32_unaligned(A + aoff[u] + 4);
+                g[u] = *reinterpret_cast<const f32x4*>(gbytes + goff[u]);
+                aoff[u] += astep;
+                goff[u] += gstep;
+            }
+        };
+        if (iters > 0) load(al0, ah0, g0);
+        for (int it = 0; it < iters; it += 2) {
+            if (it + 1 < iters) load(al1, ah1, g1);
+#pragma unroll
+            for (int u = 0; u < RU; ++u) consume(al0[u], ah0[u], g0[u]);
+            if (it + 1 < iters) {
+                if (it + 2 < iters) load(al0, ah0, g0);
+#pragma unroll
+                for (int u = 0; u < RU; ++u) consume(al1[u], ah1[u], g1[u]);
+            }
+        }
+    }
+    if (__builtin_amdgcn_ballot_w64((seen & 0x80808080u) != 0) != 0) {
+        if (lane == 0) atomicOr(&flags[1], 1u);
+    }
+
+    // row slots 0+2 and 1+3 hold the same k order: add them in registers; the two orders, the 16 waves and
+    // the column sums of gC meet in LDS (the slabs are no longer needed)
+#pragma unroll
+    for (int j = 0; j < KT; ++j)
+#pragma unroll
+        for (int c = 0; c < 4; ++c) acc[j][c] += __shfl_xor(acc[j][c], 32);
+#pragma unroll
+    for (int c = 0; c < 4; ++c) gsum[c] += __shfl_xor(gsum[c], 32);
+    __syncthreads();
+    float* red = reinterpret_cast<float*>(smem);   // [wave][slot][KT + 1][64]
+    if (rs < 2) {
+        float* r = red + (size_t)((wave * 2 + rs) * (KT + 1)) * 64 + 4 * cg;
+#pragma unroll
+        for (int j = 0; j < KT; ++j)
+#pragma unroll
+            for (int c = 0; c < 4; ++c) r[(j ^ (int)swap) * 64 + c] = acc[j][c];
+#pragma unroll
+        for (int c = 0; c < 4; ++c) r[KT * 64 + c] = gsum[c];
+    }
+    __syncthreads();
+    if (tid < KT * 64) {
+        const int kk = tid >> 6, col = tid & 63;
+        float v = 0.f, gs = 0.f;
+#pragma unroll
+        for (int w = 0; w < 32; ++w) {
+            v += red[(w * (KT + 1) + kk) * 64 + col];
+            gs += red[(w * (KT + 1) + KT) * 64 + col];
+        }
+        out[((size_t)blockIdx.z * K + k0 + kk) * N + n0 + col] = (v + kBwdHalfOffset * gs) * scale;
+    }
+}
+
 // ------------------------------------------------------------------------------------------ host
 hipError_t launch_gradB_gated(const float* gC, const uint8_t* A, const uint8_t* B, float* gB, const int16_t* lut,
                               const LutGeom& g, int M, int K, int N, float scale, const uint32_t* gate, hipStream_t stream);
@@ -210,27 +390,51 @@ bool bwd_slab_applies(const LutGeom& g, int M, int K, int N) {
     return g.bits <= 7 && M >= 4096 && K >= 4;
 }
 
-// M splits of the expanded-table gradB: enough workgroups to fill the device, at least 2048 rows each.
+// M splits of the expanded-table gradB.  A workgroup fills a CU (128 KB of LDS), so the grid runs in rounds
+// of n_cu workgroups: pick the split count whose (rounds x rows per workgroup) is smallest, charging every
+// workgroup the cost of expanding its slabs (about that of streaming 512 rows) and keeping at least 2048
+// rows per workgroup.
+static int gradB_slab_splits_kt(int M, int K, int N, int n_cu, int kt) {
+    const long per_split = (long)((N + 63) / 64) * ((K + kt - 1) / kt);
+    long max_s = M / 2048;
+    if (max_s > 64) max_s = 64;
+    if (max_s < 1) max_s = 1;
+    long best_s = 1, best_cost = -1;
+    for (long sp = 1; sp <= max_s; ++sp) {
+        long chunk = (M + sp - 1) / sp;
+        chunk = (chunk + 255) & ~255L;
+        const long zs = (M + chunk - 1) / chunk;
+        const long rounds = (per_split * zs + n_cu - 1) / n_cu;
+        const long cost = rounds * (chunk + 512);
+        if (best_cost < 0 || cost < best_cost) { best_cost = cost; best_s = sp; }
+    }
+    return (int)best_s;
+}
+
+// Upper bound over the kernels launch_gradB_slab may pick (sizes the partial-sum scratch).
 int gradB_slab_splits(int M, int K, int N, int n_cu) {
-    const long per_split = (long)((N + 63) / 64) * ((K + kBwdKT - 1) / kBwdKT);
-    long splits = (2L * n_cu + per_split - 1) / per_split;
-    const long max_rows = M / 2048 > 0 ? M / 2048 : 1;
-    if (splits > max_rows) splits = max_rows;
-    if (splits > 64) splits = 64;
-    return splits < 1 ? 1 : (int)splits;
+    const int s4 = gradB_slab_splits_kt(M, K, N, n_cu, kBwdKT), s8 = gradB_slab_splits_kt(M, K, N, n_cu, kBwdKT16);
+    return s4 > s8 ? s4 : s8;
 }
 
 hipError_t launch_gradB_slab(const float* gC, const uint8_t* A, const uint8_t* B, float* gB, const int16_t* lut,
                              const LutGeom& g, int M, int K, int N, float scale, uint32_t* flags, float* partials,
-                             int splits, hipStream_t stream) {
+                             int n_cu, hipStream_t stream) {
+    const int vec_ok = ((N & 3) == 0) && (((uintptr_t)gC & 15) == 0);
+    const bool small = (size_t)M * K < (1ull << 31) && (size_t)M * N * 4 < (1ull << 31);
+    const bool regular = vec_ok && small && (N & 63) == 0 && (M % kBwdRowsPerIter) == 0;
+    const bool half_slab = regular && (K & 7) == 0;
+    const int kt = half_slab ? kBwdKT16 : kBwdKT;
+    const int splits = gradB_slab_splits_kt(M, K, N, n_cu, kt);
     int m_chunk = (M + splits - 1) / splits;
     m_chunk = (m_chunk + 255) & ~255;
     const int zs = (M + m_chunk - 1) / m_chunk;
     float* out = zs > 1 ? partials : gB;
-    const int vec_ok = ((N & 3) == 0) && (((uintptr_t)gC & 15) == 0);
-    dim3 grid((N + 63) / 64, (K + kBwdKT - 1) / kBwdKT, zs);
-    const bool small = (size_t)M * K < (1ull << 31) && (size_t)M * N * 4 < (1ull << 31);
-    if (vec_ok && small && (K & 3) == 0 && (N & 63) == 0 && (M % kBwdRowsPerIter) == 0 && (m_chunk % kBwdRowsPerIter) == 0)
+    dim3 grid((N + 63) / 64, (K + kt - 1) / kt, zs);
+    if (half_slab)
+        hipLaunchKernelGGL(lutgemm_gradB_slab16_kernel, grid, dim3(1024), 0, stream, gC, A, B, out, lut, g.cols, 1 << g.bits,
+                           flags, M, K, N, m_chunk, scale);
+    else if (regular && (K & 3) == 0)
         hipLaunchKernelGGL(lutgemm_gradB_slab_kernel<true>, grid, dim3(1024), 0, stream, gC, A, B, out, lut, g.cols, 1 << g.bits,
                            flags, M, K, N, m_chunk, scale, vec_ok);
     else
@@ -245,7 +449,9 @@ hipError_t launch_gradB_slab(const float* gC, const uint8_t* A, const uint8_t* B
         e = hipGetLastError();
         if (e != hipSuccess) return e;
     }
-    if (g.bits == 7) return launch_gradB_gated(gC, A, B, gB, lut, g, M, K, N, scale, flags + 1, stream);
+    // 7-bit operands can hold the masked code 128, and any table can hold an entry a half cannot: the gated
+    // direct kernel covers both (for narrower tables a code 2^b is an ordinary slab row of zeros)
+    if (g.bits == 7 || half_slab) return launch_gradB_gated(gC, A, B, gB, lut, g, M, K, N, scale, flags + 1, stream);
     return hipSuccess;
 }
 

@@ -237,6 +237,47 @@ def test_backward_large_m_masked_codes(lib, oracle):
     check_backward(oracle, gpu_backward(lib, g, A, B, la, lb), g, A, B, la, lb, 7)
 
 
+# K % 8 == 0, N % 64 == 0, M % 128 == 0 and M >= 4096: gradB runs on the expanded table held as halves (entries - 1024)
+HALF_SLAB_SHAPES = [(4096, 8, 64), (4224, 24, 128), (8192, 64, 64), (16384, 16, 192)]
+
+
+@pytest.mark.parametrize("bits", [7, 6, 4])
+@pytest.mark.parametrize("shape", HALF_SLAB_SHAPES)
+def test_backward_half_slab_tables_inside_the_exact_range(lib, oracle, bits, shape):
+    print("backward half slab", bits, shape, flush=True)
+    rng, A, B, _ = rand_case(hash((bits, shape, "h")) % 2**32, *shape, bits)
+    n = 1 << bits
+    Ga, Gb = rng.integers(-1024, 3073, (n, n)), rng.integers(-1024, 3073, (n, n))
+    Gb[0, 0], Gb[1, 1], Gb[2, 2], Gb[3, 3] = -1024, 3072, 3070, -1022     # ends of the range; even values beyond +-2048
+    la, lb = oracle.pack_table(Ga, bits, np.int16), oracle.pack_table(Gb, bits, np.int16)
+    g = (rng.standard_normal((shape[0], shape[2])) + 0.25).astype(np.float32)      # non-zero column sums
+    check_backward(oracle, gpu_backward(lib, g, A, B, la, lb), g, A, B, la, lb, bits)
+    if bits == 7:   # masked codes in both operands: the gated direct kernel takes over
+        A2, B2 = A.copy(), B.copy()
+        A2[::7, 3] = 128
+        A2[-1, :] = 128
+        B2[5, ::3] = 128
+        check_backward(oracle, gpu_backward(lib, g, A2, B2, la, lb), g, A2, B2, la, lb, bits)
+
+
+@pytest.mark.parametrize("bits", [7, 6])
+def test_backward_half_slab_entry_a_half_cannot_hold(lib, oracle, bits):
+    print("backward half slab inexact entry", bits, flush=True)
+    M, K, N = 4096, 16, 64
+    rng, A, B, _ = rand_case(77 + bits, M, K, N, bits)
+    n = 1 << bits
+    Ga, Gb = rng.integers(0, 2033, (n, n)), rng.integers(0, 2033, (n, n))
+    Gb[5, 9] = 3075            # 3075 - 1024 = 2051 is not a half
+    A[100, 3], B[3, 20] = 5, 9  # ... and it is used
+    la, lb = oracle.pack_table(Ga, bits, np.int16), oracle.pack_table(Gb, bits, np.int16)
+    g = rng.standard_normal((M, N)).astype(np.float32)
+    g[100, 20] = 1000.0        # make the one product matter
+    check_backward(oracle, gpu_backward(lib, g, A, B, la, lb), g, A, B, la, lb, bits)
+    Gb[5, 9] = -20000
+    lb = oracle.pack_table(Gb, bits, np.int16)
+    check_backward(oracle, gpu_backward(lib, g, A, B, la, lb), g, A, B, la, lb, bits)
+
+
 def test_backward_config2_difference_tables_and_ste(lib, oracle):
     print("backward config2", flush=True)
     A, B, T, g = oracle.synth_gemm(4096, 576, 64, bits=7, err=64, seed=0)
