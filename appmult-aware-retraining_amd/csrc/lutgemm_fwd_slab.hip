@@ -11,41 +11,45 @@
 // ds_read_b64.  64-bit LDS reads move 256 B/clk/CU on gfx950, twice the 32 lanes/clk of 16/32-bit
 // gathers, and they are conflict-free by construction here, so the LDS no longer limits the kernel.
 //
-// Layout of E in HBM (uint16): E[n_tile][k_pair][a (128 rows)][half (k parity)][64 columns]; one
-// (n_tile, k_pair) block is 32 KB, a table row of one k is 128 B and the two k of a pair share a
-// 256 B line.  A workgroup (16 waves) owns 512 rows of A and one 64-column tile, and walks K in
-// chunks of 4 (two k-pairs = 64 KB) that are double buffered in LDS and filled by LDS-direct loads.
-// Lane l of a wave: row slot rs = l/16 (4 rows per instruction), column group cg = l%16 (4 columns).
-// Odd row slots visit the two k of a pair in swapped order, so that in every instruction two slots
-// read the low 128 B half of their 256 B line and two the high half: each half lives in its own
-// 32 banks, which makes every read conflict-free.
-// The LDS address (buffer<<16 | a<<8 | half<<7 | cg<<3) is assembled from the code byte and a
+// Layout of E in HBM (uint16): E[n_tile][k_quad][a (128 rows)][kk (4 values of k)][32 columns]; one
+// (n_tile, k_quad) block ("chunk") is 32 KB and a code owns one 256 B line in it.
+// A workgroup (16 waves) owns 1024 rows of A and one 32-column tile and walks K chunk by chunk.
+// Four chunk buffers live in LDS; chunk c+2 is requested (LDS-direct loads) when chunk c starts to be
+// consumed, so a request has two chunk periods to arrive: with one period the L2 latency, not the
+// arithmetic, set the pace.  Every chunk a workgroup fetches serves 1024 x 4 x 32 additions.
+// Lane l of a wave: row slot rs = l/8 (8 rows per instruction), column group cg = l%8 (4 columns).
+// Row slot rs visits the four k of a chunk starting at k = rs%4, so in every instruction the four
+// slots of a half-wave read four different 64 B quarters of their 256 B lines: each quarter lives in its
+// own 16 banks, which makes every read conflict-free.
+// The LDS address (buffer pair<<16 | a<<8 | kk<<6 | cg<<3) is assembled from the code byte and a
 // per-lane constant by ONE v_perm_b32.  That needs a < 128: a 7-bit operand holding the masked code
 // 128 (zero contribution) is detected, flags[1] is raised and the direct kernel, queued behind this
 // one and gated on that flag, recomputes C.
 // Accumulation: when 4 * max(lut) < 65536 (flag written by the expand kernel) the four k of a chunk
 // are first added as packed uint16 pairs (v_pk_add_u16) and widened to 32 bit once per chunk.
+#include <type_traits>
+
 #include "amr_common.h"
 
 namespace amr {
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));   // native 16-byte vector (stays in registers)
 
-constexpr int kSlabRows = 128;                       // rows per (n_tile, k_pair) block
-constexpr int kSlabPairBytes = kSlabRows * 256;      // 32 KB
-constexpr int kSlabChunkPairs = 2;                   // k-pairs per LDS buffer (4 k)
-constexpr int kSlabChunkBytes = kSlabChunkPairs * kSlabPairBytes;   // 64 KB
+constexpr int kSlabRows = 128;                       // codes per chunk
+constexpr int kSlabCols = 32;                        // columns per n tile
+constexpr int kSlabChunkBytes = kSlabRows * 256;     // 32 KB: 128 codes x 4 k x 32 columns x uint16
+constexpr int kSlabBuffers = 4;
 
 // ------------------------------------------------------------------------------------------ expand
-// grid: (n_tiles, ceil(k_pairs_padded / PAIRS_PER_WG)); 256 threads.  k_pairs_padded is a multiple of
-// kSlabChunkPairs; pairs / columns beyond K / N are written as zeros.  Block (0,0) also writes
-// flags[0] = max over the table (used to pick the packed accumulation path).
-constexpr int kExpandPairsPerWg = 4;
+// grid: (n_tiles, ceil(k_quads / kExpandQuadsPerWg)); 256 threads.  Entries of k >= K or n >= N are
+// written as zeros.  Block (0,0) also writes flags[0] = max over the table (used to pick the packed
+// accumulation path).
+constexpr int kExpandQuadsPerWg = 4;
 
 __global__ __launch_bounds__(256) void expand_fwd_kernel(const uint8_t* __restrict__ B,
                                                          const uint32_t* __restrict__ lut32, int lut_dwords,
-                                                         int lut_cols, int n_codes, uint16_t* __restrict__ E,
-                                                         uint32_t* __restrict__ flags, int K, int N, int k_pairs_padded) {
+                                                         int lut_cols, int n_codes, uint32_t* __restrict__ E,
+                                                         uint32_t* __restrict__ flags, int K, int N, int k_quads) {
     extern __shared__ __align__(16) unsigned char smem[];
     uint32_t* s32 = reinterpret_cast<uint32_t*>(smem);
     uint32_t mx = 0;
@@ -63,28 +67,31 @@ __global__ __launch_bounds__(256) void expand_fwd_kernel(const uint8_t* __restri
     }
     const uint16_t* s16 = reinterpret_cast<const uint16_t*>(smem);
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    const int n = blockIdx.x * 64 + lane;
-    for (int pp = 0; pp < kExpandPairsPerWg; ++pp) {
-        const int kp = blockIdx.y * kExpandPairsPerWg + pp;
-        if (kp >= k_pairs_padded) break;
-        uint16_t* blk = E + ((size_t)blockIdx.x * k_pairs_padded + kp) * (kSlabPairBytes / 2);
-#pragma unroll
-        for (int h = 0; h < 2; ++h) {
-            const int k = 2 * kp + h;
-            const bool live = (k < K) && (n < N);
-            const int b = live ? (int)B[(size_t)k * N + n] : 0;
-            for (int a = wave; a < kSlabRows; a += 4) {
-                uint16_t v = 0;
-                if (live && a < n_codes) v = s16[a * lut_cols + b];
-                blk[a * 128 + h * 64 + lane] = v;
+    // a wave writes whole 256 B lines: lane = (kk, column pair), one dword (two columns) per lane
+    const int kk = lane >> 4, n = blockIdx.x * kSlabCols + 2 * (lane & 15);
+    for (int qq = 0; qq < kExpandQuadsPerWg; ++qq) {
+        const int q = blockIdx.y * kExpandQuadsPerWg + qq;
+        if (q >= k_quads) break;
+        uint32_t* blk = E + ((size_t)blockIdx.x * k_quads + q) * (kSlabChunkBytes / 4);
+        const int k = 4 * q + kk;
+        const bool live0 = (k < K) && (n < N), live1 = (k < K) && (n + 1 < N);
+        const int b0 = live0 ? (int)B[(size_t)k * N + n] : 0;
+        const int b1 = live1 ? (int)B[(size_t)k * N + n + 1] : 0;
+        for (int a = wave; a < kSlabRows; a += 4) {
+            uint32_t v = 0;
+            if (a < n_codes) {
+                const uint32_t v0 = live0 ? s16[a * lut_cols + b0] : 0u;
+                const uint32_t v1 = live1 ? s16[a * lut_cols + b1] : 0u;
+                v = v0 | (v1 << 16);
             }
+            blk[a * 64 + lane] = v;
         }
     }
 }
 
-// Copies one 64 KB chunk of E from global memory straight into LDS (global_load_lds_dwordx4: the data
+// Copies one 32 KB chunk of E from global memory straight into LDS (global_load_lds_dwordx4: the data
 // of lane l lands at the wave-uniform LDS base + 16*l; no VGPRs are held while the load is in flight).
-// Completion is tracked by vmcnt; the caller waits for vmcnt(0) before the barrier.
+// Completion is tracked by vmcnt (two operations per thread and chunk with 1024 threads).
 template <int THREADS>
 __device__ __forceinline__ void slab_copy_chunk(const u32x4* src, unsigned char* lds_dst, int tid, int wave) {
     typedef const __attribute__((address_space(1))) void* gptr_t;
@@ -100,14 +107,18 @@ __device__ __forceinline__ void slab_copy_chunk(const u32x4* src, unsigned char*
 
 // Eight 64-bit LDS reads (two row groups x four k) issued back to back, NOT waited for.  Inline
 // assembly, for two reasons: the reads of the chunk being consumed must not wait for the LDS-direct
-// loads of the NEXT chunk (the compiler cannot tell the two apart, same LDS array), and the reads of
+// loads of later chunks (the compiler cannot tell the two apart, same LDS array), and the reads of
 // block b+1 are issued before block b is consumed (software pipelining with explicit counters).
+// OFF is the part of the buffer offset that does not fit the v_perm-built address (odd buffers).
+template <int OFF>
 __device__ __forceinline__ void slab_issue8(uint64_t (&d)[8], const uint32_t (&addr)[8]) {
     asm volatile(
-        "ds_read_b64 %0, %8\n ds_read_b64 %1, %9\n ds_read_b64 %2, %10 offset:32768\n ds_read_b64 %3, %11 offset:32768\n"
-        "ds_read_b64 %4, %12\n ds_read_b64 %5, %13\n ds_read_b64 %6, %14 offset:32768\n ds_read_b64 %7, %15 offset:32768"
+        "ds_read_b64 %0, %8 offset:%16\n ds_read_b64 %1, %9 offset:%16\n ds_read_b64 %2, %10 offset:%16\n"
+        "ds_read_b64 %3, %11 offset:%16\n ds_read_b64 %4, %12 offset:%16\n ds_read_b64 %5, %13 offset:%16\n"
+        "ds_read_b64 %6, %14 offset:%16\n ds_read_b64 %7, %15 offset:%16"
         : "=&v"(d[0]), "=&v"(d[1]), "=&v"(d[2]), "=&v"(d[3]), "=&v"(d[4]), "=&v"(d[5]), "=&v"(d[6]), "=&v"(d[7])
-        : "v"(addr[0]), "v"(addr[1]), "v"(addr[2]), "v"(addr[3]), "v"(addr[4]), "v"(addr[5]), "v"(addr[6]), "v"(addr[7])
+        : "v"(addr[0]), "v"(addr[1]), "v"(addr[2]), "v"(addr[3]), "v"(addr[4]), "v"(addr[5]), "v"(addr[6]), "v"(addr[7]),
+          "n"(OFF)
         : "memory");
 }
 
@@ -122,33 +133,33 @@ __device__ __forceinline__ void slab_wait8(uint64_t (&d)[8]) {
 }
 
 template <int RG>
-__device__ __forceinline__ void slab_addr8(uint32_t (&addr)[8], const uint32_t (&a_cur)[RG], int i, uint32_t b0,
-                                           uint32_t b1, const uint32_t (&sel)[4]) {
+__device__ __forceinline__ void slab_addr8(uint32_t (&addr)[8], const uint32_t (&a_cur)[RG], int i,
+                                           const uint32_t (&base)[4], const uint32_t (&sel)[4]) {
 #pragma unroll
     for (int g = 0; g < 2; ++g)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) addr[4 * g + j] = __builtin_amdgcn_perm(a_cur[i + g], (j & 1) ? b1 : b0, sel[j]);
+        for (int j = 0; j < 4; ++j) addr[4 * g + j] = __builtin_amdgcn_perm(a_cur[i + g], base[j], sel[j]);
 }
 
 // One chunk (4 k) for all RG row groups of a lane; every code is < 128.
-template <int RG, bool PACKED>
-__device__ __forceinline__ void slab_chunk_fast(uint32_t (&acc)[RG][4], const uint32_t (&a_cur)[RG], uint32_t b0,
-                                                uint32_t b1, const uint32_t (&sel)[4]) {
+template <int RG, bool PACKED, int OFF>
+__device__ __forceinline__ void slab_chunk_fast(uint32_t (&acc)[RG][4], const uint32_t (&a_cur)[RG],
+                                                const uint32_t (&base)[4], const uint32_t (&sel)[4]) {
     static_assert(RG % 2 == 0, "row groups are processed in pairs");
     constexpr int NB = RG / 2;
     uint64_t d[2][8];
     {
         uint32_t addr[8];
-        slab_addr8<RG>(addr, a_cur, 0, b0, b1, sel);
-        slab_issue8(d[0], addr);
+        slab_addr8<RG>(addr, a_cur, 0, base, sel);
+        slab_issue8<OFF>(d[0], addr);
     }
 #pragma unroll
     for (int b = 0; b < NB; ++b) {
         const int i = 2 * b;
         if (b + 1 < NB) {
             uint32_t addr[8];
-            slab_addr8<RG>(addr, a_cur, i + 2, b0, b1, sel);
-            slab_issue8(d[(b + 1) & 1], addr);
+            slab_addr8<RG>(addr, a_cur, i + 2, base, sel);
+            slab_issue8<OFF>(d[(b + 1) & 1], addr);
             slab_wait8<8>(d[b & 1]);
         } else {
             slab_wait8<0>(d[b & 1]);
@@ -190,40 +201,63 @@ __device__ __forceinline__ void slab_chunk_fast(uint32_t (&acc)[RG][4], const ui
 }
 
 // ------------------------------------------------------------------------------------------ consume
+// The codes of A take the same road as the chunks: LDS-direct loads into a small staging area, 16 bytes
+// (the codes of four chunks) per row at a time, so that a cache line of A is asked for 8 times, not 32
+// (1024 rows x 128 B per workgroup do not stay in the caches between two visits).  No load of the main loop
+// has a register destination, so all waiting is explicit: the compiler forces vmcnt(0) in front of every
+// s_barrier it knows of and in front of the first use of a loaded register once LDS-direct loads are
+// pending, either of which would serialise the loop on the memory latency.  The barrier is therefore
+// issued from inline assembly together with the one wait that is needed.
+constexpr int kSlabCodeBytes = 16 * 64 * 16;   // staging of one group of four chunks: 16 waves x 64 rows x 16 codes
+
+// Eight dwords at a stride of 128 B (the codes of this lane's eight rows for one chunk).
+__device__ __forceinline__ void slab_read_codes(uint32_t (&a)[8], uint32_t addr) {
+    asm volatile(
+        "ds_read_b32 %0, %8\n ds_read_b32 %1, %8 offset:128\n ds_read_b32 %2, %8 offset:256\n ds_read_b32 %3, %8 offset:384\n"
+        "ds_read_b32 %4, %8 offset:512\n ds_read_b32 %5, %8 offset:640\n ds_read_b32 %6, %8 offset:768\n"
+        "ds_read_b32 %7, %8 offset:896\n s_waitcnt lgkmcnt(0)"
+        : "=&v"(a[0]), "=&v"(a[1]), "=&v"(a[2]), "=&v"(a[3]), "=&v"(a[4]), "=&v"(a[5]), "=&v"(a[6]), "=&v"(a[7])
+        : "v"(addr)
+        : "memory");
+}
+
 template <int RG, int WAVES, bool PACKED>
 __global__ __launch_bounds__(WAVES * 64) void lutgemm_fwd_slab_kernel(
     const uint8_t* __restrict__ A, const u32x4* __restrict__ E, uint32_t* __restrict__ C,
-    uint32_t* __restrict__ flags, int M, int K, int N, int k_pairs_padded, int chunks_per_split, int atomic_out) {
-    __shared__ __align__(16) unsigned char smem[2 * kSlabChunkBytes];   // static: lets the compiler fold the base address
+    uint32_t* __restrict__ flags, int M, int K, int N, int k_quads, int chunks_per_split, int atomic_out) {
+    // static: lets the compiler fold the base address (chunk buffers first: their addresses come out of v_perm)
+    __shared__ __align__(16) unsigned char smem[kSlabBuffers * kSlabChunkBytes + 2 * kSlabCodeBytes];
     constexpr int THREADS = WAVES * 64;
-    constexpr int ROWS_PER_WAVE = 4 * RG;
+    constexpr int ROWS_PER_WAVE = 8 * RG;
+    static_assert(RG == 8 && WAVES == 16, "staging layout and vmcnt bookkeeping are written for 16 waves of 64 rows");
+    static_assert(kSlabChunkBytes / 16 / THREADS == 2, "two chunk-copy operations per thread and chunk");
     const int tid = threadIdx.x;
     const int wave = uniform(tid >> 6);
     const int lane = tid & 63;
-    const int rs = lane >> 4, cg = lane & 15, odd = rs & 1;
+    const int rs = lane >> 3, cg = lane & 7, rot = rs & 3;
     // A wave whose rows would stick out of M is shifted up so that all its rows exist (the host only
     // takes this path for M >= 2048); the rows it then shares with the wave above are not stored twice.
     // (a wave entirely beyond M keeps running, it takes part in the chunk copies, and stores nothing)
     const int m_first = (blockIdx.y * WAVES + wave) * ROWS_PER_WAVE;     // first row this wave must store
     const int m_wave = min(m_first, M - ROWS_PER_WAVE);
-    const int total_chunks = k_pairs_padded / kSlabChunkPairs;
     const int c_begin = blockIdx.z * chunks_per_split;
-    const int c_end = min(total_chunks, c_begin + chunks_per_split);
+    const int c_end = min(k_quads, c_begin + chunks_per_split);
     if (c_begin >= c_end) return;
     // Two instances of this kernel are queued for every GEMM; the table maximum (written by the
     // expand kernel) decides which one does the work: 16-bit packed partial sums need 4*max < 65536.
     if ((flags[0] < 16384u) != PACKED) return;
 
-    const u32x4* Eblk = E + ((size_t)blockIdx.x * k_pairs_padded) * (kSlabPairBytes / 16);
-    // chunk c_begin -> buffer 0
-    slab_copy_chunk<THREADS>(Eblk + (size_t)c_begin * (kSlabChunkBytes / 16), smem, tid, wave);
+    const u32x4* Eblk = E + ((size_t)blockIdx.x * k_quads) * (kSlabChunkBytes / 16);
 
-    // per-lane address pieces; instruction j of a chunk: pair p = j>>1, t = j&1, half h = t ^ odd, k = 2p + h
-    uint32_t base[2], sel[4];
+    // per-lane address pieces; instruction j of a chunk reads k = 4c + ((j + rot) & 3)
+    uint32_t base_lo[4], base_hi[4], sel[4];
 #pragma unroll
-    for (int t = 0; t < 2; ++t) base[t] = (uint32_t)(((t ^ odd) << 7) | (cg << 3));
-#pragma unroll
-    for (int j = 0; j < 4; ++j) sel[j] = 0x0c020000u | ((uint32_t)(4 + (j & 2) + ((j & 1) ^ odd)) << 8);
+    for (int j = 0; j < 4; ++j) {
+        const uint32_t kk = (uint32_t)((j + rot) & 3);
+        base_lo[j] = (kk << 6) | (uint32_t)(cg << 3);
+        base_hi[j] = base_lo[j] | 0x10000u;
+        sel[j] = 0x0c020000u | ((4u + kk) << 8);
+    }
 
     uint32_t acc[RG][4];
 #pragma unroll
@@ -231,60 +265,73 @@ __global__ __launch_bounds__(WAVES * 64) void lutgemm_fwd_slab_kernel(
 #pragma unroll
         for (int c = 0; c < 4; ++c) acc[i][c] = 0u;
 
-    // Row group i of this lane is row m_wave + rs + 4 i: byte offset off0 + i * 4K, i.e. a per-lane
-    // 32-bit offset plus a wave-uniform term (the host only takes this path when M*K < 2^31).
-    const uint32_t off0 = (uint32_t)(m_wave + rs) * (uint32_t)K;
-    const uint32_t row_step = 4u * (uint32_t)K;
+    // Lane (rs, cg) consumes rows m_wave + 8 rs + i, i < 8.  Lane l fetches the codes of row
+    // m_wave + 8 (l % 8) + l / 8, which land at staging position l: row 8 rs + i sits at position 8 i + rs,
+    // so the eight dword reads of a chunk are a 128 B stride apart and the eight row slots of one read hit
+    // eight different banks.  32-bit offsets: the host only takes this path when M*K < 2^31.
+    const uint32_t code_off = (uint32_t)(m_wave + 8 * (lane & 7) + (lane >> 3)) * (uint32_t)K;
+    unsigned char* code_stage = smem + kSlabBuffers * kSlabChunkBytes + wave * 1024;      // + (group & 1) * kSlabCodeBytes
+    const uint32_t code_read = (uint32_t)(kSlabBuffers * kSlabChunkBytes + wave * 1024 + rs * 16);
+
+    typedef const __attribute__((address_space(1))) void* gptr_t;
+    typedef __attribute__((address_space(3))) void* lptr_t;
+    // Chunks / groups beyond the end repeat the last one (into buffers nobody reads any more) so that every
+    // step issues the same number of operations.  K % 4 == 0 (host): a group starts at code 4 (c_begin + 4 g);
+    // the last group is moved back so that its 16 bytes stay inside the row.
+    const int g_last = (c_end - 1 - c_begin) >> 2;
+    auto group_koff = [&](int g) { return min(4 * (c_begin + 4 * min(g, g_last)), K - 16); };
+    auto request_codes = [&](int g) {
+        __builtin_amdgcn_global_load_lds((gptr_t)(A + (code_off + (uint32_t)group_koff(g))),
+                                         (lptr_t)(code_stage + (g & 1) * kSlabCodeBytes), 16, 0, 0);
+    };
+    auto request_chunk = [&](int c, int buf) {
+        slab_copy_chunk<THREADS>(Eblk + (size_t)min(c, c_end - 1) * (kSlabChunkBytes / 16), smem + (size_t)buf * kSlabChunkBytes, tid, wave);
+    };
 
     uint32_t seen = 0;   // OR of every code dword this lane consumed
-    uint32_t a_cur[RG];
-    {
-        // The last chunk may stick out of K: read the last 4 codes of the row and shift, so the load
-        // stays inside the row; the surplus positions become code 0 and meet all-zero rows of E.
-        const int k0 = c_begin * 4;
-        const int koff = min(k0, K - 4), sh = 8 * (k0 - koff);
-#pragma unroll
-        for (int i = 0; i < RG; ++i) a_cur[i] = load_u32_unaligned(A + ((uint32_t)koff + (uint32_t)i * row_step) + off0) >> sh;
-    }
-    __builtin_amdgcn_s_waitcnt(0x0f70);   // vmcnt(0)
-    __syncthreads();
 
-    for (int c = c_begin; c < c_end; ++c) {
-        const int buf = (c - c_begin) & 1;
-        const bool more = (c + 1 < c_end);
-        uint32_t a_nxt[RG];
-        int sh_nxt = 0;
-        if (more) {
-            // the next chunk streams into the other buffer while this one is consumed
-            slab_copy_chunk<THREADS>(Eblk + (size_t)(c + 1) * (kSlabChunkBytes / 16), smem + (size_t)(buf ^ 1) * kSlabChunkBytes, tid, wave);
-            const int k1 = (c + 1) * 4;
-            const int koff = min(k1, K - 4);
-            sh_nxt = 8 * (k1 - koff);
+    // vmcnt counts the operations of a thread in issue order:
+    //   codes(g0) chunk(c0) chunk(c0+1) | step 0 of group g: codes(g+1) chunk(c+2) | steps 1..3: chunk(c+2)
+    // (a chunk request is two operations).  At the top of a step chunk(c), issued two steps earlier, and the
+    // codes of its group must have landed: everything but the requests of the previous step.
+    request_codes(0);
+    request_chunk(c_begin, 0);
+    request_chunk(c_begin + 1, 1);
+
+    auto step = [&](int c, int g, auto buf_tag) {
+        constexpr int BUF = decltype(buf_tag)::value;
+        if (BUF == 1)
+            asm volatile("s_waitcnt vmcnt(3)\n s_barrier" ::: "memory");
+        else
+            asm volatile("s_waitcnt vmcnt(2)\n s_barrier" ::: "memory");
+        if (BUF == 0) request_codes(g + 1);
+        request_chunk(c + 2, (BUF + 2) & 3);
+        uint32_t mine[RG];
+        slab_read_codes(mine, code_read + (uint32_t)((g & 1) * kSlabCodeBytes + (4 * c - group_koff(g))));
 #pragma unroll
-            for (int i = 0; i < RG; ++i) a_nxt[i] = load_u32_unaligned(A + ((uint32_t)koff + (uint32_t)i * row_step) + off0);
-        }
-        const uint32_t bsel = (uint32_t)buf << 16;
-        const uint32_t b0 = base[0] | bsel, b1 = base[1] | bsel;
-#pragma unroll
-        for (int i = 0; i < RG; ++i) seen |= a_cur[i];
-        slab_chunk_fast<RG, PACKED>(acc, a_cur, b0, b1, sel);
-        if (more) {
-#pragma unroll
-            for (int i = 0; i < RG; ++i) a_cur[i] = a_nxt[i] >> sh_nxt;
-        }
-        __builtin_amdgcn_s_waitcnt(0x0f70);   // vmcnt(0): the LDS-direct loads of the next chunk have landed
-        __syncthreads();
+        for (int i = 0; i < RG; ++i) seen |= mine[i];
+        if (BUF & 2)
+            slab_chunk_fast<RG, PACKED, (BUF & 1) * kSlabChunkBytes>(acc, mine, base_hi, sel);
+        else
+            slab_chunk_fast<RG, PACKED, (BUF & 1) * kSlabChunkBytes>(acc, mine, base_lo, sel);
+    };
+    for (int c = c_begin, g = 0; c < c_end; c += 4, ++g) {
+        step(c, g, std::integral_constant<int, 0>{});
+        if (c + 1 < c_end) step(c + 1, g, std::integral_constant<int, 1>{});
+        if (c + 2 < c_end) step(c + 2, g, std::integral_constant<int, 2>{});
+        if (c + 3 < c_end) step(c + 3, g, std::integral_constant<int, 3>{});
     }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // nothing is left in flight towards LDS when the workgroup ends
 
     // A code with bit 7 set (the masked code 128 of a 7-bit table) cannot be addressed by this kernel:
     // raise flags[1]; the host has queued the direct kernel behind this one, gated on that flag.
     if (__builtin_amdgcn_ballot_w64((seen & 0x80808080u) != 0) != 0) {
         if (lane == 0) atomicOr(&flags[1], 1u);
     }
-    const int n = blockIdx.x * 64 + 4 * cg;
+    const int n = blockIdx.x * kSlabCols + 4 * cg;
 #pragma unroll
     for (int i = 0; i < RG; ++i) {
-        const int m = m_wave + 4 * i + rs;
+        const int m = m_wave + 8 * rs + i;
         if (m >= m_first) {
 #pragma unroll
             for (int c = 0; c < 4; ++c) {
@@ -307,41 +354,40 @@ hipError_t launch_fwd_gated(const uint8_t* A, const uint8_t* B, uint32_t* C, con
 size_t fwd_slab_workspace_bytes(const LutGeom& g, int M, int K, int N) {
     // Worth it when the 2^b/M expansion overhead is small and K is long enough to amortise the extra
     // launches (measured cross-over on MI355X: K around 512).
-    if (g.bits > 7 || M < 2048 || K < 512 || (size_t)M * K >= (1ull << 31)) return 0;
-    const size_t n_tiles = (N + 63) / 64;
-    const size_t kpp = (((size_t)K + 1) / 2 + kSlabChunkPairs - 1) / kSlabChunkPairs * kSlabChunkPairs;
-    return 256 + n_tiles * kpp * kSlabPairBytes;
+    // (K % 4 == 0: the codes of A are fetched four and sixteen at a time)
+    if (g.bits > 7 || M < 2048 || K < 512 || (K & 3) != 0 || (size_t)M * K >= (1ull << 31)) return 0;
+    const size_t n_tiles = (N + kSlabCols - 1) / kSlabCols;
+    const size_t k_quads = ((size_t)K + 3) / 4;
+    return 256 + n_tiles * k_quads * kSlabChunkBytes;
 }
 
 hipError_t launch_fwd_slab(const uint8_t* A, const uint8_t* B, uint32_t* C, const uint16_t* lut, const LutGeom& g,
                            int M, int K, int N, int n_cu, void* workspace, hipStream_t stream) {
-    const int n_tiles = (N + 63) / 64;
-    const int kpp = ((K + 1) / 2 + kSlabChunkPairs - 1) / kSlabChunkPairs * kSlabChunkPairs;
+    const int n_tiles = (N + kSlabCols - 1) / kSlabCols;
+    const int k_quads = (K + 3) / 4;
     uint32_t* flags = reinterpret_cast<uint32_t*>(workspace);
-    uint16_t* E = reinterpret_cast<uint16_t*>(reinterpret_cast<unsigned char*>(workspace) + 256);
+    uint32_t* E = reinterpret_cast<uint32_t*>(reinterpret_cast<unsigned char*>(workspace) + 256);
     hipError_t e = hipMemsetAsync(flags, 0, 256, stream);
     if (e != hipSuccess) return e;
     const int lut_dwords = g.rows * g.cols / 2;
-    hipLaunchKernelGGL(expand_fwd_kernel, dim3(n_tiles, (kpp + kExpandPairsPerWg - 1) / kExpandPairsPerWg), dim3(256),
+    hipLaunchKernelGGL(expand_fwd_kernel, dim3(n_tiles, (k_quads + kExpandQuadsPerWg - 1) / kExpandQuadsPerWg), dim3(256),
                        (size_t)lut_dwords * 4, stream, B, reinterpret_cast<const uint32_t*>(lut), lut_dwords, g.cols,
-                       1 << g.bits, E, flags, K, N, kpp);
+                       1 << g.bits, E, flags, K, N, k_quads);
     e = hipGetLastError();
     if (e != hipSuccess) return e;
 
-    // 512 rows per workgroup
-    const int chunks = kpp / kSlabChunkPairs;
-    // 16 waves x 32 rows = 512 rows per workgroup (measured best among 256/512/1024-row tilings)
+    // 16 waves x 64 rows = 1024 rows per workgroup
     constexpr int RG = 8, WAVES = 16;
-    const int m_tile = WAVES * 4 * RG;
+    const int m_tile = WAVES * 8 * RG;
     const long wgs = (long)n_tiles * ((M + m_tile - 1) / m_tile);
     int ksplit = 1;
     if (wgs < n_cu) {
         ksplit = (int)((n_cu + wgs - 1) / wgs);
-        const int max_split = chunks / 8 > 0 ? chunks / 8 : 1;     // at least 32 k per workgroup
+        const int max_split = k_quads / 8 > 0 ? k_quads / 8 : 1;     // at least 32 k per workgroup
         if (ksplit > max_split) ksplit = max_split;
     }
-    const int cps = (chunks + ksplit - 1) / ksplit;
-    const int zs = (chunks + cps - 1) / cps;
+    const int cps = (k_quads + ksplit - 1) / ksplit;
+    const int zs = (k_quads + cps - 1) / cps;
     if (zs > 1) {
         e = hipMemsetAsync(C, 0, (size_t)M * N * sizeof(uint32_t), stream);
         if (e != hipSuccess) return e;
@@ -349,9 +395,9 @@ hipError_t launch_fwd_slab(const uint8_t* A, const uint8_t* B, uint32_t* C, cons
     dim3 grid(n_tiles, (M + m_tile - 1) / m_tile, zs);
     // both accumulation flavours are queued; flags[0] (table maximum) decides on the device which one works
     hipLaunchKernelGGL((lutgemm_fwd_slab_kernel<RG, WAVES, true>), grid, dim3(WAVES * 64), 0, stream, A,
-                       reinterpret_cast<const u32x4*>(E), C, flags, M, K, N, kpp, cps, zs > 1 ? 1 : 0);
+                       reinterpret_cast<const u32x4*>(E), C, flags, M, K, N, k_quads, cps, zs > 1 ? 1 : 0);
     hipLaunchKernelGGL((lutgemm_fwd_slab_kernel<RG, WAVES, false>), grid, dim3(WAVES * 64), 0, stream, A,
-                       reinterpret_cast<const u32x4*>(E), C, flags, M, K, N, kpp, cps, zs > 1 ? 1 : 0);
+                       reinterpret_cast<const u32x4*>(E), C, flags, M, K, N, k_quads, cps, zs > 1 ? 1 : 0);
     e = hipGetLastError();
     if (e != hipSuccess) return e;
     if (g.bits == 7) return launch_fwd_gated(A, B, C, lut, g, M, K, N, flags + 1, stream);

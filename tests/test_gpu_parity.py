@@ -89,7 +89,10 @@ def test_forward_bit_exact_random_tables(lib, oracle, bits, shape):
 
 
 # shapes with M >= 2048 and K >= 512 take the expanded-table forward path (tables of at most 7 bits)
-BIG_M_SHAPES = [(2048, 512, 64), (2081, 515, 65), (3000, 27, 10), (4096, 640, 300), (2500, 1153, 128), (5000, 777, 1)]
+# (K % 4 == 0 and K >= 512 take the expanded-table kernels; K % 16 != 0 moves the last group of codes back; a small
+# M x N grid splits K over workgroups)
+BIG_M_SHAPES = [(2048, 512, 64), (2081, 515, 65), (2081, 516, 65), (3000, 27, 10), (4096, 640, 300), (2500, 1153, 128),
+                (2500, 1156, 128), (5000, 777, 1), (5000, 776, 1), (2048, 2056, 96), (3100, 520, 33)]
 
 
 @pytest.mark.parametrize("bits", [7, 6, 4, 8])
@@ -103,7 +106,7 @@ def test_forward_bit_exact_large_m(lib, oracle, bits, shape):
 
 def test_forward_large_m_small_table_values_masked_codes_and_own_workspace(lib, oracle):
     print("forward large M masked / workspace", flush=True)
-    M, K, N = 2600, 530, 70
+    M, K, N = 2600, 532, 70
     rng, A, B, _ = rand_case(99, M, K, N, 7)
     T = oracle.synth_lut(7, 64, rng)                      # max < 16384: packed 16-bit partial sums
     flat = oracle.pack_table(T, 7, np.uint16)
