@@ -22,6 +22,10 @@ hipError_t launch_gradB(const float* gC, const uint8_t* A, const uint8_t* B, flo
 hipError_t launch_gradA(const float* gC, const uint8_t* A, const uint8_t* B, float* gA, const int16_t* lut,
                         const LutGeom& g, int M, int K, int N, float scale, int n_cu, hipStream_t stream,
                         const uint32_t* gate = nullptr, int rows_per_image = 0);
+size_t gradA_slab_workspace_bytes(const LutGeom& g, int M, int K, int N);
+hipError_t launch_gradA_slab(const float* gC, const uint8_t* A, const uint8_t* B, float* gA, const int16_t* lut,
+                             const LutGeom& g, int M, int K, int N, float scale, int n_cu, uint32_t* flags, void* S,
+                             int rows_per_image, hipStream_t stream);
 hipError_t launch_im2col_u8_f32(const float* x, uint8_t* A, int B, int C, int H, int W, int kh, int kw, int stride, int pad,
                                 int dil, int oh, int ow, hipStream_t stream);
 bool bwd_slab_applies(const LutGeom& g, int M, int K, int N);
@@ -163,19 +167,29 @@ int amr_lut_gemm_forward(const uint8_t* A, const uint8_t* B, uint32_t* C, const 
     return amr_lut_gemm_forward_ws(A, B, C, lut, lut_elems, M, K, N, nullptr, 0, stream);
 }
 
-// Scratch layout of the backward pass: [256 B of flags][partial sums of gB over the M splits].
+// Scratch layout of the backward pass: [256 B of flags][partial sums of gB over the M splits][expanded
+// gradient table of gradA]; each part a multiple of 256 bytes.
 static size_t backward_partial_bytes(int M, int K, int N, int n_cu) {
     size_t direct = amr::gradB_workspace_bytes(M, K, N, n_cu, nullptr);
     const int s = amr::gradB_slab_splits(M, K, N, n_cu);
     size_t slab = s > 1 ? (size_t)s * K * N * sizeof(float) : 0;
-    return direct > slab ? direct : slab;
+    const size_t b = direct > slab ? direct : slab;
+    return (b + 255) & ~(size_t)255;
+}
+
+// Size of the expanded table of gradA for 7-bit tables (the widest the expanded-table kernels take); a query
+// by shape alone cannot know the table width, so the scratch is sized for it.
+static size_t backward_gradA_bytes(int M, int K, int N) {
+    amr::LutGeom g7;
+    amr::lut_geom_from_bits(7, &g7);
+    return amr::gradA_slab_workspace_bytes(g7, M, K, N);
 }
 
 size_t amr_lut_gemm_backward_workspace_bytes(int M, int K, int N) {
     if (M <= 0 || K <= 0 || N <= 0) return 0;
     const int n_cu = current_device_cus(nullptr);
     // Without a device (e.g. a host-only query) size for a 256-CU part.
-    return 256 + backward_partial_bytes(M, K, N, n_cu > 0 ? n_cu : 256);
+    return 256 + backward_partial_bytes(M, K, N, n_cu > 0 ? n_cu : 256) + backward_gradA_bytes(M, K, N);
 }
 
 int amr_lut_gemm_backward(const float* gC, const uint8_t* A, const uint8_t* B, float* gA, float* gB,
@@ -212,7 +226,8 @@ int amr_lut_gemm_backward_ex(const float* gC, const uint8_t* A, const uint8_t* B
     const int n_cu = current_device_cus(&dev);
     if (n_cu <= 0) return fail(AMR_EINVAL, "no HIP device available");
     hipError_t e;
-    const size_t need = 256 + backward_partial_bytes(M, K, N, n_cu);
+    const size_t partial_bytes = backward_partial_bytes(M, K, N, n_cu);
+    const size_t need = 256 + partial_bytes + backward_gradA_bytes(M, K, N);
     void* ws = workspace;
     if (ws) {
         if (workspace_bytes < need) return fail(AMR_EWORKSPACE, "workspace of %zu bytes is smaller than the %zu required", workspace_bytes, need);
@@ -224,12 +239,17 @@ int amr_lut_gemm_backward_ex(const float* gC, const uint8_t* A, const uint8_t* B
     uint32_t* flags = reinterpret_cast<uint32_t*>(ws);
     float* partials = reinterpret_cast<float*>(reinterpret_cast<unsigned char*>(ws) + 256);
     const bool slab = amr::bwd_slab_applies(g, M, K, N);
-    if (slab && gB) {
+    const bool slab_a = gA && amr::gradA_slab_workspace_bytes(g, M, K, N) != 0 && ((uintptr_t)gC & 15) == 0;
+    if ((slab && gB) || slab_a) {
         e = hipMemsetAsync(flags, 0, 256, s);
         if (e != hipSuccess) return hip_fail(e, "hipMemsetAsync");
     }
     if (gA) {
-        e = amr::launch_gradA(gC, A, B, gA, lut_grad_a, g, M, K, N, scale, n_cu, s, nullptr, ga_rows_per_image);
+        if (slab_a)
+            e = amr::launch_gradA_slab(gC, A, B, gA, lut_grad_a, g, M, K, N, scale, n_cu, flags,
+                                       reinterpret_cast<unsigned char*>(ws) + 256 + partial_bytes, ga_rows_per_image, s);
+        else
+            e = amr::launch_gradA(gC, A, B, gA, lut_grad_a, g, M, K, N, scale, n_cu, s, nullptr, ga_rows_per_image);
         if (e != hipSuccess) return hip_fail(e, "gradA launch");
     }
     if (gB) {

@@ -150,7 +150,8 @@ def test_im2col_codes_rejects_wrong_shapes(ops):
         approx_ops.im2col_codes(x, torch.zeros(0, 3 * 81, dtype=torch.uint8, device="cuda"), (9, 9), 1, 0, 1)
 
 
-@pytest.mark.parametrize("M,K,N,L", [(192, 40, 24, 64), (150, 33, 10, 25), (4096, 64, 64, 1024), (6, 5, 3, 1)])
+@pytest.mark.parametrize("M,K,N,L", [(192, 40, 24, 64), (150, 33, 10, 25), (4096, 64, 64, 1024), (6, 5, 3, 1),
+                                     (8192, 32, 32, 1024), (9216, 48, 64, 256)])   # the last two: expanded-table gradA
 def test_backward_image_major_ga_equals_row_major(ops, oracle, golden_dir, M, K, N, L):
     import approx_ops
     self_ops, P = ops

@@ -241,7 +241,10 @@ def test_backward_large_m_masked_codes(lib, oracle):
 
 
 # K % 8 == 0, N % 64 == 0, M % 128 == 0 and M >= 4096: gradB runs on the expanded table held as halves (entries - 1024)
-HALF_SLAB_SHAPES = [(4096, 8, 64), (4224, 24, 128), (8192, 64, 64), (16384, 16, 192)]
+# (N % 32 == 0, K % 16 == 0 and M >= 8192: gradA runs on its own expanded table, 16 or 32 k per workgroup, also with a
+# ragged last row block)
+HALF_SLAB_SHAPES = [(4096, 8, 64), (4224, 24, 128), (8192, 64, 64), (16384, 16, 192), (8200, 48, 96), (9001, 64, 32),
+                    (4100, 32, 64)]
 
 
 @pytest.mark.parametrize("bits", [7, 6, 4])
