@@ -92,13 +92,13 @@ __device__ __forceinline__ void ga_wait4(u32x4 (&d)[4]) {
 }
 
 // ------------------------------------------------------------------------------------------ consume
-// grid (ceil(M / 512), K / KT), 512 threads, KT = 16 or 32 k per workgroup.  Requires M >= 64, N % 32 == 0,
+// grid ceil(M / 512) * K / KT workgroups, 512 threads, KT = 16 or 32 k per workgroup.  Requires M >= 64, N % 32 == 0,
 // K % KT == 0, M*K < 2^31.
 // rows_per_image = 0: gA row-major [M,K]; L > 0: image-major transposed gA[m / L][k][m % L].
 template <bool VEC, int kGaKT>
 __global__ __launch_bounds__(kGaWaves * 64, 2) void lutgemm_gradA_slab_kernel(
     const float* __restrict__ gC, const uint8_t* __restrict__ A, const u32x4* __restrict__ S, float* __restrict__ gA,
-    uint32_t* __restrict__ flags, int M, int K, int N, float scale, int rows_per_image) {
+    uint32_t* __restrict__ flags, int M, int K, int N, float scale, int rows_per_image, int row_blocks) {
     __shared__ __align__(16) unsigned char smem[2 * kGaChunkBytes];
     const int tid = threadIdx.x;
     const int wave = uniform(tid >> 6);
@@ -106,9 +106,18 @@ __global__ __launch_bounds__(kGaWaves * 64, 2) void lutgemm_gradA_slab_kernel(
     // A wave whose rows would stick out of M is shifted up so that all its rows exist; the rows it then
     // shares with the wave above are not stored twice (a wave entirely beyond M stores nothing but still
     // takes part in the copies and barriers).
-    const int m_first = (blockIdx.x * kGaWaves + wave) * 64;
+    // Workgroup order: 32 neighbouring row blocks, then all k groups, then the next 32 row blocks.  The workgroups
+    // in flight at one time then share both their slabs (same k group) and their rows of gC (same row block)
+    // in the caches; with all row blocks of one k group first, gC (re-read once per k group) came from HBM.
+    const int k_groups = K / kGaKT;
+    const int band = blockIdx.x / (32 * k_groups);                 // 32 row blocks x all k groups
+    const int band_rows = min(32, row_blocks - 32 * band);
+    const int in_band = blockIdx.x - band * 32 * k_groups;
+    const int k_group = in_band / band_rows;
+    const int row_block = 32 * band + (in_band - k_group * band_rows);
+    const int m_first = (row_block * kGaWaves + wave) * 64;
     const int m = min(m_first, M - 64) + lane;
-    const int k0 = blockIdx.y * kGaKT;
+    const int k0 = k_group * kGaKT;
     const int n_tiles = N / kGaCols;
     const int total = n_tiles * (kGaKT / kGaChunkK);           // chunks this workgroup walks: (tile, four k)
 
@@ -232,13 +241,13 @@ hipError_t launch_gradA_slab(const float* gC, const uint8_t* A, const uint8_t* B
     const dim3 block(kGaWaves * 64);
     const unsigned row_blocks = (unsigned)((M + rows_per_wg - 1) / rows_per_wg);
     if ((K % 32) == 0) {
-        const dim3 grid(row_blocks, K / 32);
-        if (vec) hipLaunchKernelGGL((lutgemm_gradA_slab_kernel<true, 32>), grid, block, 0, stream, gC, A, S4, gA, flags, M, K, N, scale, rows_per_image);
-        else hipLaunchKernelGGL((lutgemm_gradA_slab_kernel<false, 32>), grid, block, 0, stream, gC, A, S4, gA, flags, M, K, N, scale, rows_per_image);
+        const dim3 grid(row_blocks * (K / 32));
+        if (vec) hipLaunchKernelGGL((lutgemm_gradA_slab_kernel<true, 32>), grid, block, 0, stream, gC, A, S4, gA, flags, M, K, N, scale, rows_per_image, (int)row_blocks);
+        else hipLaunchKernelGGL((lutgemm_gradA_slab_kernel<false, 32>), grid, block, 0, stream, gC, A, S4, gA, flags, M, K, N, scale, rows_per_image, (int)row_blocks);
     } else {
-        const dim3 grid(row_blocks, K / 16);
-        if (vec) hipLaunchKernelGGL((lutgemm_gradA_slab_kernel<true, 16>), grid, block, 0, stream, gC, A, S4, gA, flags, M, K, N, scale, rows_per_image);
-        else hipLaunchKernelGGL((lutgemm_gradA_slab_kernel<false, 16>), grid, block, 0, stream, gC, A, S4, gA, flags, M, K, N, scale, rows_per_image);
+        const dim3 grid(row_blocks * (K / 16));
+        if (vec) hipLaunchKernelGGL((lutgemm_gradA_slab_kernel<true, 16>), grid, block, 0, stream, gC, A, S4, gA, flags, M, K, N, scale, rows_per_image, (int)row_blocks);
+        else hipLaunchKernelGGL((lutgemm_gradA_slab_kernel<false, 16>), grid, block, 0, stream, gC, A, S4, gA, flags, M, K, N, scale, rows_per_image, (int)row_blocks);
     }
     e = hipGetLastError();
     if (e != hipSuccess) return e;
