@@ -38,7 +38,7 @@ class ObserverBase(nn.Module):
 
     @torch.no_grad()
     def forward(self, input):
-        lo, hi = torch.min(input), torch.max(input)
+        lo, hi = torch.aminmax(input)
         if self.num_flag == 0:
             self.num_flag = 1
             self.min_val, self.max_val = lo, hi
@@ -74,8 +74,40 @@ def _scale_and_zero_point(observer, quant_max, eps):
     return scale, torch.round(observer.min_val / scale)
 
 
+class _ToCodesFn(torch.autograd.Function):
+    """clamp(round(x / scale - zp_neg), 0, quant_max) with straight-through rounding, one device pass each way
+    (same values and gradients as the torch expression in :func:`_to_codes`)."""
+
+    @staticmethod
+    def forward(ctx, x, scale, zp_neg, quant_max):
+        import approx_ops
+        xc = x.contiguous()
+        s, z = scale.detach().reshape(1).contiguous(), zp_neg.detach().reshape(1).contiguous()
+        codes = torch.empty_like(xc)
+        approx_ops.quantize_codes(xc, s, z, quant_max, codes)
+        ctx.save_for_backward(xc, s, z)
+        ctx.quant_max = quant_max
+        return codes
+
+    @staticmethod
+    def backward(ctx, g):
+        import approx_ops
+        xc, s, z = ctx.saved_tensors
+        gx = torch.empty_like(xc)
+        approx_ops.quantize_codes_backward(g.contiguous(), xc, s, z, ctx.quant_max, gx)
+        return gx, None, None, None
+
+
 def _to_codes(x, scale, zp_neg, quant_max):
     """Affine map to [0, quant_max] with straight-through rounding; returns integer-valued floats."""
+    if x.is_cuda and x.dtype == torch.float32 and scale.is_cuda and zp_neg.is_cuda:
+        return _ToCodesFn.apply(x, scale, zp_neg, float(quant_max))
+    affine = x / scale - zp_neg
+    return torch.clamp(affine - affine.detach() + torch.round(affine), 0, quant_max)
+
+
+def _to_codes_torch(x, scale, zp_neg, quant_max):
+    """The same map written with torch operators (what the reference's quantize_v2 composes)."""
     affine = x / scale - zp_neg
     return torch.clamp(affine - affine.detach() + torch.round(affine), 0, quant_max)
 
@@ -136,6 +168,61 @@ class QuantLinear(nn.Linear, _QuantParamsMixin):
 
     def quantize(self, x, s, zpn, qmax):
         return (_to_codes(x, s, zpn, qmax) + zpn) * s
+
+    def forward(self, input):
+        self._update_ranges(input)
+        input_fq = self.quantize(input, self.activation_scale, self.activation_zp_neg, self.activation_quant_max)
+        weight_fq = self.quantize(self.weight, self.weight_scale, self.weight_zp_neg, self.weight_quant_max)
+        return F.linear(input_fq, weight_fq, self.bias)
+
+
+class ApproxConv2d(nn.Conv2d, _QuantParamsMixin):
+    """Convolution whose code products come from the approximate-multiplier table
+    (reference ``app_layers.py:116-185``)."""
+
+    def __init__(self, in_channels, out_channels, kernel_size, stride=1, padding=0, dilation=1, groups=1, bias=True,
+                 padding_mode="zeros", a_bits=8, w_bits=8, use_ste_gradient=False):
+        super().__init__(in_channels, out_channels, kernel_size, stride, padding, dilation, groups, bias, padding_mode)
+        self._init_quant(a_bits, w_bits)
+        self.conv2d_op = self_ops.approx_conv2d_baseline_op if use_ste_gradient else self_ops.approx_conv2d_op
+        self.reference_zero_point_terms = False     # True: evaluate the three correction terms as full convolutions
+
+    def quantize_v2(self, x, s, zpn, qmax):
+        return _to_codes(x, s, zpn, qmax)
+
+    def _zero_point_terms(self, x_codes, w_codes, conv_args):
+        """conv(X,Zw) + conv(Za,W) + conv(Za,Zw) without the three full convolutions: a convolution with a
+        constant operand factorises, conv(X, Zw*1) = Zw * box-sum of X over channels and window (one
+        output channel), conv(Za*1, W) = Za * (response of W to an all-ones image, batch of one), and
+        conv(Za*1, Zw*1) = Za*Zw*C * (number of taps inside the image).  All quantities are integer valued,
+        so as long as they stay below 2^24 the result is bit-identical to the literal form; autograd sees
+        ordinary torch ops and yields the same gradients for the codes."""
+        z_a, z_w = self.activation_zp_neg, self.weight_zp_neg
+        _, cin, h, w = x_codes.shape
+        cout, kh, kw = w_codes.shape[0], w_codes.shape[2], w_codes.shape[3]
+        s, p, d = conv_args["stride"], conv_args["padding"], conv_args["dilation"]
+        mask = self._tap_mask(h, w, kh, kw, s, p, d, x_codes.dtype, x_codes.device)               # [kh*kw, oh*ow]
+        oh = (h + 2 * p[0] - d[0] * (kh - 1) - 1) // s[0] + 1
+        ow = mask.shape[1] // oh
+        xs = x_codes.sum(dim=1, keepdim=True)
+        if tuple(d) == (1, 1) and 2 * p[0] <= kh and 2 * p[1] <= kw:
+            # box sum with zero padding (no single-channel convolution: the library runs those image by image)
+            x_sum = F.avg_pool2d(xs, (kh, kw), stride=s, padding=p, divisor_override=1)              # [B,1,oh,ow]
+        else:
+            x_sum = F.conv2d(xs, torch.ones(1, 1, kh, kw, dtype=xs.dtype, device=xs.device), **conv_args)
+        w_resp = (w_codes.sum(dim=1).reshape(cout, kh * kw) @ mask).view(1, cout, oh, ow)           # [1,N,oh,ow]
+        taps = (mask.sum(dim=0) * float(cin)).view(1, 1, oh, ow)
+        return z_w * x_sum + z_a * w_resp + (z_a * z_w) * taps
+
+    def _tap_mask(self, h, w, kh, kw, stride, padding, dilation, dtype, device):
+        """mask[i*kw+j, l] = 1 where tap (i,j) of output position l lies inside the h x w image (constant per
+        geometry, cached)."""
+        key = (h, w, kh, kw, tuple(stride), tuple(padding), tuple(dilation), dtype, str(device))
+        cache = self.__dict__.setdefault("_tap_masks", {})
+        if key not in cache:
+            ones = torch.ones(1, 1, h, w, dtype=dtype, device=device)
+            cache[key] = F.unfold(ones, (kh, kw), dilation=dilation, padding=padding, stride=stride)[0]
+        return cache[key]
 
     def forward(self, input):
         self._update_ranges(input)

@@ -38,6 +38,8 @@ _lib.amr_lut_gemm_forward.argtypes = [_vp, _vp, _vp, _vp, _i64, _i, _i, _i, _vp]
 _lib.amr_lut_gemm_backward.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i, _i, _i, _vp, _sz, _vp]
 _lib.amr_lut_gemm_backward_ex.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i, _i, _i, _i, _vp, _sz, _vp]
 _lib.amr_im2col_u8_f32.argtypes = [_vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp]
+_lib.amr_quantize_codes_f32.argtypes = [_vp, _vp, _vp, ctypes.c_float, _vp, _i64, _vp]
+_lib.amr_quantize_codes_backward_f32.argtypes = [_vp, _vp, _vp, _vp, ctypes.c_float, _vp, _i64, _vp]
 _lib.amr_lut_gemm_backward_workspace_bytes.argtypes = [_i, _i, _i]
 _lib.amr_lut_gemm_backward_workspace_bytes.restype = _sz
 _lib.amr_acc_gemm_forward_fp32.argtypes = [_vp, _vp, _vp, _i, _i, _i, _vp]
@@ -178,6 +180,37 @@ def im2col_codes(x_tensor, a_tensor, kernel_size, stride, padding, dilation):
         rc = _lib.amr_im2col_u8_f32(x_tensor.data_ptr(), a_tensor.data_ptr(), Bn, C, H, W, kh, kw, stride, padding, dilation,
                                     _stream_ptr(dev))
     _raise_for(rc, "im2col_codes")
+
+
+def quantize_codes(x_tensor, scale_tensor, zp_neg_tensor, quant_max, codes_tensor):
+    """codes = clamp(round(x / scale - zp_neg), 0, quant_max) in one pass (the forward value of the reference's
+    quantize_v2, micronet+/app_layers.py:147-160); scale and zp_neg are one-element float32 device tensors."""
+    for t, name in ((x_tensor, "x_tensor"), (scale_tensor, "scale_tensor"), (zp_neg_tensor, "zp_neg_tensor"), (codes_tensor, "codes_tensor")):
+        _check_input(t, torch.float32, name)
+    _check(scale_tensor.numel() == 1 and zp_neg_tensor.numel() == 1, "scale and zp_neg must hold one element")
+    _check(codes_tensor.shape == x_tensor.shape, "codes_tensor must have the shape of x_tensor")
+    dev = x_tensor.device
+    _check(all(t.device == dev for t in (scale_tensor, zp_neg_tensor, codes_tensor)), "All tensors should be on the same device")
+    with torch.cuda.device(dev):
+        rc = _lib.amr_quantize_codes_f32(x_tensor.data_ptr(), scale_tensor.data_ptr(), zp_neg_tensor.data_ptr(), float(quant_max),
+                                         codes_tensor.data_ptr(), x_tensor.numel(), _stream_ptr(dev))
+    _raise_for(rc, "quantize_codes")
+
+
+def quantize_codes_backward(g_tensor, x_tensor, scale_tensor, zp_neg_tensor, quant_max, gx_tensor):
+    """gx = g / scale where round(x / scale - zp_neg) lies in [0, quant_max], else 0 (straight-through rounding)."""
+    for t, name in ((g_tensor, "g_tensor"), (x_tensor, "x_tensor"), (scale_tensor, "scale_tensor"), (zp_neg_tensor, "zp_neg_tensor"),
+                    (gx_tensor, "gx_tensor")):
+        _check_input(t, torch.float32, name)
+    _check(scale_tensor.numel() == 1 and zp_neg_tensor.numel() == 1, "scale and zp_neg must hold one element")
+    _check(g_tensor.shape == x_tensor.shape and gx_tensor.shape == x_tensor.shape, "g, x and gx must have the same shape")
+    dev = x_tensor.device
+    _check(all(t.device == dev for t in (g_tensor, scale_tensor, zp_neg_tensor, gx_tensor)), "All tensors should be on the same device")
+    with torch.cuda.device(dev):
+        rc = _lib.amr_quantize_codes_backward_f32(g_tensor.data_ptr(), x_tensor.data_ptr(), scale_tensor.data_ptr(),
+                                                  zp_neg_tensor.data_ptr(), float(quant_max), gx_tensor.data_ptr(), x_tensor.numel(),
+                                                  _stream_ptr(dev))
+    _raise_for(rc, "quantize_codes_backward")
 
 
 def lds_gather_probe(pattern=0, waves_per_cu=16, iters=4000):

@@ -26,6 +26,10 @@ size_t gradA_slab_workspace_bytes(const LutGeom& g, int M, int K, int N);
 hipError_t launch_gradA_slab(const float* gC, const uint8_t* A, const uint8_t* B, float* gA, const int16_t* lut,
                              const LutGeom& g, int M, int K, int N, float scale, int n_cu, uint32_t* flags, void* S,
                              int rows_per_image, hipStream_t stream);
+hipError_t launch_quantize_codes(const float* x, const float* scale, const float* zp_neg, float qmax, float* codes, size_t n,
+                                 hipStream_t stream);
+hipError_t launch_quantize_codes_backward(const float* g, const float* x, const float* scale, const float* zp_neg, float qmax,
+                                          float* gx, size_t n, hipStream_t stream);
 hipError_t launch_im2col_u8_f32(const float* x, uint8_t* A, int B, int C, int H, int W, int kh, int kw, int stride, int pad,
                                 int dil, int oh, int ow, hipStream_t stream);
 bool bwd_slab_applies(const LutGeom& g, int M, int K, int N);
@@ -277,6 +281,26 @@ int amr_im2col_u8_f32(const float* x, uint8_t* A, int B, int C, int H, int W, in
     if (!x || !A) return fail(AMR_EINVAL, "null pointer argument");
     hipError_t e = amr::launch_im2col_u8_f32(x, A, B, C, H, W, kh, kw, stride, pad, dil, oh, ow, reinterpret_cast<hipStream_t>(stream));
     return e == hipSuccess ? AMR_OK : hip_fail(e, "im2col launch");
+}
+
+int amr_quantize_codes_f32(const float* x, const float* scale, const float* zp_neg, float qmax, float* codes, int64_t n,
+                           void* stream) {
+    if (n < 0 || !(qmax >= 0.f)) return fail(AMR_EINVAL, "bad element count or code range");
+    if (n == 0) return AMR_OK;
+    if (n >= ((int64_t)1 << 40)) return fail(AMR_EUNSUPPORTED, "more than 2^40 elements");
+    if (!x || !scale || !zp_neg || !codes) return fail(AMR_EINVAL, "null pointer argument");
+    hipError_t e = amr::launch_quantize_codes(x, scale, zp_neg, qmax, codes, (size_t)n, reinterpret_cast<hipStream_t>(stream));
+    return e == hipSuccess ? AMR_OK : hip_fail(e, "quantize launch");
+}
+
+int amr_quantize_codes_backward_f32(const float* g, const float* x, const float* scale, const float* zp_neg, float qmax,
+                                    float* gx, int64_t n, void* stream) {
+    if (n < 0 || !(qmax >= 0.f)) return fail(AMR_EINVAL, "bad element count or code range");
+    if (n == 0) return AMR_OK;
+    if (n >= ((int64_t)1 << 40)) return fail(AMR_EUNSUPPORTED, "more than 2^40 elements");
+    if (!g || !x || !scale || !zp_neg || !gx) return fail(AMR_EINVAL, "null pointer argument");
+    hipError_t e = amr::launch_quantize_codes_backward(g, x, scale, zp_neg, qmax, gx, (size_t)n, reinterpret_cast<hipStream_t>(stream));
+    return e == hipSuccess ? AMR_OK : hip_fail(e, "quantize backward launch");
 }
 
 int amr_acc_gemm_forward_fp32(const float* A, const float* B, float* C, int M, int K, int N, void* stream) {

@@ -1,0 +1,84 @@
+// Quantiser of the layer in front of the LUT GEMM, gfx950: real values -> integer codes in one pass.
+//
+// Forward: codes = clamp(round(x / scale - zp_neg), 0, qmax), the value of the reference's quantize_v2 with
+// its straight-through rounding (micronet+/app_layers.py:147-160: "x / s - zpn", Round.apply, clamp); scale and
+// zp_neg are read from device memory (they come out of the observers without a host round trip).
+// Backward of that expression: the rounding passes the gradient through, the clamp passes it where the
+// rounded value lies inside [0, qmax], and x / scale contributes 1 / scale:  gx = inside ? g / scale : 0.
+// Both kernels are a single streaming pass (16 bytes per lane and access); the tail is done element-wise.
+#include "amr_common.h"
+
+namespace amr {
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ float quant_code(float x, float s, float zp, float qmax, bool* inside) {
+    const float r = rintf(x / s - zp);          // round half to even, as torch.round
+    *inside = (r >= 0.f) && (r <= qmax);
+    return fminf(fmaxf(r, 0.f), qmax);
+}
+
+__global__ __launch_bounds__(256) void quantize_codes_kernel(const float* __restrict__ x, const float* __restrict__ scale,
+                                                             const float* __restrict__ zp_neg, float qmax,
+                                                             float* __restrict__ codes, size_t n, int vec) {
+    const float s = *scale, zp = *zp_neg;
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    bool in;
+    if (vec) {
+        if (4 * i + 3 < n) {
+            const f32x4 v = reinterpret_cast<const f32x4*>(x)[i];
+            f32x4 o = {quant_code(v.x, s, zp, qmax, &in), quant_code(v.y, s, zp, qmax, &in), quant_code(v.z, s, zp, qmax, &in),
+                       quant_code(v.w, s, zp, qmax, &in)};
+            reinterpret_cast<f32x4*>(codes)[i] = o;
+        } else {
+            for (size_t j = 4 * i; j < n; ++j) codes[j] = quant_code(x[j], s, zp, qmax, &in);
+        }
+    } else if (i < n) {
+        codes[i] = quant_code(x[i], s, zp, qmax, &in);
+    }
+}
+
+__global__ __launch_bounds__(256) void quantize_codes_backward_kernel(const float* __restrict__ g, const float* __restrict__ x,
+                                                                      const float* __restrict__ scale,
+                                                                      const float* __restrict__ zp_neg, float qmax,
+                                                                      float* __restrict__ gx, size_t n, int vec) {
+    const float s = *scale, zp = *zp_neg;
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    auto one = [&](float gv, float xv) {
+        bool in;
+        (void)quant_code(xv, s, zp, qmax, &in);
+        return in ? gv / s : 0.f;
+    };
+    if (vec) {
+        if (4 * i + 3 < n) {
+            const f32x4 gv = reinterpret_cast<const f32x4*>(g)[i];
+            const f32x4 xv = reinterpret_cast<const f32x4*>(x)[i];
+            f32x4 o = {one(gv.x, xv.x), one(gv.y, xv.y), one(gv.z, xv.z), one(gv.w, xv.w)};
+            reinterpret_cast<f32x4*>(gx)[i] = o;
+        } else {
+            for (size_t j = 4 * i; j < n; ++j) gx[j] = one(g[j], x[j]);
+        }
+    } else if (i < n) {
+        gx[i] = one(g[i], x[i]);
+    }
+}
+
+hipError_t launch_quantize_codes(const float* x, const float* scale, const float* zp_neg, float qmax, float* codes, size_t n,
+                                 hipStream_t stream) {
+    const int vec = ((((uintptr_t)x) | ((uintptr_t)codes)) & 15) == 0;
+    const size_t items = vec ? (n + 3) / 4 : n;
+    hipLaunchKernelGGL(quantize_codes_kernel, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, stream, x, scale, zp_neg, qmax,
+                       codes, n, vec);
+    return hipGetLastError();
+}
+
+hipError_t launch_quantize_codes_backward(const float* g, const float* x, const float* scale, const float* zp_neg, float qmax,
+                                          float* gx, size_t n, hipStream_t stream) {
+    const int vec = ((((uintptr_t)x) | ((uintptr_t)g) | ((uintptr_t)gx)) & 15) == 0;
+    const size_t items = vec ? (n + 3) / 4 : n;
+    hipLaunchKernelGGL(quantize_codes_backward_kernel, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, stream, g, x, scale,
+                       zp_neg, qmax, gx, n, vec);
+    return hipGetLastError();
+}
+
+}  // namespace amr

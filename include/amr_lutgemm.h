@@ -113,6 +113,18 @@ int amr_im2col_u8_f32(const float *x, uint8_t *A, int B, int C, int H, int W, in
                       int dil, void *stream);
 
 /*
+ * Quantiser in front of the LUT GEMM: codes[i] = clamp(round(x[i] / *scale - *zp_neg), 0, qmax) as float32,
+ * round half to even; scale and zp_neg are device pointers to one float each.  One pass instead of the
+ * divide / subtract / round / straight-through / clamp chain of the reference's quantize_v2
+ * (micronet+/app_layers.py:147-160).  The backward entry point gives the gradient of that expression with
+ * straight-through rounding: gx[i] = g[i] / *scale where the rounded value lies in [0, qmax], else 0.
+ */
+int amr_quantize_codes_f32(const float *x, const float *scale, const float *zp_neg, float qmax, float *codes,
+                           int64_t n, void *stream);
+int amr_quantize_codes_backward_f32(const float *g, const float *x, const float *scale, const float *zp_neg,
+                                    float qmax, float *gx, int64_t n, void *stream);
+
+/*
  * Accurate fp32 GEMM  C = A . B  (row-major), kept for API parity only.
  * Replaces acc_gemm_forward_fp32_gpu (self_ops/src/approx_gemm_forward.cu:494-571), bound as
  * approx_ops.acc_gemm_forward_fp32 (self_ops/src/op_register.cpp:18).

@@ -224,6 +224,32 @@ def test_conv_op_rejects_bias_and_groups(ops):
         self_ops.approx_conv2d_op(x, w, None, (1, 1), (1, 1), (1, 1), 2)
 
 
+@pytest.mark.parametrize("shape", [(7,), (4, 3, 5, 5), (64, 16, 32, 32), (1023,), (2, 1026)])
+def test_fused_quantiser_equals_torch_expression(ops, shape):
+    """The one-pass quantiser against the operator chain the reference composes (app_layers.py:147-160):
+    bit-identical codes and gradients, including values that land exactly on .5 and outside the range."""
+    import app_layers
+    print("quantiser", shape, flush=True)
+    g = torch.Generator(device="cuda").manual_seed(3)
+    x = (torch.randn(shape, device="cuda", generator=g) * 3).requires_grad_()
+    with torch.no_grad():
+        x.view(-1)[::5] = (torch.arange(x.numel(), device="cuda")[::5] % 200 - 30).float() * 0.05 + 0.025   # ties after scaling
+    scale, zp = torch.tensor([0.05], device="cuda"), torch.tensor([-17.0], device="cuda")
+    x2 = x.detach().clone().requires_grad_()
+    y = app_layers._to_codes(x, scale, zp, 127.0)
+    y2 = app_layers._to_codes_torch(x2, scale, zp, 127.0)
+    assert torch.equal(y, y2) and y.min() >= 0 and y.max() <= 127
+    gy = torch.randn(shape, device="cuda", generator=g)
+    y.backward(gy)
+    y2.backward(gy)
+    assert torch.equal(x.grad, x2.grad)
+    assert (x.grad == 0).any() and (x.grad != 0).any()
+    # non-contiguous input
+    if len(shape) == 4:
+        xt = x.detach().transpose(1, 3)
+        assert torch.equal(app_layers._to_codes(xt, scale, zp, 127.0), app_layers._to_codes_torch(xt, scale, zp, 127.0))
+
+
 def test_acc_gemm_op(ops):
     self_ops, P = ops
     a = torch.randn(70, 40, device="cuda", requires_grad=True)
