@@ -12,7 +12,7 @@
 namespace amr {
 hipError_t launch_fwd(const uint8_t* A, const uint8_t* B, uint32_t* C, const uint16_t* lut, const LutGeom& g, int M,
                       int K, int N, int n_cu, hipStream_t stream);
-size_t fwd_slab_workspace_bytes(const LutGeom& g, int M, int K, int N);
+size_t fwd_slab_workspace_bytes(const LutGeom& g, int M, int K, int N, bool force);
 hipError_t launch_fwd_slab(const uint8_t* A, const uint8_t* B, uint32_t* C, const uint16_t* lut, const LutGeom& g,
                            int M, int K, int N, int n_cu, void* workspace, hipStream_t stream);
 size_t gradB_workspace_bytes(int M, int K, int N, int n_cu, int* splits_out);
@@ -22,7 +22,7 @@ hipError_t launch_gradB(const float* gC, const uint8_t* A, const uint8_t* B, flo
 hipError_t launch_gradA(const float* gC, const uint8_t* A, const uint8_t* B, float* gA, const int16_t* lut,
                         const LutGeom& g, int M, int K, int N, float scale, int n_cu, hipStream_t stream,
                         const uint32_t* gate = nullptr, int rows_per_image = 0);
-size_t gradA_slab_workspace_bytes(const LutGeom& g, int M, int K, int N);
+size_t gradA_slab_workspace_bytes(const LutGeom& g, int M, int K, int N, bool force);
 hipError_t launch_gradA_slab(const float* gC, const uint8_t* A, const uint8_t* B, float* gA, const int16_t* lut,
                              const LutGeom& g, int M, int K, int N, float scale, int n_cu, uint32_t* flags, void* S,
                              int rows_per_image, hipStream_t stream);
@@ -118,6 +118,16 @@ int amr_lut_geometry(int bits, int* rows, int* cols, int64_t* elem_num) {
     return AMR_OK;
 }
 
+// Process-wide switch (diagnostics, tests, benchmarks): 0 sends every call to the direct gather kernels, 1 picks by
+// problem size, 2 takes the expanded-table kernels wherever the shape allows (also where they are slower).
+static int g_expanded_kernels = 1;
+
+int amr_set_expanded_table_kernels(int mode) {
+    const int old = g_expanded_kernels;
+    g_expanded_kernels = mode <= 0 ? 0 : (mode >= 2 ? 2 : 1);
+    return old;
+}
+
 int amr_bits_from_lut_elems(int64_t lut_elems) {
     amr::LutGeom g;
     if (!amr::lut_geom_from_elems(lut_elems, &g))
@@ -128,7 +138,7 @@ int amr_bits_from_lut_elems(int64_t lut_elems) {
 size_t amr_lut_gemm_forward_workspace_bytes(int64_t lut_elems, int M, int K, int N) {
     amr::LutGeom g;
     if (M <= 0 || K <= 0 || N <= 0 || !amr::lut_geom_from_elems(lut_elems, &g)) return 0;
-    return amr::fwd_slab_workspace_bytes(g, M, K, N);
+    return g_expanded_kernels ? amr::fwd_slab_workspace_bytes(g, M, K, N, g_expanded_kernels == 2) : 0;
 }
 
 int amr_lut_gemm_forward_ws(const uint8_t* A, const uint8_t* B, uint32_t* C, const uint16_t* lut, int64_t lut_elems,
@@ -148,7 +158,7 @@ int amr_lut_gemm_forward_ws(const uint8_t* A, const uint8_t* B, uint32_t* C, con
     int dev = 0;
     const int n_cu = current_device_cus(&dev);
     if (n_cu <= 0) return fail(AMR_EINVAL, "no HIP device available");
-    const size_t need = amr::fwd_slab_workspace_bytes(g, M, K, N);
+    const size_t need = g_expanded_kernels ? amr::fwd_slab_workspace_bytes(g, M, K, N, g_expanded_kernels == 2) : 0;
     hipError_t e;
     if (need > 0) {
         void* ws = workspace;
@@ -184,9 +194,10 @@ static size_t backward_partial_bytes(int M, int K, int N, int n_cu) {
 // Size of the expanded table of gradA for 7-bit tables (the widest the expanded-table kernels take); a query
 // by shape alone cannot know the table width, so the scratch is sized for it.
 static size_t backward_gradA_bytes(int M, int K, int N) {
+    if (!g_expanded_kernels) return 0;
     amr::LutGeom g7;
     amr::lut_geom_from_bits(7, &g7);
-    return amr::gradA_slab_workspace_bytes(g7, M, K, N);
+    return amr::gradA_slab_workspace_bytes(g7, M, K, N, g_expanded_kernels == 2);
 }
 
 size_t amr_lut_gemm_backward_workspace_bytes(int M, int K, int N) {
@@ -242,8 +253,8 @@ int amr_lut_gemm_backward_ex(const float* gC, const uint8_t* A, const uint8_t* B
     }
     uint32_t* flags = reinterpret_cast<uint32_t*>(ws);
     float* partials = reinterpret_cast<float*>(reinterpret_cast<unsigned char*>(ws) + 256);
-    const bool slab = amr::bwd_slab_applies(g, M, K, N);
-    const bool slab_a = gA && amr::gradA_slab_workspace_bytes(g, M, K, N) != 0 && ((uintptr_t)gC & 15) == 0;
+    const bool slab = g_expanded_kernels && amr::bwd_slab_applies(g, M, K, N);
+    const bool slab_a = g_expanded_kernels && gA && amr::gradA_slab_workspace_bytes(g, M, K, N, g_expanded_kernels == 2) != 0 && ((uintptr_t)gC & 15) == 0;
     if ((slab && gB) || slab_a) {
         e = hipMemsetAsync(flags, 0, 256, s);
         if (e != hipSuccess) return hip_fail(e, "hipMemsetAsync");

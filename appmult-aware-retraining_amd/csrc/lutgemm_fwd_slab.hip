@@ -351,11 +351,14 @@ hipError_t launch_fwd_gated(const uint8_t* A, const uint8_t* B, uint32_t* C, con
 
 // ------------------------------------------------------------------------------------------ host
 // Workspace layout: [256 B flags][E].  Returns 0 when the expanded-table path does not apply.
-size_t fwd_slab_workspace_bytes(const LutGeom& g, int M, int K, int N) {
+size_t fwd_slab_workspace_bytes(const LutGeom& g, int M, int K, int N, bool force) {
     // Worth it when the 2^b/M expansion overhead is small and K is long enough to amortise the extra
     // launches (measured cross-over on MI355X: K around 512).
     // (K % 4 == 0: the codes of A are fetched four and sixteen at a time)
     if (g.bits > 7 || M < 2048 || K < 512 || (K & 3) != 0 || (size_t)M * K >= (1ull << 31)) return 0;
+    // below about 1.6e9 multiply-adds the extra launches (flags, expansion, second flavour, gated fall-back) cost
+    // more than the faster kernel gains (measured cross-over on MI355X between 1.2e9 and 2.4e9)
+    if (!force && (size_t)M * K * N < (3ull << 29)) return 0;
     const size_t n_tiles = (N + kSlabCols - 1) / kSlabCols;
     const size_t k_quads = ((size_t)K + 3) / 4;
     return 256 + n_tiles * k_quads * kSlabChunkBytes;

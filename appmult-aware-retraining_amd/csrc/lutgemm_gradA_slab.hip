@@ -219,9 +219,9 @@ hipError_t launch_gradA(const float* gC, const uint8_t* A, const uint8_t* B, flo
                         const uint32_t* gate, int rows_per_image);
 
 // Bytes of the expanded table S, or 0 when the expanded-table gradA does not apply.
-size_t gradA_slab_workspace_bytes(const LutGeom& g, int M, int K, int N) {
+size_t gradA_slab_workspace_bytes(const LutGeom& g, int M, int K, int N, bool force) {
     // (below about 8192 rows the expansion, 2^b / M of the work but all of it HBM writes, costs more than it saves)
-    if (g.bits > 7 || M < 8192 || (N % kGaCols) != 0 || (K % kGaKTmin) != 0 || (size_t)M * K >= (1ull << 31)) return 0;
+    if (g.bits > 7 || M < (force ? 2048 : 8192) || (N % kGaCols) != 0 || (K % kGaKTmin) != 0 || (size_t)M * K >= (1ull << 31)) return 0;
     return (size_t)(N / kGaCols) * K * kGaSlabBytes;
 }
 

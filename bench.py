@@ -41,6 +41,10 @@ LDS_GATHER_PEAK = 256 * 2.4e9 * 32      # gathers/s: CUs x peak clock x conflict
 HBM_PEAK = 8.0e12
 
 
+# measured on MI355X with the counters named above, bytes per conv2_x launch (read + written)
+MEASURED_TRAFFIC_CONV2X = {"forward": (1584 + 72) * 2**20, "gradA": (1884 + 576) * 2**20, "gradB": (2141 + 1) * 2**20}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -216,7 +220,11 @@ def main():
         "frac_of_lds_gather_roofline": rate / LDS_GATHER_PEAK,
         "kernel_ms_per_step": {k: round(v, 4) for k, v in kernels.items()},
         "roofline": {"bound": "lds", "kernel": dominant, "achieved": dom_rate / 1e9, "peak": LDS_GATHER_PEAK / 1e9,
-                     "unit": "Ggather/s", "frac": dom_rate / LDS_GATHER_PEAK, "traffic": None,
+                     "unit": "Ggather/s", "frac": dom_rate / LDS_GATHER_PEAK,
+                     # bytes the L2s fetched + wrote for the conv2_x launch of that kernel kind (rocprofv3 FETCH_SIZE x 2.00,
+                     # WRITE_SIZE x 1.00 against plain copies; profiles/conv2x_hbm_traffic.md), beside its algorithmic bytes
+                     "traffic": MEASURED_TRAFFIC_CONV2X[dominant],
+                     "traffic_launch": "conv2_x (M=262144,K=576,N=64)", "traffic_algorithmic": hbm_bytes(dominant, 262144, 576, 64),
                      "avg_launch_ms": dom_ms / launches,
                      "hbm": {"achieved": dom_bytes / (dom_ms * 1e-3) / 1e9, "peak": HBM_PEAK / 1e9, "unit": "GB/s",
                              "frac": dom_bytes / (dom_ms * 1e-3) / HBM_PEAK},

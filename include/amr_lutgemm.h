@@ -113,6 +113,16 @@ int amr_im2col_u8_f32(const float *x, uint8_t *A, int B, int C, int H, int W, in
                       int dil, void *stream);
 
 /*
+ * Process-wide switch for diagnostics, tests and benchmarks.  mode 0 sends every later call to the direct
+ * gather kernels (the formulation of the reference's kernels, approx_gemm_forward.cu:45-229); 1 (the default)
+ * lets the library pick by problem size; 2 takes the expanded-table kernels wherever the shape allows, also
+ * where they are slower.  Returns the previous mode.  Results are the same in every mode (forward bit-exact,
+ * backward to summation order); the workspace size queries answer for the mode in force.  No counterpart in
+ * the reference.
+ */
+int amr_set_expanded_table_kernels(int mode);
+
+/*
  * Quantiser in front of the LUT GEMM: codes[i] = clamp(round(x[i] / *scale - *zp_neg), 0, qmax) as float32,
  * round half to even; scale and zp_neg are device pointers to one float each.  One pass instead of the
  * divide / subtract / round / straight-through / clamp chain of the reference's quantize_v2

@@ -32,7 +32,11 @@ def lib():
     L.amr_lut_gemm_backward_workspace_bytes.argtypes = [i, i, i]
     L.amr_lut_gemm_backward_workspace_bytes.restype = sz
     L.amr_acc_gemm_forward_fp32.argtypes = [vp, vp, vp, i, i, i, vp]
-    return L
+    # mode 2: the expanded-table kernels wherever the shape allows, so that the test sizes (small next to the sizes
+    # at which the library would pick them by itself) exercise them; mode 0 / 1 have tests of their own below
+    L.amr_set_expanded_table_kernels(2)
+    yield L
+    L.amr_set_expanded_table_kernels(1)
 
 
 def dev(x):
@@ -327,6 +331,42 @@ def test_backward_deterministic_and_skippable_outputs(lib, oracle):
                                      t.numel(), 3000, 64, 64, None, 0, None) == 0
     torch.cuda.synchronize()
     assert (gb.cpu().numpy() == r1[1]).all()
+
+
+@pytest.mark.parametrize("shape", [(2048, 512, 64), (4096, 640, 300), (8200, 48, 96), (5000, 130, 65)])
+def test_direct_kernels_at_large_m(lib, oracle, shape):
+    """Mode 0: the direct gather kernels on shapes that otherwise take the expanded-table kernels."""
+    print("direct kernels, large M", shape, flush=True)
+    M, K, N = shape
+    rng, A, B, T = rand_case(hash((shape, "d")) % 2**32, M, K, N, 7)
+    flat = oracle.pack_table(T, 7, np.uint16)
+    la = oracle.pack_table(rng.integers(-1024, 3073, (128, 128)), 7, np.int16)
+    lb = oracle.pack_table(rng.integers(-1024, 3073, (128, 128)), 7, np.int16)
+    g = rng.standard_normal((M, N)).astype(np.float32)
+    assert lib.amr_set_expanded_table_kernels(0) == 2
+    try:
+        assert lib.amr_lut_gemm_forward_workspace_bytes(flat.size, M, K, N) == 0
+        c0 = gpu_forward(lib, A, B, flat)
+        r0 = gpu_backward(lib, g, A, B, la, lb)
+    finally:
+        lib.amr_set_expanded_table_kernels(2)
+    assert (c0 == oracle.forward_c(A, B, flat, 7)).all()
+    check_backward(oracle, r0, g, A, B, la, lb, 7)
+    assert (gpu_forward(lib, A, B, flat) == c0).all()            # expanded-table kernels: same bits
+
+
+def test_default_mode_picks_kernels_by_problem_size(lib, oracle):
+    print("kernel selection by size", flush=True)
+    assert lib.amr_set_expanded_table_kernels(1) == 2
+    try:
+        # configs[1]-sized GEMM: too small for the expanded forward table to pay; a conv2_x-sized one is not
+        assert lib.amr_lut_gemm_forward_workspace_bytes(17408, 4096, 576, 64) == 0
+        assert lib.amr_lut_gemm_forward_workspace_bytes(17408, 262144, 576, 64) == 256 + 2 * 144 * 32768
+        rng, A, B, T = rand_case(5, 4096, 576, 64, 7)
+        flat = oracle.pack_table(T, 7, np.uint16)
+        assert (gpu_forward(lib, A, B, flat) == oracle.forward_c(A, B, flat, 7)).all()
+    finally:
+        lib.amr_set_expanded_table_kernels(2)
 
 
 def test_accgemm_matches_torch(lib):
