@@ -128,34 +128,40 @@ def approx_gemm_backward(gc_tensor, a_tensor, b_tensor, ga_tensor, gb_tensor, lu
     _check_input(gc_tensor, torch.float32, "gc_tensor")
     _check_input(a_tensor, torch.uint8, "a_tensor")
     _check_input(b_tensor, torch.uint8, "b_tensor")
-    _check_input(ga_tensor, torch.float32, "ga_tensor")
-    _check_input(gb_tensor, torch.float32, "gb_tensor")
+    # ga_tensor / gb_tensor may be None (an extension): that gradient is then not computed
+    _check(ga_tensor is not None or gb_tensor is not None, "ga_tensor and gb_tensor must not both be None")
+    if ga_tensor is not None:
+        _check_input(ga_tensor, torch.float32, "ga_tensor")
+    if gb_tensor is not None:
+        _check_input(gb_tensor, torch.float32, "gb_tensor")
     _check_input(lut_grad_a_tensor, torch.int16, "lut_grad_a_tensor")
     _check_input(lut_grad_b_tensor, torch.int16, "lut_grad_b_tensor")
     L = int(ga_rows_per_image)
-    _check(all(t.dim() == 2 for t in (gc_tensor, a_tensor, b_tensor, gb_tensor)), "gc, a, b and gb must be 2-D")
+    _check(all(t.dim() == 2 for t in (gc_tensor, a_tensor, b_tensor)) and (gb_tensor is None or gb_tensor.dim() == 2), "gc, a, b and gb must be 2-D")
     M, K = a_tensor.shape
     N = b_tensor.size(1)
     _check(gc_tensor.size(0) == M and gc_tensor.size(1) == N, f"gc_tensor's shape should be {M} x {N}")
     _check(K == b_tensor.size(0), f"b_tensor's shape should be {K} x {N}")
+    _check(L >= 0, "ga_rows_per_image must not be negative")
     if L > 0:
         _check(M % L == 0, f"ga_rows_per_image={L} must divide {M}")
+    if ga_tensor is not None and L > 0:
         _check(tuple(ga_tensor.shape) == (M // L, K, L), f"ga_tensor's shape should be {M // L} x {K} x {L}")
-    else:
-        _check(L == 0, "ga_rows_per_image must not be negative")
+    elif ga_tensor is not None:
         _check(ga_tensor.dim() == 2 and ga_tensor.size(0) == M and ga_tensor.size(1) == K, f"ga_tensor's shape should be {M} x {K}")
-    _check(gb_tensor.size(0) == K and gb_tensor.size(1) == N, f"gb_tensor's shape should be {K} x {N}")
+    _check(gb_tensor is None or (gb_tensor.size(0) == K and gb_tensor.size(1) == N), f"gb_tensor's shape should be {K} x {N}")
     _lut_len_check(lut_grad_a_tensor, "lut_grad_a_tensor")
     _lut_len_check(lut_grad_b_tensor, "lut_grad_b_tensor")
     _check(lut_grad_a_tensor.size(0) == lut_grad_b_tensor.size(0), "the two gradient tables must have the same length")
     dev = gc_tensor.device
-    _check(all(t.device == dev for t in (a_tensor, b_tensor, ga_tensor, gb_tensor, lut_grad_a_tensor, lut_grad_b_tensor)),
+    _check(all(t.device == dev for t in (a_tensor, b_tensor, ga_tensor, gb_tensor, lut_grad_a_tensor, lut_grad_b_tensor) if t is not None),
            "All tensors should be on the same device")
     with torch.cuda.device(dev):
         need = _lib.amr_lut_gemm_backward_workspace_bytes(M, K, N)
         ws = torch.empty(need, dtype=torch.uint8, device=dev) if need else None
         rc = _lib.amr_lut_gemm_backward_ex(gc_tensor.data_ptr(), a_tensor.data_ptr(), b_tensor.data_ptr(),
-                                           ga_tensor.data_ptr(), gb_tensor.data_ptr(), lut_grad_a_tensor.data_ptr(),
+                                           ga_tensor.data_ptr() if ga_tensor is not None else None,
+                                           gb_tensor.data_ptr() if gb_tensor is not None else None, lut_grad_a_tensor.data_ptr(),
                                            lut_grad_b_tensor.data_ptr(), lut_grad_a_tensor.size(0), M, K, N, L,
                                            ws.data_ptr() if ws is not None else None, need, _stream_ptr(dev))
     _raise_for(rc, "approx_gemm_backward")

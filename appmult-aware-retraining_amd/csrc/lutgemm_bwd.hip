@@ -101,14 +101,14 @@ __global__ void reduce_partials_kernel(const float* __restrict__ partial, float*
 }
 
 // ------------------------------------------------------------------------------------------ gradA
-// VEC: N % 4 == 0, K % 4 == 0 and gC / gA 16-byte aligned, so the per-lane rows of gC are read and the
-// per-lane rows of gA are written 16 bytes at a time (a lane owns a row, so every scalar access would
+// VEC: N % 4 == 0 and gC 16-byte aligned, so the per-lane rows of gC are read 16 bytes at a time; vec_store: K % 4 == 0
+// and gA 16-byte aligned, so the per-lane rows of gA are written 16 bytes at a time (a lane owns a row, so every scalar access would
 // touch 64 different cache lines per instruction).
 template <int KT, int RM, int WAVES, bool VEC>
 __global__ __launch_bounds__(WAVES * 64) void lutgemm_gradA_kernel(
     const float* __restrict__ gC, const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
     float* __restrict__ gA, const uint16_t* __restrict__ lut, int rows, int cols, int M, int K, int N, float scale,
-    const uint32_t* __restrict__ gate, int rows_per_image) {
+    const uint32_t* __restrict__ gate, int rows_per_image, int vec_store) {
     extern __shared__ __align__(16) unsigned char smem[];
     if (gate != nullptr && *gate == 0u) return;   // queued as a fallback that turned out not to be needed
     // Transposed staging: entry (a,b) of the row-major table goes to T[b][a], T row stride = cols
@@ -196,7 +196,7 @@ __global__ __launch_bounds__(WAVES * 64) void lutgemm_gradA_kernel(
             for (int kk = 0; kk < KT; ++kk)
                 if (k0 + kk < K) o[(size_t)kk * rows_per_image] = acc[r][kk] * scale;
         } else if (m < M) {
-            if (VEC) {
+            if (vec_store) {   // K % 4 == 0 and gA 16-byte aligned
                 typedef float f32x4 __attribute__((ext_vector_type(4)));
 #pragma unroll
                 for (int d = 0; d < KT / 4; ++d) {
@@ -276,6 +276,7 @@ template <int KT, int RM, int WAVES, bool VEC>
 static hipError_t launch_gradA_t(const float* gC, const uint8_t* A, const uint8_t* B, float* gA, const int16_t* lut,
                                  const LutGeom& g, int M, int K, int N, float scale, hipStream_t stream, const uint32_t* gate,
                                  int rows_per_image) {
+    const int vec_store = ((K & 3) == 0) && (((uintptr_t)gA & 15) == 0);
     auto kern = lutgemm_gradA_kernel<KT, RM, WAVES, VEC>;
     static bool done = false;
     if (!done) {
@@ -286,7 +287,7 @@ static hipError_t launch_gradA_t(const float* gC, const uint8_t* A, const uint8_
     const int rows_per_wg = 64 * RM * WAVES;
     dim3 grid((K + KT - 1) / KT, (M + rows_per_wg - 1) / rows_per_wg);
     hipLaunchKernelGGL(kern, grid, dim3(WAVES * 64), (size_t)g.cols * g.cols * 2, stream, gC, A, B, gA,
-                       reinterpret_cast<const uint16_t*>(lut), g.rows, g.cols, M, K, N, scale, gate, rows_per_image);
+                       reinterpret_cast<const uint16_t*>(lut), g.rows, g.cols, M, K, N, scale, gate, rows_per_image, vec_store);
     return hipGetLastError();
 }
 
@@ -294,7 +295,7 @@ hipError_t launch_gradA(const float* gC, const uint8_t* A, const uint8_t* B, flo
                         const LutGeom& g, int M, int K, int N, float scale, int n_cu, hipStream_t stream,
                         const uint32_t* gate = nullptr, int rows_per_image = 0) {
     constexpr int KT = 16;
-    const bool vec = ((N & 3) == 0) && ((K & 3) == 0) && (((uintptr_t)gC & 15) == 0) && (((uintptr_t)gA & 15) == 0);
+    const bool vec = ((N & 3) == 0) && (((uintptr_t)gC & 15) == 0);   // rows of gC are read 16 bytes at a time
     const int ktiles = (K + KT - 1) / KT;
     if (g.bits == 8) {
         return vec ? launch_gradA_t<KT, 1, 16, true>(gC, A, B, gA, lut, g, M, K, N, scale, stream, gate, rows_per_image)

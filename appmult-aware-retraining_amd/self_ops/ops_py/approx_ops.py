@@ -229,12 +229,16 @@ class ApproxConv2dFn(Function):
         a_c, b_c = ctx.saved_tensors
         s, p, d, batch, cin, h, w, cout, kh, kw, oh, ow = ctx.geo
         g_c = _conv_grad_rows(g_out, ctx.geo)
-        g_a = torch.empty((batch, cin * kh * kw, oh * ow), dtype=torch.float32, device=g_c.device)
-        g_b = torch.empty(b_c.shape, dtype=torch.float32, device=g_c.device)
-        approx_ops.approx_gemm_backward(g_c, a_c, b_c, g_a, g_b, lut_grad_a, lut_grad_b, ga_rows_per_image=oh * ow)
-        g_in = F.fold(g_a, (h, w), kernel_size=(kh, kw), dilation=(d, d), padding=(p, p), stride=(s, s))
-        g_w = g_b.t().reshape(cout, cin, kh, kw)
-        return g_in.to(ctx.dtypes[0]), g_w.to(ctx.dtypes[1]), None, None, None
+        # a gradient nobody asked for (the images in front of the first layer) is not computed: the reference
+        # always runs both kernels (approx_gemm_backward.cu:561,588)
+        need_in, need_w = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
+        g_a = torch.empty((batch, cin * kh * kw, oh * ow), dtype=torch.float32, device=g_c.device) if need_in else None
+        g_b = torch.empty(b_c.shape, dtype=torch.float32, device=g_c.device) if need_w else None
+        if need_in or need_w:
+            approx_ops.approx_gemm_backward(g_c, a_c, b_c, g_a, g_b, lut_grad_a, lut_grad_b, ga_rows_per_image=oh * ow)
+        g_in = F.fold(g_a, (h, w), kernel_size=(kh, kw), dilation=(d, d), padding=(p, p), stride=(s, s)).to(ctx.dtypes[0]) if need_in else None
+        g_w = g_b.t().reshape(cout, cin, kh, kw).to(ctx.dtypes[1]) if need_w else None
+        return g_in, g_w, None, None, None
 
 
 class ApproxConv2dBaselineFn(Function):

@@ -215,6 +215,24 @@ def test_conv_op_matches_reference_composition(ops, oracle, golden_dir, shape, c
     torch.testing.assert_close(wb.grad, wb2.grad, rtol=1e-4, atol=1e-4 * float(wb2.grad.abs().max()))
 
 
+def test_conv_op_skips_the_gradient_nobody_needs(ops):
+    """Images in front of the first layer need no gradient: only the weight gradient is computed then (and equals
+    the one computed together with the input gradient)."""
+    self_ops, P = ops
+    x = torch.randint(0, 128, (4, 3, 12, 12), device="cuda").float()
+    w = torch.randint(0, 128, (8, 3, 3, 3), device="cuda").float().requires_grad_()
+    args = (None, (1, 1), (1, 1), (1, 1), 1)
+    g = torch.randn(4, 8, 12, 12, device="cuda")
+    self_ops.approx_conv2d_op(x, w, *args).backward(g)
+    x2, w2 = x.clone().requires_grad_(), w.detach().clone().requires_grad_()
+    self_ops.approx_conv2d_op(x2, w2, *args).backward(g)
+    assert torch.equal(w.grad, w2.grad) and x2.grad is not None
+    w3 = w.detach().clone()
+    x3 = x.clone().requires_grad_()
+    self_ops.approx_conv2d_op(x3, w3, *args).backward(g)
+    assert torch.equal(x3.grad, x2.grad)
+
+
 def test_conv_op_rejects_bias_and_groups(ops):
     self_ops, P = ops
     x, w = torch.zeros(1, 2, 4, 4, device="cuda"), torch.zeros(2, 2, 3, 3, device="cuda")
