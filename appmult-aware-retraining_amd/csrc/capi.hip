@@ -30,6 +30,7 @@ hipError_t launch_quantize_codes(const float* x, const float* scale, const float
                                  hipStream_t stream);
 hipError_t launch_quantize_codes_backward(const float* g, const float* x, const float* scale, const float* zp_neg, float qmax,
                                           float* gx, size_t n, hipStream_t stream);
+hipError_t launch_zero_u32(void* p, size_t n_dwords, hipStream_t stream);
 hipError_t launch_im2col_u8_f32(const float* x, uint8_t* A, int B, int C, int H, int W, int kh, int kw, int stride, int pad,
                                 int dil, int oh, int ow, hipStream_t stream);
 bool bwd_slab_applies(const LutGeom& g, int M, int K, int N);
@@ -152,8 +153,8 @@ int amr_lut_gemm_forward_ws(const uint8_t* A, const uint8_t* B, uint32_t* C, con
     if ((uintptr_t)lut & 3) return fail(AMR_EINVAL, "lut must be 4-byte aligned");
     hipStream_t s = reinterpret_cast<hipStream_t>(stream);
     if (K == 0) {
-        hipError_t e = hipMemsetAsync(C, 0, (size_t)M * N * sizeof(uint32_t), s);
-        return e == hipSuccess ? AMR_OK : hip_fail(e, "hipMemsetAsync");
+        hipError_t e = amr::launch_zero_u32(C, (size_t)M * N, s);
+        return e == hipSuccess ? AMR_OK : hip_fail(e, "zero fill launch");
     }
     int dev = 0;
     const int n_cu = current_device_cus(&dev);
@@ -231,9 +232,9 @@ int amr_lut_gemm_backward_ex(const float* gC, const uint8_t* A, const uint8_t* B
     // Degenerate reductions: an empty sum is zero.
     if (M == 0 || K == 0 || N == 0) {
         hipError_t e = hipSuccess;
-        if (gA && (size_t)M * K) e = hipMemsetAsync(gA, 0, (size_t)M * K * sizeof(float), s);
-        if (e == hipSuccess && gB && (size_t)K * N) e = hipMemsetAsync(gB, 0, (size_t)K * N * sizeof(float), s);
-        return e == hipSuccess ? AMR_OK : hip_fail(e, "hipMemsetAsync");
+        if (gA && (size_t)M * K) e = amr::launch_zero_u32(gA, (size_t)M * K, s);
+        if (e == hipSuccess && gB && (size_t)K * N) e = amr::launch_zero_u32(gB, (size_t)K * N, s);
+        return e == hipSuccess ? AMR_OK : hip_fail(e, "zero fill launch");
     }
     if (!gC || !A || !B) return fail(AMR_EINVAL, "null pointer argument");
     if (!gA && !gB) return AMR_OK;
@@ -256,8 +257,8 @@ int amr_lut_gemm_backward_ex(const float* gC, const uint8_t* A, const uint8_t* B
     const bool slab = g_expanded_kernels && amr::bwd_slab_applies(g, M, K, N);
     const bool slab_a = g_expanded_kernels && gA && amr::gradA_slab_workspace_bytes(g, M, K, N, g_expanded_kernels == 2) != 0 && ((uintptr_t)gC & 15) == 0;
     if ((slab && gB) || slab_a) {
-        e = hipMemsetAsync(flags, 0, 256, s);
-        if (e != hipSuccess) return hip_fail(e, "hipMemsetAsync");
+        e = amr::launch_zero_u32(flags, 64, s);
+        if (e != hipSuccess) return hip_fail(e, "zero fill launch");
     }
     if (gA) {
         if (slab_a)
@@ -320,8 +321,8 @@ int amr_acc_gemm_forward_fp32(const float* A, const float* B, float* C, int M, i
     if (!C || (K > 0 && (!A || !B))) return fail(AMR_EINVAL, "null pointer argument");
     hipStream_t s = reinterpret_cast<hipStream_t>(stream);
     if (K == 0) {
-        hipError_t e = hipMemsetAsync(C, 0, (size_t)M * N * sizeof(float), s);
-        return e == hipSuccess ? AMR_OK : hip_fail(e, "hipMemsetAsync");
+        hipError_t e = amr::launch_zero_u32(C, (size_t)M * N, s);
+        return e == hipSuccess ? AMR_OK : hip_fail(e, "zero fill launch");
     }
     hipError_t e = amr::launch_accgemm(A, B, C, M, K, N, s);
     return e == hipSuccess ? AMR_OK : hip_fail(e, "accgemm launch");

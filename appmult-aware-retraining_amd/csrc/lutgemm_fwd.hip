@@ -16,6 +16,8 @@
 
 namespace amr {
 
+hipError_t launch_zero_u32(void* p, size_t n_dwords, hipStream_t stream);
+
 template <int R, int TN, int WAVES>
 __global__ __launch_bounds__(WAVES * 64) void lutgemm_fwd_kernel(
     const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, uint32_t* __restrict__ C,
@@ -139,7 +141,7 @@ static hipError_t launch_fwd_t(const uint8_t* A, const uint8_t* B, uint32_t* C, 
     const int zs = (K + k_chunk - 1) / k_chunk;
     dim3 grid((N + 64 * TN - 1) / (64 * TN), (M + WAVES * R - 1) / (WAVES * R), zs);
     if (zs > 1) {
-        hipError_t e = hipMemsetAsync(C, 0, (size_t)M * N * sizeof(uint32_t), stream);
+        hipError_t e = launch_zero_u32(C, (size_t)M * N, stream);
         if (e != hipSuccess) return e;
     }
     hipLaunchKernelGGL(kern, grid, dim3(WAVES * 64), lds, stream, A, B, C, reinterpret_cast<const uint32_t*>(lut),

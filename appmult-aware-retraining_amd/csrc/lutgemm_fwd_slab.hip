@@ -33,6 +33,8 @@
 
 namespace amr {
 
+hipError_t launch_zero_u32(void* p, size_t n_dwords, hipStream_t stream);
+
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));   // native 16-byte vector (stays in registers)
 
 constexpr int kSlabRows = 128;                       // codes per chunk
@@ -370,7 +372,7 @@ hipError_t launch_fwd_slab(const uint8_t* A, const uint8_t* B, uint32_t* C, cons
     const int k_quads = (K + 3) / 4;
     uint32_t* flags = reinterpret_cast<uint32_t*>(workspace);
     uint32_t* E = reinterpret_cast<uint32_t*>(reinterpret_cast<unsigned char*>(workspace) + 256);
-    hipError_t e = hipMemsetAsync(flags, 0, 256, stream);
+    hipError_t e = launch_zero_u32(flags, 64, stream);
     if (e != hipSuccess) return e;
     const int lut_dwords = g.rows * g.cols / 2;
     hipLaunchKernelGGL(expand_fwd_kernel, dim3(n_tiles, (k_quads + kExpandQuadsPerWg - 1) / kExpandQuadsPerWg), dim3(256),
@@ -392,7 +394,7 @@ hipError_t launch_fwd_slab(const uint8_t* A, const uint8_t* B, uint32_t* C, cons
     const int cps = (k_quads + ksplit - 1) / ksplit;
     const int zs = (k_quads + cps - 1) / cps;
     if (zs > 1) {
-        e = hipMemsetAsync(C, 0, (size_t)M * N * sizeof(uint32_t), stream);
+        e = launch_zero_u32(C, (size_t)M * N, stream);
         if (e != hipSuccess) return e;
     }
     dim3 grid(n_tiles, (M + m_tile - 1) / m_tile, zs);
