@@ -369,6 +369,58 @@ def test_default_mode_picks_kernels_by_problem_size(lib, oracle):
         lib.amr_set_expanded_table_kernels(2)
 
 
+def test_calls_can_be_recorded_into_a_device_graph(lib, oracle):
+    """Forward and backward with caller-provided scratch, recorded once into a graph and replayed with new operand
+    contents (with eager work and synchronisations in between): every replay equals the eager result."""
+    print("graph capture", flush=True)
+    M, K, N = 4096, 576, 64
+    rng, A, B, T = rand_case(31, M, K, N, 7)
+    T = oracle.synth_lut(7, 64, rng)
+    flat = oracle.pack_table(T, 7, np.uint16)
+    Gx, Gy = oracle.gen_bp_lut(T, 8)
+    la, lb = oracle.pack_table(Gx, 7, np.int16), oracle.pack_table(Gy, 7, np.int16)
+    a, b, l, ta, tb = dev(A), dev(B), dev(flat), dev(la), dev(lb)
+    g = torch.randn(M, N, device="cuda")
+    c = torch.zeros(M, N, dtype=torch.int32, device="cuda")
+    ga, gb = torch.zeros(M, K, device="cuda"), torch.zeros(K, N, device="cuda")
+    need_f = lib.amr_lut_gemm_forward_workspace_bytes(l.numel(), M, K, N)
+    need_b = lib.amr_lut_gemm_backward_workspace_bytes(M, K, N)
+    assert need_f > 0 and need_b > 0
+    ws_f = torch.empty(need_f, dtype=torch.uint8, device="cuda")
+    ws_b = torch.empty(need_b, dtype=torch.uint8, device="cuda")
+
+    def run(stream):
+        sp = ctypes.c_void_p(stream.cuda_stream)
+        assert lib.amr_lut_gemm_forward_ws(a.data_ptr(), b.data_ptr(), c.data_ptr(), l.data_ptr(), l.numel(), M, K, N,
+                                           ws_f.data_ptr(), need_f, sp) == 0, lib.amr_last_error()
+        assert lib.amr_lut_gemm_backward(g.data_ptr(), a.data_ptr(), b.data_ptr(), ga.data_ptr(), gb.data_ptr(), ta.data_ptr(),
+                                         tb.data_ptr(), ta.numel(), M, K, N, ws_b.data_ptr(), need_b, sp) == 0, lib.amr_last_error()
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        run(side)                                   # warm-up: one-time attribute calls happen outside the capture
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        run(torch.cuda.current_stream())
+    for rep in range(3):
+        a.copy_(torch.randint(0, 128, (M, K), dtype=torch.uint8, device="cuda"))
+        if rep == 1:
+            a[5, 7] = 128                           # a masked code: the gated fall-back kernels do the work in this replay
+        g.copy_(torch.randn(M, N, device="cuda"))
+        c.zero_(); ga.zero_(); gb.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        got = (c.clone(), ga.clone(), gb.clone())
+        c.zero_(); ga.zero_(); gb.zero_()
+        run(torch.cuda.current_stream())
+        torch.cuda.synchronize()
+        assert torch.equal(got[0], c) and torch.equal(got[1], ga) and torch.equal(got[2], gb), f"replay {rep} differs from the eager call"
+        assert (c.cpu().numpy().view(np.uint32) == oracle.forward_c(a.cpu().numpy(), B, flat, 7)).all()
+
+
 def test_accgemm_matches_torch(lib):
     print("accgemm", flush=True)
     torch.manual_seed(0)
