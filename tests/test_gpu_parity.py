@@ -473,3 +473,47 @@ def test_full_size_resnet_layer_properties(lib, oracle):
     torch.cuda.synchronize()
     assert torch.equal(ga.double(), g.double() @ b.double().t())
     assert torch.equal(gb.double(), a.double().t() @ g.double())
+
+
+# The GEMM shapes of the benchmark step (ResNet-18 / CIFAR at batch 256), in the library's own kernel selection.
+RESNET18_B256_SHAPES = [(262144, 27, 64), (262144, 576, 64), (65536, 576, 128), (65536, 1152, 128), (65536, 64, 128),
+                        (16384, 1152, 256), (16384, 2304, 256), (16384, 128, 256), (4096, 2304, 512), (4096, 4608, 512),
+                        (4096, 256, 512), (256, 512, 10)]
+
+
+@pytest.mark.parametrize("shape", RESNET18_B256_SHAPES)
+def test_benchmark_shapes_against_oracle_on_row_samples(lib, oracle, shape):
+    """Full-size layers are too big for the CPU oracle, but every output row of the forward pass and of gA depends on
+    its own row of A / gC only, and gB is a sum over rows: with gC non-zero on a sample of rows only (spread over all
+    row blocks and M splits), the oracle on that sample gives the forward rows, the gA rows and the whole of gB."""
+    print("benchmark shape", shape, flush=True)
+    M, K, N = shape
+    gen = torch.Generator(device="cuda").manual_seed(M + K + N)
+    rng = np.random.default_rng(M + 3 * K + 7 * N)
+    T = oracle.synth_lut(7, 64, rng)
+    Gx, Gy = oracle.gen_bp_lut(T, 8)
+    flat, la, lb = oracle.pack_table(T, 7, np.uint16), oracle.pack_table(Gx, 7, np.int16), oracle.pack_table(Gy, 7, np.int16)
+    a = torch.randint(0, 128, (M, K), dtype=torch.uint8, device="cuda", generator=gen)
+    b = torch.randint(0, 128, (K, N), dtype=torch.uint8, device="cuda", generator=gen)
+    rows = np.unique(np.r_[0:96, np.arange(37, M, max(M // 1500, 1)), M // 2 - 70:M // 2 + 70, M - 96:M].clip(0, M - 1))
+    rows_t = torch.from_numpy(rows).cuda()
+    g = torch.zeros((M, N), device="cuda")
+    g[rows_t] = torch.randn((len(rows), N), device="cuda", generator=gen)
+    c = torch.empty((M, N), dtype=torch.int32, device="cuda")
+    ga = torch.full((M, K), float("nan"), device="cuda")
+    gb = torch.full((K, N), float("nan"), device="cuda")
+    l, ta, tb = dev(flat), dev(la), dev(lb)
+    assert lib.amr_set_expanded_table_kernels(1) == 2
+    try:
+        assert lib.amr_lut_gemm_forward(a.data_ptr(), b.data_ptr(), c.data_ptr(), l.data_ptr(), l.numel(), M, K, N, None) == 0
+        assert lib.amr_lut_gemm_backward(g.data_ptr(), a.data_ptr(), b.data_ptr(), ga.data_ptr(), gb.data_ptr(), ta.data_ptr(),
+                                         tb.data_ptr(), ta.numel(), M, K, N, None, 0, None) == 0, lib.amr_last_error()
+        torch.cuda.synchronize()
+    finally:
+        lib.amr_set_expanded_table_kernels(2)
+    As, Bn, gs = a[rows_t].cpu().numpy(), b.cpu().numpy(), g[rows_t].cpu().numpy()
+    assert (c[rows_t].cpu().numpy().view(np.uint32) == oracle.forward_c(As, Bn, flat, 7)).all()
+    mask = torch.ones(M, dtype=torch.bool, device="cuda")
+    mask[rows_t] = False
+    assert (ga[mask] == 0).all()                              # rows without gradient: exactly zero
+    check_backward(oracle, (ga[rows_t].cpu().numpy(), gb.cpu().numpy()), gs, As, Bn, la, lb, 7)
