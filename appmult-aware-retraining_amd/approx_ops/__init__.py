@@ -35,6 +35,9 @@ _vp, _i, _i64, _sz = ctypes.c_void_p, ctypes.c_int, ctypes.c_int64, ctypes.c_siz
 _lib.amr_last_error.restype = ctypes.c_char_p
 _lib.amr_target_arch.restype = ctypes.c_char_p
 _lib.amr_lut_gemm_forward.argtypes = [_vp, _vp, _vp, _vp, _i64, _i, _i, _i, _vp]
+_lib.amr_lut_gemm_forward_ws.argtypes = [_vp, _vp, _vp, _vp, _i64, _i, _i, _i, _vp, _sz, _vp]
+_lib.amr_lut_gemm_forward_workspace_bytes.argtypes = [_i64, _i, _i, _i]
+_lib.amr_lut_gemm_forward_workspace_bytes.restype = _sz
 _lib.amr_lut_gemm_backward.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i, _i, _i, _vp, _sz, _vp]
 _lib.amr_lut_gemm_backward_ex.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i, _i, _i, _i, _vp, _sz, _vp]
 _lib.amr_im2col_u8_f32.argtypes = [_vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp]
@@ -96,8 +99,13 @@ def approx_gemm_forward(a_tensor, b_tensor, c_tensor, lut_appmult_tensor):
     dev = a_tensor.device
     _check(dev == b_tensor.device and dev == c_tensor.device and dev == lut_appmult_tensor.device, "device id not match")
     with torch.cuda.device(dev):
-        rc = _lib.amr_lut_gemm_forward(a_tensor.data_ptr(), b_tensor.data_ptr(), c_tensor.data_ptr(),
-                                       lut_appmult_tensor.data_ptr(), lut_appmult_tensor.size(0), M, K, N, _stream_ptr(dev))
+        # scratch (the expanded table of large problems) comes from torch's caching allocator, so that it is
+        # ordered with the stream like any other tensor and freed with the process' other device memory
+        need = _lib.amr_lut_gemm_forward_workspace_bytes(lut_appmult_tensor.size(0), M, K, N)
+        ws = torch.empty(need, dtype=torch.uint8, device=dev) if need else None
+        rc = _lib.amr_lut_gemm_forward_ws(a_tensor.data_ptr(), b_tensor.data_ptr(), c_tensor.data_ptr(),
+                                          lut_appmult_tensor.data_ptr(), lut_appmult_tensor.size(0), M, K, N,
+                                          ws.data_ptr() if ws is not None else None, need, _stream_ptr(dev))
     _raise_for(rc, "approx_gemm_forward")
 
 
