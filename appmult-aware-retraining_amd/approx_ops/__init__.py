@@ -41,6 +41,7 @@ _lib.amr_lut_gemm_forward_workspace_bytes.restype = _sz
 _lib.amr_lut_gemm_backward.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i, _i, _i, _vp, _sz, _vp]
 _lib.amr_lut_gemm_backward_ex.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i, _i, _i, _i, _vp, _sz, _vp]
 _lib.amr_im2col_u8_f32.argtypes = [_vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp]
+_lib.amr_col2im_f32.argtypes = [_vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp]
 _lib.amr_quantize_codes_f32.argtypes = [_vp, _vp, _vp, ctypes.c_float, _vp, _i64, _vp]
 _lib.amr_quantize_codes_backward_f32.argtypes = [_vp, _vp, _vp, _vp, ctypes.c_float, _vp, _i64, _vp]
 _lib.amr_lut_gemm_backward_workspace_bytes.argtypes = [_i, _i, _i]
@@ -194,6 +195,26 @@ def im2col_codes(x_tensor, a_tensor, kernel_size, stride, padding, dilation):
         rc = _lib.amr_im2col_u8_f32(x_tensor.data_ptr(), a_tensor.data_ptr(), Bn, C, H, W, kh, kw, stride, padding, dilation,
                                     _stream_ptr(dev))
     _raise_for(rc, "im2col_codes")
+
+
+def col2im(cols_tensor, x_tensor, kernel_size, stride, padding, dilation):
+    """x[b,c,y,x] = sum of the window entries cols[b, c*kh*kw + i*kw + j, oy*ow + ox] that pixel fed (the adjoint of
+    im2col_codes; torch.nn.functional.fold of the same arguments).  cols float32 [B, C*kh*kw, oh*ow], x float32 [B,C,H,W]."""
+    _check_input(cols_tensor, torch.float32, "cols_tensor")
+    _check_input(x_tensor, torch.float32, "x_tensor")
+    _check(cols_tensor.dim() == 3 and x_tensor.dim() == 4, "cols must be 3-D and x 4-D")
+    kh, kw = kernel_size
+    Bn, C, H, W = x_tensor.shape
+    oh = (H + 2 * padding - dilation * (kh - 1) - 1) // stride + 1
+    ow = (W + 2 * padding - dilation * (kw - 1) - 1) // stride + 1
+    _check(oh > 0 and ow > 0, "empty convolution output")
+    _check(tuple(cols_tensor.shape) == (Bn, C * kh * kw, oh * ow), f"cols_tensor's shape should be {Bn} x {C * kh * kw} x {oh * ow}")
+    dev = x_tensor.device
+    _check(dev == cols_tensor.device, "device id not match")
+    with torch.cuda.device(dev):
+        rc = _lib.amr_col2im_f32(cols_tensor.data_ptr(), x_tensor.data_ptr(), Bn, C, H, W, kh, kw, stride, padding, dilation,
+                                 _stream_ptr(dev))
+    _raise_for(rc, "col2im")
 
 
 def quantize_codes(x_tensor, scale_tensor, zp_neg_tensor, quant_max, codes_tensor):

@@ -31,6 +31,8 @@ hipError_t launch_quantize_codes(const float* x, const float* scale, const float
 hipError_t launch_quantize_codes_backward(const float* g, const float* x, const float* scale, const float* zp_neg, float qmax,
                                           float* gx, size_t n, hipStream_t stream);
 hipError_t launch_zero_u32(void* p, size_t n_dwords, hipStream_t stream);
+hipError_t launch_col2im_f32(const float* cols, float* x, int B, int C, int H, int W, int kh, int kw, int stride, int pad, int dil,
+                             int oh, int ow, hipStream_t stream);
 hipError_t launch_im2col_u8_f32(const float* x, uint8_t* A, int B, int C, int H, int W, int kh, int kw, int stride, int pad,
                                 int dil, int oh, int ow, hipStream_t stream);
 bool bwd_slab_applies(const LutGeom& g, int M, int K, int N);
@@ -293,6 +295,20 @@ int amr_im2col_u8_f32(const float* x, uint8_t* A, int B, int C, int H, int W, in
     if (!x || !A) return fail(AMR_EINVAL, "null pointer argument");
     hipError_t e = amr::launch_im2col_u8_f32(x, A, B, C, H, W, kh, kw, stride, pad, dil, oh, ow, reinterpret_cast<hipStream_t>(stream));
     return e == hipSuccess ? AMR_OK : hip_fail(e, "im2col launch");
+}
+
+int amr_col2im_f32(const float* cols, float* x, int B, int C, int H, int W, int kh, int kw, int stride, int pad, int dil,
+                   void* stream) {
+    if (B < 0 || C <= 0 || H <= 0 || W <= 0 || kh <= 0 || kw <= 0 || stride <= 0 || pad < 0 || dil <= 0)
+        return fail(AMR_EINVAL, "bad convolution geometry");
+    const int oh = (H + 2 * pad - dil * (kh - 1) - 1) / stride + 1;
+    const int ow = (W + 2 * pad - dil * (kw - 1) - 1) / stride + 1;
+    if (oh <= 0 || ow <= 0) return fail(AMR_EINVAL, "empty convolution output");
+    if (B == 0) return AMR_OK;
+    if ((size_t)B * C * H * W >= ((size_t)1 << 40)) return fail(AMR_EUNSUPPORTED, "more than 2^40 pixels");
+    if (!cols || !x) return fail(AMR_EINVAL, "null pointer argument");
+    hipError_t e = amr::launch_col2im_f32(cols, x, B, C, H, W, kh, kw, stride, pad, dil, oh, ow, reinterpret_cast<hipStream_t>(stream));
+    return e == hipSuccess ? AMR_OK : hip_fail(e, "col2im launch");
 }
 
 int amr_quantize_codes_f32(const float* x, const float* scale, const float* zp_neg, float qmax, float* codes, int64_t n,

@@ -78,4 +78,47 @@ hipError_t launch_im2col_u8_f32(const float* x, uint8_t* A, int B, int C, int H,
     return hipGetLastError();
 }
 
+// ------------------------------------------------------------------------------------------ col2im
+// Adjoint of the window extraction for the input gradient of the LUT convolution: cols [B][C*kh*kw][oh*ow] (the
+// image-major layout gradA writes) -> x [B,C,H,W], x[b,c,y,x] = sum over the taps (i,j) whose window position
+// (oy,ox) = ((y + pad - i*dil)/stride, (x + pad - j*dil)/stride) exists.  What the reference gets from autograd
+// through F.unfold (self_ops/ops_py/approx_ops.py:558); a gather, so no atomics and a fixed summation order.
+// One thread per input pixel; consecutive threads read consecutive window positions of the same tap row.
+__global__ __launch_bounds__(256) void col2im_f32_kernel(const float* __restrict__ cols, float* __restrict__ x, int C, int H, int W,
+                                                         int kh, int kw, int stride, int pad, int dil, int oh, int ow, size_t total) {
+    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= total) return;
+    const int xx = (int)(idx % W);
+    size_t r = idx / W;
+    const int yy = (int)(r % H);
+    r /= H;
+    const int c = (int)(r % C);
+    const size_t b = r / C;
+    const size_t L = (size_t)oh * ow;
+    const float* base = cols + (b * C + c) * (size_t)(kh * kw) * L;
+    float acc = 0.f;
+    for (int i = 0; i < kh; ++i) {
+        const int ty = yy + pad - i * dil;
+        if (ty < 0 || ty % stride != 0) continue;
+        const int oy = ty / stride;
+        if (oy >= oh) continue;
+        for (int j = 0; j < kw; ++j) {
+            const int tx = xx + pad - j * dil;
+            if (tx < 0 || tx % stride != 0) continue;
+            const int ox = tx / stride;
+            if (ox >= ow) continue;
+            acc += base[(size_t)(i * kw + j) * L + (size_t)oy * ow + ox];
+        }
+    }
+    x[idx] = acc;
+}
+
+hipError_t launch_col2im_f32(const float* cols, float* x, int B, int C, int H, int W, int kh, int kw, int stride, int pad, int dil,
+                             int oh, int ow, hipStream_t stream) {
+    const size_t total = (size_t)B * C * H * W;
+    hipLaunchKernelGGL(col2im_f32_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, cols, x, C, H, W, kh, kw,
+                       stride, pad, dil, oh, ow, total);
+    return hipGetLastError();
+}
+
 }  // namespace amr

@@ -236,7 +236,11 @@ class ApproxConv2dFn(Function):
         g_b = torch.empty(b_c.shape, dtype=torch.float32, device=g_c.device) if need_w else None
         if need_in or need_w:
             approx_ops.approx_gemm_backward(g_c, a_c, b_c, g_a, g_b, lut_grad_a, lut_grad_b, ga_rows_per_image=oh * ow)
-        g_in = F.fold(g_a, (h, w), kernel_size=(kh, kw), dilation=(d, d), padding=(p, p), stride=(s, s)).to(ctx.dtypes[0]) if need_in else None
+        g_in = None
+        if need_in:
+            g_in = torch.empty((batch, cin, h, w), dtype=torch.float32, device=g_c.device)
+            approx_ops.col2im(g_a, g_in, (kh, kw), s, p, d)          # = F.fold(g_a, (h, w), (kh, kw), d, p, s)
+            g_in = g_in.to(ctx.dtypes[0])
         g_w = g_b.t().reshape(cout, cin, kh, kw).to(ctx.dtypes[1]) if need_w else None
         return g_in, g_w, None, None, None
 

@@ -113,6 +113,15 @@ int amr_im2col_u8_f32(const float *x, uint8_t *A, int B, int C, int H, int W, in
                       int dil, void *stream);
 
 /*
+ * Adjoint of amr_im2col_u8_f32 for gradients: cols [B][C*kh*kw][oh*ow] float32 (the layout amr_lut_gemm_backward_ex
+ * writes with ga_rows_per_image = oh*ow) -> x [B,C,H,W], every pixel the sum of the window entries it fed.  The
+ * input-gradient step the reference leaves to autograd through F.unfold (self_ops/ops_py/approx_ops.py:558).
+ * Overwrites x; fixed summation order (no atomics).
+ */
+int amr_col2im_f32(const float *cols, float *x, int B, int C, int H, int W, int kh, int kw, int stride, int pad,
+                   int dil, void *stream);
+
+/*
  * Process-wide switch for diagnostics, tests and benchmarks.  mode 0 sends every later call to the direct
  * gather kernels (the formulation of the reference's kernels, approx_gemm_forward.cu:45-229); 1 (the default)
  * lets the library pick by problem size; 2 takes the expanded-table kernels wherever the shape allows, also

@@ -139,6 +139,27 @@ def test_im2col_codes_against_oracle(ops, oracle, shape, k, stride, padding, dil
     assert torch.equal(a, cols.transpose(1, 2).reshape(-1, want.shape[1]).to(torch.uint8))
 
 
+@pytest.mark.parametrize("shape,k,stride,padding,dilation", [
+    ((3, 5, 10, 10), 3, 1, 1, 1), ((2, 4, 9, 7), 3, 2, 1, 1), ((2, 8, 12, 12), 1, 2, 0, 1), ((1, 3, 16, 16), 7, 2, 3, 1),
+    ((2, 6, 11, 11), 3, 1, 2, 2), ((2, 64, 8, 8), 3, 1, 1, 1), ((4, 16, 32, 32), 3, 1, 1, 1)])
+def test_col2im_equals_fold(ops, shape, k, stride, padding, dilation):
+    import approx_ops
+    print("col2im", shape, k, stride, padding, dilation, flush=True)
+    Bn, C, H, W = shape
+    oh = (H + 2 * padding - dilation * (k - 1) - 1) // stride + 1
+    ow = (W + 2 * padding - dilation * (k - 1) - 1) // stride + 1
+    g = torch.Generator(device="cuda").manual_seed(1)
+    cols = torch.randn(Bn, C * k * k, oh * ow, device="cuda", generator=g)
+    x = torch.full(shape, float("nan"), device="cuda")
+    approx_ops.col2im(cols, x, (k, k), stride, padding, dilation)
+    want = F.fold(cols.double(), (H, W), (k, k), dilation=dilation, padding=padding, stride=stride)
+    torch.testing.assert_close(x.double(), want, rtol=0, atol=1e-6 * float(want.abs().max()))
+    # integer-valued windows: every order of the sums gives the same bits
+    ci = torch.randint(-8, 9, cols.shape, device="cuda", generator=g).float()
+    approx_ops.col2im(ci, x, (k, k), stride, padding, dilation)
+    assert torch.equal(x, F.fold(ci, (H, W), (k, k), dilation=dilation, padding=padding, stride=stride))
+
+
 def test_im2col_codes_rejects_wrong_shapes(ops):
     import approx_ops
     x = torch.zeros(2, 3, 8, 8, device="cuda")
