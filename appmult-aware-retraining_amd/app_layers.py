@@ -176,6 +176,31 @@ class QuantLinear(nn.Linear, _QuantParamsMixin):
         return F.linear(input_fq, weight_fq, self.bias)
 
 
+class ApproxLinear(QuantLinear):
+    """Fully connected layer whose code products come from the approximate-multiplier table, the way ApproxConv2d
+    treats a convolution.  The reference keeps its linear layers on exact products (``app_layers.py:109-111``);
+    this variant is opt-in (``prepare(..., approx_linear=True)``) for models whose classifier is to run on the
+    approximate multiplier as well:  y = s_a*s_w*(AM(X,W^T) + X.Zw + Za.W^T + K*Za*Zw) + bias."""
+
+    def __init__(self, in_features, out_features, bias=True, a_bits=8, w_bits=8, use_ste_gradient=False):
+        super().__init__(in_features, out_features, bias, a_bits=a_bits, w_bits=w_bits)
+        self.gemm_op = self_ops.approx_gemm_baseline_op if use_ste_gradient else self_ops.approx_gemm_op
+
+    def forward(self, input):
+        self._update_ranges(input)
+        lead = input.shape[:-1]
+        x_codes = _to_codes(input.reshape(-1, self.in_features), self.activation_scale, self.activation_zp_neg, self.activation_quant_max)
+        w_codes = _to_codes(self.weight, self.weight_scale, self.weight_zp_neg, self.weight_quant_max)
+        z_a, z_w = self.activation_zp_neg, self.weight_zp_neg
+        total = self.gemm_op(x_codes, w_codes.t())
+        total = total + (z_w * x_codes.sum(dim=1, keepdim=True) + z_a * w_codes.sum(dim=1).unsqueeze(0)
+                         + (z_a * z_w) * float(self.in_features))
+        output = self.activation_scale * self.weight_scale * total
+        if self.bias is not None:
+            output = output + self.bias
+        return output.reshape(*lead, self.out_features)
+
+
 class ApproxConv2d(nn.Conv2d, _QuantParamsMixin):
     """Convolution whose code products come from the approximate-multiplier table
     (reference ``app_layers.py:116-185``)."""
@@ -229,6 +254,31 @@ class ApproxConv2d(nn.Conv2d, _QuantParamsMixin):
         input_fq = self.quantize(input, self.activation_scale, self.activation_zp_neg, self.activation_quant_max)
         weight_fq = self.quantize(self.weight, self.weight_scale, self.weight_zp_neg, self.weight_quant_max)
         return F.linear(input_fq, weight_fq, self.bias)
+
+
+class ApproxLinear(QuantLinear):
+    """Fully connected layer whose code products come from the approximate-multiplier table, the way ApproxConv2d
+    treats a convolution.  The reference keeps its linear layers on exact products (``app_layers.py:109-111``);
+    this variant is opt-in (``prepare(..., approx_linear=True)``) for models whose classifier is to run on the
+    approximate multiplier as well:  y = s_a*s_w*(AM(X,W^T) + X.Zw + Za.W^T + K*Za*Zw) + bias."""
+
+    def __init__(self, in_features, out_features, bias=True, a_bits=8, w_bits=8, use_ste_gradient=False):
+        super().__init__(in_features, out_features, bias, a_bits=a_bits, w_bits=w_bits)
+        self.gemm_op = self_ops.approx_gemm_baseline_op if use_ste_gradient else self_ops.approx_gemm_op
+
+    def forward(self, input):
+        self._update_ranges(input)
+        lead = input.shape[:-1]
+        x_codes = _to_codes(input.reshape(-1, self.in_features), self.activation_scale, self.activation_zp_neg, self.activation_quant_max)
+        w_codes = _to_codes(self.weight, self.weight_scale, self.weight_zp_neg, self.weight_quant_max)
+        z_a, z_w = self.activation_zp_neg, self.weight_zp_neg
+        total = self.gemm_op(x_codes, w_codes.t())
+        total = total + (z_w * x_codes.sum(dim=1, keepdim=True) + z_a * w_codes.sum(dim=1).unsqueeze(0)
+                         + (z_a * z_w) * float(self.in_features))
+        output = self.activation_scale * self.weight_scale * total
+        if self.bias is not None:
+            output = output + self.bias
+        return output.reshape(*lead, self.out_features)
 
 
 class ApproxConv2d(nn.Conv2d, _QuantParamsMixin):
@@ -310,14 +360,17 @@ class QuantAvgPool2d(nn.AvgPool2d):
 
 # ------------------------------------------------------------------------------------------ model rewriting
 def add_quant_op(module, a_bits=8, w_bits=8, q_type=0, q_level=0, weight_observer=0, bn_fuse=False, bn_fuse_calib=False,
-                 pretrained_model=False, qaft=False, ptq=False, percentile=0.9999, use_ste_gradient=False):
+                 pretrained_model=False, qaft=False, ptq=False, percentile=0.9999, use_ste_gradient=False, approx_linear=False):
     """Replace, in place and recursively, Linear / Conv2d / MaxPool2d / AvgPool2d children by their quantised
     versions; parameters are shared with the replaced module (reference ``app_layers.py:285-339``)."""
     opts = dict(a_bits=a_bits, w_bits=w_bits, q_type=q_type, q_level=q_level, weight_observer=weight_observer, bn_fuse=bn_fuse,
                 bn_fuse_calib=bn_fuse_calib, pretrained_model=pretrained_model, qaft=qaft, ptq=ptq, percentile=percentile,
-                use_ste_gradient=use_ste_gradient)
+                use_ste_gradient=use_ste_gradient, approx_linear=approx_linear)
     for name, child in module.named_children():
-        if isinstance(child, nn.Linear):
+        if isinstance(child, nn.Linear) and approx_linear:
+            new = ApproxLinear(child.in_features, child.out_features, bias=child.bias is not None, a_bits=a_bits, w_bits=w_bits,
+                               use_ste_gradient=use_ste_gradient)
+        elif isinstance(child, nn.Linear):
             new = QuantLinear(child.in_features, child.out_features, bias=child.bias is not None, a_bits=a_bits, w_bits=w_bits)
         elif isinstance(child, nn.Conv2d):
             new = ApproxConv2d(child.in_channels, child.out_channels, child.kernel_size, stride=child.stride, padding=child.padding,
@@ -340,13 +393,13 @@ def add_quant_op(module, a_bits=8, w_bits=8, q_type=0, q_level=0, weight_observe
 
 
 def prepare(model, inplace=False, a_bits=8, w_bits=8, q_type=0, q_level=0, weight_observer=0, bn_fuse=False, bn_fuse_calib=False,
-            pretrained_model=False, qaft=False, ptq=False, percentile=0.9999, use_ste_gradient=False):
+            pretrained_model=False, qaft=False, ptq=False, percentile=0.9999, use_ste_gradient=False, approx_linear=False):
     """Return ``model`` (a deep copy unless ``inplace``) with every supported layer quantised
-    (reference ``app_layers.py:342-377``)."""
+    (reference ``app_layers.py:342-377``; ``approx_linear`` is an addition: linear layers on the table as well)."""
     print(f'Quantizing model with a_bits={a_bits}, w_bits={w_bits}, use_ste_gradient={use_ste_gradient}')
     if not inplace:
         model = copy.deepcopy(model)
     add_quant_op(model, a_bits=a_bits, w_bits=w_bits, q_type=q_type, q_level=q_level, weight_observer=weight_observer,
                  bn_fuse=bn_fuse, bn_fuse_calib=bn_fuse_calib, pretrained_model=pretrained_model, qaft=qaft, ptq=ptq,
-                 percentile=percentile, use_ste_gradient=use_ste_gradient)
+                 percentile=percentile, use_ste_gradient=use_ste_gradient, approx_linear=approx_linear)
     return model

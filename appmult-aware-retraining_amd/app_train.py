@@ -25,10 +25,11 @@ import models  # noqa: E402
 import self_ops  # noqa: E402
 
 
-def build_model(arch, bits, use_ste_gradient, device, num_classes=10):
+def build_model(arch, bits, use_ste_gradient, device, num_classes=10, approx_linear=False):
     net = models.resnet18(num_classes) if arch == "resnet18" else models.vgg16(num_classes)
     net = net.to(device)
-    return app_layers.prepare(net, inplace=True, a_bits=bits, w_bits=bits, use_ste_gradient=use_ste_gradient)
+    return app_layers.prepare(net, inplace=True, a_bits=bits, w_bits=bits, use_ste_gradient=use_ste_gradient,
+                              approx_linear=approx_linear)
 
 
 @torch.no_grad()
@@ -69,12 +70,13 @@ def main(argv=None):
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--ste", action="store_true", help="straight-through gradients instead of the gradient tables")
     ap.add_argument("--optimizer", default="adam", choices=["adam", "sgd"])
+    ap.add_argument("--approx-linear", action="store_true", help="run the classifier on the table as well (the reference keeps it exact)")
     args = ap.parse_args(argv)
     assert torch.cuda.is_available(), "a GPU is required"
     device = torch.device("cuda")
     torch.manual_seed(199608224)
     self_ops.init_lookup_tables(device, args.lut, args.bits)
-    model = build_model(args.arch, args.bits, args.ste, device)
+    model = build_model(args.arch, args.bits, args.ste, device, approx_linear=args.approx_linear)
     xs, ys = synthetic_batches(args.steps + 1, args.batch, device)
     calibrate(model, xs[:1])
     opt = (torch.optim.Adam(model.parameters(), lr=1e-3, weight_decay=0.0) if args.optimizer == "adam"

@@ -358,3 +358,34 @@ def test_synthetic_training_steps_reduce_loss(ops, golden_dir):
     opt = torch.optim.Adam(net.parameters(), lr=1e-2)
     losses = [float(l) for l in T.train_steps(net, opt, xs * 12, ys * 12)]
     assert all(np.isfinite(losses)) and losses[-1] < losses[0]
+
+
+def test_approx_linear_equals_fake_quant_linear_with_exact_multiplier(ops, oracle):
+    """With LUT[a][b] = a*b the table classifier computes the same function as the fake-quantised one (the reference's
+    QuantLinear, app_layers.py:101-111), values and gradients, up to fp32 rounding of the scaling."""
+    import app_layers
+    self_ops, P = ops
+    keep = (P.lut_appmult, P.lut_grad_a, P.lut_grad_b)
+    try:
+        n = np.arange(128)
+        Sx, Sy = oracle.ste_tables16(7)
+        P.set_lookup_tables("cuda", oracle.pack_table(n[:, None] * n[None, :], 7, np.uint16),
+                            oracle.pack_table(Sx, 7, np.int16), oracle.pack_table(Sy, 7, np.int16))
+        torch.manual_seed(0)
+        ref = app_layers.QuantLinear(96, 10, bias=True, a_bits=7, w_bits=7).cuda()
+        lin = app_layers.ApproxLinear(96, 10, bias=True, a_bits=7, w_bits=7).cuda()
+        lin.load_state_dict(ref.state_dict())
+        x = torch.randn(33, 96, device="cuda")
+        x1, x2 = x.clone().requires_grad_(), x.clone().requires_grad_()
+        ref.train(); lin.train()
+        y1, y2 = ref(x1), lin(x2)
+        torch.testing.assert_close(y2, y1, rtol=1e-4, atol=1e-4 * float(y1.detach().abs().max()))
+        g = torch.randn_like(y1)
+        y1.backward(g); y2.backward(g)
+        torch.testing.assert_close(x2.grad, x1.grad, rtol=1e-3, atol=1e-4 * float(x1.grad.abs().max()))
+        torch.testing.assert_close(lin.weight.grad, ref.weight.grad, rtol=1e-3, atol=1e-4 * float(ref.weight.grad.abs().max()))
+        torch.testing.assert_close(lin.bias.grad, ref.bias.grad)
+        net = app_layers.prepare(torch.nn.Sequential(torch.nn.Linear(8, 4)), a_bits=7, w_bits=7, approx_linear=True)
+        assert isinstance(net[0], app_layers.ApproxLinear)
+    finally:
+        P.lut_appmult, P.lut_grad_a, P.lut_grad_b = keep
