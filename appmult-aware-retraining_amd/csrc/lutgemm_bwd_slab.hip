@@ -227,7 +227,7 @@ constexpr float kBwdHalfOffset = 1024.f;
 __global__ __launch_bounds__(1024) void lutgemm_gradB_slab16_kernel(
     const float* __restrict__ gC, const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, float* __restrict__ out,
     const int16_t* __restrict__ G, int lut_cols, int n_codes, uint32_t* __restrict__ flags, int M, int K, int N,
-    int m_chunk, float scale) {
+    int m_chunk, float scale, int n_tiles, int k_tiles, int splits) {
     constexpr int KT = kBwdKT16;
     __shared__ __align__(16) unsigned char smem[KT * 16384];
     const int tid = threadIdx.x;
@@ -235,9 +235,19 @@ __global__ __launch_bounds__(1024) void lutgemm_gradB_slab16_kernel(
     const int lane = tid & 63;
     const int rs = lane >> 4, cg = lane & 15;
     const uint32_t swap = (uint32_t)(rs & 1);
-    const int n0 = blockIdx.x * 64;
-    const int k0 = blockIdx.y * KT;
-    const int mb = blockIdx.z * m_chunk;
+    // Workgroups are dealt to the 8 XCDs round-robin by their index; the workgroups of one XCD (same index mod 8) take
+    // consecutive k tiles of one (column tile, M split), so that the rows of gC and A they all stream are shared in
+    // that XCD's L2 instead of being fetched once per XCD.
+    const int total = n_tiles * k_tiles * splits;
+    const int per_xcd = (total + 7) / 8;
+    const int logical = (int)(blockIdx.x % 8) * per_xcd + (int)(blockIdx.x / 8);
+    if (logical >= total) return;
+    const int k_tile = logical % k_tiles;
+    const int n_tile = (logical / k_tiles) % n_tiles;
+    const int split = logical / (k_tiles * n_tiles);
+    const int n0 = n_tile * 64;
+    const int k0 = k_tile * KT;
+    const int mb = split * m_chunk;
     const int me = min(M, mb + m_chunk);
 
     {   // expansion: wave-uniform code a, lanes = columns (the gathers of a wave stay inside one table row).
@@ -376,7 +386,7 @@ __global__ __launch_bounds__(1024) void lutgemm_gradB_slab16_kernel(
             v += red[(w * (KT + 1) + kk) * 64 + col];
             gs += red[(w * (KT + 1) + KT) * 64 + col];
         }
-        out[((size_t)blockIdx.z * K + k0 + kk) * N + n0 + col] = (v + kBwdHalfOffset * gs) * scale;
+        out[((size_t)split * K + k0 + kk) * N + n0 + col] = (v + kBwdHalfOffset * gs) * scale;
     }
 }
 
@@ -431,9 +441,11 @@ hipError_t launch_gradB_slab(const float* gC, const uint8_t* A, const uint8_t* B
     const int zs = (M + m_chunk - 1) / m_chunk;
     float* out = zs > 1 ? partials : gB;
     dim3 grid((N + 63) / 64, (K + kt - 1) / kt, zs);
-    if (half_slab)
-        hipLaunchKernelGGL(lutgemm_gradB_slab16_kernel, grid, dim3(1024), 0, stream, gC, A, B, out, lut, g.cols, 1 << g.bits,
-                           flags, M, K, N, m_chunk, scale);
+    if (half_slab) {
+        const int total = (int)(grid.x * grid.y * grid.z);
+        hipLaunchKernelGGL(lutgemm_gradB_slab16_kernel, dim3(8 * ((total + 7) / 8)), dim3(1024), 0, stream, gC, A, B, out, lut, g.cols,
+                           1 << g.bits, flags, M, K, N, m_chunk, scale, (int)grid.x, (int)grid.y, (int)grid.z);
+    }
     else if (regular && (K & 3) == 0)
         hipLaunchKernelGGL(lutgemm_gradB_slab_kernel<true>, grid, dim3(1024), 0, stream, gC, A, B, out, lut, g.cols, 1 << g.bits,
                            flags, M, K, N, m_chunk, scale, vec_ok);
