@@ -22,6 +22,8 @@
 // different rows at the same time; with 64 B rows they would all meet in the same few banks).
 // A workgroup (8 waves = 512 rows; two per CU, so that one computes while the other waits) owns 16 or 32 consecutive k and walks all column tiles; the slabs of four k
 // (40 KB) are double buffered in LDS and filled by LDS-direct loads while the previous four are consumed.
+#include <type_traits>
+
 #include "amr_common.h"
 
 namespace amr {
@@ -35,7 +37,6 @@ constexpr int kGaRowBytes = 2 * kGaCols + 16;             // 80
 constexpr int kGaSlabBytes = 128 * kGaRowBytes;           // one k: 10 KB
 constexpr int kGaChunkK = 4;
 constexpr int kGaChunkBytes = kGaChunkK * kGaSlabBytes;   // 40 KB
-constexpr int kGaKTmin = 16;                              // k per workgroup: 32 when K allows, else 16
 constexpr float kGaHalfOffset = 1024.f;
 constexpr int kGaWaves = 8;                               // 512 rows per workgroup; two workgroups share a CU (80 KB of LDS each)
 
@@ -98,7 +99,7 @@ __device__ __forceinline__ void ga_wait4(u32x4 (&d)[4]) {
 template <bool VEC, int kGaKT>
 __global__ __launch_bounds__(kGaWaves * 64, 2) void lutgemm_gradA_slab_kernel(
     const float* __restrict__ gC, const uint8_t* __restrict__ A, const u32x4* __restrict__ S, float* __restrict__ gA,
-    uint32_t* __restrict__ flags, int M, int K, int N, float scale, int rows_per_image, int row_blocks) {
+    uint32_t* __restrict__ flags, int M, int K, int N, float scale, int rows_per_image, int row_blocks, int xcd_order) {
     __shared__ __align__(16) unsigned char smem[2 * kGaChunkBytes];
     const int tid = threadIdx.x;
     const int wave = uniform(tid >> 6);
@@ -106,13 +107,21 @@ __global__ __launch_bounds__(kGaWaves * 64, 2) void lutgemm_gradA_slab_kernel(
     // A wave whose rows would stick out of M is shifted up so that all its rows exist; the rows it then
     // shares with the wave above are not stored twice (a wave entirely beyond M stores nothing but still
     // takes part in the copies and barriers).
-    // Workgroup order: 32 neighbouring row blocks, then all k groups, then the next 32 row blocks.  The workgroups
-    // in flight at one time then share both their slabs (same k group) and their rows of gC (same row block)
-    // in the caches; with all row blocks of one k group first, gC (re-read once per k group) came from HBM.
+    // Workgroup order: 32 neighbouring row blocks, then all k groups, then the next 32 row blocks, so that the workgroups
+    // in flight at one time share their slabs (same k group) and their rows of gC (same row block) in the caches.
+    // The hardware deals workgroups to the 8 XCDs round-robin by index; the workgroups of one XCD (same index mod 8)
+    // take consecutive positions of that order when there are few row blocks (xcd_order), so that the row blocks of
+    // one k group meet in ONE L2 and its slabs are fetched from memory once: with 8 row blocks every workgroup
+    // fetched its own copy otherwise.  With many row blocks each XCD already holds several per k group, and keeping
+    // a k group on one XCD measured a little slower.
     const int k_groups = K / kGaKT;
-    const int band = blockIdx.x / (32 * k_groups);                 // 32 row blocks x all k groups
+    const int total_wgs = row_blocks * k_groups;
+    const int per_xcd = (total_wgs + 7) / 8;
+    const int logical = xcd_order ? (int)(blockIdx.x % 8) * per_xcd + (int)(blockIdx.x / 8) : (int)blockIdx.x;
+    if (logical >= total_wgs) return;
+    const int band = logical / (32 * k_groups);                    // 32 row blocks x all k groups
     const int band_rows = min(32, row_blocks - 32 * band);
-    const int in_band = blockIdx.x - band * 32 * k_groups;
+    const int in_band = logical - band * 32 * k_groups;
     const int k_group = in_band / band_rows;
     const int row_block = 32 * band + (in_band - k_group * band_rows);
     const int m_first = (row_block * kGaWaves + wave) * 64;
@@ -220,8 +229,10 @@ hipError_t launch_gradA(const float* gC, const uint8_t* A, const uint8_t* B, flo
 
 // Bytes of the expanded table S, or 0 when the expanded-table gradA does not apply.
 size_t gradA_slab_workspace_bytes(const LutGeom& g, int M, int K, int N, bool force) {
-    // (below about 8192 rows the expansion, 2^b / M of the work but all of it HBM writes, costs more than it saves)
-    if (g.bits > 7 || M < (force ? 2048 : 8192) || (N % kGaCols) != 0 || (K % kGaKTmin) != 0 || (size_t)M * K >= (1ull << 31)) return 0;
+    // (below about 4096 rows, or 8192 for short K, the expansion, 2^b / M of the work but all of it HBM writes plus two
+    // more launches, costs more than it saves)
+    if (!force && M < 8192 && K < 1024) return 0;
+    if (g.bits > 7 || M < (force ? 2048 : 4096) || (N % kGaCols) != 0 || (K % 8) != 0 || ((K % 16) != 0 && (K % 24) != 0) || (size_t)M * K >= (1ull << 31)) return 0;
     return (size_t)(N / kGaCols) * K * kGaSlabBytes;
 }
 
@@ -240,17 +251,22 @@ hipError_t launch_gradA_slab(const float* gC, const uint8_t* A, const uint8_t* B
     const u32x4* S4 = reinterpret_cast<const u32x4*>(S);
     const dim3 block(kGaWaves * 64);
     const unsigned row_blocks = (unsigned)((M + rows_per_wg - 1) / rows_per_wg);
-    // 32 k per workgroup halve the gC reloads and the start-up cost per multiply-add (measured better than 16 k
-    // with twice the workgroups also where the last round of workgroups is half empty)
-    if ((K % 32) == 0) {
-        const dim3 grid(row_blocks * (K / 32));
-        if (vec) hipLaunchKernelGGL((lutgemm_gradA_slab_kernel<true, 32>), grid, block, 0, stream, gC, A, S4, gA, flags, M, K, N, scale, rows_per_image, (int)row_blocks);
-        else hipLaunchKernelGGL((lutgemm_gradA_slab_kernel<false, 32>), grid, block, 0, stream, gC, A, S4, gA, flags, M, K, N, scale, rows_per_image, (int)row_blocks);
-    } else {
-        const dim3 grid(row_blocks * (K / 16));
-        if (vec) hipLaunchKernelGGL((lutgemm_gradA_slab_kernel<true, 16>), grid, block, 0, stream, gC, A, S4, gA, flags, M, K, N, scale, rows_per_image, (int)row_blocks);
-        else hipLaunchKernelGGL((lutgemm_gradA_slab_kernel<false, 16>), grid, block, 0, stream, gC, A, S4, gA, flags, M, K, N, scale, rows_per_image, (int)row_blocks);
-    }
+    // k per workgroup: 32 halve the gC reloads and the start-up cost per multiply-add against 16 (measured better
+    // also where the last round of workgroups is half empty); 24 for few row blocks (measured).
+    const int xcd_order = row_blocks <= 16;
+    auto launch = [&](auto kt_tag) {
+        constexpr int KT = decltype(kt_tag)::value;
+        const dim3 grid(8 * ((row_blocks * (K / KT) + 7) / 8));
+        if (vec) hipLaunchKernelGGL((lutgemm_gradA_slab_kernel<true, KT>), grid, block, 0, stream, gC, A, S4, gA, flags, M, K, N, scale, rows_per_image, (int)row_blocks, xcd_order);
+        else hipLaunchKernelGGL((lutgemm_gradA_slab_kernel<false, KT>), grid, block, 0, stream, gC, A, S4, gA, flags, M, K, N, scale, rows_per_image, (int)row_blocks, xcd_order);
+    };
+    (void)n_cu;
+    int kt = (K % 32) == 0 ? 32 : 16;
+    if (row_blocks <= 16 && (K % 24) == 0) kt = 24;    // few row blocks: more, shorter workgroups fill the last round better
+    if ((K % kt) != 0) kt = (K % 24) == 0 ? 24 : 16;
+    if (kt == 32) launch(std::integral_constant<int, 32>{});
+    else if (kt == 24) launch(std::integral_constant<int, 24>{});
+    else launch(std::integral_constant<int, 16>{});
     e = hipGetLastError();
     if (e != hipSuccess) return e;
     // masked codes in A or table entries a half cannot hold: the gated direct kernel recomputes gA
