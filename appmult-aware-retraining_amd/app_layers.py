@@ -251,69 +251,6 @@ class ApproxConv2d(nn.Conv2d, _QuantParamsMixin):
 
     def forward(self, input):
         self._update_ranges(input)
-        input_fq = self.quantize(input, self.activation_scale, self.activation_zp_neg, self.activation_quant_max)
-        weight_fq = self.quantize(self.weight, self.weight_scale, self.weight_zp_neg, self.weight_quant_max)
-        return F.linear(input_fq, weight_fq, self.bias)
-
-
-class ApproxLinear(QuantLinear):
-    """Fully connected layer whose code products come from the approximate-multiplier table, the way ApproxConv2d
-    treats a convolution.  The reference keeps its linear layers on exact products (``app_layers.py:109-111``);
-    this variant is opt-in (``prepare(..., approx_linear=True)``) for models whose classifier is to run on the
-    approximate multiplier as well:  y = s_a*s_w*(AM(X,W^T) + X.Zw + Za.W^T + K*Za*Zw) + bias."""
-
-    def __init__(self, in_features, out_features, bias=True, a_bits=8, w_bits=8, use_ste_gradient=False):
-        super().__init__(in_features, out_features, bias, a_bits=a_bits, w_bits=w_bits)
-        self.gemm_op = self_ops.approx_gemm_baseline_op if use_ste_gradient else self_ops.approx_gemm_op
-
-    def forward(self, input):
-        self._update_ranges(input)
-        lead = input.shape[:-1]
-        x_codes = _to_codes(input.reshape(-1, self.in_features), self.activation_scale, self.activation_zp_neg, self.activation_quant_max)
-        w_codes = _to_codes(self.weight, self.weight_scale, self.weight_zp_neg, self.weight_quant_max)
-        z_a, z_w = self.activation_zp_neg, self.weight_zp_neg
-        total = self.gemm_op(x_codes, w_codes.t())
-        total = total + (z_w * x_codes.sum(dim=1, keepdim=True) + z_a * w_codes.sum(dim=1).unsqueeze(0)
-                         + (z_a * z_w) * float(self.in_features))
-        output = self.activation_scale * self.weight_scale * total
-        if self.bias is not None:
-            output = output + self.bias
-        return output.reshape(*lead, self.out_features)
-
-
-class ApproxConv2d(nn.Conv2d, _QuantParamsMixin):
-    """Convolution whose code products come from the approximate-multiplier table
-    (reference ``app_layers.py:116-185``)."""
-
-    def __init__(self, in_channels, out_channels, kernel_size, stride=1, padding=0, dilation=1, groups=1, bias=True,
-                 padding_mode="zeros", a_bits=8, w_bits=8, use_ste_gradient=False):
-        super().__init__(in_channels, out_channels, kernel_size, stride, padding, dilation, groups, bias, padding_mode)
-        self._init_quant(a_bits, w_bits)
-        self.conv2d_op = self_ops.approx_conv2d_baseline_op if use_ste_gradient else self_ops.approx_conv2d_op
-        self.reference_zero_point_terms = False     # True: evaluate the three correction terms as full convolutions
-
-    def quantize_v2(self, x, s, zpn, qmax):
-        return _to_codes(x, s, zpn, qmax)
-
-    def _zero_point_terms(self, x_codes, w_codes, conv_args):
-        """conv(X,Zw) + conv(Za,W) + conv(Za,Zw) without the three full convolutions: a convolution with a
-        constant operand factorises, conv(X, Zw*1) = Zw * box-sum of X over channels and window (one
-        output channel), conv(Za*1, W) = Za * (response of W to an all-ones image, batch of one), and
-        conv(Za*1, Zw*1) = Za*Zw*C * (number of taps inside the image).  All quantities are integer valued,
-        so as long as they stay below 2^24 the result is bit-identical to the literal form; autograd sees
-        ordinary torch ops and yields the same gradients for the codes."""
-        z_a, z_w = self.activation_zp_neg, self.weight_zp_neg
-        _, cin, h, w = x_codes.shape
-        kh, kw = w_codes.shape[2], w_codes.shape[3]
-        ones_k = torch.ones(1, 1, kh, kw, dtype=x_codes.dtype, device=x_codes.device)
-        ones_img = torch.ones(1, 1, h, w, dtype=x_codes.dtype, device=x_codes.device)
-        x_sum = F.conv2d(x_codes.sum(dim=1, keepdim=True), ones_k, **conv_args)                 # [B,1,oh,ow]
-        w_resp = F.conv2d(ones_img.expand(1, cin, h, w), w_codes, **conv_args)                  # [1,N,oh,ow]
-        taps = F.conv2d(ones_img, ones_k, **conv_args) * float(cin)                             # [1,1,oh,ow]
-        return z_w * x_sum + z_a * w_resp + (z_a * z_w) * taps
-
-    def forward(self, input):
-        self._update_ranges(input)
         conv_args = dict(bias=None, stride=self.stride, padding=self.padding, dilation=self.dilation, groups=self.groups)
         x_codes = self.quantize_v2(input, self.activation_scale, self.activation_zp_neg, self.activation_quant_max)
         w_codes = self.quantize_v2(self.weight, self.weight_scale, self.weight_zp_neg, self.weight_quant_max)
