@@ -112,6 +112,43 @@ def _to_codes_torch(x, scale, zp_neg, quant_max):
     return torch.clamp(affine - affine.detach() + torch.round(affine), 0, quant_max)
 
 
+class _ConvDequantFn(torch.autograd.Function):
+    """(s_a*s_w) * (c + z_w*x_sum + z_a*w_resp + z_a*z_w*taps) + bias from the GEMM's [B*L, N] rows to a contiguous
+    [B,N,oh,ow] activation in one device pass (same operations in the same order as the torch expression of
+    ApproxConv2d.forward, so the same bits); backward: one transposing pass for the rows plus three reductions."""
+
+    @staticmethod
+    def forward(ctx, c_rows, x_sum, w_resp, taps, z_a, z_w, s_a, s_w, bias, out_shape):
+        import approx_ops
+        one = lambda t: t.detach().reshape(1).contiguous()
+        z_a, z_w, s_a, s_w = one(z_a), one(z_w), one(s_a), one(s_w)
+        out = torch.empty(out_shape, dtype=torch.float32, device=c_rows.device)
+        approx_ops.conv_dequant(c_rows.contiguous(), x_sum.contiguous(), w_resp.contiguous(), taps.contiguous(), z_a, z_w, s_a, s_w,
+                                None if bias is None else bias.detach().contiguous(), out)
+        ctx.save_for_backward(z_a, z_w, s_a, s_w)
+        ctx.shapes = (c_rows.shape, x_sum.shape, w_resp.shape, bias is not None)
+        return out
+
+    @staticmethod
+    def backward(ctx, g):
+        import approx_ops
+        z_a, z_w, s_a, s_w = ctx.saved_tensors
+        c_shape, xs_shape, wr_shape, has_bias = ctx.shapes
+        g = g.contiguous()
+        s = s_a * s_w
+        g_rows = g_xs = g_wr = g_bias = None
+        if ctx.needs_input_grad[0]:
+            g_rows = torch.empty(c_shape, dtype=torch.float32, device=g.device)
+            approx_ops.conv_dequant_backward(g, s_a, s_w, g_rows)
+        if ctx.needs_input_grad[1]:
+            g_xs = ((z_w * s) * g.sum(dim=1, keepdim=True)).reshape(xs_shape)
+        if ctx.needs_input_grad[2]:
+            g_wr = ((z_a * s) * g.sum(dim=0, keepdim=True)).reshape(wr_shape)
+        if has_bias and ctx.needs_input_grad[8]:
+            g_bias = g.sum(dim=(0, 2, 3))
+        return g_rows, g_xs, g_wr, None, None, None, None, None, g_bias, None
+
+
 # ------------------------------------------------------------------------------------------ quantiser module
 class AsymmetricQuantizer(nn.Module):
     """Fake quantiser used in front of the pooling layers (reference ``app_layers.py:56-74``; note that its
@@ -211,18 +248,18 @@ class ApproxConv2d(nn.Conv2d, _QuantParamsMixin):
         self._init_quant(a_bits, w_bits)
         self.conv2d_op = self_ops.approx_conv2d_baseline_op if use_ste_gradient else self_ops.approx_conv2d_op
         self.reference_zero_point_terms = False     # True: evaluate the three correction terms as full convolutions
+        self.fused_dequant = True                   # False: zero-point terms and scaling as torch operators
 
     def quantize_v2(self, x, s, zpn, qmax):
         return _to_codes(x, s, zpn, qmax)
 
-    def _zero_point_terms(self, x_codes, w_codes, conv_args):
-        """conv(X,Zw) + conv(Za,W) + conv(Za,Zw) without the three full convolutions: a convolution with a
+    def _zero_point_parts(self, x_codes, w_codes, conv_args):
+        """The three factors of conv(X,Zw) + conv(Za,W) + conv(Za,Zw) = Zw*x_sum + Za*w_resp + Za*Zw*taps: a convolution with a
         constant operand factorises, conv(X, Zw*1) = Zw * box-sum of X over channels and window (one
         output channel), conv(Za*1, W) = Za * (response of W to an all-ones image, batch of one), and
         conv(Za*1, Zw*1) = Za*Zw*C * (number of taps inside the image).  All quantities are integer valued,
         so as long as they stay below 2^24 the result is bit-identical to the literal form; autograd sees
         ordinary torch ops and yields the same gradients for the codes."""
-        z_a, z_w = self.activation_zp_neg, self.weight_zp_neg
         _, cin, h, w = x_codes.shape
         cout, kh, kw = w_codes.shape[0], w_codes.shape[2], w_codes.shape[3]
         s, p, d = conv_args["stride"], conv_args["padding"], conv_args["dilation"]
@@ -237,7 +274,7 @@ class ApproxConv2d(nn.Conv2d, _QuantParamsMixin):
             x_sum = F.conv2d(xs, torch.ones(1, 1, kh, kw, dtype=xs.dtype, device=xs.device), **conv_args)
         w_resp = (w_codes.sum(dim=1).reshape(cout, kh * kw) @ mask).view(1, cout, oh, ow)           # [1,N,oh,ow]
         taps = (mask.sum(dim=0) * float(cin)).view(1, 1, oh, ow)
-        return z_w * x_sum + z_a * w_resp + (z_a * z_w) * taps
+        return x_sum, w_resp, taps
 
     def _tap_mask(self, h, w, kh, kw, stride, padding, dilation, dtype, device):
         """mask[i*kw+j, l] = 1 where tap (i,j) of output position l lies inside the h x w image (constant per
@@ -261,7 +298,13 @@ class ApproxConv2d(nn.Conv2d, _QuantParamsMixin):
             w_zp = torch.full_like(w_codes, self.weight_zp_neg)
             total = total + F.conv2d(x_codes, w_zp, **conv_args) + F.conv2d(x_zp, w_codes, **conv_args) + F.conv2d(x_zp, w_zp, **conv_args)
         else:
-            total = total + self._zero_point_terms(x_codes, w_codes, conv_args)
+            z_a, z_w = self.activation_zp_neg, self.weight_zp_neg
+            x_sum, w_resp, taps = self._zero_point_parts(x_codes, w_codes, conv_args)
+            if total.is_cuda and total.dtype == torch.float32 and self.fused_dequant:
+                rows = total.permute(0, 2, 3, 1).reshape(-1, total.shape[1])     # the GEMM's own rows: a view of the op's result
+                return _ConvDequantFn.apply(rows, x_sum, w_resp, taps, z_a, z_w, self.activation_scale, self.weight_scale,
+                                            self.bias, tuple(total.shape))
+            total = total + (z_w * x_sum + z_a * w_resp + (z_a * z_w) * taps)
         output = self.activation_scale * self.weight_scale * total
         if self.bias is not None:
             output += self.bias.view(1, -1, 1, 1)

@@ -42,6 +42,8 @@ _lib.amr_lut_gemm_backward.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, 
 _lib.amr_lut_gemm_backward_ex.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i, _i, _i, _i, _vp, _sz, _vp]
 _lib.amr_im2col_u8_f32.argtypes = [_vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp]
 _lib.amr_col2im_f32.argtypes = [_vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp]
+_lib.amr_conv_dequant_f32.argtypes = [_vp] * 10 + [_i, _i, _i, _vp]
+_lib.amr_conv_dequant_backward_f32.argtypes = [_vp, _vp, _vp, _vp, _i, _i, _i, _vp]
 _lib.amr_quantize_codes_f32.argtypes = [_vp, _vp, _vp, ctypes.c_float, _vp, _i64, _vp]
 _lib.amr_quantize_codes_backward_f32.argtypes = [_vp, _vp, _vp, _vp, ctypes.c_float, _vp, _i64, _vp]
 _lib.amr_lut_gemm_backward_workspace_bytes.argtypes = [_i, _i, _i]
@@ -215,6 +217,45 @@ def col2im(cols_tensor, x_tensor, kernel_size, stride, padding, dilation):
         rc = _lib.amr_col2im_f32(cols_tensor.data_ptr(), x_tensor.data_ptr(), Bn, C, H, W, kh, kw, stride, padding, dilation,
                                  _stream_ptr(dev))
     _raise_for(rc, "col2im")
+
+
+def conv_dequant(c_rows, x_sum, w_resp, taps, z_a, z_w, s_a, s_w, bias, out_tensor):
+    """out[b,n,pos] = (s_a*s_w) * (c_rows[b*L+pos, n] + ((z_w*x_sum[b,pos] + z_a*w_resp[n,pos]) + (z_a*z_w)*taps[pos])) + bias[n]:
+    the zero-point terms and scaling of the reference's ApproxConv2d.forward (micronet+/app_layers.py:175-183) in one pass.
+    c_rows float32 [B*L, N]; x_sum B*L elements; w_resp N*L; taps L; scalars one element each; out float32 [B, N, oh, ow]."""
+    tensors = [(c_rows, "c_rows"), (x_sum, "x_sum"), (w_resp, "w_resp"), (taps, "taps"), (z_a, "z_a"), (z_w, "z_w"), (s_a, "s_a"),
+               (s_w, "s_w"), (out_tensor, "out_tensor")] + ([(bias, "bias")] if bias is not None else [])
+    for t, name in tensors:
+        _check_input(t, torch.float32, name)
+    _check(out_tensor.dim() == 4 and c_rows.dim() == 2, "out must be 4-D and c_rows 2-D")
+    Bn, N = out_tensor.size(0), out_tensor.size(1)
+    L = out_tensor.size(2) * out_tensor.size(3)
+    _check(tuple(c_rows.shape) == (Bn * L, N), f"c_rows's shape should be {Bn * L} x {N}")
+    _check(x_sum.numel() == Bn * L and w_resp.numel() == N * L and taps.numel() == L, "x_sum, w_resp or taps has the wrong size")
+    _check(all(t.numel() == 1 for t in (z_a, z_w, s_a, s_w)), "z_a, z_w, s_a and s_w must hold one element")
+    _check(bias is None or bias.numel() == N, f"bias should have {N} elements")
+    dev = out_tensor.device
+    _check(all(t.device == dev for t, _ in tensors), "All tensors should be on the same device")
+    with torch.cuda.device(dev):
+        rc = _lib.amr_conv_dequant_f32(c_rows.data_ptr(), x_sum.data_ptr(), w_resp.data_ptr(), taps.data_ptr(), z_a.data_ptr(),
+                                       z_w.data_ptr(), s_a.data_ptr(), s_w.data_ptr(), bias.data_ptr() if bias is not None else None,
+                                       out_tensor.data_ptr(), Bn, N, L, _stream_ptr(dev))
+    _raise_for(rc, "conv_dequant")
+
+
+def conv_dequant_backward(g_tensor, s_a, s_w, gc_rows):
+    """gc_rows[b*L+pos, n] = (s_a*s_w) * g[b,n,pos]; g float32 [B,N,oh,ow] contiguous, gc_rows float32 [B*L, N]."""
+    for t, name in ((g_tensor, "g_tensor"), (s_a, "s_a"), (s_w, "s_w"), (gc_rows, "gc_rows")):
+        _check_input(t, torch.float32, name)
+    _check(g_tensor.dim() == 4 and gc_rows.dim() == 2, "g must be 4-D and gc_rows 2-D")
+    Bn, N = g_tensor.size(0), g_tensor.size(1)
+    L = g_tensor.size(2) * g_tensor.size(3)
+    _check(tuple(gc_rows.shape) == (Bn * L, N), f"gc_rows's shape should be {Bn * L} x {N}")
+    dev = g_tensor.device
+    with torch.cuda.device(dev):
+        rc = _lib.amr_conv_dequant_backward_f32(g_tensor.data_ptr(), s_a.data_ptr(), s_w.data_ptr(), gc_rows.data_ptr(), Bn, N, L,
+                                                _stream_ptr(dev))
+    _raise_for(rc, "conv_dequant_backward")
 
 
 def quantize_codes(x_tensor, scale_tensor, zp_neg_tensor, quant_max, codes_tensor):

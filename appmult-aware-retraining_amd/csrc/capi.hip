@@ -31,6 +31,9 @@ hipError_t launch_quantize_codes(const float* x, const float* scale, const float
 hipError_t launch_quantize_codes_backward(const float* g, const float* x, const float* scale, const float* zp_neg, float qmax,
                                           float* gx, size_t n, hipStream_t stream);
 hipError_t launch_zero_u32(void* p, size_t n_dwords, hipStream_t stream);
+hipError_t launch_dequant(const float* c, const float* xs, const float* wr, const float* tp, const float* za, const float* zw,
+                          const float* sa, const float* sw, const float* bias, float* out, int M, int N, int L, hipStream_t stream);
+hipError_t launch_dequant_grad(const float* g, const float* sa, const float* sw, float* gc, int M, int N, int L, hipStream_t stream);
 hipError_t launch_col2im_f32(const float* cols, float* x, int B, int C, int H, int W, int kh, int kw, int stride, int pad, int dil,
                              int oh, int ow, hipStream_t stream);
 hipError_t launch_im2col_u8_f32(const float* x, uint8_t* A, int B, int C, int H, int W, int kh, int kw, int stride, int pad,
@@ -309,6 +312,28 @@ int amr_col2im_f32(const float* cols, float* x, int B, int C, int H, int W, int 
     if (!cols || !x) return fail(AMR_EINVAL, "null pointer argument");
     hipError_t e = amr::launch_col2im_f32(cols, x, B, C, H, W, kh, kw, stride, pad, dil, oh, ow, reinterpret_cast<hipStream_t>(stream));
     return e == hipSuccess ? AMR_OK : hip_fail(e, "col2im launch");
+}
+
+int amr_conv_dequant_f32(const float* c, const float* x_sum, const float* w_resp, const float* taps, const float* z_a,
+                         const float* z_w, const float* s_a, const float* s_w, const float* bias, float* out, int batch,
+                         int out_channels, int positions, void* stream) {
+    if (batch < 0 || out_channels <= 0 || positions <= 0) return fail(AMR_EINVAL, "bad shape");
+    if (batch == 0) return AMR_OK;
+    if ((long)batch * positions >= (1L << 31)) return fail(AMR_EUNSUPPORTED, "more than 2^31 output positions");
+    if (!c || !x_sum || !w_resp || !taps || !z_a || !z_w || !s_a || !s_w || !out) return fail(AMR_EINVAL, "null pointer argument");
+    hipError_t e = amr::launch_dequant(c, x_sum, w_resp, taps, z_a, z_w, s_a, s_w, bias, out, batch * positions, out_channels, positions,
+                                       reinterpret_cast<hipStream_t>(stream));
+    return e == hipSuccess ? AMR_OK : hip_fail(e, "dequant launch");
+}
+
+int amr_conv_dequant_backward_f32(const float* g, const float* s_a, const float* s_w, float* g_c, int batch, int out_channels,
+                                  int positions, void* stream) {
+    if (batch < 0 || out_channels <= 0 || positions <= 0) return fail(AMR_EINVAL, "bad shape");
+    if (batch == 0) return AMR_OK;
+    if ((long)batch * positions >= (1L << 31)) return fail(AMR_EUNSUPPORTED, "more than 2^31 output positions");
+    if (!g || !s_a || !s_w || !g_c) return fail(AMR_EINVAL, "null pointer argument");
+    hipError_t e = amr::launch_dequant_grad(g, s_a, s_w, g_c, batch * positions, out_channels, positions, reinterpret_cast<hipStream_t>(stream));
+    return e == hipSuccess ? AMR_OK : hip_fail(e, "dequant backward launch");
 }
 
 int amr_quantize_codes_f32(const float* x, const float* scale, const float* zp_neg, float qmax, float* codes, int64_t n,

@@ -132,6 +132,20 @@ int amr_col2im_f32(const float *cols, float *x, int B, int C, int H, int W, int 
 int amr_set_expanded_table_kernels(int mode);
 
 /*
+ * Dequantisation behind the LUT convolution, from the GEMM's row layout to the NCHW activation in one pass:
+ *   out[b,n,pos] = (*s_a * *s_w) * (c[b*L+pos, n] + ((*z_w * x_sum[b*L+pos] + *z_a * w_resp[n*L+pos]) + (*z_a * *z_w) * taps[pos])) + bias[n]
+ * with L = positions; c [batch*L, out_channels], x_sum [batch*L], w_resp [out_channels*L], taps [L], out [batch,
+ * out_channels, L]; bias may be NULL; the four scalars are device pointers.  These are the zero-point terms and the
+ * scaling of the reference's ApproxConv2d.forward (micronet+/app_layers.py:175-183), every operation rounded on its
+ * own in that order.  The backward entry point gives g_c[b*L+pos, n] = (*s_a * *s_w) * g[b,n,pos].
+ */
+int amr_conv_dequant_f32(const float *c, const float *x_sum, const float *w_resp, const float *taps, const float *z_a,
+                         const float *z_w, const float *s_a, const float *s_w, const float *bias, float *out,
+                         int batch, int out_channels, int positions, void *stream);
+int amr_conv_dequant_backward_f32(const float *g, const float *s_a, const float *s_w, float *g_c, int batch,
+                                  int out_channels, int positions, void *stream);
+
+/*
  * Quantiser in front of the LUT GEMM: codes[i] = clamp(round(x[i] / *scale - *zp_neg), 0, qmax) as float32,
  * round half to even; scale and zp_neg are device pointers to one float each.  One pass instead of the
  * divide / subtract / round / straight-through / clamp chain of the reference's quantize_v2

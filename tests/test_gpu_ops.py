@@ -328,17 +328,20 @@ def test_approx_conv_layer_equals_fake_quant_conv_with_exact_multiplier(ops, ora
         layer.eval()                                   # freeze the observers: both forms see the same scales
         grads = []
         outs = []
-        for literal in (False, True):
+        for fused, literal in ((True, False), (False, False), (False, True)):   # one-pass kernel, torch operators, literal
             x.grad = None
             layer.weight.grad = None
-            layer.reference_zero_point_terms = literal
+            layer.bias.grad = None
+            layer.fused_dequant, layer.reference_zero_point_terms = fused, literal
             out = layer(x)
             out.square().mean().backward()
             outs.append(out.detach())
-            grads.append((x.grad.clone(), layer.weight.grad.clone()))
-        assert torch.equal(outs[0], outs[1])           # integer-valued terms below 2^24: bit-identical
-        torch.testing.assert_close(grads[0][0], grads[1][0], rtol=1e-5, atol=1e-6)
-        torch.testing.assert_close(grads[0][1], grads[1][1], rtol=1e-5, atol=1e-6)
+            grads.append((x.grad.clone(), layer.weight.grad.clone(), layer.bias.grad.clone()))
+        assert outs[0].is_contiguous()
+        assert torch.equal(outs[0], outs[1]) and torch.equal(outs[1], outs[2])   # integer-valued terms below 2^24: bit-identical
+        for k in (1, 2):
+            for a, b in zip(grads[0], grads[k]):
+                torch.testing.assert_close(a, b, rtol=1e-5, atol=1e-6)
     finally:
         P.lut_appmult, P.lut_grad_a, P.lut_grad_b = keep
 
@@ -389,3 +392,28 @@ def test_approx_linear_equals_fake_quant_linear_with_exact_multiplier(ops, oracl
         assert isinstance(net[0], app_layers.ApproxLinear)
     finally:
         P.lut_appmult, P.lut_grad_a, P.lut_grad_b = keep
+
+
+@pytest.mark.parametrize("cin,cout,k,stride,padding,hw,bias", [(6, 40, 3, 2, 1, 9, True), (16, 33, 1, 2, 0, 8, False), (3, 64, 3, 1, 1, 32, True)])
+def test_one_pass_dequantisation_equals_torch_operators(ops, golden_dir, cin, cout, k, stride, padding, hw, bias):
+    """ApproxConv2d with the shipped table: zero-point terms and scaling in one pass (contiguous NCHW result) against the
+    same expression in torch operators, on shapes whose channel and position counts are no multiples of the 32 x 32 tile."""
+    import app_layers as L
+    print("dequant", cin, cout, k, stride, padding, hw, bias, flush=True)
+    torch.manual_seed(1)
+    layer = L.ApproxConv2d(cin, cout, k, stride=stride, padding=padding, bias=bias, a_bits=7, w_bits=7).cuda().train()
+    x = torch.randn(5, cin, hw, hw, device="cuda", requires_grad=True)
+    layer(x)                                        # observers see data once
+    layer.eval()
+    res = []
+    for fused in (True, False):
+        layer.fused_dequant = fused
+        layer.zero_grad()
+        x.grad = None
+        y = layer(x)
+        y.square().mean().backward()
+        res.append((y.detach(), x.grad.clone(), layer.weight.grad.clone(), None if not bias else layer.bias.grad.clone()))
+    assert res[0][0].is_contiguous() and torch.equal(res[0][0], res[1][0])
+    for a, b in zip(res[0][1:], res[1][1:]):
+        if a is not None:
+            torch.testing.assert_close(a, b, rtol=1e-4, atol=1e-6 * float(b.abs().max()) + 1e-12)
