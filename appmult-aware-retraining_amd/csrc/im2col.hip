@@ -6,8 +6,8 @@
 // k = c*kh*kw + i*kw + j, padding positions hold code 0 (as F.pad(value=0) does there).
 //
 // A workgroup transposes a tile of 64 consecutive rows x up to 512 columns through LDS: for one column
-// the 64 lanes read 64 neighbouring pixels (coalesced), the finished tile is written out as contiguous
-// row segments with 32-bit stores.
+// the 64 lanes read 64 neighbouring pixels (coalesced), four columns are packed into a dword, and the
+// finished tile is written out as contiguous row segments with 32-bit stores.
 #include "amr_common.h"
 
 namespace amr {
@@ -17,12 +17,21 @@ constexpr int kIm2colKC = 512;
 __global__ __launch_bounds__(256) void im2col_u8_f32_kernel(const float* __restrict__ x, uint8_t* __restrict__ A, int C,
                                                             int H, int W, int kh, int kw, int stride, int pad, int dil, int oh,
                                                             int ow, int M, int K) {
-    __shared__ __align__(4) uint8_t tile[64][kIm2colKC + 4];
+    __shared__ uint32_t tile[64][kIm2colKC / 4 + 1];     // 64 rows x 512 codes, one dword = four columns (+1: no bank conflicts)
+    __shared__ int2 taps[kIm2colKC];                      // per column of the chunk: offset inside the image, (dy << 16 | dx)
     const int lane = threadIdx.x & 63;
     const int wave = uniform(threadIdx.x >> 6);
     const int m0 = blockIdx.x * 64;
     const int kc0 = blockIdx.y * kIm2colKC;
     const int kc = min(kIm2colKC, K - kc0);
+    // the column -> (channel, tap) decomposition is done once per workgroup, not once per load
+    for (int kk = threadIdx.x; kk < kIm2colKC; kk += 256) {
+        const int k = min(kc0 + kk, K - 1);
+        const int c = k / (kh * kw);
+        const int t = k - c * (kh * kw);
+        const int i = t / kw, j = t - i * kw;
+        taps[kk] = make_int2((c * H + i * dil) * W + j * dil, ((i * dil) << 16) | (j * dil));
+    }
     const int m = m0 + lane;
     const bool valid = m < M;
     const int mm = valid ? m : M - 1;
@@ -30,42 +39,42 @@ __global__ __launch_bounds__(256) void im2col_u8_f32_kernel(const float* __restr
     const int r = mm - b * (oh * ow);
     const int oy = r / ow, ox = r - oy * ow;
     const int y0 = oy * stride - pad, x0 = ox * stride - pad;
-    const float* xb = x + (size_t)b * C * H * W;
-    const int khw = kh * kw;
-    // Each wave takes every 4th column; kU columns per trip so that kU independent loads are in flight.
-    // Out-of-image taps read a clamped (valid) address and are zeroed by a select: no divergent branch.
-    constexpr int kU = 8;
-    for (int kb = wave; kb < kc; kb += 4 * kU) {
-        float v[kU];
-        bool in[kU];
+    const float* xb = x + (size_t)b * C * H * W + y0 * W + x0;      // window origin (may lie outside the image)
+    __syncthreads();
+    // A wave takes every 4th group of four columns, four groups (16 loads in flight) per trip.  Taps outside the
+    // image read the image's first pixel instead and are zeroed by a select: no divergent branch.
+    const int quads = (kc + 3) >> 2;
+    for (int q0 = wave; q0 < quads; q0 += 16) {
+        float v[4][4];
 #pragma unroll
-        for (int u = 0; u < kU; ++u) {
-            const int k = min(kc0 + kb + 4 * u, K - 1);   // wave-uniform: the divisions below are scalar
-            const int c = k / khw;
-            const int t = k - c * khw;
-            const int i = t / kw, j = t - i * kw;
-            const int yy = y0 + i * dil, xx = x0 + j * dil;
-            in[u] = valid && yy >= 0 && yy < H && xx >= 0 && xx < W;
-            const int yc = min(max(yy, 0), H - 1), xc = min(max(xx, 0), W - 1);
-            v[u] = xb[((size_t)c * H + yc) * W + xc];
+        for (int u = 0; u < 4; ++u)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int2 tp = taps[min(4 * (q0 + 4 * u) + e, kIm2colKC - 1)];      // wave-uniform address: one broadcast read
+                const int yy = y0 + (tp.y >> 16), xx = x0 + (tp.y & 0xffff);
+                const bool in = valid && yy >= 0 && yy < H && xx >= 0 && xx < W;
+                const float val = xb[in ? tp.x : -(y0 * W + x0)];
+                v[u][e] = in ? val : 0.f;
+            }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int q = q0 + 4 * u;
+            if (q < quads)
+                tile[lane][q] = (uint32_t)(int)v[u][0] | ((uint32_t)(int)v[u][1] << 8) | ((uint32_t)(int)v[u][2] << 16) |
+                                ((uint32_t)(int)v[u][3] << 24);
         }
-#pragma unroll
-        for (int u = 0; u < kU; ++u)
-            if (kb + 4 * u < kc) tile[lane][kb + 4 * u] = in[u] ? (uint8_t)(int)v[u] : (uint8_t)0;
     }
     __syncthreads();
     const int rows = min(64, M - m0);
     if (((K | kc0) & 3) == 0 && (((uintptr_t)A) & 3) == 0) {
-        const int dw = kc >> 2;              // kc is a multiple of 4 here
-        for (int idx = threadIdx.x; idx < rows * dw; idx += 256) {
-            const int rr = idx / dw, q = idx - rr * dw;
-            *reinterpret_cast<uint32_t*>(A + (size_t)(m0 + rr) * K + kc0 + 4 * q) = *reinterpret_cast<const uint32_t*>(&tile[rr][4 * q]);
-        }
+        // kc is a multiple of 4 here: a wave writes the dwords of a row, 256 contiguous bytes per store
+        for (int rr = wave; rr < rows; rr += 4)
+            for (int q = lane; q < (kc >> 2); q += 64)
+                *reinterpret_cast<uint32_t*>(A + (size_t)(m0 + rr) * K + kc0 + 4 * q) = tile[rr][q];
     } else {
-        for (int idx = threadIdx.x; idx < rows * kc; idx += 256) {
-            const int rr = idx / kc, q = idx - rr * kc;
-            A[(size_t)(m0 + rr) * K + kc0 + q] = tile[rr][q];
-        }
+        for (int rr = wave; rr < rows; rr += 4)
+            for (int q = lane; q < kc; q += 64)
+                A[(size_t)(m0 + rr) * K + kc0 + q] = (uint8_t)(tile[rr][q >> 2] >> (8 * (q & 3)));
     }
 }
 
