@@ -48,6 +48,7 @@ class ObserverBase(nn.Module):
 
 class MinMaxObserver(ObserverBase):
     """Running extremes."""
+    fused_mode = 1
 
     def __init__(self, q_level, out_channels):
         super().__init__(q_level)
@@ -59,6 +60,7 @@ class MinMaxObserver(ObserverBase):
 
 class MovingAverageMinMaxObserver(ObserverBase):
     """Exponential moving average of the per-batch extremes."""
+    fused_mode = 2
 
     def __init__(self, q_level, out_channels, momentum=0.1):
         super().__init__(q_level)
@@ -72,6 +74,30 @@ class MovingAverageMinMaxObserver(ObserverBase):
 def _scale_and_zero_point(observer, quant_max, eps):
     scale = torch.max((observer.max_val - observer.min_val) / quant_max, eps)
     return scale, torch.round(observer.min_val / scale)
+
+
+def _observe(observer, x, quant_max, eps, scale, zp_neg):
+    """One observer step on ``x`` followed by the scale / zero point it implies; returns (scale, zp_neg).
+    On the GPU the scalar arithmetic (range update, scale, zero point: a dozen one-element tensor operations in the
+    reference, ``app_layers.py:21-53,154-160``) is one launch that updates the observer's buffers and the given
+    ``scale`` / ``zp_neg`` buffers in place; the values are those of the tensor expressions."""
+    fused_mode = getattr(observer, "fused_mode", None)
+    ok = (fused_mode is not None and x.is_cuda and x.dtype == torch.float32 and
+          all(t.is_cuda and t.dtype == torch.float32 and t.numel() == 1 and t.is_contiguous()
+              for t in (observer.min_val, observer.max_val, scale, zp_neg)))
+    if not ok:
+        observer(x)
+        return _scale_and_zero_point(observer, quant_max, eps)
+    import approx_ops
+    with torch.no_grad():
+        lo, hi = torch.aminmax(x)
+        mode = 0 if observer.num_flag == 0 else fused_mode
+        observer.num_flag = 1
+        approx_ops.observer_update(lo.reshape(1), hi.reshape(1), observer.min_val, observer.max_val, scale, zp_neg, mode,
+                                   getattr(observer, "momentum", 0.0), float(quant_max), float(eps),
+                                   # torch divides by a host-side scalar through its reciprocal rounded to float32
+                                   0.0 if quant_max.is_cuda else float(torch.tensor(1.0, dtype=torch.float32) / quant_max.to(torch.float32)))
+    return scale, zp_neg
 
 
 class _ToCodesFn(torch.autograd.Function):
@@ -164,8 +190,8 @@ class AsymmetricQuantizer(nn.Module):
 
     def forward(self, input):
         if self.training:
-            self.observer(input)
-            self.scale, self.zero_point_neg = _scale_and_zero_point(self.observer, self.quant_max_val, self.eps)
+            self.scale, self.zero_point_neg = _observe(self.observer, input, self.quant_max_val, self.eps, self.scale,
+                                                       self.zero_point_neg)
         q = input / self.scale - self.zero_point_neg
         q = q - q.detach() + torch.round(q)
         return (torch.clamp(q, 0, self.quant_max_val) + self.zero_point_neg) * self.scale
@@ -187,12 +213,10 @@ class _QuantParamsMixin:
 
     def _update_ranges(self, input):
         if self.training:
-            self.activation_observer(input)
-            self.activation_scale, self.activation_zp_neg = _scale_and_zero_point(
-                self.activation_observer, self.activation_quant_max, self.eps)
-            self.weight_observer(self.weight)
-            self.weight_scale, self.weight_zp_neg = _scale_and_zero_point(
-                self.weight_observer, self.weight_quant_max, self.eps)
+            self.activation_scale, self.activation_zp_neg = _observe(
+                self.activation_observer, input, self.activation_quant_max, self.eps, self.activation_scale, self.activation_zp_neg)
+            self.weight_scale, self.weight_zp_neg = _observe(
+                self.weight_observer, self.weight, self.weight_quant_max, self.eps, self.weight_scale, self.weight_zp_neg)
 
 
 # ------------------------------------------------------------------------------------------ layers
@@ -294,8 +318,8 @@ class ApproxConv2d(nn.Conv2d, _QuantParamsMixin):
         total = self.conv2d_op(x_codes, w_codes, **conv_args)       # approximate products of the codes
         if self.reference_zero_point_terms:
             # the reference's literal form: three full convolutions with constant operands
-            x_zp = torch.full_like(x_codes, self.activation_zp_neg)
-            w_zp = torch.full_like(w_codes, self.weight_zp_neg)
+            x_zp = torch.ones_like(x_codes) * self.activation_zp_neg
+            w_zp = torch.ones_like(w_codes) * self.weight_zp_neg
             total = total + F.conv2d(x_codes, w_zp, **conv_args) + F.conv2d(x_zp, w_codes, **conv_args) + F.conv2d(x_zp, w_zp, **conv_args)
         else:
             z_a, z_w = self.activation_zp_neg, self.weight_zp_neg

@@ -44,6 +44,7 @@ _lib.amr_im2col_u8_f32.argtypes = [_vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i,
 _lib.amr_col2im_f32.argtypes = [_vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp]
 _lib.amr_conv_dequant_f32.argtypes = [_vp] * 10 + [_i, _i, _i, _vp]
 _lib.amr_conv_dequant_backward_f32.argtypes = [_vp, _vp, _vp, _vp, _i, _i, _i, _vp]
+_lib.amr_observer_update_f32.argtypes = [_vp] * 6 + [_i] + [ctypes.c_float] * 5 + [_vp]
 _lib.amr_quantize_codes_f32.argtypes = [_vp, _vp, _vp, ctypes.c_float, _vp, _i64, _vp]
 _lib.amr_quantize_codes_backward_f32.argtypes = [_vp, _vp, _vp, _vp, ctypes.c_float, _vp, _i64, _vp]
 _lib.amr_lut_gemm_backward_workspace_bytes.argtypes = [_i, _i, _i]
@@ -256,6 +257,22 @@ def conv_dequant_backward(g_tensor, s_a, s_w, gc_rows):
         rc = _lib.amr_conv_dequant_backward_f32(g_tensor.data_ptr(), s_a.data_ptr(), s_w.data_ptr(), gc_rows.data_ptr(), Bn, N, L,
                                                 _stream_ptr(dev))
     _raise_for(rc, "conv_dequant_backward")
+
+
+def observer_update(cur_min, cur_max, min_val, max_val, scale, zp_neg, mode, momentum, quant_max, eps, inv_quant_max=0.0):
+    """One launch for the range update of an observer (mode 0 first batch, 1 running extremes, 2 moving average) and the
+    scale / zero point that follow from it; all tensors one float32 element on the device, the last four updated in place.
+    inv_quant_max != 0: the range is multiplied by it instead of divided by quant_max."""
+    for t, name in ((cur_min, "cur_min"), (cur_max, "cur_max"), (min_val, "min_val"), (max_val, "max_val"), (scale, "scale"),
+                    (zp_neg, "zp_neg")):
+        _check_input(t, torch.float32, name)
+        _check(t.numel() == 1, f"{name} must hold one element")
+    dev = cur_min.device
+    with torch.cuda.device(dev):
+        rc = _lib.amr_observer_update_f32(cur_min.data_ptr(), cur_max.data_ptr(), min_val.data_ptr(), max_val.data_ptr(),
+                                          scale.data_ptr(), zp_neg.data_ptr(), int(mode), float(1 - momentum), float(momentum),
+                                          float(quant_max), float(inv_quant_max), float(eps), _stream_ptr(dev))
+    _raise_for(rc, "observer_update")
 
 
 def quantize_codes(x_tensor, scale_tensor, zp_neg_tensor, quant_max, codes_tensor):

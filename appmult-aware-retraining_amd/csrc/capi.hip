@@ -26,6 +26,9 @@ size_t gradA_slab_workspace_bytes(const LutGeom& g, int M, int K, int N, bool fo
 hipError_t launch_gradA_slab(const float* gC, const uint8_t* A, const uint8_t* B, float* gA, const int16_t* lut,
                              const LutGeom& g, int M, int K, int N, float scale, int n_cu, uint32_t* flags, void* S,
                              int rows_per_image, hipStream_t stream);
+hipError_t launch_observer_update(const float* cur_min, const float* cur_max, float* min_val, float* max_val, float* scale,
+                                  float* zp_neg, int mode, float keep, float momentum, float qmax, float inv_qmax, float eps,
+                                  hipStream_t stream);
 hipError_t launch_quantize_codes(const float* x, const float* scale, const float* zp_neg, float qmax, float* codes, size_t n,
                                  hipStream_t stream);
 hipError_t launch_quantize_codes_backward(const float* g, const float* x, const float* scale, const float* zp_neg, float qmax,
@@ -334,6 +337,16 @@ int amr_conv_dequant_backward_f32(const float* g, const float* s_a, const float*
     if (!g || !s_a || !s_w || !g_c) return fail(AMR_EINVAL, "null pointer argument");
     hipError_t e = amr::launch_dequant_grad(g, s_a, s_w, g_c, batch * positions, out_channels, positions, reinterpret_cast<hipStream_t>(stream));
     return e == hipSuccess ? AMR_OK : hip_fail(e, "dequant backward launch");
+}
+
+int amr_observer_update_f32(const float* cur_min, const float* cur_max, float* min_val, float* max_val, float* scale,
+                            float* zp_neg, int mode, float keep, float momentum, float quant_max, float inv_quant_max, float eps,
+                            void* stream) {
+    if (mode < 0 || mode > 2 || !(quant_max > 0.f)) return fail(AMR_EINVAL, "bad observer mode or code range");
+    if (!cur_min || !cur_max || !min_val || !max_val || !scale || !zp_neg) return fail(AMR_EINVAL, "null pointer argument");
+    hipError_t e = amr::launch_observer_update(cur_min, cur_max, min_val, max_val, scale, zp_neg, mode, keep, momentum, quant_max, inv_quant_max, eps,
+                                               reinterpret_cast<hipStream_t>(stream));
+    return e == hipSuccess ? AMR_OK : hip_fail(e, "observer update launch");
 }
 
 int amr_quantize_codes_f32(const float* x, const float* scale, const float* zp_neg, float qmax, float* codes, int64_t n,

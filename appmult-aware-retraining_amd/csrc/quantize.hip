@@ -63,6 +63,41 @@ __global__ __launch_bounds__(256) void quantize_codes_backward_kernel(const floa
     }
 }
 
+// Observer step + quantisation parameters in one launch (one thread): the scalar updates the reference spreads over a
+// dozen tensor operations per layer and step (micronet+/app_layers.py:21-53 observers, :154-160 scale / zero point).
+//   mode 0: first batch, min/max := current;  mode 1: running extremes;  mode 2: keep * old + momentum * current
+//   (keep = 1 - momentum, rounded by the caller the way the tensor expression rounds it)
+//   scale = max((max - min) / qmax, eps)  [or (max - min) * inv_qmax when inv_qmax != 0];  zp_neg = round(min / scale)
+// Same operations in the same order as the tensor expressions, each rounded on its own.
+__global__ void observer_update_kernel(const float* __restrict__ cur_min, const float* __restrict__ cur_max, float* __restrict__ min_val,
+                                       float* __restrict__ max_val, float* __restrict__ scale, float* __restrict__ zp_neg, int mode,
+                                       float keep, float momentum, float qmax, float inv_qmax, float eps) {
+    if (threadIdx.x != 0 || blockIdx.x != 0) return;
+    float lo = *cur_min, hi = *cur_max;
+    if (mode == 1) {
+        lo = fminf(lo, *min_val);
+        hi = fmaxf(hi, *max_val);
+    } else if (mode == 2) {
+        lo = __fadd_rn(__fmul_rn(keep, *min_val), __fmul_rn(momentum, lo));
+        hi = __fadd_rn(__fmul_rn(keep, *max_val), __fmul_rn(momentum, hi));
+    }
+    *min_val = lo;
+    *max_val = hi;
+    // (a division by a host-side scalar is a multiplication by its rounded reciprocal in the tensor library: inv_qmax != 0)
+    const float range = __fsub_rn(hi, lo);
+    const float s = fmaxf(inv_qmax != 0.f ? __fmul_rn(range, inv_qmax) : __fdiv_rn(range, qmax), eps);
+    *scale = s;
+    *zp_neg = rintf(__fdiv_rn(lo, s));
+}
+
+hipError_t launch_observer_update(const float* cur_min, const float* cur_max, float* min_val, float* max_val, float* scale,
+                                  float* zp_neg, int mode, float keep, float momentum, float qmax, float inv_qmax, float eps,
+                                  hipStream_t stream) {
+    hipLaunchKernelGGL(observer_update_kernel, dim3(1), dim3(64), 0, stream, cur_min, cur_max, min_val, max_val, scale, zp_neg, mode,
+                       keep, momentum, qmax, inv_qmax, eps);
+    return hipGetLastError();
+}
+
 hipError_t launch_quantize_codes(const float* x, const float* scale, const float* zp_neg, float qmax, float* codes, size_t n,
                                  hipStream_t stream) {
     const int vec = ((((uintptr_t)x) | ((uintptr_t)codes)) & 15) == 0;

@@ -146,6 +146,17 @@ int amr_conv_dequant_backward_f32(const float *g, const float *s_a, const float 
                                   int out_channels, int positions, void *stream);
 
 /*
+ * Range tracking and quantisation parameters of one tensor in one launch (all pointers: one float in device memory).
+ * mode 0: min_val/max_val := cur_min/cur_max (first batch); 1: running extremes; 2: keep * old + momentum * current;
+ * then *scale = max((max - min) / quant_max, eps) -- or (max - min) * inv_quant_max when inv_quant_max != 0, which is
+ * what the tensor library computes for a division by a host-side scalar -- and *zp_neg = round(min / *scale).  The scalar tensor operations of the
+ * reference's observers and quantisers (micronet+/app_layers.py:21-53, :154-160), each rounded on its own in that order.
+ */
+int amr_observer_update_f32(const float *cur_min, const float *cur_max, float *min_val, float *max_val, float *scale,
+                            float *zp_neg, int mode, float keep, float momentum, float quant_max, float inv_quant_max,
+                            float eps, void *stream);
+
+/*
  * Quantiser in front of the LUT GEMM: codes[i] = clamp(round(x[i] / *scale - *zp_neg), 0, qmax) as float32,
  * round half to even; scale and zp_neg are device pointers to one float each.  One pass instead of the
  * divide / subtract / round / straight-through / clamp chain of the reference's quantize_v2

@@ -417,3 +417,32 @@ def test_one_pass_dequantisation_equals_torch_operators(ops, golden_dir, cin, co
     for a, b in zip(res[0][1:], res[1][1:]):
         if a is not None:
             torch.testing.assert_close(a, b, rtol=1e-4, atol=1e-6 * float(b.abs().max()) + 1e-12)
+
+
+@pytest.mark.parametrize("qmax_on_device", [False, True])
+@pytest.mark.parametrize("kind", ["ema", "extremes"])
+def test_one_launch_observer_update_equals_tensor_expressions(ops, kind, qmax_on_device):
+    """Range tracking + scale + zero point in one launch against the reference's tensor expressions
+    (app_layers.py:21-53, :154-160) over several batches: the same bits in every buffer."""
+    import app_layers as L
+    make = (lambda: L.MovingAverageMinMaxObserver("L", None)) if kind == "ema" else (lambda: L.MinMaxObserver("L", None))
+    fused, plain = make().cuda(), make().cuda()
+    plain.fused_mode = None                                   # tensor expressions
+    qmax, eps = torch.tensor(127.0), torch.tensor(torch.finfo(torch.float32).eps)
+    if qmax_on_device:                                        # the pooling quantisers hold it as a device buffer: true division
+        qmax, eps = qmax.cuda(), eps.cuda()
+    sc, zp = torch.ones(1, device="cuda"), torch.zeros(1, device="cuda")
+    g = torch.Generator(device="cuda").manual_seed(4)
+    for step in range(6):
+        x = torch.randn(64, 33, device="cuda", generator=g) * (1 + step) + 0.3 * step
+        s1, z1 = L._observe(fused, x, qmax, eps, sc, zp)
+        s2, z2 = L._observe(plain, x, qmax, eps, None, None)
+        assert s1.data_ptr() == sc.data_ptr()                 # updated in place
+        assert torch.equal(s1.reshape(1), s2.reshape(1)) and torch.equal(z1.reshape(1), z2.reshape(1)), step
+        assert torch.equal(fused.min_val.reshape(1), plain.min_val.reshape(1)) and torch.equal(fused.max_val.reshape(1), plain.max_val.reshape(1))
+    x = torch.zeros(8, device="cuda")                         # constant input: scale falls back to eps
+    fused2, plain2 = make().cuda(), make().cuda()
+    plain2.fused_mode = None
+    s1, z1 = L._observe(fused2, x, qmax, eps, sc, zp)
+    s2, z2 = L._observe(plain2, x, qmax, eps, None, None)
+    assert torch.equal(s1.reshape(1), s2.reshape(1)) and torch.equal(z1.reshape(1), z2.reshape(1))
