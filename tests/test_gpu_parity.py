@@ -245,19 +245,22 @@ def test_backward_large_m_masked_codes(lib, oracle):
 
 
 # K % 8 == 0, N % 64 == 0, M % 128 == 0 and M >= 4096: gradB runs on the expanded table held as halves (entries - 1024)
-# (N % 32 == 0, K % 16 == 0 and M >= 8192: gradA runs on its own expanded table, 16 or 32 k per workgroup, also with a
-# ragged last row block)
+# (N % 32 == 0, K % 16 == 0 and M >= 2048: gradA runs on its own expanded table, 16, 32 or 48 k per workgroup and one to
+# six column tiles, also with a ragged last row block)
 HALF_SLAB_SHAPES = [(4096, 8, 64), (4224, 24, 128), (8192, 64, 64), (16384, 16, 192), (8200, 48, 96), (9001, 64, 32),
-                    (4100, 32, 64)]
+                    (4100, 32, 64), (2148, 144, 160), (5000, 80, 128)]
 
 
 @pytest.mark.parametrize("bits", [7, 6, 4])
+@pytest.mark.parametrize("low", [-1024, -2048])
 @pytest.mark.parametrize("shape", HALF_SLAB_SHAPES)
-def test_backward_half_slab_tables_inside_the_exact_range(lib, oracle, bits, shape):
-    print("backward half slab", bits, shape, flush=True)
+def test_backward_half_slab_tables_inside_the_exact_range(lib, oracle, bits, shape, low):
+    print("backward half slab", bits, shape, low, flush=True)
     rng, A, B, _ = rand_case(hash((bits, shape, "h")) % 2**32, *shape, bits)
     n = 1 << bits
-    Ga, Gb = rng.integers(-1024, 3073, (n, n)), rng.integers(-1024, 3073, (n, n))
+    # [-1024, 3072]: halves of the entries - 1024; [-2048, 2048]: gradA holds the entries themselves
+    Ga, Gb = rng.integers(low, low + 4097, (n, n)), rng.integers(-1024, 3073, (n, n))
+    Ga[0, 0], Ga[1, 1], Ga[2, 2], Ga[3, 3] = low, low + 4096, low + 4094, low + 2
     Gb[0, 0], Gb[1, 1], Gb[2, 2], Gb[3, 3] = -1024, 3072, 3070, -1022     # ends of the range; even values beyond +-2048
     la, lb = oracle.pack_table(Ga, bits, np.int16), oracle.pack_table(Gb, bits, np.int16)
     g = (rng.standard_normal((shape[0], shape[2])) + 0.25).astype(np.float32)      # non-zero column sums
