@@ -55,12 +55,11 @@ constexpr int kGaStageBytes = kGaRows * kGaCols * 4;      // 64 KB
 static_assert(kGaStageBase + kGaStageBytes == 160 * 1024, "the workgroup uses the whole LDS of a CU");
 
 // ------------------------------------------------------------------------------------------ expand
-// grid (n_tiles, K / 8), 256 threads.  Requires N % 32 == 0 and K % 8 == 0.
-constexpr int kGaExpandK = 8;
+// grid (n_tiles, ceil(K / 4 / quads_per_wg)), 256 threads.  Requires N % 32 == 0 and K % 4 == 0.
 
 __global__ __launch_bounds__(256) void expand_gradA_kernel(const uint8_t* __restrict__ B, const uint32_t* __restrict__ lut32,
                                                            int lut_dwords, int lut_cols, int n_codes,
-                                                           uint32_t* __restrict__ S, uint32_t* __restrict__ flags, int K, int N) {
+                                                           uint32_t* __restrict__ S, uint32_t* __restrict__ flags, int K, int N, int quads_per_wg) {
     extern __shared__ __align__(16) unsigned char smem[];
     __shared__ int extremes[2];
     uint32_t* s32 = reinterpret_cast<uint32_t*>(smem);
@@ -86,8 +85,9 @@ __global__ __launch_bounds__(256) void expand_gradA_kernel(const uint8_t* __rest
     const int ks = lane >> 4, cp = lane & 15;
     const int n = blockIdx.x * kGaCols + 2 * cp;
     bool inexact = false;
-    for (int pp = 0; pp < kGaExpandK / 4; ++pp) {
-        const int kq = blockIdx.y * (kGaExpandK / 4) + pp;
+    for (int pp = 0; pp < quads_per_wg; ++pp) {
+        const int kq = blockIdx.y * quads_per_wg + pp;
+        if (4 * kq >= K) break;
         const int k = 4 * kq + ks;
         const int b0 = (int)B[(size_t)k * N + n], b1 = (int)B[(size_t)k * N + n + 1];
         uint32_t* chunk = S + ((size_t)blockIdx.x * (K / 4) + kq) * (kGaChunkBytes / 4);
@@ -122,44 +122,56 @@ __device__ __forceinline__ void ga_read(u32x4& d, uint32_t codeword, uint32_t la
                  : "memory");
 }
 
-// grid: row_blocks * K / KT workgroups (rounded up to a multiple of 8), 1024 threads.  Requires N % 32 == 0,
-// K % KT == 0, M*K < 2^31, gC 16-byte aligned.
+// grid: 8 * (workgroups per XCD, at most one per CU) workgroups of 1024 threads; every workgroup walks several tiles
+// (512 rows x KT k) one after the other.  Requires N % 32 == 0, K % KT == 0, M >= 32, M*K < 2^31, gC 16-byte aligned.
 // rows_per_image = 0: gA row-major [M,K]; L > 0: image-major transposed gA[m / L][k][m % L].
 template <int kGaKT>
 __global__ __launch_bounds__(kGaWaves * 64) void lutgemm_gradA_slab_kernel(
     const float* __restrict__ gC, const uint8_t* __restrict__ A, const u32x4* __restrict__ S, float* __restrict__ gA,
-    uint32_t* __restrict__ flags, int M, int K, int N, float scale, int rows_per_image, int row_blocks, int band_rows_max,
-    int xcd_order) {
+    uint32_t* __restrict__ flags, int M, int K, int N, float scale, int rows_per_image, int row_blocks, int band_rows_max) {
     __shared__ __align__(16) unsigned char smem[kGaStageBase + kGaStageBytes];
     constexpr int CH = kGaKT / kGaChunkK;                  // chunks per column tile
     constexpr int NTU = (CH % kGaBufs) == 0 ? 1 : kGaBufs; // column tiles per unrolled pass: the buffer of a chunk is then static
+    constexpr int NST = 2 * CH;                            // stores per lane at the end of a tile
     static_assert(CH >= 4, "the bookkeeping of outstanding loads assumes at least four chunks per column tile");
     const int tid = threadIdx.x;
     const int wave = uniform(tid >> 6);
     const int lane = tid & 63;
     const int quad = lane >> 2, c = lane & 3;
 
-    // Workgroup order: a band of row blocks, then all k groups, then the next band, so that the workgroups in
-    // flight at one time share their chunks (same k group) and their rows of gC (same row block) in the caches.
-    // The hardware deals workgroups to the 8 XCDs round-robin by index; with xcd_order the workgroups of one XCD
-    // (same index mod 8) take consecutive positions of that order, so that they meet in ONE L2.
+    // Tile order: a band of row blocks, then all k groups, then the next band, so that the tiles in flight at one
+    // time share their chunks (same k group) and their rows of gC (same row block) in the caches.  The hardware deals
+    // workgroups to the 8 XCDs round-robin by index; the workgroups of one XCD (same index mod 8) walk ONE eighth of
+    // that order together, so that they meet in one L2.  A workgroup keeps its CU for all its tiles: the loads of
+    // the next tile are under way while the current one is finished (a fresh workgroup per tile spent 7 us, a third
+    // of a tile of two column tiles, on start-up, first loads and drain).
     const int k_groups = K / kGaKT;
-    const int total_wgs = row_blocks * k_groups;
-    const int per_xcd = (total_wgs + 7) / 8;
-    const int logical = xcd_order ? (int)(blockIdx.x % 8) * per_xcd + (int)(blockIdx.x / 8) : (int)blockIdx.x;
-    if (logical >= total_wgs) return;
-    const int band = logical / (band_rows_max * k_groups);
-    const int band_rows = min(band_rows_max, row_blocks - band_rows_max * band);
-    const int in_band = logical - band * band_rows_max * k_groups;
-    const int k_group = in_band / band_rows;
-    const int row_block = band_rows_max * band + (in_band - k_group * band_rows);
-    const int m_wave = row_block * kGaRows + wave * kGaRowsPerWave;
-    const int k0 = k_group * kGaKT;
+    const int total_tiles = row_blocks * k_groups;
+    const int per_xcd = (total_tiles + 7) / 8;
+    const int xcd = (int)(blockIdx.x % 8), pos_stride = (int)(gridDim.x / 8);
     const int n_tiles = N / kGaCols;
-    const int total = n_tiles * CH;                          // chunks this workgroup walks: (tile, four k)
+    const int total = n_tiles * CH;                          // chunks of a tile: (column tile, four k)
     const float offset = (float)flags[3];
+    struct Tile { int k0, m_wave; bool valid; };
+    auto decode = [&](int pos) {
+        Tile t;
+        const int logical = xcd * per_xcd + pos;
+        t.valid = pos < per_xcd && logical < total_tiles;
+        const int lg = t.valid ? logical : 0;
+        const int band = lg / (band_rows_max * k_groups);
+        const int band_rows = min(band_rows_max, row_blocks - band_rows_max * band);
+        const int in_band = lg - band * band_rows_max * k_groups;
+        const int k_group = in_band / band_rows;
+        const int row_block = band_rows_max * band + (in_band - k_group * band_rows);
+        t.k0 = k_group * kGaKT;
+        t.m_wave = row_block * kGaRows + wave * kGaRowsPerWave;
+        return t;
+    };
+    int pos = (int)(blockIdx.x / 8);
+    Tile cur = decode(pos);
+    if (!cur.valid) return;
+    Tile nxt = decode(pos + pos_stride);
 
-    // Rows of this lane: m_wave + 16 r + quad (clamped for the loads; rows beyond M are not stored).
     // per-lane address constants: window c, piece (quad + s) % 4 at step s; byte 3 = 1 (see ga_read)
     uint32_t lane_const[4];
 #pragma unroll
@@ -167,37 +179,67 @@ __global__ __launch_bounds__(kGaWaves * 64) void lutgemm_gradA_slab_kernel(
 
     typedef const __attribute__((address_space(1))) void* gptr_t;
     typedef __attribute__((address_space(3))) void* lptr_t;
-    // The waves share the requests by kind, since vmcnt counts the operations of a wave in issue order and a slow one
-    // holds up the count for every later one: waves 0-7 fetch the chunks (needed two steps later, from L2), waves
-    // 8-15 the rows of gC (from HBM, needed a whole column tile later).
-    const bool chunk_wave = wave < kGaWaves / 2;
-    // chunk q = (tile, four k of the workgroup's range): 32 KB = 32 wave-wide 16-byte loads, four per wave.
-    // Requests beyond the end repeat the last chunk (into a buffer nobody reads any more) so that every step
-    // issues the same number of operations.
-    const u32x4* Sgroup = S + (size_t)(k0 / kGaChunkK) * (kGaChunkBytes / 16);
+    // A wave whose rows would stick out of M is shifted up so that all its rows exist; the rows it then shares with
+    // the wave above are not stored twice (a wave entirely beyond M stores nothing but still takes part in the copies
+    // and barriers).  Rows of a lane: m_base + 16 r + quad.
+    auto m_base_of = [&](const Tile& t) { return min(t.m_wave, M - kGaRowsPerWave); };
+    // chunk q of the current tile: 32 KB = 32 wave-wide 16-byte loads, two per wave; beyond the end: the first chunks
+    // of the next tile (the last chunk again when there is none, into a buffer nobody reads any more), so that every
+    // step issues the same number of operations
     auto request_chunk = [&](int q, int buf) {
-        if (!chunk_wave) return;
-        q = min(q, total - 1);
+        int k0 = cur.k0;
+        if (q >= total) {
+            if (nxt.valid) { q -= total; k0 = nxt.k0; } else q = total - 1;
+        }
         const int nt = q / CH, kc = q - nt * CH;
-        const u32x4* src = Sgroup + ((size_t)nt * (K / kGaChunkK) + kc) * (kGaChunkBytes / 16);
+        const u32x4* src = S + ((size_t)nt * (K / kGaChunkK) + k0 / kGaChunkK + kc) * (kGaChunkBytes / 16);
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+            __builtin_amdgcn_global_load_lds((gptr_t)(src + (wave + kGaWaves * i) * 64 + lane),
+                                             (lptr_t)(smem + buf * kGaChunkBytes + (wave + kGaWaves * i) * 1024), 16, 0, 0);
+    };
+    // the 32 rows of this wave, 128 B (32 columns of tile nt) each: four wave-wide loads, lane = (row % 8, 16 B piece);
+    // beyond the last column tile: the first one of the next tile
+    const uint32_t glane = (uint32_t)(lane >> 3) * (uint32_t)N + 4u * (uint32_t)(lane & 7);
+    auto request_rows = [&](int nt) {
+        int m_base = m_base_of(cur);
+        if (nt >= n_tiles) {
+            if (nxt.valid) { nt = 0; m_base = m_base_of(nxt); } else nt = n_tiles - 1;
+        }
+        const float* base = gC + (size_t)m_base * N + nt * kGaCols;
 #pragma unroll
         for (int i = 0; i < 4; ++i)
-            __builtin_amdgcn_global_load_lds((gptr_t)(src + (wave + 8 * i) * 64 + lane),
-                                             (lptr_t)(smem + buf * kGaChunkBytes + (wave + 8 * i) * 1024), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds((gptr_t)(base + (size_t)(8 * i) * N + glane),
+                                             (lptr_t)(smem + kGaStageBase + wave * 4096 + i * 1024), 16, 0, 0);
     };
-    // the 512 rows of the workgroup, 128 B (32 columns of tile nt) each: 64 wave-wide loads of 8 rows, eight per wave,
-    // lane = (row % 8, 16 B piece); rows beyond M repeat the last one
-    int grow = row_block * kGaRows + (wave & 7) * 64 + (lane >> 3);
-    auto request_rows = [&](int nt) {
-        if (chunk_wave) return;
-        nt = min(nt, n_tiles - 1);
-        // (opaque to the compiler: the eight offsets are computed here, once per column tile, not kept in registers)
-        asm volatile("" : "+v"(grow));
-        const float* base = gC + nt * kGaCols + 4 * (lane & 7);
+    // The codes of a tile: A[m][k0 + 4 j + c], one byte per chunk and row, packed four to a register.  Assembly loads:
+    // the waiting is explicit (the compiler would wait for everything in flight).
+    uint32_t codes[2][(CH + 3) / 4];
+    auto load_codes = [&](const Tile& t, uint32_t (&raw)[2][CH]) {
+        const int m_base = m_base_of(t);
 #pragma unroll
-        for (int i = 0; i < 8; ++i)
-            __builtin_amdgcn_global_load_lds((gptr_t)(base + (size_t)((uint32_t)min(grow + 8 * i, M - 1) * (uint32_t)N)),
-                                             (lptr_t)(smem + kGaStageBase + ((wave & 7) * 8 + i) * 1024), 16, 0, 0);
+        for (int r = 0; r < 2; ++r) {
+            const uint8_t* arow = A + (size_t)(m_base + 16 * r + quad) * K + t.k0;
+#pragma unroll
+            for (int j = 0; j < CH; ++j) asm volatile("global_load_dword %0, %1, off" : "=v"(raw[r][j]) : "v"(arow + 4 * j) : "memory");
+        }
+    };
+    auto pack_codes = [&](uint32_t (&raw)[2][CH]) {
+        uint32_t high_bits = 0;
+#pragma unroll
+        for (int r = 0; r < 2; ++r) {
+#pragma unroll
+            for (int w = 0; w < (CH + 3) / 4; ++w) codes[r][w] = 0;
+#pragma unroll
+            for (int j = 0; j < CH; ++j) {
+                const uint32_t a = (raw[r][j] >> (8 * c)) & 0xffu;
+                high_bits |= a;
+                codes[r][j >> 2] |= a << (8 * (j & 3));
+            }
+        }
+        if (__builtin_amdgcn_ballot_w64((high_bits & 0x80u) != 0) != 0) {
+            if (lane == 0) atomicOr(&flags[2], 1u);
+        }
     };
 
     float acc[2][CH];
@@ -213,32 +255,26 @@ __global__ __launch_bounds__(kGaWaves * 64) void lutgemm_gradA_slab_kernel(
     float row_sum[2] = {0.f, 0.f};
     u32x4 d[4] = {{0, 0, 0, 0}, {0, 0, 0, 0}, {0, 0, 0, 0}, {0, 0, 0, 0}};
 
-    // Operations of a thread towards LDS, in issue order (vmcnt counts them in this order):
-    //   rows(0) chunk(0) chunk(1) | top of chunk q: chunk(q + 2); top of the second chunk of tile nt also: rows(nt + 1)
-    // (a chunk request is two operations, a row request four).  At the top of chunk q, chunk q (requested two
-    // chunks earlier) must have landed: all but the requests of the previous top may be outstanding.
+    // Operations of a wave towards memory, in issue order (vmcnt counts them in this order):
+    //   rows(0) chunk(0) chunk(1) codes | step q: chunk(q + 2); second step of column tile nt also: rows(nt + 1)
+    //   | end of a tile: codes of the next tile, NST stores | ...
+    // (a chunk request is two operations, a row request four).  At the top of step q, chunk q (requested two steps
+    // earlier) must have landed: all but the requests of the previous step may be outstanding; in the first two
+    // steps of a tile the stores of the previous one as well.
     request_rows(0);
     request_chunk(0, 0);
     request_chunk(1, 1);
-    // (the codes after the first requests: both then travel at the same time)
-    uint32_t codes[2][(CH + 3) / 4];
-    uint32_t high_bits = 0;
+    {
+        uint32_t raw[2][CH];
+        load_codes(cur, raw);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 #pragma unroll
-    for (int r = 0; r < 2; ++r) {
-        const uint8_t* arow = A + (size_t)min(m_wave + 16 * r + quad, M - 1) * K + k0;
+        for (int r = 0; r < 2; ++r)
 #pragma unroll
-        for (int w = 0; w < (CH + 3) / 4; ++w) codes[r][w] = 0;
-#pragma unroll
-        for (int j = 0; j < CH; ++j) {
-            const uint32_t a = (load_u32_unaligned(arow + 4 * j) >> (8 * c)) & 0xffu;      // A[m][k0 + 4 j + c]
-            high_bits |= a;
-            codes[r][j >> 2] |= a << (8 * (j & 3));
-        }
+            for (int j = 0; j < CH; ++j) asm volatile("" : "+v"(raw[r][j]));
+        pack_codes(raw);
     }
-    if (__builtin_amdgcn_ballot_w64((high_bits & 0x80u) != 0) != 0) {
-        if (lane == 0) atomicOr(&flags[2], 1u);
-    }
-
+    bool after_stores = false;     // the previous tile's stores may still be on their way (this wave issued all NST of them)
 
     // Read i of a chunk (i = 0..7): step s = i / 2, row r = i % 2; data in d[i % 4].  Two pairs of reads are in flight;
     // the last pair of a chunk is consumed after the barrier of the next one, while its first reads travel.  The two
@@ -260,25 +296,27 @@ __global__ __launch_bounds__(kGaWaves * 64) void lutgemm_gradA_slab_kernel(
         acc[0][KC] = s0;
         acc[1][KC] = s1;
     };
-    auto chunk_step = [&](int nt, auto kc_tag, auto buf_tag) {
+    auto chunk_step = [&](int nt, auto kc_tag, auto buf_tag) __attribute__((always_inline)) {
         constexpr int KC = decltype(kc_tag)::value;
         constexpr int BUF = decltype(buf_tag)::value;
         constexpr int KP = (KC + CH - 1) % CH;            // the previous chunk's k quad (its last pair of reads is consumed here)
         const int q = nt * CH + KC;
         // the last pair of the previous chunk has landed (nobody reads its buffer any more), chunk q has landed for
         // this wave; behind the barrier: for every wave
-        if (chunk_wave)
-            asm volatile("s_waitcnt lgkmcnt(0)\n s_waitcnt vmcnt(4)\n s_barrier" : "+v"(d[2]), "+v"(d[3]) : : "memory");
-        else if (KC == 0)
-            asm volatile("s_waitcnt lgkmcnt(0)\n s_waitcnt vmcnt(0)\n s_barrier" : "+v"(d[2]), "+v"(d[3]) : : "memory");
-        else
-            asm volatile("s_waitcnt lgkmcnt(0)\n s_barrier" : "+v"(d[2]), "+v"(d[3]) : : "memory");
+        if (KC < 2 && nt == 0 && after_stores) {
+            if (KC == 0) asm volatile("s_waitcnt lgkmcnt(0)\n s_waitcnt vmcnt(%2)\n s_barrier" : "+v"(d[2]), "+v"(d[3]) : "n"(NST) : "memory");
+            else asm volatile("s_waitcnt lgkmcnt(0)\n s_waitcnt vmcnt(%2)\n s_barrier" : "+v"(d[2]), "+v"(d[3]) : "n"(NST + 2) : "memory");
+        } else if (KC == 2 || KC == 3) {
+            asm volatile("s_waitcnt lgkmcnt(0)\n s_waitcnt vmcnt(6)\n s_barrier" : "+v"(d[2]), "+v"(d[3]) : : "memory");
+        } else {
+            asm volatile("s_waitcnt lgkmcnt(0)\n s_waitcnt vmcnt(2)\n s_barrier" : "+v"(d[2]), "+v"(d[3]) : : "memory");
+        }
         request_chunk(q + 2, (BUF + 2) % kGaBufs);
         if (KC == 1) request_rows(nt + 1);
         __builtin_amdgcn_s_setprio(3);
         ga_read<KC & 3, BUF>(d[0], codes[0][KC >> 2], lane_const[0]);
         ga_read<KC & 3, BUF>(d[1], codes[1][KC >> 2], lane_const[0]);
-        pair_fma(std::integral_constant<int, KP>{}, std::integral_constant<int, 3>{}, d[2], d[3]);
+        if (KC != 0 || nt != 0) pair_fma(std::integral_constant<int, KP>{}, std::integral_constant<int, 3>{}, d[2], d[3]);
         ga_read<KC & 3, BUF>(d[2], codes[0][KC >> 2], lane_const[1]);
         ga_read<KC & 3, BUF>(d[3], codes[1][KC >> 2], lane_const[1]);
         if (KC == 0) {
@@ -328,46 +366,88 @@ __global__ __launch_bounds__(kGaWaves * 64) void lutgemm_gradA_slab_kernel(
         asm volatile("s_waitcnt lgkmcnt(2)" : "+v"(d[0]), "+v"(d[1]) : : "memory");
         pair_fma(kc_tag, std::integral_constant<int, 2>{}, d[0], d[1]);
     };
-    auto tile_steps = [&](int nt, auto j_tag) {
-        constexpr int J = decltype(j_tag)::value;            // position of the tile in the unrolled pass
+    // End of a tile: last multiply-adds, the codes of the next tile are asked for, gA of this one is stored meanwhile.
+    // Returns false when the workgroup has no further tile.
+    auto finish_tile = [&]() __attribute__((always_inline)) {
+        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(d[2]), "+v"(d[3]) : : "memory");
+        pair_fma(std::integral_constant<int, CH - 1>{}, std::integral_constant<int, 3>{}, d[2], d[3]);
+        uint32_t raw[2][CH];
+        if (nxt.valid) load_codes(nxt, raw);
+        const int m_base = m_base_of(cur);
+        const bool whole = m_base == cur.m_wave;             // every lane of the wave stores: NST store instructions, no more, no less
+        // (k outside, row inside: the two stores of a k then fill the same 128 B lines of the image-major layout)
+        float* o[2];
+        float corr[2];
+        size_t k_stride = 4;
+#pragma unroll
+        for (int r = 0; r < 2; ++r) {
+            const int m = m_base + 16 * r + quad;
+            corr[r] = offset * row_sum[r];
+            if (m < cur.m_wave) {
+                o[r] = nullptr;          // row stored by the wave above
+            } else if (rows_per_image > 0) {
+                const int img = m / rows_per_image, l = m - img * rows_per_image;
+                o[r] = gA + ((size_t)img * K + cur.k0 + c) * rows_per_image + l;
+                k_stride = (size_t)4 * rows_per_image;
+            } else {
+                o[r] = gA + (size_t)m * K + cur.k0 + c;
+            }
+        }
+        if (whole) {
+#pragma unroll
+            for (int j = 0; j < CH; ++j)
+#pragma unroll
+                for (int r = 0; r < 2; ++r) {
+                    const float v = (acc[r][j] + corr[r]) * scale;
+                    asm volatile("global_store_dword %0, %1, off" : : "v"(o[r] + j * k_stride), "v"(v) : "memory");
+                }
+        } else {
+#pragma unroll
+            for (int j = 0; j < CH; ++j)
+#pragma unroll
+                for (int r = 0; r < 2; ++r)
+                    if (o[r]) o[r][j * k_stride] = (acc[r][j] + corr[r]) * scale;
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        }
+        if (!nxt.valid) return false;
+        // the codes have arrived (they were asked for before the stores)
+        if (whole) asm volatile("s_waitcnt vmcnt(%0)" : : "n"(NST) : "memory");
+#pragma unroll
+        for (int r = 0; r < 2; ++r)
+#pragma unroll
+            for (int j = 0; j < CH; ++j) asm volatile("" : "+v"(raw[r][j]));
+        pack_codes(raw);
+        after_stores = whole;
+#pragma unroll
+        for (int r = 0; r < 2; ++r) {
+            row_sum[r] = 0.f;
+#pragma unroll
+            for (int j = 0; j < CH; ++j) acc[r][j] = 0.f;
+        }
+        cur = nxt;
+        pos += pos_stride;
+        nxt = decode(pos + pos_stride);
+        return true;
+    };
+    int nt = 0;
+    // one column tile; J = its position in the unrolled pass (the buffers rotate with period three across tiles)
+    auto tile_step = [&](auto j_tag) __attribute__((always_inline)) {
+        constexpr int J = decltype(j_tag)::value;
         [&]<int... KC>(std::integer_sequence<int, KC...>) {
             (chunk_step(nt, std::integral_constant<int, KC>{}, std::integral_constant<int, (J * CH + KC) % kGaBufs>{}), ...);
         }(std::make_integer_sequence<int, CH>{});
+        if (++nt < n_tiles) return true;
+        nt = 0;
+        return finish_tile();
     };
-    for (int nt0 = 0; nt0 < n_tiles; nt0 += NTU) {
-        tile_steps(nt0, std::integral_constant<int, 0>{});
+    for (;;) {
+        if (!tile_step(std::integral_constant<int, 0>{})) break;
         if (NTU > 1) {
-            if (nt0 + 1 < n_tiles) tile_steps(nt0 + 1, std::integral_constant<int, 1 % NTU>{});
-            if (nt0 + 2 < n_tiles) tile_steps(nt0 + 2, std::integral_constant<int, 2 % NTU>{});
+            if (!tile_step(std::integral_constant<int, 1 % NTU>{})) break;
+            if (!tile_step(std::integral_constant<int, 2 % NTU>{})) break;
         }
     }
-    // the last pair of reads of the last chunk
-    asm volatile("s_waitcnt lgkmcnt(0)\n s_waitcnt vmcnt(0)" : "+v"(d[2]), "+v"(d[3]) : : "memory");
-    pair_fma(std::integral_constant<int, CH - 1>{}, std::integral_constant<int, 3>{}, d[2], d[3]);
-
-    // (k outside, row inside: the two stores of a k then fill the same 128 B lines of the image-major layout)
-    float* o[2];
-    float corr[2];
-    size_t k_stride = 4;
-#pragma unroll
-    for (int r = 0; r < 2; ++r) {
-        const int m = m_wave + 16 * r + quad;
-        corr[r] = offset * row_sum[r];
-        if (m >= M) {
-            o[r] = nullptr;
-        } else if (rows_per_image > 0) {
-            const int img = m / rows_per_image, l = m - img * rows_per_image;
-            o[r] = gA + ((size_t)img * K + k0 + c) * rows_per_image + l;
-            k_stride = (size_t)4 * rows_per_image;
-        } else {
-            o[r] = gA + (size_t)m * K + k0 + c;
-        }
-    }
-#pragma unroll
-    for (int j = 0; j < CH; ++j)
-#pragma unroll
-        for (int r = 0; r < 2; ++r)
-            if (o[r]) o[r][j * k_stride] = (acc[r][j] + corr[r]) * scale;
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // nothing is left in flight towards LDS when the workgroup ends
 }
 
 // ------------------------------------------------------------------------------------------ host
@@ -388,29 +468,29 @@ hipError_t launch_gradA_slab(const float* gC, const uint8_t* A, const uint8_t* B
                              const LutGeom& g, int M, int K, int N, float scale, int n_cu, uint32_t* flags, void* S,
                              int rows_per_image, hipStream_t stream) {
     const int lut_dwords = g.rows * g.cols / 2;
-    hipLaunchKernelGGL(expand_gradA_kernel, dim3(N / kGaCols, K / kGaExpandK), dim3(256), (size_t)lut_dwords * 4, stream, B,
+    const int qpw = 4;     // 16 k per workgroup (measured: 8 k is 15 % slower for long K, 64 k 20 % slower)
+    hipLaunchKernelGGL(expand_gradA_kernel, dim3(N / kGaCols, (K / 4 + qpw - 1) / qpw), dim3(256), (size_t)lut_dwords * 4, stream, B,
                        reinterpret_cast<const uint32_t*>(lut), lut_dwords, g.cols, 1 << g.bits, reinterpret_cast<uint32_t*>(S),
-                       flags, K, N);
+                       flags, K, N, qpw);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     if (((uintptr_t)gC & 15) != 0) return hipErrorInvalidValue;   // callers check: rows of gC are fetched 16 bytes at a time
     const u32x4* S4 = reinterpret_cast<const u32x4*>(S);
     const dim3 block(kGaWaves * 64);
     const int row_blocks = (M + kGaRows - 1) / kGaRows;
-    // 16 row blocks x 2 k groups are in flight on an XCD at a time (measured: 8 to 32 row blocks make no difference,
-    // the XCD order gains 15 % where there are few row blocks)
-    const int band_rows = 16, xcd_order = 1;
-    auto launch = [&](auto kt_tag) {
-        constexpr int KT = decltype(kt_tag)::value;
-        const dim3 grid(8 * ((row_blocks * (K / KT) + 7) / 8));
-        hipLaunchKernelGGL((lutgemm_gradA_slab_kernel<KT>), grid, block, 0, stream, gC, A, S4, gA, flags, M, K, N, scale,
-                           rows_per_image, row_blocks, band_rows, xcd_order);
-    };
-    (void)n_cu;
+    // 16 row blocks x 2 k groups are in flight on an XCD at a time (measured: 8 to 32 row blocks make no difference)
+    const int band_rows = 16;
     // (48 k per workgroup would need more registers than a wave of a 1024-thread workgroup has)
     const int kt = (K % 32) == 0 ? 32 : 16;
-    if (kt == 32) launch(std::integral_constant<int, 32>{});
-    else launch(std::integral_constant<int, 16>{});
+    const int tiles = row_blocks * (K / kt);
+    const int per_xcd = (tiles + 7) / 8, cus_per_xcd = n_cu >= 8 ? n_cu / 8 : 1;
+    const dim3 grid(8 * (per_xcd < cus_per_xcd ? per_xcd : cus_per_xcd));
+    if (kt == 32)
+        hipLaunchKernelGGL((lutgemm_gradA_slab_kernel<32>), grid, block, 0, stream, gC, A, S4, gA, flags, M, K, N, scale,
+                           rows_per_image, row_blocks, band_rows);
+    else
+        hipLaunchKernelGGL((lutgemm_gradA_slab_kernel<16>), grid, block, 0, stream, gC, A, S4, gA, flags, M, K, N, scale,
+                           rows_per_image, row_blocks, band_rows);
     e = hipGetLastError();
     if (e != hipSuccess) return e;
     // masked codes in A or table entries a half cannot hold: the gated direct kernel recomputes gA
