@@ -34,6 +34,7 @@ hipError_t launch_quantize_codes(const float* x, const float* scale, const float
 hipError_t launch_quantize_codes_backward(const float* g, const float* x, const float* scale, const float* zp_neg, float qmax,
                                           float* gx, size_t n, hipStream_t stream);
 hipError_t launch_zero_u32(void* p, size_t n_dwords, hipStream_t stream);
+hipError_t launch_bwd_header(const int16_t* lut_a, const int16_t* lut_b, const LutGeom& g, uint32_t* flags, hipStream_t stream);
 hipError_t launch_dequant(const float* c, const float* xs, const float* wr, const float* tp, const float* za, const float* zw,
                           const float* sa, const float* sw, const float* bias, float* out, int M, int N, int L, hipStream_t stream);
 hipError_t launch_dequant_grad(const float* g, const float* sa, const float* sw, float* gc, int M, int N, int L, hipStream_t stream);
@@ -265,8 +266,9 @@ int amr_lut_gemm_backward_ex(const float* gC, const uint8_t* A, const uint8_t* B
     const bool slab = g_expanded_kernels && amr::bwd_slab_applies(g, M, K, N);
     const bool slab_a = g_expanded_kernels && gA && amr::gradA_slab_workspace_bytes(g, M, K, N, g_expanded_kernels == 2) != 0 && ((uintptr_t)gC & 15) == 0;
     if ((slab && gB) || slab_a) {
-        e = amr::launch_zero_u32(flags, 64, s);
-        if (e != hipSuccess) return hip_fail(e, "zero fill launch");
+        // flags cleared, offsets of the half-precision tables decided from the tables' extremes
+        e = amr::launch_bwd_header(slab_a ? lut_grad_a : nullptr, (slab && gB) ? lut_grad_b : nullptr, g, flags, s);
+        if (e != hipSuccess) return hip_fail(e, "scratch header launch");
     }
     if (gA) {
         if (slab_a)

@@ -18,6 +18,8 @@
 // queued behind this one and gated on that flag, recomputes the result.
 // (The gradient of A has no such formulation that pays off: its reduction runs over n, so the rows of
 // gC would have to be re-read once per k tile; it stays with the direct gather kernel.)
+#include <type_traits>
+
 #include "amr_common.h"
 
 namespace amr {
@@ -207,14 +209,16 @@ __global__ __launch_bounds__(1024) void lutgemm_gradB_slab_kernel(
 
 
 // ------------------------------------------------------------------------------------------ gradB, half-precision slab
-// Same scheme with the expanded table held as IEEE half, S16[kk][a][c] = half(G[a][b] - 1024), so that
+// Same scheme with the expanded table held as IEEE half, S16[kk][a][c] = half(G[a][b] - offset), so that
 // eight k fit the 128 KB (half the gC traffic per multiply-add: every row of gC a workgroup streams is
 // used for 8 instead of 4 values of k) and one 64-bit LDS read brings four entries.  Exact: a half holds
-// every integer of magnitude <= 2048, i.e. table entries in [-1024, 3072] (16 x the gradient of a 7-bit
+// every integer of magnitude <= 2048, i.e. table entries in [-2048, 2048] with offset 0 and in [-1024, 3072] with
+// offset 1024, picked from the table's extremes by bwd_header_kernel (16 x the gradient of a 7-bit
 // multiplier is about 16*b <= 2032); an entry outside that range raises flags[1] like a masked code does
 // and the direct kernel recomputes.  The multiply-add takes the half straight into an fp32 fma
 // (v_fma_mix_f32), products and sums are the same fp32 values as with an fp32 table, and the offset is
-// undone at the end with the column sums of gC:  sum_m g*(G-1024) + 1024 * sum_m g.
+// undone at the end with the column sums of gC:  sum_m g*(G-offset) + offset * sum_m g (nothing to undo and no
+// column sums for offset 0).
 //
 // LDS layout: byte address = (kk>>1)*32768 + a*256 + (kk&1)*128 + 2*c: the two k of a pair share a 256 B
 // row.  Row slots 1 and 3 of a wave visit the two k of every pair in the other order than slots 0 and 2,
@@ -222,7 +226,6 @@ __global__ __launch_bounds__(1024) void lutgemm_gradB_slab_kernel(
 // Requires K % 8 == 0, N % 64 == 0, row counts that are multiples of the rows per iteration, gC 16-byte
 // aligned and 32-bit offsets (the launcher checks).
 constexpr int kBwdKT16 = 8;
-constexpr float kBwdHalfOffset = 1024.f;
 
 __global__ __launch_bounds__(1024) void lutgemm_gradB_slab16_kernel(
     const float* __restrict__ gC, const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, float* __restrict__ out,
@@ -249,6 +252,7 @@ __global__ __launch_bounds__(1024) void lutgemm_gradB_slab16_kernel(
     const int k0 = k_tile * KT;
     const int mb = split * m_chunk;
     const int me = min(M, mb + m_chunk);
+    const float offset = (float)flags[4];        // 0 or 1024 (bwd_header_kernel)
 
     {   // expansion: wave-uniform code a, lanes = columns (the gathers of a wave stay inside one table row).
         // All loads of a step are issued before the first is used: the table sits in L2 and a dependent
@@ -271,8 +275,8 @@ __global__ __launch_bounds__(1024) void lutgemm_gradB_slab16_kernel(
             for (int i = 0; i < kBwdSlabRows / 16; ++i) {
                 const int a = wave + 16 * i;
                 const float v = (a < n_codes) ? (float)e[i] : 0.f;
-                const _Float16 h = (_Float16)(v - kBwdHalfOffset);
-                inexact |= ((float)h != v - kBwdHalfOffset);
+                const _Float16 h = (_Float16)(v - offset);
+                inexact |= ((float)h != v - offset);
                 *reinterpret_cast<_Float16*>(s + a * 256) = h;
             }
         }
@@ -298,7 +302,7 @@ __global__ __launch_bounds__(1024) void lutgemm_gradB_slab16_kernel(
     uint32_t seen = 0;
 
     constexpr int RU = kBwdRU;
-    auto consume = [&](uint32_t alo, uint32_t ahi, const f32x4& gvec) {
+    auto consume = [&](auto sums_tag, uint32_t alo, uint32_t ahi, const f32x4& gvec) __attribute__((always_inline)) {
         seen |= alo | ahi;
         const uint32_t a4[2] = {alo, ahi};
         f16x4 s[KT];
@@ -315,10 +319,10 @@ __global__ __launch_bounds__(1024) void lutgemm_gradB_slab16_kernel(
             acc[j][2] = __builtin_fmaf(gvec.z, (float)s[j].z, acc[j][2]);
             acc[j][3] = __builtin_fmaf(gvec.w, (float)s[j].w, acc[j][3]);
         }
-        gsum[0] += gvec.x; gsum[1] += gvec.y; gsum[2] += gvec.z; gsum[3] += gvec.w;
+        if (decltype(sums_tag)::value) { gsum[0] += gvec.x; gsum[1] += gvec.y; gsum[2] += gvec.z; gsum[3] += gvec.w; }
     };
 
-    {
+    auto stream_rows = [&](auto sums_tag) __attribute__((always_inline)) {
         const int iters = (me - mb) / (16 * RU * 4);
         uint32_t aoff[RU], goff[RU];
 #pragma unroll
@@ -346,14 +350,16 @@ __global__ __launch_bounds__(1024) void lutgemm_gradB_slab16_kernel(
         for (int it = 0; it < iters; it += 2) {
             if (it + 1 < iters) load(al1, ah1, g1);
 #pragma unroll
-            for (int u = 0; u < RU; ++u) consume(al0[u], ah0[u], g0[u]);
+            for (int u = 0; u < RU; ++u) consume(sums_tag, al0[u], ah0[u], g0[u]);
             if (it + 1 < iters) {
                 if (it + 2 < iters) load(al0, ah0, g0);
 #pragma unroll
-                for (int u = 0; u < RU; ++u) consume(al1[u], ah1[u], g1[u]);
+                for (int u = 0; u < RU; ++u) consume(sums_tag, al1[u], ah1[u], g1[u]);
             }
         }
-    }
+    };
+    // (two copies of the loop: without the column sums of gC when the table is stored without offset)
+    if (offset != 0.f) stream_rows(std::true_type{}); else stream_rows(std::false_type{});
     if (__builtin_amdgcn_ballot_w64((seen & 0x80808080u) != 0) != 0) {
         if (lane == 0) atomicOr(&flags[1], 1u);
     }
@@ -386,8 +392,49 @@ __global__ __launch_bounds__(1024) void lutgemm_gradB_slab16_kernel(
             v += red[(w * (KT + 1) + kk) * 64 + col];
             gs += red[(w * (KT + 1) + KT) * 64 + col];
         }
-        out[((size_t)split * K + k0 + kk) * N + n0 + col] = (v + kBwdHalfOffset * gs) * scale;
+        out[((size_t)split * K + k0 + kk) * N + n0 + col] = (v + offset * gs) * scale;
     }
+}
+
+// ------------------------------------------------------------------------------------------ scratch header
+// One workgroup: clears the 64 flag words of the backward scratch and leaves the offsets the half-precision tables
+// are stored with: flags[3] for the table of gradA, flags[4] for the table of gradB.  A half holds every integer
+// of magnitude <= 2048: offset 0 when the whole table lies in [-2048, 2048] (the correction term with the sums
+// of gC then drops out of the kernels), else 1024, exact for [-1024, 3072].
+__global__ __launch_bounds__(256) void bwd_header_kernel(const uint32_t* __restrict__ lut_a, const uint32_t* __restrict__ lut_b,
+                                                         int lut_dwords, uint32_t* __restrict__ flags) {
+    __shared__ int extremes[4];
+    if (threadIdx.x < 4) extremes[threadIdx.x] = 0;
+    __syncthreads();
+    for (int t = 0; t < 2; ++t) {
+        const uint32_t* lut = t ? lut_b : lut_a;
+        int lo = 0, hi = 0;
+        if (lut) {
+            for (int i = threadIdx.x; i < lut_dwords; i += 256) {
+                const uint32_t w = lut[i];
+                const int v0 = (int)(int16_t)(w & 0xffffu), v1 = (int)(int16_t)(w >> 16);
+                lo = min(lo, min(v0, v1));
+                hi = max(hi, max(v0, v1));
+            }
+        }
+        atomicMin(&extremes[2 * t], lo);
+        atomicMax(&extremes[2 * t + 1], hi);
+    }
+    __syncthreads();
+    if (threadIdx.x < 64) {
+        uint32_t v = 0;
+        if (threadIdx.x == 3 || threadIdx.x == 4) {
+            const int t = threadIdx.x - 3;
+            v = (extremes[2 * t] >= -2048 && extremes[2 * t + 1] <= 2048) ? 0u : 1024u;
+        }
+        flags[threadIdx.x] = v;
+    }
+}
+
+hipError_t launch_bwd_header(const int16_t* lut_a, const int16_t* lut_b, const LutGeom& g, uint32_t* flags, hipStream_t stream) {
+    hipLaunchKernelGGL(bwd_header_kernel, dim3(1), dim3(256), 0, stream, reinterpret_cast<const uint32_t*>(lut_a),
+                       reinterpret_cast<const uint32_t*>(lut_b), g.rows * g.cols / 2, flags);
+    return hipGetLastError();
 }
 
 // ------------------------------------------------------------------------------------------ host

@@ -13,7 +13,7 @@
 // instead of gathering 32 single entries.  The multiply-add takes the half straight into an fp32 fma
 // (v_fma_mix_f32); a half holds every integer of magnitude <= 2048, so with offset 0 table entries in
 // [-2048, 2048] are exact (16 x the gradient of a 7-bit multiplier is about 16*b <= 2032), with offset 1024
-// entries in [-1024, 3072]; the expansion picks the offset from the extremes of the table and leaves it in
+// entries in [-1024, 3072]; the offset is picked from the extremes of the table (bwd_header_kernel) and sits in
 // flags[3].  Products and sums are then the fp32 values an fp32 table would give.  An entry a half cannot
 // hold, or a masked code 128 in A (not addressable here), raises flags[2] and the direct kernel, queued
 // behind and gated on that flag, recomputes gA.
@@ -61,24 +61,10 @@ __global__ __launch_bounds__(256) void expand_gradA_kernel(const uint8_t* __rest
                                                            int lut_dwords, int lut_cols, int n_codes,
                                                            uint32_t* __restrict__ S, uint32_t* __restrict__ flags, int K, int N, int quads_per_wg) {
     extern __shared__ __align__(16) unsigned char smem[];
-    __shared__ int extremes[2];
     uint32_t* s32 = reinterpret_cast<uint32_t*>(smem);
-    if (threadIdx.x == 0) { extremes[0] = 0; extremes[1] = 0; }
+    for (int i = threadIdx.x; i < lut_dwords; i += 256) s32[i] = lut32[i];
     __syncthreads();
-    int lo = 0, hi = 0;
-    for (int i = threadIdx.x; i < lut_dwords; i += 256) {
-        const uint32_t w = lut32[i];
-        s32[i] = w;
-        const int v0 = (int)(int16_t)(w & 0xffffu), v1 = (int)(int16_t)(w >> 16);
-        lo = min(lo, min(v0, v1));
-        hi = max(hi, max(v0, v1));
-    }
-    atomicMin(&extremes[0], lo);
-    atomicMax(&extremes[1], hi);
-    __syncthreads();
-    // every workgroup finds the same offset; the consumer reads it from flags[3]
-    const float offset = (extremes[0] >= -2048 && extremes[1] <= 2048) ? 0.f : 1024.f;
-    if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) flags[3] = (uint32_t)offset;
+    const float offset = (float)flags[3];        // 0 or 1024, decided from the table's extremes by bwd_header_kernel
     const int16_t* s16 = reinterpret_cast<const int16_t*>(smem);
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     // a wave writes the 256 B row of one code: lane = (k % 4, column pair), one dword (two columns) per lane
