@@ -401,24 +401,44 @@ __global__ __launch_bounds__(1024) void lutgemm_gradB_slab16_kernel(
 // are stored with: flags[3] for the table of gradA, flags[4] for the table of gradB.  A half holds every integer
 // of magnitude <= 2048: offset 0 when the whole table lies in [-2048, 2048] (the correction term with the sums
 // of gC then drops out of the kernels), else 1024, exact for [-1024, 3072].
-__global__ __launch_bounds__(256) void bwd_header_kernel(const uint32_t* __restrict__ lut_a, const uint32_t* __restrict__ lut_b,
-                                                         int lut_dwords, uint32_t* __restrict__ flags) {
+__global__ __launch_bounds__(1024) void bwd_header_kernel(const uint32_t* __restrict__ lut_a, const uint32_t* __restrict__ lut_b,
+                                                          int lut_dwords, uint32_t* __restrict__ flags) {
     __shared__ int extremes[4];
     if (threadIdx.x < 4) extremes[threadIdx.x] = 0;
     __syncthreads();
-    for (int t = 0; t < 2; ++t) {
-        const uint32_t* lut = t ? lut_b : lut_a;
-        int lo = 0, hi = 0;
-        if (lut) {
-            for (int i = threadIdx.x; i < lut_dwords; i += 256) {
-                const uint32_t w = lut[i];
-                const int v0 = (int)(int16_t)(w & 0xffffu), v1 = (int)(int16_t)(w >> 16);
+    // all loads of both tables are issued before the first is used (one dependent load at a time would pay the
+    // memory latency 66 times: 19 us instead of 5)
+    constexpr int PER = 9;                       // 9 x 1024 dwords cover a 7-bit table (8385) in one round; an 8-bit table takes four
+    uint32_t w[2][PER];
+    for (int base = 0; base < lut_dwords; base += PER * 1024) {
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            const uint32_t* lut = t ? lut_b : lut_a;
+#pragma unroll
+            for (int i = 0; i < PER; ++i) {
+                const int idx = base + i * 1024 + (int)threadIdx.x;
+                w[t][i] = (lut && idx < lut_dwords) ? lut[idx] : 0u;
+            }
+        }
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            int lo = 0, hi = 0;
+#pragma unroll
+            for (int i = 0; i < PER; ++i) {
+                const int v0 = (int)(int16_t)(w[t][i] & 0xffffu), v1 = (int)(int16_t)(w[t][i] >> 16);
                 lo = min(lo, min(v0, v1));
                 hi = max(hi, max(v0, v1));
             }
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) {
+                lo = min(lo, __shfl_xor(lo, o));
+                hi = max(hi, __shfl_xor(hi, o));
+            }
+            if ((threadIdx.x & 63) == 0) {
+                atomicMin(&extremes[2 * t], lo);
+                atomicMax(&extremes[2 * t + 1], hi);
+            }
         }
-        atomicMin(&extremes[2 * t], lo);
-        atomicMax(&extremes[2 * t + 1], hi);
     }
     __syncthreads();
     if (threadIdx.x < 64) {
@@ -432,7 +452,7 @@ __global__ __launch_bounds__(256) void bwd_header_kernel(const uint32_t* __restr
 }
 
 hipError_t launch_bwd_header(const int16_t* lut_a, const int16_t* lut_b, const LutGeom& g, uint32_t* flags, hipStream_t stream) {
-    hipLaunchKernelGGL(bwd_header_kernel, dim3(1), dim3(256), 0, stream, reinterpret_cast<const uint32_t*>(lut_a),
+    hipLaunchKernelGGL(bwd_header_kernel, dim3(1), dim3(1024), 0, stream, reinterpret_cast<const uint32_t*>(lut_a),
                        reinterpret_cast<const uint32_t*>(lut_b), g.rows * g.cols / 2, flags);
     return hipGetLastError();
 }
