@@ -289,13 +289,16 @@ __global__ __launch_bounds__(kGaWaves * 64) void lutgemm_gradA_slab_kernel(
         const int q = nt * CH + KC;
         // the last pair of the previous chunk has landed (nobody reads its buffer any more), chunk q has landed for
         // this wave; behind the barrier: for every wave
+        // (the wait for the reads in flight stands alone, ahead of the branch: where the blocks below tie the registers
+        // of those reads as operands, the register allocator may copy them, i.e. read them, in front of the block)
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         if (KC < 2 && nt == 0 && after_stores) {
-            if (KC == 0) asm volatile("s_waitcnt lgkmcnt(0)\n s_waitcnt vmcnt(%2)\n s_barrier" : "+v"(d[2]), "+v"(d[3]) : "n"(NST) : "memory");
-            else asm volatile("s_waitcnt lgkmcnt(0)\n s_waitcnt vmcnt(%2)\n s_barrier" : "+v"(d[2]), "+v"(d[3]) : "n"(NST + 2) : "memory");
+            if (KC == 0) asm volatile("s_waitcnt vmcnt(%2)\n s_barrier" : "+v"(d[2]), "+v"(d[3]) : "n"(NST) : "memory");
+            else asm volatile("s_waitcnt vmcnt(%2)\n s_barrier" : "+v"(d[2]), "+v"(d[3]) : "n"(NST + 2) : "memory");
         } else if (KC == 2 || KC == 3) {
-            asm volatile("s_waitcnt lgkmcnt(0)\n s_waitcnt vmcnt(6)\n s_barrier" : "+v"(d[2]), "+v"(d[3]) : : "memory");
+            asm volatile("s_waitcnt vmcnt(6)\n s_barrier" : "+v"(d[2]), "+v"(d[3]) : : "memory");
         } else {
-            asm volatile("s_waitcnt lgkmcnt(0)\n s_waitcnt vmcnt(2)\n s_barrier" : "+v"(d[2]), "+v"(d[3]) : : "memory");
+            asm volatile("s_waitcnt vmcnt(2)\n s_barrier" : "+v"(d[2]), "+v"(d[3]) : : "memory");
         }
         request_chunk(q + 2, (BUF + 2) % kGaBufs);
         if (KC == 1) request_rows(nt + 1);
@@ -310,25 +313,26 @@ __global__ __launch_bounds__(kGaWaves * 64) void lutgemm_gradA_slab_kernel(
             const uint32_t gbase = (uint32_t)(kGaStageBase + wave * 4096 + quad * 128);
 #pragma unroll
             for (int r = 0; r < 2; ++r) {
-                u32x4 t[8];
+                // (two pieces at a time: eight more registers in flight would not fit)
 #pragma unroll
-                for (int s = 0; s < 4; ++s) {
-                    const uint32_t ga = gbase + (uint32_t)(((quad + s) & 3) << 5);
-                    if (r == 0) {
-                        asm volatile("ds_read_b128 %0, %2\n ds_read_b128 %1, %2 offset:16" : "=&v"(t[2 * s]), "=&v"(t[2 * s + 1]) : "v"(ga) : "memory");
-                    } else {
-                        asm volatile("ds_read_b128 %0, %2 offset:2048\n ds_read_b128 %1, %2 offset:2064" : "=&v"(t[2 * s]), "=&v"(t[2 * s + 1]) : "v"(ga) : "memory");
+                for (int hf = 0; hf < 2; ++hf) {
+                    u32x4 t[4];
+#pragma unroll
+                    for (int s2 = 0; s2 < 2; ++s2) {
+                        const int s = 2 * hf + s2;
+                        const uint32_t ga = gbase + (uint32_t)(((quad + s) & 3) << 5);
+                        if (r == 0) {
+                            asm volatile("ds_read_b128 %0, %2\n ds_read_b128 %1, %2 offset:16" : "=&v"(t[2 * s2]), "=&v"(t[2 * s2 + 1]) : "v"(ga) : "memory");
+                        } else {
+                            asm volatile("ds_read_b128 %0, %2 offset:2048\n ds_read_b128 %1, %2 offset:2064" : "=&v"(t[2 * s2]), "=&v"(t[2 * s2 + 1]) : "v"(ga) : "memory");
+                        }
                     }
-                }
-                asm volatile("s_waitcnt lgkmcnt(0)"
-                             : "+v"(t[0]), "+v"(t[1]), "+v"(t[2]), "+v"(t[3]), "+v"(t[4]), "+v"(t[5]), "+v"(t[6]), "+v"(t[7]), "+v"(d[0]),
-                               "+v"(d[1]), "+v"(d[2]), "+v"(d[3])
-                             :
-                             : "memory");
+                    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(t[0]), "+v"(t[1]), "+v"(t[2]), "+v"(t[3]), "+v"(d[0]), "+v"(d[1]), "+v"(d[2]), "+v"(d[3]) : : "memory");
 #pragma unroll
-                for (int i = 0; i < 8; ++i) {
-                    const f32x4 v = __builtin_bit_cast(f32x4, t[i]);
-                    g[r][4 * i] = v.x; g[r][4 * i + 1] = v.y; g[r][4 * i + 2] = v.z; g[r][4 * i + 3] = v.w;
+                    for (int i = 0; i < 4; ++i) {
+                        const f32x4 v = __builtin_bit_cast(f32x4, t[i]);
+                        g[r][16 * hf + 4 * i] = v.x; g[r][16 * hf + 4 * i + 1] = v.y; g[r][16 * hf + 4 * i + 2] = v.z; g[r][16 * hf + 4 * i + 3] = v.w;
+                    }
                 }
                 if (offset != 0.f) {
                     float s = row_sum[r];
@@ -388,6 +392,7 @@ __global__ __launch_bounds__(kGaWaves * 64) void lutgemm_gradA_slab_kernel(
                     asm volatile("global_store_dword %0, %1, off" : : "v"(o[r] + j * k_stride), "v"(v) : "memory");
                 }
         } else {
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 #pragma unroll
             for (int j = 0; j < CH; ++j)
 #pragma unroll
