@@ -69,24 +69,22 @@ __global__ __launch_bounds__(256) void expand_fwd_kernel(const uint8_t* __restri
     }
     const uint16_t* s16 = reinterpret_cast<const uint16_t*>(smem);
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    // a wave writes whole 256 B lines: lane = (kk, column pair), one dword (two columns) per lane
+    // a wave writes whole 256 B lines: lane = (kk, column pair), one dword (two columns) per lane.  Per entry: two
+    // 16-bit LDS reads, one shift-or, the store (the kernel should run at the speed of its writes).  Positions
+    // beyond K or N and codes beyond the table read the table's all-zero pad column / pad row.
     const int kk = lane >> 4, n = blockIdx.x * kSlabCols + 2 * (lane & 15);
     for (int qq = 0; qq < kExpandQuadsPerWg; ++qq) {
         const int q = blockIdx.y * kExpandQuadsPerWg + qq;
         if (q >= k_quads) break;
-        uint32_t* blk = E + ((size_t)blockIdx.x * k_quads + q) * (kSlabChunkBytes / 4);
+        uint32_t* blk = E + ((size_t)blockIdx.x * k_quads + q) * (kSlabChunkBytes / 4) + lane;
         const int k = 4 * q + kk;
         const bool live0 = (k < K) && (n < N), live1 = (k < K) && (n + 1 < N);
-        const int b0 = live0 ? (int)B[(size_t)k * N + n] : 0;
-        const int b1 = live1 ? (int)B[(size_t)k * N + n + 1] : 0;
+        const uint16_t* p0 = s16 + (live0 ? (int)B[(size_t)k * N + n] : n_codes);
+        const uint16_t* p1 = s16 + (live1 ? (int)B[(size_t)k * N + n + 1] : n_codes);
+#pragma unroll 8
         for (int a = wave; a < kSlabRows; a += 4) {
-            uint32_t v = 0;
-            if (a < n_codes) {
-                const uint32_t v0 = live0 ? s16[a * lut_cols + b0] : 0u;
-                const uint32_t v1 = live1 ? s16[a * lut_cols + b1] : 0u;
-                v = v0 | (v1 << 16);
-            }
-            blk[a * 64 + lane] = v;
+            const int row = min(a, n_codes) * lut_cols;
+            blk[a * 64] = (uint32_t)p0[row] | ((uint32_t)p1[row] << 16);
         }
     }
 }

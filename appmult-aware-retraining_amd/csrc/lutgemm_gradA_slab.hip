@@ -62,32 +62,40 @@ __global__ __launch_bounds__(256) void expand_gradA_kernel(const uint8_t* __rest
                                                            uint32_t* __restrict__ S, uint32_t* __restrict__ flags, int K, int N, int quads_per_wg) {
     extern __shared__ __align__(16) unsigned char smem[];
     uint32_t* s32 = reinterpret_cast<uint32_t*>(smem);
-    for (int i = threadIdx.x; i < lut_dwords; i += 256) s32[i] = lut32[i];
-    __syncthreads();
     const float offset = (float)flags[3];        // 0 or 1024, decided from the table's extremes by bwd_header_kernel
-    const int16_t* s16 = reinterpret_cast<const int16_t*>(smem);
+    // The table goes to LDS as halves, converted once per workgroup; what is left per entry of S is two 16-bit LDS
+    // reads, one shift-or and the store (the kernel writes 256 B per code and k quad and should run at the speed of
+    // the writes: 6.8 TB/s measured for a plain fill).
+    bool inexact = false;
+    for (int i = threadIdx.x; i < lut_dwords; i += 256) {
+        const uint32_t w = lut32[i];
+        const float v0 = (float)(int16_t)(w & 0xffffu) - offset, v1 = (float)(int16_t)(w >> 16) - offset;
+        const _Float16 h0 = (_Float16)v0, h1 = (_Float16)v1;
+        inexact |= ((float)h0 != v0) | ((float)h1 != v1);
+        s32[i] = (uint32_t)__builtin_bit_cast(uint16_t, h0) | ((uint32_t)__builtin_bit_cast(uint16_t, h1) << 16);
+    }
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    if (__builtin_amdgcn_ballot_w64(inexact) != 0 && lane == 0) atomicOr(&flags[2], 1u);
+    __syncthreads();
+    const uint16_t* s16 = reinterpret_cast<const uint16_t*>(smem);
     // a wave writes the 256 B row of one code: lane = (k % 4, column pair), one dword (two columns) per lane
     const int ks = lane >> 4, cp = lane & 15;
     const int n = blockIdx.x * kGaCols + 2 * cp;
-    bool inexact = false;
     for (int pp = 0; pp < quads_per_wg; ++pp) {
         const int kq = blockIdx.y * quads_per_wg + pp;
         if (4 * kq >= K) break;
         const int k = 4 * kq + ks;
-        const int b0 = (int)B[(size_t)k * N + n], b1 = (int)B[(size_t)k * N + n + 1];
-        uint32_t* chunk = S + ((size_t)blockIdx.x * (K / 4) + kq) * (kGaChunkBytes / 4);
+        const uint8_t* bp = B + (size_t)k * N + n;
+        const uint16_t* p0 = s16 + (int)bp[0];
+        const uint16_t* p1 = s16 + (int)bp[1];
+        uint32_t* chunk = S + ((size_t)blockIdx.x * (K / 4) + kq) * (kGaChunkBytes / 4) + lane;
+#pragma unroll 8
         for (int a = wave; a < 128; a += 4) {
-            // codes beyond the table (only the pad code 2^b of a narrower table can occur) contribute zero
-            const float v0 = (a < n_codes) ? (float)s16[a * lut_cols + b0] : 0.f;
-            const float v1 = (a < n_codes) ? (float)s16[a * lut_cols + b1] : 0.f;
-            const _Float16 h0 = (_Float16)(v0 - offset), h1 = (_Float16)(v1 - offset);
-            inexact |= ((float)h0 != v0 - offset) | ((float)h1 != v1 - offset);
-            const uint32_t w = (uint32_t)__builtin_bit_cast(uint16_t, h0) | ((uint32_t)__builtin_bit_cast(uint16_t, h1) << 16);
-            chunk[a * 64 + ks * 16 + cp] = w;
+            // codes beyond the table (only the pad code 2^b of a narrower table can occur) read its all-zero pad row
+            const int row = min(a, n_codes) * lut_cols;
+            chunk[a * 64] = (uint32_t)p0[row] | ((uint32_t)p1[row] << 16);
         }
     }
-    if (__builtin_amdgcn_ballot_w64(inexact) != 0 && lane == 0) atomicOr(&flags[2], 1u);
 }
 
 // ------------------------------------------------------------------------------------------ consume
