@@ -42,7 +42,7 @@ HBM_PEAK = 8.0e12
 
 
 # measured on MI355X with the counters named above, bytes per conv2_x launch (read + written)
-MEASURED_TRAFFIC_CONV2X = {"forward": (1581 + 65) * 2**20, "gradA": (1265 + 615) * 2**20, "gradB": (433 + 1) * 2**20}
+MEASURED_TRAFFIC_CONV2X = {"forward": (1581 + 65) * 2**20, "gradA": (1144 + 576) * 2**20, "gradB": (433 + 1) * 2**20}
 
 
 def main():
