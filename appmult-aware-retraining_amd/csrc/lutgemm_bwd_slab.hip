@@ -336,25 +336,43 @@ __global__ __launch_bounds__(1024) void lutgemm_gradB_slab16_kernel(
         const unsigned char* gbytes = reinterpret_cast<const unsigned char*>(gC);
         uint32_t al0[RU], ah0[RU], al1[RU], ah1[RU];
         f32x4 g0[RU], g1[RU];
+        // Every load batch is issued unconditionally (beyond the end: the last rows again, nobody consumes them): behind
+        // a branch around the loads the compiler's wait in front of the consumer has to cover the path without new
+        // loads too, and on the other path it then waits for the first of the loads it has just issued -- no prefetch
+        // at all (measured: the waves spent half their time in s_waitcnt).
+        int next = 0;
         auto load = [&](uint32_t (&al)[RU], uint32_t (&ah)[RU], f32x4 (&g)[RU]) {
 #pragma unroll
             for (int u = 0; u < RU; ++u) {
                 al[u] = load_u32_unaligned(A + aoff[u]);
                 ah[u] = load_u32_unaligned(A + aoff[u] + 4);
                 g[u] = *reinterpret_cast<const f32x4*>(gbytes + goff[u]);
-                aoff[u] += astep;
-                goff[u] += gstep;
             }
-        };
-        if (iters > 0) load(al0, ah0, g0);
-        for (int it = 0; it < iters; it += 2) {
-            if (it + 1 < iters) load(al1, ah1, g1);
+            ++next;
+            const uint32_t as = next < iters ? astep : 0u, gs = next < iters ? gstep : 0u;
 #pragma unroll
-            for (int u = 0; u < RU; ++u) consume(sums_tag, al0[u], ah0[u], g0[u]);
-            if (it + 1 < iters) {
-                if (it + 2 < iters) load(al0, ah0, g0);
+            for (int u = 0; u < RU; ++u) {
+                aoff[u] += as;
+                goff[u] += gs;
+            }
+            // (the scheduler would otherwise start on the consumer first, i.e. wait for the previous batch, and issue
+            // these loads behind that wait)
+            __builtin_amdgcn_sched_barrier(0);
+        };
+        if (iters > 0) {
+            load(al0, ah0, g0);
+            int it = 0;
+            for (; it + 2 <= iters; it += 2) {
+                load(al1, ah1, g1);
+#pragma unroll
+                for (int u = 0; u < RU; ++u) consume(sums_tag, al0[u], ah0[u], g0[u]);
+                load(al0, ah0, g0);
 #pragma unroll
                 for (int u = 0; u < RU; ++u) consume(sums_tag, al1[u], ah1[u], g1[u]);
+            }
+            if (it < iters) {
+#pragma unroll
+                for (int u = 0; u < RU; ++u) consume(sums_tag, al0[u], ah0[u], g0[u]);
             }
         }
     };
