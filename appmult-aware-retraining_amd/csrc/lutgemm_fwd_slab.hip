@@ -156,6 +156,12 @@ __device__ __forceinline__ void slab_chunk_fast(uint32_t (&acc)[RG][4], const ui
 #pragma unroll
     for (int b = 0; b < NB; ++b) {
         const int i = 2 * b;
+        // waves that are behind go first: the four waves of a SIMD then move through a chunk in step instead of one
+        // after the other (oldest first), and the last one does not run alone, latencies exposed, before the barrier
+        if (b == 0) __builtin_amdgcn_s_setprio(3);
+        else if (b == 1) __builtin_amdgcn_s_setprio(2);
+        else if (b == 2) __builtin_amdgcn_s_setprio(1);
+        else __builtin_amdgcn_s_setprio(0);
         if (b + 1 < NB) {
             uint32_t addr[8];
             slab_addr8<RG>(addr, a_cur, i + 2, base, sel);

@@ -456,10 +456,11 @@ hipError_t launch_gradA(const float* gC, const uint8_t* A, const uint8_t* B, flo
 
 // Bytes of the expanded table S, or 0 when the expanded-table gradA does not apply.
 size_t gradA_slab_workspace_bytes(const LutGeom& g, int M, int K, int N, bool force) {
-    // (below about 4096 rows, or 8192 for short K, the expansion, 2^b / M of the work but all of it HBM writes plus two
-    // more launches, costs more than it saves)
-    if (!force && M < 8192 && K < 1024) return 0;
-    if (g.bits > 7 || M < (force ? 2048 : 4096) || (N % kGaCols) != 0 || (K % 16) != 0 || (size_t)M * K >= (1ull << 31)) return 0;
+    // (below the thresholds the expansion, 2^b / M of the work but all of it HBM writes plus two more launches, costs
+    // more than it saves: measured cross-over on MI355X at about 1000 rows and 1e8 multiply-adds; with `force` only
+    // what the kernel cannot do is excluded)
+    if (!force && (M < 1024 || (double)M * K * N < 1e8)) return 0;
+    if (g.bits > 7 || M < 512 || (N % kGaCols) != 0 || (K % 16) != 0 || (size_t)M * K >= (1ull << 31)) return 0;
     return (size_t)(N / kGaCols) * (K / kGaChunkK) * kGaChunkBytes;
 }
 
@@ -480,7 +481,8 @@ hipError_t launch_gradA_slab(const float* gC, const uint8_t* A, const uint8_t* B
     // 16 row blocks x 2 k groups are in flight on an XCD at a time (measured: 8 to 32 row blocks make no difference)
     const int band_rows = 16;
     // (48 k per workgroup would need more registers than a wave of a 1024-thread workgroup has)
-    const int kt = (K % 32) == 0 ? 32 : 16;
+    // (fewer tiles than CUs: 16 k per tile, twice the tiles)
+    const int kt = ((K % 32) == 0 && row_blocks * (K / 32) >= n_cu) ? 32 : 16;
     const int tiles = row_blocks * (K / kt);
     const int per_xcd = (tiles + 7) / 8, cus_per_xcd = n_cu >= 8 ? n_cu / 8 : 1;
     const dim3 grid(8 * (per_xcd < cus_per_xcd ? per_xcd : cus_per_xcd));
