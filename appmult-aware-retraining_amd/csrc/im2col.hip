@@ -122,9 +122,57 @@ __global__ __launch_bounds__(256) void col2im_f32_kernel(const float* __restrict
     x[idx] = acc;
 }
 
+// The same gather for the usual window sizes, without branches: every thread issues the loads of all its taps at once
+// (addresses of taps that do not exist are clamped to the first entry and their values dropped), so that the kernel
+// runs at the speed of its reads, 9 x the size of the result for a 3x3 window, instead of one dependent load after the
+// other.  Same summation order as the generic kernel.
+template <int KH, int KW, int STRIDE>
+__global__ __launch_bounds__(256) void col2im_f32_taps_kernel(const float* __restrict__ cols, float* __restrict__ x, int C, int H, int W,
+                                                              int pad, int dil, int oh, int ow, size_t total) {
+    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= total) return;
+    const int xx = (int)(idx % W);
+    size_t r = idx / W;
+    const int yy = (int)(r % H);
+    r /= H;                                   // = b * C + c
+    const size_t L = (size_t)oh * ow;
+    const float* base = cols + r * (size_t)(KH * KW) * L;
+    float v[KH * KW];
+    bool ok[KH * KW];
+#pragma unroll
+    for (int i = 0; i < KH; ++i) {
+        const int ty = yy + pad - i * dil;
+        const int oy = ty / STRIDE;
+        const bool oky = ty >= 0 && (STRIDE == 1 || ty % STRIDE == 0) && oy < oh;
+#pragma unroll
+        for (int j = 0; j < KW; ++j) {
+            const int tx = xx + pad - j * dil;
+            const int ox = tx / STRIDE;
+            const int tap = i * KW + j;
+            ok[tap] = oky && tx >= 0 && (STRIDE == 1 || tx % STRIDE == 0) && ox < ow;
+            v[tap] = base[ok[tap] ? (size_t)tap * L + (size_t)oy * ow + ox : 0];
+        }
+    }
+    float acc = 0.f;
+#pragma unroll
+    for (int tap = 0; tap < KH * KW; ++tap) acc += ok[tap] ? v[tap] : 0.f;
+    x[idx] = acc;
+}
+
 hipError_t launch_col2im_f32(const float* cols, float* x, int B, int C, int H, int W, int kh, int kw, int stride, int pad, int dil,
                              int oh, int ow, hipStream_t stream) {
     const size_t total = (size_t)B * C * H * W;
+    const dim3 grid((unsigned)((total + 255) / 256));
+    if (total == 0) return hipSuccess;
+    if (kh == 3 && kw == 3 && stride == 1)
+        hipLaunchKernelGGL((col2im_f32_taps_kernel<3, 3, 1>), grid, dim3(256), 0, stream, cols, x, C, H, W, pad, dil, oh, ow, total);
+    else if (kh == 3 && kw == 3 && stride == 2)
+        hipLaunchKernelGGL((col2im_f32_taps_kernel<3, 3, 2>), grid, dim3(256), 0, stream, cols, x, C, H, W, pad, dil, oh, ow, total);
+    else if (kh == 1 && kw == 1 && stride == 1)
+        hipLaunchKernelGGL((col2im_f32_taps_kernel<1, 1, 1>), grid, dim3(256), 0, stream, cols, x, C, H, W, pad, dil, oh, ow, total);
+    else if (kh == 1 && kw == 1 && stride == 2)
+        hipLaunchKernelGGL((col2im_f32_taps_kernel<1, 1, 2>), grid, dim3(256), 0, stream, cols, x, C, H, W, pad, dil, oh, ow, total);
+    else
     hipLaunchKernelGGL(col2im_f32_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, cols, x, C, H, W, kh, kw,
                        stride, pad, dil, oh, ow, total);
     return hipGetLastError();
