@@ -232,7 +232,7 @@ __global__ __launch_bounds__(1024) void lutgemm_gradB_slab16_kernel(
     const int16_t* __restrict__ G, int lut_cols, int n_codes, uint32_t* __restrict__ flags, int M, int K, int N,
     int m_chunk, float scale, int n_tiles, int k_tiles, int splits) {
     constexpr int KT = kBwdKT16;
-    __shared__ __align__(16) unsigned char smem[KT * 16384];
+    __shared__ __align__(16) unsigned char smem[KT * 16384 + 32768];     // slabs + the table as halves
     const int tid = threadIdx.x;
     const int wave = uniform(tid >> 6);
     const int lane = tid & 63;
@@ -254,33 +254,40 @@ __global__ __launch_bounds__(1024) void lutgemm_gradB_slab16_kernel(
     const int me = min(M, mb + m_chunk);
     const float offset = (float)flags[4];        // 0 or 1024 (bwd_header_kernel)
 
-    {   // expansion: wave-uniform code a, lanes = columns (the gathers of a wave stay inside one table row).
-        // All loads of a step are issued before the first is used: the table sits in L2 and a dependent
-        // load-convert-store chain would pay that latency 64 times per workgroup.
-        const int col = lane;
+    {   // expansion.  First the table itself goes to LDS, as halves, 128 x 128 without the padding (32 KB behind the
+        // slabs; codes the table does not have read as zero): 16 independent loads per thread, one trip to L2.
+        // The slabs are then gathered from that copy: wave-uniform code a, lanes = columns.  (Gathering them from
+        // the table in global memory took 64 loads per thread in 8 dependent rounds: 5 of the 12 us a workgroup
+        // spends outside its streaming loop, a third of the run time of a layer of 4096 rows.)
+        _Float16* tab = reinterpret_cast<_Float16*>(smem + KT * 16384);
         bool inexact = false;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int idx = tid + 1024 * i, a = idx >> 7, b = idx & 127;
+            const float v = (a < n_codes && b < n_codes) ? (float)G[a * lut_cols + b] - offset : -offset;
+            const _Float16 h = (_Float16)v;
+            inexact |= ((float)h != v);
+            tab[idx] = h;
+        }
+        if (__builtin_amdgcn_ballot_w64(inexact) != 0 && lane == 0) atomicOr(&flags[1], 1u);
+        const int col = lane;
         int bcode[KT];
 #pragma unroll
         for (int kk = 0; kk < KT; ++kk) bcode[kk] = (int)B[(size_t)(k0 + kk) * N + n0 + col];
+        __syncthreads();
+        const _Float16 zero = (_Float16)(-offset);
 #pragma unroll
         for (int kk = 0; kk < KT; ++kk) {
             unsigned char* s = smem + (kk >> 1) * 32768 + (kk & 1) * 128 + 2 * col;
-            int16_t e[kBwdSlabRows / 16];
-#pragma unroll
-            for (int i = 0; i < kBwdSlabRows / 16; ++i) {
-                const int a = min(wave + 16 * i, n_codes - 1);
-                e[i] = G[a * lut_cols + bcode[kk]];
-            }
+            const bool masked = bcode[kk] > 127;           // the masked code of a 7-bit operand: the table's zero column
+            const _Float16* t = tab + min(bcode[kk], 127);
 #pragma unroll
             for (int i = 0; i < kBwdSlabRows / 16; ++i) {
                 const int a = wave + 16 * i;
-                const float v = (a < n_codes) ? (float)e[i] : 0.f;
-                const _Float16 h = (_Float16)(v - offset);
-                inexact |= ((float)h != v - offset);
-                *reinterpret_cast<_Float16*>(s + a * 256) = h;
+                const _Float16 h = t[a * 128];
+                *reinterpret_cast<_Float16*>(s + a * 256) = masked ? zero : h;
             }
         }
-        if (__builtin_amdgcn_ballot_w64(inexact) != 0 && lane == 0) atomicOr(&flags[1], 1u);
     }
     __syncthreads();
 
