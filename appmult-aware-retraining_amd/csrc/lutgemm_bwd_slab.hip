@@ -489,7 +489,8 @@ __global__ void reduce_partials_kernel(const float* __restrict__ partial, float*
 
 bool bwd_slab_applies(const LutGeom& g, int M, int K, int N) {
     (void)N;
-    return g.bits <= 7 && M >= 4096 && K >= 4;
+    // (measured cross-over against the direct kernel on MI355X: between 512 and 1024 rows)
+    return g.bits <= 7 && M >= 1024 && K >= 4;
 }
 
 // M splits of the expanded-table gradB.  A workgroup fills a CU (128 KB of LDS), so the grid runs in rounds

@@ -213,8 +213,9 @@ def test_backward_within_tolerance_random_tables(lib, oracle, bits, shape):
     check_backward(oracle, gpu_backward(lib, g, A, B, la, lb), g, A, B, la, lb, bits)
 
 
-# M >= 4096 takes the expanded-table backward kernels (tables of at most 7 bits); N > 256 needs two passes of gradA
-BWD_BIG_M_SHAPES = [(4096, 8, 64), (4100, 27, 10), (5000, 130, 65), (4096, 64, 300), (4500, 70, 129), (4096, 33, 513), (9000, 5, 200)]
+# M >= 1024 takes the expanded-table backward kernels (tables of at most 7 bits)
+BWD_BIG_M_SHAPES = [(4096, 8, 64), (4100, 27, 10), (5000, 130, 65), (4096, 64, 300), (4500, 70, 129), (4096, 33, 513), (9000, 5, 200),
+                    (1024, 64, 64), (1500, 40, 70), (3000, 130, 65), (1100, 9, 200)]
 
 
 @pytest.mark.parametrize("bits", [7, 6, 8])
@@ -248,7 +249,7 @@ def test_backward_large_m_masked_codes(lib, oracle):
 # (N % 32 == 0, K % 16 == 0 and M >= 2048: gradA runs on its own expanded table, 16, 32 or 48 k per workgroup and one to
 # six column tiles, also with a ragged last row block)
 HALF_SLAB_SHAPES = [(4096, 8, 64), (4224, 24, 128), (8192, 64, 64), (16384, 16, 192), (8200, 48, 96), (9001, 64, 32),
-                    (4100, 32, 64), (2148, 144, 160), (5000, 80, 128)]
+                    (4100, 32, 64), (2148, 144, 160), (5000, 80, 128), (1024, 16, 64), (2048, 48, 128), (1280, 64, 192)]
 
 
 @pytest.mark.parametrize("bits", [7, 6, 4])
