@@ -36,6 +36,7 @@ _lib.amr_last_error.restype = ctypes.c_char_p
 _lib.amr_target_arch.restype = ctypes.c_char_p
 _lib.amr_lut_gemm_forward.argtypes = [_vp, _vp, _vp, _vp, _i64, _i, _i, _i, _vp]
 _lib.amr_lut_gemm_forward_ws.argtypes = [_vp, _vp, _vp, _vp, _i64, _i, _i, _i, _vp, _sz, _vp]
+_lib.amr_lut_gemm_forward_f32_ws.argtypes = [_vp, _vp, _vp, _vp, _i64, _i, _i, _i, _vp, _sz, _vp]
 _lib.amr_lut_gemm_forward_workspace_bytes.argtypes = [_i64, _i, _i, _i]
 _lib.amr_lut_gemm_forward_workspace_bytes.restype = _sz
 _lib.amr_lut_gemm_backward.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i, _i, _i, _vp, _sz, _vp]
@@ -89,10 +90,13 @@ def _stream_ptr(device):
 
 def approx_gemm_forward(a_tensor, b_tensor, c_tensor, lut_appmult_tensor):
     """c[m,n] = sum_k lut[a[m,k]][b[k,n]]; a u8 [M,K], b u8 [K,N], c u32 [M,N] (out), lut u16 padded table.
-    Contract of approx_gemm_forward_gpu (self_ops/src/approx_gemm_forward.cu:241-259)."""
+    Contract of approx_gemm_forward_gpu (self_ops/src/approx_gemm_forward.cu:241-259).
+    A float32 c_tensor receives the same sums converted to float32 (what the reference's callers do with the uint32
+    result at once, self_ops/ops_py/approx_ops.py:569) without the extra pass over it."""
     _check_input(a_tensor, torch.uint8, "a_tensor")
     _check_input(b_tensor, torch.uint8, "b_tensor")
-    _check_input(c_tensor, torch.uint32, "c_tensor")
+    as_float = c_tensor.dtype == torch.float32
+    _check_input(c_tensor, torch.float32 if as_float else torch.uint32, "c_tensor")
     _check_input(lut_appmult_tensor, torch.uint16, "lut_appmult_tensor")
     _check(a_tensor.dim() == 2 and b_tensor.dim() == 2 and c_tensor.dim() == 2, "a, b and c must be 2-D")
     M, K = a_tensor.shape
@@ -107,9 +111,9 @@ def approx_gemm_forward(a_tensor, b_tensor, c_tensor, lut_appmult_tensor):
         # ordered with the stream like any other tensor and freed with the process' other device memory
         need = _lib.amr_lut_gemm_forward_workspace_bytes(lut_appmult_tensor.size(0), M, K, N)
         ws = torch.empty(need, dtype=torch.uint8, device=dev) if need else None
-        rc = _lib.amr_lut_gemm_forward_ws(a_tensor.data_ptr(), b_tensor.data_ptr(), c_tensor.data_ptr(),
-                                          lut_appmult_tensor.data_ptr(), lut_appmult_tensor.size(0), M, K, N,
-                                          ws.data_ptr() if ws is not None else None, need, _stream_ptr(dev))
+        entry = _lib.amr_lut_gemm_forward_f32_ws if as_float else _lib.amr_lut_gemm_forward_ws
+        rc = entry(a_tensor.data_ptr(), b_tensor.data_ptr(), c_tensor.data_ptr(), lut_appmult_tensor.data_ptr(),
+                   lut_appmult_tensor.size(0), M, K, N, ws.data_ptr() if ws is not None else None, need, _stream_ptr(dev))
     _raise_for(rc, "approx_gemm_forward")
 
 

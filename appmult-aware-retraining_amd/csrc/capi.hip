@@ -11,10 +11,10 @@
 
 namespace amr {
 hipError_t launch_fwd(const uint8_t* A, const uint8_t* B, uint32_t* C, const uint16_t* lut, const LutGeom& g, int M,
-                      int K, int N, int n_cu, hipStream_t stream);
+                      int K, int N, int n_cu, hipStream_t stream, int out_f32);
 size_t fwd_slab_workspace_bytes(const LutGeom& g, int M, int K, int N, bool force);
 hipError_t launch_fwd_slab(const uint8_t* A, const uint8_t* B, uint32_t* C, const uint16_t* lut, const LutGeom& g,
-                           int M, int K, int N, int n_cu, void* workspace, hipStream_t stream);
+                           int M, int K, int N, int n_cu, void* workspace, hipStream_t stream, int out_f32);
 size_t gradB_workspace_bytes(int M, int K, int N, int n_cu, int* splits_out);
 hipError_t launch_gradB(const float* gC, const uint8_t* A, const uint8_t* B, float* gB, const int16_t* lut,
                         const LutGeom& g, int M, int K, int N, float scale, void* workspace, int splits,
@@ -151,8 +151,8 @@ size_t amr_lut_gemm_forward_workspace_bytes(int64_t lut_elems, int M, int K, int
     return g_expanded_kernels ? amr::fwd_slab_workspace_bytes(g, M, K, N, g_expanded_kernels == 2) : 0;
 }
 
-int amr_lut_gemm_forward_ws(const uint8_t* A, const uint8_t* B, uint32_t* C, const uint16_t* lut, int64_t lut_elems,
-                            int M, int K, int N, void* workspace, size_t workspace_bytes, void* stream) {
+static int forward_impl(const uint8_t* A, const uint8_t* B, uint32_t* C, const uint16_t* lut, int64_t lut_elems, int M, int K, int N,
+                        void* workspace, size_t workspace_bytes, void* stream, int out_f32) {
     if (M < 0 || K < 0 || N < 0) return fail(AMR_EINVAL, "negative dimension M=%d K=%d N=%d", M, K, N);
     amr::LutGeom g;
     if (!amr::lut_geom_from_elems(lut_elems, &g))
@@ -179,11 +179,22 @@ int amr_lut_gemm_forward_ws(const uint8_t* A, const uint8_t* B, uint32_t* C, con
             ws = internal_workspace(dev, need, &e);
             if (!ws) return hip_fail(e, "workspace hipMalloc");
         }
-        e = amr::launch_fwd_slab(A, B, C, lut, g, M, K, N, n_cu, ws, s);
+        e = amr::launch_fwd_slab(A, B, C, lut, g, M, K, N, n_cu, ws, s, out_f32);
     } else {
-        e = amr::launch_fwd(A, B, C, lut, g, M, K, N, n_cu, s);
+        e = amr::launch_fwd(A, B, C, lut, g, M, K, N, n_cu, s, out_f32);
     }
     return e == hipSuccess ? AMR_OK : hip_fail(e, "forward launch");
+}
+
+int amr_lut_gemm_forward_ws(const uint8_t* A, const uint8_t* B, uint32_t* C, const uint16_t* lut, int64_t lut_elems,
+                            int M, int K, int N, void* workspace, size_t workspace_bytes, void* stream) {
+    return forward_impl(A, B, C, lut, lut_elems, M, K, N, workspace, workspace_bytes, stream, 0);
+}
+
+int amr_lut_gemm_forward_f32_ws(const uint8_t* A, const uint8_t* B, float* C, const uint16_t* lut, int64_t lut_elems,
+                                int M, int K, int N, void* workspace, size_t workspace_bytes, void* stream) {
+    // (a zero of either type has the same bits: the empty sums of K == 0 need no conversion)
+    return forward_impl(A, B, reinterpret_cast<uint32_t*>(C), lut, lut_elems, M, K, N, workspace, workspace_bytes, stream, 1);
 }
 
 int amr_lut_gemm_forward(const uint8_t* A, const uint8_t* B, uint32_t* C, const uint16_t* lut, int64_t lut_elems,

@@ -17,12 +17,15 @@
 namespace amr {
 
 hipError_t launch_zero_u32(void* p, size_t n_dwords, hipStream_t stream);
+hipError_t launch_u32_to_f32(void* p, size_t n_dwords, hipStream_t stream);
 
+// out_f32: C receives the sums converted to float32 (what the reference's callers do with the result at once,
+// self_ops/ops_py/approx_ops.py:569), not the uint32 sums.
 template <int R, int TN, int WAVES>
 __global__ __launch_bounds__(WAVES * 64) void lutgemm_fwd_kernel(
     const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, uint32_t* __restrict__ C,
     const uint32_t* __restrict__ lut32, int lut_dwords, int row_bytes, int M, int K, int N, int k_chunk,
-    int atomic_out, const uint32_t* __restrict__ gate) {
+    int atomic_out, const uint32_t* __restrict__ gate, int out_f32) {
     extern __shared__ __align__(16) unsigned char smem[];
     if (gate != nullptr && *gate == 0u) return;   // queued as a fallback that turned out not to be needed
     {
@@ -118,6 +121,8 @@ __global__ __launch_bounds__(WAVES * 64) void lutgemm_fwd_kernel(
             if (n < N) {
                 if (atomic_out)
                     atomicAdd(&C[(size_t)m * N + n], acc[i][j]);
+                else if (out_f32)
+                    C[(size_t)m * N + n] = __float_as_uint((float)acc[i][j]);
                 else
                     C[(size_t)m * N + n] = acc[i][j];
             }
@@ -127,7 +132,7 @@ __global__ __launch_bounds__(WAVES * 64) void lutgemm_fwd_kernel(
 
 template <int R, int TN, int WAVES>
 static hipError_t launch_fwd_t(const uint8_t* A, const uint8_t* B, uint32_t* C, const uint16_t* lut, const LutGeom& g,
-                               int M, int K, int N, int ksplit, hipStream_t stream, const uint32_t* gate = nullptr) {
+                               int M, int K, int N, int ksplit, hipStream_t stream, const uint32_t* gate = nullptr, int out_f32 = 0) {
     const int lut_dwords = g.rows * g.cols / 2;  // rows*cols is even for every supported bit-width
     const size_t lds = (size_t)lut_dwords * 4;
     auto kern = lutgemm_fwd_kernel<R, TN, WAVES>;
@@ -145,15 +150,17 @@ static hipError_t launch_fwd_t(const uint8_t* A, const uint8_t* B, uint32_t* C, 
         if (e != hipSuccess) return e;
     }
     hipLaunchKernelGGL(kern, grid, dim3(WAVES * 64), lds, stream, A, B, C, reinterpret_cast<const uint32_t*>(lut),
-                       lut_dwords, g.cols * 2, M, K, N, k_chunk, zs > 1 ? 1 : 0, gate);
-    return hipGetLastError();
+                       lut_dwords, g.cols * 2, M, K, N, k_chunk, zs > 1 ? 1 : 0, gate, out_f32);
+    hipError_t e = hipGetLastError();
+    if (e == hipSuccess && zs > 1 && out_f32) e = launch_u32_to_f32(C, (size_t)M * N, stream);
+    return e;
 }
 
 // Tile selection.  n_cu: compute units of the device.  The table occupies 33.5 KB (7-bit) so four
 // 256-thread workgroups fit a CU; the 8-bit table (132.6 KB) leaves room for one workgroup, which
 // is therefore made 1024 threads wide.
 hipError_t launch_fwd(const uint8_t* A, const uint8_t* B, uint32_t* C, const uint16_t* lut, const LutGeom& g, int M,
-                      int K, int N, int n_cu, hipStream_t stream) {
+                      int K, int N, int n_cu, hipStream_t stream, int out_f32) {
     const bool big = g.bits == 8;
     const int waves = big ? 16 : 4;
     int R, TN;
@@ -173,8 +180,8 @@ hipError_t launch_fwd(const uint8_t* A, const uint8_t* B, uint32_t* C, const uin
     }
 #define AMR_FWD_CASE(r, tn)                                                                                   \
     if (R == r && TN == tn)                                                                                   \
-        return big ? launch_fwd_t<r, tn, 16>(A, B, C, lut, g, M, K, N, ksplit, stream)                         \
-                   : launch_fwd_t<r, tn, 4>(A, B, C, lut, g, M, K, N, ksplit, stream);
+        return big ? launch_fwd_t<r, tn, 16>(A, B, C, lut, g, M, K, N, ksplit, stream, nullptr, out_f32)       \
+                   : launch_fwd_t<r, tn, 4>(A, B, C, lut, g, M, K, N, ksplit, stream, nullptr, out_f32);
     AMR_FWD_CASE(32, 1)
     AMR_FWD_CASE(16, 1)
     AMR_FWD_CASE(32, 2)
@@ -187,10 +194,10 @@ hipError_t launch_fwd(const uint8_t* A, const uint8_t* B, uint32_t* C, const uin
 // Direct kernel queued behind the expanded-table kernel: it runs only when *gate != 0 (the operand
 // held a masked code) and then overwrites all of C, so it must not split K.
 hipError_t launch_fwd_gated(const uint8_t* A, const uint8_t* B, uint32_t* C, const uint16_t* lut, const LutGeom& g,
-                            int M, int K, int N, const uint32_t* gate, hipStream_t stream) {
-    if (N <= 64) return launch_fwd_t<32, 1, 4>(A, B, C, lut, g, M, K, N, 1, stream, gate);
-    if (N <= 128) return launch_fwd_t<32, 2, 4>(A, B, C, lut, g, M, K, N, 1, stream, gate);
-    return launch_fwd_t<16, 4, 4>(A, B, C, lut, g, M, K, N, 1, stream, gate);
+                            int M, int K, int N, const uint32_t* gate, hipStream_t stream, int out_f32) {
+    if (N <= 64) return launch_fwd_t<32, 1, 4>(A, B, C, lut, g, M, K, N, 1, stream, gate, out_f32);
+    if (N <= 128) return launch_fwd_t<32, 2, 4>(A, B, C, lut, g, M, K, N, 1, stream, gate, out_f32);
+    return launch_fwd_t<16, 4, 4>(A, B, C, lut, g, M, K, N, 1, stream, gate, out_f32);
 }
 
 }  // namespace amr

@@ -34,6 +34,7 @@
 namespace amr {
 
 hipError_t launch_zero_u32(void* p, size_t n_dwords, hipStream_t stream);
+hipError_t launch_u32_to_f32(void* p, size_t n_dwords, hipStream_t stream);
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));   // native 16-byte vector (stays in registers)
 
@@ -230,7 +231,7 @@ __device__ __forceinline__ void slab_read_codes(uint32_t (&a)[8], uint32_t addr)
 template <int RG, int WAVES, bool PACKED>
 __global__ __launch_bounds__(WAVES * 64) void lutgemm_fwd_slab_kernel(
     const uint8_t* __restrict__ A, const u32x4* __restrict__ E, uint32_t* __restrict__ C,
-    uint32_t* __restrict__ flags, int M, int K, int N, int k_quads, int chunks_per_split, int atomic_out) {
+    uint32_t* __restrict__ flags, int M, int K, int N, int k_quads, int chunks_per_split, int atomic_out, int out_f32) {
     // static: lets the compiler fold the base address (chunk buffers first: their addresses come out of v_perm)
     __shared__ __align__(16) unsigned char smem[kSlabBuffers * kSlabChunkBytes + 2 * kSlabCodeBytes];
     constexpr int THREADS = WAVES * 64;
@@ -344,6 +345,8 @@ __global__ __launch_bounds__(WAVES * 64) void lutgemm_fwd_slab_kernel(
                 if (n + c < N) {
                     if (atomic_out)
                         atomicAdd(&C[(size_t)m * N + n + c], acc[i][c]);
+                    else if (out_f32)
+                        C[(size_t)m * N + n + c] = __float_as_uint((float)acc[i][c]);
                     else
                         C[(size_t)m * N + n + c] = acc[i][c];
                 }
@@ -353,7 +356,7 @@ __global__ __launch_bounds__(WAVES * 64) void lutgemm_fwd_slab_kernel(
 }
 
 hipError_t launch_fwd_gated(const uint8_t* A, const uint8_t* B, uint32_t* C, const uint16_t* lut, const LutGeom& g,
-                            int M, int K, int N, const uint32_t* gate, hipStream_t stream);
+                            int M, int K, int N, const uint32_t* gate, hipStream_t stream, int out_f32);
 
 // ------------------------------------------------------------------------------------------ host
 // Workspace layout: [256 B flags][E].  Returns 0 when the expanded-table path does not apply.
@@ -371,7 +374,7 @@ size_t fwd_slab_workspace_bytes(const LutGeom& g, int M, int K, int N, bool forc
 }
 
 hipError_t launch_fwd_slab(const uint8_t* A, const uint8_t* B, uint32_t* C, const uint16_t* lut, const LutGeom& g,
-                           int M, int K, int N, int n_cu, void* workspace, hipStream_t stream) {
+                           int M, int K, int N, int n_cu, void* workspace, hipStream_t stream, int out_f32) {
     const int n_tiles = (N + kSlabCols - 1) / kSlabCols;
     const int k_quads = (K + 3) / 4;
     uint32_t* flags = reinterpret_cast<uint32_t*>(workspace);
@@ -404,12 +407,17 @@ hipError_t launch_fwd_slab(const uint8_t* A, const uint8_t* B, uint32_t* C, cons
     dim3 grid(n_tiles, (M + m_tile - 1) / m_tile, zs);
     // both accumulation flavours are queued; flags[0] (table maximum) decides on the device which one works
     hipLaunchKernelGGL((lutgemm_fwd_slab_kernel<RG, WAVES, true>), grid, dim3(WAVES * 64), 0, stream, A,
-                       reinterpret_cast<const u32x4*>(E), C, flags, M, K, N, k_quads, cps, zs > 1 ? 1 : 0);
+                       reinterpret_cast<const u32x4*>(E), C, flags, M, K, N, k_quads, cps, zs > 1 ? 1 : 0, out_f32);
     hipLaunchKernelGGL((lutgemm_fwd_slab_kernel<RG, WAVES, false>), grid, dim3(WAVES * 64), 0, stream, A,
-                       reinterpret_cast<const u32x4*>(E), C, flags, M, K, N, k_quads, cps, zs > 1 ? 1 : 0);
+                       reinterpret_cast<const u32x4*>(E), C, flags, M, K, N, k_quads, cps, zs > 1 ? 1 : 0, out_f32);
     e = hipGetLastError();
     if (e != hipSuccess) return e;
-    if (g.bits == 7) return launch_fwd_gated(A, B, C, lut, g, M, K, N, flags + 1, stream);
+    // (partial sums over a split K met as integers: converted before the fall-back, which stores floats itself)
+    if (zs > 1 && out_f32) {
+        e = launch_u32_to_f32(C, (size_t)M * N, stream);
+        if (e != hipSuccess) return e;
+    }
+    if (g.bits == 7) return launch_fwd_gated(A, B, C, lut, g, M, K, N, flags + 1, stream, out_f32);
     return hipGetLastError();
 }
 

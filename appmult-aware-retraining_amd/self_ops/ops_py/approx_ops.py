@@ -93,9 +93,10 @@ def _codes(x):
 
 def _lut_forward(a_codes, b_codes):
     M, N = a_codes.shape[0], b_codes.shape[1]
-    c = torch.empty((M, N), dtype=torch.uint32, device=a_codes.device)
+    # float32 output: the uint32 sums converted by the kernel's store (the reference converts them in a pass of its own)
+    c = torch.empty((M, N), dtype=torch.float32, device=a_codes.device)
     approx_ops.approx_gemm_forward(a_codes, b_codes, c, lut_appmult)
-    return c.to(torch.float32)
+    return c
 
 
 class AccGemm(Function):

@@ -71,6 +71,15 @@ int amr_lut_gemm_forward_ws(const uint8_t *A, const uint8_t *B, uint32_t *C, con
                             void *stream);
 
 /*
+ * Same sums, stored as float32: C[m,n] = (float)(uint32 sum), rounded to nearest even above 2^24, i.e. the
+ * bits of the `.to(torch.float32)` the reference's callers apply to the result at once
+ * (self_ops/ops_py/approx_ops.py:569, :165) without the pass over C that conversion costs.
+ */
+int amr_lut_gemm_forward_f32_ws(const uint8_t *A, const uint8_t *B, float *C, const uint16_t *lut,
+                                int64_t lut_elems, int M, int K, int N, void *workspace, size_t workspace_bytes,
+                                void *stream);
+
+/*
  * Backward (both gradients, as the reference always produces both):
  *   gA[m,k] = (1/16) * sum_{n<N} gC[m,n] * (float)lut_grad_a[A[m,k] * cols + B[k,n]]
  *   gB[k,n] = (1/16) * sum_{m<M} (float)lut_grad_b[A[m,k] * cols + B[k,n]] * gC[m,n]

@@ -26,6 +26,7 @@ def lib():
     L.amr_last_error.restype = ctypes.c_char_p
     L.amr_lut_gemm_forward.argtypes = [vp, vp, vp, vp, i64, i, i, i, vp]
     L.amr_lut_gemm_forward_ws.argtypes = [vp, vp, vp, vp, i64, i, i, i, vp, sz, vp]
+    L.amr_lut_gemm_forward_f32_ws.argtypes = [vp, vp, vp, vp, i64, i, i, i, vp, sz, vp]
     L.amr_lut_gemm_forward_workspace_bytes.argtypes = [i64, i, i, i]
     L.amr_lut_gemm_forward_workspace_bytes.restype = sz
     L.amr_lut_gemm_backward.argtypes = [vp, vp, vp, vp, vp, vp, vp, i64, i, i, i, vp, sz, vp]
@@ -176,6 +177,37 @@ def test_forward_golden_shipped_tables(lib, oracle, golden_dir):
     _, A, B, _ = rand_case(6, 200, 150, 80, 8)
     flat = oracle.pack_table(z["fwd"], 8, np.uint16)
     assert (gpu_forward(lib, A, B, flat) == oracle.forward_np(A, B, z["fwd"])).all()
+
+
+# the float32 output of the forward pass = the uint32 sums converted with round-to-nearest-even (what torch's
+# .to(float32) does): direct kernels, K split over workgroups (small M), expanded-table kernels, both table widths of the
+# packed / unpacked flavours, the masked-code fall-back, sums beyond 2^24 and wrapped sums
+@pytest.mark.parametrize("bits,shape,big", [(7, (37, 530, 70), False), (7, (300, 2048, 64), True), (8, (100, 300, 130), True),
+                                            (7, (4096, 576, 64), False), (7, (2048, 4608, 96), True), (6, (2100, 600, 33), False),
+                                            (7, (2048, 1024, 64), True), (4, (4100, 512, 40), False)])
+def test_forward_float_output_is_the_converted_integer_sum(lib, oracle, bits, shape, big):
+    print("forward f32", bits, shape, big, flush=True)
+    M, K, N = shape
+    rng, A, B, _ = rand_case(hash((bits, shape, "f32")) % 2**32, M, K, N, bits)
+    n = 1 << bits
+    T = rng.integers(60000, 65536, (n, n)) if big else rng.integers(0, 300, (n, n))      # big: sums pass 2^24 (and 2^32 for long K)
+    flat = oracle.pack_table(T, bits, np.uint16)
+    if bits == 7:
+        A[::9, 5] = 128            # masked codes: the fall-back kernel stores the floats itself
+    want = gpu_forward(lib, A, B, flat)
+    assert (want == oracle.forward_c(A, B, flat, bits)).all()
+    a, b, l = dev(A), dev(B), dev(flat)
+    c = torch.full((M, N), float("nan"), device="cuda")
+    need = lib.amr_lut_gemm_forward_workspace_bytes(l.numel(), M, K, N)
+    ws = torch.empty(max(need, 1), dtype=torch.uint8, device="cuda")
+    rc = lib.amr_lut_gemm_forward_f32_ws(a.data_ptr(), b.data_ptr(), c.data_ptr(), l.data_ptr(), l.numel(), M, K, N, ws.data_ptr(),
+                                         need, None)
+    assert rc == 0, lib.amr_last_error()
+    torch.cuda.synchronize()
+    ref = torch.from_numpy(want.astype(np.int64)).to(torch.float32)          # int64 -> float32: round to nearest even
+    assert torch.equal(c.cpu(), ref)
+    if big:
+        assert (want > 2**24).any()
 
 
 def test_forward_wraparound_and_k_zero(lib, oracle):
