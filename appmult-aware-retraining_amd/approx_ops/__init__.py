@@ -41,6 +41,7 @@ _lib.amr_lut_gemm_forward_workspace_bytes.argtypes = [_i64, _i, _i, _i]
 _lib.amr_lut_gemm_forward_workspace_bytes.restype = _sz
 _lib.amr_lut_gemm_backward.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i, _i, _i, _vp, _sz, _vp]
 _lib.amr_lut_gemm_backward_ex.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i, _i, _i, _i, _vp, _sz, _vp]
+_lib.amr_lut_gemm_backward_f32tab.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, ctypes.c_float, _i, _i, _i, _i, _vp, _sz, _vp]
 _lib.amr_im2col_u8_f32.argtypes = [_vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp]
 _lib.amr_col2im_f32.argtypes = [_vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp]
 _lib.amr_conv_dequant_f32.argtypes = [_vp] * 10 + [_i, _i, _i, _vp]
@@ -135,9 +136,13 @@ def acc_gemm_forward_fp32(a_tensor, b_tensor, c_tensor):
 
 
 def approx_gemm_backward(gc_tensor, a_tensor, b_tensor, ga_tensor, gb_tensor, lut_grad_a_tensor, lut_grad_b_tensor,
-                         ga_rows_per_image=0):
+                         ga_rows_per_image=0, grad_scale=None):
     """ga[m,k] = 1/16 sum_n gc[m,n]*lutA[a][b], gb[k,n] = 1/16 sum_m lutB[a][b]*gc[m,n]; outputs overwritten.
     Contract of approx_gemm_backward_gpu (self_ops/src/approx_gemm_backward.cu:506-529).
+
+    The tables are int16 (slope x 16, as the reference's) or, as an extension, both float32: then the entries are the
+    slopes themselves and the factor in front of the sums is grad_scale (default 1).  grad_scale is not accepted
+    with int16 tables (their factor is the reference's 1/16).
 
     ga_rows_per_image = L > 0 (an extension; the reference has no such argument) makes ga_tensor the image-major
     transposed gradient of shape [M/L, K, L], the layout torch's fold takes."""
@@ -150,8 +155,10 @@ def approx_gemm_backward(gc_tensor, a_tensor, b_tensor, ga_tensor, gb_tensor, lu
         _check_input(ga_tensor, torch.float32, "ga_tensor")
     if gb_tensor is not None:
         _check_input(gb_tensor, torch.float32, "gb_tensor")
-    _check_input(lut_grad_a_tensor, torch.int16, "lut_grad_a_tensor")
-    _check_input(lut_grad_b_tensor, torch.int16, "lut_grad_b_tensor")
+    float_tables = lut_grad_a_tensor.dtype == torch.float32 and lut_grad_b_tensor.dtype == torch.float32
+    _check_input(lut_grad_a_tensor, torch.float32 if float_tables else torch.int16, "lut_grad_a_tensor")
+    _check_input(lut_grad_b_tensor, torch.float32 if float_tables else torch.int16, "lut_grad_b_tensor")
+    _check(float_tables or grad_scale is None, "grad_scale needs float32 gradient tables")
     L = int(ga_rows_per_image)
     _check(all(t.dim() == 2 for t in (gc_tensor, a_tensor, b_tensor)) and (gb_tensor is None or gb_tensor.dim() == 2), "gc, a, b and gb must be 2-D")
     M, K = a_tensor.shape
@@ -175,11 +182,18 @@ def approx_gemm_backward(gc_tensor, a_tensor, b_tensor, ga_tensor, gb_tensor, lu
     with torch.cuda.device(dev):
         need = _lib.amr_lut_gemm_backward_workspace_bytes(M, K, N)
         ws = torch.empty(need, dtype=torch.uint8, device=dev) if need else None
-        rc = _lib.amr_lut_gemm_backward_ex(gc_tensor.data_ptr(), a_tensor.data_ptr(), b_tensor.data_ptr(),
-                                           ga_tensor.data_ptr() if ga_tensor is not None else None,
-                                           gb_tensor.data_ptr() if gb_tensor is not None else None, lut_grad_a_tensor.data_ptr(),
-                                           lut_grad_b_tensor.data_ptr(), lut_grad_a_tensor.size(0), M, K, N, L,
-                                           ws.data_ptr() if ws is not None else None, need, _stream_ptr(dev))
+        ga_ptr = ga_tensor.data_ptr() if ga_tensor is not None else None
+        gb_ptr = gb_tensor.data_ptr() if gb_tensor is not None else None
+        ws_ptr = ws.data_ptr() if ws is not None else None
+        if float_tables:
+            rc = _lib.amr_lut_gemm_backward_f32tab(gc_tensor.data_ptr(), a_tensor.data_ptr(), b_tensor.data_ptr(), ga_ptr, gb_ptr,
+                                                   lut_grad_a_tensor.data_ptr(), lut_grad_b_tensor.data_ptr(),
+                                                   lut_grad_a_tensor.size(0), 1.0 if grad_scale is None else float(grad_scale),
+                                                   M, K, N, L, ws_ptr, need, _stream_ptr(dev))
+        else:
+            rc = _lib.amr_lut_gemm_backward_ex(gc_tensor.data_ptr(), a_tensor.data_ptr(), b_tensor.data_ptr(), ga_ptr, gb_ptr,
+                                               lut_grad_a_tensor.data_ptr(), lut_grad_b_tensor.data_ptr(),
+                                               lut_grad_a_tensor.size(0), M, K, N, L, ws_ptr, need, _stream_ptr(dev))
     _raise_for(rc, "approx_gemm_backward")
 
 

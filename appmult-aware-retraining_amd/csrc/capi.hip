@@ -47,6 +47,15 @@ int gradB_slab_splits(int M, int K, int N, int n_cu);
 hipError_t launch_gradB_slab(const float* gC, const uint8_t* A, const uint8_t* B, float* gB, const int16_t* lut,
                              const LutGeom& g, int M, int K, int N, float scale, uint32_t* flags, float* partials,
                              int n_cu, hipStream_t stream);
+hipError_t launch_gradB_f32tab(const float* gC, const uint8_t* A, const uint8_t* B, float* gB, const float* lut, const LutGeom& g,
+                               int M, int K, int N, float scale, void* workspace, int splits, hipStream_t stream,
+                               const uint32_t* gate);
+hipError_t launch_gradA_f32tab(const float* gC, const uint8_t* A, const uint8_t* B, float* gA, const float* lut, const LutGeom& g,
+                               int M, int K, int N, float scale, int n_cu, hipStream_t stream, const uint32_t* gate,
+                               int rows_per_image);
+hipError_t launch_gradB_slab_f32tab(const float* gC, const uint8_t* A, const uint8_t* B, float* gB, const float* lut,
+                                    const LutGeom& g, int M, int K, int N, float scale, uint32_t* flags, float* partials,
+                                    int n_cu, hipStream_t stream);
 hipError_t launch_accgemm(const float* A, const float* B, float* C, int M, int K, int N, hipStream_t stream);
 hipError_t run_lds_probe(int pattern, int waves_per_cu, int iters, int n_cu, float* ms_out, double* gathers_out,
                          hipStream_t stream);
@@ -296,6 +305,60 @@ int amr_lut_gemm_backward_ex(const float* gC, const uint8_t* A, const uint8_t* B
             int splits = 1;
             amr::gradB_workspace_bytes(M, K, N, n_cu, &splits);
             e = amr::launch_gradB(gC, A, B, gB, lut_grad_b, g, M, K, N, scale, partials, splits, s);
+        }
+        if (e != hipSuccess) return hip_fail(e, "gradB launch");
+    }
+    return AMR_OK;
+}
+
+int amr_lut_gemm_backward_f32tab(const float* gC, const uint8_t* A, const uint8_t* B, float* gA, float* gB,
+                                 const float* lut_grad_a, const float* lut_grad_b, int64_t lut_elems, float scale, int M, int K,
+                                 int N, int ga_rows_per_image, void* workspace, size_t workspace_bytes, void* stream) {
+    if (ga_rows_per_image < 0 || (ga_rows_per_image > 0 && M % ga_rows_per_image != 0))
+        return fail(AMR_EINVAL, "ga_rows_per_image=%d must divide M=%d", ga_rows_per_image, M);
+    if (M < 0 || K < 0 || N < 0) return fail(AMR_EINVAL, "negative dimension M=%d K=%d N=%d", M, K, N);
+    amr::LutGeom g;
+    if (!amr::lut_geom_from_elems(lut_elems, &g))
+        return fail(AMR_ELUTLEN, "lut size should be one of 1024/5120/17408/66306, got %lld", (long long)lut_elems);
+    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    if (gA && !lut_grad_a) return fail(AMR_EINVAL, "lut_grad_a is null");
+    if (gB && !lut_grad_b) return fail(AMR_EINVAL, "lut_grad_b is null");
+    if (((uintptr_t)lut_grad_a & 3) || ((uintptr_t)lut_grad_b & 3)) return fail(AMR_EINVAL, "gradient tables must be 4-byte aligned");
+    if (M == 0 || K == 0 || N == 0) {   // an empty sum is zero
+        hipError_t e = hipSuccess;
+        if (gA && (size_t)M * K) e = amr::launch_zero_u32(gA, (size_t)M * K, s);
+        if (e == hipSuccess && gB && (size_t)K * N) e = amr::launch_zero_u32(gB, (size_t)K * N, s);
+        return e == hipSuccess ? AMR_OK : hip_fail(e, "zero fill launch");
+    }
+    if (!gC || !A || !B) return fail(AMR_EINVAL, "null pointer argument");
+    if (!gA && !gB) return AMR_OK;
+    int dev = 0;
+    const int n_cu = current_device_cus(&dev);
+    if (n_cu <= 0) return fail(AMR_EINVAL, "no HIP device available");
+    hipError_t e;
+    const size_t partial_bytes = backward_partial_bytes(M, K, N, n_cu);
+    const size_t need = 256 + partial_bytes;
+    void* ws = workspace;
+    if (ws) {
+        if (workspace_bytes < need) return fail(AMR_EWORKSPACE, "workspace of %zu bytes is smaller than the %zu required", workspace_bytes, need);
+        if ((uintptr_t)ws & 255) return fail(AMR_EINVAL, "workspace must be 256-byte aligned");
+    } else {
+        ws = internal_workspace(dev, need, &e);
+        if (!ws) return hip_fail(e, "workspace hipMalloc");
+    }
+    uint32_t* flags = reinterpret_cast<uint32_t*>(ws);
+    float* partials = reinterpret_cast<float*>(reinterpret_cast<unsigned char*>(ws) + 256);
+    if (gA) {
+        e = amr::launch_gradA_f32tab(gC, A, B, gA, lut_grad_a, g, M, K, N, scale, n_cu, s, nullptr, ga_rows_per_image);
+        if (e != hipSuccess) return hip_fail(e, "gradA launch");
+    }
+    if (gB) {
+        if (g_expanded_kernels && amr::bwd_slab_applies(g, M, K, N)) {
+            e = amr::launch_gradB_slab_f32tab(gC, A, B, gB, lut_grad_b, g, M, K, N, scale, flags, partials, n_cu, s);
+        } else {
+            int splits = 1;
+            amr::gradB_workspace_bytes(M, K, N, n_cu, &splits);
+            e = amr::launch_gradB_f32tab(gC, A, B, gB, lut_grad_b, g, M, K, N, scale, partials, splits, s, nullptr);
         }
         if (e != hipSuccess) return hip_fail(e, "gradB launch");
     }

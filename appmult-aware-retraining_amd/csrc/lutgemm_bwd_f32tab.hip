@@ -1,0 +1,329 @@
+// Backward LUT-GEMM with float32 gradient tables, gfx950.
+//
+//   gA[m,k] = scale * sum_n gC[m,n] * Gx[A[m,k]][B[k,n]]     (lutgemm_gradA_f32tab_kernel)
+//   gB[k,n] = scale * sum_m Gy[A[m,k]][B[k,n]] * gC[m,n]     (lutgemm_gradB_f32tab_kernel)
+//
+// The same sums as ApproxGemmBackwardKernelForGA / ...ForGB (self_ops/src/approx_gemm_backward.cu:21-258 and
+// :269-492) with the table entries given as float32 (unrounded slopes) instead of int16 = round(16 x slope), and the
+// caller's scale in place of FACTOR (self_ops/src/approx_mult.h:41).  Tables keep the reference's padded geometry
+// (self_ops/src/approx_mult.h:12-40), four bytes per entry.
+//
+// Both kernels are the "uniform-row gather" of lutgemm_bwd.hip: one operand code is wave-uniform per gather and picks
+// the table row, the lanes' own codes pick the entry inside the row.  What is new is the size of the table: a 7-bit
+// float table (67 KB) fits the LDS of a workgroup, an 8-bit one (265 KB) does not fit the 160 KB of a CU.  It is
+// split along the uniform operand into `passes` bands of `rows_pp` rows (8 bit: 2 x 129 rows = 133 KB): the workgroup
+// stages band 0, walks its whole reduction taking only the gathers whose uniform code falls into the band (a scalar
+// branch: the skipped gathers cost no LDS access), stages band 1 and walks it again.  Every gather is done exactly
+// once; the accumulators stay in registers across the bands, the codes are read once per band.
+#include "amr_common.h"
+
+namespace amr {
+
+__global__ void reduce_partials_kernel(const float* __restrict__ partial, float* __restrict__ out, size_t count, int splits);
+
+// ------------------------------------------------------------------------------------------ gradB
+// Lanes own columns n, the uniform operand is a = A[m,k]; band p holds table rows a in [p*rows_pp, (p+1)*rows_pp).
+template <int KT, int WAVES, bool SPLIT>
+__global__ __launch_bounds__(WAVES * 64) void lutgemm_gradB_f32tab_kernel(
+    const float* __restrict__ gC, const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, float* __restrict__ out,
+    const float* __restrict__ lut, int n_rows, int cols, int rows_pp, int passes, int M, int K, int N, int m_chunk,
+    float scale, const uint32_t* __restrict__ gate) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    if (gate != nullptr && *gate == 0u) return;   // queued as a fallback that turned out not to be needed
+    const int wave = uniform(threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    const int k0 = (blockIdx.y * WAVES + wave) * KT;
+    const bool active = k0 < K;            // idle waves still take part in the barriers between bands
+    const int n = blockIdx.x * 64 + lane;
+    const int nc = min(n, N - 1);
+    const int mb = blockIdx.z * m_chunk;
+    const int me = min(M, mb + m_chunk);
+    const uint32_t row_bytes = (uint32_t)cols * 4u;
+
+    constexpr int DW = KT / 4;        // code dwords per row in this k tile
+    constexpr int RPL = 64 / DW;      // rows covered by one loader instruction
+    const int ldw = lane % DW;
+    const int lrow = lane / DW;
+
+    uint32_t boff[KT];
+#pragma unroll
+    for (int kk = 0; kk < KT; ++kk) boff[kk] = 4u * (uint32_t)B[(size_t)min(k0 + kk, K - 1) * N + nc];
+    float acc[KT];
+#pragma unroll
+    for (int kk = 0; kk < KT; ++kk) acc[kk] = 0.f;
+
+    for (int p = 0; p < passes; ++p) {
+        const int lo = p * rows_pp;
+        const uint32_t nr = (uint32_t)min(rows_pp, n_rows - lo);
+        if (p) __syncthreads();
+        {
+            float* s = reinterpret_cast<float*>(smem);
+            const float* src = lut + (size_t)lo * cols;
+            const int count = (int)nr * cols;
+            for (int i = threadIdx.x; i < count; i += WAVES * 64) s[i] = src[i];
+        }
+        __syncthreads();
+        if (!active) continue;
+        for (int m = mb; m < me; m += RPL) {
+            const int r = min(m + lrow, me - 1);
+            const uint32_t a4 = load_codes4_clamped(A + (size_t)r * K, k0 + 4 * ldw, K);
+            // rows of gC in groups of IU: all rows of the loader instruction at once for a whole table; four at a time
+            // for a band (the scalar state of the band tests of 16 unrolled rows does not fit the scalar registers)
+            constexpr int IU = SPLIT ? 4 : RPL;
+#pragma unroll 1
+            for (int i0 = 0; i0 < RPL; i0 += IU) {
+            float g[IU];
+#pragma unroll
+            for (int u = 0; u < IU; ++u) g[u] = (m + i0 + u < me) ? gC[(size_t)(m + i0 + u) * N + nc] : 0.f;
+#pragma unroll
+            for (int u = 0; u < IU; ++u) {
+                const int i = i0 + u;
+                float t[KT];
+                uint32_t in = 0;      // wave-uniform: bit kk = the code of k0+kk lies in this band
+#pragma unroll
+                for (int d = 0; d < DW; ++d) {
+                    const uint32_t aw = __builtin_amdgcn_readlane(a4, i * DW + d);
+#pragma unroll
+                    for (int kk = 0; kk < 4; ++kk) {
+                        const uint32_t rel = ((aw >> (8 * kk)) & 0xffu) - (uint32_t)lo;    // wave-uniform
+                        const bool here = !SPLIT || rel < nr;
+                        in |= (uint32_t)here << (4 * d + kk);
+                        t[4 * d + kk] = here ? *reinterpret_cast<const float*>(smem + rel * row_bytes + boff[4 * d + kk]) : 0.f;
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int kk = 0; kk < KT; ++kk)
+                    if (!SPLIT || ((in >> kk) & 1u)) acc[kk] = __builtin_fmaf(t[kk], g[u], acc[kk]);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            }
+        }
+    }
+    if (active && n < N) {
+        float* o = out + (size_t)blockIdx.z * K * N;
+#pragma unroll
+        for (int kk = 0; kk < KT; ++kk)
+            if (k0 + kk < K) o[(size_t)(k0 + kk) * N + n] = acc[kk] * scale;
+    }
+}
+
+// ------------------------------------------------------------------------------------------ gradA
+// Lanes own rows m, the uniform operand is b = B[k,n]; the table is transposed while it is staged, T[b - lo][a], so that
+// the uniform code again picks the row; band p holds b in [p*rows_pp, (p+1)*rows_pp).
+template <int KT, int RM, int WAVES, bool VEC, bool SPLIT>
+__global__ __launch_bounds__(WAVES * 64) void lutgemm_gradA_f32tab_kernel(
+    const float* __restrict__ gC, const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, float* __restrict__ gA,
+    const float* __restrict__ lut, int n_rows, int cols, int rows_pp, int passes, int M, int K, int N, float scale,
+    const uint32_t* __restrict__ gate, int rows_per_image, int vec_store) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    if (gate != nullptr && *gate == 0u) return;
+    const int wave = uniform(threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    const int k0 = blockIdx.x * KT;
+    const int m0 = (blockIdx.y * WAVES + wave) * (64 * RM);
+    const bool active = m0 < M;
+    const uint32_t trow_bytes = (uint32_t)cols * 4u;
+
+    int mr[RM];
+    uint32_t aoff[RM][KT];
+    float acc[RM][KT];
+#pragma unroll
+    for (int r = 0; r < RM; ++r) {
+        mr[r] = min(m0 + lane + 64 * r, M - 1);
+        const uint8_t* arow = A + (size_t)mr[r] * K;
+#pragma unroll
+        for (int d = 0; d < KT / 4; ++d) {
+            const uint32_t a4 = load_codes4_clamped(arow, k0 + 4 * d, K);
+#pragma unroll
+            for (int kk = 0; kk < 4; ++kk) {
+                aoff[r][4 * d + kk] = 4u * ((a4 >> (8 * kk)) & 0xffu);
+                acc[r][4 * d + kk] = 0.f;
+            }
+        }
+    }
+    // Loader lane kk (< KT) carries four B codes of row k0+kk; rows beyond K are clamped (never stored).
+    const uint8_t* brow = B + (size_t)min(k0 + (lane % KT), K - 1) * N;
+
+    for (int p = 0; p < passes; ++p) {
+        const int lo = p * rows_pp;
+        const uint32_t nr = (uint32_t)min(rows_pp, n_rows - lo);
+        if (p) __syncthreads();
+        {
+            // entry (a, b) of the row-major table goes to T[b - lo][a], T row stride = cols entries
+            float* t32 = reinterpret_cast<float*>(smem);
+            const int total = n_rows * (int)nr;
+            for (int i = threadIdx.x; i < total; i += WAVES * 64) {
+                const int a = i / (int)nr;
+                const int bb = i - a * (int)nr;
+                t32[bb * cols + a] = lut[(size_t)a * cols + lo + bb];
+            }
+        }
+        __syncthreads();
+        if (!active) continue;
+        for (int n = 0; n < N; n += 4) {
+            const uint32_t b4 = load_codes4_clamped(brow, n, N);
+            float g[RM][4];
+#pragma unroll
+            for (int r = 0; r < RM; ++r) {
+                if (VEC) {
+                    typedef float f32x4 __attribute__((ext_vector_type(4)));
+                    const f32x4 v = *reinterpret_cast<const f32x4*>(gC + (size_t)mr[r] * N + n);
+                    g[r][0] = v.x; g[r][1] = v.y; g[r][2] = v.z; g[r][3] = v.w;
+                } else {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) g[r][j] = (n + j < N) ? gC[(size_t)mr[r] * N + n + j] : 0.f;
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                float t[RM][KT];
+                uint32_t in = 0;      // wave-uniform: bit kk = the code of k0+kk lies in this band
+#pragma unroll
+                for (int kk = 0; kk < KT; ++kk) {
+                    const uint32_t bw = __builtin_amdgcn_readlane(b4, kk);
+                    const uint32_t rel = ((bw >> (8 * j)) & 0xffu) - (uint32_t)lo;    // wave-uniform
+                    const bool here = !SPLIT || rel < nr;
+                    in |= (uint32_t)here << kk;
+#pragma unroll
+                    for (int r = 0; r < RM; ++r)
+                        t[r][kk] = here ? *reinterpret_cast<const float*>(smem + rel * trow_bytes + aoff[r][kk]) : 0.f;
+                }
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int kk = 0; kk < KT; ++kk)
+                    if (!SPLIT || ((in >> kk) & 1u)) {
+#pragma unroll
+                        for (int r = 0; r < RM; ++r) acc[r][kk] = __builtin_fmaf(g[r][j], t[r][kk], acc[r][kk]);
+                    }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+    }
+    if (!active) return;
+#pragma unroll
+    for (int r = 0; r < RM; ++r) {
+        const int m = m0 + lane + 64 * r;
+        if (m < M && rows_per_image > 0) {
+            // image-major transposed output gA_T[m / L][k][m % L] (L = rows_per_image)
+            const int img = m / rows_per_image, l = m - img * rows_per_image;
+            float* o = gA + ((size_t)img * K + k0) * rows_per_image + l;
+#pragma unroll
+            for (int kk = 0; kk < KT; ++kk)
+                if (k0 + kk < K) o[(size_t)kk * rows_per_image] = acc[r][kk] * scale;
+        } else if (m < M) {
+            if (vec_store) {   // K % 4 == 0 and gA 16-byte aligned
+                typedef float f32x4 __attribute__((ext_vector_type(4)));
+#pragma unroll
+                for (int d = 0; d < KT / 4; ++d) {
+                    if (k0 + 4 * d < K) {
+                        f32x4 v = {acc[r][4 * d] * scale, acc[r][4 * d + 1] * scale, acc[r][4 * d + 2] * scale, acc[r][4 * d + 3] * scale};
+                        *reinterpret_cast<f32x4*>(gA + (size_t)m * K + k0 + 4 * d) = v;
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int kk = 0; kk < KT; ++kk)
+                    if (k0 + kk < K) gA[(size_t)m * K + k0 + kk] = acc[r][kk] * scale;
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------ host
+constexpr size_t kF32TabLdsCap = 140 * 1024;   // table band per workgroup (the 8-bit band of 129 rows needs 133 128 bytes)
+
+// Bands of the table along the uniform operand: all n_rows rows when they fit, else the fewest equal bands that do.
+static void f32tab_bands(const LutGeom& g, int* rows_pp, int* passes) {
+    const size_t row = (size_t)g.cols * 4;
+    int p = 1;
+    while ((size_t)((g.rows + p - 1) / p) * row > kF32TabLdsCap) ++p;
+    *passes = p;
+    *rows_pp = (g.rows + p - 1) / p;
+}
+
+template <typename Kern>
+static hipError_t allow_big_lds(Kern kern, bool* done) {
+    if (*done) return hipSuccess;
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    if (e == hipSuccess) *done = true;
+    return e;
+}
+
+hipError_t launch_gradB_f32tab(const float* gC, const uint8_t* A, const uint8_t* B, float* gB, const float* lut, const LutGeom& g,
+                               int M, int K, int N, float scale, void* workspace, int splits, hipStream_t stream,
+                               const uint32_t* gate) {
+    constexpr int KT = 16;
+    int rows_pp, passes;
+    f32tab_bands(g, &rows_pp, &passes);
+    const size_t lds = (size_t)rows_pp * g.cols * 4;
+    int m_chunk = (M + splits - 1) / splits;
+    m_chunk = (m_chunk + 15) & ~15;
+    const int zs = (M + m_chunk - 1) / m_chunk;
+    float* out = zs > 1 ? reinterpret_cast<float*>(workspace) : gB;
+    const int ktiles = (K + KT - 1) / KT;
+    hipError_t e;
+    if (passes > 1 || lds > 80 * 1024) {
+        // one 1024-thread workgroup per CU shares the staged band
+        static bool done = false;
+        auto kern = lutgemm_gradB_f32tab_kernel<KT, 16, true>;
+        if ((e = allow_big_lds(kern, &done)) != hipSuccess) return e;
+        hipLaunchKernelGGL(kern, dim3((N + 63) / 64, (ktiles + 15) / 16, zs), dim3(1024), lds, stream, gC, A, B, out, lut, g.rows,
+                           g.cols, rows_pp, passes, M, K, N, m_chunk, scale, gate);
+    } else {
+        static bool done = false;
+        auto kern = lutgemm_gradB_f32tab_kernel<KT, 4, false>;
+        if ((e = allow_big_lds(kern, &done)) != hipSuccess) return e;
+        hipLaunchKernelGGL(kern, dim3((N + 63) / 64, (ktiles + 3) / 4, zs), dim3(256), lds, stream, gC, A, B, out, lut, g.rows,
+                           g.cols, rows_pp, passes, M, K, N, m_chunk, scale, gate);
+    }
+    e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    if (zs > 1) {
+        const size_t count = (size_t)K * N;
+        hipLaunchKernelGGL(reduce_partials_kernel, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, stream,
+                           reinterpret_cast<const float*>(workspace), gB, count, zs);
+        e = hipGetLastError();
+    }
+    return e;
+}
+
+template <int KT, int RM, int WAVES, bool VEC, bool SPLIT>
+static hipError_t launch_gradA_f32tab_t(const float* gC, const uint8_t* A, const uint8_t* B, float* gA, const float* lut,
+                                        const LutGeom& g, int rows_pp, int passes, int M, int K, int N, float scale,
+                                        hipStream_t stream, const uint32_t* gate, int rows_per_image) {
+    const int vec_store = ((K & 3) == 0) && (((uintptr_t)gA & 15) == 0);
+    auto kern = lutgemm_gradA_f32tab_kernel<KT, RM, WAVES, VEC, SPLIT>;
+    static bool done = false;
+    hipError_t e = allow_big_lds(kern, &done);
+    if (e != hipSuccess) return e;
+    const int rows_per_wg = 64 * RM * WAVES;
+    dim3 grid((K + KT - 1) / KT, (M + rows_per_wg - 1) / rows_per_wg);
+    hipLaunchKernelGGL(kern, grid, dim3(WAVES * 64), (size_t)rows_pp * g.cols * 4, stream, gC, A, B, gA, lut, g.rows, g.cols, rows_pp,
+                       passes, M, K, N, scale, gate, rows_per_image, vec_store);
+    return hipGetLastError();
+}
+
+hipError_t launch_gradA_f32tab(const float* gC, const uint8_t* A, const uint8_t* B, float* gA, const float* lut, const LutGeom& g,
+                               int M, int K, int N, float scale, int n_cu, hipStream_t stream, const uint32_t* gate,
+                               int rows_per_image) {
+    constexpr int KT = 16;
+    int rows_pp, passes;
+    f32tab_bands(g, &rows_pp, &passes);
+    const bool vec = ((N & 3) == 0) && (((uintptr_t)gC & 15) == 0);   // rows of gC are read 16 bytes at a time
+    const int ktiles = (K + KT - 1) / KT;
+    if (passes > 1 || (size_t)rows_pp * g.cols * 4 > 80 * 1024) {
+        return vec ? launch_gradA_f32tab_t<KT, 1, 16, true, true>(gC, A, B, gA, lut, g, rows_pp, passes, M, K, N, scale, stream, gate, rows_per_image)
+                   : launch_gradA_f32tab_t<KT, 1, 16, false, true>(gC, A, B, gA, lut, g, rows_pp, passes, M, K, N, scale, stream, gate, rows_per_image);
+    }
+    // Two rows per lane amortise the scalar work per gather; one when that would leave CUs idle.
+    const long wg2 = (long)ktiles * ((M + 511) / 512);
+    if (wg2 >= 2L * n_cu) {
+        return vec ? launch_gradA_f32tab_t<KT, 2, 4, true, false>(gC, A, B, gA, lut, g, rows_pp, passes, M, K, N, scale, stream, gate, rows_per_image)
+                   : launch_gradA_f32tab_t<KT, 2, 4, false, false>(gC, A, B, gA, lut, g, rows_pp, passes, M, K, N, scale, stream, gate, rows_per_image);
+    }
+    return vec ? launch_gradA_f32tab_t<KT, 1, 4, true, false>(gC, A, B, gA, lut, g, rows_pp, passes, M, K, N, scale, stream, gate, rows_per_image)
+               : launch_gradA_f32tab_t<KT, 1, 4, false, false>(gC, A, B, gA, lut, g, rows_pp, passes, M, K, N, scale, stream, gate, rows_per_image);
+}
+
+}  // namespace amr

@@ -34,7 +34,9 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 // S[kk][a][c] for kk < KT, built by all 1024 threads straight from the table in global memory (it is
 // 33 KB and stays in the L2; the expansion is 2^b / M of the streaming work).
-__device__ __forceinline__ void build_bwd_slab(float* slab, const int16_t* __restrict__ G, int lut_cols, int n_codes,
+// (T: int16 entries of the reference's tables, or float32 entries)
+template <typename T>
+__device__ __forceinline__ void build_bwd_slab(float* slab, const T* __restrict__ G, int lut_cols, int n_codes,
                                                const uint8_t* __restrict__ B, int K, int N, int k0, int n0, int kt) {
     const int col = threadIdx.x & 63;
     const int a0 = threadIdx.x >> 6;
@@ -44,7 +46,7 @@ __device__ __forceinline__ void build_bwd_slab(float* slab, const int16_t* __res
         const bool live = (k0 + kk < K) && (n0 + col < N);
         const int b = live ? (int)B[(size_t)(k0 + kk) * N + n0 + col] : 0;
         float* s = slab + kk * (kBwdSlabBytes / 4);
-        int16_t e[kBwdSlabRows / 16];
+        T e[kBwdSlabRows / 16];
 #pragma unroll
         for (int i = 0; i < kBwdSlabRows / 16; ++i) e[i] = G[min(a0 + 16 * i, n_codes - 1) * lut_cols + b];
 #pragma unroll
@@ -61,10 +63,10 @@ __device__ __forceinline__ void build_bwd_slab(float* slab, const int16_t* __res
 // FAST: K % 4 == 0, N % 64 == 0, M % 128 == 0, gC 16-byte aligned and M*K, 4*M*N < 2^31, so every
 // operand load is an unconditional dword / 128-bit load at a 32-bit offset (no tail handling in the
 // streaming loop).
-template <bool FAST>
+template <bool FAST, typename T>
 __global__ __launch_bounds__(1024) void lutgemm_gradB_slab_kernel(
     const float* __restrict__ gC, const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, float* __restrict__ out,
-    const int16_t* __restrict__ G, int lut_cols, int n_codes, uint32_t* __restrict__ flags, int M, int K, int N,
+    const T* __restrict__ G, int lut_cols, int n_codes, uint32_t* __restrict__ flags, int M, int K, int N,
     int m_chunk, float scale, int vec_ok) {
     __shared__ __align__(16) unsigned char smem[kBwdKT * kBwdSlabBytes];
     float* slab = reinterpret_cast<float*>(smem);
@@ -540,10 +542,10 @@ hipError_t launch_gradB_slab(const float* gC, const uint8_t* A, const uint8_t* B
                            1 << g.bits, flags, M, K, N, m_chunk, scale, (int)grid.x, (int)grid.y, (int)grid.z);
     }
     else if (regular && (K & 3) == 0)
-        hipLaunchKernelGGL(lutgemm_gradB_slab_kernel<true>, grid, dim3(1024), 0, stream, gC, A, B, out, lut, g.cols, 1 << g.bits,
+        hipLaunchKernelGGL((lutgemm_gradB_slab_kernel<true, int16_t>), grid, dim3(1024), 0, stream, gC, A, B, out, lut, g.cols, 1 << g.bits,
                            flags, M, K, N, m_chunk, scale, vec_ok);
     else
-        hipLaunchKernelGGL(lutgemm_gradB_slab_kernel<false>, grid, dim3(1024), 0, stream, gC, A, B, out, lut, g.cols, 1 << g.bits,
+        hipLaunchKernelGGL((lutgemm_gradB_slab_kernel<false, int16_t>), grid, dim3(1024), 0, stream, gC, A, B, out, lut, g.cols, 1 << g.bits,
                            flags, M, K, N, m_chunk, scale, vec_ok);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
@@ -557,6 +559,47 @@ hipError_t launch_gradB_slab(const float* gC, const uint8_t* A, const uint8_t* B
     // 7-bit operands can hold the masked code 128, and any table can hold an entry a half cannot: the gated
     // direct kernel covers both (for narrower tables a code 2^b is an ordinary slab row of zeros)
     if (g.bits == 7 || half_slab) return launch_gradB_gated(gC, A, B, gB, lut, g, M, K, N, scale, flags + 1, stream);
+    return hipSuccess;
+}
+
+// The same for float32 tables: the fp32 slab holds the entries themselves, so the products and sums are the ones the
+// direct kernel forms (the half-precision slab cannot hold arbitrary float entries).  flags[1] is cleared here; the
+// direct float-table kernel queued behind is gated on it (7-bit operands holding the masked code 128).
+hipError_t launch_gradB_f32tab(const float* gC, const uint8_t* A, const uint8_t* B, float* gB, const float* lut, const LutGeom& g,
+                               int M, int K, int N, float scale, void* workspace, int splits, hipStream_t stream,
+                               const uint32_t* gate);
+hipError_t launch_zero_u32(void* p, size_t n_dwords, hipStream_t stream);
+
+hipError_t launch_gradB_slab_f32tab(const float* gC, const uint8_t* A, const uint8_t* B, float* gB, const float* lut,
+                                    const LutGeom& g, int M, int K, int N, float scale, uint32_t* flags, float* partials,
+                                    int n_cu, hipStream_t stream) {
+    hipError_t e = launch_zero_u32(flags, 64, stream);
+    if (e != hipSuccess) return e;
+    const int vec_ok = ((N & 3) == 0) && (((uintptr_t)gC & 15) == 0);
+    const bool small = (size_t)M * K < (1ull << 31) && (size_t)M * N * 4 < (1ull << 31);
+    const bool regular = vec_ok && small && (N & 63) == 0 && (M % kBwdRowsPerIter) == 0;
+    const int splits = gradB_slab_splits_kt(M, K, N, n_cu, kBwdKT);
+    int m_chunk = (M + splits - 1) / splits;
+    m_chunk = (m_chunk + 255) & ~255;
+    const int zs = (M + m_chunk - 1) / m_chunk;
+    float* out = zs > 1 ? partials : gB;
+    dim3 grid((N + 63) / 64, (K + kBwdKT - 1) / kBwdKT, zs);
+    if (regular && (K & 3) == 0)
+        hipLaunchKernelGGL((lutgemm_gradB_slab_kernel<true, float>), grid, dim3(1024), 0, stream, gC, A, B, out, lut, g.cols, 1 << g.bits,
+                           flags, M, K, N, m_chunk, scale, vec_ok);
+    else
+        hipLaunchKernelGGL((lutgemm_gradB_slab_kernel<false, float>), grid, dim3(1024), 0, stream, gC, A, B, out, lut, g.cols, 1 << g.bits,
+                           flags, M, K, N, m_chunk, scale, vec_ok);
+    e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    if (zs > 1) {
+        const size_t count = (size_t)K * N;
+        hipLaunchKernelGGL(reduce_partials_kernel, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, stream, partials, gB,
+                           count, zs);
+        e = hipGetLastError();
+        if (e != hipSuccess) return e;
+    }
+    if (g.bits == 7) return launch_gradB_f32tab(gC, A, B, gB, lut, g, M, K, N, scale, nullptr, 1, stream, flags + 1);
     return hipSuccess;
 }
 

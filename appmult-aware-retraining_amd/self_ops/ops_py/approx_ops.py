@@ -71,11 +71,16 @@ def read_lut_file(file_name, quantization_bit):
 
 
 def set_lookup_tables(device, appmult, grad_a, grad_b):
-    """Install padded tables given as arrays/tensors (uint16, int16, int16); one copy per table."""
+    """Install padded tables given as arrays/tensors (uint16, int16, int16); one copy per table.
+
+    Gradient tables of a floating dtype are installed as float32 and taken as the slopes themselves (no factor 1/16):
+    the backward pass then runs on the native float-table entry point."""
     global lut_appmult, lut_grad_a, lut_grad_b
     lut_appmult = torch.as_tensor(np.ascontiguousarray(appmult, np.uint16)).to(device)
-    lut_grad_a = torch.as_tensor(np.ascontiguousarray(grad_a, np.int16)).to(device)
-    lut_grad_b = torch.as_tensor(np.ascontiguousarray(grad_b, np.int16)).to(device)
+    as_float = np.issubdtype(np.asarray(grad_a).dtype, np.floating) and np.issubdtype(np.asarray(grad_b).dtype, np.floating)
+    gdt = np.float32 if as_float else np.int16
+    lut_grad_a = torch.as_tensor(np.ascontiguousarray(grad_a, gdt)).to(device)
+    lut_grad_b = torch.as_tensor(np.ascontiguousarray(grad_b, gdt)).to(device)
 
 
 def init_lookup_tables(device, file_name, quantization_bit):

@@ -54,6 +54,9 @@ def main():
     ap.add_argument("--layers", action="store_true", help="also print a per-layer table to stderr")
     ap.add_argument("--calib", action="store_true", help="also run three plain 256 MiB device copies (reference for scaling FETCH_SIZE/WRITE_SIZE counters)")
     ap.add_argument("--only", default="", help="comma-separated layer names: restrict the step to them (profiling aid; the JSON line then describes that subset)")
+    ap.add_argument("--grad-tables", choices=["i16", "f32"], default="i16",
+                    help="i16: the reference's int16 x16 gradient tables (the headline metric); f32: the unrounded float32 slopes "
+                         "through the float-table entry point")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures the one-GPU hot path only: every box of this build has one GPU; run with --gpus 1")
@@ -82,8 +85,12 @@ def main():
     T = O.synth_lut(7, 64, rng)
     Gx, Gy = O.gen_bp_lut(T, 8)
     lut = torch.from_numpy(O.pack_table(T, 7, np.uint16)).to(dev)
-    lga = torch.from_numpy(O.pack_table(Gx, 7, np.int16)).to(dev)
-    lgb = torch.from_numpy(O.pack_table(Gy, 7, np.int16)).to(dev)
+    f32_tables = args.grad_tables == "f32"
+    if f32_tables:
+        Gx, Gy = O.gen_bp_lut(T, 8, rounded=False)
+    gdt = np.float32 if f32_tables else np.int16
+    lga = torch.from_numpy(O.pack_table(Gx, 7, gdt)).to(dev)
+    lgb = torch.from_numpy(O.pack_table(Gy, 7, gdt)).to(dev)
     L = lut.numel()
 
     # operands, resident in HBM --------------------------------------------------------------------
@@ -108,9 +115,14 @@ def main():
 
     def bwd(name, M, K, N, want_a=True, want_b=True):
         b = bufs[name]
-        rc = lib.amr_lut_gemm_backward(b["gC"].data_ptr(), b["A"].data_ptr(), b["B"].data_ptr(),
-                                       b["gA"].data_ptr() if want_a else None, b["gB"].data_ptr() if want_b else None,
-                                       lga.data_ptr(), lgb.data_ptr(), L, M, K, N, ws.data_ptr(), ws.numel(), stream)
+        if f32_tables:
+            rc = lib.amr_lut_gemm_backward_f32tab(b["gC"].data_ptr(), b["A"].data_ptr(), b["B"].data_ptr(),
+                                                  b["gA"].data_ptr() if want_a else None, b["gB"].data_ptr() if want_b else None,
+                                                  lga.data_ptr(), lgb.data_ptr(), L, 1.0, M, K, N, 0, ws.data_ptr(), ws.numel(), stream)
+        else:
+            rc = lib.amr_lut_gemm_backward(b["gC"].data_ptr(), b["A"].data_ptr(), b["B"].data_ptr(),
+                                           b["gA"].data_ptr() if want_a else None, b["gB"].data_ptr() if want_b else None,
+                                           lga.data_ptr(), lgb.data_ptr(), L, M, K, N, ws.data_ptr(), ws.numel(), stream)
         assert rc == 0, lib.amr_last_error()
 
     def step():
@@ -215,7 +227,7 @@ def main():
         "dtype": "u8 codes; u16 table -> int32 sums (fwd); i16 table x f32 -> f32 sums (bwd)",
         "data": "synthetic",
         "config": {"workload": "resnet18_cifar_b256_7bit_lutgemm_fwd_bwd (BASELINE.json configs[2]: 20 conv + 1 fc GEMMs)" if full else "subset: " + args.only,
-                   "batch": BATCH, "lut_macs_per_step": macs_step, "codes": "uniform random", "grad_tables": "int16 x16 difference-based, half window 8"},
+                   "batch": BATCH, "lut_macs_per_step": macs_step, "codes": "uniform random", "grad_tables": ("float32 unrounded difference slopes, half window 8" if f32_tables else "int16 x16 difference-based, half window 8")},
         "images_per_s": BATCH * args.steps / dt,
         "frac_of_lds_gather_roofline": rate / LDS_GATHER_PEAK,
         "kernel_ms_per_step": {k: round(v, 4) for k, v in kernels.items()},

@@ -113,6 +113,23 @@ int amr_lut_gemm_backward_ex(const float *gC, const uint8_t *A, const uint8_t *B
                              void *stream);
 
 /*
+ * Backward with float32 gradient tables: the same two sums with lut_grad_a / lut_grad_b holding the slopes themselves
+ * (padded tables of lut_elems float32 entries, entry (a,b) at a * cols + b) and `scale` in place of the 1/16:
+ *   gA[m,k] = scale * sum_{n<N} gC[m,n] * lut_grad_a[A[m,k] * cols + B[k,n]]
+ *   gB[k,n] = scale * sum_{m<M} lut_grad_b[A[m,k] * cols + B[k,n]] * gC[m,n]
+ * The reference's entry point (approx_gemm_backward_gpu, self_ops/src/approx_gemm_backward.cu:506-624) takes int16
+ * tables only, rounded from float slopes by scripts/gen_bp_lut.py:172-183; this one takes the unrounded slopes
+ * (scale = 1) or any other float table.  A float table of int16 values with scale = 1/16 gives the results of
+ * amr_lut_gemm_backward up to fp32 summation order.  An 8-bit float table (265 KB) exceeds the LDS of a CU and is
+ * processed in two bands of rows.  Arguments otherwise as amr_lut_gemm_backward_ex; the workspace size is
+ * amr_lut_gemm_backward_workspace_bytes(M,K,N).
+ */
+int amr_lut_gemm_backward_f32tab(const float *gC, const uint8_t *A, const uint8_t *B, float *gA, float *gB,
+                                 const float *lut_grad_a, const float *lut_grad_b, int64_t lut_elems, float scale,
+                                 int M, int K, int N, int ga_rows_per_image, void *workspace, size_t workspace_bytes,
+                                 void *stream);
+
+/*
  * im2col of operand codes: x [B,C,H,W] float32 holding integer codes 0..255 -> A [B*oh*ow, C*kh*kw] uint8,
  * row (b,oy,ox), column c*kh*kw + i*kw + j, same stride / padding / dilation on both axes, padding
  * positions = code 0.  One pass instead of the reference's pad + unfold + transpose + reshape + cast

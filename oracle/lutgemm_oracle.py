@@ -108,9 +108,10 @@ def parse_lut_file(path: str, bits: int):
 # Gradient tables (scripts/gen_bp_lut.py:7-62 smoothing + central difference, :172-183 x16 rounding)
 # Pinned by: the shipped (forward section -> gradient sections) pairs inside every "+bp" file.
 # ----------------------------------------------------------------------------------------------
-def gen_bp_lut(fwd: np.ndarray, half_ws: int):
+def gen_bp_lut(fwd: np.ndarray, half_ws: int, rounded: bool = True):
     """Literal (loop-for-loop) restatement; float32 arithmetic exactly as NumPy does it there.
-    Returns (grad_a16, grad_b16) as int64 = round(16 * slope)."""
+    Returns (grad_a16, grad_b16) as int64 = round(16 * slope); with rounded=False the float32 slopes themselves
+    (the values the reference's script holds just before its x16 rounding, gen_bp_lut.py:172-183)."""
     lut = fwd.astype(np.float32)
     R, Cn = lut.shape
     smooth_a = np.zeros((R, Cn), np.float32)
@@ -137,6 +138,8 @@ def gen_bp_lut(fwd: np.ndarray, half_ws: int):
                 grad_b[a][b] = (smooth_b[a][b + 1] - smooth_b[a][b - 1]) / 2
             else:
                 grad_b[a][b] = (np.max(lut[a][0:Cn]) - np.min(lut[a][0:Cn])) / Cn
+    if not rounded:
+        return grad_a, grad_b
     ga16 = np.round(grad_a * np.float32(16.0)).astype(np.int64)
     gb16 = np.round(grad_b * np.float32(16.0)).astype(np.int64)
     return ga16, gb16

@@ -60,6 +60,49 @@ def test_gemm_op_forward_and_backward_against_oracle(ops, oracle, golden_dir):
     np.testing.assert_allclose(bt.grad.cpu().numpy().T, b64, rtol=0, atol=1e-5 * np.abs(b64).max())
 
 
+def test_gemm_and_conv_ops_with_float_gradient_tables(ops, oracle, golden_dir):
+    """Float32 gradient tables installed with set_lookup_tables: slopes themselves, no 1/16."""
+    self_ops, P = ops
+    print("gemm / conv op, float gradient tables", flush=True)
+    fwd, _, _ = oracle.parse_lut_file(os.path.join(golden_dir, "lut7_resub_63_bp8.txt.gz"), 7)
+    Gx, Gy = oracle.gen_bp_lut(fwd, 8, rounded=False)
+    saved = (P.lut_appmult, P.lut_grad_a, P.lut_grad_b)
+    try:
+        P.set_lookup_tables("cuda", oracle.pack_table(fwd, 7, np.uint16), oracle.pack_table(Gx, 7, np.float32),
+                            oracle.pack_table(Gy, 7, np.float32))
+        assert P.lut_grad_a.dtype == torch.float32 and P.lut_grad_b.dtype == torch.float32
+        rng = np.random.default_rng(3)
+        A = rng.integers(0, 128, (200, 72)).astype(np.uint8)
+        B = rng.integers(0, 128, (72, 48)).astype(np.uint8)
+        a = torch.tensor(A, dtype=torch.float32, device="cuda", requires_grad=True)
+        b = torch.tensor(B, dtype=torch.float32, device="cuda", requires_grad=True)
+        out = self_ops.approx_gemm_op(a, b)
+        g = torch.randn(200, 48, device="cuda")
+        out.backward(g)
+        a64, b64 = oracle.backward_np(g.cpu().numpy(), A, B, Gx, Gy, factor=1.0)
+        np.testing.assert_allclose(a.grad.cpu().numpy(), a64, rtol=0, atol=1e-5 * np.abs(a64).max())
+        np.testing.assert_allclose(b.grad.cpu().numpy(), b64, rtol=0, atol=1e-5 * np.abs(b64).max())
+        # the convolution on the same tables: its gradients are those of the GEMM of its im2col matrix
+        x = torch.tensor(rng.integers(0, 128, (2, 3, 9, 9)), dtype=torch.float32, device="cuda", requires_grad=True)
+        w = torch.tensor(rng.integers(0, 128, (5, 3, 3, 3)), dtype=torch.float32, device="cuda", requires_grad=True)
+        y = self_ops.approx_conv2d_op(x, w, None, (1, 1), (1, 1), (1, 1), 1)
+        gy = torch.randn_like(y)
+        y.backward(gy)
+        cols, oh, ow = oracle.im2col_np(x.detach().cpu().numpy().astype(np.uint8), 3, 3, 1, 1, 1)
+        Wm = w.detach().cpu().numpy().astype(np.uint8).reshape(5, -1).T.copy()
+        gm = gy.permute(0, 2, 3, 1).reshape(-1, 5).cpu().numpy()
+        ga64, gb64 = oracle.backward_np(gm, cols, Wm, Gx, Gy, factor=1.0)
+        np.testing.assert_allclose(w.grad.cpu().numpy().reshape(5, -1).T, gb64, rtol=0, atol=1e-5 * np.abs(gb64).max())
+        fold = F.fold(torch.tensor(ga64.reshape(2, oh * ow, -1).transpose(0, 2, 1).copy()), (9, 9), (3, 3), padding=1)
+        np.testing.assert_allclose(x.grad.cpu().numpy(), fold.numpy(), rtol=0, atol=1e-5 * float(fold.abs().max()))
+        import approx_ops
+        with pytest.raises(RuntimeError, match="grad_scale needs float32"):
+            approx_ops.approx_gemm_backward(g, a.detach().to(torch.uint8), b.detach().to(torch.uint8), torch.empty_like(a),
+                                            torch.empty_like(b), saved[1], saved[2], grad_scale=0.5)
+    finally:
+        P.lut_appmult, P.lut_grad_a, P.lut_grad_b = saved
+
+
 def test_baseline_op_uses_dense_ste_gradients(ops):
     self_ops, P = ops
     print("baseline op", flush=True)

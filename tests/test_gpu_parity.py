@@ -30,6 +30,7 @@ def lib():
     L.amr_lut_gemm_forward_workspace_bytes.argtypes = [i64, i, i, i]
     L.amr_lut_gemm_forward_workspace_bytes.restype = sz
     L.amr_lut_gemm_backward.argtypes = [vp, vp, vp, vp, vp, vp, vp, i64, i, i, i, vp, sz, vp]
+    L.amr_lut_gemm_backward_f32tab.argtypes = [vp, vp, vp, vp, vp, vp, vp, i64, ctypes.c_float, i, i, i, i, vp, sz, vp]
     L.amr_lut_gemm_backward_workspace_bytes.argtypes = [i, i, i]
     L.amr_lut_gemm_backward_workspace_bytes.restype = sz
     L.amr_acc_gemm_forward_fp32.argtypes = [vp, vp, vp, i, i, i, vp]
@@ -219,9 +220,9 @@ def test_forward_wraparound_and_k_zero(lib, oracle):
     assert (gpu_forward(lib, np.zeros((4, 0), np.uint8), np.zeros((0, 6), np.uint8), flat) == 0).all()
 
 
-def check_backward(oracle, got, g, A, B, la, lb, bits):
+def check_backward(oracle, got, g, A, B, la, lb, bits, factor=1.0 / 16):
     gA, gB = got
-    a64, b64, absA, absB = oracle.backward_c_f64(g, A, B, la, lb, bits, want_abs=True)
+    a64, b64, absA, absB = oracle.backward_c_f64(g, A, B, la, lb, bits, factor=factor, want_abs=True)
     assert np.isfinite(gA).all() and np.isfinite(gB).all()
     for x, r, ab in ((gA, a64, absA), (gB, b64, absB)):
         err = np.abs(x - r)
@@ -351,6 +352,113 @@ def test_backward_golden_shipped_tables(lib, oracle, golden_dir):
     g = rng.standard_normal((300, 70)).astype(np.float32)
     la, lb = oracle.pack_table(z["grad_a"], 8, np.int16), oracle.pack_table(z["grad_b"], 8, np.int16)
     check_backward(oracle, gpu_backward(lib, g, A, B, la, lb), g, A, B, la, lb, 8)
+
+
+# ------------------------------------------------------------------------------------------ float32 gradient tables
+def gpu_backward_f32tab(lib, g, A, B, la, lb, scale, own_workspace=True, rows_per_image=0):
+    M, K = A.shape
+    N = B.shape[1]
+    gd, a, b, ta, tb = dev(g), dev(A), dev(B), dev(np.asarray(la, np.float32)), dev(np.asarray(lb, np.float32))
+    ga = torch.full((M, K), float("nan"), device="cuda")
+    gb = torch.full((K, N), float("nan"), device="cuda")
+    need = lib.amr_lut_gemm_backward_workspace_bytes(M, K, N)
+    ws = torch.empty(max(need, 1), dtype=torch.uint8, device="cuda") if own_workspace else None
+    rc = lib.amr_lut_gemm_backward_f32tab(gd.data_ptr(), a.data_ptr(), b.data_ptr(), ga.data_ptr(), gb.data_ptr(), ta.data_ptr(),
+                                          tb.data_ptr(), ta.numel(), scale, M, K, N, rows_per_image,
+                                          ws.data_ptr() if ws is not None else None, need if ws is not None else 0, None)
+    assert rc == 0, lib.amr_last_error()
+    torch.cuda.synchronize()
+    return ga.cpu().numpy(), gb.cpu().numpy()
+
+
+# small and ragged shapes (direct kernels), K below one workgroup's share (idle waves at the band barriers), and
+# M >= 1024 (gradB on the fp32 expanded table for tables of at most 7 bits)
+F32TAB_SHAPES = [(1, 1, 1), (3, 5, 7), (9, 27, 10), (64, 64, 64), (33, 130, 65), (600, 96, 64), (257, 100, 129), (300, 288, 256),
+                 (70, 50, 513), (1100, 27, 64), (4096, 8, 64), (4100, 27, 10), (5000, 130, 65), (2048, 48, 128), (1500, 40, 70)]
+
+
+@pytest.mark.parametrize("bits", [7, 8, 6, 4])
+@pytest.mark.parametrize("shape", F32TAB_SHAPES)
+def test_backward_float_tables_within_tolerance(lib, oracle, bits, shape):
+    print("backward float tables", bits, shape, flush=True)
+    rng, A, B, _ = rand_case(hash((bits, shape, "f")) % 2**32, *shape, bits)
+    n = 1 << bits
+    la = oracle.pack_table(rng.standard_normal((n, n)) * 40 + 3, bits, np.float32)
+    lb = oracle.pack_table(rng.standard_normal((n, n)) * 40 - 5, bits, np.float32)
+    g = rng.standard_normal((shape[0], shape[2])).astype(np.float32)
+    scale = 0.37
+    check_backward(oracle, gpu_backward_f32tab(lib, g, A, B, la, lb, scale), g, A, B, la, lb, bits, factor=np.float32(scale))
+
+
+@pytest.mark.parametrize("bits", [7, 8])
+def test_backward_float_tables_masked_codes_and_both_bands(lib, oracle, bits):
+    print("backward float tables, masked codes", bits, flush=True)
+    n = 1 << bits
+    M, K, N = 4300, 40, 70
+    rng, A, B, _ = rand_case(500 + bits, M, K, N, bits)
+    la = oracle.pack_table(rng.standard_normal((n, n)) * 10, bits, np.float32)
+    lb = oracle.pack_table(rng.standard_normal((n, n)) * 10, bits, np.float32)
+    g = rng.standard_normal((M, N)).astype(np.float32)
+    if bits < 8:           # masked code 2^b: zero contribution (the pad row / column of the table); a uint8 cannot hold 256
+        A[::5, 7] = n
+        A[4000, :] = n
+        B[3, ::2] = n
+    else:                  # an 8-bit float table is staged in two bands of 129 rows: 128 is the last of the first band
+        A[::5, 7], A[4000, :], B[3, ::2] = 128, 129, 128
+        B[:, 5], B[:, 6] = 129, 128
+    A[17, :] = n - 1
+    A[18, :] = 0
+    check_backward(oracle, gpu_backward_f32tab(lib, g, A, B, la, lb, 1.0), g, A, B, la, lb, bits, factor=1.0)
+    check_backward(oracle, gpu_backward_f32tab(lib, g, A, B, la, lb, 1.0, own_workspace=False), g, A, B, la, lb, bits, factor=1.0)
+
+
+@pytest.mark.parametrize("bits", [7, 8])
+def test_backward_float_tables_ste_is_the_dense_product_and_int16_values_agree(lib, oracle, bits):
+    print("backward float tables, STE / int16 values", bits, flush=True)
+    n = 1 << bits
+    M, K, N = 1300, 72, 96
+    rng, A, B, _ = rand_case(600 + bits, M, K, N, bits)
+    # Gx[a][b] = b, Gy[a][b] = a, scale 1, small integer gC: every partial sum is exact -> the dense products, bit for bit
+    Sx = np.broadcast_to(np.arange(n, dtype=np.float32)[None, :], (n, n))
+    Sy = np.broadcast_to(np.arange(n, dtype=np.float32)[:, None], (n, n))
+    gi = rng.integers(-4, 5, (M, N)).astype(np.float32)
+    gA, gB = gpu_backward_f32tab(lib, gi, A, B, oracle.pack_table(Sx, bits, np.float32), oracle.pack_table(Sy, bits, np.float32), 1.0)
+    assert (gA == gi.astype(np.int64) @ B.astype(np.int64).T).all()
+    assert (gB == A.astype(np.int64).T @ gi.astype(np.int64)).all()
+    # a float table holding int16 values with scale 1/16 is the reference's backward pass
+    Ga, Gb = rng.integers(-32768, 32768, (n, n)), rng.integers(-32768, 32768, (n, n))
+    g = rng.standard_normal((M, N)).astype(np.float32)
+    la16, lb16 = oracle.pack_table(Ga, bits, np.int16), oracle.pack_table(Gb, bits, np.int16)
+    got = gpu_backward_f32tab(lib, g, A, B, la16.astype(np.float32), lb16.astype(np.float32), 1.0 / 16)
+    check_backward(oracle, got, g, A, B, la16, lb16, bits)
+    ref = gpu_backward(lib, g, A, B, la16, lb16)
+    for x, r in zip(got, ref):
+        assert np.max(np.abs(x - r)) <= 2e-5 * np.max(np.abs(r))
+
+
+def test_backward_float_tables_unrounded_difference_slopes_and_image_major_layout(lib, oracle):
+    """The GEMM of BASELINE configs[1] with the float32 difference slopes (half window 8) before their x16 rounding."""
+    print("backward float tables, config2 slopes", flush=True)
+    A, B, T, g = oracle.synth_gemm(4096, 576, 64, bits=7, err=64, seed=0)
+    Gx, Gy = oracle.gen_bp_lut(T, 8, rounded=False)
+    assert Gx.dtype == np.float32 and not (Gx * 16 == np.round(Gx * 16)).all()      # really unrounded
+    la, lb = oracle.pack_table(Gx, 7, np.float32), oracle.pack_table(Gy, 7, np.float32)
+    gA, gB = gpu_backward_f32tab(lib, g, A, B, la, lb, 1.0)
+    check_backward(oracle, (gA, gB), g, A, B, la, lb, 7, factor=1.0)
+    # image-major gA (the layout col2im takes): [M/L][K][L]
+    L = 1024
+    M, K = A.shape
+    gd, a, b, ta, tb = dev(g), dev(A), dev(B), dev(la), dev(lb)
+    gat = torch.full((M // L, K, L), float("nan"), device="cuda")
+    assert lib.amr_lut_gemm_backward_f32tab(gd.data_ptr(), a.data_ptr(), b.data_ptr(), gat.data_ptr(), None, ta.data_ptr(), tb.data_ptr(),
+                                            ta.numel(), 1.0, M, K, 64, L, None, 0, None) == 0
+    torch.cuda.synchronize()
+    assert (gat.cpu().numpy().transpose(0, 2, 1).reshape(M, K) == gA).all()
+    # argument checks
+    assert lib.amr_lut_gemm_backward_f32tab(gd.data_ptr(), a.data_ptr(), b.data_ptr(), gat.data_ptr(), None, ta.data_ptr(), tb.data_ptr(),
+                                            ta.numel() - 1, 1.0, M, K, 64, L, None, 0, None) != 0
+    assert lib.amr_lut_gemm_backward_f32tab(gd.data_ptr(), a.data_ptr(), b.data_ptr(), gat.data_ptr(), None, ta.data_ptr(), tb.data_ptr(),
+                                            ta.numel(), 1.0, M, K, 64, 1000, None, 0, None) != 0
 
 
 def test_backward_deterministic_and_skippable_outputs(lib, oracle):
