@@ -12,9 +12,12 @@
 // the table row, the lanes' own codes pick the entry inside the row.  What is new is the size of the table: a 7-bit
 // float table (67 KB) fits the LDS of a workgroup, an 8-bit one (265 KB) does not fit the 160 KB of a CU.  It is
 // split along the uniform operand into `passes` bands of `rows_pp` rows (8 bit: 2 x 129 rows = 133 KB): the workgroup
-// stages band 0, walks its whole reduction taking only the gathers whose uniform code falls into the band (a scalar
-// branch: the skipped gathers cost no LDS access), stages band 1 and walks it again.  Every gather is done exactly
-// once; the accumulators stay in registers across the bands, the codes are read once per band.
+// stages band 0, walks its whole reduction, stages band 1 and walks it again; the accumulators stay in registers
+// across the bands, the codes are read once per band.  A gather whose uniform code lies outside the staged band is
+// not skipped by a branch (every conditional read would have to be waited for where its branch ends, one LDS latency
+// per gather, and the band tests are a dozen scalar instructions per gather): its row index is clamped to a row of
+// zeros staged behind the band (one s_min_u32), so that it adds 0 x gC -- the reads of a row stay in flight together.
+// (For a non-finite gC value that product is NaN where the reference, which has the whole table, adds nothing.)
 #include "amr_common.h"
 
 namespace amr {
@@ -61,42 +64,34 @@ __global__ __launch_bounds__(WAVES * 64) void lutgemm_gradB_f32tab_kernel(
             const float* src = lut + (size_t)lo * cols;
             const int count = (int)nr * cols;
             for (int i = threadIdx.x; i < count; i += WAVES * 64) s[i] = src[i];
+            if (SPLIT)
+                for (int i = threadIdx.x; i < cols; i += WAVES * 64) s[count + i] = 0.f;      // the row of zeros behind the band
         }
         __syncthreads();
         if (!active) continue;
         for (int m = mb; m < me; m += RPL) {
             const int r = min(m + lrow, me - 1);
             const uint32_t a4 = load_codes4_clamped(A + (size_t)r * K, k0 + 4 * ldw, K);
-            // rows of gC in groups of IU: all rows of the loader instruction at once for a whole table; four at a time
-            // for a band (the scalar state of the band tests of 16 unrolled rows does not fit the scalar registers)
-            constexpr int IU = SPLIT ? 4 : RPL;
-#pragma unroll 1
-            for (int i0 = 0; i0 < RPL; i0 += IU) {
-            float g[IU];
+            float g[RPL];
 #pragma unroll
-            for (int u = 0; u < IU; ++u) g[u] = (m + i0 + u < me) ? gC[(size_t)(m + i0 + u) * N + nc] : 0.f;
+            for (int i = 0; i < RPL; ++i) g[i] = (m + i < me) ? gC[(size_t)(m + i) * N + nc] : 0.f;
 #pragma unroll
-            for (int u = 0; u < IU; ++u) {
-                const int i = i0 + u;
+            for (int i = 0; i < RPL; ++i) {
                 float t[KT];
-                uint32_t in = 0;      // wave-uniform: bit kk = the code of k0+kk lies in this band
 #pragma unroll
                 for (int d = 0; d < DW; ++d) {
                     const uint32_t aw = __builtin_amdgcn_readlane(a4, i * DW + d);
 #pragma unroll
                     for (int kk = 0; kk < 4; ++kk) {
-                        const uint32_t rel = ((aw >> (8 * kk)) & 0xffu) - (uint32_t)lo;    // wave-uniform
-                        const bool here = !SPLIT || rel < nr;
-                        in |= (uint32_t)here << (4 * d + kk);
-                        t[4 * d + kk] = here ? *reinterpret_cast<const float*>(smem + rel * row_bytes + boff[4 * d + kk]) : 0.f;
+                        uint32_t rel = ((aw >> (8 * kk)) & 0xffu) - (uint32_t)lo;    // wave-uniform; below the band: wraps to a huge value
+                        if (SPLIT) rel = min(rel, nr);                                // outside the band: the row of zeros
+                        t[4 * d + kk] = *reinterpret_cast<const float*>(smem + rel * row_bytes + boff[4 * d + kk]);
                     }
                 }
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                for (int kk = 0; kk < KT; ++kk)
-                    if (!SPLIT || ((in >> kk) & 1u)) acc[kk] = __builtin_fmaf(t[kk], g[u], acc[kk]);
+                for (int kk = 0; kk < KT; ++kk) acc[kk] = __builtin_fmaf(t[kk], g[i], acc[kk]);
                 __builtin_amdgcn_sched_barrier(0);
-            }
             }
         }
     }
@@ -158,6 +153,8 @@ __global__ __launch_bounds__(WAVES * 64) void lutgemm_gradA_f32tab_kernel(
                 const int bb = i - a * (int)nr;
                 t32[bb * cols + a] = lut[(size_t)a * cols + lo + bb];
             }
+            if (SPLIT)
+                for (int i = threadIdx.x; i < cols; i += WAVES * 64) t32[(int)nr * cols + i] = 0.f;      // the row of zeros behind the band
         }
         __syncthreads();
         if (!active) continue;
@@ -178,24 +175,19 @@ __global__ __launch_bounds__(WAVES * 64) void lutgemm_gradA_f32tab_kernel(
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 float t[RM][KT];
-                uint32_t in = 0;      // wave-uniform: bit kk = the code of k0+kk lies in this band
 #pragma unroll
                 for (int kk = 0; kk < KT; ++kk) {
                     const uint32_t bw = __builtin_amdgcn_readlane(b4, kk);
-                    const uint32_t rel = ((bw >> (8 * j)) & 0xffu) - (uint32_t)lo;    // wave-uniform
-                    const bool here = !SPLIT || rel < nr;
-                    in |= (uint32_t)here << kk;
+                    uint32_t rel = ((bw >> (8 * j)) & 0xffu) - (uint32_t)lo;    // wave-uniform; below the band: wraps to a huge value
+                    if (SPLIT) rel = min(rel, nr);                               // outside the band: the row of zeros
 #pragma unroll
-                    for (int r = 0; r < RM; ++r)
-                        t[r][kk] = here ? *reinterpret_cast<const float*>(smem + rel * trow_bytes + aoff[r][kk]) : 0.f;
+                    for (int r = 0; r < RM; ++r) t[r][kk] = *reinterpret_cast<const float*>(smem + rel * trow_bytes + aoff[r][kk]);
                 }
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int kk = 0; kk < KT; ++kk)
-                    if (!SPLIT || ((in >> kk) & 1u)) {
 #pragma unroll
-                        for (int r = 0; r < RM; ++r) acc[r][kk] = __builtin_fmaf(g[r][j], t[r][kk], acc[r][kk]);
-                    }
+                    for (int r = 0; r < RM; ++r) acc[r][kk] = __builtin_fmaf(g[r][j], t[r][kk], acc[r][kk]);
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
@@ -256,7 +248,7 @@ hipError_t launch_gradB_f32tab(const float* gC, const uint8_t* A, const uint8_t*
     constexpr int KT = 16;
     int rows_pp, passes;
     f32tab_bands(g, &rows_pp, &passes);
-    const size_t lds = (size_t)rows_pp * g.cols * 4;
+    const size_t lds = (size_t)(rows_pp + 1) * g.cols * 4;      // + the row of zeros
     int m_chunk = (M + splits - 1) / splits;
     m_chunk = (m_chunk + 15) & ~15;
     const int zs = (M + m_chunk - 1) / m_chunk;
@@ -299,7 +291,7 @@ static hipError_t launch_gradA_f32tab_t(const float* gC, const uint8_t* A, const
     if (e != hipSuccess) return e;
     const int rows_per_wg = 64 * RM * WAVES;
     dim3 grid((K + KT - 1) / KT, (M + rows_per_wg - 1) / rows_per_wg);
-    hipLaunchKernelGGL(kern, grid, dim3(WAVES * 64), (size_t)rows_pp * g.cols * 4, stream, gC, A, B, gA, lut, g.rows, g.cols, rows_pp,
+    hipLaunchKernelGGL(kern, grid, dim3(WAVES * 64), (size_t)(rows_pp + 1) * g.cols * 4, stream, gC, A, B, gA, lut, g.rows, g.cols, rows_pp,
                        passes, M, K, N, scale, gate, rows_per_image, vec_store);
     return hipGetLastError();
 }
@@ -313,6 +305,10 @@ hipError_t launch_gradA_f32tab(const float* gC, const uint8_t* A, const uint8_t*
     const bool vec = ((N & 3) == 0) && (((uintptr_t)gC & 15) == 0);   // rows of gC are read 16 bytes at a time
     const int ktiles = (K + KT - 1) / KT;
     if (passes > 1 || (size_t)rows_pp * g.cols * 4 > 80 * 1024) {
+        // one 1024-thread workgroup per CU shares the staged band; two rows per lane when that still fills the CUs
+        if ((long)ktiles * ((M + 2047) / 2048) >= n_cu)
+            return vec ? launch_gradA_f32tab_t<KT, 2, 16, true, true>(gC, A, B, gA, lut, g, rows_pp, passes, M, K, N, scale, stream, gate, rows_per_image)
+                       : launch_gradA_f32tab_t<KT, 2, 16, false, true>(gC, A, B, gA, lut, g, rows_pp, passes, M, K, N, scale, stream, gate, rows_per_image);
         return vec ? launch_gradA_f32tab_t<KT, 1, 16, true, true>(gC, A, B, gA, lut, g, rows_pp, passes, M, K, N, scale, stream, gate, rows_per_image)
                    : launch_gradA_f32tab_t<KT, 1, 16, false, true>(gC, A, B, gA, lut, g, rows_pp, passes, M, K, N, scale, stream, gate, rows_per_image);
     }

@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the LUT-GEMM hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--layers]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--layers] [--grad-tables f32] [--workload vgg16_b128_8bit]
 
 One "step" = forward + backward (gradA and gradB) LUT-GEMM of every conv layer and the fc layer of a
 CIFAR-style ResNet-18 at batch 256, 7-bit tables (BASELINE.json configs[2]: 21 GEMMs,
@@ -37,6 +37,12 @@ RESNET18_B256 = [
     ("fc", 1, 256, 512, 10),
 ]
 BATCH = 256
+# VGG-16 conv stack on 32x32 inputs + fc at batch 128 (BASELINE.json configs[3], 8-bit tables): 120 269 438 976 LUT-MACs
+VGG16_B128 = [
+    ("conv1_1", 1, 131072, 27, 64), ("conv1_2", 1, 131072, 576, 64), ("conv2_1", 1, 32768, 576, 128), ("conv2_2", 1, 32768, 1152, 128),
+    ("conv3_1", 1, 8192, 1152, 256), ("conv3_x", 2, 8192, 2304, 256), ("conv4_1", 1, 2048, 2304, 512), ("conv4_x", 2, 2048, 4608, 512),
+    ("conv5_x", 3, 512, 4608, 512), ("fc", 1, 128, 512, 10),
+]
 LDS_GATHER_PEAK = 256 * 2.4e9 * 32      # gathers/s: CUs x peak clock x conflict-free lanes per clock
 HBM_PEAK = 8.0e12
 
@@ -57,6 +63,9 @@ def main():
     ap.add_argument("--grad-tables", choices=["i16", "f32"], default="i16",
                     help="i16: the reference's int16 x16 gradient tables (the headline metric); f32: the unrounded float32 slopes "
                          "through the float-table entry point")
+    ap.add_argument("--workload", choices=["resnet18_b256_7bit", "vgg16_b128_8bit"], default="resnet18_b256_7bit",
+                    help="resnet18_b256_7bit: the headline configuration; vgg16_b128_8bit: the 8-bit stress configuration "
+                         "(forward error +-256, half window 16)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures the one-GPU hot path only: every box of this build has one GPU; run with --gpus 1")
@@ -64,7 +73,12 @@ def main():
     import numpy as np
     import torch
 
-    global RESNET18_B256
+    global RESNET18_B256, BATCH
+    headline = args.workload == "resnet18_b256_7bit"
+    BITS, ERR, HALF_WS = (7, 64, 8) if headline else (8, 256, 16)
+    NCODE = 1 << BITS
+    if not headline:
+        RESNET18_B256, BATCH = VGG16_B128, 128      # the layer list of the step
     full = not args.only
     if args.only:
         keep = set(args.only.split(","))
@@ -82,15 +96,15 @@ def main():
 
     # tables (config 1 recipe) -------------------------------------------------------------------
     rng = np.random.default_rng(0)
-    T = O.synth_lut(7, 64, rng)
-    Gx, Gy = O.gen_bp_lut(T, 8)
-    lut = torch.from_numpy(O.pack_table(T, 7, np.uint16)).to(dev)
+    T = O.synth_lut(BITS, ERR, rng)
+    Gx, Gy = O.gen_bp_lut(T, HALF_WS)
+    lut = torch.from_numpy(O.pack_table(T, BITS, np.uint16)).to(dev)
     f32_tables = args.grad_tables == "f32"
     if f32_tables:
-        Gx, Gy = O.gen_bp_lut(T, 8, rounded=False)
+        Gx, Gy = O.gen_bp_lut(T, HALF_WS, rounded=False)
     gdt = np.float32 if f32_tables else np.int16
-    lga = torch.from_numpy(O.pack_table(Gx, 7, gdt)).to(dev)
-    lgb = torch.from_numpy(O.pack_table(Gy, 7, gdt)).to(dev)
+    lga = torch.from_numpy(O.pack_table(Gx, BITS, gdt)).to(dev)
+    lgb = torch.from_numpy(O.pack_table(Gy, BITS, gdt)).to(dev)
     L = lut.numel()
 
     # operands, resident in HBM --------------------------------------------------------------------
@@ -99,8 +113,8 @@ def main():
     ws_need = 0
     for name, cnt, M, K, N in RESNET18_B256:
         bufs[name] = dict(
-            A=torch.randint(0, 128, (M, K), dtype=torch.uint8, device=dev, generator=gen),
-            B=torch.randint(0, 128, (K, N), dtype=torch.uint8, device=dev, generator=gen),
+            A=torch.randint(0, NCODE, (M, K), dtype=torch.uint8, device=dev, generator=gen),
+            B=torch.randint(0, NCODE, (K, N), dtype=torch.uint8, device=dev, generator=gen),
             C=torch.empty((M, N), dtype=torch.int32, device=dev),
             gC=torch.randn((M, N), dtype=torch.float32, device=dev, generator=gen),
             gA=torch.empty((M, K), dtype=torch.float32, device=dev),
@@ -134,16 +148,16 @@ def main():
                 bwd(name, M, K, N)
 
     macs_fwd = sum(c * M * K * N for _, c, M, K, N in RESNET18_B256)
-    assert macs_fwd == 142188216320 or not full
+    assert macs_fwd == (142188216320 if headline else 40089812992) or not full
     macs_step = 3 * macs_fwd
 
     # quick parity guard on a row sample of one layer (the full parity suite is tests/ -m gpu) ---------
-    gname, _, gM, gK, gN = RESNET18_B256[-1] if not full else RESNET18_B256[4]
+    gname, _, gM, gK, gN = RESNET18_B256[-1] if not full else RESNET18_B256[4 if headline else 2]
     fwd(gname, gM, gK, gN)
     torch.cuda.synchronize()
     b = bufs[gname]
     rows = slice(100, 164)
-    want = O.forward_c(b["A"][rows].cpu().numpy(), b["B"].cpu().numpy(), lut.cpu().numpy(), 7)
+    want = O.forward_c(b["A"][rows].cpu().numpy(), b["B"].cpu().numpy(), lut.cpu().numpy(), BITS)
     assert (b["C"][rows].cpu().numpy().view(np.uint32) == want).all(), "forward parity guard failed"
 
     if args.calib:
@@ -212,8 +226,8 @@ def main():
 
     # single-GEMM configuration (BASELINE configs[1]: M=4096, K=576, N=64 forward+backward) ---------------
     M1, K1, N1 = 4096, 576, 64
-    bufs["single"] = dict(A=torch.randint(0, 128, (M1, K1), dtype=torch.uint8, device=dev, generator=gen),
-                          B=torch.randint(0, 128, (K1, N1), dtype=torch.uint8, device=dev, generator=gen),
+    bufs["single"] = dict(A=torch.randint(0, NCODE, (M1, K1), dtype=torch.uint8, device=dev, generator=gen),
+                          B=torch.randint(0, NCODE, (K1, N1), dtype=torch.uint8, device=dev, generator=gen),
                           C=torch.empty((M1, N1), dtype=torch.int32, device=dev),
                           gC=torch.randn((M1, N1), dtype=torch.float32, device=dev, generator=gen),
                           gA=torch.empty((M1, K1), dtype=torch.float32, device=dev),
@@ -221,13 +235,15 @@ def main():
     t_single = timed(lambda: (fwd("single", M1, K1, N1), bwd("single", M1, K1, N1)), reps=50)
 
     out = {
-        "metric": "LUT-MAC/s fwd+bwd (ResNet-18 conv shapes, 7-bit)",
+        "metric": "LUT-MAC/s fwd+bwd (ResNet-18 conv shapes, 7-bit)" if headline else "LUT-MAC/s fwd+bwd (VGG-16 conv shapes, 8-bit)",
         "value": rate, "unit": "LUT-MAC/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "u8 codes; u16 table -> int32 sums (fwd); i16 table x f32 -> f32 sums (bwd)",
         "data": "synthetic",
-        "config": {"workload": "resnet18_cifar_b256_7bit_lutgemm_fwd_bwd (BASELINE.json configs[2]: 20 conv + 1 fc GEMMs)" if full else "subset: " + args.only,
-                   "batch": BATCH, "lut_macs_per_step": macs_step, "codes": "uniform random", "grad_tables": ("float32 unrounded difference slopes, half window 8" if f32_tables else "int16 x16 difference-based, half window 8")},
+        "config": {"workload": ("subset: " + args.only) if not full else
+                   "resnet18_cifar_b256_7bit_lutgemm_fwd_bwd (BASELINE.json configs[2]: 20 conv + 1 fc GEMMs)" if headline else
+                   "vgg16_cifar_b128_8bit_lutgemm_fwd_bwd (BASELINE.json configs[3]: 13 conv + 1 fc GEMMs)",
+                   "batch": BATCH, "lut_macs_per_step": macs_step, "codes": "uniform random", "grad_tables": (f"float32 unrounded difference slopes, half window {HALF_WS}" if f32_tables else f"int16 x16 difference-based, half window {HALF_WS}")},
         "images_per_s": BATCH * args.steps / dt,
         "frac_of_lds_gather_roofline": rate / LDS_GATHER_PEAK,
         "kernel_ms_per_step": {k: round(v, 4) for k, v in kernels.items()},
@@ -235,26 +251,28 @@ def main():
                      "unit": "Ggather/s", "frac": dom_rate / LDS_GATHER_PEAK,
                      # bytes the L2s fetched + wrote for the conv2_x launch of that kernel kind (rocprofv3 FETCH_SIZE x 2.00,
                      # WRITE_SIZE x 1.00 against plain copies; profiles/conv2x_hbm_traffic.md), beside its algorithmic bytes
-                     "traffic": MEASURED_TRAFFIC_CONV2X[dominant],
+                     # (measured for the headline workload's kernels only)
+                     "traffic": MEASURED_TRAFFIC_CONV2X[dominant] if headline and not f32_tables else None,
                      "traffic_launch": "conv2_x (M=262144,K=576,N=64)", "traffic_algorithmic": hbm_bytes(dominant, 262144, 576, 64),
                      "avg_launch_ms": dom_ms / launches,
                      "hbm": {"achieved": dom_bytes / (dom_ms * 1e-3) / 1e9, "peak": HBM_PEAK / 1e9, "unit": "GB/s",
                              "frac": dom_bytes / (dom_ms * 1e-3) / HBM_PEAK},
                      "lds_probe_gathers_per_s": {"conflict_free": probe_free, "uniform_row_256B": probe_row}},
-        "single_gemm": {"workload": "M=4096 K=576 N=64 fwd+bwd (BASELINE.json configs[1])", "us": t_single * 1e3,
+        "single_gemm": {"workload": f"M=4096 K=576 N=64 fwd+bwd, {BITS}-bit (BASELINE.json configs[1] shape)", "us": t_single * 1e3,
                         "lut_mac_per_s": 3 * M1 * K1 * N1 / (t_single * 1e-3),
                         "frac_of_lds_gather_roofline": 3 * M1 * K1 * N1 / (t_single * 1e-3) / LDS_GATHER_PEAK},
     }
 
     # CPU baseline: the C oracle (port of the reference formulation) on the host cores ----------------------
     if not args.no_cpu:
-        A, B, Tc, g = O.synth_gemm(M1, K1, N1, bits=7, err=64, seed=0)
-        f16, a16, b16 = O.pack_table(Tc, 7, np.uint16), O.pack_table(Gx, 7, np.int16), O.pack_table(Gy, 7, np.int16)
-        O.forward_c(A, B, f16, 7)
+        A, B, Tc, g = O.synth_gemm(M1, K1, N1, bits=BITS, err=ERR, seed=0)
+        Gx16, Gy16 = O.gen_bp_lut(Tc, HALF_WS)
+        f16, a16, b16 = O.pack_table(Tc, BITS, np.uint16), O.pack_table(Gx16, BITS, np.int16), O.pack_table(Gy16, BITS, np.int16)
+        O.forward_c(A, B, f16, BITS)
         reps, t0 = 0, time.perf_counter()
         while time.perf_counter() - t0 < 10.0:
-            O.forward_c(A, B, f16, 7)
-            O.backward_c_f32(g, A, B, a16, b16, 7)
+            O.forward_c(A, B, f16, BITS)
+            O.backward_c_f32(g, A, B, a16, b16, BITS)
             reps += 1
         el = time.perf_counter() - t0
         out["cpu_baseline"] = {"value": reps * 3 * M1 * K1 * N1 / el, "unit": "LUT-MAC/s", "cores": O.c_lib().oracle_num_threads(),
