@@ -30,10 +30,7 @@ __global__ __launch_bounds__(WAVES * 64) void lutgemm_gradB_kernel(
     int m_chunk, float scale, const uint32_t* __restrict__ gate) {
     extern __shared__ __align__(16) unsigned char smem[];
     if (gate != nullptr && *gate == 0u) return;   // queued as a fallback that turned out not to be needed
-    {
-        uint32_t* s32 = reinterpret_cast<uint32_t*>(smem);
-        for (int i = threadIdx.x; i < lut_dwords; i += WAVES * 64) s32[i] = lut32[i];
-    }
+    stage_table_dwords<WAVES * 64>(smem, lut32, lut_dwords);
     __syncthreads();
 
     const int wave = uniform(threadIdx.x >> 6);
@@ -59,12 +56,18 @@ __global__ __launch_bounds__(WAVES * 64) void lutgemm_gradB_kernel(
 #pragma unroll
     for (int kk = 0; kk < KT; ++kk) acc[kk] = 0.f;
 
-    for (int m = mb; m < me; m += RPL) {
+    // The codes and gC values of the next RPL rows are loaded while the current ones are consumed (two register sets
+    // alternate); without that every trip of a wave pays the memory latency before its first gather.
+    auto load_rows = [&](int m, uint32_t& a4, float (&g)[RPL]) __attribute__((always_inline)) {
         const int r = min(m + lrow, me - 1);
-        const uint32_t a4 = load_codes4_clamped(A + (size_t)r * K, k0 + 4 * ldw, K);
-        float g[RPL];
+        a4 = load_codes4_clamped(A + (size_t)r * K, k0 + 4 * ldw, K);
 #pragma unroll
-        for (int i = 0; i < RPL; ++i) g[i] = (m + i < me) ? gC[(size_t)(m + i) * N + nc] : 0.f;
+        for (int i = 0; i < RPL; ++i) {
+            const float v = gC[(size_t)min(m + i, me - 1) * N + nc];
+            g[i] = (m + i < me) ? v : 0.f;
+        }
+    };
+    auto consume_rows = [&](uint32_t a4, const float (&g)[RPL]) __attribute__((always_inline)) {
 #pragma unroll
         for (int i = 0; i < RPL; ++i) {
             float t[KT];
@@ -81,6 +84,21 @@ __global__ __launch_bounds__(WAVES * 64) void lutgemm_gradB_kernel(
 #pragma unroll
             for (int kk = 0; kk < KT; ++kk) acc[kk] = __builtin_fmaf(t[kk], g[i], acc[kk]);
             __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    {
+        uint32_t a4x, a4y;
+        float gx[RPL], gy[RPL];
+        int m = mb;
+        if (m < me) load_rows(m, a4x, gx);
+        while (m < me) {
+            if (m + RPL < me) load_rows(m + RPL, a4y, gy);
+            consume_rows(a4x, gx);
+            m += RPL;
+            if (m >= me) break;
+            if (m + RPL < me) load_rows(m + RPL, a4x, gx);
+            consume_rows(a4y, gy);
+            m += RPL;
         }
     }
     if (n < N) {
@@ -114,12 +132,27 @@ __global__ __launch_bounds__(WAVES * 64) void lutgemm_gradA_kernel(
     // Transposed staging: entry (a,b) of the row-major table goes to T[b][a], T row stride = cols
     // entries (cols is even, so T rows stay dword aligned).  T needs cols rows of `rows` entries.
     {
+        // a dword of the table holds the entries (a, b) and (a, b + 1) (cols is even); eight loads of a thread are in
+        // flight before the first entry is stored
         uint16_t* t16 = reinterpret_cast<uint16_t*>(smem);
-        const int total = rows * cols;
-        for (int i = threadIdx.x; i < total; i += WAVES * 64) {
-            const int a = i / cols;
-            const int b = i - a * cols;
-            t16[b * cols + a] = lut[i];
+        const uint32_t* lut32 = reinterpret_cast<const uint32_t*>(lut);
+        const int hc = cols >> 1, total = rows * hc;
+        const float inv_hc = 1.0f / (float)hc;
+        constexpr int U = 8, THREADS = WAVES * 64;
+        for (int base = 0; base < total; base += U * THREADS) {
+            uint32_t v[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) v[u] = lut32[min(base + u * THREADS + (int)threadIdx.x, total - 1)];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int j = base + u * THREADS + (int)threadIdx.x;
+                if (j < total) {
+                    const int a = div_small(j, hc, inv_hc);
+                    const int b = 2 * (j - a * hc);
+                    t16[b * cols + a] = (uint16_t)v[u];
+                    t16[(b + 1) * cols + a] = (uint16_t)(v[u] >> 16);
+                }
+            }
         }
     }
     __syncthreads();
@@ -221,11 +254,12 @@ static hipError_t set_lds_attr(const void* f) {
 
 size_t gradB_workspace_bytes(int M, int K, int N, int n_cu, int* splits_out) {
     // Split M so that the launch has about 4 workgroups (of 4 waves) per CU and every split keeps
-    // at least 256 rows.
+    // at least 32 rows (two trips of a wave's row loop: a wave walks its rows one group of 16 after the other,
+    // about 4 us per group, so few long chunks leave a small problem latency-bound on a handful of CUs).
     constexpr int KT = 16;
     const long wg_per_split = (long)((N + 63) / 64) * (((K + KT - 1) / KT + 3) / 4);
     long splits = (4L * n_cu + wg_per_split - 1) / wg_per_split;
-    const long max_by_rows = M / 256 > 0 ? M / 256 : 1;
+    const long max_by_rows = M / 32 > 0 ? M / 32 : 1;
     if (splits > max_by_rows) splits = max_by_rows;
     if (splits > 256) splits = 256;
     if (splits < 1) splits = 1;

@@ -63,7 +63,7 @@ __global__ __launch_bounds__(WAVES * 64) void lutgemm_gradB_f32tab_kernel(
             float* s = reinterpret_cast<float*>(smem);
             const float* src = lut + (size_t)lo * cols;
             const int count = (int)nr * cols;
-            for (int i = threadIdx.x; i < count; i += WAVES * 64) s[i] = src[i];
+            stage_table_dwords<WAVES * 64>(s, src, count);
             if (SPLIT)
                 for (int i = threadIdx.x; i < cols; i += WAVES * 64) s[count + i] = 0.f;      // the row of zeros behind the band
         }
@@ -148,10 +148,21 @@ __global__ __launch_bounds__(WAVES * 64) void lutgemm_gradA_f32tab_kernel(
             // entry (a, b) of the row-major table goes to T[b - lo][a], T row stride = cols entries
             float* t32 = reinterpret_cast<float*>(smem);
             const int total = n_rows * (int)nr;
-            for (int i = threadIdx.x; i < total; i += WAVES * 64) {
-                const int a = i / (int)nr;
-                const int bb = i - a * (int)nr;
-                t32[bb * cols + a] = lut[(size_t)a * cols + lo + bb];
+            const float inv_nr = 1.0f / (float)nr;
+            constexpr int U = 8, THREADS = WAVES * 64;
+            for (int base = 0; base < total; base += U * THREADS) {      // eight loads of a thread in flight
+                float v[U];
+                int a[U], bb[U];
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    const int i = min(base + u * THREADS + (int)threadIdx.x, total - 1);
+                    a[u] = div_small(i, (int)nr, inv_nr);
+                    bb[u] = i - a[u] * (int)nr;
+                    v[u] = lut[(size_t)a[u] * cols + lo + bb[u]];
+                }
+#pragma unroll
+                for (int u = 0; u < U; ++u)
+                    if (base + u * THREADS + (int)threadIdx.x < total) t32[bb[u] * cols + a[u]] = v[u];
             }
             if (SPLIT)
                 for (int i = threadIdx.x; i < cols; i += WAVES * 64) t32[(int)nr * cols + i] = 0.f;      // the row of zeros behind the band

@@ -28,10 +28,7 @@ __global__ __launch_bounds__(WAVES * 64) void lutgemm_fwd_kernel(
     int atomic_out, const uint32_t* __restrict__ gate, int out_f32) {
     extern __shared__ __align__(16) unsigned char smem[];
     if (gate != nullptr && *gate == 0u) return;   // queued as a fallback that turned out not to be needed
-    {
-        uint32_t* s32 = reinterpret_cast<uint32_t*>(smem);
-        for (int i = threadIdx.x; i < lut_dwords; i += WAVES * 64) s32[i] = lut32[i];
-    }
+    stage_table_dwords<WAVES * 64>(smem, lut32, lut_dwords);
     __syncthreads();
 
     const int wave = uniform(threadIdx.x >> 6);
