@@ -54,6 +54,38 @@ def test_c_abi_rejects_bad_arguments_without_touching_a_device():
     assert lib.amr_lut_gemm_forward(None, None, None, None, 17408, 2, 2, 2, None) == -1     # null pointers
 
 
+def test_float_table_entry_point_checks_arguments_without_touching_a_device():
+    lib = _lib()
+    vp, i64, i, sz = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_size_t
+    lib.amr_lut_gemm_backward_f32tab.argtypes = [vp, vp, vp, vp, vp, vp, vp, i64, ctypes.c_float, i, i, i, i, vp, sz, vp]
+    call = lambda elems, M, K, N, L: lib.amr_lut_gemm_backward_f32tab(None, None, None, None, None, None, None, elems, 1.0, M, K, N, L,
+                                                                        None, 0, None)
+    assert call(66306, -1, 2, 2, 0) == -1          # negative dimension
+    assert call(66000, 2, 2, 2, 0) == -2           # not a padded table length
+    assert call(66306, 10, 2, 2, 3) == -1          # rows per image must divide M
+    assert call(66306, 0, 5, 0, 0) == 0            # empty problem
+    assert call(17408, 2, 2, 2, 0) == -1           # null pointers
+
+
+def test_gradient_tables_keep_their_kind_and_float_tables_need_both(golden_dir):
+    import approx_ops
+    from self_ops.ops_py import approx_ops as P
+    fwd, ga, gb = P.read_lut_file(os.path.join(golden_dir, "lut6_vert_trunc_bp2.txt.gz"), 6)
+    saved = (P.lut_appmult, P.lut_grad_a, P.lut_grad_b)
+    try:
+        P.set_lookup_tables("cpu", fwd, ga.astype(np.float64) / 16, gb.astype(np.float32) / 16)
+        assert P.lut_grad_a.dtype == torch.float32 and P.lut_grad_b.dtype == torch.float32
+        assert (P.lut_grad_a.numpy() * 16 == ga).all()
+        P.set_lookup_tables("cpu", fwd, ga, gb.astype(np.float32))       # one integer table: both stay int16
+        assert P.lut_grad_a.dtype == torch.int16 and P.lut_grad_b.dtype == torch.int16
+    finally:
+        P.lut_appmult, P.lut_grad_a, P.lut_grad_b = saved
+    # the dtype checks come after the device checks, as in the reference: a CPU tensor is reported first
+    with pytest.raises(RuntimeError, match="gc_tensor must be a CUDAtensor"):
+        approx_ops.approx_gemm_backward(torch.zeros(2, 2), torch.zeros(2, 2, dtype=torch.uint8), torch.zeros(2, 2, dtype=torch.uint8),
+                                        torch.zeros(2, 2), torch.zeros(2, 2), torch.zeros(5120), torch.zeros(5120), grad_scale=0.5)
+
+
 def test_python_surface_matches_reference_names():
     import approx_ops
     import self_ops
