@@ -56,6 +56,10 @@ hipError_t launch_gradA_f32tab(const float* gC, const uint8_t* A, const uint8_t*
 hipError_t launch_gradB_slab_f32tab(const float* gC, const uint8_t* A, const uint8_t* B, float* gB, const float* lut,
                                     const LutGeom& g, int M, int K, int N, float scale, uint32_t* flags, float* partials,
                                     int n_cu, hipStream_t stream);
+size_t gradA_slab_f32_workspace_bytes(const LutGeom& g, int M, int K, int N, bool force);
+hipError_t launch_gradA_slab_f32tab(const float* gC, const uint8_t* A, const uint8_t* B, float* gA, const float* lut,
+                                    const LutGeom& g, int M, int K, int N, float scale, int n_cu, uint32_t* flags, void* S,
+                                    int rows_per_image, hipStream_t stream);
 hipError_t launch_accgemm(const float* A, const float* B, float* C, int M, int K, int N, hipStream_t stream);
 hipError_t run_lds_probe(int pattern, int waves_per_cu, int iters, int n_cu, float* ms_out, double* gathers_out,
                          hipStream_t stream);
@@ -311,6 +315,20 @@ int amr_lut_gemm_backward_ex(const float* gC, const uint8_t* A, const uint8_t* B
     return AMR_OK;
 }
 
+// Scratch of the float-table backward pass: [256 B of flags][partial sums of gB][float32 expanded table of gradA].
+static size_t backward_gradA_f32_bytes(int M, int K, int N) {
+    if (!g_expanded_kernels) return 0;
+    amr::LutGeom g7;
+    amr::lut_geom_from_bits(7, &g7);
+    return amr::gradA_slab_f32_workspace_bytes(g7, M, K, N, g_expanded_kernels == 2);
+}
+
+size_t amr_lut_gemm_backward_f32tab_workspace_bytes(int M, int K, int N) {
+    if (M <= 0 || K <= 0 || N <= 0) return 0;
+    const int n_cu = current_device_cus(nullptr);
+    return 256 + backward_partial_bytes(M, K, N, n_cu > 0 ? n_cu : 256) + backward_gradA_f32_bytes(M, K, N);
+}
+
 int amr_lut_gemm_backward_f32tab(const float* gC, const uint8_t* A, const uint8_t* B, float* gA, float* gB,
                                  const float* lut_grad_a, const float* lut_grad_b, int64_t lut_elems, float scale, int M, int K,
                                  int N, int ga_rows_per_image, void* workspace, size_t workspace_bytes, void* stream) {
@@ -337,7 +355,7 @@ int amr_lut_gemm_backward_f32tab(const float* gC, const uint8_t* A, const uint8_
     if (n_cu <= 0) return fail(AMR_EINVAL, "no HIP device available");
     hipError_t e;
     const size_t partial_bytes = backward_partial_bytes(M, K, N, n_cu);
-    const size_t need = 256 + partial_bytes;
+    const size_t need = 256 + partial_bytes + backward_gradA_f32_bytes(M, K, N);
     void* ws = workspace;
     if (ws) {
         if (workspace_bytes < need) return fail(AMR_EWORKSPACE, "workspace of %zu bytes is smaller than the %zu required", workspace_bytes, need);
@@ -348,12 +366,23 @@ int amr_lut_gemm_backward_f32tab(const float* gC, const uint8_t* A, const uint8_
     }
     uint32_t* flags = reinterpret_cast<uint32_t*>(ws);
     float* partials = reinterpret_cast<float*>(reinterpret_cast<unsigned char*>(ws) + 256);
+    const bool slab_b = g_expanded_kernels && gB && amr::bwd_slab_applies(g, M, K, N);
+    const bool slab_a = g_expanded_kernels && gA && amr::gradA_slab_f32_workspace_bytes(g, M, K, N, g_expanded_kernels == 2) != 0 &&
+                        ((uintptr_t)gC & 15) == 0;
+    if (slab_a || slab_b) {
+        e = amr::launch_zero_u32(flags, 64, s);
+        if (e != hipSuccess) return hip_fail(e, "scratch header launch");
+    }
     if (gA) {
-        e = amr::launch_gradA_f32tab(gC, A, B, gA, lut_grad_a, g, M, K, N, scale, n_cu, s, nullptr, ga_rows_per_image);
+        if (slab_a)
+            e = amr::launch_gradA_slab_f32tab(gC, A, B, gA, lut_grad_a, g, M, K, N, scale, n_cu, flags,
+                                              reinterpret_cast<unsigned char*>(ws) + 256 + partial_bytes, ga_rows_per_image, s);
+        else
+            e = amr::launch_gradA_f32tab(gC, A, B, gA, lut_grad_a, g, M, K, N, scale, n_cu, s, nullptr, ga_rows_per_image);
         if (e != hipSuccess) return hip_fail(e, "gradA launch");
     }
     if (gB) {
-        if (g_expanded_kernels && amr::bwd_slab_applies(g, M, K, N)) {
+        if (slab_b) {
             e = amr::launch_gradB_slab_f32tab(gC, A, B, gB, lut_grad_b, g, M, K, N, scale, flags, partials, n_cu, s);
         } else {
             int splits = 1;

@@ -568,13 +568,10 @@ hipError_t launch_gradB_slab(const float* gC, const uint8_t* A, const uint8_t* B
 hipError_t launch_gradB_f32tab(const float* gC, const uint8_t* A, const uint8_t* B, float* gB, const float* lut, const LutGeom& g,
                                int M, int K, int N, float scale, void* workspace, int splits, hipStream_t stream,
                                const uint32_t* gate);
-hipError_t launch_zero_u32(void* p, size_t n_dwords, hipStream_t stream);
-
 hipError_t launch_gradB_slab_f32tab(const float* gC, const uint8_t* A, const uint8_t* B, float* gB, const float* lut,
                                     const LutGeom& g, int M, int K, int N, float scale, uint32_t* flags, float* partials,
                                     int n_cu, hipStream_t stream) {
-    hipError_t e = launch_zero_u32(flags, 64, stream);
-    if (e != hipSuccess) return e;
+    hipError_t e;
     const int vec_ok = ((N & 3) == 0) && (((uintptr_t)gC & 15) == 0);
     const bool small = (size_t)M * K < (1ull << 31) && (size_t)M * N * 4 < (1ull << 31);
     const bool regular = vec_ok && small && (N & 63) == 0 && (M % kBwdRowsPerIter) == 0;

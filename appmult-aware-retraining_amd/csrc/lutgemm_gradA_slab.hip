@@ -43,15 +43,16 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 
-constexpr int kGaCols = 32;                               // columns per tile
+constexpr int kGaCols = 32;                               // columns per tile (half entries; 16 for float32 entries)
+constexpr int kGaColsF32 = 16;
 constexpr int kGaChunkK = 4;
-constexpr int kGaChunkBytes = 128 * kGaChunkK * 2 * kGaCols;   // 32 KB
+constexpr int kGaChunkBytes = 128 * kGaChunkK * 2 * kGaCols;   // 32 KB (= 128 codes x 4 k x 16 columns x 4 bytes as well)
 constexpr int kGaBufs = 3;
 constexpr int kGaWaves = 16;
 constexpr int kGaRowsPerWave = 32;                        // 16 quads x 2 rows
 constexpr int kGaRows = kGaWaves * kGaRowsPerWave;        // 512 rows per workgroup
 constexpr int kGaStageBase = kGaBufs * kGaChunkBytes;     // 96 KB: the rows of gC of one column tile, 128 B per row
-constexpr int kGaStageBytes = kGaRows * kGaCols * 4;      // 64 KB
+constexpr int kGaStageBytes = kGaRows * kGaCols * 4;      // 64 KB (half of it used with float32 entries)
 static_assert(kGaStageBase + kGaStageBytes == 160 * 1024, "the workgroup uses the whole LDS of a CU");
 
 // ------------------------------------------------------------------------------------------ expand
@@ -98,6 +99,29 @@ __global__ __launch_bounds__(256) void expand_gradA_kernel(const uint8_t* __rest
     }
 }
 
+// The same for a float32 table: S[n_tile][k / 4][a][k % 4][16 columns] float32, the entries themselves (no offset, nothing
+// inexact).  grid (N / 16, ceil(K / 4 / quads_per_wg)), 256 threads, the table (rows x cols floats) in dynamic LDS.
+__global__ __launch_bounds__(256) void expand_gradA_f32_kernel(const uint8_t* __restrict__ B, const float* __restrict__ lut,
+                                                               int lut_entries, int lut_cols, int n_codes, uint32_t* __restrict__ S,
+                                                               int K, int N, int quads_per_wg) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    stage_table_dwords<256>(smem, lut, lut_entries);
+    __syncthreads();
+    const uint32_t* s32 = reinterpret_cast<const uint32_t*>(smem);
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    // a wave writes the 256 B row of one code: lane = (k % 4, column), one dword per lane
+    const int ks = lane >> 4, col = lane & 15;
+    const int n = blockIdx.x * kGaColsF32 + col;
+    for (int pp = 0; pp < quads_per_wg; ++pp) {
+        const int kq = blockIdx.y * quads_per_wg + pp;
+        if (4 * kq >= K) break;
+        const uint32_t* p0 = s32 + (int)B[(size_t)(4 * kq + ks) * N + n];
+        uint32_t* chunk = S + ((size_t)blockIdx.x * (K / 4) + kq) * (kGaChunkBytes / 4) + lane;
+#pragma unroll 8
+        for (int a = wave; a < 128; a += 4) chunk[a * 64] = p0[min(a, n_codes) * lut_cols];
+    }
+}
+
 // ------------------------------------------------------------------------------------------ consume
 // One 128-bit LDS read of a chunk, issued and NOT waited for.  The address comes out of ONE v_perm_b32:
 // byte 0 = the lane's constant (window and piece), byte 1 = the code (BYTE of codeword; < 128), byte 2 = 1 for
@@ -119,7 +143,9 @@ __device__ __forceinline__ void ga_read(u32x4& d, uint32_t codeword, uint32_t la
 // grid: 8 * (workgroups per XCD, at most one per CU) workgroups of 1024 threads; every workgroup walks several tiles
 // (512 rows x KT k) one after the other.  Requires N % 32 == 0, K % KT == 0, M >= 32, M*K < 2^31, gC 16-byte aligned.
 // rows_per_image = 0: gA row-major [M,K]; L > 0: image-major transposed gA[m / L][k][m % L].
-template <int kGaKT>
+// F32: S holds float32 entries, 16 columns per tile (a 64 B window is 16 floats, a 128-bit read feeds four v_fma_f32 instead
+// of eight v_fma_mix_f32); no offset.
+template <int kGaKT, bool F32>
 __global__ __launch_bounds__(kGaWaves * 64) void lutgemm_gradA_slab_kernel(
     const float* __restrict__ gC, const uint8_t* __restrict__ A, const u32x4* __restrict__ S, float* __restrict__ gA,
     uint32_t* __restrict__ flags, int M, int K, int N, float scale, int rows_per_image, int row_blocks, int band_rows_max) {
@@ -127,6 +153,9 @@ __global__ __launch_bounds__(kGaWaves * 64) void lutgemm_gradA_slab_kernel(
     constexpr int CH = kGaKT / kGaChunkK;                  // chunks per column tile
     constexpr int NTU = (CH % kGaBufs) == 0 ? 1 : kGaBufs; // column tiles per unrolled pass: the buffer of a chunk is then static
     constexpr int NST = 2 * CH;                            // stores per lane at the end of a tile
+    constexpr int COLS = F32 ? kGaColsF32 : kGaCols;       // columns per tile
+    constexpr int STAGE_WAVE = kGaRowsPerWave * COLS * 4;  // bytes of gC rows a wave stages per column tile (4 KB / 2 KB)
+    constexpr int ROWOPS = STAGE_WAVE / 1024;              // wave-wide 16-byte loads of a row request (4 / 2)
     static_assert(CH >= 4, "the bookkeeping of outstanding loads assumes at least four chunks per column tile");
     const int tid = threadIdx.x;
     const int wave = uniform(tid >> 6);
@@ -143,9 +172,9 @@ __global__ __launch_bounds__(kGaWaves * 64) void lutgemm_gradA_slab_kernel(
     const int total_tiles = row_blocks * k_groups;
     const int per_xcd = (total_tiles + 7) / 8;
     const int xcd = (int)(blockIdx.x % 8), pos_stride = (int)(gridDim.x / 8);
-    const int n_tiles = N / kGaCols;
+    const int n_tiles = N / COLS;
     const int total = n_tiles * CH;                          // chunks of a tile: (column tile, four k)
-    const float offset = (float)flags[3];
+    const float offset = F32 ? 0.f : (float)flags[3];
     struct Tile { int k0, m_wave; bool valid; };
     auto decode = [&](int pos) {
         Tile t;
@@ -192,19 +221,21 @@ __global__ __launch_bounds__(kGaWaves * 64) void lutgemm_gradA_slab_kernel(
             __builtin_amdgcn_global_load_lds((gptr_t)(src + (wave + kGaWaves * i) * 64 + lane),
                                              (lptr_t)(smem + buf * kGaChunkBytes + (wave + kGaWaves * i) * 1024), 16, 0, 0);
     };
-    // the 32 rows of this wave, 128 B (32 columns of tile nt) each: four wave-wide loads, lane = (row % 8, 16 B piece);
+    // the 32 rows of this wave, 128 B (32 columns of tile nt) each: four wave-wide loads, lane = (row % 8, 16 B piece)
+    // (float32 entries: 64 B of 16 columns, two loads, lane = (row % 16, piece));
     // beyond the last column tile: the first one of the next tile
-    const uint32_t glane = (uint32_t)(lane >> 3) * (uint32_t)N + 4u * (uint32_t)(lane & 7);
+    constexpr int RPO = 64 * 16 / (COLS * 4);                // rows per wave-wide load (8 / 16)
+    const uint32_t glane = (uint32_t)(lane / (64 / RPO)) * (uint32_t)N + 4u * (uint32_t)(lane % (64 / RPO));
     auto request_rows = [&](int nt) {
         int m_base = m_base_of(cur);
         if (nt >= n_tiles) {
             if (nxt.valid) { nt = 0; m_base = m_base_of(nxt); } else nt = n_tiles - 1;
         }
-        const float* base = gC + (size_t)m_base * N + nt * kGaCols;
+        const float* base = gC + (size_t)m_base * N + nt * COLS;
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
-            __builtin_amdgcn_global_load_lds((gptr_t)(base + (size_t)(8 * i) * N + glane),
-                                             (lptr_t)(smem + kGaStageBase + wave * 4096 + i * 1024), 16, 0, 0);
+        for (int i = 0; i < ROWOPS; ++i)
+            __builtin_amdgcn_global_load_lds((gptr_t)(base + (size_t)(RPO * i) * N + glane),
+                                             (lptr_t)(smem + kGaStageBase + wave * STAGE_WAVE + i * 1024), 16, 0, 0);
     };
     // The codes of a tile: A[m][k0 + 4 j + c], one byte per chunk and row, packed four to a register.  Assembly loads:
     // the waiting is explicit (the compiler would wait for everything in flight).
@@ -241,18 +272,18 @@ __global__ __launch_bounds__(kGaWaves * 64) void lutgemm_gradA_slab_kernel(
     for (int r = 0; r < 2; ++r)
 #pragma unroll
         for (int j = 0; j < CH; ++j) acc[r][j] = 0.f;
-    float g[2][kGaCols];
+    float g[2][COLS];
 #pragma unroll
     for (int r = 0; r < 2; ++r)
 #pragma unroll
-        for (int i = 0; i < kGaCols; ++i) g[r][i] = 0.f;
+        for (int i = 0; i < COLS; ++i) g[r][i] = 0.f;
     float row_sum[2] = {0.f, 0.f};
     u32x4 d[4] = {{0, 0, 0, 0}, {0, 0, 0, 0}, {0, 0, 0, 0}, {0, 0, 0, 0}};
 
     // Operations of a wave towards memory, in issue order (vmcnt counts them in this order):
     //   rows(0) chunk(0) chunk(1) codes | step q: chunk(q + 2); second step of column tile nt also: rows(nt + 1)
     //   | end of a tile: codes of the next tile, NST stores | ...
-    // (a chunk request is two operations, a row request four).  At the top of step q, chunk q (requested two steps
+    // (a chunk request is two operations, a row request ROWOPS = four, two with float32 entries).  At the top of step q, chunk q (requested two steps
     // earlier) must have landed: all but the requests of the previous step may be outstanding; in the first two
     // steps of a tile the stores of the previous one as well.
     request_rows(0);
@@ -276,13 +307,23 @@ __global__ __launch_bounds__(kGaWaves * 64) void lutgemm_gradA_slab_kernel(
     // every 9 clocks.
     auto pair_fma = [&](auto kc_tag, auto s_tag, const u32x4& d0, const u32x4& d1) {
         constexpr int KC = decltype(kc_tag)::value;
-        constexpr int S8 = 8 * decltype(s_tag)::value;
-        const f16x8 h0 = __builtin_bit_cast(f16x8, d0), h1 = __builtin_bit_cast(f16x8, d1);
         float s0 = acc[0][KC], s1 = acc[1][KC];
+        if constexpr (F32) {
+            constexpr int S4 = 4 * decltype(s_tag)::value;
+            const f32x4 f0 = __builtin_bit_cast(f32x4, d0), f1 = __builtin_bit_cast(f32x4, d1);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            s0 = __builtin_fmaf(g[0][S8 + e], (float)h0[e], s0);
-            s1 = __builtin_fmaf(g[1][S8 + e], (float)h1[e], s1);
+            for (int e = 0; e < 4; ++e) {
+                s0 = __builtin_fmaf(g[0][S4 + e], f0[e], s0);
+                s1 = __builtin_fmaf(g[1][S4 + e], f1[e], s1);
+            }
+        } else {
+            constexpr int S8 = 8 * decltype(s_tag)::value;
+            const f16x8 h0 = __builtin_bit_cast(f16x8, d0), h1 = __builtin_bit_cast(f16x8, d1);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                s0 = __builtin_fmaf(g[0][S8 + e], (float)h0[e], s0);
+                s1 = __builtin_fmaf(g[1][S8 + e], (float)h1[e], s1);
+            }
         }
         // pin: the sums are finished before the next volatile read is issued (otherwise the compiler keeps the
         // results of several reads live and runs out of registers)
@@ -304,7 +345,7 @@ __global__ __launch_bounds__(kGaWaves * 64) void lutgemm_gradA_slab_kernel(
             if (KC == 0) asm volatile("s_waitcnt vmcnt(%2)\n s_barrier" : "+v"(d[2]), "+v"(d[3]) : "n"(NST) : "memory");
             else asm volatile("s_waitcnt vmcnt(%2)\n s_barrier" : "+v"(d[2]), "+v"(d[3]) : "n"(NST + 2) : "memory");
         } else if (KC == 2 || KC == 3) {
-            asm volatile("s_waitcnt vmcnt(6)\n s_barrier" : "+v"(d[2]), "+v"(d[3]) : : "memory");
+            asm volatile("s_waitcnt vmcnt(%2)\n s_barrier" : "+v"(d[2]), "+v"(d[3]) : "n"(2 + ROWOPS) : "memory");
         } else {
             asm volatile("s_waitcnt vmcnt(2)\n s_barrier" : "+v"(d[2]), "+v"(d[3]) : : "memory");
         }
@@ -318,9 +359,25 @@ __global__ __launch_bounds__(kGaWaves * 64) void lutgemm_gradA_slab_kernel(
         ga_read<KC & 3, BUF>(d[3], codes[1][KC >> 2], lane_const[1]);
         if (KC == 0) {
             // new column tile: the rows of gC from the staging area, pieces in this lane's rotated order
-            const uint32_t gbase = (uint32_t)(kGaStageBase + wave * 4096 + quad * 128);
+            const uint32_t gbase = (uint32_t)(kGaStageBase + wave * STAGE_WAVE + quad * (COLS * 4));
 #pragma unroll
             for (int r = 0; r < 2; ++r) {
+                if constexpr (F32) {
+                    // a row is 64 B: piece (quad + s) % 4 for step s, one 128-bit read each
+                    u32x4 t[4];
+#pragma unroll
+                    for (int s = 0; s < 4; ++s) {
+                        const uint32_t ga = gbase + (uint32_t)(((quad + s) & 3) << 4);
+                        if (r == 0) asm volatile("ds_read_b128 %0, %1" : "=&v"(t[s]) : "v"(ga) : "memory");
+                        else asm volatile("ds_read_b128 %0, %1 offset:1024" : "=&v"(t[s]) : "v"(ga) : "memory");
+                    }
+                    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(t[0]), "+v"(t[1]), "+v"(t[2]), "+v"(t[3]), "+v"(d[0]), "+v"(d[1]), "+v"(d[2]), "+v"(d[3]) : : "memory");
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const f32x4 v = __builtin_bit_cast(f32x4, t[i]);
+                        g[r][4 * i] = v.x; g[r][4 * i + 1] = v.y; g[r][4 * i + 2] = v.z; g[r][4 * i + 3] = v.w;
+                    }
+                } else {
                 // (two pieces at a time: eight more registers in flight would not fit)
 #pragma unroll
                 for (int hf = 0; hf < 2; ++hf) {
@@ -345,8 +402,9 @@ __global__ __launch_bounds__(kGaWaves * 64) void lutgemm_gradA_slab_kernel(
                 if (offset != 0.f) {
                     float s = row_sum[r];
 #pragma unroll
-                    for (int i = 0; i < kGaCols; ++i) s += g[r][i];
+                    for (int i = 0; i < COLS; ++i) s += g[r][i];
                     row_sum[r] = s;
+                }
                 }
             }
         }
@@ -487,15 +545,66 @@ hipError_t launch_gradA_slab(const float* gC, const uint8_t* A, const uint8_t* B
     const int per_xcd = (tiles + 7) / 8, cus_per_xcd = n_cu >= 8 ? n_cu / 8 : 1;
     const dim3 grid(8 * (per_xcd < cus_per_xcd ? per_xcd : cus_per_xcd));
     if (kt == 32)
-        hipLaunchKernelGGL((lutgemm_gradA_slab_kernel<32>), grid, block, 0, stream, gC, A, S4, gA, flags, M, K, N, scale,
+        hipLaunchKernelGGL((lutgemm_gradA_slab_kernel<32, false>), grid, block, 0, stream, gC, A, S4, gA, flags, M, K, N, scale,
                            rows_per_image, row_blocks, band_rows);
     else
-        hipLaunchKernelGGL((lutgemm_gradA_slab_kernel<16>), grid, block, 0, stream, gC, A, S4, gA, flags, M, K, N, scale,
+        hipLaunchKernelGGL((lutgemm_gradA_slab_kernel<16, false>), grid, block, 0, stream, gC, A, S4, gA, flags, M, K, N, scale,
                            rows_per_image, row_blocks, band_rows);
     e = hipGetLastError();
     if (e != hipSuccess) return e;
     // masked codes in A or table entries a half cannot hold: the gated direct kernel recomputes gA
     return launch_gradA(gC, A, B, gA, lut, g, M, K, N, scale, n_cu, stream, flags + 2, rows_per_image);
+}
+
+// ------------------------------------------------------------------------------------------ float32 tables
+hipError_t launch_gradA_f32tab(const float* gC, const uint8_t* A, const uint8_t* B, float* gA, const float* lut, const LutGeom& g,
+                               int M, int K, int N, float scale, int n_cu, hipStream_t stream, const uint32_t* gate,
+                               int rows_per_image);
+
+// Bytes of the float32 expanded table, or 0 when that kernel does not apply.  It is twice the size of the half one and
+// every block of 512 rows streams all of it, so it pays for fewer shapes: with 4096 rows and K*N = 4608 x 512 the
+// table alone is 1.2 GB.
+size_t gradA_slab_f32_workspace_bytes(const LutGeom& g, int M, int K, int N, bool force) {
+    if (!force && (M < 4096 || (double)M * K * N < 2e8)) return 0;
+    if (g.bits > 7 || M < 512 || (N % kGaColsF32) != 0 || (K % 16) != 0 || (size_t)M * K >= (1ull << 31)) return 0;
+    return (size_t)(N / kGaColsF32) * (K / kGaChunkK) * kGaChunkBytes;
+}
+
+// flags[2] must be zero on entry (masked codes in A raise it; the gated direct kernel then recomputes gA).
+hipError_t launch_gradA_slab_f32tab(const float* gC, const uint8_t* A, const uint8_t* B, float* gA, const float* lut,
+                                    const LutGeom& g, int M, int K, int N, float scale, int n_cu, uint32_t* flags, void* S,
+                                    int rows_per_image, hipStream_t stream) {
+    if (((uintptr_t)gC & 15) != 0) return hipErrorInvalidValue;   // callers check: rows of gC are fetched 16 bytes at a time
+    const int lut_entries = g.rows * g.cols;
+    static bool attr_done = false;
+    if (!attr_done) {
+        hipError_t ea = hipFuncSetAttribute(reinterpret_cast<const void*>(expand_gradA_f32_kernel),
+                                            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        if (ea != hipSuccess) return ea;
+        attr_done = true;
+    }
+    const int qpw = 4;
+    hipLaunchKernelGGL(expand_gradA_f32_kernel, dim3(N / kGaColsF32, (K / 4 + qpw - 1) / qpw), dim3(256), (size_t)lut_entries * 4,
+                       stream, B, lut, lut_entries, g.cols, 1 << g.bits, reinterpret_cast<uint32_t*>(S), K, N, qpw);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    const u32x4* S4 = reinterpret_cast<const u32x4*>(S);
+    const dim3 block(kGaWaves * 64);
+    const int row_blocks = (M + kGaRows - 1) / kGaRows;
+    const int band_rows = 16;
+    const int kt = ((K % 32) == 0 && row_blocks * (K / 32) >= n_cu) ? 32 : 16;
+    const int tiles = row_blocks * (K / kt);
+    const int per_xcd = (tiles + 7) / 8, cus_per_xcd = n_cu >= 8 ? n_cu / 8 : 1;
+    const dim3 grid(8 * (per_xcd < cus_per_xcd ? per_xcd : cus_per_xcd));
+    if (kt == 32)
+        hipLaunchKernelGGL((lutgemm_gradA_slab_kernel<32, true>), grid, block, 0, stream, gC, A, S4, gA, flags, M, K, N, scale,
+                           rows_per_image, row_blocks, band_rows);
+    else
+        hipLaunchKernelGGL((lutgemm_gradA_slab_kernel<16, true>), grid, block, 0, stream, gC, A, S4, gA, flags, M, K, N, scale,
+                           rows_per_image, row_blocks, band_rows);
+    e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    return launch_gradA_f32tab(gC, A, B, gA, lut, g, M, K, N, scale, n_cu, stream, flags + 2, rows_per_image);
 }
 
 }  // namespace amr

@@ -119,7 +119,7 @@ def main():
             gC=torch.randn((M, N), dtype=torch.float32, device=dev, generator=gen),
             gA=torch.empty((M, K), dtype=torch.float32, device=dev),
             gB=torch.empty((K, N), dtype=torch.float32, device=dev))
-        ws_need = max(ws_need, lib.amr_lut_gemm_backward_workspace_bytes(M, K, N))
+        ws_need = max(ws_need, (lib.amr_lut_gemm_backward_f32tab_workspace_bytes if f32_tables else lib.amr_lut_gemm_backward_workspace_bytes)(M, K, N))
     ws = torch.empty(max(ws_need, 256), dtype=torch.uint8, device=dev)
 
     def fwd(name, M, K, N):

@@ -122,8 +122,10 @@ int amr_lut_gemm_backward_ex(const float *gC, const uint8_t *A, const uint8_t *B
  * (scale = 1) or any other float table.  A float table of int16 values with scale = 1/16 gives the results of
  * amr_lut_gemm_backward up to fp32 summation order.  An 8-bit float table (265 KB) exceeds the LDS of a CU and is
  * processed in two bands of rows.  Arguments otherwise as amr_lut_gemm_backward_ex; the workspace size is
- * amr_lut_gemm_backward_workspace_bytes(M,K,N).
+ * amr_lut_gemm_backward_f32tab_workspace_bytes(M,K,N) (partial sums of gB and, for large M, the float32 expanded table
+ * of gradA, twice the size of the int16 path's).
  */
+size_t amr_lut_gemm_backward_f32tab_workspace_bytes(int M, int K, int N);
 int amr_lut_gemm_backward_f32tab(const float *gC, const uint8_t *A, const uint8_t *B, float *gA, float *gB,
                                  const float *lut_grad_a, const float *lut_grad_b, int64_t lut_elems, float scale,
                                  int M, int K, int N, int ga_rows_per_image, void *workspace, size_t workspace_bytes,

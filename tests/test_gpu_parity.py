@@ -31,6 +31,8 @@ def lib():
     L.amr_lut_gemm_forward_workspace_bytes.restype = sz
     L.amr_lut_gemm_backward.argtypes = [vp, vp, vp, vp, vp, vp, vp, i64, i, i, i, vp, sz, vp]
     L.amr_lut_gemm_backward_f32tab.argtypes = [vp, vp, vp, vp, vp, vp, vp, i64, ctypes.c_float, i, i, i, i, vp, sz, vp]
+    L.amr_lut_gemm_backward_f32tab_workspace_bytes.argtypes = [i, i, i]
+    L.amr_lut_gemm_backward_f32tab_workspace_bytes.restype = sz
     L.amr_lut_gemm_backward_workspace_bytes.argtypes = [i, i, i]
     L.amr_lut_gemm_backward_workspace_bytes.restype = sz
     L.amr_acc_gemm_forward_fp32.argtypes = [vp, vp, vp, i, i, i, vp]
@@ -361,7 +363,7 @@ def gpu_backward_f32tab(lib, g, A, B, la, lb, scale, own_workspace=True, rows_pe
     gd, a, b, ta, tb = dev(g), dev(A), dev(B), dev(np.asarray(la, np.float32)), dev(np.asarray(lb, np.float32))
     ga = torch.full((M, K), float("nan"), device="cuda")
     gb = torch.full((K, N), float("nan"), device="cuda")
-    need = lib.amr_lut_gemm_backward_workspace_bytes(M, K, N)
+    need = lib.amr_lut_gemm_backward_f32tab_workspace_bytes(M, K, N)
     ws = torch.empty(max(need, 1), dtype=torch.uint8, device="cuda") if own_workspace else None
     rc = lib.amr_lut_gemm_backward_f32tab(gd.data_ptr(), a.data_ptr(), b.data_ptr(), ga.data_ptr(), gb.data_ptr(), ta.data_ptr(),
                                           tb.data_ptr(), ta.numel(), scale, M, K, N, rows_per_image,
@@ -373,8 +375,11 @@ def gpu_backward_f32tab(lib, g, A, B, la, lb, scale, own_workspace=True, rows_pe
 
 # small and ragged shapes (direct kernels), K below one workgroup's share (idle waves at the band barriers), and
 # M >= 1024 (gradB on the fp32 expanded table for tables of at most 7 bits)
+# (N % 16 == 0, K % 16 == 0 and M >= 512: gradA on the float32 expanded table, 16 or 32 k per tile, one to ten column tiles, also
+# with a ragged last row block)
 F32TAB_SHAPES = [(1, 1, 1), (3, 5, 7), (9, 27, 10), (64, 64, 64), (33, 130, 65), (600, 96, 64), (257, 100, 129), (300, 288, 256),
-                 (70, 50, 513), (1100, 27, 64), (4096, 8, 64), (4100, 27, 10), (5000, 130, 65), (2048, 48, 128), (1500, 40, 70)]
+                 (70, 50, 513), (1100, 27, 64), (4096, 8, 64), (4100, 27, 10), (5000, 130, 65), (2048, 48, 128), (1500, 40, 70),
+                 (1024, 16, 16), (5000, 80, 48), (4096, 64, 32), (9001, 64, 16), (2148, 144, 160), (16384, 32, 64), (8192, 576, 64)]
 
 
 @pytest.mark.parametrize("bits", [7, 8, 6, 4])
@@ -410,6 +415,31 @@ def test_backward_float_tables_masked_codes_and_both_bands(lib, oracle, bits):
     A[18, :] = 0
     check_backward(oracle, gpu_backward_f32tab(lib, g, A, B, la, lb, 1.0), g, A, B, la, lb, bits, factor=1.0)
     check_backward(oracle, gpu_backward_f32tab(lib, g, A, B, la, lb, 1.0, own_workspace=False), g, A, B, la, lb, bits, factor=1.0)
+
+
+def test_backward_float_tables_expanded_gradA_masked_codes(lib, oracle):
+    print("backward float tables, expanded gradA with masked codes", flush=True)
+    M, K, N = 4224, 32, 64
+    rng, A, B, _ = rand_case(700, M, K, N, 7)
+    la = oracle.pack_table(rng.standard_normal((128, 128)) * 10, 7, np.float32)
+    lb = oracle.pack_table(rng.standard_normal((128, 128)) * 10, 7, np.float32)
+    g = rng.standard_normal((M, N)).astype(np.float32)
+    assert lib.amr_lut_gemm_backward_f32tab_workspace_bytes(M, K, N) > lib.amr_lut_gemm_backward_workspace_bytes(M, K, N) > 0
+    check_backward(oracle, gpu_backward_f32tab(lib, g, A, B, la, lb, 1.0), g, A, B, la, lb, 7, factor=1.0)
+    A2, B2 = A.copy(), B.copy()
+    A2[::7, 3] = 128
+    A2[-1, :] = 128
+    B2[5, ::3] = 128
+    check_backward(oracle, gpu_backward_f32tab(lib, g, A2, B2, la, lb, 1.0), g, A2, B2, la, lb, 7, factor=1.0)
+    check_backward(oracle, gpu_backward_f32tab(lib, g, A, B, la, lb, 1.0), g, A, B, la, lb, 7, factor=1.0)     # clean again
+    # image-major gA from the expanded-table kernel equals the row-major one
+    L = 64
+    gd, a, b, ta, tb = dev(g), dev(A), dev(B), dev(la), dev(lb)
+    gat = torch.full((M // L, K, L), float("nan"), device="cuda")
+    assert lib.amr_lut_gemm_backward_f32tab(gd.data_ptr(), a.data_ptr(), b.data_ptr(), gat.data_ptr(), None, ta.data_ptr(), tb.data_ptr(),
+                                            ta.numel(), 1.0, M, K, N, L, None, 0, None) == 0
+    torch.cuda.synchronize()
+    assert (gat.cpu().numpy().transpose(0, 2, 1).reshape(M, K) == gpu_backward_f32tab(lib, g, A, B, la, lb, 1.0)[0]).all()
 
 
 @pytest.mark.parametrize("bits", [7, 8])
