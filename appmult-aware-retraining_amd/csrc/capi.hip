@@ -15,9 +15,9 @@ hipError_t launch_fwd(const uint8_t* A, const uint8_t* B, uint32_t* C, const uin
 size_t fwd_slab_workspace_bytes(const LutGeom& g, int M, int K, int N, bool force);
 hipError_t launch_fwd_slab(const uint8_t* A, const uint8_t* B, uint32_t* C, const uint16_t* lut, const LutGeom& g,
                            int M, int K, int N, int n_cu, void* workspace, hipStream_t stream, int out_f32);
-size_t gradB_workspace_bytes(int M, int K, int N, int n_cu, int* splits_out);
+size_t gradB_workspace_bytes(int M, int K, int N, int n_cu);
 hipError_t launch_gradB(const float* gC, const uint8_t* A, const uint8_t* B, float* gB, const int16_t* lut,
-                        const LutGeom& g, int M, int K, int N, float scale, void* workspace, int splits,
+                        const LutGeom& g, int M, int K, int N, float scale, void* workspace, int n_cu,
                         hipStream_t stream, const uint32_t* gate = nullptr);
 hipError_t launch_gradA(const float* gC, const uint8_t* A, const uint8_t* B, float* gA, const int16_t* lut,
                         const LutGeom& g, int M, int K, int N, float scale, int n_cu, hipStream_t stream,
@@ -48,7 +48,7 @@ hipError_t launch_gradB_slab(const float* gC, const uint8_t* A, const uint8_t* B
                              const LutGeom& g, int M, int K, int N, float scale, uint32_t* flags, float* partials,
                              int n_cu, hipStream_t stream);
 hipError_t launch_gradB_f32tab(const float* gC, const uint8_t* A, const uint8_t* B, float* gB, const float* lut, const LutGeom& g,
-                               int M, int K, int N, float scale, void* workspace, int splits, hipStream_t stream,
+                               int M, int K, int N, float scale, void* workspace, int n_cu, hipStream_t stream,
                                const uint32_t* gate);
 hipError_t launch_gradA_f32tab(const float* gC, const uint8_t* A, const uint8_t* B, float* gA, const float* lut, const LutGeom& g,
                                int M, int K, int N, float scale, int n_cu, hipStream_t stream, const uint32_t* gate,
@@ -218,7 +218,7 @@ int amr_lut_gemm_forward(const uint8_t* A, const uint8_t* B, uint32_t* C, const 
 // Scratch layout of the backward pass: [256 B of flags][partial sums of gB over the M splits][expanded
 // gradient table of gradA]; each part a multiple of 256 bytes.
 static size_t backward_partial_bytes(int M, int K, int N, int n_cu) {
-    size_t direct = amr::gradB_workspace_bytes(M, K, N, n_cu, nullptr);
+    size_t direct = amr::gradB_workspace_bytes(M, K, N, n_cu);
     const int s = amr::gradB_slab_splits(M, K, N, n_cu);
     size_t slab = s > 1 ? (size_t)s * K * N * sizeof(float) : 0;
     const size_t b = direct > slab ? direct : slab;
@@ -306,9 +306,7 @@ int amr_lut_gemm_backward_ex(const float* gC, const uint8_t* A, const uint8_t* B
         if (slab) {
             e = amr::launch_gradB_slab(gC, A, B, gB, lut_grad_b, g, M, K, N, scale, flags, partials, n_cu, s);
         } else {
-            int splits = 1;
-            amr::gradB_workspace_bytes(M, K, N, n_cu, &splits);
-            e = amr::launch_gradB(gC, A, B, gB, lut_grad_b, g, M, K, N, scale, partials, splits, s);
+            e = amr::launch_gradB(gC, A, B, gB, lut_grad_b, g, M, K, N, scale, partials, n_cu, s);
         }
         if (e != hipSuccess) return hip_fail(e, "gradB launch");
     }
@@ -385,9 +383,7 @@ int amr_lut_gemm_backward_f32tab(const float* gC, const uint8_t* A, const uint8_
         if (slab_b) {
             e = amr::launch_gradB_slab_f32tab(gC, A, B, gB, lut_grad_b, g, M, K, N, scale, flags, partials, n_cu, s);
         } else {
-            int splits = 1;
-            amr::gradB_workspace_bytes(M, K, N, n_cu, &splits);
-            e = amr::launch_gradB_f32tab(gC, A, B, gB, lut_grad_b, g, M, K, N, scale, partials, splits, s, nullptr);
+            e = amr::launch_gradB_f32tab(gC, A, B, gB, lut_grad_b, g, M, K, N, scale, partials, n_cu, s, nullptr);
         }
         if (e != hipSuccess) return hip_fail(e, "gradB launch");
     }

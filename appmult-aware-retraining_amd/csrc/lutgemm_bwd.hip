@@ -252,28 +252,52 @@ static hipError_t set_lds_attr(const void* f) {
     return hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
 }
 
-size_t gradB_workspace_bytes(int M, int K, int N, int n_cu, int* splits_out) {
-    // Split M so that the launch has about 4 workgroups (of 4 waves) per CU and every split keeps
-    // at least 32 rows (two trips of a wave's row loop: a wave walks its rows one group of 16 after the other,
-    // about 4 us per group, so few long chunks leave a small problem latency-bound on a handful of CUs).
+// M splits of a direct gradB launch whose workgroups have `waves` waves (each owning 16 k) and of which `wgs_per_cu` fit a
+// CU at a time.  The grid runs in rounds of n_cu * wgs_per_cu workgroups: the split count is the one whose
+// (rounds x rows per workgroup) is smallest -- 290 workgroups on 256 CUs take as long as 512 -- with every split keeping
+// at least 32 rows (two trips of a wave's row loop: a wave walks its rows one group of 16 after the other, about 4 us
+// per group, so few long chunks leave a small problem latency-bound on a handful of CUs).
+int gradB_direct_splits(int M, int K, int N, int n_cu, int waves, int wgs_per_cu) {
     constexpr int KT = 16;
-    const long wg_per_split = (long)((N + 63) / 64) * (((K + KT - 1) / KT + 3) / 4);
-    long splits = (4L * n_cu + wg_per_split - 1) / wg_per_split;
-    const long max_by_rows = M / 32 > 0 ? M / 32 : 1;
-    if (splits > max_by_rows) splits = max_by_rows;
-    if (splits > 256) splits = 256;
-    if (splits < 1) splits = 1;
-    if (splits_out) *splits_out = (int)splits;
-    return splits > 1 ? (size_t)splits * K * N * sizeof(float) : 0;
+    const long ktiles = (K + KT - 1) / KT;
+    const long per_split = (long)((N + 63) / 64) * ((ktiles + waves - 1) / waves);
+    const long slots = (long)n_cu * wgs_per_cu;
+    long max_s = M / 32;
+    if (max_s > 256) max_s = 256;
+    if (max_s < 1) max_s = 1;
+    long best_s = 1, best_cost = -1;
+    for (long sp = 1; sp <= max_s; ++sp) {
+        long chunk = (M + sp - 1) / sp;
+        chunk = (chunk + 15) & ~15L;
+        const long zs = (M + chunk - 1) / chunk;
+        const long rounds = (per_split * zs + slots - 1) / slots;
+        // (+16 rows: staging the table and the reduction pass over one more partial result)
+        const long cost = rounds * (chunk + 16);
+        if (best_cost < 0 || cost < best_cost) { best_cost = cost; best_s = sp; }
+    }
+    return (int)best_s;
 }
 
+// Scratch for the partial sums of the direct gradB kernels: the largest split count any of their launch shapes picks
+// (4 waves and four workgroups per CU: int16 tables of at most 7 bits; two per CU: float tables of at most 7 bits; 16 waves,
+// one per CU: 8-bit tables).
+size_t gradB_workspace_bytes(int M, int K, int N, int n_cu) {
+    int s = gradB_direct_splits(M, K, N, n_cu, 4, 4);
+    const int s2 = gradB_direct_splits(M, K, N, n_cu, 4, 2), s3 = gradB_direct_splits(M, K, N, n_cu, 16, 1);
+    if (s2 > s) s = s2;
+    if (s3 > s) s = s3;
+    return s > 1 ? (size_t)s * K * N * sizeof(float) : 0;
+}
+
+// workspace: room for the partial sums (gradB_workspace_bytes), or nullptr: no split over M.
 hipError_t launch_gradB(const float* gC, const uint8_t* A, const uint8_t* B, float* gB, const int16_t* lut,
-                        const LutGeom& g, int M, int K, int N, float scale, void* workspace, int splits,
+                        const LutGeom& g, int M, int K, int N, float scale, void* workspace, int n_cu,
                         hipStream_t stream, const uint32_t* gate = nullptr) {
     constexpr int KT = 16;
     const int lut_dwords = g.rows * g.cols / 2;
     const size_t lds = (size_t)lut_dwords * 4;
     const bool big = g.bits == 8;
+    const int splits = workspace ? gradB_direct_splits(M, K, N, n_cu, big ? 16 : 4, big ? 1 : 4) : 1;
     int m_chunk = (M + splits - 1) / splits;
     m_chunk = (m_chunk + 15) & ~15;
     const int zs = (M + m_chunk - 1) / m_chunk;
@@ -332,6 +356,13 @@ hipError_t launch_gradA(const float* gC, const uint8_t* A, const uint8_t* B, flo
     const bool vec = ((N & 3) == 0) && (((uintptr_t)gC & 15) == 0);   // rows of gC are read 16 bytes at a time
     const int ktiles = (K + KT - 1) / KT;
     if (g.bits == 8) {
+        // one 1024-thread workgroup per CU; two rows per lane (half the scalar work per gather) unless one row per lane
+        // needs fewer (rounds of n_cu workgroups) x (rows per workgroup)
+        const long cost2 = (((long)ktiles * ((M + 2047) / 2048) + n_cu - 1) / n_cu) * 2048;
+        const long cost1 = (((long)ktiles * ((M + 1023) / 1024) + n_cu - 1) / n_cu) * 1024;
+        if (cost2 <= cost1)
+            return vec ? launch_gradA_t<KT, 2, 16, true>(gC, A, B, gA, lut, g, M, K, N, scale, stream, gate, rows_per_image)
+                       : launch_gradA_t<KT, 2, 16, false>(gC, A, B, gA, lut, g, M, K, N, scale, stream, gate, rows_per_image);
         return vec ? launch_gradA_t<KT, 1, 16, true>(gC, A, B, gA, lut, g, M, K, N, scale, stream, gate, rows_per_image)
                    : launch_gradA_t<KT, 1, 16, false>(gC, A, B, gA, lut, g, M, K, N, scale, stream, gate, rows_per_image);
     }
@@ -349,7 +380,7 @@ hipError_t launch_gradA(const float* gC, const uint8_t* A, const uint8_t* B, flo
 // held a masked code) and then overwrites the whole result (no M split: no scratch).
 hipError_t launch_gradB_gated(const float* gC, const uint8_t* A, const uint8_t* B, float* gB, const int16_t* lut,
                               const LutGeom& g, int M, int K, int N, float scale, const uint32_t* gate, hipStream_t stream) {
-    return launch_gradB(gC, A, B, gB, lut, g, M, K, N, scale, nullptr, 1, stream, gate);
+    return launch_gradB(gC, A, B, gB, lut, g, M, K, N, scale, nullptr, 0, stream, gate);
 }
 
 }  // namespace amr

@@ -253,20 +253,25 @@ static hipError_t allow_big_lds(Kern kern, bool* done) {
     return e;
 }
 
+int gradB_direct_splits(int M, int K, int N, int n_cu, int waves, int wgs_per_cu);
+
+// workspace: room for the partial sums (gradB_workspace_bytes), or nullptr: no split over M.
 hipError_t launch_gradB_f32tab(const float* gC, const uint8_t* A, const uint8_t* B, float* gB, const float* lut, const LutGeom& g,
-                               int M, int K, int N, float scale, void* workspace, int splits, hipStream_t stream,
+                               int M, int K, int N, float scale, void* workspace, int n_cu, hipStream_t stream,
                                const uint32_t* gate) {
     constexpr int KT = 16;
     int rows_pp, passes;
     f32tab_bands(g, &rows_pp, &passes);
     const size_t lds = (size_t)(rows_pp + 1) * g.cols * 4;      // + the row of zeros
+    const bool wide = passes > 1 || lds > 80 * 1024;            // one 1024-thread workgroup per CU
+    const int splits = workspace ? gradB_direct_splits(M, K, N, n_cu, wide ? 16 : 4, wide ? 1 : 2) : 1;
     int m_chunk = (M + splits - 1) / splits;
     m_chunk = (m_chunk + 15) & ~15;
     const int zs = (M + m_chunk - 1) / m_chunk;
     float* out = zs > 1 ? reinterpret_cast<float*>(workspace) : gB;
     const int ktiles = (K + KT - 1) / KT;
     hipError_t e;
-    if (passes > 1 || lds > 80 * 1024) {
+    if (wide) {
         // one 1024-thread workgroup per CU shares the staged band
         static bool done = false;
         auto kern = lutgemm_gradB_f32tab_kernel<KT, 16, true>;
@@ -316,8 +321,11 @@ hipError_t launch_gradA_f32tab(const float* gC, const uint8_t* A, const uint8_t*
     const bool vec = ((N & 3) == 0) && (((uintptr_t)gC & 15) == 0);   // rows of gC are read 16 bytes at a time
     const int ktiles = (K + KT - 1) / KT;
     if (passes > 1 || (size_t)rows_pp * g.cols * 4 > 80 * 1024) {
-        // one 1024-thread workgroup per CU shares the staged band; two rows per lane when that still fills the CUs
-        if ((long)ktiles * ((M + 2047) / 2048) >= n_cu)
+        // one 1024-thread workgroup per CU shares the staged band; two rows per lane (half the scalar work per gather) unless
+        // one row per lane needs fewer (rounds of n_cu workgroups) x (rows per workgroup)
+        const long cost2 = (((long)ktiles * ((M + 2047) / 2048) + n_cu - 1) / n_cu) * 2048;
+        const long cost1 = (((long)ktiles * ((M + 1023) / 1024) + n_cu - 1) / n_cu) * 1024;
+        if (cost2 <= cost1)
             return vec ? launch_gradA_f32tab_t<KT, 2, 16, true, true>(gC, A, B, gA, lut, g, rows_pp, passes, M, K, N, scale, stream, gate, rows_per_image)
                        : launch_gradA_f32tab_t<KT, 2, 16, false, true>(gC, A, B, gA, lut, g, rows_pp, passes, M, K, N, scale, stream, gate, rows_per_image);
         return vec ? launch_gradA_f32tab_t<KT, 1, 16, true, true>(gC, A, B, gA, lut, g, rows_pp, passes, M, K, N, scale, stream, gate, rows_per_image)

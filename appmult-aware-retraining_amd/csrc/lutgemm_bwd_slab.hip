@@ -566,7 +566,7 @@ hipError_t launch_gradB_slab(const float* gC, const uint8_t* A, const uint8_t* B
 // direct kernel forms (the half-precision slab cannot hold arbitrary float entries).  flags[1] is cleared here; the
 // direct float-table kernel queued behind is gated on it (7-bit operands holding the masked code 128).
 hipError_t launch_gradB_f32tab(const float* gC, const uint8_t* A, const uint8_t* B, float* gB, const float* lut, const LutGeom& g,
-                               int M, int K, int N, float scale, void* workspace, int splits, hipStream_t stream,
+                               int M, int K, int N, float scale, void* workspace, int n_cu, hipStream_t stream,
                                const uint32_t* gate);
 hipError_t launch_gradB_slab_f32tab(const float* gC, const uint8_t* A, const uint8_t* B, float* gB, const float* lut,
                                     const LutGeom& g, int M, int K, int N, float scale, uint32_t* flags, float* partials,
@@ -596,7 +596,7 @@ hipError_t launch_gradB_slab_f32tab(const float* gC, const uint8_t* A, const uin
         e = hipGetLastError();
         if (e != hipSuccess) return e;
     }
-    if (g.bits == 7) return launch_gradB_f32tab(gC, A, B, gB, lut, g, M, K, N, scale, nullptr, 1, stream, flags + 1);
+    if (g.bits == 7) return launch_gradB_f32tab(gC, A, B, gB, lut, g, M, K, N, scale, nullptr, n_cu, stream, flags + 1);
     return hipSuccess;
 }
 

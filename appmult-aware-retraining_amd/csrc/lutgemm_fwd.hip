@@ -173,7 +173,7 @@ hipError_t launch_fwd(const uint8_t* A, const uint8_t* B, uint32_t* C, const uin
         ksplit = (int)((target_wg + wgs - 1) / wgs);
         const int max_split = K / 64 > 0 ? K / 64 : 1;  // keep at least 64 k per workgroup
         if (ksplit > max_split) ksplit = max_split;
-        if (ksplit > 16) ksplit = 16;
+        if (ksplit > 64) ksplit = 64;
     }
 #define AMR_FWD_CASE(r, tn)                                                                                   \
     if (R == r && TN == tn)                                                                                   \
