@@ -1,7 +1,7 @@
 """Synthetic-data AppMult-aware retraining loop (counterpart of the reference's ``micronet+/app_train.py``
 minus datasets and checkpoints, which need the network): prepare -> calibrate -> train steps.
 
-    python app_train.py --lut <table file> --bits 7 --batch 512 --steps 10 [--ste] [--optimizer sgd|adam]
+    python app_train.py --lut <table file> --bits 7 --batch 512 --steps 10 [--ste] [--optimizer sgd|adam] [--float-grad-window W]
 
 Flow as in the reference (``app_train.py:231-266``): ``init_lookup_tables`` -> ``app_layers.prepare`` ->
 one calibration pass in training mode without gradients -> optimiser steps of
@@ -71,11 +71,27 @@ def main(argv=None):
     ap.add_argument("--ste", action="store_true", help="straight-through gradients instead of the gradient tables")
     ap.add_argument("--optimizer", default="adam", choices=["adam", "sgd"])
     ap.add_argument("--approx-linear", action="store_true", help="run the classifier on the table as well (the reference keeps it exact)")
+    ap.add_argument("--float-grad-window", type=int, default=0, metavar="W",
+                    help="replace the file's int16 gradient tables by the float32 difference slopes of its forward table, "
+                         "half window W (the float-table backward pass; no counterpart in the reference)")
     args = ap.parse_args(argv)
     assert torch.cuda.is_available(), "a GPU is required"
     device = torch.device("cuda")
     torch.manual_seed(199608224)
     self_ops.init_lookup_tables(device, args.lut, args.bits)
+    if args.float_grad_window > 0:
+        import numpy as np
+        import gen_bp_lut
+        from self_ops.ops_py import approx_ops as P
+        rows, cols, _ = P.lut_geometry(args.bits)
+        n = 1 << args.bits
+        flat = P.lut_appmult.cpu().numpy()
+        fwd = flat[:rows * cols].reshape(rows, cols)[:n, :n]
+        ga, gb = gen_bp_lut.gradient_tables(fwd, args.float_grad_window, rounded=False)
+        pa, pb = np.zeros(flat.size, np.float32), np.zeros(flat.size, np.float32)
+        idx = (np.arange(n)[:, None] * cols + np.arange(n)[None, :]).ravel()
+        pa[idx], pb[idx] = ga.ravel(), gb.ravel()
+        P.set_lookup_tables(device, flat, pa, pb)
     model = build_model(args.arch, args.bits, args.ste, device, approx_linear=args.approx_linear)
     xs, ys = synthetic_batches(args.steps + 1, args.batch, device)
     calibrate(model, xs[:1])

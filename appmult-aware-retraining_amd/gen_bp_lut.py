@@ -38,8 +38,9 @@ def _window_mean(F32, h, axis):
     return (sums.astype(np.float32) / cnt.reshape(shape)).astype(np.float32)
 
 
-def gradient_tables(fwd, half_ws):
-    """fwd: (N, N) integer table.  Returns (grad_a16, grad_b16) int64 = round(16 * slope)."""
+def gradient_tables(fwd, half_ws, rounded=True):
+    """fwd: (N, N) integer table.  Returns (grad_a16, grad_b16) int64 = round(16 * slope), the encoding of the reference's
+    table files; rounded=False returns the float32 slopes themselves (for the float-table backward pass)."""
     assert half_ws >= 1
     F32 = np.asarray(fwd).astype(np.float32)
     n = F32.shape[0]
@@ -57,6 +58,8 @@ def gradient_tables(fwd, half_ws):
     if hi >= lo:
         ga[lo:hi + 1, :] = (sa[lo + 1:hi + 2, :] - sa[lo - 1:hi, :]) / np.float32(2)
         gb[:, lo:hi + 1] = (sb[:, lo + 1:hi + 2] - sb[:, lo - 1:hi]) / np.float32(2)
+    if not rounded:
+        return ga, gb
     return (np.round(ga * np.float32(16.0)).astype(np.int64), np.round(gb * np.float32(16.0)).astype(np.int64))
 
 

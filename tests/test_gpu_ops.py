@@ -406,6 +406,27 @@ def test_synthetic_training_steps_reduce_loss(ops, golden_dir):
     assert all(np.isfinite(losses)) and losses[-1] < losses[0]
 
 
+def test_training_harness_cli_with_float_gradient_tables(ops, golden_dir, tmp_path, capsys):
+    """The command-line harness end to end on a small batch, with the file's int16 tables and with float32 slopes."""
+    import gzip
+    import shutil
+    import app_train as T
+    from self_ops.ops_py import approx_ops as P
+    print("train harness cli", flush=True)
+    lut = tmp_path / "lut7.txt"
+    with gzip.open(os.path.join(golden_dir, "lut7_resub_63_bp8.txt.gz"), "rb") as f, open(lut, "wb") as o:
+        shutil.copyfileobj(f, o)
+    saved = (P.lut_appmult, P.lut_grad_a, P.lut_grad_b)
+    try:
+        for extra, dtype in ([], torch.int16), (["--float-grad-window", "8"], torch.float32):
+            T.main(["--lut", str(lut), "--bits", "7", "--batch", "32", "--steps", "2", "--optimizer", "sgd"] + extra)
+            assert P.lut_grad_a.dtype == dtype
+            out = capsys.readouterr().out
+            assert "img/s" in out and "nan" not in out.lower()
+    finally:
+        P.lut_appmult, P.lut_grad_a, P.lut_grad_b = saved
+
+
 def test_approx_linear_equals_fake_quant_linear_with_exact_multiplier(ops, oracle):
     """With LUT[a][b] = a*b the table classifier computes the same function as the fake-quantised one (the reference's
     QuantLinear, app_layers.py:101-111), values and gradients, up to fp32 rounding of the scaling."""

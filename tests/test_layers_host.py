@@ -28,6 +28,18 @@ def test_gradient_table_generator_equals_oracle_loops_on_random_table(oracle):
         assert (a == ao).all() and (b == bo).all()
 
 
+def test_gradient_table_generator_float_slopes_equal_oracle_loops(oracle):
+    import gen_bp_lut as G
+    rng = np.random.default_rng(4)
+    T = oracle.synth_lut(6, 16, rng)
+    for hw in (1, 3, 8):
+        a, b = G.gradient_tables(T, hw, rounded=False)
+        a0, b0 = oracle.gen_bp_lut(T, hw, rounded=False)
+        assert a.dtype == np.float32 and (a == a0).all() and (b == b0).all()
+        a16, b16 = G.gradient_tables(T, hw)
+        assert (a16 == np.round(a * np.float32(16))).all() and (b16 == np.round(b * np.float32(16))).all()
+
+
 def test_generator_cli_round_trip(tmp_path, oracle, golden_dir, capsys):
     import gzip
     import gen_bp_lut as G
