@@ -231,7 +231,8 @@ __device__ __forceinline__ void slab_read_codes(uint32_t (&a)[8], uint32_t addr)
 template <int RG, int WAVES, bool PACKED>
 __global__ __launch_bounds__(WAVES * 64) void lutgemm_fwd_slab_kernel(
     const uint8_t* __restrict__ A, const u32x4* __restrict__ E, uint32_t* __restrict__ C,
-    uint32_t* __restrict__ flags, int M, int K, int N, int k_quads, int chunks_per_split, int atomic_out, int out_f32) {
+    uint32_t* __restrict__ flags, int M, int K, int N, int k_quads, int chunks_per_split, int atomic_out, int out_f32,
+    int n_tiles_grouped, int row_blocks) {
     // static: lets the compiler fold the base address (chunk buffers first: their addresses come out of v_perm)
     __shared__ __align__(16) unsigned char smem[kSlabBuffers * kSlabChunkBytes + 2 * kSlabCodeBytes];
     constexpr int THREADS = WAVES * 64;
@@ -242,19 +243,31 @@ __global__ __launch_bounds__(WAVES * 64) void lutgemm_fwd_slab_kernel(
     const int wave = uniform(tid >> 6);
     const int lane = tid & 63;
     const int rs = lane >> 3, cg = lane & 7, rot = rs & 3;
+    // Workgroup -> (column tile, row block, K split).  Plain: the grid's three dimensions.  Grouped (n_tiles_grouped > 0,
+    // 1-D grid, no K split): the hardware deals workgroups to the 8 XCDs round-robin by index; the column tiles of one
+    // row block get consecutive slots of ONE XCD, so that they run at the same time behind the same L2 and fetch their
+    // rows of A once between them (chosen by the host when A is larger than the expanded table).
+    int tile_x = blockIdx.x, rb_y = blockIdx.y;
+    const int split_z = blockIdx.z;
+    if (n_tiles_grouped > 0) {
+        const int xcd = (int)(blockIdx.x & 7), slot = (int)(blockIdx.x >> 3);
+        tile_x = slot % n_tiles_grouped;
+        rb_y = xcd + 8 * (slot / n_tiles_grouped);
+        if (rb_y >= row_blocks) return;
+    }
     // A wave whose rows would stick out of M is shifted up so that all its rows exist (the host only
     // takes this path for M >= 2048); the rows it then shares with the wave above are not stored twice.
     // (a wave entirely beyond M keeps running, it takes part in the chunk copies, and stores nothing)
-    const int m_first = (blockIdx.y * WAVES + wave) * ROWS_PER_WAVE;     // first row this wave must store
+    const int m_first = (rb_y * WAVES + wave) * ROWS_PER_WAVE;     // first row this wave must store
     const int m_wave = min(m_first, M - ROWS_PER_WAVE);
-    const int c_begin = blockIdx.z * chunks_per_split;
+    const int c_begin = split_z * chunks_per_split;
     const int c_end = min(k_quads, c_begin + chunks_per_split);
     if (c_begin >= c_end) return;
     // Two instances of this kernel are queued for every GEMM; the table maximum (written by the
     // expand kernel) decides which one does the work: 16-bit packed partial sums need 4*max < 65536.
     if ((flags[0] < 16384u) != PACKED) return;
 
-    const u32x4* Eblk = E + ((size_t)blockIdx.x * k_quads) * (kSlabChunkBytes / 16);
+    const u32x4* Eblk = E + ((size_t)tile_x * k_quads) * (kSlabChunkBytes / 16);
 
     // per-lane address pieces; instruction j of a chunk reads k = 4c + ((j + rot) & 3)
     uint32_t base_lo[4], base_hi[4], sel[4];
@@ -335,7 +348,7 @@ __global__ __launch_bounds__(WAVES * 64) void lutgemm_fwd_slab_kernel(
     if (__builtin_amdgcn_ballot_w64((seen & 0x80808080u) != 0) != 0) {
         if (lane == 0) atomicOr(&flags[1], 1u);
     }
-    const int n = blockIdx.x * kSlabCols + 4 * cg;
+    const int n = tile_x * kSlabCols + 4 * cg;
 #pragma unroll
     for (int i = 0; i < RG; ++i) {
         const int m = m_wave + 8 * rs + i;
@@ -404,12 +417,20 @@ hipError_t launch_fwd_slab(const uint8_t* A, const uint8_t* B, uint32_t* C, cons
         e = launch_zero_u32(C, (size_t)M * N, stream);
         if (e != hipSuccess) return e;
     }
-    dim3 grid(n_tiles, (M + m_tile - 1) / m_tile, zs);
+    const int row_blocks = (M + m_tile - 1) / m_tile;
+    dim3 grid(n_tiles, row_blocks, zs);
+    // A larger than the expanded table (M > 256 N) and several column tiles: the tiles of a row block share an XCD
+    int grouped = 0;
+    // (measured: conv2_x 0.40 -> 0.38 ms, conv3_x 0.395 -> 0.37 ms; with a split K the rows are few and A is small)
+    if (zs == 1 && n_tiles > 1 && (size_t)M > (size_t)256 * N) {
+        grouped = n_tiles;
+        grid = dim3(8 * ((row_blocks + 7) / 8) * n_tiles);
+    }
     // both accumulation flavours are queued; flags[0] (table maximum) decides on the device which one works
     hipLaunchKernelGGL((lutgemm_fwd_slab_kernel<RG, WAVES, true>), grid, dim3(WAVES * 64), 0, stream, A,
-                       reinterpret_cast<const u32x4*>(E), C, flags, M, K, N, k_quads, cps, zs > 1 ? 1 : 0, out_f32);
+                       reinterpret_cast<const u32x4*>(E), C, flags, M, K, N, k_quads, cps, zs > 1 ? 1 : 0, out_f32, grouped, row_blocks);
     hipLaunchKernelGGL((lutgemm_fwd_slab_kernel<RG, WAVES, false>), grid, dim3(WAVES * 64), 0, stream, A,
-                       reinterpret_cast<const u32x4*>(E), C, flags, M, K, N, k_quads, cps, zs > 1 ? 1 : 0, out_f32);
+                       reinterpret_cast<const u32x4*>(E), C, flags, M, K, N, k_quads, cps, zs > 1 ? 1 : 0, out_f32, grouped, row_blocks);
     e = hipGetLastError();
     if (e != hipSuccess) return e;
     // (partial sums over a split K met as integers: converted before the fall-back, which stores floats itself)
