@@ -691,3 +691,58 @@ def test_benchmark_shapes_against_oracle_on_row_samples(lib, oracle, shape):
     mask[rows_t] = False
     assert (ga[mask] == 0).all()                              # rows without gradient: exactly zero
     check_backward(oracle, (ga[rows_t].cpu().numpy(), gb.cpu().numpy()), gs, As, Bn, la, lb, 7)
+
+
+VGG16_B128_SHAPES = [(131072, 27, 64), (131072, 576, 64), (32768, 576, 128), (32768, 1152, 128), (8192, 1152, 256), (8192, 2304, 256),
+                     (2048, 2304, 512), (2048, 4608, 512), (512, 4608, 512), (128, 512, 10)]
+
+
+@pytest.mark.parametrize("kind,bits,shape", [("f32", 7, s) for s in RESNET18_B256_SHAPES] + [("i16", 8, s) for s in VGG16_B128_SHAPES] +
+                         [("f32", 8, s) for s in VGG16_B128_SHAPES])
+def test_benchmark_shapes_other_table_formats_on_row_samples(lib, oracle, kind, bits, shape):
+    """The same row-sample check for the other two workloads of the benchmark: float32 gradient tables on the ResNet-18
+    shapes (7 bit) and the VGG-16 shapes at batch 128 with 8-bit tables, int16 and float32 gradient tables (unrounded
+    difference slopes, half window 8 / 16), in the library's own kernel selection."""
+    print("benchmark shape", kind, bits, shape, flush=True)
+    M, K, N = shape
+    n = 1 << bits
+    gen = torch.Generator(device="cuda").manual_seed(M + K + N + bits)
+    rng = np.random.default_rng(M + 3 * K + 7 * N + bits)
+    T = oracle.synth_lut(bits, 64 if bits == 7 else 256, rng)
+    hw = 8 if bits == 7 else 16
+    if kind == "f32":
+        Gx, Gy = oracle.gen_bp_lut(T, hw, rounded=False)
+        la, lb, factor = oracle.pack_table(Gx, bits, np.float32), oracle.pack_table(Gy, bits, np.float32), 1.0
+    else:
+        Gx, Gy = oracle.gen_bp_lut(T, hw)
+        la, lb, factor = oracle.pack_table(Gx, bits, np.int16), oracle.pack_table(Gy, bits, np.int16), 1.0 / 16
+    flat = oracle.pack_table(T, bits, np.uint16)
+    a = torch.randint(0, n, (M, K), dtype=torch.uint8, device="cuda", generator=gen)
+    b = torch.randint(0, n, (K, N), dtype=torch.uint8, device="cuda", generator=gen)
+    rows = np.unique(np.r_[0:96, np.arange(37, M, max(M // 1200, 1)), M // 2 - 70:M // 2 + 70, M - 96:M].clip(0, M - 1))
+    rows_t = torch.from_numpy(rows).cuda()
+    g = torch.zeros((M, N), device="cuda")
+    g[rows_t] = torch.randn((len(rows), N), device="cuda", generator=gen)
+    c = torch.empty((M, N), dtype=torch.int32, device="cuda")
+    ga = torch.full((M, K), float("nan"), device="cuda")
+    gb = torch.full((K, N), float("nan"), device="cuda")
+    l, ta, tb = dev(flat), dev(la), dev(lb)
+    assert lib.amr_set_expanded_table_kernels(1) == 2
+    try:
+        assert lib.amr_lut_gemm_forward(a.data_ptr(), b.data_ptr(), c.data_ptr(), l.data_ptr(), l.numel(), M, K, N, None) == 0
+        if kind == "f32":
+            rc = lib.amr_lut_gemm_backward_f32tab(g.data_ptr(), a.data_ptr(), b.data_ptr(), ga.data_ptr(), gb.data_ptr(), ta.data_ptr(),
+                                                  tb.data_ptr(), ta.numel(), 1.0, M, K, N, 0, None, 0, None)
+        else:
+            rc = lib.amr_lut_gemm_backward(g.data_ptr(), a.data_ptr(), b.data_ptr(), ga.data_ptr(), gb.data_ptr(), ta.data_ptr(),
+                                           tb.data_ptr(), ta.numel(), M, K, N, None, 0, None)
+        assert rc == 0, lib.amr_last_error()
+        torch.cuda.synchronize()
+    finally:
+        lib.amr_set_expanded_table_kernels(2)
+    As, Bn, gs = a[rows_t].cpu().numpy(), b.cpu().numpy(), g[rows_t].cpu().numpy()
+    assert (c[rows_t].cpu().numpy().view(np.uint32) == oracle.forward_c(As, Bn, flat, bits)).all()
+    mask = torch.ones(M, dtype=torch.bool, device="cuda")
+    mask[rows_t] = False
+    assert (ga[mask] == 0).all()                              # rows without gradient: exactly zero
+    check_backward(oracle, (ga[rows_t].cpu().numpy(), gb.cpu().numpy()), gs, As, Bn, la, lb, bits, factor=factor)
