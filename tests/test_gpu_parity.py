@@ -417,6 +417,65 @@ def test_backward_float_tables_masked_codes_and_both_bands(lib, oracle, bits):
     check_backward(oracle, gpu_backward_f32tab(lib, g, A, B, la, lb, 1.0, own_workspace=False), g, A, B, la, lb, bits, factor=1.0)
 
 
+@pytest.mark.parametrize("bits,shape", [(7, (700, 96, 64)), (8, (300, 40, 48)), (7, (4224, 32, 64)), (6, (129, 17, 33))])
+def test_backward_float_tables_pointers_aligned_to_four_bytes_only(lib, oracle, bits, shape):
+    """Tables, gC, gA and gB at addresses that are multiples of 4 but not of 16: no 128-bit access may be assumed."""
+    print("backward float tables, 4-byte aligned pointers", bits, shape, flush=True)
+    M, K, N = shape
+    n = 1 << bits
+    rng, A, B, _ = rand_case(800 + bits + M, M, K, N, bits)
+    la = oracle.pack_table(rng.standard_normal((n, n)) * 7, bits, np.float32)
+    lb = oracle.pack_table(rng.standard_normal((n, n)) * 7, bits, np.float32)
+    g = rng.standard_normal((M, N)).astype(np.float32)
+
+    def shifted(x, fill=None):
+        t = torch.empty(x.size + 1, dtype=torch.float32, device="cuda")
+        v = t[1:]
+        if fill is None:
+            v.copy_(torch.from_numpy(np.ascontiguousarray(x).ravel()))
+        else:
+            v.fill_(fill)
+        assert v.data_ptr() % 16 == 4
+        return t, v
+    keep = []
+    ptr = {}
+    for name, arr, fill in (("g", g, None), ("ta", la, None), ("tb", lb, None), ("ga", np.empty((M, K), np.float32), float("nan")),
+                            ("gb", np.empty((K, N), np.float32), float("nan"))):
+        t, v = shifted(arr, fill)
+        keep.append(t)
+        ptr[name] = v
+    a, b = dev(A), dev(B)
+    rc = lib.amr_lut_gemm_backward_f32tab(ptr["g"].data_ptr(), a.data_ptr(), b.data_ptr(), ptr["ga"].data_ptr(), ptr["gb"].data_ptr(),
+                                          ptr["ta"].data_ptr(), ptr["tb"].data_ptr(), la.size, 0.5, M, K, N, 0, None, 0, None)
+    assert rc == 0, lib.amr_last_error()
+    torch.cuda.synchronize()
+    got = (ptr["ga"].cpu().numpy().reshape(M, K), ptr["gb"].cpu().numpy().reshape(K, N))
+    check_backward(oracle, got, g, A, B, la, lb, bits, factor=0.5)
+
+
+@pytest.mark.parametrize("bits,shape", [(7, (700, 96, 64)), (8, (300, 40, 48)), (7, (4224, 32, 64)), (6, (1290, 17, 33))])
+def test_backward_int16_tables_pointers_aligned_to_four_bytes_only(lib, oracle, bits, shape):
+    print("backward, 4-byte aligned pointers", bits, shape, flush=True)
+    M, K, N = shape
+    n = 1 << bits
+    rng, A, B, _ = rand_case(900 + bits + M, M, K, N, bits)
+    la = oracle.pack_table(rng.integers(-2000, 2000, (n, n)), bits, np.int16)
+    lb = oracle.pack_table(rng.integers(-2000, 2000, (n, n)), bits, np.int16)
+    g = rng.standard_normal((M, N)).astype(np.float32)
+    tg = torch.empty(g.size + 1, device="cuda"); vg = tg[1:]; vg.copy_(torch.from_numpy(g.ravel()))
+    tga = torch.full((M * K + 1,), float("nan"), device="cuda"); vga = tga[1:]
+    tgb = torch.full((K * N + 1,), float("nan"), device="cuda"); vgb = tgb[1:]
+    tta = torch.empty(la.size + 2, dtype=torch.int16, device="cuda"); vta = tta[2:]; vta.copy_(torch.from_numpy(la))
+    ttb = torch.empty(lb.size + 2, dtype=torch.int16, device="cuda"); vtb = ttb[2:]; vtb.copy_(torch.from_numpy(lb))
+    assert vg.data_ptr() % 16 == 4 and vta.data_ptr() % 16 == 4
+    a, b = dev(A), dev(B)
+    rc = lib.amr_lut_gemm_backward(vg.data_ptr(), a.data_ptr(), b.data_ptr(), vga.data_ptr(), vgb.data_ptr(), vta.data_ptr(),
+                                   vtb.data_ptr(), la.size, M, K, N, None, 0, None)
+    assert rc == 0, lib.amr_last_error()
+    torch.cuda.synchronize()
+    check_backward(oracle, (vga.cpu().numpy().reshape(M, K), vgb.cpu().numpy().reshape(K, N)), g, A, B, la, lb, bits)
+
+
 def test_backward_float_tables_expanded_gradA_masked_codes(lib, oracle):
     print("backward float tables, expanded gradA with masked codes", flush=True)
     M, K, N = 4224, 32, 64
