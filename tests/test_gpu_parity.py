@@ -476,6 +476,28 @@ def test_backward_int16_tables_pointers_aligned_to_four_bytes_only(lib, oracle, 
     check_backward(oracle, (vga.cpu().numpy().reshape(M, K), vgb.cpu().numpy().reshape(K, N)), g, A, B, la, lb, bits)
 
 
+@pytest.mark.parametrize("bits,shape", [(7, (3000, 64, 64)), (8, (3000, 64, 64)), (7, (300, 200, 40))])
+def test_backward_float_tables_deterministic_and_skippable_outputs(lib, oracle, bits, shape):
+    print("backward float tables, determinism", bits, shape, flush=True)
+    M, K, N = shape
+    n = 1 << bits
+    rng, A, B, _ = rand_case(1000 + bits + M, M, K, N, bits)
+    la = oracle.pack_table(rng.standard_normal((n, n)) * 30, bits, np.float32)
+    g = rng.standard_normal((M, N)).astype(np.float32)
+    r1 = gpu_backward_f32tab(lib, g, A, B, la, la, 0.25)
+    r2 = gpu_backward_f32tab(lib, g, A, B, la, la, 0.25)
+    assert (r1[0] == r2[0]).all() and (r1[1] == r2[1]).all()
+    gd, a, b, t = dev(g), dev(A), dev(B), dev(la)
+    gb = torch.zeros(K, N, device="cuda")
+    ga = torch.zeros(M, K, device="cuda")
+    assert lib.amr_lut_gemm_backward_f32tab(gd.data_ptr(), a.data_ptr(), b.data_ptr(), None, gb.data_ptr(), None, t.data_ptr(),
+                                            t.numel(), 0.25, M, K, N, 0, None, 0, None) == 0
+    assert lib.amr_lut_gemm_backward_f32tab(gd.data_ptr(), a.data_ptr(), b.data_ptr(), ga.data_ptr(), None, t.data_ptr(), None,
+                                            t.numel(), 0.25, M, K, N, 0, None, 0, None) == 0
+    torch.cuda.synchronize()
+    assert (gb.cpu().numpy() == r1[1]).all() and (ga.cpu().numpy() == r1[0]).all()
+
+
 def test_backward_float_tables_expanded_gradA_masked_codes(lib, oracle):
     print("backward float tables, expanded gradA with masked codes", flush=True)
     M, K, N = 4224, 32, 64
