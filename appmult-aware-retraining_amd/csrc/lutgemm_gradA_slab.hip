@@ -125,18 +125,18 @@ __global__ __launch_bounds__(256) void expand_gradA_f32_kernel(const uint8_t* __
 // ------------------------------------------------------------------------------------------ consume
 // One 128-bit LDS read of a chunk, issued and NOT waited for.  The address comes out of ONE v_perm_b32:
 // byte 0 = the lane's constant (window and piece), byte 1 = the code (BYTE of codeword; < 128), byte 2 = 1 for
-// the third buffer (byte 3 of the lane's constant holds that 1), the second buffer goes into the offset field.
+// the third and fourth buffer (byte 3 of the lane's constant holds that 1), the odd buffers go into the offset field.
 // Inline assembly: the compiler must not make these reads wait for the LDS-direct loads that fill the other
 // buffers (same LDS array to it).
 template <int BYTE, int BUF>
 __device__ __forceinline__ void ga_read(u32x4& d, uint32_t codeword, uint32_t lane_const) {
-    constexpr uint32_t sel = (BUF == 2 ? 0x0c030000u : 0x0c020000u) | ((4u + BYTE) << 8);
+    constexpr uint32_t sel = (BUF >= 2 ? 0x0c030000u : 0x0c020000u) | ((4u + BYTE) << 8);
     uint32_t addr;
     // (the address computation sits inside the volatile block so that it stays where it is used: computed ahead
     // of the loop, as the compiler would, the addresses of all reads of a workgroup occupy registers that do not exist)
     asm volatile("v_perm_b32 %1, %2, %3, %4\n ds_read_b128 %0, %1 offset:%5"
                  : "=v"(d), "=&v"(addr)
-                 : "v"(codeword), "v"(lane_const), "s"(sel), "n"(BUF == 1 ? kGaChunkBytes : 0)
+                 : "v"(codeword), "v"(lane_const), "s"(sel), "n"((BUF & 1) ? kGaChunkBytes : 0)
                  : "memory");
 }
 
@@ -151,7 +151,15 @@ __global__ __launch_bounds__(kGaWaves * 64) void lutgemm_gradA_slab_kernel(
     uint32_t* __restrict__ flags, int M, int K, int N, float scale, int rows_per_image, int row_blocks, int band_rows_max) {
     __shared__ __align__(16) unsigned char smem[kGaStageBase + kGaStageBytes];
     constexpr int CH = kGaKT / kGaChunkK;                  // chunks per column tile
-    constexpr int NTU = (CH % kGaBufs) == 0 ? 1 : kGaBufs; // column tiles per unrolled pass: the buffer of a chunk is then static
+    // Chunk buffers: three, requested two chunks ahead; with float32 entries the staging area is half the size and a fourth
+    // buffer fits: three chunks ahead (the loop is bound by the delivery of the chunks, 36 KB per 32 K multiply-adds).
+    constexpr int BUFS = F32 ? 4 : kGaBufs;
+    constexpr int DIST = BUFS - 1;                         // chunks between a request and its use
+    constexpr int OUT = 2 * (DIST - 1);                    // chunk operations issued after the request of the chunk a step needs
+    constexpr int STAGE_BASE = BUFS * kGaChunkBytes;
+    static_assert(STAGE_BASE + kGaRows * (F32 ? kGaColsF32 : kGaCols) * 4 <= kGaStageBase + kGaStageBytes, "LDS budget");
+    constexpr int NTU = (CH % BUFS) == 0 ? 1 : BUFS;       // column tiles per unrolled pass: the buffer of a chunk is then static
+    static_assert(NTU == 1 || NTU == 3, "the tile loop below unrolls one or three column tiles");
     constexpr int NST = 2 * CH;                            // stores per lane at the end of a tile
     constexpr int COLS = F32 ? kGaColsF32 : kGaCols;       // columns per tile
     constexpr int STAGE_WAVE = kGaRowsPerWave * COLS * 4;  // bytes of gC rows a wave stages per column tile (4 KB / 2 KB)
@@ -235,7 +243,7 @@ __global__ __launch_bounds__(kGaWaves * 64) void lutgemm_gradA_slab_kernel(
 #pragma unroll
         for (int i = 0; i < ROWOPS; ++i)
             __builtin_amdgcn_global_load_lds((gptr_t)(base + (size_t)(RPO * i) * N + glane),
-                                             (lptr_t)(smem + kGaStageBase + wave * STAGE_WAVE + i * 1024), 16, 0, 0);
+                                             (lptr_t)(smem + STAGE_BASE + wave * STAGE_WAVE + i * 1024), 16, 0, 0);
     };
     // The codes of a tile: A[m][k0 + 4 j + c], one byte per chunk and row, packed four to a register.  Assembly loads:
     // the waiting is explicit (the compiler would wait for everything in flight).
@@ -279,16 +287,17 @@ __global__ __launch_bounds__(kGaWaves * 64) void lutgemm_gradA_slab_kernel(
         for (int i = 0; i < COLS; ++i) g[r][i] = 0.f;
     float row_sum[2] = {0.f, 0.f};
     u32x4 d[4] = {{0, 0, 0, 0}, {0, 0, 0, 0}, {0, 0, 0, 0}, {0, 0, 0, 0}};
+    u32x4 e[4] = {{0, 0, 0, 0}, {0, 0, 0, 0}, {0, 0, 0, 0}, {0, 0, 0, 0}};      // float32 entries: the second half of a chunk's reads
 
     // Operations of a wave towards memory, in issue order (vmcnt counts them in this order):
-    //   rows(0) chunk(0) chunk(1) codes | step q: chunk(q + 2); second step of column tile nt also: rows(nt + 1)
+    //   rows(0) chunk(0) .. chunk(DIST - 1) codes | step q: chunk(q + DIST); second step of column tile nt also: rows(nt + 1)
     //   | end of a tile: codes of the next tile, NST stores | ...
     // (a chunk request is two operations, a row request ROWOPS = four, two with float32 entries).  At the top of step q, chunk q (requested two steps
     // earlier) must have landed: all but the requests of the previous step may be outstanding; in the first two
     // steps of a tile the stores of the previous one as well.
     request_rows(0);
-    request_chunk(0, 0);
-    request_chunk(1, 1);
+#pragma unroll
+    for (int i = 0; i < DIST; ++i) request_chunk(i, i);
     {
         uint32_t raw[2][CH];
         load_codes(cur, raw);
@@ -344,13 +353,55 @@ __global__ __launch_bounds__(kGaWaves * 64) void lutgemm_gradA_slab_kernel(
         if (KC < 2 && nt == 0 && after_stores) {
             if (KC == 0) asm volatile("s_waitcnt vmcnt(%2)\n s_barrier" : "+v"(d[2]), "+v"(d[3]) : "n"(NST) : "memory");
             else asm volatile("s_waitcnt vmcnt(%2)\n s_barrier" : "+v"(d[2]), "+v"(d[3]) : "n"(NST + 2) : "memory");
-        } else if (KC == 2 || KC == 3) {
-            asm volatile("s_waitcnt vmcnt(%2)\n s_barrier" : "+v"(d[2]), "+v"(d[3]) : "n"(2 + ROWOPS) : "memory");
+        } else if (KC >= 2 && KC <= DIST + 1) {
+            // the row request of step 1 was issued after the request of the chunk this step needs
+            asm volatile("s_waitcnt vmcnt(%2)\n s_barrier" : "+v"(d[2]), "+v"(d[3]) : "n"(OUT + ROWOPS) : "memory");
         } else {
-            asm volatile("s_waitcnt vmcnt(2)\n s_barrier" : "+v"(d[2]), "+v"(d[3]) : : "memory");
+            asm volatile("s_waitcnt vmcnt(%2)\n s_barrier" : "+v"(d[2]), "+v"(d[3]) : "n"(OUT) : "memory");
         }
-        request_chunk(q + 2, (BUF + 2) % kGaBufs);
+        request_chunk(q + DIST, (BUF + DIST) % BUFS);
         if (KC == 1) request_rows(nt + 1);
+        if constexpr (F32) {
+            // float32 entries: a read feeds four multiply-adds only, so the loop is bound by the latency of the LDS, not by
+            // arithmetic: all eight reads of the chunk are issued at once (the registers are there: 16 values of gC per row
+            // instead of 32) and consumed in order; nothing is carried over the barrier.
+            if (KC == 0) {
+                const uint32_t gbase = (uint32_t)(STAGE_BASE + wave * STAGE_WAVE + quad * (COLS * 4));
+#pragma unroll
+                for (int r = 0; r < 2; ++r) {
+                    u32x4 t[4];
+#pragma unroll
+                    for (int s4 = 0; s4 < 4; ++s4) {
+                        const uint32_t ga = gbase + (uint32_t)(((quad + s4) & 3) << 4);
+                        if (r == 0) asm volatile("ds_read_b128 %0, %1" : "=&v"(t[s4]) : "v"(ga) : "memory");
+                        else asm volatile("ds_read_b128 %0, %1 offset:1024" : "=&v"(t[s4]) : "v"(ga) : "memory");
+                    }
+                    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(t[0]), "+v"(t[1]), "+v"(t[2]), "+v"(t[3]) : : "memory");
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const f32x4 v = __builtin_bit_cast(f32x4, t[i]);
+                        g[r][4 * i] = v.x; g[r][4 * i + 1] = v.y; g[r][4 * i + 2] = v.z; g[r][4 * i + 3] = v.w;
+                    }
+                }
+            }
+            ga_read<KC & 3, BUF>(d[0], codes[0][KC >> 2], lane_const[0]);
+            ga_read<KC & 3, BUF>(d[1], codes[1][KC >> 2], lane_const[0]);
+            ga_read<KC & 3, BUF>(d[2], codes[0][KC >> 2], lane_const[1]);
+            ga_read<KC & 3, BUF>(d[3], codes[1][KC >> 2], lane_const[1]);
+            ga_read<KC & 3, BUF>(e[0], codes[0][KC >> 2], lane_const[2]);
+            ga_read<KC & 3, BUF>(e[1], codes[1][KC >> 2], lane_const[2]);
+            ga_read<KC & 3, BUF>(e[2], codes[0][KC >> 2], lane_const[3]);
+            ga_read<KC & 3, BUF>(e[3], codes[1][KC >> 2], lane_const[3]);
+            asm volatile("s_waitcnt lgkmcnt(6)" : "+v"(d[0]), "+v"(d[1]) : : "memory");
+            pair_fma(kc_tag, std::integral_constant<int, 0>{}, d[0], d[1]);
+            asm volatile("s_waitcnt lgkmcnt(4)" : "+v"(d[2]), "+v"(d[3]) : : "memory");
+            pair_fma(kc_tag, std::integral_constant<int, 1>{}, d[2], d[3]);
+            asm volatile("s_waitcnt lgkmcnt(2)" : "+v"(e[0]), "+v"(e[1]) : : "memory");
+            pair_fma(kc_tag, std::integral_constant<int, 2>{}, e[0], e[1]);
+            asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(e[2]), "+v"(e[3]) : : "memory");
+            pair_fma(kc_tag, std::integral_constant<int, 3>{}, e[2], e[3]);
+            return;
+        }
         __builtin_amdgcn_s_setprio(3);
         ga_read<KC & 3, BUF>(d[0], codes[0][KC >> 2], lane_const[0]);
         ga_read<KC & 3, BUF>(d[1], codes[1][KC >> 2], lane_const[0]);
@@ -359,7 +410,7 @@ __global__ __launch_bounds__(kGaWaves * 64) void lutgemm_gradA_slab_kernel(
         ga_read<KC & 3, BUF>(d[3], codes[1][KC >> 2], lane_const[1]);
         if (KC == 0) {
             // new column tile: the rows of gC from the staging area, pieces in this lane's rotated order
-            const uint32_t gbase = (uint32_t)(kGaStageBase + wave * STAGE_WAVE + quad * (COLS * 4));
+            const uint32_t gbase = (uint32_t)(STAGE_BASE + wave * STAGE_WAVE + quad * (COLS * 4));
 #pragma unroll
             for (int r = 0; r < 2; ++r) {
                 if constexpr (F32) {
@@ -425,8 +476,10 @@ __global__ __launch_bounds__(kGaWaves * 64) void lutgemm_gradA_slab_kernel(
     // End of a tile: last multiply-adds, the codes of the next tile are asked for, gA of this one is stored meanwhile.
     // Returns false when the workgroup has no further tile.
     auto finish_tile = [&]() __attribute__((always_inline)) {
-        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(d[2]), "+v"(d[3]) : : "memory");
-        pair_fma(std::integral_constant<int, CH - 1>{}, std::integral_constant<int, 3>{}, d[2], d[3]);
+        if constexpr (!F32) {
+            asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(d[2]), "+v"(d[3]) : : "memory");
+            pair_fma(std::integral_constant<int, CH - 1>{}, std::integral_constant<int, 3>{}, d[2], d[3]);
+        }
         uint32_t raw[2][CH];
         if (nxt.valid) load_codes(nxt, raw);
         const int m_base = m_base_of(cur);
@@ -491,7 +544,7 @@ __global__ __launch_bounds__(kGaWaves * 64) void lutgemm_gradA_slab_kernel(
     auto tile_step = [&](auto j_tag) __attribute__((always_inline)) {
         constexpr int J = decltype(j_tag)::value;
         [&]<int... KC>(std::integer_sequence<int, KC...>) {
-            (chunk_step(nt, std::integral_constant<int, KC>{}, std::integral_constant<int, (J * CH + KC) % kGaBufs>{}), ...);
+            (chunk_step(nt, std::integral_constant<int, KC>{}, std::integral_constant<int, (J * CH + KC) % BUFS>{}), ...);
         }(std::make_integer_sequence<int, CH>{});
         if (++nt < n_tiles) return true;
         nt = 0;
