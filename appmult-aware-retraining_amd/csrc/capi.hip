@@ -44,6 +44,7 @@ hipError_t launch_im2col_u8_f32(const float* x, uint8_t* A, int B, int C, int H,
                                 int dil, int oh, int ow, hipStream_t stream);
 bool bwd_slab_applies(const LutGeom& g, int M, int K, int N);
 int gradB_slab_splits(int M, int K, int N, int n_cu);
+size_t gradB_slab_colsum_floats(int N);
 hipError_t launch_gradB_slab(const float* gC, const uint8_t* A, const uint8_t* B, float* gB, const int16_t* lut,
                              const LutGeom& g, int M, int K, int N, float scale, uint32_t* flags, float* partials,
                              int n_cu, hipStream_t stream);
@@ -220,7 +221,7 @@ int amr_lut_gemm_forward(const uint8_t* A, const uint8_t* B, uint32_t* C, const 
 static size_t backward_partial_bytes(int M, int K, int N, int n_cu) {
     size_t direct = amr::gradB_workspace_bytes(M, K, N, n_cu);
     const int s = amr::gradB_slab_splits(M, K, N, n_cu);
-    size_t slab = s > 1 ? (size_t)s * K * N * sizeof(float) : 0;
+    size_t slab = (s > 1 ? (size_t)s * K * N * sizeof(float) : 0) + amr::gradB_slab_colsum_floats(N) * sizeof(float);
     const size_t b = direct > slab ? direct : slab;
     return (b + 255) & ~(size_t)255;
 }

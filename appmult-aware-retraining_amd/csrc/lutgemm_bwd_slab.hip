@@ -228,11 +228,12 @@ __global__ __launch_bounds__(1024) void lutgemm_gradB_slab_kernel(
 // Requires K % 8 == 0, N % 64 == 0, row counts that are multiples of the rows per iteration, gC 16-byte
 // aligned and 32-bit offsets (the launcher checks).
 constexpr int kBwdKT16 = 8;
+constexpr int kBwdColsumSplits = 64;      // the most M splits the launcher picks
 
 __global__ __launch_bounds__(1024) void lutgemm_gradB_slab16_kernel(
     const float* __restrict__ gC, const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, float* __restrict__ out,
     const int16_t* __restrict__ G, int lut_cols, int n_codes, uint32_t* __restrict__ flags, int M, int K, int N,
-    int m_chunk, float scale, int n_tiles, int k_tiles, int splits) {
+    int m_chunk, float scale, int n_tiles, int k_tiles, int splits, float* __restrict__ colsum) {
     constexpr int KT = kBwdKT16;
     __shared__ __align__(16) unsigned char smem[KT * 16384 + 32768];     // slabs + the table as halves
     const int tid = threadIdx.x;
@@ -385,8 +386,11 @@ __global__ __launch_bounds__(1024) void lutgemm_gradB_slab16_kernel(
             }
         }
     };
-    // (two copies of the loop: without the column sums of gC when the table is stored without offset)
-    if (offset != 0.f) stream_rows(std::true_type{}); else stream_rows(std::false_type{});
+    // (two copies of the loop.  The column sums of gC, needed to undo a non-zero offset, are the same for all k tiles
+    // of a (column tile, M split): only the workgroup of k tile 0 forms them (4 % more work in its loop) and leaves them
+    // in colsum[split][n]; gradB_finish_kernel adds offset * colsum to every k afterwards.)
+    const bool do_sums = offset != 0.f && k_tile == 0;
+    if (do_sums) stream_rows(std::true_type{}); else stream_rows(std::false_type{});
     if (__builtin_amdgcn_ballot_w64((seen & 0x80808080u) != 0) != 0) {
         if (lane == 0) atomicOr(&flags[1], 1u);
     }
@@ -419,8 +423,30 @@ __global__ __launch_bounds__(1024) void lutgemm_gradB_slab16_kernel(
             v += red[(w * (KT + 1) + kk) * 64 + col];
             gs += red[(w * (KT + 1) + KT) * 64 + col];
         }
-        out[((size_t)split * K + k0 + kk) * N + n0 + col] = (v + offset * gs) * scale;
+        out[((size_t)split * K + k0 + kk) * N + n0 + col] = v * scale;
+        if (do_sums && kk == 0) colsum[(size_t)split * N + n0 + col] = gs;
     }
+}
+
+// gB[k][n] = sum over the M splits of the partial results (fixed order) + scale * offset * sum over the splits of the
+// column sums of gC (offset = flags[4]; nothing to add for offset 0).  partial == nullptr: one split, the kernel wrote gB itself.
+__global__ __launch_bounds__(256) void gradB_finish_kernel(const float* __restrict__ partial, float* __restrict__ gB,
+                                                           const float* __restrict__ colsum, const uint32_t* __restrict__ flags,
+                                                           int K, int N, int splits, float scale) {
+    const float offset = (float)flags[4];
+    if (partial == nullptr && offset == 0.f) return;
+    const size_t count = (size_t)K * N;
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= count) return;
+    const int n = (int)(i % (size_t)N);
+    float v = partial ? partial[i] : gB[i];
+    for (int p = 1; p < splits && partial; ++p) v += partial[(size_t)p * count + i];
+    if (offset != 0.f) {
+        float cs = colsum[n];
+        for (int p = 1; p < splits; ++p) cs += colsum[(size_t)p * N + n];
+        v += scale * offset * cs;
+    }
+    gB[i] = v;
 }
 
 // ------------------------------------------------------------------------------------------ scratch header
@@ -489,6 +515,9 @@ hipError_t launch_gradB_gated(const float* gC, const uint8_t* A, const uint8_t* 
                               const LutGeom& g, int M, int K, int N, float scale, const uint32_t* gate, hipStream_t stream);
 __global__ void reduce_partials_kernel(const float* __restrict__ partial, float* __restrict__ out, size_t count, int splits);
 
+// Floats of scratch the half-slab kernel keeps in front of its partial results (column sums of gC per M split).
+size_t gradB_slab_colsum_floats(int N) { return kBwdColsumSplits * (size_t)N; }
+
 bool bwd_slab_applies(const LutGeom& g, int M, int K, int N) {
     (void)N;
     // (measured cross-over against the direct kernel on MI355X: between 512 and 1024 rows)
@@ -537,9 +566,21 @@ hipError_t launch_gradB_slab(const float* gC, const uint8_t* A, const uint8_t* B
     float* out = zs > 1 ? partials : gB;
     dim3 grid((N + 63) / 64, (K + kt - 1) / kt, zs);
     if (half_slab) {
+        // scratch of this kernel: [column sums of gC: 64 splits x N][partial results]
+        float* colsum = partials;
+        float* part16 = partials + kBwdColsumSplits * (size_t)N;
+        out = zs > 1 ? part16 : gB;
         const int total = (int)(grid.x * grid.y * grid.z);
         hipLaunchKernelGGL(lutgemm_gradB_slab16_kernel, dim3(8 * ((total + 7) / 8)), dim3(1024), 0, stream, gC, A, B, out, lut, g.cols,
-                           1 << g.bits, flags, M, K, N, m_chunk, scale, (int)grid.x, (int)grid.y, (int)grid.z);
+                           1 << g.bits, flags, M, K, N, m_chunk, scale, (int)grid.x, (int)grid.y, (int)grid.z, colsum);
+        hipError_t e16 = hipGetLastError();
+        if (e16 != hipSuccess) return e16;
+        const size_t count = (size_t)K * N;
+        hipLaunchKernelGGL(gradB_finish_kernel, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, stream,
+                           zs > 1 ? (const float*)part16 : (const float*)nullptr, gB, colsum, flags, K, N, zs, scale);
+        e16 = hipGetLastError();
+        if (e16 != hipSuccess) return e16;
+        return launch_gradB_gated(gC, A, B, gB, lut, g, M, K, N, scale, flags + 1, stream);
     }
     else if (regular && (K & 3) == 0)
         hipLaunchKernelGGL((lutgemm_gradB_slab_kernel<true, int16_t>), grid, dim3(1024), 0, stream, gC, A, B, out, lut, g.cols, 1 << g.bits,
