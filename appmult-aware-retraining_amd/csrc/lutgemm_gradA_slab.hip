@@ -285,7 +285,10 @@ __global__ __launch_bounds__(kGaWaves * 64) void lutgemm_gradA_slab_kernel(
     for (int r = 0; r < 2; ++r)
 #pragma unroll
         for (int i = 0; i < COLS; ++i) g[r][i] = 0.f;
+    // sums of the lane's rows of gC over all columns (to undo a non-zero offset): formed during the first tile a workgroup
+    // walks on a block of rows and kept while its next tiles stay on the same rows (with the order above, every other k group)
     float row_sum[2] = {0.f, 0.f};
+    bool sum_rows = offset != 0.f;
     u32x4 d[4] = {{0, 0, 0, 0}, {0, 0, 0, 0}, {0, 0, 0, 0}, {0, 0, 0, 0}};
     u32x4 e[4] = {{0, 0, 0, 0}, {0, 0, 0, 0}, {0, 0, 0, 0}, {0, 0, 0, 0}};      // float32 entries: the second half of a chunk's reads
 
@@ -450,7 +453,7 @@ __global__ __launch_bounds__(kGaWaves * 64) void lutgemm_gradA_slab_kernel(
                         g[r][16 * hf + 4 * i] = v.x; g[r][16 * hf + 4 * i + 1] = v.y; g[r][16 * hf + 4 * i + 2] = v.z; g[r][16 * hf + 4 * i + 3] = v.w;
                     }
                 }
-                if (offset != 0.f) {
+                if (sum_rows) {
                     float s = row_sum[r];
 #pragma unroll
                     for (int i = 0; i < COLS; ++i) s += g[r][i];
@@ -528,9 +531,11 @@ __global__ __launch_bounds__(kGaWaves * 64) void lutgemm_gradA_slab_kernel(
             for (int j = 0; j < CH; ++j) asm volatile("" : "+v"(raw[r][j]));
         pack_codes(raw);
         after_stores = whole;
+        const bool same_rows = nxt.m_wave == cur.m_wave;
+        sum_rows = offset != 0.f && !same_rows;
 #pragma unroll
         for (int r = 0; r < 2; ++r) {
-            row_sum[r] = 0.f;
+            if (!same_rows) row_sum[r] = 0.f;
 #pragma unroll
             for (int j = 0; j < CH; ++j) acc[r][j] = 0.f;
         }
