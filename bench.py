@@ -48,7 +48,7 @@ HBM_PEAK = 8.0e12
 
 
 # measured on MI355X with the counters named above, bytes per conv2_x launch (read + written)
-MEASURED_TRAFFIC_CONV2X = {"forward": (337 + 65) * 2**20, "gradA": (1162 + 576) * 2**20, "gradB": (443 + 1) * 2**20}
+MEASURED_TRAFFIC_CONV2X = {"forward": (337 + 65) * 2**20, "gradA": (1146 + 576) * 2**20, "gradB": (450 + 1) * 2**20}
 
 
 def main():
