@@ -56,10 +56,19 @@ __global__ __launch_bounds__(256) void expand_fwd_kernel(const uint8_t* __restri
     extern __shared__ __align__(16) unsigned char smem[];
     uint32_t* s32 = reinterpret_cast<uint32_t*>(smem);
     uint32_t mx = 0;
-    for (int i = threadIdx.x; i < lut_dwords; i += 256) {
-        const uint32_t v = lut32[i];
-        s32[i] = v;
-        mx = max(mx, max(v & 0xffffu, v >> 16));
+    // (eight loads of a thread in flight before the first is stored: a load-wait-store loop pays the memory latency 33 times)
+    for (int base = 0; base < lut_dwords; base += 8 * 256) {
+        uint32_t v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = lut32[min(base + u * 256 + (int)threadIdx.x, lut_dwords - 1)];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int i = base + u * 256 + (int)threadIdx.x;
+            if (i < lut_dwords) {
+                s32[i] = v[u];
+                mx = max(mx, max(v[u] & 0xffffu, v[u] >> 16));
+            }
+        }
     }
     __syncthreads();
     if (blockIdx.x == 0 && blockIdx.y == 0) {

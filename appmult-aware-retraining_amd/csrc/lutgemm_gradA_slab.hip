@@ -68,12 +68,22 @@ __global__ __launch_bounds__(256) void expand_gradA_kernel(const uint8_t* __rest
     // reads, one shift-or and the store (the kernel writes 256 B per code and k quad and should run at the speed of
     // the writes: 6.8 TB/s measured for a plain fill).
     bool inexact = false;
-    for (int i = threadIdx.x; i < lut_dwords; i += 256) {
-        const uint32_t w = lut32[i];
-        const float v0 = (float)(int16_t)(w & 0xffffu) - offset, v1 = (float)(int16_t)(w >> 16) - offset;
-        const _Float16 h0 = (_Float16)v0, h1 = (_Float16)v1;
-        inexact |= ((float)h0 != v0) | ((float)h1 != v1);
-        s32[i] = (uint32_t)__builtin_bit_cast(uint16_t, h0) | ((uint32_t)__builtin_bit_cast(uint16_t, h1) << 16);
+    // (eight loads of a thread in flight before the first is converted and stored)
+    for (int base = 0; base < lut_dwords; base += 8 * 256) {
+        uint32_t w8[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) w8[u] = lut32[min(base + u * 256 + (int)threadIdx.x, lut_dwords - 1)];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int i = base + u * 256 + (int)threadIdx.x;
+            const uint32_t w = w8[u];
+            const float v0 = (float)(int16_t)(w & 0xffffu) - offset, v1 = (float)(int16_t)(w >> 16) - offset;
+            const _Float16 h0 = (_Float16)v0, h1 = (_Float16)v1;
+            if (i < lut_dwords) {
+                inexact |= ((float)h0 != v0) | ((float)h1 != v1);
+                s32[i] = (uint32_t)__builtin_bit_cast(uint16_t, h0) | ((uint32_t)__builtin_bit_cast(uint16_t, h1) << 16);
+            }
+        }
     }
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     if (__builtin_amdgcn_ballot_w64(inexact) != 0 && lane == 0) atomicOr(&flags[2], 1u);
