@@ -83,14 +83,22 @@ __global__ __launch_bounds__(256) void expand_fwd_kernel(const uint8_t* __restri
     // 16-bit LDS reads, one shift-or, the store (the kernel should run at the speed of its writes).  Positions
     // beyond K or N and codes beyond the table read the table's all-zero pad column / pad row.
     const int kk = lane >> 4, n = blockIdx.x * kSlabCols + 2 * (lane & 15);
+    // the codes of B for all k quads of the workgroup first (one trip to memory instead of one per quad)
+    int b0[kExpandQuadsPerWg], b1[kExpandQuadsPerWg];
+#pragma unroll
+    for (int qq = 0; qq < kExpandQuadsPerWg; ++qq) {
+        const int k = 4 * (blockIdx.y * kExpandQuadsPerWg + qq) + kk;
+        const bool live0 = (k < K) && (n < N), live1 = (k < K) && (n + 1 < N);
+        b0[qq] = live0 ? (int)B[(size_t)k * N + n] : n_codes;
+        b1[qq] = live1 ? (int)B[(size_t)k * N + n + 1] : n_codes;
+    }
+#pragma unroll
     for (int qq = 0; qq < kExpandQuadsPerWg; ++qq) {
         const int q = blockIdx.y * kExpandQuadsPerWg + qq;
         if (q >= k_quads) break;
         uint32_t* blk = E + ((size_t)blockIdx.x * k_quads + q) * (kSlabChunkBytes / 4) + lane;
-        const int k = 4 * q + kk;
-        const bool live0 = (k < K) && (n < N), live1 = (k < K) && (n + 1 < N);
-        const uint16_t* p0 = s16 + (live0 ? (int)B[(size_t)k * N + n] : n_codes);
-        const uint16_t* p1 = s16 + (live1 ? (int)B[(size_t)k * N + n + 1] : n_codes);
+        const uint16_t* p0 = s16 + b0[qq];
+        const uint16_t* p1 = s16 + b1[qq];
 #pragma unroll 8
         for (int a = wave; a < kSlabRows; a += 4) {
             const int row = min(a, n_codes) * lut_cols;

@@ -92,13 +92,22 @@ __global__ __launch_bounds__(256) void expand_gradA_kernel(const uint8_t* __rest
     // a wave writes the 256 B row of one code: lane = (k % 4, column pair), one dword (two columns) per lane
     const int ks = lane >> 4, cp = lane & 15;
     const int n = blockIdx.x * kGaCols + 2 * cp;
-    for (int pp = 0; pp < quads_per_wg; ++pp) {
+    // the codes of B for all k quads of the workgroup first (one trip to memory instead of one per quad)
+    constexpr int kMaxQuads = 4;
+    uint16_t bpair[kMaxQuads];
+#pragma unroll
+    for (int pp = 0; pp < kMaxQuads; ++pp) {
+        const int kq = min(blockIdx.y * quads_per_wg + min(pp, quads_per_wg - 1), K / 4 - 1);
+        const uint8_t* bp = B + (size_t)(4 * kq + ks) * N + n;
+        bpair[pp] = (uint16_t)((uint32_t)bp[0] | ((uint32_t)bp[1] << 8));
+    }
+#pragma unroll
+    for (int pp = 0; pp < kMaxQuads; ++pp) {
+        if (pp >= quads_per_wg) break;
         const int kq = blockIdx.y * quads_per_wg + pp;
         if (4 * kq >= K) break;
-        const int k = 4 * kq + ks;
-        const uint8_t* bp = B + (size_t)k * N + n;
-        const uint16_t* p0 = s16 + (int)bp[0];
-        const uint16_t* p1 = s16 + (int)bp[1];
+        const uint16_t* p0 = s16 + (int)(bpair[pp] & 0xffu);
+        const uint16_t* p1 = s16 + (int)(bpair[pp] >> 8);
         uint32_t* chunk = S + ((size_t)blockIdx.x * (K / 4) + kq) * (kGaChunkBytes / 4) + lane;
 #pragma unroll 8
         for (int a = wave; a < 128; a += 4) {
