@@ -131,10 +131,20 @@ __global__ __launch_bounds__(256) void expand_gradA_f32_kernel(const uint8_t* __
     // a wave writes the 256 B row of one code: lane = (k % 4, column), one dword per lane
     const int ks = lane >> 4, col = lane & 15;
     const int n = blockIdx.x * kGaColsF32 + col;
-    for (int pp = 0; pp < quads_per_wg; ++pp) {
+    // (the codes of B for all k quads of the workgroup first)
+    constexpr int kMaxQuads = 4;
+    int bcode[kMaxQuads];
+#pragma unroll
+    for (int pp = 0; pp < kMaxQuads; ++pp) {
+        const int kq = min(blockIdx.y * quads_per_wg + min(pp, quads_per_wg - 1), K / 4 - 1);
+        bcode[pp] = (int)B[(size_t)(4 * kq + ks) * N + n];
+    }
+#pragma unroll
+    for (int pp = 0; pp < kMaxQuads; ++pp) {
+        if (pp >= quads_per_wg) break;
         const int kq = blockIdx.y * quads_per_wg + pp;
         if (4 * kq >= K) break;
-        const uint32_t* p0 = s32 + (int)B[(size_t)(4 * kq + ks) * N + n];
+        const uint32_t* p0 = s32 + bcode[pp];
         uint32_t* chunk = S + ((size_t)blockIdx.x * (K / 4) + kq) * (kGaChunkBytes / 4) + lane;
 #pragma unroll 8
         for (int a = wave; a < 128; a += 4) chunk[a * 64] = p0[min(a, n_codes) * lut_cols];
