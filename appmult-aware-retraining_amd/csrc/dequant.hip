@@ -8,7 +8,8 @@
 // The operations and their order are those of the torch expression this replaces (every product and sum rounded on
 // its own, no fused multiply-add), so the values are bit-identical to it.  The backward kernel is the transpose back
 // with the scale: g_c[m,n] = (s_a*s_w) * g[b,n,pos].
-// Both go through a 32 x 32 LDS tile so that reads run along n (rows of c) and writes along pos (NCHW), or the reverse.
+// Both go through 32 x 32 LDS tiles so that reads run along n (rows of c) and writes along pos (NCHW), or the reverse; a
+// workgroup takes four such tiles along m and issues the 16 loads of a thread before the first is used.
 #include "amr_common.h"
 
 namespace amr {
@@ -17,30 +18,42 @@ __global__ __launch_bounds__(256) void dequant_rows_to_nchw_kernel(
     const float* __restrict__ c, const float* __restrict__ xs, const float* __restrict__ wr, const float* __restrict__ tp,
     const float* __restrict__ za_p, const float* __restrict__ zw_p, const float* __restrict__ sa_p, const float* __restrict__ sw_p,
     const float* __restrict__ bias, float* __restrict__ out, int M, int N, int L) {
-    __shared__ float tile[32][33];
+    __shared__ float tile[4][32][33];
     const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
-    const int m0 = blockIdx.x * 32, n0 = blockIdx.y * 32;
-#pragma unroll
-    for (int r = 0; r < 4; ++r) {
-        const int m = m0 + ty + 8 * r, n = n0 + tx;
-        if (m < M && n < N) tile[ty + 8 * r][tx] = c[(size_t)m * N + n];
-    }
-    __syncthreads();
+    const int m0 = blockIdx.x * 128, n0 = blockIdx.y * 32;
     const float za = *za_p, zw = *zw_p;
     const float s = __fmul_rn(*sa_p, *sw_p), zz = __fmul_rn(za, zw);
-    const int m = m0 + tx;
-    if (m >= M) return;
-    const int b = m / L, pos = m - b * L;
-    const float x_term = __fmul_rn(zw, xs[m]);
-    const float t_term = __fmul_rn(zz, tp[pos]);
+    {
+        float v[4][4];
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
-        const int n = n0 + ty + 8 * r;
-        if (n < N) {
-            const float terms = __fadd_rn(__fadd_rn(x_term, __fmul_rn(za, wr[(size_t)n * L + pos])), t_term);
-            float v = __fmul_rn(s, __fadd_rn(tile[tx][ty + 8 * r], terms));
-            if (bias != nullptr) v = __fadd_rn(v, bias[n]);
-            out[((size_t)b * N + n) * L + pos] = v;
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int m = min(m0 + 32 * t + ty + 8 * r, M - 1), n = min(n0 + tx, N - 1);
+                v[t][r] = c[(size_t)m * N + n];
+            }
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) tile[t][ty + 8 * r][tx] = v[t][r];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+        const int m = m0 + 32 * t + tx;
+        if (m >= M) break;
+        const int b = m / L, pos = m - b * L;
+        const float x_term = __fmul_rn(zw, xs[m]);
+        const float t_term = __fmul_rn(zz, tp[pos]);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int n = n0 + ty + 8 * r;
+            if (n < N) {
+                const float terms = __fadd_rn(__fadd_rn(x_term, __fmul_rn(za, wr[(size_t)n * L + pos])), t_term);
+                float v = __fmul_rn(s, __fadd_rn(tile[t][tx][ty + 8 * r], terms));
+                if (bias != nullptr) v = __fadd_rn(v, bias[n]);
+                out[((size_t)b * N + n) * L + pos] = v;
+            }
         }
     }
 }
@@ -48,38 +61,46 @@ __global__ __launch_bounds__(256) void dequant_rows_to_nchw_kernel(
 __global__ __launch_bounds__(256) void dequant_grad_nchw_to_rows_kernel(const float* __restrict__ g, const float* __restrict__ sa_p,
                                                                         const float* __restrict__ sw_p, float* __restrict__ gc,
                                                                         int M, int N, int L) {
-    __shared__ float tile[32][33];
+    __shared__ float tile[4][32][33];
     const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
-    const int m0 = blockIdx.x * 32, n0 = blockIdx.y * 32;
+    const int m0 = blockIdx.x * 128, n0 = blockIdx.y * 32;
     const float s = __fmul_rn(*sa_p, *sw_p);
     {
-        const int m = m0 + tx;
-        if (m < M) {
+        float v[4][4];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const int m = min(m0 + 32 * t + tx, M - 1);
             const int b = m / L, pos = m - b * L;
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                const int n = n0 + ty + 8 * r;
-                if (n < N) tile[tx][ty + 8 * r] = __fmul_rn(s, g[((size_t)b * N + n) * L + pos]);
+                const int n = min(n0 + ty + 8 * r, N - 1);
+                v[t][r] = g[((size_t)b * N + n) * L + pos];
             }
         }
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) tile[t][tx][ty + 8 * r] = __fmul_rn(s, v[t][r]);
     }
     __syncthreads();
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
-        const int m = m0 + ty + 8 * r, n = n0 + tx;
-        if (m < M && n < N) gc[(size_t)m * N + n] = tile[ty + 8 * r][tx];
-    }
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int m = m0 + 32 * t + ty + 8 * r, n = n0 + tx;
+            if (m < M && n < N) gc[(size_t)m * N + n] = tile[t][ty + 8 * r][tx];
+        }
 }
 
 hipError_t launch_dequant(const float* c, const float* xs, const float* wr, const float* tp, const float* za, const float* zw,
                           const float* sa, const float* sw, const float* bias, float* out, int M, int N, int L, hipStream_t stream) {
-    hipLaunchKernelGGL(dequant_rows_to_nchw_kernel, dim3((M + 31) / 32, (N + 31) / 32), dim3(256), 0, stream, c, xs, wr, tp, za, zw, sa,
+    hipLaunchKernelGGL(dequant_rows_to_nchw_kernel, dim3((M + 127) / 128, (N + 31) / 32), dim3(256), 0, stream, c, xs, wr, tp, za, zw, sa,
                        sw, bias, out, M, N, L);
     return hipGetLastError();
 }
 
 hipError_t launch_dequant_grad(const float* g, const float* sa, const float* sw, float* gc, int M, int N, int L, hipStream_t stream) {
-    hipLaunchKernelGGL(dequant_grad_nchw_to_rows_kernel, dim3((M + 31) / 32, (N + 31) / 32), dim3(256), 0, stream, g, sa, sw, gc, M, N, L);
+    hipLaunchKernelGGL(dequant_grad_nchw_to_rows_kernel, dim3((M + 127) / 128, (N + 31) / 32), dim3(256), 0, stream, g, sa, sw, gc, M, N, L);
     return hipGetLastError();
 }
 
