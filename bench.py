@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the LUT-GEMM hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--layers] [--grad-tables f32] [--workload vgg16_b128_8bit]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--layers] [--grad-tables f32] [--workload vgg16_b128_8bit] [--codes captured]
 
 One "step" = forward + backward (gradA and gradB) LUT-GEMM of every conv layer and the fc layer of a
 CIFAR-style ResNet-18 at batch 256, 7-bit tables (BASELINE.json configs[2]: 21 GEMMs,
@@ -51,6 +51,32 @@ HBM_PEAK = 8.0e12
 MEASURED_TRAFFIC_CONV2X = {"forward": (337 + 65) * 2**20, "gradA": (1146 + 576) * 2**20, "gradB": (450 + 1) * 2**20}
 
 
+def capture_codes(torch, dev, bits, tables, arch, batch):
+    """Operand codes of every LUT GEMM of one training-mode forward pass of this package's network on N(0,1) images:
+    {(M, K, N): (A codes, B codes)}, the first GEMM of each shape."""
+    import app_train
+    from self_ops.ops_py import approx_ops as ops
+    ops.set_lookup_tables(dev, *tables)
+    torch.manual_seed(0)
+    model = app_train.build_model(arch, bits, False, dev, approx_linear=True)
+    x = torch.randn(batch, 3, 32, 32, device=dev, generator=torch.Generator(device=dev).manual_seed(1))
+    seen = {}
+    native = ops.approx_ops.approx_gemm_forward
+
+    def spy(a, b, c, lut):
+        seen.setdefault((a.shape[0], a.shape[1], b.shape[1]), (a.clone(), b.clone()))
+        return native(a, b, c, lut)
+
+    ops.approx_ops.approx_gemm_forward = spy
+    try:
+        model.train()
+        with torch.no_grad():
+            model(x)
+    finally:
+        ops.approx_ops.approx_gemm_forward = native
+    return seen
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -66,6 +92,10 @@ def main():
     ap.add_argument("--workload", choices=["resnet18_b256_7bit", "vgg16_b128_8bit"], default="resnet18_b256_7bit",
                     help="resnet18_b256_7bit: the headline configuration; vgg16_b128_8bit: the 8-bit stress configuration "
                          "(forward error +-256, half window 16)")
+    ap.add_argument("--codes", choices=["uniform", "captured"], default="uniform",
+                    help="uniform: independent uniform random codes (the headline figure; worst case for LDS conflicts); captured: the "
+                         "operand codes one forward pass of this package's network produces on N(0,1) images with random-init weights "
+                         "(post-ReLU activations and bell-shaped weights: skewed codes)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures the one-GPU hot path only: every box of this build has one GPU; run with --gpus 1")
@@ -121,6 +151,13 @@ def main():
             gB=torch.empty((K, N), dtype=torch.float32, device=dev))
         ws_need = max(ws_need, (lib.amr_lut_gemm_backward_f32tab_workspace_bytes if f32_tables else lib.amr_lut_gemm_backward_workspace_bytes)(M, K, N))
     ws = torch.empty(max(ws_need, 256), dtype=torch.uint8, device=dev)
+
+    if args.codes == "captured":
+        seen = capture_codes(torch, dev, BITS, (lut.cpu().numpy(), lga.cpu().numpy(), lgb.cpu().numpy()),
+                             "resnet18" if headline else "vgg16", BATCH)
+        for name, cnt, M, K, N in RESNET18_B256:
+            assert (M, K, N) in seen, f"the network's forward pass ran no LUT GEMM of shape {(M, K, N)} ({name})"
+            bufs[name]["A"], bufs[name]["B"] = seen[(M, K, N)]
 
     def fwd(name, M, K, N):
         b = bufs[name]
@@ -243,7 +280,7 @@ def main():
         "config": {"workload": ("subset: " + args.only) if not full else
                    "resnet18_cifar_b256_7bit_lutgemm_fwd_bwd (BASELINE.json configs[2]: 20 conv + 1 fc GEMMs)" if headline else
                    "vgg16_cifar_b128_8bit_lutgemm_fwd_bwd (BASELINE.json configs[3]: 13 conv + 1 fc GEMMs)",
-                   "batch": BATCH, "lut_macs_per_step": macs_step, "codes": "uniform random", "grad_tables": (f"float32 unrounded difference slopes, half window {HALF_WS}" if f32_tables else f"int16 x16 difference-based, half window {HALF_WS}")},
+                   "batch": BATCH, "lut_macs_per_step": macs_step, "codes": "uniform random" if args.codes == "uniform" else "captured from one forward pass of the network (N(0,1) images, random-init weights, min/max quantisation)", "grad_tables": (f"float32 unrounded difference slopes, half window {HALF_WS}" if f32_tables else f"int16 x16 difference-based, half window {HALF_WS}")},
         "images_per_s": BATCH * args.steps / dt,
         "frac_of_lds_gather_roofline": rate / LDS_GATHER_PEAK,
         "kernel_ms_per_step": {k: round(v, 4) for k, v in kernels.items()},

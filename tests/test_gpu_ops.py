@@ -510,3 +510,19 @@ def test_one_launch_observer_update_equals_tensor_expressions(ops, kind, qmax_on
     s1, z1 = L._observe(fused2, x, qmax, eps, sc, zp)
     s2, z2 = L._observe(plain2, x, qmax, eps, None, None)
     assert torch.equal(s1.reshape(1), s2.reshape(1)) and torch.equal(z1.reshape(1), z2.reshape(1))
+
+
+def test_bench_captured_codes_cover_every_benchmark_layer(ops):
+    """bench.py --codes captured: one forward pass of the package's ResNet-18 yields operand codes for each of the 12
+    benchmark GEMM shapes (here at batch 4), uint8 below 2^7, and post-ReLU activations pile up on one code."""
+    import bench
+    _, P = ops
+    print("captured codes", flush=True)
+    tables = tuple(t.cpu().numpy() for t in (P.lut_appmult, P.lut_grad_a, P.lut_grad_b))
+    seen = bench.capture_codes(torch, torch.device("cuda"), 7, tables, "resnet18", 4)
+    for name, cnt, M, K, N in bench.RESNET18_B256:
+        a, b = seen[(M // 64, K, N)]
+        assert a.dtype == torch.uint8 and b.dtype == torch.uint8 and a.is_contiguous() and b.is_contiguous(), name
+        assert int(a.max()) < 128 and int(b.max()) < 128, name
+    a, _ = seen[(4096, 576, 64)]                      # conv2_x: its input went through a ReLU (and the padding adds zeros)
+    assert float(torch.bincount(a.flatten().int(), minlength=128).max()) / a.numel() > 0.25
