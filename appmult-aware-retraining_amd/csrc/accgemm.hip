@@ -12,7 +12,9 @@ __global__ __launch_bounds__(256) void accgemm_f32_kernel(const float* __restric
     __shared__ float As[BK][BM + 1];
     __shared__ float Bs[BK][BN + 1];
     const int tx = threadIdx.x % 16, ty = threadIdx.x / 16;
-    const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+    int tile_n, tile_m;
+    folded_tile_xy((N + BN - 1) / BN, &tile_n, &tile_m);
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
     float acc[4][4] = {};
     for (int k0 = 0; k0 < K; k0 += BK) {
         for (int i = threadIdx.x; i < BM * BK; i += 256) {
@@ -48,7 +50,7 @@ __global__ __launch_bounds__(256) void accgemm_f32_kernel(const float* __restric
 }
 
 hipError_t launch_accgemm(const float* A, const float* B, float* C, int M, int K, int N, hipStream_t stream) {
-    dim3 grid((N + 63) / 64, (M + 63) / 64);
+    dim3 grid((unsigned)((N + 63) / 64) * (unsigned)((M + 63) / 64));   // column tiles x row tiles, folded into x
     hipLaunchKernelGGL(accgemm_f32_kernel, grid, dim3(256), 0, stream, A, B, C, M, K, N);
     return hipGetLastError();
 }

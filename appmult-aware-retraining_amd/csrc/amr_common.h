@@ -110,4 +110,13 @@ __device__ __forceinline__ int div_small(int j, int d, float inv) {
     return q;
 }
 
+// Tile coordinates of a workgroup whose (x, y) tile grid is folded into blockIdx.x, x fastest -- the order in which a
+// two-dimensional grid is dealt out, without its limit of 65535 workgroups along y.
+__device__ __forceinline__ void folded_tile_xy(int tiles_x, int* x, int* y) {
+    const uint32_t id = blockIdx.x;
+    const uint32_t q = id / (uint32_t)tiles_x;
+    *y = (int)q;
+    *x = (int)(id - q * (uint32_t)tiles_x);
+}
+
 }  // namespace amr

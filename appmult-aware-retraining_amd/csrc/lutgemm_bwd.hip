@@ -160,8 +160,10 @@ __global__ __launch_bounds__(WAVES * 64) void lutgemm_gradA_kernel(
 
     const int wave = uniform(threadIdx.x >> 6);
     const int lane = threadIdx.x & 63;
-    const int k0 = blockIdx.x * KT;
-    const int m0 = (blockIdx.y * WAVES + wave) * (64 * RM);
+    int tile_k, tile_m;
+    folded_tile_xy((K + KT - 1) / KT, &tile_k, &tile_m);
+    const int k0 = tile_k * KT;
+    const int m0 = (tile_m * WAVES + wave) * (64 * RM);
     if (m0 >= M) return;
 
     int mr[RM];
@@ -343,7 +345,7 @@ static hipError_t launch_gradA_t(const float* gC, const uint8_t* A, const uint8_
         done = true;
     }
     const int rows_per_wg = 64 * RM * WAVES;
-    dim3 grid((K + KT - 1) / KT, (M + rows_per_wg - 1) / rows_per_wg);
+    dim3 grid((unsigned)((K + KT - 1) / KT) * (unsigned)((M + rows_per_wg - 1) / rows_per_wg));   // k tiles x row blocks, folded into x
     hipLaunchKernelGGL(kern, grid, dim3(WAVES * 64), (size_t)g.cols * g.cols * 2, stream, gC, A, B, gA,
                        reinterpret_cast<const uint16_t*>(lut), g.rows, g.cols, M, K, N, scale, gate, rows_per_image, vec_store);
     return hipGetLastError();

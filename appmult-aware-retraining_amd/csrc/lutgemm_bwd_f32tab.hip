@@ -115,8 +115,10 @@ __global__ __launch_bounds__(WAVES * 64) void lutgemm_gradA_f32tab_kernel(
     if (gate != nullptr && *gate == 0u) return;
     const int wave = uniform(threadIdx.x >> 6);
     const int lane = threadIdx.x & 63;
-    const int k0 = blockIdx.x * KT;
-    const int m0 = (blockIdx.y * WAVES + wave) * (64 * RM);
+    int tile_k, tile_m;
+    folded_tile_xy((K + KT - 1) / KT, &tile_k, &tile_m);
+    const int k0 = tile_k * KT;
+    const int m0 = (tile_m * WAVES + wave) * (64 * RM);
     const bool active = m0 < M;
     const uint32_t trow_bytes = (uint32_t)cols * 4u;
 
@@ -306,7 +308,7 @@ static hipError_t launch_gradA_f32tab_t(const float* gC, const uint8_t* A, const
     hipError_t e = allow_big_lds(kern, &done);
     if (e != hipSuccess) return e;
     const int rows_per_wg = 64 * RM * WAVES;
-    dim3 grid((K + KT - 1) / KT, (M + rows_per_wg - 1) / rows_per_wg);
+    dim3 grid((unsigned)((K + KT - 1) / KT) * (unsigned)((M + rows_per_wg - 1) / rows_per_wg));   // k tiles x row blocks, folded into x
     hipLaunchKernelGGL(kern, grid, dim3(WAVES * 64), (size_t)(rows_pp + 1) * g.cols * 4, stream, gC, A, B, gA, lut, g.rows, g.cols, rows_pp,
                        passes, M, K, N, scale, gate, rows_per_image, vec_store);
     return hipGetLastError();

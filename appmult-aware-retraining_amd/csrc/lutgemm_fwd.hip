@@ -33,9 +33,11 @@ __global__ __launch_bounds__(WAVES * 64) void lutgemm_fwd_kernel(
 
     const int wave = uniform(threadIdx.x >> 6);
     const int lane = threadIdx.x & 63;
-    const int m0 = (blockIdx.y * WAVES + wave) * R;
+    int tile_n, tile_m;
+    folded_tile_xy((N + 64 * TN - 1) / (64 * TN), &tile_n, &tile_m);
+    const int m0 = (tile_m * WAVES + wave) * R;
     if (m0 >= M) return;
-    const int n0 = blockIdx.x * (64 * TN);
+    const int n0 = tile_n * (64 * TN);
     const int kb = blockIdx.z * k_chunk;
     const int ke = min(K, kb + k_chunk);
     if (kb >= ke) return;
@@ -141,7 +143,8 @@ static hipError_t launch_fwd_t(const uint8_t* A, const uint8_t* B, uint32_t* C, 
     }
     const int k_chunk = ((K + ksplit - 1) / ksplit + 3) & ~3;
     const int zs = (K + k_chunk - 1) / k_chunk;
-    dim3 grid((N + 64 * TN - 1) / (64 * TN), (M + WAVES * R - 1) / (WAVES * R), zs);
+    // (column tiles x row blocks folded into x: a grid may be 65535 workgroups along y, and M / 64 can exceed that)
+    dim3 grid((unsigned)((N + 64 * TN - 1) / (64 * TN)) * (unsigned)((M + WAVES * R - 1) / (WAVES * R)), 1, zs);
     if (zs > 1) {
         hipError_t e = launch_zero_u32(C, (size_t)M * N, stream);
         if (e != hipSuccess) return e;

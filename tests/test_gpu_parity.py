@@ -610,6 +610,88 @@ def test_direct_kernels_at_large_m(lib, oracle, shape):
     assert (gpu_forward(lib, A, B, flat) == c0).all()            # expanded-table kernels: same bits
 
 
+def test_operands_beyond_2_31_elements(lib, oracle):
+    """M * K just above 2^31 (2 GiB of codes, 8 GiB of gA): the kernels that take 32-bit offsets step aside and the rows whose
+    offsets need more than 32 bits come out right.  Forward and gA are checked against the oracle on row samples (first rows,
+    middle, and the rows beyond offset 2^31); gB, a sum over all rows, against the sum of the two halves of the rows computed
+    by launches whose offsets fit 32 bits, within the tolerance measured against the sum of term magnitudes (the same
+    launch on |gC| and |table|)."""
+    print("M*K > 2^31", flush=True)
+    M, K, N, bits = 4194432, 512, 20, 7
+    assert M * K > 2**31 and M % 2 == 0
+    rng = np.random.default_rng(77)
+    gen = torch.Generator(device="cuda").manual_seed(77)
+    a = torch.randint(0, 128, (M, K), dtype=torch.uint8, device="cuda", generator=gen)
+    B = rng.integers(0, 128, (K, N)).astype(np.uint8)
+    T = rng.integers(0, 65536, (128, 128))
+    flat = oracle.pack_table(T, bits, np.uint16)
+    la = oracle.pack_table(rng.integers(-1024, 3073, (128, 128)), bits, np.int16)
+    lb = oracle.pack_table(rng.integers(-1024, 3073, (128, 128)), bits, np.int16)
+    gd = torch.randn((M, N), device="cuda", generator=gen)
+    b, l, ta, tb = dev(B), dev(flat), dev(la), dev(lb)
+    idx = np.concatenate([np.arange(64), np.arange(M // 2 - 32, M // 2 + 32), np.arange(M - 192, M)])
+    assert (idx[-128:] * K >= 2**31).all()
+    tidx = torch.from_numpy(idx).cuda()
+    A_s, g_s = a[tidx].cpu().numpy(), gd[tidx].cpu().numpy()
+
+    assert lib.amr_lut_gemm_forward_workspace_bytes(l.numel(), M, K, N) == 0
+    c = torch.full((M, N), -1, dtype=torch.int32, device="cuda")
+    assert lib.amr_lut_gemm_forward(a.data_ptr(), b.data_ptr(), c.data_ptr(), l.data_ptr(), l.numel(), M, K, N, None) == 0, lib.amr_last_error()
+    torch.cuda.synchronize()
+    assert (c[tidx].cpu().numpy().view(np.uint32) == oracle.forward_c(A_s, B, flat, bits)).all()
+    del c
+
+    def backward(gc, codes, table_b, rows, want_a):
+        ga = torch.full((rows, K), float("nan"), device="cuda") if want_a else None
+        gb = torch.full((K, N), float("nan"), device="cuda")
+        need = lib.amr_lut_gemm_backward_workspace_bytes(rows, K, N)
+        ws = torch.empty(max(need, 1), dtype=torch.uint8, device="cuda")
+        rc = lib.amr_lut_gemm_backward(gc.data_ptr(), codes.data_ptr(), b.data_ptr(), ga.data_ptr() if want_a else None, gb.data_ptr(),
+                                       ta.data_ptr(), table_b.data_ptr(), ta.numel(), rows, K, N, ws.data_ptr(), need, None)
+        assert rc == 0, lib.amr_last_error()
+        torch.cuda.synchronize()
+        return ga, gb
+
+    ga, gb = backward(gd, a, tb, M, True)
+    a64, _, absA, _ = oracle.backward_c_f64(g_s, A_s, B, la, lb, bits, want_abs=True)
+    err = np.abs(ga[tidx].cpu().numpy() - a64)
+    assert np.max(err / np.maximum(absA, 1e-30)) < TOL
+    assert bool(torch.isfinite(ga).all())
+    del ga
+    h = M // 2
+    _, gb0 = backward(gd[:h], a[:h], tb, h, False)
+    _, gb1 = backward(gd[h:], a[h:], tb, h, False)
+    _, gb_abs = backward(gd.abs(), a, dev(np.abs(lb)), M, False)
+    err = (gb.double() - (gb0.double() + gb1.double())).abs()
+    assert float((err / gb_abs.double().clamp_min(1e-30)).max()) < 2 * TOL
+    assert bool(torch.isfinite(gb).all()) and float(gb_abs.min()) > 0
+
+
+def test_row_counts_beyond_65535_row_blocks(lib, oracle):
+    """More row blocks than a grid may have workgroups along y (65535): the direct kernels fold their tile grid into x."""
+    print("row blocks > 65535", flush=True)
+    # 64 rows per workgroup in the forward kernel for N > 128 and in the fp32 GEMM: 65538 row blocks
+    M, K, N = 4194432, 8, 130
+    rng, A, B, T = rand_case(31, M, K, N, 7)
+    flat = oracle.pack_table(T, 7, np.uint16)
+    assert (gpu_forward(lib, A, B, flat) == oracle.forward_c(A, B, flat, 7)).all()
+    a, b = dev(A.astype(np.float32)), dev(B.astype(np.float32))
+    c = torch.full((M, N), float("nan"), device="cuda")
+    assert lib.amr_acc_gemm_forward_fp32(a.data_ptr(), b.data_ptr(), c.data_ptr(), M, K, N, None) == 0, lib.amr_last_error()
+    torch.cuda.synchronize()
+    assert torch.equal(c.cpu(), torch.from_numpy(A.astype(np.float32) @ B.astype(np.float32)))     # small integers: exact
+    del a, b, c
+    # 512 rows per workgroup in the direct gradA kernel, 128 in the forward kernel for N <= 64: 65537 and 262145 row blocks
+    M, K, N = 33554496, 3, 2
+    rng, A, B, T = rand_case(32, M, K, N, 7)
+    flat = oracle.pack_table(T, 7, np.uint16)
+    assert (gpu_forward(lib, A, B, flat) == oracle.forward_c(A, B, flat, 7)).all()
+    la = oracle.pack_table(rng.integers(-1024, 3073, (128, 128)), 7, np.int16)
+    lb = oracle.pack_table(rng.integers(-1024, 3073, (128, 128)), 7, np.int16)
+    g = rng.standard_normal((M, N)).astype(np.float32)
+    check_backward(oracle, gpu_backward(lib, g, A, B, la, lb), g, A, B, la, lb, 7)
+
+
 def test_default_mode_picks_kernels_by_problem_size(lib, oracle):
     print("kernel selection by size", flush=True)
     assert lib.amr_set_expanded_table_kernels(1) == 2
