@@ -692,6 +692,49 @@ def test_row_counts_beyond_65535_row_blocks(lib, oracle):
     check_backward(oracle, gpu_backward(lib, g, A, B, la, lb), g, A, B, la, lb, 7)
 
 
+def _seeded_case(seed):
+    """A pseudo-random problem: bit width, shape (half of them with the divisibilities the expanded-table kernels want),
+    table value range and kernel-selection mode all drawn from the seed."""
+    rng = np.random.default_rng(1000 + seed)
+    bits = int(rng.choice([7, 7, 7, 8, 6, 4]))
+    M = int(np.exp(rng.uniform(0, np.log(7000))))
+    K = int(np.exp(rng.uniform(0, np.log(1400))))
+    N = int(np.exp(rng.uniform(0, np.log(320))))
+    if rng.random() < 0.5:
+        M, K, N = max(1024, M // 128 * 128 + int(rng.choice([0, 0, 5]))), max(16, K // 16 * 16), max(32, N // 32 * 32)
+    lo, hi = [(-2048, 2049), (-1024, 3073), (-32768, 32768), (0, 4081)][int(rng.integers(0, 4))]
+    mode = int(rng.choice([1, 2, 2]))
+    return rng, bits, max(M, 1), max(K, 1), max(N, 1), lo, hi, mode
+
+
+@pytest.mark.parametrize("seed", range(48))
+def test_seeded_random_problems(lib, oracle, seed):
+    """Forward bit-exact and both backward entry points within tolerance on 48 problems drawn from seeds."""
+    rng, bits, M, K, N, lo, hi, mode = _seeded_case(seed)
+    print("seeded problem", seed, bits, (M, K, N), (lo, hi), "mode", mode, flush=True)
+    n = 1 << bits
+    A = rng.integers(0, n, (M, K)).astype(np.uint8)
+    B = rng.integers(0, n, (K, N)).astype(np.uint8)
+    if bits < 8 and seed % 5 == 0:                       # the masked code 2^b here and there
+        A[rng.integers(0, M), rng.integers(0, K)] = n
+        B[rng.integers(0, K), rng.integers(0, N)] = n
+    flat = oracle.pack_table(rng.integers(0, 65536 if seed % 2 else 16384, (n, n)), bits, np.uint16)
+    la = oracle.pack_table(rng.integers(lo, hi, (n, n)), bits, np.int16)
+    lb = oracle.pack_table(rng.integers(lo, hi, (n, n)), bits, np.int16)
+    g = rng.standard_normal((M, N)).astype(np.float32)
+    assert lib.amr_set_expanded_table_kernels(mode) == 2
+    try:
+        c = gpu_forward(lib, A, B, flat)
+        r16 = gpu_backward(lib, g, A, B, la, lb)
+        fa, fb = (la.astype(np.float32) * np.float32(0.37)), (lb.astype(np.float32) * np.float32(-1.3))
+        r32 = gpu_backward_f32tab(lib, g, A, B, fa, fb, 0.5)
+    finally:
+        lib.amr_set_expanded_table_kernels(2)
+    assert (c == oracle.forward_c(A, B, flat, bits)).all()
+    check_backward(oracle, r16, g, A, B, la, lb, bits)
+    check_backward(oracle, r32, g, A, B, fa, fb, bits, factor=0.5)
+
+
 def test_default_mode_picks_kernels_by_problem_size(lib, oracle):
     print("kernel selection by size", flush=True)
     assert lib.amr_set_expanded_table_kernels(1) == 2
