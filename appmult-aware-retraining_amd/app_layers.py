@@ -77,13 +77,15 @@ def _scale_and_zero_point(observer, quant_max, eps):
 
 
 def _observe(observer, x, quant_max, eps, scale, zp_neg):
-    """One observer step on ``x`` followed by the scale / zero point it implies; returns (scale, zp_neg).
-    On the GPU the scalar arithmetic (range update, scale, zero point: a dozen one-element tensor operations in the
-    reference, ``app_layers.py:21-53,154-160``) is one launch that updates the observer's buffers and the given
-    ``scale`` / ``zp_neg`` buffers in place; the values are those of the tensor expressions."""
+    """One observer step on ``x`` followed by the scale / zero point it implies; returns (scale, zp_neg) as NEW tensors,
+    like the reference's ``self.activation_scale = torch.max(...)`` (``app_layers.py:154-160``): an autograd graph built by
+    an earlier forward pass keeps the values it saw.  ``scale`` / ``zp_neg`` (the layer's current buffers) only say where the
+    results live.  On the GPU the scalar arithmetic (range update, scale, zero point: a dozen one-element tensor operations
+    in the reference, ``app_layers.py:21-53,154-160``) is one launch that updates the observer's range buffers in place
+    (no graph ever holds those) and writes the two results; the values are those of the tensor expressions."""
     fused_mode = getattr(observer, "fused_mode", None)
     ok = (fused_mode is not None and x.is_cuda and x.dtype == torch.float32 and
-          all(t.is_cuda and t.dtype == torch.float32 and t.numel() == 1 and t.is_contiguous()
+          all(t is not None and t.is_cuda and t.dtype == torch.float32 and t.numel() == 1 and t.is_contiguous()
               for t in (observer.min_val, observer.max_val, scale, zp_neg)))
     if not ok:
         observer(x)
@@ -93,11 +95,13 @@ def _observe(observer, x, quant_max, eps, scale, zp_neg):
         lo, hi = torch.aminmax(x)
         mode = 0 if observer.num_flag == 0 else fused_mode
         observer.num_flag = 1
-        approx_ops.observer_update(lo.reshape(1), hi.reshape(1), observer.min_val, observer.max_val, scale, zp_neg, mode,
+        fresh = torch.empty(2, dtype=torch.float32, device=x.device)
+        new_scale, new_zp = fresh[0:1], fresh[1:2]
+        approx_ops.observer_update(lo.reshape(1), hi.reshape(1), observer.min_val, observer.max_val, new_scale, new_zp, mode,
                                    getattr(observer, "momentum", 0.0), float(quant_max), float(eps),
                                    # torch divides by a host-side scalar through its reciprocal rounded to float32
                                    0.0 if quant_max.is_cuda else float(torch.tensor(1.0, dtype=torch.float32) / quant_max.to(torch.float32)))
-    return scale, zp_neg
+    return new_scale, new_zp
 
 
 class _ToCodesFn(torch.autograd.Function):

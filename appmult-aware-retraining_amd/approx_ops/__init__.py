@@ -53,6 +53,10 @@ _lib.amr_quantize_codes_f32.argtypes = [_vp, _vp, _vp, ctypes.c_float, _vp, _i64
 _lib.amr_quantize_codes_backward_f32.argtypes = [_vp, _vp, _vp, _vp, ctypes.c_float, _vp, _i64, _vp]
 _lib.amr_lut_gemm_backward_workspace_bytes.argtypes = [_i, _i, _i]
 _lib.amr_lut_gemm_backward_workspace_bytes.restype = _sz
+_lib.amr_lut_gemm_backward_workspace_bytes_for.argtypes = [_i64, _i, _i, _i]
+_lib.amr_lut_gemm_backward_workspace_bytes_for.restype = _sz
+_lib.amr_lut_gemm_backward_f32tab_workspace_bytes_for.argtypes = [_i64, _i, _i, _i]
+_lib.amr_lut_gemm_backward_f32tab_workspace_bytes_for.restype = _sz
 _lib.amr_acc_gemm_forward_fp32.argtypes = [_vp, _vp, _vp, _i, _i, _i, _vp]
 _lib.amr_bits_from_lut_elems.argtypes = [_i64]
 _lib.amr_lut_geometry.argtypes = [_i, ctypes.POINTER(_i), ctypes.POINTER(_i), ctypes.POINTER(_i64)]
@@ -182,7 +186,8 @@ def approx_gemm_backward(gc_tensor, a_tensor, b_tensor, ga_tensor, gb_tensor, lu
     _check(all(t.device == dev for t in (a_tensor, b_tensor, ga_tensor, gb_tensor, lut_grad_a_tensor, lut_grad_b_tensor) if t is not None),
            "All tensors should be on the same device")
     with torch.cuda.device(dev):
-        need = (_lib.amr_lut_gemm_backward_f32tab_workspace_bytes if float_tables else _lib.amr_lut_gemm_backward_workspace_bytes)(M, K, N)
+        need = (_lib.amr_lut_gemm_backward_f32tab_workspace_bytes_for if float_tables else
+                _lib.amr_lut_gemm_backward_workspace_bytes_for)(lut_grad_a_tensor.size(0), M, K, N)
         ws = torch.empty(need, dtype=torch.uint8, device=dev) if need else None
         ga_ptr = ga_tensor.data_ptr() if ga_tensor is not None else None
         gb_ptr = gb_tensor.data_ptr() if gb_tensor is not None else None

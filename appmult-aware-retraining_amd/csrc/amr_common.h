@@ -3,6 +3,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 namespace amr {
 
 constexpr int kWave = 64;  // CDNA4 wavefront width
@@ -40,6 +42,19 @@ inline bool lut_geom_from_elems(int64_t elems, LutGeom* g) {
         if (lut_geom_from_bits(bits, g) && g->elems == elems) return true;
     }
     return false;
+}
+
+// Lets a kernel use up to 160 KB of dynamic LDS: set once per kernel and device (bit d of `done` = device d), from
+// whichever host thread gets there first; setting it twice is harmless, so concurrent first calls need no lock.
+inline hipError_t allow_full_lds(const void* kernel, std::atomic<uint64_t>& done) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    const uint64_t bit = 1ull << (dev & 63);
+    if (done.load(std::memory_order_acquire) & bit) return hipSuccess;
+    e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    if (e == hipSuccess) done.fetch_or(bit, std::memory_order_release);
+    return e;
 }
 
 __device__ __forceinline__ int uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }

@@ -2,7 +2,9 @@
 // bit-width dispatch from the table length, per-device caches, launches on the caller's stream.
 #include "../../include/amr_lutgemm.h"
 
+#include <atomic>
 #include <mutex>
+#include <vector>
 #include <stdarg.h>
 #include <stdio.h>
 #include <string.h>
@@ -84,10 +86,19 @@ int hip_fail(hipError_t e, const char* where) {
 }
 
 constexpr int kMaxDevices = 64;
+// Scratch the library owns for callers that pass none: one buffer per (device, stream).  Work queued on a stream runs
+// in order, so calls on one stream can share a buffer; calls on different streams (possibly from different host
+// threads) never do.  A buffer that has become too small is replaced by a larger one and kept until the process ends:
+// launches already queued may still be using it, and freeing it would need a device-wide wait in the middle of an
+// asynchronous call.
+struct StreamScratch {
+    hipStream_t stream;
+    void* ptr;
+    size_t bytes;
+};
 struct DeviceState {
     int n_cu = 0;
-    void* ws = nullptr;
-    size_t ws_bytes = 0;
+    std::vector<StreamScratch> scratch;
 };
 DeviceState g_dev[kMaxDevices];
 std::mutex g_mu;
@@ -106,23 +117,25 @@ int current_device_cus(int* dev_out) {
     return g_dev[dev].n_cu;
 }
 
-// Library-owned scratch for callers that pass no workspace: grown on demand, kept until exit.
-void* internal_workspace(int dev, size_t bytes, hipError_t* err) {
+// Library-owned scratch of `stream` on device `dev`, at least `bytes` large.  Grows by allocation only (hipMalloc: not
+// possible while the stream is being captured into a graph -- the first call of a given size has to happen before the
+// capture, or the caller passes a workspace); never waits for the device and never frees.
+void* internal_workspace(int dev, hipStream_t stream, size_t bytes, hipError_t* err) {
     std::lock_guard<std::mutex> lk(g_mu);
     DeviceState& d = g_dev[dev];
     *err = hipSuccess;
-    if (d.ws_bytes >= bytes) return d.ws;
-    if (d.ws) {
-        (void)hipDeviceSynchronize();
-        (void)hipFree(d.ws);
-        d.ws = nullptr;
-        d.ws_bytes = 0;
-    }
+    StreamScratch* slot = nullptr;
+    for (StreamScratch& sc : d.scratch)
+        if (sc.stream == stream) slot = &sc;
+    if (slot && slot->bytes >= bytes) return slot->ptr;
     size_t want = bytes + bytes / 4;
-    *err = hipMalloc(&d.ws, want);
-    if (*err != hipSuccess) { d.ws = nullptr; return nullptr; }
-    d.ws_bytes = want;
-    return d.ws;
+    if (slot && want < 2 * slot->bytes) want = 2 * slot->bytes;    // geometric growth: all retired buffers together stay below the live one
+    void* p = nullptr;
+    *err = hipMalloc(&p, want);
+    if (*err != hipSuccess) return nullptr;
+    if (slot) { slot->ptr = p; slot->bytes = want; }               // the old buffer stays allocated (see above)
+    else d.scratch.push_back({stream, p, want});
+    return p;
 }
 
 }  // namespace
@@ -144,12 +157,10 @@ int amr_lut_geometry(int bits, int* rows, int* cols, int64_t* elem_num) {
 
 // Process-wide switch (diagnostics, tests, benchmarks): 0 sends every call to the direct gather kernels, 1 picks by
 // problem size, 2 takes the expanded-table kernels wherever the shape allows (also where they are slower).
-static int g_expanded_kernels = 1;
+static std::atomic<int> g_expanded_kernels{1};
 
 int amr_set_expanded_table_kernels(int mode) {
-    const int old = g_expanded_kernels;
-    g_expanded_kernels = mode <= 0 ? 0 : (mode >= 2 ? 2 : 1);
-    return old;
+    return g_expanded_kernels.exchange(mode <= 0 ? 0 : (mode >= 2 ? 2 : 1));
 }
 
 int amr_bits_from_lut_elems(int64_t lut_elems) {
@@ -162,7 +173,8 @@ int amr_bits_from_lut_elems(int64_t lut_elems) {
 size_t amr_lut_gemm_forward_workspace_bytes(int64_t lut_elems, int M, int K, int N) {
     amr::LutGeom g;
     if (M <= 0 || K <= 0 || N <= 0 || !amr::lut_geom_from_elems(lut_elems, &g)) return 0;
-    return g_expanded_kernels ? amr::fwd_slab_workspace_bytes(g, M, K, N, g_expanded_kernels == 2) : 0;
+    const int mode = g_expanded_kernels.load();
+    return mode ? amr::fwd_slab_workspace_bytes(g, M, K, N, mode == 2) : 0;
 }
 
 static int forward_impl(const uint8_t* A, const uint8_t* B, uint32_t* C, const uint16_t* lut, int64_t lut_elems, int M, int K, int N,
@@ -182,7 +194,8 @@ static int forward_impl(const uint8_t* A, const uint8_t* B, uint32_t* C, const u
     int dev = 0;
     const int n_cu = current_device_cus(&dev);
     if (n_cu <= 0) return fail(AMR_EINVAL, "no HIP device available");
-    const size_t need = g_expanded_kernels ? amr::fwd_slab_workspace_bytes(g, M, K, N, g_expanded_kernels == 2) : 0;
+    const int mode = g_expanded_kernels.load();
+    const size_t need = mode ? amr::fwd_slab_workspace_bytes(g, M, K, N, mode == 2) : 0;
     hipError_t e;
     if (need > 0) {
         void* ws = workspace;
@@ -190,7 +203,7 @@ static int forward_impl(const uint8_t* A, const uint8_t* B, uint32_t* C, const u
             if (workspace_bytes < need) return fail(AMR_EWORKSPACE, "workspace of %zu bytes is smaller than the %zu required", workspace_bytes, need);
             if ((uintptr_t)ws & 255) return fail(AMR_EINVAL, "workspace must be 256-byte aligned");
         } else {
-            ws = internal_workspace(dev, need, &e);
+            ws = internal_workspace(dev, s, need, &e);
             if (!ws) return hip_fail(e, "workspace hipMalloc");
         }
         e = amr::launch_fwd_slab(A, B, C, lut, g, M, K, N, n_cu, ws, s, out_f32);
@@ -226,20 +239,27 @@ static size_t backward_partial_bytes(int M, int K, int N, int n_cu) {
     return (b + 255) & ~(size_t)255;
 }
 
-// Size of the expanded table of gradA for 7-bit tables (the widest the expanded-table kernels take); a query
-// by shape alone cannot know the table width, so the scratch is sized for it.
-static size_t backward_gradA_bytes(int M, int K, int N) {
-    if (!g_expanded_kernels) return 0;
-    amr::LutGeom g7;
-    amr::lut_geom_from_bits(7, &g7);
-    return amr::gradA_slab_workspace_bytes(g7, M, K, N, g_expanded_kernels == 2);
+// Size of the expanded table of gradA.  bits == 0: the table width is not known (a query by shape alone), so the scratch
+// is sized for 7-bit tables, the widest the expanded-table kernels take.
+static size_t backward_gradA_bytes(int mode, int bits, int M, int K, int N) {
+    if (!mode) return 0;
+    amr::LutGeom g;
+    amr::lut_geom_from_bits(bits ? bits : 7, &g);
+    return amr::gradA_slab_workspace_bytes(g, M, K, N, mode == 2);
 }
 
 size_t amr_lut_gemm_backward_workspace_bytes(int M, int K, int N) {
     if (M <= 0 || K <= 0 || N <= 0) return 0;
     const int n_cu = current_device_cus(nullptr);
     // Without a device (e.g. a host-only query) size for a 256-CU part.
-    return 256 + backward_partial_bytes(M, K, N, n_cu > 0 ? n_cu : 256) + backward_gradA_bytes(M, K, N);
+    return 256 + backward_partial_bytes(M, K, N, n_cu > 0 ? n_cu : 256) + backward_gradA_bytes(g_expanded_kernels.load(), 0, M, K, N);
+}
+
+size_t amr_lut_gemm_backward_workspace_bytes_for(int64_t lut_elems, int M, int K, int N) {
+    amr::LutGeom g;
+    if (M <= 0 || K <= 0 || N <= 0 || !amr::lut_geom_from_elems(lut_elems, &g)) return 0;
+    const int n_cu = current_device_cus(nullptr);
+    return 256 + backward_partial_bytes(M, K, N, n_cu > 0 ? n_cu : 256) + backward_gradA_bytes(g_expanded_kernels.load(), g.bits, M, K, N);
 }
 
 int amr_lut_gemm_backward(const float* gC, const uint8_t* A, const uint8_t* B, float* gA, float* gB,
@@ -249,9 +269,12 @@ int amr_lut_gemm_backward(const float* gC, const uint8_t* A, const uint8_t* B, f
                                     workspace_bytes, stream);
 }
 
-int amr_lut_gemm_backward_ex(const float* gC, const uint8_t* A, const uint8_t* B, float* gA, float* gB,
-                             const int16_t* lut_grad_a, const int16_t* lut_grad_b, int64_t lut_elems, int M, int K,
-                             int N, int ga_rows_per_image, void* workspace, size_t workspace_bytes, void* stream) {
+// where the scratch of a backward call comes from
+enum class ScratchFrom { Caller, Library };
+
+static int backward_impl(const float* gC, const uint8_t* A, const uint8_t* B, float* gA, float* gB,
+                         const int16_t* lut_grad_a, const int16_t* lut_grad_b, int64_t lut_elems, int M, int K,
+                         int N, int ga_rows_per_image, ScratchFrom from, void* workspace, size_t workspace_bytes, void* stream) {
     if (ga_rows_per_image < 0 || (ga_rows_per_image > 0 && M % ga_rows_per_image != 0))
         return fail(AMR_EINVAL, "ga_rows_per_image=%d must divide M=%d", ga_rows_per_image, M);
     if (M < 0 || K < 0 || N < 0) return fail(AMR_EINVAL, "negative dimension M=%d K=%d N=%d", M, K, N);
@@ -276,20 +299,24 @@ int amr_lut_gemm_backward_ex(const float* gC, const uint8_t* A, const uint8_t* B
     const int n_cu = current_device_cus(&dev);
     if (n_cu <= 0) return fail(AMR_EINVAL, "no HIP device available");
     hipError_t e;
+    const int mode = g_expanded_kernels.load();
     const size_t partial_bytes = backward_partial_bytes(M, K, N, n_cu);
-    const size_t need = 256 + partial_bytes + backward_gradA_bytes(M, K, N);
+    // (what this table width needs: never more than the shape-only query answers)
+    const size_t gradA_bytes = backward_gradA_bytes(mode, g.bits, M, K, N);
+    const bool allow_slab_a = true;
     void* ws = workspace;
-    if (ws) {
+    const size_t need = 256 + partial_bytes + gradA_bytes;
+    if (from == ScratchFrom::Caller) {
         if (workspace_bytes < need) return fail(AMR_EWORKSPACE, "workspace of %zu bytes is smaller than the %zu required", workspace_bytes, need);
         if ((uintptr_t)ws & 255) return fail(AMR_EINVAL, "workspace must be 256-byte aligned");
-    } else {
-        ws = internal_workspace(dev, need, &e);
+    } else if (from == ScratchFrom::Library) {
+        ws = internal_workspace(dev, s, need, &e);
         if (!ws) return hip_fail(e, "workspace hipMalloc");
     }
     uint32_t* flags = reinterpret_cast<uint32_t*>(ws);
     float* partials = reinterpret_cast<float*>(reinterpret_cast<unsigned char*>(ws) + 256);
-    const bool slab = g_expanded_kernels && amr::bwd_slab_applies(g, M, K, N);
-    const bool slab_a = g_expanded_kernels && gA && amr::gradA_slab_workspace_bytes(g, M, K, N, g_expanded_kernels == 2) != 0 && ((uintptr_t)gC & 15) == 0;
+    const bool slab = mode && amr::bwd_slab_applies(g, M, K, N);
+    const bool slab_a = mode && allow_slab_a && gA && amr::gradA_slab_workspace_bytes(g, M, K, N, mode == 2) != 0 && ((uintptr_t)gC & 15) == 0;
     if ((slab && gB) || slab_a) {
         // flags cleared, offsets of the half-precision tables decided from the tables' extremes
         e = amr::launch_bwd_header(slab_a ? lut_grad_a : nullptr, (slab && gB) ? lut_grad_b : nullptr, g, flags, s);
@@ -314,18 +341,32 @@ int amr_lut_gemm_backward_ex(const float* gC, const uint8_t* A, const uint8_t* B
     return AMR_OK;
 }
 
+int amr_lut_gemm_backward_ex(const float* gC, const uint8_t* A, const uint8_t* B, float* gA, float* gB,
+                             const int16_t* lut_grad_a, const int16_t* lut_grad_b, int64_t lut_elems, int M, int K,
+                             int N, int ga_rows_per_image, void* workspace, size_t workspace_bytes, void* stream) {
+    return backward_impl(gC, A, B, gA, gB, lut_grad_a, lut_grad_b, lut_elems, M, K, N, ga_rows_per_image,
+                         workspace ? ScratchFrom::Caller : ScratchFrom::Library, workspace, workspace_bytes, stream);
+}
+
 // Scratch of the float-table backward pass: [256 B of flags][partial sums of gB][float32 expanded table of gradA].
-static size_t backward_gradA_f32_bytes(int M, int K, int N) {
-    if (!g_expanded_kernels) return 0;
-    amr::LutGeom g7;
-    amr::lut_geom_from_bits(7, &g7);
-    return amr::gradA_slab_f32_workspace_bytes(g7, M, K, N, g_expanded_kernels == 2);
+static size_t backward_gradA_f32_bytes(int mode, int bits, int M, int K, int N) {
+    if (!mode) return 0;
+    amr::LutGeom g;
+    amr::lut_geom_from_bits(bits ? bits : 7, &g);
+    return amr::gradA_slab_f32_workspace_bytes(g, M, K, N, mode == 2);
 }
 
 size_t amr_lut_gemm_backward_f32tab_workspace_bytes(int M, int K, int N) {
     if (M <= 0 || K <= 0 || N <= 0) return 0;
     const int n_cu = current_device_cus(nullptr);
-    return 256 + backward_partial_bytes(M, K, N, n_cu > 0 ? n_cu : 256) + backward_gradA_f32_bytes(M, K, N);
+    return 256 + backward_partial_bytes(M, K, N, n_cu > 0 ? n_cu : 256) + backward_gradA_f32_bytes(g_expanded_kernels.load(), 0, M, K, N);
+}
+
+size_t amr_lut_gemm_backward_f32tab_workspace_bytes_for(int64_t lut_elems, int M, int K, int N) {
+    amr::LutGeom g;
+    if (M <= 0 || K <= 0 || N <= 0 || !amr::lut_geom_from_elems(lut_elems, &g)) return 0;
+    const int n_cu = current_device_cus(nullptr);
+    return 256 + backward_partial_bytes(M, K, N, n_cu > 0 ? n_cu : 256) + backward_gradA_f32_bytes(g_expanded_kernels.load(), g.bits, M, K, N);
 }
 
 int amr_lut_gemm_backward_f32tab(const float* gC, const uint8_t* A, const uint8_t* B, float* gA, float* gB,
@@ -354,19 +395,20 @@ int amr_lut_gemm_backward_f32tab(const float* gC, const uint8_t* A, const uint8_
     if (n_cu <= 0) return fail(AMR_EINVAL, "no HIP device available");
     hipError_t e;
     const size_t partial_bytes = backward_partial_bytes(M, K, N, n_cu);
-    const size_t need = 256 + partial_bytes + backward_gradA_f32_bytes(M, K, N);
+    const int mode = g_expanded_kernels.load();
+    const size_t need = 256 + partial_bytes + backward_gradA_f32_bytes(mode, g.bits, M, K, N);
     void* ws = workspace;
     if (ws) {
         if (workspace_bytes < need) return fail(AMR_EWORKSPACE, "workspace of %zu bytes is smaller than the %zu required", workspace_bytes, need);
         if ((uintptr_t)ws & 255) return fail(AMR_EINVAL, "workspace must be 256-byte aligned");
     } else {
-        ws = internal_workspace(dev, need, &e);
+        ws = internal_workspace(dev, s, need, &e);
         if (!ws) return hip_fail(e, "workspace hipMalloc");
     }
     uint32_t* flags = reinterpret_cast<uint32_t*>(ws);
     float* partials = reinterpret_cast<float*>(reinterpret_cast<unsigned char*>(ws) + 256);
-    const bool slab_b = g_expanded_kernels && gB && amr::bwd_slab_applies(g, M, K, N);
-    const bool slab_a = g_expanded_kernels && gA && amr::gradA_slab_f32_workspace_bytes(g, M, K, N, g_expanded_kernels == 2) != 0 &&
+    const bool slab_b = mode && gB && amr::bwd_slab_applies(g, M, K, N);
+    const bool slab_a = mode && gA && amr::gradA_slab_f32_workspace_bytes(g, M, K, N, mode == 2) != 0 &&
                         ((uintptr_t)gC & 15) == 0;
     if (slab_a || slab_b) {
         e = amr::launch_zero_u32(flags, 64, s);

@@ -250,10 +250,6 @@ __global__ __launch_bounds__(WAVES * 64) void lutgemm_gradA_kernel(
 }
 
 // ------------------------------------------------------------------------------------------ host
-static hipError_t set_lds_attr(const void* f) {
-    return hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-}
-
 // M splits of a direct gradB launch whose workgroups have `waves` waves (each owning 16 k) and of which `wgs_per_cu` fit a
 // CU at a time.  The grid runs in rounds of n_cu * wgs_per_cu workgroups: the split count is the one whose
 // (rounds x rows per workgroup) is smallest -- 290 workgroups on 256 CUs take as long as 512 -- with every split keeping
@@ -308,15 +304,15 @@ hipError_t launch_gradB(const float* gC, const uint8_t* A, const uint8_t* B, flo
     hipError_t e;
     if (big) {
         auto kern = lutgemm_gradB_kernel<KT, 16>;
-        static bool done = false;
-        if (!done) { e = set_lds_attr(reinterpret_cast<const void*>(kern)); if (e != hipSuccess) return e; done = true; }
+        static std::atomic<uint64_t> done{0};
+        if ((e = allow_full_lds(reinterpret_cast<const void*>(kern), done)) != hipSuccess) return e;
         dim3 grid((N + 63) / 64, (ktiles + 15) / 16, zs);
         hipLaunchKernelGGL(kern, grid, dim3(1024), lds, stream, gC, A, B, out, reinterpret_cast<const uint32_t*>(lut),
                            lut_dwords, g.cols * 2, M, K, N, m_chunk, scale, gate);
     } else {
         auto kern = lutgemm_gradB_kernel<KT, 4>;
-        static bool done = false;
-        if (!done) { e = set_lds_attr(reinterpret_cast<const void*>(kern)); if (e != hipSuccess) return e; done = true; }
+        static std::atomic<uint64_t> done{0};
+        if ((e = allow_full_lds(reinterpret_cast<const void*>(kern), done)) != hipSuccess) return e;
         dim3 grid((N + 63) / 64, (ktiles + 3) / 4, zs);
         hipLaunchKernelGGL(kern, grid, dim3(256), lds, stream, gC, A, B, out, reinterpret_cast<const uint32_t*>(lut),
                            lut_dwords, g.cols * 2, M, K, N, m_chunk, scale, gate);
@@ -338,12 +334,8 @@ static hipError_t launch_gradA_t(const float* gC, const uint8_t* A, const uint8_
                                  int rows_per_image) {
     const int vec_store = ((K & 3) == 0) && (((uintptr_t)gA & 15) == 0);
     auto kern = lutgemm_gradA_kernel<KT, RM, WAVES, VEC>;
-    static bool done = false;
-    if (!done) {
-        hipError_t e = set_lds_attr(reinterpret_cast<const void*>(kern));
-        if (e != hipSuccess) return e;
-        done = true;
-    }
+    static std::atomic<uint64_t> done{0};
+    if (hipError_t ea = allow_full_lds(reinterpret_cast<const void*>(kern), done); ea != hipSuccess) return ea;
     const int rows_per_wg = 64 * RM * WAVES;
     dim3 grid((unsigned)((K + KT - 1) / KT) * (unsigned)((M + rows_per_wg - 1) / rows_per_wg));   // k tiles x row blocks, folded into x
     hipLaunchKernelGGL(kern, grid, dim3(WAVES * 64), (size_t)g.cols * g.cols * 2, stream, gC, A, B, gA,

@@ -248,11 +248,8 @@ static void f32tab_bands(const LutGeom& g, int* rows_pp, int* passes) {
 }
 
 template <typename Kern>
-static hipError_t allow_big_lds(Kern kern, bool* done) {
-    if (*done) return hipSuccess;
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-    if (e == hipSuccess) *done = true;
-    return e;
+static hipError_t allow_big_lds(Kern kern, std::atomic<uint64_t>* done) {
+    return allow_full_lds(reinterpret_cast<const void*>(kern), *done);
 }
 
 int gradB_direct_splits(int M, int K, int N, int n_cu, int waves, int wgs_per_cu);
@@ -275,13 +272,13 @@ hipError_t launch_gradB_f32tab(const float* gC, const uint8_t* A, const uint8_t*
     hipError_t e;
     if (wide) {
         // one 1024-thread workgroup per CU shares the staged band
-        static bool done = false;
+        static std::atomic<uint64_t> done{0};
         auto kern = lutgemm_gradB_f32tab_kernel<KT, 16, true>;
         if ((e = allow_big_lds(kern, &done)) != hipSuccess) return e;
         hipLaunchKernelGGL(kern, dim3((N + 63) / 64, (ktiles + 15) / 16, zs), dim3(1024), lds, stream, gC, A, B, out, lut, g.rows,
                            g.cols, rows_pp, passes, M, K, N, m_chunk, scale, gate);
     } else {
-        static bool done = false;
+        static std::atomic<uint64_t> done{0};
         auto kern = lutgemm_gradB_f32tab_kernel<KT, 4, false>;
         if ((e = allow_big_lds(kern, &done)) != hipSuccess) return e;
         hipLaunchKernelGGL(kern, dim3((N + 63) / 64, (ktiles + 3) / 4, zs), dim3(256), lds, stream, gC, A, B, out, lut, g.rows,
@@ -304,7 +301,7 @@ static hipError_t launch_gradA_f32tab_t(const float* gC, const uint8_t* A, const
                                         hipStream_t stream, const uint32_t* gate, int rows_per_image) {
     const int vec_store = ((K & 3) == 0) && (((uintptr_t)gA & 15) == 0);
     auto kern = lutgemm_gradA_f32tab_kernel<KT, RM, WAVES, VEC, SPLIT>;
-    static bool done = false;
+    static std::atomic<uint64_t> done{0};
     hipError_t e = allow_big_lds(kern, &done);
     if (e != hipSuccess) return e;
     const int rows_per_wg = 64 * RM * WAVES;

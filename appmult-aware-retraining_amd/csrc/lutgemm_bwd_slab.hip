@@ -255,7 +255,8 @@ __global__ __launch_bounds__(1024) void lutgemm_gradB_slab16_kernel(
     const int k0 = k_tile * KT;
     const int mb = split * m_chunk;
     const int me = min(M, mb + m_chunk);
-    const float offset = (float)flags[4];        // 0 or 1024 (bwd_header_kernel)
+    if (flags[6] != 0u) return;                  // the table cannot be held as halves (bwd_header_kernel): the direct kernel does it
+    const float offset = (float)(int)flags[4];   // bwd_header_kernel
 
     {   // expansion.  First the table itself goes to LDS, as halves, 128 x 128 without the padding (32 KB behind the
         // slabs; codes the table does not have read as zero): 16 independent loads per thread, one trip to L2.
@@ -433,8 +434,8 @@ __global__ __launch_bounds__(1024) void lutgemm_gradB_slab16_kernel(
 __global__ __launch_bounds__(256) void gradB_finish_kernel(const float* __restrict__ partial, float* __restrict__ gB,
                                                            const float* __restrict__ colsum, const uint32_t* __restrict__ flags,
                                                            int K, int N, int splits, float scale) {
-    const float offset = (float)flags[4];
-    if (partial == nullptr && offset == 0.f) return;
+    const float offset = (float)(int)flags[4];
+    if (flags[6] != 0u || (partial == nullptr && offset == 0.f)) return;
     const size_t count = (size_t)K * N;
     const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
     if (i >= count) return;
@@ -450,14 +451,21 @@ __global__ __launch_bounds__(256) void gradB_finish_kernel(const float* __restri
 }
 
 // ------------------------------------------------------------------------------------------ scratch header
-// One workgroup: clears the 64 flag words of the backward scratch and leaves the offsets the half-precision tables
-// are stored with: flags[3] for the table of gradA, flags[4] for the table of gradB.  A half holds every integer
-// of magnitude <= 2048: offset 0 when the whole table lies in [-2048, 2048] (the correction term with the sums
-// of gC then drops out of the kernels), else 1024, exact for [-1024, 3072].
+// One workgroup: clears the 64 flag words of the backward scratch and decides how the half-precision tables are stored.
+// A half holds every integer of magnitude <= 2048.  offset (flags[3] for the table of gradA, flags[4] for the table of
+// gradB, as int32): 0 when the whole table lies in [-2048, 2048] (the correction term with the sums of gC then drops out
+// of the kernels); else the value of smallest magnitude that brings every entry into that range, max - 2048 or
+// min + 2048, when the table spans no more than 4096.  The kernels then compute sum g * (entry - offset) + offset * sum g,
+// whose rounding errors grow with |offset| while the true terms have the size of the entries: the offset is only taken
+// when |offset| <= 8 x the mean magnitude of the entries.  A table that fails either test is not held as halves at all:
+// flags[5] (gradA) / flags[6] (gradB) tell the expanded-table kernels to leave at once, and flags[2] / flags[1] make the
+// direct kernels queued behind them compute the result.
 __global__ __launch_bounds__(1024) void bwd_header_kernel(const uint32_t* __restrict__ lut_a, const uint32_t* __restrict__ lut_b,
-                                                          int lut_dwords, uint32_t* __restrict__ flags) {
+                                                          int lut_dwords, int n_entries, uint32_t* __restrict__ flags) {
     __shared__ int extremes[4];
+    __shared__ float magnitude[2];
     if (threadIdx.x < 4) extremes[threadIdx.x] = 0;
+    if (threadIdx.x < 2) magnitude[threadIdx.x] = 0.f;
     __syncthreads();
     // all loads of both tables are issued before the first is used (one dependent load at a time would pay the
     // memory latency 66 times: 19 us instead of 5)
@@ -475,38 +483,55 @@ __global__ __launch_bounds__(1024) void bwd_header_kernel(const uint32_t* __rest
         }
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
-            int lo = 0, hi = 0;
+            int lo = 0, hi = 0, mag = 0;
 #pragma unroll
             for (int i = 0; i < PER; ++i) {
                 const int v0 = (int)(int16_t)(w[t][i] & 0xffffu), v1 = (int)(int16_t)(w[t][i] >> 16);
                 lo = min(lo, min(v0, v1));
                 hi = max(hi, max(v0, v1));
+                mag += abs(v0) + abs(v1);
             }
 #pragma unroll
             for (int o = 32; o > 0; o >>= 1) {
                 lo = min(lo, __shfl_xor(lo, o));
                 hi = max(hi, __shfl_xor(hi, o));
+                mag += __shfl_xor(mag, o);           // at most 64 lanes x 18 entries x 32768: fits 32 bits
             }
             if ((threadIdx.x & 63) == 0) {
                 atomicMin(&extremes[2 * t], lo);
                 atomicMax(&extremes[2 * t + 1], hi);
+                atomicAdd(&magnitude[t], (float)mag);
             }
         }
     }
     __syncthreads();
     if (threadIdx.x < 64) {
-        uint32_t v = 0;
-        if (threadIdx.x == 3 || threadIdx.x == 4) {
-            const int t = threadIdx.x - 3;
-            v = (extremes[2 * t] >= -2048 && extremes[2 * t + 1] <= 2048) ? 0u : 1024u;
+        int off[2], unusable[2];
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            const int lo = extremes[2 * t], hi = extremes[2 * t + 1];
+            off[t] = 0;
+            unusable[t] = 0;
+            if (lo < -2048 || hi > 2048) {
+                if (hi - lo > 4096) unusable[t] = 1;
+                else off[t] = hi > 2048 ? hi - 2048 : lo + 2048;
+                if ((float)abs(off[t]) * (float)n_entries > 8.f * magnitude[t]) unusable[t] = 1;
+            }
+            if (unusable[t]) off[t] = 0;
         }
-        flags[threadIdx.x] = v;
+        uint32_t v = 0;
+        const int i = threadIdx.x;
+        if (i == 3) v = (uint32_t)off[0];
+        if (i == 4) v = (uint32_t)off[1];
+        if (i == 5 || i == 2) v = lut_a ? (uint32_t)unusable[0] : 0u;
+        if (i == 6 || i == 1) v = lut_b ? (uint32_t)unusable[1] : 0u;
+        flags[i] = v;
     }
 }
 
 hipError_t launch_bwd_header(const int16_t* lut_a, const int16_t* lut_b, const LutGeom& g, uint32_t* flags, hipStream_t stream) {
     hipLaunchKernelGGL(bwd_header_kernel, dim3(1), dim3(1024), 0, stream, reinterpret_cast<const uint32_t*>(lut_a),
-                       reinterpret_cast<const uint32_t*>(lut_b), g.rows * g.cols / 2, flags);
+                       reinterpret_cast<const uint32_t*>(lut_b), g.rows * g.cols / 2, (1 << g.bits) * (1 << g.bits), flags);
     return hipGetLastError();
 }
 

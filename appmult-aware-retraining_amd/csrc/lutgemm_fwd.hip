@@ -135,12 +135,8 @@ static hipError_t launch_fwd_t(const uint8_t* A, const uint8_t* B, uint32_t* C, 
     const int lut_dwords = g.rows * g.cols / 2;  // rows*cols is even for every supported bit-width
     const size_t lds = (size_t)lut_dwords * 4;
     auto kern = lutgemm_fwd_kernel<R, TN, WAVES>;
-    static bool attr_done = false;
-    if (!attr_done) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-        if (e != hipSuccess) return e;
-        attr_done = true;
-    }
+    static std::atomic<uint64_t> attr_done{0};
+    if (hipError_t ea = allow_full_lds(reinterpret_cast<const void*>(kern), attr_done); ea != hipSuccess) return ea;
     const int k_chunk = ((K + ksplit - 1) / ksplit + 3) & ~3;
     const int zs = (K + k_chunk - 1) / k_chunk;
     // (column tiles x row blocks folded into x: a grid may be 65535 workgroups along y, and M / 64 can exceed that)

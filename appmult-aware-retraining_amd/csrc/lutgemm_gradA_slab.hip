@@ -63,7 +63,8 @@ __global__ __launch_bounds__(256) void expand_gradA_kernel(const uint8_t* __rest
                                                            uint32_t* __restrict__ S, uint32_t* __restrict__ flags, int K, int N, int quads_per_wg) {
     extern __shared__ __align__(16) unsigned char smem[];
     uint32_t* s32 = reinterpret_cast<uint32_t*>(smem);
-    const float offset = (float)flags[3];        // 0 or 1024, decided from the table's extremes by bwd_header_kernel
+    if (flags[5] != 0u) return;                  // the table cannot be held as halves (bwd_header_kernel): the direct kernel does it
+    const float offset = (float)(int)flags[3];   // decided from the table's extremes by bwd_header_kernel
     // The table goes to LDS as halves, converted once per workgroup; what is left per entry of S is two 16-bit LDS
     // reads, one shift-or and the store (the kernel writes 256 B per code and k quad and should run at the speed of
     // the writes: 6.8 TB/s measured for a plain fill).
@@ -211,7 +212,8 @@ __global__ __launch_bounds__(kGaWaves * 64) void lutgemm_gradA_slab_kernel(
     const int xcd = (int)(blockIdx.x % 8), pos_stride = (int)(gridDim.x / 8);
     const int n_tiles = N / COLS;
     const int total = n_tiles * CH;                          // chunks of a tile: (column tile, four k)
-    const float offset = F32 ? 0.f : (float)flags[3];
+    if (!F32 && flags[5] != 0u) return;                      // (set before this launch and never changed during it: every wave sees the same)
+    const float offset = F32 ? 0.f : (float)(int)flags[3];
     struct Tile { int k0, m_wave; bool valid; };
     auto decode = [&](int pos) {
         Tile t;
@@ -663,13 +665,8 @@ hipError_t launch_gradA_slab_f32tab(const float* gC, const uint8_t* A, const uin
                                     int rows_per_image, hipStream_t stream) {
     if (((uintptr_t)gC & 15) != 0) return hipErrorInvalidValue;   // callers check: rows of gC are fetched 16 bytes at a time
     const int lut_entries = g.rows * g.cols;
-    static bool attr_done = false;
-    if (!attr_done) {
-        hipError_t ea = hipFuncSetAttribute(reinterpret_cast<const void*>(expand_gradA_f32_kernel),
-                                            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-        if (ea != hipSuccess) return ea;
-        attr_done = true;
-    }
+    static std::atomic<uint64_t> attr_done{0};
+    if (hipError_t ea = allow_full_lds(reinterpret_cast<const void*>(expand_gradA_f32_kernel), attr_done); ea != hipSuccess) return ea;
     const int qpw = 4;
     hipLaunchKernelGGL(expand_gradA_f32_kernel, dim3(N / kGaColsF32, (K / 4 + qpw - 1) / qpw), dim3(256), (size_t)lut_entries * 4,
                        stream, B, lut, lut_entries, g.cols, 1 << g.bits, reinterpret_cast<uint32_t*>(S), K, N, qpw);

@@ -15,7 +15,8 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ float quant_code(float x, float s, float zp, float qmax, bool* inside) {
     const float r = rintf(x / s - zp);          // round half to even, as torch.round
     *inside = (r >= 0.f) && (r <= qmax);
-    return fminf(fmaxf(r, 0.f), qmax);
+    // (a NaN stays a NaN, as in torch.clamp; fminf / fmaxf alone would turn it into a code)
+    return r != r ? r : fminf(fmaxf(r, 0.f), qmax);
 }
 
 __global__ __launch_bounds__(256) void quantize_codes_kernel(const float* __restrict__ x, const float* __restrict__ scale,
@@ -75,8 +76,10 @@ __global__ void observer_update_kernel(const float* __restrict__ cur_min, const 
     if (threadIdx.x != 0 || blockIdx.x != 0) return;
     float lo = *cur_min, hi = *cur_max;
     if (mode == 1) {
-        lo = fminf(lo, *min_val);
-        hi = fmaxf(hi, *max_val);
+        // torch.min / torch.max hand a NaN on; fminf / fmaxf would drop it
+        const float old_lo = *min_val, old_hi = *max_val;
+        lo = (lo != lo || old_lo != old_lo) ? __builtin_nanf("") : fminf(lo, old_lo);
+        hi = (hi != hi || old_hi != old_hi) ? __builtin_nanf("") : fmaxf(hi, old_hi);
     } else if (mode == 2) {
         lo = __fadd_rn(__fmul_rn(keep, *min_val), __fmul_rn(momentum, lo));
         hi = __fadd_rn(__fmul_rn(keep, *max_val), __fmul_rn(momentum, hi));
@@ -85,7 +88,8 @@ __global__ void observer_update_kernel(const float* __restrict__ cur_min, const 
     *max_val = hi;
     // (a division by a host-side scalar is a multiplication by its rounded reciprocal in the tensor library: inv_qmax != 0)
     const float range = __fsub_rn(hi, lo);
-    const float s = fmaxf(inv_qmax != 0.f ? __fmul_rn(range, inv_qmax) : __fdiv_rn(range, qmax), eps);
+    const float raw = inv_qmax != 0.f ? __fmul_rn(range, inv_qmax) : __fdiv_rn(range, qmax);
+    const float s = raw != raw ? raw : fmaxf(raw, eps);
     *scale = s;
     *zp_neg = rintf(__fdiv_rn(lo, s));
 }

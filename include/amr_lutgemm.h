@@ -61,8 +61,9 @@ int amr_lut_gemm_forward(const uint8_t *A, const uint8_t *B, uint32_t *C, const 
  * Same operation with caller-provided scratch.  For large M and tables of at most 7 bits the forward
  * pass first expands the table along B (E[k][a][n] = lut[a][B[k,n]]) into `workspace` and then adds
  * rows of E; amr_lut_gemm_forward_workspace_bytes gives the size that needs (0 = no scratch used for
- * this shape).  workspace must be 256-byte aligned; NULL makes the library use its own per-device
- * buffer, grown with hipMalloc when needed (amr_lut_gemm_forward does exactly that).
+ * this shape).  workspace must be 256-byte aligned; NULL makes the library use its own buffer for this
+ * (device, stream), grown with hipMalloc when needed and never freed or waited for (amr_lut_gemm_forward does
+ * exactly that; see amr_lut_gemm_backward for the rules).
  * No counterpart in the reference, whose forward kernel needs no scratch.
  */
 size_t amr_lut_gemm_forward_workspace_bytes(int64_t lut_elems, int M, int K, int N);
@@ -90,12 +91,18 @@ int amr_lut_gemm_forward_f32_ws(const uint8_t *A, const uint8_t *B, float *C, co
  *   gC [M,N] fp32   A [M,K] uint8   B [K,N] uint8   gA [M,K] fp32 (overwritten)   gB [K,N] fp32 (overwritten)
  *   lut_grad_a / lut_grad_b: padded tables, int16 (slope x 16), length lut_elems, 4-byte aligned.
  * gA or gB may be NULL to skip that gradient (extension; the reference computes both).
- * workspace: device scratch for the split-M partial sums of gB, at least
+ * workspace: device scratch for the split-M partial sums of gB and the expanded table of gradA, at least
  *   amr_lut_gemm_backward_workspace_bytes(M,K,N) bytes, 256-byte aligned; or NULL, in which case the
- *   library keeps a per-device buffer that it grows with hipMalloc when needed (not stream-safe
- *   across concurrent streams; pass a workspace for that).
+ *   library uses a buffer of its own, one per (device, stream): calls on one stream share it in stream order,
+ *   calls on different streams (also from different host threads) never do.  The library grows such a buffer with
+ *   hipMalloc when a call needs more than any earlier call on that stream did, keeps the old one until the
+ *   process ends (queued work may still use it) and never waits for the device.  hipMalloc cannot run while the
+ *   stream is being captured into a graph: capture with a workspace, or after an uncaptured call of the same size.
  */
 size_t amr_lut_gemm_backward_workspace_bytes(int M, int K, int N);
+/* The same for a known table width (lut_elems as passed to the call): 8-bit tables never use the expanded table of gradA,
+ * so this answer can be much smaller; the shape-only query above is an upper bound over all widths. */
+size_t amr_lut_gemm_backward_workspace_bytes_for(int64_t lut_elems, int M, int K, int N);
 int amr_lut_gemm_backward(const float *gC, const uint8_t *A, const uint8_t *B, float *gA, float *gB,
                           const int16_t *lut_grad_a, const int16_t *lut_grad_b, int64_t lut_elems,
                           int M, int K, int N, void *workspace, size_t workspace_bytes, void *stream);
@@ -126,6 +133,7 @@ int amr_lut_gemm_backward_ex(const float *gC, const uint8_t *A, const uint8_t *B
  * of gradA, twice the size of the int16 path's).
  */
 size_t amr_lut_gemm_backward_f32tab_workspace_bytes(int M, int K, int N);
+size_t amr_lut_gemm_backward_f32tab_workspace_bytes_for(int64_t lut_elems, int M, int K, int N);   /* for a known table width */
 int amr_lut_gemm_backward_f32tab(const float *gC, const uint8_t *A, const uint8_t *B, float *gA, float *gB,
                                  const float *lut_grad_a, const float *lut_grad_b, int64_t lut_elems, float scale,
                                  int M, int K, int N, int ga_rows_per_image, void *workspace, size_t workspace_bytes,

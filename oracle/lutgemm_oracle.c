@@ -113,6 +113,39 @@ void oracle_lutgemm_backward_f64(const float *gC, const uint8_t *A, const uint8_
     }
 }
 
+/* gB alone, same float64 sums as oracle_lutgemm_backward_f64 (self_ops/src/approx_gemm_backward.cu:447-461
+ * accumulate, :469-475 scale), walking A and gC row by row so that layers with hundreds of thousands of rows
+ * finish in seconds: every thread owns a block of k and keeps its [k][n] sums; the order of the additions over m
+ * is the reference's (m ascending).  Pinned by tests/test_oracle.py against oracle_lutgemm_backward_f64. */
+void oracle_lutgemm_gradB_f64_rows(const float *gC, const uint8_t *A, const uint8_t *B, double *gB, double *absB,
+                                   const double *lutB, int lut_cols, double factor, int M, int K, int N) {
+    const int KB = 8;
+#pragma omp parallel for schedule(dynamic, 1)
+    for (int kb = 0; kb < K; kb += KB) {
+        const int ke = kb + KB < K ? kb + KB : K;
+        double *acc = (double *)calloc((size_t)2 * KB * N, sizeof(double));
+        for (int m = 0; m < M; ++m) {
+            const float *g = gC + (size_t)m * N;
+            for (int k = kb; k < ke; ++k) {
+                const double *lrow = lutB + (size_t)A[(size_t)m * K + k] * lut_cols;
+                const uint8_t *brow = B + (size_t)k * N;
+                double *s = acc + (size_t)2 * (k - kb) * N;
+                for (int n = 0; n < N; ++n) {
+                    const double t = lrow[brow[n]] * (double)g[n];
+                    s[n] += t;
+                    s[N + n] += fabs(t);
+                }
+            }
+        }
+        for (int k = kb; k < ke; ++k)
+            for (int n = 0; n < N; ++n) {
+                gB[(size_t)k * N + n] = acc[(size_t)2 * (k - kb) * N + n] * factor;
+                if (absB) absB[(size_t)k * N + n] = acc[(size_t)2 * (k - kb) * N + N + n] * factor;
+            }
+        free(acc);
+    }
+}
+
 /* Accurate fp32 GEMM C = A.B, sequential fp32 FMA over k
  * (self_ops/src/approx_gemm_forward.cu:456-470). */
 void oracle_accgemm_forward_f32(const float *A, const float *B, float *C, int M, int K, int N) {

@@ -320,6 +320,22 @@ def backward_c_f64(gC, A, B, lutA_flat, lutB_flat, bits, factor=FACTOR, want_abs
     return gA, gB
 
 
+def gradB_c_f64_rows(gC, A, B, lutB_flat, bits, factor=FACTOR):
+    """gB and the sums of |terms| of gB in float64 for layers with very many rows (row-streaming loop order)."""
+    rows, cols, elems = geometry(bits)
+    gC = np.ascontiguousarray(gC, np.float32)
+    A = np.ascontiguousarray(A, np.uint8)
+    B = np.ascontiguousarray(B, np.uint8)
+    lb = np.ascontiguousarray(lutB_flat, np.float64)
+    M, K = A.shape
+    N = B.shape[1]
+    gB = np.empty((K, N), np.float64)
+    aB = np.empty((K, N), np.float64)
+    c_lib().oracle_lutgemm_gradB_f64_rows(_p(gC), _p(A), _p(B), _p(gB), _p(aB), _p(lb), ctypes.c_int(cols),
+                                          ctypes.c_double(factor), ctypes.c_int(M), ctypes.c_int(K), ctypes.c_int(N))
+    return gB, aB
+
+
 def accgemm_c(A, B):
     A = np.ascontiguousarray(A, np.float32)
     B = np.ascontiguousarray(B, np.float32)

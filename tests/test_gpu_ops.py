@@ -316,20 +316,25 @@ def test_fused_quantiser_equals_torch_expression(ops, shape):
     x = (torch.randn(shape, device="cuda", generator=g) * 3).requires_grad_()
     with torch.no_grad():
         x.view(-1)[::5] = (torch.arange(x.numel(), device="cuda")[::5] % 200 - 30).float() * 0.05 + 0.025   # ties after scaling
+        # non-finite inputs: torch.clamp hands a NaN on and sends the infinities to the ends of the range
+        x.view(-1)[7], x.view(-1)[x.numel() // 2], x.view(-1)[-3] = float("nan"), float("inf"), float("-inf")
     scale, zp = torch.tensor([0.05], device="cuda"), torch.tensor([-17.0], device="cuda")
     x2 = x.detach().clone().requires_grad_()
     y = app_layers._to_codes(x, scale, zp, 127.0)
     y2 = app_layers._to_codes_torch(x2, scale, zp, 127.0)
-    assert torch.equal(y, y2) and y.min() >= 0 and y.max() <= 127
+    assert torch.equal(torch.isnan(y), torch.isnan(y2)) and int(torch.isnan(y).sum()) == 1
+    assert torch.equal(torch.nan_to_num(y, nan=-1.0), torch.nan_to_num(y2, nan=-1.0))
+    assert torch.nan_to_num(y, nan=0.0).min() >= 0 and torch.nan_to_num(y, nan=0.0).max() <= 127
     gy = torch.randn(shape, device="cuda", generator=g)
     y.backward(gy)
     y2.backward(gy)
-    assert torch.equal(x.grad, x2.grad)
+    assert torch.equal(torch.nan_to_num(x.grad, nan=-7.0), torch.nan_to_num(x2.grad, nan=-7.0))
     assert (x.grad == 0).any() and (x.grad != 0).any()
     # non-contiguous input
     if len(shape) == 4:
         xt = x.detach().transpose(1, 3)
-        assert torch.equal(app_layers._to_codes(xt, scale, zp, 127.0), app_layers._to_codes_torch(xt, scale, zp, 127.0))
+        assert torch.equal(torch.nan_to_num(app_layers._to_codes(xt, scale, zp, 127.0), nan=-1.0),
+                           torch.nan_to_num(app_layers._to_codes_torch(xt, scale, zp, 127.0), nan=-1.0))
 
 
 def test_acc_gemm_op(ops):
@@ -387,6 +392,36 @@ def test_approx_conv_layer_equals_fake_quant_conv_with_exact_multiplier(ops, ora
                 torch.testing.assert_close(a, b, rtol=1e-5, atol=1e-6)
     finally:
         P.lut_appmult, P.lut_grad_a, P.lut_grad_b = keep
+
+
+def test_two_training_forwards_before_one_backward_keep_their_own_scales(ops):
+    """A layer called twice in training mode before backward (shared layer, two-view losses): the second call moves the
+    observers, and the graph of the first call must still use the scale and zero point it was built with -- the reference
+    binds new tensors on every forward (app_layers.py:154-160).  Checked against the same computation with every
+    quantisation step written in torch operators."""
+    import app_layers as L
+    print("two forwards, one backward", flush=True)
+    torch.manual_seed(3)
+    fused = L.ApproxConv2d(5, 12, 3, padding=1, bias=True, a_bits=7, w_bits=7).cuda().train()
+    plain = L.ApproxConv2d(5, 12, 3, padding=1, bias=True, a_bits=7, w_bits=7).cuda().train()
+    plain.load_state_dict(fused.state_dict())
+    plain.fused_dequant = False
+    plain.quantize_v2 = lambda x, s, z, q: L._to_codes_torch(x, s, z, q)       # torch operators all the way
+    plain.activation_observer.fused_mode = None
+    plain.weight_observer.fused_mode = None
+    x1 = torch.randn(4, 5, 9, 9, device="cuda")
+    x2 = torch.randn(4, 5, 9, 9, device="cuda") * 3 + 1                        # a different range: the second call moves the scale
+    res = []
+    for layer in (fused, plain):
+        a, b = x1.clone().requires_grad_(), x2.clone().requires_grad_()
+        y1 = layer(a)
+        s_first = layer.activation_scale.clone()
+        y2 = layer(b)
+        assert not torch.equal(layer.activation_scale, s_first)
+        (y1.square().mean() + y2.square().mean()).backward()
+        res.append((y1.detach(), y2.detach(), a.grad, b.grad, layer.weight.grad, layer.bias.grad))
+    for u, v in zip(*res):
+        torch.testing.assert_close(u, v, rtol=1e-4, atol=1e-6 * float(v.abs().max()) + 1e-12)
 
 
 def test_synthetic_training_steps_reduce_loss(ops, golden_dir):
@@ -501,9 +536,16 @@ def test_one_launch_observer_update_equals_tensor_expressions(ops, kind, qmax_on
         x = torch.randn(64, 33, device="cuda", generator=g) * (1 + step) + 0.3 * step
         s1, z1 = L._observe(fused, x, qmax, eps, sc, zp)
         s2, z2 = L._observe(plain, x, qmax, eps, None, None)
-        assert s1.data_ptr() == sc.data_ptr()                 # updated in place
+        assert s1.data_ptr() != sc.data_ptr() and float(sc) == 1.0 and float(zp) == 0.0   # new tensors: graphs of earlier passes keep theirs
         assert torch.equal(s1.reshape(1), s2.reshape(1)) and torch.equal(z1.reshape(1), z2.reshape(1)), step
         assert torch.equal(fused.min_val.reshape(1), plain.min_val.reshape(1)) and torch.equal(fused.max_val.reshape(1), plain.max_val.reshape(1))
+    # a NaN in the data reaches the range, the scale and the zero point, as it does through torch.min / torch.max
+    x = torch.randn(40, device="cuda", generator=g)
+    x[3] = float("nan")
+    s1, z1 = L._observe(fused, x, qmax, eps, sc, zp)
+    s2, z2 = L._observe(plain, x, qmax, eps, None, None)
+    assert bool(torch.isnan(s1).all()) and bool(torch.isnan(s2).all()) and bool(torch.isnan(z1).all()) and bool(torch.isnan(z2).all())
+    assert bool(torch.isnan(fused.min_val).all()) and bool(torch.isnan(plain.min_val).all())
     x = torch.zeros(8, device="cuda")                         # constant input: scale falls back to eps
     fused2, plain2 = make().cuda(), make().cuda()
     plain2.fused_mode = None

@@ -188,6 +188,28 @@ def test_backward_c_f64_equals_numpy(oracle, bits):
     np.testing.assert_allclose(b, bn, rtol=1e-12, atol=1e-9)
 
 
+@pytest.mark.parametrize("bits,shape", [(7, (301, 19, 13)), (8, (64, 33, 70)), (6, (1000, 8, 5))])
+def test_row_streaming_gradB_equals_brute_force_and_ste_matmul(oracle, bits, shape):
+    # the loop order used for full-size layers: against the numpy brute force (asymmetric random table: catches a / b swapped),
+    # its |terms| sums against the same brute force on absolute values, and STE tables against the dense integer product
+    M, K, N = shape
+    rng = np.random.default_rng(80 + bits)
+    n = 1 << bits
+    A, B, _ = _rand_case(rng, M, K, N, bits)
+    Gb = rng.integers(-4000, 4000, (n, n))
+    g = rng.standard_normal((M, N)).astype(np.float32)
+    lb = oracle.pack_table(Gb, bits, np.int16)
+    b, ab = oracle.gradB_c_f64_rows(g, A, B, lb, bits)
+    _, bn = oracle.backward_np(g, A, B, Gb, Gb)
+    _, abn = oracle.backward_np(np.abs(g), A, B, np.abs(Gb), np.abs(Gb))
+    np.testing.assert_allclose(b, bn, rtol=1e-12, atol=1e-9)
+    np.testing.assert_allclose(ab, abn, rtol=1e-12, atol=1e-9)
+    gi = rng.integers(-8, 9, (M, N)).astype(np.float32)
+    _, Gy = oracle.ste_tables16(bits)
+    bs, _ = oracle.gradB_c_f64_rows(gi, A, B, oracle.pack_table(Gy, bits, np.int16), bits)
+    assert (bs == A.astype(np.int64).T @ gi.astype(np.int64)).all()
+
+
 def test_backward_ste_tables_reduce_to_dense_matmuls_bit_exact(oracle):
     # the author's known-answer idea (approx_ops.py:81-86): Gx = 16 b, Gy = 16 a  =>  gA = gC B^T, gB = A^T gC.
     # With small integer gC every fp32 partial sum is exact, so the fp32 oracle must match bit for bit.
