@@ -455,7 +455,7 @@ __global__ __launch_bounds__(256) void gradB_finish_kernel(const float* __restri
 // A half holds every integer of magnitude <= 2048.  offset (flags[3] for the table of gradA, flags[4] for the table of
 // gradB, as int32): 0 when the whole table lies in [-2048, 2048] (the correction term with the sums of gC then drops out
 // of the kernels); else the value of smallest magnitude that brings every entry into that range, max - 2048 or
-// min + 2048, when the table spans no more than 4096.  The kernels then compute sum g * (entry - offset) + offset * sum g,
+// min + 2048 (rounded up to a power of two when that still fits), when the table spans no more than 4096.  The kernels then compute sum g * (entry - offset) + offset * sum g,
 // whose rounding errors grow with |offset| while the true terms have the size of the entries: the offset is only taken
 // when |offset| <= 8 x the mean magnitude of the entries.  A table that fails either test is not held as halves at all:
 // flags[5] (gradA) / flags[6] (gradB) tell the expanded-table kernels to leave at once, and flags[2] / flags[1] make the
@@ -514,7 +514,16 @@ __global__ __launch_bounds__(1024) void bwd_header_kernel(const uint32_t* __rest
             unusable[t] = 0;
             if (lo < -2048 || hi > 2048) {
                 if (hi - lo > 4096) unusable[t] = 1;
-                else off[t] = hi > 2048 ? hi - 2048 : lo + 2048;
+                else {
+                    // the value of smallest magnitude that works, rounded up to a power of two when one fits: g * 2^j is
+                    // exact, so a row of zeros (the pad row a masked code reads) still sums to exactly -offset * sum g and
+                    // cancels against the correction term
+                    const int need = hi > 2048 ? hi - 2048 : -(lo + 2048), room = hi > 2048 ? lo + 2048 : -(hi - 2048);
+                    int p = 1;
+                    while (p < need) p <<= 1;
+                    const int mag_off = p <= room ? p : need;
+                    off[t] = hi > 2048 ? mag_off : -mag_off;
+                }
                 if ((float)abs(off[t]) * (float)n_entries > 8.f * magnitude[t]) unusable[t] = 1;
             }
             if (unusable[t]) off[t] = 0;

@@ -13,7 +13,10 @@ namespace amr {
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ float quant_code(float x, float s, float zp, float qmax, bool* inside) {
-    const float r = rintf(x / s - zp);          // round half to even, as torch.round
+    const float q = x / s - zp;
+    // round half to even, as torch.round; the reference's straight-through form q - q.detach() + round(q) turns an
+    // infinite q into a NaN (inf - inf), so does this
+    const float r = __builtin_isinf(q) ? __builtin_nanf("") : rintf(q);
     *inside = (r >= 0.f) && (r <= qmax);
     // (a NaN stays a NaN, as in torch.clamp; fminf / fmaxf alone would turn it into a code)
     return r != r ? r : fminf(fmaxf(r, 0.f), qmax);
