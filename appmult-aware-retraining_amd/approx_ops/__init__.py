@@ -57,6 +57,8 @@ _lib.amr_lut_gemm_backward_workspace_bytes_for.argtypes = [_i64, _i, _i, _i]
 _lib.amr_lut_gemm_backward_workspace_bytes_for.restype = _sz
 _lib.amr_lut_gemm_backward_f32tab_workspace_bytes_for.argtypes = [_i64, _i, _i, _i]
 _lib.amr_lut_gemm_backward_f32tab_workspace_bytes_for.restype = _sz
+_lib.amr_lut_gemm_backward_static.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i, _i, _i, _i, _vp]
+_lib.amr_static_scratch_bytes.restype = _sz
 _lib.amr_acc_gemm_forward_fp32.argtypes = [_vp, _vp, _vp, _i, _i, _i, _vp]
 _lib.amr_bits_from_lut_elems.argtypes = [_i64]
 _lib.amr_lut_geometry.argtypes = [_i, ctypes.POINTER(_i), ctypes.POINTER(_i), ctypes.POINTER(_i64)]

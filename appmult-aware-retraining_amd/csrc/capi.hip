@@ -99,6 +99,7 @@ struct StreamScratch {
 struct DeviceState {
     int n_cu = 0;
     std::vector<StreamScratch> scratch;
+    void* static_scratch = nullptr;     // address of the file-scope device array on this device (amr_lut_gemm_backward_static)
 };
 DeviceState g_dev[kMaxDevices];
 std::mutex g_mu;
@@ -269,8 +270,26 @@ int amr_lut_gemm_backward(const float* gC, const uint8_t* A, const uint8_t* B, f
                                     workspace_bytes, stream);
 }
 
+// File-scope scratch of amr_lut_gemm_backward_static: every device the library runs on holds its own copy until the
+// process ends.  Host code never uses the array's name as an address: static_scratch_ptr() asks the runtime once per
+// device where that device's copy lives.
+constexpr size_t kStaticScratchBytes = (size_t)AMR_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+static void* static_scratch_ptr(int dev, hipError_t* err) {
+    std::lock_guard<std::mutex> lk(g_mu);
+    *err = hipSuccess;
+    if (!g_dev[dev].static_scratch) {
+        void* p = nullptr;
+        *err = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));     // (the caller's device `dev` is current)
+        if (*err != hipSuccess) return nullptr;
+        g_dev[dev].static_scratch = p;
+    }
+    return g_dev[dev].static_scratch;
+}
+
 // where the scratch of a backward call comes from
-enum class ScratchFrom { Caller, Library };
+enum class ScratchFrom { Caller, Library, Static };
 
 static int backward_impl(const float* gC, const uint8_t* A, const uint8_t* B, float* gA, float* gB,
                          const int16_t* lut_grad_a, const int16_t* lut_grad_b, int64_t lut_elems, int M, int K,
@@ -302,9 +321,20 @@ static int backward_impl(const float* gC, const uint8_t* A, const uint8_t* B, fl
     const int mode = g_expanded_kernels.load();
     const size_t partial_bytes = backward_partial_bytes(M, K, N, n_cu);
     // (what this table width needs: never more than the shape-only query answers)
-    const size_t gradA_bytes = backward_gradA_bytes(mode, g.bits, M, K, N);
-    const bool allow_slab_a = true;
+    size_t gradA_bytes = backward_gradA_bytes(mode, g.bits, M, K, N);
+    bool allow_slab_a = true;
     void* ws = workspace;
+    if (from == ScratchFrom::Static) {
+        if (256 + partial_bytes + gradA_bytes > kStaticScratchBytes) {   // without the expanded table of gradA (direct kernel) it may still fit
+            gradA_bytes = 0;
+            allow_slab_a = false;
+        }
+        if (256 + partial_bytes > kStaticScratchBytes)
+            return fail(AMR_EWORKSPACE, "this shape needs %zu bytes of scratch, the static scratch holds %zu: use amr_lut_gemm_backward with a workspace",
+                        256 + partial_bytes, kStaticScratchBytes);
+        ws = static_scratch_ptr(dev, &e);
+        if (!ws) return hip_fail(e, "hipGetSymbolAddress(scratch)");
+    }
     const size_t need = 256 + partial_bytes + gradA_bytes;
     if (from == ScratchFrom::Caller) {
         if (workspace_bytes < need) return fail(AMR_EWORKSPACE, "workspace of %zu bytes is smaller than the %zu required", workspace_bytes, need);
@@ -346,6 +376,15 @@ int amr_lut_gemm_backward_ex(const float* gC, const uint8_t* A, const uint8_t* B
                              int N, int ga_rows_per_image, void* workspace, size_t workspace_bytes, void* stream) {
     return backward_impl(gC, A, B, gA, gB, lut_grad_a, lut_grad_b, lut_elems, M, K, N, ga_rows_per_image,
                          workspace ? ScratchFrom::Caller : ScratchFrom::Library, workspace, workspace_bytes, stream);
+}
+
+size_t amr_static_scratch_bytes(void) { return kStaticScratchBytes; }
+
+int amr_lut_gemm_backward_static(const float* gC, const uint8_t* A, const uint8_t* B, float* gA, float* gB,
+                                 const int16_t* lut_grad_a, const int16_t* lut_grad_b, int64_t lut_elems, int M, int K,
+                                 int N, int ga_rows_per_image, void* stream) {
+    return backward_impl(gC, A, B, gA, gB, lut_grad_a, lut_grad_b, lut_elems, M, K, N, ga_rows_per_image, ScratchFrom::Static,
+                         nullptr, 0, stream);
 }
 
 // Scratch of the float-table backward pass: [256 B of flags][partial sums of gB][float32 expanded table of gradA].

@@ -97,7 +97,8 @@ int amr_lut_gemm_forward_f32_ws(const uint8_t *A, const uint8_t *B, float *C, co
  *   calls on different streams (also from different host threads) never do.  The library grows such a buffer with
  *   hipMalloc when a call needs more than any earlier call on that stream did, keeps the old one until the
  *   process ends (queued work may still use it) and never waits for the device.  hipMalloc cannot run while the
- *   stream is being captured into a graph: capture with a workspace, or after an uncaptured call of the same size.
+ *   stream is being captured into a graph: capture with a workspace, after an uncaptured call of the same size,
+ *   or through amr_lut_gemm_backward_static.
  */
 size_t amr_lut_gemm_backward_workspace_bytes(int M, int K, int N);
 /* The same for a known table width (lut_elems as passed to the call): 8-bit tables never use the expanded table of gradA,
@@ -118,6 +119,21 @@ int amr_lut_gemm_backward_ex(const float *gC, const uint8_t *A, const uint8_t *B
                              const int16_t *lut_grad_a, const int16_t *lut_grad_b, int64_t lut_elems,
                              int M, int K, int N, int ga_rows_per_image, void *workspace, size_t workspace_bytes,
                              void *stream);
+
+/*
+ * amr_lut_gemm_backward_ex for callers that cannot allocate: code under HIP graph capture, tight serving loops, harnesses
+ * that forbid hipMalloc.  It has no counterpart in the reference.  Same arguments, results and kernels; the scratch
+ * (flags, partial sums of gB, expanded table of gradA) is a file-scope device array of AMR_STATIC_SCRATCH_BYTES inside the
+ * library, one copy per GPU, held until the process ends.  The call allocates and frees nothing.  A shape whose expanded
+ * table of gradA does not fit runs gradA on the direct kernel instead; a shape whose partial sums of gB alone exceed the
+ * array is rejected with AMR_EWORKSPACE.  All calls on one GPU share that array: calls that overlap in time on one
+ * GPU (two streams, two threads) race; calls queued on one stream do not.
+ */
+#define AMR_STATIC_SCRATCH_BYTES (32u << 20)
+size_t amr_static_scratch_bytes(void);
+int amr_lut_gemm_backward_static(const float *gC, const uint8_t *A, const uint8_t *B, float *gA, float *gB,
+                                 const int16_t *lut_grad_a, const int16_t *lut_grad_b, int64_t lut_elems,
+                                 int M, int K, int N, int ga_rows_per_image, void *stream);
 
 /*
  * Backward with float32 gradient tables: the same two sums with lut_grad_a / lut_grad_b holding the slopes themselves
