@@ -441,6 +441,48 @@ def test_synthetic_training_steps_reduce_loss(ops, golden_dir):
     assert all(np.isfinite(losses)) and losses[-1] < losses[0]
 
 
+def test_resnet18_batch512_training_step_expanded_kernels_agree_with_direct_kernels(ops):
+    """The training-step configuration (ResNet-18, batch 512, SGD, the shipped 7-bit table with its gradient tables): one
+    step -- forward, cross-entropy, backward, update -- of the same model state on the same batch, once with the library's own
+    kernel selection and once with the direct gather kernels only (the formulation the oracle tests pin shape by shape).
+    The forward pass is integer arithmetic, so the logits are bit-identical; every parameter gradient agrees norm-wise to
+    1e-5 (the two differ in summation order only, through 20 layers of backward)."""
+    import copy
+    import approx_ops
+    import app_train as T
+    print("resnet18 batch 512 step", flush=True)
+    dev = torch.device("cuda")
+    torch.manual_seed(7)
+    base = T.build_model("resnet18", 7, False, dev)
+    xs, ys = T.synthetic_batches(2, 512, dev, seed=3)
+    T.calibrate(base, xs[:1])
+    results = []
+    for mode in (1, 0):
+        model = copy.deepcopy(base)
+        opt = torch.optim.SGD(model.parameters(), lr=1e-2, momentum=0.9)
+        prev = approx_ops._lib.amr_set_expanded_table_kernels(mode)
+        try:
+            model.train()
+            opt.zero_grad()
+            logits = model(xs[1])
+            loss = torch.nn.functional.cross_entropy(logits, ys[1])
+            loss.backward()
+            grads = {n: p.grad.detach().clone() for n, p in model.named_parameters()}
+            opt.step()
+            torch.cuda.synchronize()
+        finally:
+            approx_ops._lib.amr_set_expanded_table_kernels(prev)
+        results.append((logits.detach(), grads, {n: p.detach().clone() for n, p in model.named_parameters()}))
+    (l1, g1, p1), (l0, g0, p0) = results
+    assert torch.equal(l1, l0) and bool(torch.isfinite(l1).all())
+    assert len(g1) > 60
+    for n in g0:
+        ref = g0[n].double()
+        assert float((g1[n].double() - ref).norm()) <= 1e-5 * float(ref.norm()) + 1e-30, n
+        assert float(ref.norm()) > 0, n
+        assert float((p1[n].double() - p0[n].double()).norm()) <= 1e-5 * float(p0[n].double().norm()) + 1e-30, n
+
+
 def test_training_harness_cli_with_float_gradient_tables(ops, golden_dir, tmp_path, capsys):
     """The command-line harness end to end on a small batch, with the file's int16 tables and with float32 slopes."""
     import gzip
