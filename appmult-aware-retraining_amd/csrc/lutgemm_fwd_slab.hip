@@ -1,4 +1,5 @@
-// Forward LUT-GEMM for large M on gfx950: "expanded-table" formulation (7-bit tables and narrower).
+// Forward LUT-GEMM for large M on gfx950: "expanded-table" formulation (7-bit tables and narrower; 8-bit tables: the
+// variant at the end of the file).
 //
 // Same result as lutgemm_fwd_kernel (and as the reference's ApproxGemmForwardKernel,
 // self_ops/src/approx_gemm_forward.cu:45-229), different work decomposition:
@@ -52,7 +53,7 @@ constexpr int kExpandQuadsPerWg = 4;
 __global__ __launch_bounds__(256) void expand_fwd_kernel(const uint8_t* __restrict__ B,
                                                          const uint32_t* __restrict__ lut32, int lut_dwords,
                                                          int lut_cols, int n_codes, uint32_t* __restrict__ E,
-                                                         uint32_t* __restrict__ flags, int K, int N, int k_quads) {
+                                                         uint32_t* __restrict__ flags, int K, int N, int k_quads, int chunk_rows) {
     extern __shared__ __align__(16) unsigned char smem[];
     uint32_t* s32 = reinterpret_cast<uint32_t*>(smem);
     uint32_t mx = 0;
@@ -96,11 +97,12 @@ __global__ __launch_bounds__(256) void expand_fwd_kernel(const uint8_t* __restri
     for (int qq = 0; qq < kExpandQuadsPerWg; ++qq) {
         const int q = blockIdx.y * kExpandQuadsPerWg + qq;
         if (q >= k_quads) break;
-        uint32_t* blk = E + ((size_t)blockIdx.x * k_quads + q) * (kSlabChunkBytes / 4) + lane;
+        // (a chunk holds chunk_rows codes, 256 B each: 128 for tables of at most 7 bits, 256 for 8-bit tables)
+        uint32_t* blk = E + ((size_t)blockIdx.x * k_quads + q) * (size_t)(chunk_rows * 64) + lane;
         const uint16_t* p0 = s16 + b0[qq];
         const uint16_t* p1 = s16 + b1[qq];
 #pragma unroll 8
-        for (int a = wave; a < kSlabRows; a += 4) {
+        for (int a = wave; a < chunk_rows; a += 4) {
             const int row = min(a, n_codes) * lut_cols;
             blk[a * 64] = (uint32_t)p0[row] | ((uint32_t)p1[row] << 16);
         }
@@ -110,11 +112,11 @@ __global__ __launch_bounds__(256) void expand_fwd_kernel(const uint8_t* __restri
 // Copies one 32 KB chunk of E from global memory straight into LDS (global_load_lds_dwordx4: the data
 // of lane l lands at the wave-uniform LDS base + 16*l; no VGPRs are held while the load is in flight).
 // Completion is tracked by vmcnt (two operations per thread and chunk with 1024 threads).
-template <int THREADS>
+template <int THREADS, int BYTES = kSlabChunkBytes>
 __device__ __forceinline__ void slab_copy_chunk(const u32x4* src, unsigned char* lds_dst, int tid, int wave) {
     typedef const __attribute__((address_space(1))) void* gptr_t;
     typedef __attribute__((address_space(3))) void* lptr_t;
-    constexpr int CPT = kSlabChunkBytes / 16 / THREADS;
+    constexpr int CPT = BYTES / 16 / THREADS;
 #pragma unroll
     for (int i = 0; i < CPT; ++i) {
         const u32x4* g = src + tid + THREADS * i;
@@ -385,6 +387,114 @@ __global__ __launch_bounds__(WAVES * 64) void lutgemm_fwd_slab_kernel(
     }
 }
 
+// ------------------------------------------------------------------------------------------ 8-bit tables
+// The same scheme for 256 codes: a chunk (four k, 32 columns) is 256 lines of 256 B = 64 KB, the code byte still
+// lands in byte 1 of the LDS address through the one v_perm_b32, and the chunk buffer is picked by byte 2.  Two chunk
+// buffers and the code staging fill the 160 KB of a CU exactly, so a chunk is requested one chunk period ahead only
+// (chunk c+1 when chunk c starts): the kernel runs at the pace the chunks arrive (0.5 B per multiply-add, twice the
+// volume of the 7-bit kernel).  Every code of a uint8 operand has its line: no masked code, no fall-back.
+constexpr int kSlab8Rows = 256;
+constexpr int kSlab8ChunkBytes = kSlab8Rows * 256;   // 64 KB
+
+template <bool PACKED>
+__global__ __launch_bounds__(1024) void lutgemm_fwd_slab8_kernel(
+    const uint8_t* __restrict__ A, const u32x4* __restrict__ E, uint32_t* __restrict__ C,
+    const uint32_t* __restrict__ flags, int M, int K, int N, int k_quads, int chunks_per_split, int atomic_out, int out_f32) {
+    __shared__ __align__(16) unsigned char smem[2 * kSlab8ChunkBytes + 2 * kSlabCodeBytes];
+    constexpr int RG = 8, WAVES = 16, THREADS = WAVES * 64, ROWS_PER_WAVE = 8 * RG;
+    static_assert(2 * kSlab8ChunkBytes + 2 * kSlabCodeBytes == 160 * 1024, "the workgroup uses the whole LDS of a CU");
+    const int tid = threadIdx.x;
+    const int wave = uniform(tid >> 6);
+    const int lane = tid & 63;
+    const int rs = lane >> 3, cg = lane & 7, rot = rs & 3;
+    const int tile_x = blockIdx.x, rb_y = blockIdx.y, split_z = blockIdx.z;
+    // (a wave whose rows would stick out of M is shifted up; the rows it shares with the wave above are stored once)
+    const int m_first = (rb_y * WAVES + wave) * ROWS_PER_WAVE;
+    const int m_wave = min(m_first, M - ROWS_PER_WAVE);
+    const int c_begin = split_z * chunks_per_split;
+    const int c_end = min(k_quads, c_begin + chunks_per_split);
+    if (c_begin >= c_end) return;
+    if ((flags[0] < 16384u) != PACKED) return;     // both flavours are queued; the table maximum picks one
+
+    const u32x4* Eblk = E + ((size_t)tile_x * k_quads) * (kSlab8ChunkBytes / 16);
+    // instruction j of a chunk reads k = 4c + ((j + rot) & 3); byte 2 of the address = chunk buffer
+    uint32_t base0[4], base1[4], sel[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const uint32_t kk = (uint32_t)((j + rot) & 3);
+        base0[j] = (kk << 6) | (uint32_t)(cg << 3);
+        base1[j] = base0[j] | 0x10000u;
+        sel[j] = 0x0c020000u | ((4u + kk) << 8);
+    }
+    uint32_t acc[RG][4];
+#pragma unroll
+    for (int i = 0; i < RG; ++i)
+#pragma unroll
+        for (int c = 0; c < 4; ++c) acc[i][c] = 0u;
+
+    // codes: as in the 7-bit kernel (16 bytes = four chunks per row and request, staged so that a lane's eight rows are
+    // 128 B apart)
+    const uint32_t code_off = (uint32_t)(m_wave + 8 * (lane & 7) + (lane >> 3)) * (uint32_t)K;
+    unsigned char* code_stage = smem + 2 * kSlab8ChunkBytes + wave * 1024;
+    const uint32_t code_read = (uint32_t)(2 * kSlab8ChunkBytes + wave * 1024 + rs * 16);
+    typedef const __attribute__((address_space(1))) void* gptr_t;
+    typedef __attribute__((address_space(3))) void* lptr_t;
+    const int g_last = (c_end - 1 - c_begin) >> 2;
+    auto group_koff = [&](int g) { return min(4 * (c_begin + 4 * min(g, g_last)), K - 16); };
+    auto request_codes = [&](int g) {
+        __builtin_amdgcn_global_load_lds((gptr_t)(A + (code_off + (uint32_t)group_koff(g))),
+                                         (lptr_t)(code_stage + (g & 1) * kSlabCodeBytes), 16, 0, 0);
+    };
+    auto request_chunk = [&](int c, int buf) {
+        slab_copy_chunk<THREADS, kSlab8ChunkBytes>(Eblk + (size_t)min(c, c_end - 1) * (kSlab8ChunkBytes / 16),
+                                                   smem + (size_t)buf * kSlab8ChunkBytes, tid, wave);
+    };
+    // Operations of a thread towards memory, in issue order: codes(0) chunk(c0) | step c: [codes(g+1) in the first step of
+    // a group] chunk(c+1).  At the top of a step everything issued so far must have landed (chunk c was the last request of
+    // the previous step); behind the barrier every wave has finished reading the buffer the next request overwrites.
+    request_codes(0);
+    request_chunk(c_begin, 0);
+    auto step = [&](int c, int g, auto buf_tag, bool first_of_group) {
+        constexpr int BUF = decltype(buf_tag)::value;
+        asm volatile("s_waitcnt vmcnt(0)\n s_barrier" ::: "memory");
+        if (first_of_group) request_codes(g + 1);
+        request_chunk(c + 1, BUF ^ 1);
+        uint32_t mine[RG];
+        slab_read_codes(mine, code_read + (uint32_t)((g & 1) * kSlabCodeBytes + (4 * c - group_koff(g))));
+        if (BUF)
+            slab_chunk_fast<RG, PACKED, 0>(acc, mine, base1, sel);
+        else
+            slab_chunk_fast<RG, PACKED, 0>(acc, mine, base0, sel);
+    };
+    // (chunk c of the split sits in buffer (c - c_begin) & 1; a group of codes covers four chunks)
+    for (int c = c_begin, g = 0; c < c_end; c += 4, ++g) {
+        step(c, g, std::integral_constant<int, 0>{}, true);
+        if (c + 1 < c_end) step(c + 1, g, std::integral_constant<int, 1>{}, false);
+        if (c + 2 < c_end) step(c + 2, g, std::integral_constant<int, 0>{}, false);
+        if (c + 3 < c_end) step(c + 3, g, std::integral_constant<int, 1>{}, false);
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // nothing is left in flight towards LDS when the workgroup ends
+
+    const int n = tile_x * kSlabCols + 4 * cg;
+#pragma unroll
+    for (int i = 0; i < RG; ++i) {
+        const int m = m_wave + 8 * rs + i;
+        if (m >= m_first) {
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                if (n + c < N) {
+                    if (atomic_out)
+                        atomicAdd(&C[(size_t)m * N + n + c], acc[i][c]);
+                    else if (out_f32)
+                        C[(size_t)m * N + n + c] = __float_as_uint((float)acc[i][c]);
+                    else
+                        C[(size_t)m * N + n + c] = acc[i][c];
+                }
+            }
+        }
+    }
+}
+
 hipError_t launch_fwd_gated(const uint8_t* A, const uint8_t* B, uint32_t* C, const uint16_t* lut, const LutGeom& g,
                             int M, int K, int N, const uint32_t* gate, hipStream_t stream, int out_f32);
 
@@ -394,7 +504,13 @@ size_t fwd_slab_workspace_bytes(const LutGeom& g, int M, int K, int N, bool forc
     // Worth it when the 2^b/M expansion overhead is small and K is long enough to amortise the extra
     // launches (measured cross-over on MI355X: K around 512).
     // (K % 4 == 0: the codes of A are fetched four and sixteen at a time)
-    if (g.bits > 7 || M < 2048 || K < 512 || (K & 3) != 0 || (size_t)M * K >= (1ull << 31)) return 0;
+    if (M < 2048 || K < 512 || (K & 3) != 0 || (size_t)M * K >= (1ull << 31)) return 0;
+    if (g.bits == 8) {
+        // 8-bit tables: 64 KB per (column tile, four k); every block of 1024 rows streams all of it, so the rows have to
+        // outnumber the 256 codes well (measured against the direct kernel on MI355X)
+        if (!force && (M < 4096 || (size_t)M * K * N < (3ull << 29))) return 0;
+        return 256 + (size_t)((N + kSlabCols - 1) / kSlabCols) * (((size_t)K + 3) / 4) * kSlab8ChunkBytes;
+    }
     // below about 1.6e9 multiply-adds the extra launches (flags, expansion, second flavour, gated fall-back) cost
     // more than the faster kernel gains (measured cross-over on MI355X between 1.2e9 and 2.4e9)
     if (!force && (size_t)M * K * N < (3ull << 29)) return 0;
@@ -412,9 +528,36 @@ hipError_t launch_fwd_slab(const uint8_t* A, const uint8_t* B, uint32_t* C, cons
     hipError_t e = launch_zero_u32(flags, 64, stream);
     if (e != hipSuccess) return e;
     const int lut_dwords = g.rows * g.cols / 2;
+    if (g.bits == 8) {
+        static std::atomic<uint64_t> attr_done{0};
+        if ((e = allow_full_lds(reinterpret_cast<const void*>(expand_fwd_kernel), attr_done)) != hipSuccess) return e;
+        hipLaunchKernelGGL(expand_fwd_kernel, dim3(n_tiles, (k_quads + kExpandQuadsPerWg - 1) / kExpandQuadsPerWg), dim3(256),
+                           (size_t)lut_dwords * 4, stream, B, reinterpret_cast<const uint32_t*>(lut), lut_dwords, g.cols,
+                           1 << g.bits, E, flags, K, N, k_quads, kSlab8Rows);
+        if ((e = hipGetLastError()) != hipSuccess) return e;
+        const int row_blocks8 = (M + 1023) / 1024;
+        const long wgs8 = (long)n_tiles * row_blocks8;
+        int ksplit8 = 1;
+        if (wgs8 < n_cu) {
+            ksplit8 = (int)((n_cu + wgs8 - 1) / wgs8);
+            const int max_split = k_quads / 8 > 0 ? k_quads / 8 : 1;     // at least 32 k per workgroup
+            if (ksplit8 > max_split) ksplit8 = max_split;
+        }
+        const int cps8 = (k_quads + ksplit8 - 1) / ksplit8;
+        const int zs8 = (k_quads + cps8 - 1) / cps8;
+        if (zs8 > 1 && (e = launch_zero_u32(C, (size_t)M * N, stream)) != hipSuccess) return e;
+        const dim3 grid8(n_tiles, row_blocks8, zs8);
+        hipLaunchKernelGGL((lutgemm_fwd_slab8_kernel<true>), grid8, dim3(1024), 0, stream, A, reinterpret_cast<const u32x4*>(E), C, flags,
+                           M, K, N, k_quads, cps8, zs8 > 1 ? 1 : 0, out_f32);
+        hipLaunchKernelGGL((lutgemm_fwd_slab8_kernel<false>), grid8, dim3(1024), 0, stream, A, reinterpret_cast<const u32x4*>(E), C, flags,
+                           M, K, N, k_quads, cps8, zs8 > 1 ? 1 : 0, out_f32);
+        if ((e = hipGetLastError()) != hipSuccess) return e;
+        if (zs8 > 1 && out_f32) return launch_u32_to_f32(C, (size_t)M * N, stream);
+        return hipSuccess;
+    }
     hipLaunchKernelGGL(expand_fwd_kernel, dim3(n_tiles, (k_quads + kExpandQuadsPerWg - 1) / kExpandQuadsPerWg), dim3(256),
                        (size_t)lut_dwords * 4, stream, B, reinterpret_cast<const uint32_t*>(lut), lut_dwords, g.cols,
-                       1 << g.bits, E, flags, K, N, k_quads);
+                       1 << g.bits, E, flags, K, N, k_quads, kSlabRows);
     e = hipGetLastError();
     if (e != hipSuccess) return e;
 
