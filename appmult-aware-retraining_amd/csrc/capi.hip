@@ -96,9 +96,17 @@ struct StreamScratch {
     void* ptr;
     size_t bytes;
 };
+// A second stream and two events per (device, caller's stream): small backward calls run their gradB launches there,
+// beside the gradA launches on the caller's stream, and join the caller's stream again before the call returns.
+struct StreamFork {
+    hipStream_t stream;       // the caller's
+    hipStream_t side;
+    hipEvent_t forked, joined;
+};
 struct DeviceState {
     int n_cu = 0;
     std::vector<StreamScratch> scratch;
+    std::vector<StreamFork> forks;
     void* static_scratch = nullptr;     // address of the file-scope device array on this device (amr_lut_gemm_backward_static)
 };
 DeviceState g_dev[kMaxDevices];
@@ -139,6 +147,24 @@ void* internal_workspace(int dev, hipStream_t stream, size_t bytes, hipError_t* 
     return p;
 }
 
+// The side stream of `stream` on device `dev` (created on first use, default priority, kept until the process ends).
+bool stream_fork(int dev, hipStream_t stream, StreamFork* out) {
+    std::lock_guard<std::mutex> lk(g_mu);
+    DeviceState& d = g_dev[dev];
+    for (const StreamFork& f : d.forks)
+        if (f.stream == stream) { *out = f; return true; }
+    StreamFork f{stream, nullptr, nullptr, nullptr};
+    if (hipStreamCreateWithFlags(&f.side, hipStreamNonBlocking) != hipSuccess) return false;
+    if (hipEventCreateWithFlags(&f.forked, hipEventDisableTiming) != hipSuccess ||
+        hipEventCreateWithFlags(&f.joined, hipEventDisableTiming) != hipSuccess) {
+        (void)hipGetLastError();
+        return false;
+    }
+    d.forks.push_back(f);
+    *out = f;
+    return true;
+}
+
 }  // namespace
 
 extern "C" {
@@ -159,10 +185,14 @@ int amr_lut_geometry(int bits, int* rows, int* cols, int64_t* elem_num) {
 // Process-wide switch (diagnostics, tests, benchmarks): 0 sends every call to the direct gather kernels, 1 picks by
 // problem size, 2 takes the expanded-table kernels wherever the shape allows (also where they are slower).
 static std::atomic<int> g_expanded_kernels{1};
+// 1: small backward calls run gradB on a side stream beside gradA (amr_set_backward_fork)
+static std::atomic<int> g_fork_small{1};
 
 int amr_set_expanded_table_kernels(int mode) {
     return g_expanded_kernels.exchange(mode <= 0 ? 0 : (mode >= 2 ? 2 : 1));
 }
+
+int amr_set_backward_fork(int on) { return g_fork_small.exchange(on ? 1 : 0); }
 
 int amr_bits_from_lut_elems(int64_t lut_elems) {
     amr::LutGeom g;
@@ -352,22 +382,41 @@ static int backward_impl(const float* gC, const uint8_t* A, const uint8_t* B, fl
         e = amr::launch_bwd_header(slab_a ? lut_grad_a : nullptr, (slab && gB) ? lut_grad_b : nullptr, g, flags, s);
         if (e != hipSuccess) return hip_fail(e, "scratch header launch");
     }
+    // Small problems are bound by the latency of their launches (three or four dependent ones per gradient), not by
+    // arithmetic: the launches of gradB then go to a side stream and run beside those of gradA (the two gradients share
+    // inputs only; their parts of the scratch are disjoint), and the caller's stream waits for the side stream before
+    // the call returns, so that everything stays ordered with the caller's stream.
+    hipStream_t sb = s;
+    StreamFork fork{};
+    const bool forked = gA && gB && from != ScratchFrom::Static && (double)M * K * N < 2.0e9 && g_fork_small.load() &&
+                        stream_fork(dev, s, &fork);
+    if (forked) {
+        if ((e = hipEventRecord(fork.forked, s)) != hipSuccess || (e = hipStreamWaitEvent(fork.side, fork.forked, 0)) != hipSuccess)
+            return hip_fail(e, "side stream fork");
+        sb = fork.side;
+    }
     if (gA) {
         if (slab_a)
             e = amr::launch_gradA_slab(gC, A, B, gA, lut_grad_a, g, M, K, N, scale, n_cu, flags,
                                        reinterpret_cast<unsigned char*>(ws) + 256 + partial_bytes, ga_rows_per_image, s);
         else
             e = amr::launch_gradA(gC, A, B, gA, lut_grad_a, g, M, K, N, scale, n_cu, s, nullptr, ga_rows_per_image);
-        if (e != hipSuccess) return hip_fail(e, "gradA launch");
     }
-    if (gB) {
+    hipError_t eb = hipSuccess;
+    if (gB) {     // (queued also when the gradA launch failed: a forked side stream must be joined again either way)
         if (slab) {
-            e = amr::launch_gradB_slab(gC, A, B, gB, lut_grad_b, g, M, K, N, scale, flags, partials, n_cu, s);
+            eb = amr::launch_gradB_slab(gC, A, B, gB, lut_grad_b, g, M, K, N, scale, flags, partials, n_cu, sb);
         } else {
-            e = amr::launch_gradB(gC, A, B, gB, lut_grad_b, g, M, K, N, scale, partials, n_cu, s);
+            eb = amr::launch_gradB(gC, A, B, gB, lut_grad_b, g, M, K, N, scale, partials, n_cu, sb);
         }
-        if (e != hipSuccess) return hip_fail(e, "gradB launch");
     }
+    if (forked) {
+        hipError_t ej;
+        if ((ej = hipEventRecord(fork.joined, fork.side)) != hipSuccess || (ej = hipStreamWaitEvent(s, fork.joined, 0)) != hipSuccess)
+            return hip_fail(ej, "side stream join");
+    }
+    if (gA && e != hipSuccess) return hip_fail(e, "gradA launch");
+    if (eb != hipSuccess) return hip_fail(eb, "gradB launch");
     return AMR_OK;
 }
 

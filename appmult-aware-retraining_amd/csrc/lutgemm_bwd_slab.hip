@@ -560,11 +560,11 @@ bool bwd_slab_applies(const LutGeom& g, int M, int K, int N) {
 
 // M splits of the expanded-table gradB.  A workgroup fills a CU (128 KB of LDS), so the grid runs in rounds
 // of n_cu workgroups: pick the split count whose (rounds x rows per workgroup) is smallest, charging every
-// workgroup the cost of expanding its slabs (about that of streaming 512 rows) and keeping at least 2048
+// workgroup the cost of expanding its slabs (about that of streaming 512 rows) and keeping at least 1024
 // rows per workgroup.
 static int gradB_slab_splits_kt(int M, int K, int N, int n_cu, int kt) {
     const long per_split = (long)((N + 63) / 64) * ((K + kt - 1) / kt);
-    long max_s = M / 2048;
+    long max_s = M / 1024;
     if (max_s > 64) max_s = 64;
     if (max_s < 1) max_s = 1;
     long best_s = 1, best_cost = -1;

@@ -170,7 +170,7 @@ hipError_t launch_fwd(const uint8_t* A, const uint8_t* B, uint32_t* C, const uin
     int ksplit = 1;
     if (wgs < target_wg) {
         ksplit = (int)((target_wg + wgs - 1) / wgs);
-        const int max_split = K / 64 > 0 ? K / 64 : 1;  // keep at least 64 k per workgroup
+        const int max_split = K / 32 > 0 ? K / 32 : 1;  // keep at least 32 k per workgroup
         if (ksplit > max_split) ksplit = max_split;
         if (ksplit > 64) ksplit = 64;
     }

@@ -615,7 +615,8 @@ hipError_t launch_gradA_slab(const float* gC, const uint8_t* A, const uint8_t* B
                              const LutGeom& g, int M, int K, int N, float scale, int n_cu, uint32_t* flags, void* S,
                              int rows_per_image, hipStream_t stream) {
     const int lut_dwords = g.rows * g.cols / 2;
-    const int qpw = 4;     // 16 k per workgroup (measured: 8 k is 15 % slower for long K, 64 k 20 % slower)
+    // 16 k per workgroup (measured: 8 k is 15 % slower for long K, 64 k 20 % slower); 4 k where that would leave most CUs idle
+    const int qpw = (long)(N / kGaCols) * ((K / 4 + 3) / 4) >= n_cu ? 4 : 1;
     hipLaunchKernelGGL(expand_gradA_kernel, dim3(N / kGaCols, (K / 4 + qpw - 1) / qpw), dim3(256), (size_t)lut_dwords * 4, stream, B,
                        reinterpret_cast<const uint32_t*>(lut), lut_dwords, g.cols, 1 << g.bits, reinterpret_cast<uint32_t*>(S),
                        flags, K, N, qpw);

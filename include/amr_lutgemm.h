@@ -184,6 +184,17 @@ int amr_col2im_f32(const float *cols, float *x, int B, int C, int H, int W, int 
 int amr_set_expanded_table_kernels(int mode);
 
 /*
+ * Process-wide switch, on by default: a backward call that computes both gradients of a small problem (M*K*N < 2e9,
+ * where the latencies of the dependent launches outweigh the arithmetic) queues its gradB launches on a stream of the
+ * library's own beside the gradA launches on the caller's stream; the caller's stream waits for that side stream before
+ * the call returns, so results and stream order are those of the serial form (and the fork / join is captured like any
+ * other cross-stream dependency when the caller's stream is being captured into a graph).  0 switches it off.  Returns
+ * the previous setting.  No counterpart in the reference, which launches both kernels on the default stream
+ * (self_ops/src/approx_gemm_backward.cu:560-608).
+ */
+int amr_set_backward_fork(int on);
+
+/*
  * Dequantisation behind the LUT convolution, from the GEMM's row layout to the NCHW activation in one pass:
  *   out[b,n,pos] = (*s_a * *s_w) * (c[b*L+pos, n] + ((*z_w * x_sum[b*L+pos] + *z_a * w_resp[n*L+pos]) + (*z_a * *z_w) * taps[pos])) + bias[n]
  * with L = positions; c [batch*L, out_channels], x_sum [batch*L], w_resp [out_channels*L], taps [L], out [batch,
