@@ -334,7 +334,8 @@ def quantize_codes_backward(g_tensor, x_tensor, scale_tensor, zp_neg_tensor, qua
 
 
 def lds_gather_probe(pattern=0, waves_per_cu=16, iters=4000):
-    """Measured LDS gather rate (gathers per second) of the current device; see amr_lds_gather_probe."""
+    """Measured LDS gather rate (gathers per second; pattern 2: bytes per second of LDS-direct chunk loads from the L2) of
+    the current device; see amr_lds_gather_probe."""
     ms, n = ctypes.c_float(0), ctypes.c_double(0)
     rc = _lib.amr_lds_gather_probe(pattern, waves_per_cu, iters, ctypes.byref(ms), ctypes.byref(n),
                                    _stream_ptr(torch.device("cuda", torch.cuda.current_device())))

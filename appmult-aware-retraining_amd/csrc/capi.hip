@@ -66,6 +66,7 @@ hipError_t launch_gradA_slab_f32tab(const float* gC, const uint8_t* A, const uin
 hipError_t launch_accgemm(const float* A, const float* B, float* C, int M, int K, int N, hipStream_t stream);
 hipError_t run_lds_probe(int pattern, int waves_per_cu, int iters, int n_cu, float* ms_out, double* gathers_out,
                          hipStream_t stream);
+hipError_t run_lds_direct_probe(int n_chunks, int iters, int n_cu, float* ms_out, double* bytes_out, hipStream_t stream);
 }  // namespace amr
 
 namespace {
@@ -615,9 +616,13 @@ int amr_acc_gemm_forward_fp32(const float* A, const float* B, float* C, int M, i
 }
 
 int amr_lds_gather_probe(int pattern, int waves_per_cu, int iters, float* ms_out, double* gathers_out, void* stream) {
-    if (pattern < 0 || pattern > 1 || iters <= 0) return fail(AMR_EINVAL, "bad probe arguments");
+    if (pattern < 0 || pattern > 3 || iters <= 0) return fail(AMR_EINVAL, "bad probe arguments");
     const int n_cu = current_device_cus(nullptr);
     if (n_cu <= 0) return fail(AMR_EINVAL, "no HIP device available");
+    if (pattern >= 2) {
+        hipError_t e2 = amr::run_lds_direct_probe(pattern == 2 ? 288 : 32, iters, n_cu, ms_out, gathers_out, reinterpret_cast<hipStream_t>(stream));
+        return e2 == hipSuccess ? AMR_OK : hip_fail(e2, "lds-direct probe");
+    }
     hipError_t e = amr::run_lds_probe(pattern, waves_per_cu, iters, n_cu, ms_out, gathers_out, reinterpret_cast<hipStream_t>(stream));
     return e == hipSuccess ? AMR_OK : hip_fail(e, "lds probe");
 }

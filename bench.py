@@ -336,6 +336,7 @@ def main():
 
     probe_free = approx_ops.lds_gather_probe(0, 16, 4000)
     probe_row = approx_ops.lds_gather_probe(1, 16, 4000)
+    probe_delivery = approx_ops.lds_gather_probe(2, 16, 4000)      # bytes/s of LDS-direct 32 KB chunk loads from the L2, all CUs
 
     # single-GEMM configuration (BASELINE configs[1]: M=4096, K=576, N=64 forward+backward) ---------------
     M1, K1, N1 = 4096, 576, 64
@@ -374,7 +375,8 @@ def main():
                      "avg_launch_ms": dom_ms / launches,
                      "hbm": {"achieved": dom_bytes / (dom_ms * 1e-3) / 1e9, "peak": HBM_PEAK / 1e9, "unit": "GB/s",
                              "frac": dom_bytes / (dom_ms * 1e-3) / HBM_PEAK},
-                     "lds_probe_gathers_per_s": {"conflict_free": probe_free, "uniform_row_256B": probe_row}},
+                     "lds_probe_gathers_per_s": {"conflict_free": probe_free, "uniform_row_256B": probe_row},
+                     "lds_direct_chunk_delivery_probe_GBps": probe_delivery / 1e9},
         "single_gemm": {"workload": f"M=4096 K=576 N=64 fwd+bwd, {BITS}-bit (BASELINE.json configs[1] shape)", "us": t_single * 1e3,
                         "lut_mac_per_s": 3 * M1 * K1 * N1 / (t_single * 1e-3),
                         "frac_of_lds_gather_roofline": 3 * M1 * K1 * N1 / (t_single * 1e-3) / LDS_GATHER_PEAK},
@@ -394,6 +396,18 @@ def main():
                      "lds_read": {"achieved_GBps": 2 * mac_rate / 1e9, "frac": 2 * mac_rate / LDS_READ_PEAK},
                      "gather_equivalent_vs_direct_gather_peak": mac_rate / LDS_GATHER_PEAK,
                      "l2_traffic_bytes": traffic, "algorithmic_bytes": hbm_bytes(kind, M2, K2, N2)}
+            # bytes the kernel has delivered from the L2 straight into LDS (expanded-table chunks of 32 KB per 4 k x 32 columns and
+            # block of rows, plus the rows of gC / the codes of A that take the same road) against the rate the probe measures for
+            # such loads alone; gradB streams its operands through registers instead
+            if kind == "forward":
+                direct_bytes = ((M2 + 1023) // 1024) * ((N2 + 31) // 32) * (K2 // 4) * 32768 + M2 * K2 * ((N2 + 31) // 32)
+            elif kind == "gradA":
+                direct_bytes = ((M2 + 511) // 512) * (N2 // 32) * (K2 // 4) * 32768 + ((M2 + 511) // 512) * (K2 // 32) * 512 * N2 * 4
+            else:
+                direct_bytes = 0
+            if direct_bytes:
+                entry["lds_direct_delivery"] = {"achieved_GBps": direct_bytes / (ms * 1e-3) / 1e9, "probe_GBps": probe_delivery / 1e9,
+                                                "frac": direct_bytes / (ms * 1e-3) / probe_delivery}
             if valu_per_lds is not None:
                 valu_per_mac = valu_per_lds / CONV2X_KERNEL[kind][1]
                 entry["valu_issue"] = {"valu_per_mac": round(valu_per_mac, 3), "frac": mac_rate * valu_per_mac / VALU_ISSUE_PEAK}

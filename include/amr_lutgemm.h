@@ -243,6 +243,10 @@ int amr_acc_gemm_forward_fp32(const float *A, const float *B, float *C, int M, i
  * ds_read_u16 per wave with conflict-free (pattern 0) or uniform-random-in-a-256-byte-row
  * (pattern 1) addresses on every CU and writes the kernel time in milliseconds to *ms_out (host
  * pointer; the call synchronises the stream).  gathers = waves_per_cu * n_cu * iters * 8 * 64.
+ * Patterns 2 and 3 measure the delivery of 32 KB chunks from the L2 into LDS by LDS-direct loads instead (one
+ * 1024-thread workgroup per CU, two chunks in flight, `iters` chunks per CU, waves_per_cu ignored; every workgroup
+ * walks the same 9 MB (pattern 2) or 1 MB (pattern 3, resident in every L2) of chunks): *gathers_out then receives
+ * the BYTES delivered over all CUs.
  * No counterpart in the reference.
  */
 int amr_lds_gather_probe(int pattern, int waves_per_cu, int iters, float *ms_out, double *gathers_out, void *stream);
