@@ -46,8 +46,8 @@ constexpr int kSlabBuffers = 4;
 
 // ------------------------------------------------------------------------------------------ expand
 // grid: (n_tiles, ceil(k_quads / kExpandQuadsPerWg)); 256 threads.  Entries of k >= K or n >= N are
-// written as zeros.  Block (0,0) also writes flags[0] = max over the table (used to pick the packed
-// accumulation path).
+// written as zeros.  Block (0,0) also writes the scratch header: flags[0] = max over the table (used to pick the
+// packed accumulation path), flags[1] = 0.
 constexpr int kExpandQuadsPerWg = 4;
 
 __global__ __launch_bounds__(256) void expand_fwd_kernel(const uint8_t* __restrict__ B,
@@ -71,12 +71,16 @@ __global__ __launch_bounds__(256) void expand_fwd_kernel(const uint8_t* __restri
             }
         }
     }
-    __syncthreads();
-    if (blockIdx.x == 0 && blockIdx.y == 0) {
-        // wave-level max, then one atomicMax per wave (flags[0] is zeroed by the host before launch)
+    // Workgroup (0,0) leaves the scratch header for the kernels queued behind this launch: flags[0] = maximum of the table,
+    // flags[1] = 0 (no fall-back requested yet); no separate launch clears them.
+    __shared__ uint32_t wave_max[4];
 #pragma unroll
-        for (int o = 32; o > 0; o >>= 1) mx = max(mx, (uint32_t)__shfl_xor((int)mx, o));
-        if ((threadIdx.x & 63) == 0) atomicMax(&flags[0], mx);
+    for (int o = 32; o > 0; o >>= 1) mx = max(mx, (uint32_t)__shfl_xor((int)mx, o));
+    if ((threadIdx.x & 63) == 0) wave_max[threadIdx.x >> 6] = mx;
+    __syncthreads();
+    if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) {
+        flags[0] = max(max(wave_max[0], wave_max[1]), max(wave_max[2], wave_max[3]));
+        flags[1] = 0u;
     }
     const uint16_t* s16 = reinterpret_cast<const uint16_t*>(smem);
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -525,8 +529,7 @@ hipError_t launch_fwd_slab(const uint8_t* A, const uint8_t* B, uint32_t* C, cons
     const int k_quads = (K + 3) / 4;
     uint32_t* flags = reinterpret_cast<uint32_t*>(workspace);
     uint32_t* E = reinterpret_cast<uint32_t*>(reinterpret_cast<unsigned char*>(workspace) + 256);
-    hipError_t e = launch_zero_u32(flags, 64, stream);
-    if (e != hipSuccess) return e;
+    hipError_t e;
     const int lut_dwords = g.rows * g.cols / 2;
     if (g.bits == 8) {
         static std::atomic<uint64_t> attr_done{0};
