@@ -73,7 +73,7 @@ __global__ __launch_bounds__(256) void expand_fwd_kernel(const uint8_t* __restri
     }
     // Workgroup (0,0) leaves the scratch header for the kernels queued behind this launch: flags[0] = maximum of the table,
     // flags[1] = 0 (no fall-back requested yet); no separate launch clears them.
-    __shared__ uint32_t wave_max[4];
+    uint32_t* wave_max = s32 + lut_dwords;         // four words behind the table (the launch asks for them)
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) mx = max(mx, (uint32_t)__shfl_xor((int)mx, o));
     if ((threadIdx.x & 63) == 0) wave_max[threadIdx.x >> 6] = mx;
@@ -535,7 +535,7 @@ hipError_t launch_fwd_slab(const uint8_t* A, const uint8_t* B, uint32_t* C, cons
         static std::atomic<uint64_t> attr_done{0};
         if ((e = allow_full_lds(reinterpret_cast<const void*>(expand_fwd_kernel), attr_done)) != hipSuccess) return e;
         hipLaunchKernelGGL(expand_fwd_kernel, dim3(n_tiles, (k_quads + kExpandQuadsPerWg - 1) / kExpandQuadsPerWg), dim3(256),
-                           (size_t)lut_dwords * 4, stream, B, reinterpret_cast<const uint32_t*>(lut), lut_dwords, g.cols,
+                           (size_t)lut_dwords * 4 + 16, stream, B, reinterpret_cast<const uint32_t*>(lut), lut_dwords, g.cols,
                            1 << g.bits, E, flags, K, N, k_quads, kSlab8Rows);
         if ((e = hipGetLastError()) != hipSuccess) return e;
         const int row_blocks8 = (M + 1023) / 1024;
@@ -559,7 +559,7 @@ hipError_t launch_fwd_slab(const uint8_t* A, const uint8_t* B, uint32_t* C, cons
         return hipSuccess;
     }
     hipLaunchKernelGGL(expand_fwd_kernel, dim3(n_tiles, (k_quads + kExpandQuadsPerWg - 1) / kExpandQuadsPerWg), dim3(256),
-                       (size_t)lut_dwords * 4, stream, B, reinterpret_cast<const uint32_t*>(lut), lut_dwords, g.cols,
+                       (size_t)lut_dwords * 4 + 16, stream, B, reinterpret_cast<const uint32_t*>(lut), lut_dwords, g.cols,
                        1 << g.bits, E, flags, K, N, k_quads, kSlabRows);
     e = hipGetLastError();
     if (e != hipSuccess) return e;
