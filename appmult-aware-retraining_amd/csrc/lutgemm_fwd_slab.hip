@@ -204,10 +204,10 @@ __device__ __forceinline__ void slab_chunk_fast(uint32_t (&acc)[RG][4], const ui
             }
             if (PACKED) {
                 typedef unsigned short us2 __attribute__((ext_vector_type(2)));
-                const us2 l = (__builtin_bit_cast(us2, lo[0]) + __builtin_bit_cast(us2, lo[1])) +
-                              (__builtin_bit_cast(us2, lo[2]) + __builtin_bit_cast(us2, lo[3]));
-                const us2 h = (__builtin_bit_cast(us2, hi[0]) + __builtin_bit_cast(us2, hi[1])) +
-                              (__builtin_bit_cast(us2, hi[2]) + __builtin_bit_cast(us2, hi[3]));
+                // (no 16-bit half of these sums overflows, so one 32-bit addition adds both halves and a three-operand
+                // addition saves an instruction per pair of columns over packed 16-bit additions)
+                const us2 l = __builtin_bit_cast(us2, (lo[0] + lo[1] + lo[2]) + lo[3]);
+                const us2 h = __builtin_bit_cast(us2, (hi[0] + hi[1] + hi[2]) + hi[3]);
                 acc[i + g][0] += l.x;
                 acc[i + g][1] += l.y;
                 acc[i + g][2] += h.x;
