@@ -8,8 +8,8 @@
 //   step 2  lutgemm_fwd_slab_kernel:  C[m, :] = sum_k E[k][A[m,k]][:]             (M * K row additions)
 //
 // Step 1 costs 2^b / M of the M*K*N gathers of the direct kernel.  Step 2 never gathers single
-// entries: for one (m,k) a lane reads FOUR adjacent uint16 entries of row a = A[m,k] with one
-// ds_read_b64.  64-bit LDS reads move 256 B/clk/CU on gfx950, twice the 32 lanes/clk of 16/32-bit
+// entries: for one (m,k) a lane reads EIGHT adjacent uint16 entries of row a = A[m,k] with one
+// ds_read_b128.  Wide LDS reads move 256 B/clk/CU on gfx950, twice the 32 lanes/clk of 16/32-bit
 // gathers, and they are conflict-free by construction here, so the LDS no longer limits the kernel.
 //
 // Layout of E in HBM (uint16): E[n_tile][k_quad][a (128 rows)][kk (4 values of k)][32 columns]; one
@@ -18,16 +18,18 @@
 // Four chunk buffers live in LDS; chunk c+2 is requested (LDS-direct loads) when chunk c starts to be
 // consumed, so a request has two chunk periods to arrive: with one period the L2 latency, not the
 // arithmetic, set the pace.  Every chunk a workgroup fetches serves 1024 x 4 x 32 additions.
-// Lane l of a wave: row slot rs = l/8 (8 rows per instruction), column group cg = l%8 (4 columns).
-// Row slot rs visits the four k of a chunk starting at k = rs%4, so in every instruction the four
-// slots of a half-wave read four different 64 B quarters of their 256 B lines: each quarter lives in its
-// own 16 banks, which makes every read conflict-free.
-// The LDS address (buffer pair<<16 | a<<8 | kk<<6 | cg<<3) is assembled from the code byte and a
-// per-lane constant by ONE v_perm_b32.  That needs a < 128: a 7-bit operand holding the masked code
-// 128 (zero contribution) is detected, flags[1] is raised and the direct kernel, queued behind this
-// one and gated on that flag, recomputes C.
+// Lane l of a wave: row slot rs = l/4 (16 rows per instruction), column group cg = l%4 (8 columns).
+// Row slot rs visits the four k of a chunk starting at k = rs%4, so the four slots that the LDS serves
+// together (16 lanes of a 128-bit read) read four different 64 B quarters of their 256 B lines: each
+// quarter lives in its own 16 banks, which makes every read conflict-free.
+// The LDS address (buffer pair<<16 | a<<8 | kk<<6 | cg<<4) is assembled from the code byte and a
+// per-lane constant by ONE v_perm_b32 per eight entries.  That needs a < 128: a 7-bit operand holding
+// the masked code 128 (zero contribution) is detected, flags[1] is raised and the direct kernel, queued
+// behind this one and gated on that flag, recomputes C.
 // Accumulation: when 4 * max(lut) < 65536 (flag written by the expand kernel) the four k of a chunk
-// are first added as packed uint16 pairs (v_pk_add_u16) and widened to 32 bit once per chunk.
+// are first added as packed uint16 pairs (plain 32-bit additions: no half overflows) and widened to 32
+// bit once per chunk: 2.5 vector instructions per four entries (one address, two additions, two widening
+// additions per pair of columns and four k), which is what bounds the kernel.
 #include <type_traits>
 
 #include "amr_common.h"
@@ -129,104 +131,86 @@ __device__ __forceinline__ void slab_copy_chunk(const u32x4* src, unsigned char*
     }
 }
 
-// Eight 64-bit LDS reads (two row groups x four k) issued back to back, NOT waited for.  Inline
+// Four 128-bit LDS reads (one row group x four k) issued back to back, NOT waited for.  Inline
 // assembly, for two reasons: the reads of the chunk being consumed must not wait for the LDS-direct
 // loads of later chunks (the compiler cannot tell the two apart, same LDS array), and the reads of
 // block b+1 are issued before block b is consumed (software pipelining with explicit counters).
 // OFF is the part of the buffer offset that does not fit the v_perm-built address (odd buffers).
 template <int OFF>
-__device__ __forceinline__ void slab_issue8(uint64_t (&d)[8], const uint32_t (&addr)[8]) {
+__device__ __forceinline__ void slab_issue4(u32x4 (&d)[4], const uint32_t (&addr)[4]) {
     asm volatile(
-        "ds_read_b64 %0, %8 offset:%16\n ds_read_b64 %1, %9 offset:%16\n ds_read_b64 %2, %10 offset:%16\n"
-        "ds_read_b64 %3, %11 offset:%16\n ds_read_b64 %4, %12 offset:%16\n ds_read_b64 %5, %13 offset:%16\n"
-        "ds_read_b64 %6, %14 offset:%16\n ds_read_b64 %7, %15 offset:%16"
-        : "=&v"(d[0]), "=&v"(d[1]), "=&v"(d[2]), "=&v"(d[3]), "=&v"(d[4]), "=&v"(d[5]), "=&v"(d[6]), "=&v"(d[7])
-        : "v"(addr[0]), "v"(addr[1]), "v"(addr[2]), "v"(addr[3]), "v"(addr[4]), "v"(addr[5]), "v"(addr[6]), "v"(addr[7]),
-          "n"(OFF)
+        "ds_read_b128 %0, %4 offset:%8\n ds_read_b128 %1, %5 offset:%8\n ds_read_b128 %2, %6 offset:%8\n"
+        "ds_read_b128 %3, %7 offset:%8"
+        : "=&v"(d[0]), "=&v"(d[1]), "=&v"(d[2]), "=&v"(d[3])
+        : "v"(addr[0]), "v"(addr[1]), "v"(addr[2]), "v"(addr[3]), "n"(OFF)
         : "memory");
 }
 
-// Waits until at most PENDING LDS operations are outstanding.  The eight results are passed through
+// Waits until at most PENDING LDS operations are outstanding.  The four results are passed through
 // as in/out operands so that every use of them is ordered after the wait.
 template <int PENDING>
-__device__ __forceinline__ void slab_wait8(uint64_t (&d)[8]) {
-    asm volatile("s_waitcnt lgkmcnt(%8)"
-                 : "+v"(d[0]), "+v"(d[1]), "+v"(d[2]), "+v"(d[3]), "+v"(d[4]), "+v"(d[5]), "+v"(d[6]), "+v"(d[7])
-                 : "n"(PENDING)
-                 : "memory");
+__device__ __forceinline__ void slab_wait4(u32x4 (&d)[4]) {
+    asm volatile("s_waitcnt lgkmcnt(%4)" : "+v"(d[0]), "+v"(d[1]), "+v"(d[2]), "+v"(d[3]) : "n"(PENDING) : "memory");
 }
 
-template <int RG>
-__device__ __forceinline__ void slab_addr8(uint32_t (&addr)[8], const uint32_t (&a_cur)[RG], int i,
-                                           const uint32_t (&base)[4], const uint32_t (&sel)[4]) {
+__device__ __forceinline__ void slab_addr4(uint32_t (&addr)[4], uint32_t codes4, const uint32_t (&base)[4],
+                                           const uint32_t (&sel)[4]) {
 #pragma unroll
-    for (int g = 0; g < 2; ++g)
-#pragma unroll
-        for (int j = 0; j < 4; ++j) addr[4 * g + j] = __builtin_amdgcn_perm(a_cur[i + g], base[j], sel[j]);
+    for (int j = 0; j < 4; ++j) addr[j] = __builtin_amdgcn_perm(codes4, base[j], sel[j]);
 }
 
-// One chunk (4 k) for all RG row groups of a lane; every code is < 128.
+// One pair of columns (one dword of each of the four reads of a row group) into its two sums.
+template <bool PACKED>
+__device__ __forceinline__ void slab_add_pair(uint32_t& even, uint32_t& odd, uint32_t x0, uint32_t x1, uint32_t x2, uint32_t x3) {
+    if (PACKED) {
+        // (no 16-bit half of these sums overflows, so one 32-bit addition adds both halves and a three-operand
+        // addition saves an instruction per pair of columns over packed 16-bit additions)
+        typedef unsigned short us2 __attribute__((ext_vector_type(2)));
+        const us2 s = __builtin_bit_cast(us2, (x0 + x1 + x2) + x3);
+        even += s.x;
+        odd += s.y;
+    } else {
+        even += (x0 & 0xffffu) + (x1 & 0xffffu) + (x2 & 0xffffu) + (x3 & 0xffffu);
+        odd += (x0 >> 16) + (x1 >> 16) + (x2 >> 16) + (x3 >> 16);
+    }
+}
+
+// One chunk (4 k) for all RG row groups of a lane; every code is < 128 (8-bit kernel: < 256).
 template <int RG, bool PACKED, int OFF>
-__device__ __forceinline__ void slab_chunk_fast(uint32_t (&acc)[RG][4], const uint32_t (&a_cur)[RG],
+__device__ __forceinline__ void slab_chunk_fast(uint32_t (&acc)[RG][8], const uint32_t (&a_cur)[RG],
                                                 const uint32_t (&base)[4], const uint32_t (&sel)[4]) {
-    static_assert(RG % 2 == 0, "row groups are processed in pairs");
-    constexpr int NB = RG / 2;
-    uint64_t d[2][8];
+    u32x4 d[2][4];
     {
-        uint32_t addr[8];
-        slab_addr8<RG>(addr, a_cur, 0, base, sel);
-        slab_issue8<OFF>(d[0], addr);
+        uint32_t addr[4];
+        slab_addr4(addr, a_cur[0], base, sel);
+        slab_issue4<OFF>(d[0], addr);
     }
 #pragma unroll
-    for (int b = 0; b < NB; ++b) {
-        const int i = 2 * b;
+    for (int b = 0; b < RG; ++b) {
         // waves that are behind go first: the four waves of a SIMD then move through a chunk in step instead of one
         // after the other (oldest first), and the last one does not run alone, latencies exposed, before the barrier
         if (b == 0) __builtin_amdgcn_s_setprio(3);
         else if (b == 1) __builtin_amdgcn_s_setprio(2);
         else if (b == 2) __builtin_amdgcn_s_setprio(1);
         else __builtin_amdgcn_s_setprio(0);
-        if (b + 1 < NB) {
-            uint32_t addr[8];
-            slab_addr8<RG>(addr, a_cur, i + 2, base, sel);
-            slab_issue8<OFF>(d[(b + 1) & 1], addr);
-            slab_wait8<8>(d[b & 1]);
+        if (b + 1 < RG) {
+            uint32_t addr[4];
+            slab_addr4(addr, a_cur[b + 1], base, sel);
+            slab_issue4<OFF>(d[(b + 1) & 1], addr);
+            slab_wait4<4>(d[b & 1]);
         } else {
-            slab_wait8<0>(d[b & 1]);
+            slab_wait4<0>(d[b & 1]);
         }
-#pragma unroll
-        for (int g = 0; g < 2; ++g) {
-            uint32_t lo[4], hi[4];
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                lo[j] = (uint32_t)d[b & 1][4 * g + j];
-                hi[j] = (uint32_t)(d[b & 1][4 * g + j] >> 32);
-            }
-            if (PACKED) {
-                typedef unsigned short us2 __attribute__((ext_vector_type(2)));
-                // (no 16-bit half of these sums overflows, so one 32-bit addition adds both halves and a three-operand
-                // addition saves an instruction per pair of columns over packed 16-bit additions)
-                const us2 l = __builtin_bit_cast(us2, (lo[0] + lo[1] + lo[2]) + lo[3]);
-                const us2 h = __builtin_bit_cast(us2, (hi[0] + hi[1] + hi[2]) + hi[3]);
-                acc[i + g][0] += l.x;
-                acc[i + g][1] += l.y;
-                acc[i + g][2] += h.x;
-                acc[i + g][3] += h.y;
-            } else {
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    acc[i + g][0] += lo[j] & 0xffffu;
-                    acc[i + g][1] += lo[j] >> 16;
-                    acc[i + g][2] += hi[j] & 0xffffu;
-                    acc[i + g][3] += hi[j] >> 16;
-                }
-            }
-        }
+        const u32x4 x0 = d[b & 1][0], x1 = d[b & 1][1], x2 = d[b & 1][2], x3 = d[b & 1][3];
+        slab_add_pair<PACKED>(acc[b][0], acc[b][1], x0.x, x1.x, x2.x, x3.x);
+        slab_add_pair<PACKED>(acc[b][2], acc[b][3], x0.y, x1.y, x2.y, x3.y);
+        slab_add_pair<PACKED>(acc[b][4], acc[b][5], x0.z, x1.z, x2.z, x3.z);
+        slab_add_pair<PACKED>(acc[b][6], acc[b][7], x0.w, x1.w, x2.w, x3.w);
         // Pin the accumulation here: an empty volatile asm that "modifies" the eight accumulators cannot
         // be moved across the volatile read blocks, so the sums are not postponed until all reads of
         // the chunk are done (which would keep every result live and overflow the register file).
-        asm volatile("" : "+v"(acc[i][0]), "+v"(acc[i][1]), "+v"(acc[i][2]), "+v"(acc[i][3]), "+v"(acc[i + 1][0]),
-                          "+v"(acc[i + 1][1]), "+v"(acc[i + 1][2]), "+v"(acc[i + 1][3]));
+        asm volatile("" : "+v"(acc[b][0]), "+v"(acc[b][1]), "+v"(acc[b][2]), "+v"(acc[b][3]), "+v"(acc[b][4]),
+                          "+v"(acc[b][5]), "+v"(acc[b][6]), "+v"(acc[b][7]));
     }
 }
 
@@ -240,15 +224,50 @@ __device__ __forceinline__ void slab_chunk_fast(uint32_t (&acc)[RG][4], const ui
 // issued from inline assembly together with the one wait that is needed.
 constexpr int kSlabCodeBytes = 16 * 64 * 16;   // staging of one group of four chunks: 16 waves x 64 rows x 16 codes
 
-// Eight dwords at a stride of 128 B (the codes of this lane's eight rows for one chunk).
-__device__ __forceinline__ void slab_read_codes(uint32_t (&a)[8], uint32_t addr) {
+// Four dwords at a stride of 256 B (the codes of this lane's four rows for one chunk).
+__device__ __forceinline__ void slab_read_codes(uint32_t (&a)[4], uint32_t addr) {
     asm volatile(
-        "ds_read_b32 %0, %8\n ds_read_b32 %1, %8 offset:128\n ds_read_b32 %2, %8 offset:256\n ds_read_b32 %3, %8 offset:384\n"
-        "ds_read_b32 %4, %8 offset:512\n ds_read_b32 %5, %8 offset:640\n ds_read_b32 %6, %8 offset:768\n"
-        "ds_read_b32 %7, %8 offset:896\n s_waitcnt lgkmcnt(0)"
-        : "=&v"(a[0]), "=&v"(a[1]), "=&v"(a[2]), "=&v"(a[3]), "=&v"(a[4]), "=&v"(a[5]), "=&v"(a[6]), "=&v"(a[7])
+        "ds_read_b32 %0, %4\n ds_read_b32 %1, %4 offset:256\n ds_read_b32 %2, %4 offset:512\n ds_read_b32 %3, %4 offset:768\n"
+        "s_waitcnt lgkmcnt(0)"
+        : "=&v"(a[0]), "=&v"(a[1]), "=&v"(a[2]), "=&v"(a[3])
         : "v"(addr)
         : "memory");
+}
+
+// The sums of a wave (64 rows x 32 columns) leave through LDS, 8 KB per wave in the chunk buffers nobody reads any more,
+// so that every store or atomic instruction of a wave covers two whole 128 B lines of C (straight from the accumulators an
+// instruction would touch 16 rows and four dwords in each; a split K adds its sums with atomics, which pay per line).
+// The caller has waited for its loads towards LDS and passed a workgroup barrier.
+template <int RG>
+__device__ __forceinline__ void slab_store_tile(const uint32_t (&acc)[RG][8], unsigned char* wave_lds, int lane, int rs, int cg,
+                                                uint32_t* __restrict__ C, int m_wave, int m_first, int n0, int N, int atomic_out,
+                                                int out_f32) {
+#pragma unroll
+    for (int i = 0; i < RG; ++i) {
+        u32x4* dst = reinterpret_cast<u32x4*>(wave_lds + (16 * i + rs) * 128 + cg * 32);
+        u32x4 lo, hi;
+        lo.x = acc[i][0]; lo.y = acc[i][1]; lo.z = acc[i][2]; lo.w = acc[i][3];
+        hi.x = acc[i][4]; hi.y = acc[i][5]; hi.z = acc[i][6]; hi.w = acc[i][7];
+        dst[0] = lo;
+        dst[1] = hi;
+    }
+    const uint32_t* w32 = reinterpret_cast<const uint32_t*>(wave_lds);
+    const int col = lane & 31, half = lane >> 5;
+    const int n = n0 + col;
+#pragma unroll 8
+    for (int p = 0; p < 8 * RG; ++p) {
+        const int row = 2 * p + half;
+        const int m = m_wave + row;
+        const uint32_t v = w32[row * 32 + col];
+        if (m >= m_first && n < N) {
+            if (atomic_out)
+                atomicAdd(&C[(size_t)m * N + n], v);
+            else if (out_f32)
+                C[(size_t)m * N + n] = __float_as_uint((float)v);
+            else
+                C[(size_t)m * N + n] = v;
+        }
+    }
 }
 
 template <int RG, int WAVES, bool PACKED>
@@ -259,13 +278,13 @@ __global__ __launch_bounds__(WAVES * 64) void lutgemm_fwd_slab_kernel(
     // static: lets the compiler fold the base address (chunk buffers first: their addresses come out of v_perm)
     __shared__ __align__(16) unsigned char smem[kSlabBuffers * kSlabChunkBytes + 2 * kSlabCodeBytes];
     constexpr int THREADS = WAVES * 64;
-    constexpr int ROWS_PER_WAVE = 8 * RG;
-    static_assert(RG == 8 && WAVES == 16, "staging layout and vmcnt bookkeeping are written for 16 waves of 64 rows");
+    constexpr int ROWS_PER_WAVE = 16 * RG;
+    static_assert(RG == 4 && WAVES == 16, "staging layout and vmcnt bookkeeping are written for 16 waves of 64 rows");
     static_assert(kSlabChunkBytes / 16 / THREADS == 2, "two chunk-copy operations per thread and chunk");
     const int tid = threadIdx.x;
     const int wave = uniform(tid >> 6);
     const int lane = tid & 63;
-    const int rs = lane >> 3, cg = lane & 7, rot = rs & 3;
+    const int rs = lane >> 2, cg = lane & 3, rot = rs & 3;
     // Workgroup -> (column tile, row block, K split).  Plain: the grid's three dimensions.  Grouped (n_tiles_grouped > 0,
     // 1-D grid, no K split): the hardware deals workgroups to the 8 XCDs round-robin by index; the column tiles of one
     // row block get consecutive slots of ONE XCD, so that they run at the same time behind the same L2 and fetch their
@@ -297,22 +316,22 @@ __global__ __launch_bounds__(WAVES * 64) void lutgemm_fwd_slab_kernel(
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
         const uint32_t kk = (uint32_t)((j + rot) & 3);
-        base_lo[j] = (kk << 6) | (uint32_t)(cg << 3);
+        base_lo[j] = (kk << 6) | (uint32_t)(cg << 4);
         base_hi[j] = base_lo[j] | 0x10000u;
         sel[j] = 0x0c020000u | ((4u + kk) << 8);
     }
 
-    uint32_t acc[RG][4];
+    uint32_t acc[RG][8];
 #pragma unroll
     for (int i = 0; i < RG; ++i)
 #pragma unroll
-        for (int c = 0; c < 4; ++c) acc[i][c] = 0u;
+        for (int c = 0; c < 8; ++c) acc[i][c] = 0u;
 
-    // Lane (rs, cg) consumes rows m_wave + 8 rs + i, i < 8.  Lane l fetches the codes of row
-    // m_wave + 8 (l % 8) + l / 8, which land at staging position l: row 8 rs + i sits at position 8 i + rs,
-    // so the eight dword reads of a chunk are a 128 B stride apart and the eight row slots of one read hit
-    // eight different banks.  32-bit offsets: the host only takes this path when M*K < 2^31.
-    const uint32_t code_off = (uint32_t)(m_wave + 8 * (lane & 7) + (lane >> 3)) * (uint32_t)K;
+    // Lane (rs, cg) consumes rows m_wave + 16 i + rs, i < 4.  Lane l fetches the codes of row m_wave + l,
+    // which land at staging position l (16 B each): the four dword reads of a chunk are 256 B apart and the
+    // eight row slots that one pass of a read serves are 16 B apart, in eight different banks.
+    // 32-bit offsets: the host only takes this path when M*K < 2^31.
+    const uint32_t code_off = (uint32_t)(m_wave + lane) * (uint32_t)K;
     unsigned char* code_stage = smem + kSlabBuffers * kSlabChunkBytes + wave * 1024;      // + (group & 1) * kSlabCodeBytes
     const uint32_t code_read = (uint32_t)(kSlabBuffers * kSlabChunkBytes + wave * 1024 + rs * 16);
 
@@ -364,31 +383,15 @@ __global__ __launch_bounds__(WAVES * 64) void lutgemm_fwd_slab_kernel(
         if (c + 2 < c_end) step(c + 2, g, std::integral_constant<int, 2>{});
         if (c + 3 < c_end) step(c + 3, g, std::integral_constant<int, 3>{});
     }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // nothing is left in flight towards LDS when the workgroup ends
+    // nothing is left in flight towards LDS and every wave has read its last chunk: the buffers take the sums
+    asm volatile("s_waitcnt vmcnt(0)\n s_barrier" ::: "memory");
 
     // A code with bit 7 set (the masked code 128 of a 7-bit table) cannot be addressed by this kernel:
     // raise flags[1]; the host has queued the direct kernel behind this one, gated on that flag.
     if (__builtin_amdgcn_ballot_w64((seen & 0x80808080u) != 0) != 0) {
         if (lane == 0) atomicOr(&flags[1], 1u);
     }
-    const int n = tile_x * kSlabCols + 4 * cg;
-#pragma unroll
-    for (int i = 0; i < RG; ++i) {
-        const int m = m_wave + 8 * rs + i;
-        if (m >= m_first) {
-#pragma unroll
-            for (int c = 0; c < 4; ++c) {
-                if (n + c < N) {
-                    if (atomic_out)
-                        atomicAdd(&C[(size_t)m * N + n + c], acc[i][c]);
-                    else if (out_f32)
-                        C[(size_t)m * N + n + c] = __float_as_uint((float)acc[i][c]);
-                    else
-                        C[(size_t)m * N + n + c] = acc[i][c];
-                }
-            }
-        }
-    }
+    slab_store_tile<RG>(acc, smem + wave * 8192, lane, rs, cg, C, m_wave, m_first, tile_x * kSlabCols, N, atomic_out, out_f32);
 }
 
 // ------------------------------------------------------------------------------------------ 8-bit tables
@@ -405,12 +408,12 @@ __global__ __launch_bounds__(1024) void lutgemm_fwd_slab8_kernel(
     const uint8_t* __restrict__ A, const u32x4* __restrict__ E, uint32_t* __restrict__ C,
     const uint32_t* __restrict__ flags, int M, int K, int N, int k_quads, int chunks_per_split, int atomic_out, int out_f32) {
     __shared__ __align__(16) unsigned char smem[2 * kSlab8ChunkBytes + 2 * kSlabCodeBytes];
-    constexpr int RG = 8, WAVES = 16, THREADS = WAVES * 64, ROWS_PER_WAVE = 8 * RG;
+    constexpr int RG = 4, WAVES = 16, THREADS = WAVES * 64, ROWS_PER_WAVE = 16 * RG;
     static_assert(2 * kSlab8ChunkBytes + 2 * kSlabCodeBytes == 160 * 1024, "the workgroup uses the whole LDS of a CU");
     const int tid = threadIdx.x;
     const int wave = uniform(tid >> 6);
     const int lane = tid & 63;
-    const int rs = lane >> 3, cg = lane & 7, rot = rs & 3;
+    const int rs = lane >> 2, cg = lane & 3, rot = rs & 3;
     const int tile_x = blockIdx.x, rb_y = blockIdx.y, split_z = blockIdx.z;
     // (a wave whose rows would stick out of M is shifted up; the rows it shares with the wave above are stored once)
     const int m_first = (rb_y * WAVES + wave) * ROWS_PER_WAVE;
@@ -426,19 +429,18 @@ __global__ __launch_bounds__(1024) void lutgemm_fwd_slab8_kernel(
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
         const uint32_t kk = (uint32_t)((j + rot) & 3);
-        base0[j] = (kk << 6) | (uint32_t)(cg << 3);
+        base0[j] = (kk << 6) | (uint32_t)(cg << 4);
         base1[j] = base0[j] | 0x10000u;
         sel[j] = 0x0c020000u | ((4u + kk) << 8);
     }
-    uint32_t acc[RG][4];
+    uint32_t acc[RG][8];
 #pragma unroll
     for (int i = 0; i < RG; ++i)
 #pragma unroll
-        for (int c = 0; c < 4; ++c) acc[i][c] = 0u;
+        for (int c = 0; c < 8; ++c) acc[i][c] = 0u;
 
-    // codes: as in the 7-bit kernel (16 bytes = four chunks per row and request, staged so that a lane's eight rows are
-    // 128 B apart)
-    const uint32_t code_off = (uint32_t)(m_wave + 8 * (lane & 7) + (lane >> 3)) * (uint32_t)K;
+    // codes: as in the 7-bit kernel (16 bytes = four chunks per row and request; row r of the wave at staging position r)
+    const uint32_t code_off = (uint32_t)(m_wave + lane) * (uint32_t)K;
     unsigned char* code_stage = smem + 2 * kSlab8ChunkBytes + wave * 1024;
     const uint32_t code_read = (uint32_t)(2 * kSlab8ChunkBytes + wave * 1024 + rs * 16);
     typedef const __attribute__((address_space(1))) void* gptr_t;
@@ -477,26 +479,9 @@ __global__ __launch_bounds__(1024) void lutgemm_fwd_slab8_kernel(
         if (c + 2 < c_end) step(c + 2, g, std::integral_constant<int, 0>{}, false);
         if (c + 3 < c_end) step(c + 3, g, std::integral_constant<int, 1>{}, false);
     }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // nothing is left in flight towards LDS when the workgroup ends
-
-    const int n = tile_x * kSlabCols + 4 * cg;
-#pragma unroll
-    for (int i = 0; i < RG; ++i) {
-        const int m = m_wave + 8 * rs + i;
-        if (m >= m_first) {
-#pragma unroll
-            for (int c = 0; c < 4; ++c) {
-                if (n + c < N) {
-                    if (atomic_out)
-                        atomicAdd(&C[(size_t)m * N + n + c], acc[i][c]);
-                    else if (out_f32)
-                        C[(size_t)m * N + n + c] = __float_as_uint((float)acc[i][c]);
-                    else
-                        C[(size_t)m * N + n + c] = acc[i][c];
-                }
-            }
-        }
-    }
+    // nothing is left in flight towards LDS and every wave has read its last chunk: the buffers take the sums
+    asm volatile("s_waitcnt vmcnt(0)\n s_barrier" ::: "memory");
+    slab_store_tile<RG>(acc, smem + wave * 8192, lane, rs, cg, C, m_wave, m_first, tile_x * kSlabCols, N, atomic_out, out_f32);
 }
 
 hipError_t launch_fwd_gated(const uint8_t* A, const uint8_t* B, uint32_t* C, const uint16_t* lut, const LutGeom& g,
@@ -565,8 +550,8 @@ hipError_t launch_fwd_slab(const uint8_t* A, const uint8_t* B, uint32_t* C, cons
     if (e != hipSuccess) return e;
 
     // 16 waves x 64 rows = 1024 rows per workgroup
-    constexpr int RG = 8, WAVES = 16;
-    const int m_tile = WAVES * 8 * RG;
+    constexpr int RG = 4, WAVES = 16;
+    const int m_tile = WAVES * 16 * RG;
     const long wgs = (long)n_tiles * ((M + m_tile - 1) / m_tile);
     int ksplit = 1;
     if (wgs < n_cu) {
