@@ -490,19 +490,18 @@ hipError_t launch_fwd_gated(const uint8_t* A, const uint8_t* B, uint32_t* C, con
 // ------------------------------------------------------------------------------------------ host
 // Workspace layout: [256 B flags][E].  Returns 0 when the expanded-table path does not apply.
 size_t fwd_slab_workspace_bytes(const LutGeom& g, int M, int K, int N, bool force) {
-    // Worth it when the 2^b/M expansion overhead is small and K is long enough to amortise the extra
-    // launches (measured cross-over on MI355X: K around 512).
+    // Worth it when the 2^b/M expansion overhead is small and there is enough work to amortise the extra launches.
     // (K % 4 == 0: the codes of A are fetched four and sixteen at a time)
-    if (M < 2048 || K < 512 || (K & 3) != 0 || (size_t)M * K >= (1ull << 31)) return 0;
+    if (M < 2048 || K < (force ? 32 : 64) || (K & 3) != 0 || (size_t)M * K >= (1ull << 31)) return 0;
     if (g.bits == 8) {
         // 8-bit tables: 64 KB per (column tile, four k); every block of 1024 rows streams all of it, so the rows have to
         // outnumber the 256 codes well (measured against the direct kernel on MI355X)
         if (!force && (M < 4096 || (size_t)M * K * N < (3ull << 29))) return 0;
         return 256 + (size_t)((N + kSlabCols - 1) / kSlabCols) * (((size_t)K + 3) / 4) * kSlab8ChunkBytes;
     }
-    // below about 1.6e9 multiply-adds the extra launches (flags, expansion, second flavour, gated fall-back) cost
-    // more than the faster kernel gains (measured cross-over on MI355X between 1.2e9 and 2.4e9)
-    if (!force && (size_t)M * K * N < (3ull << 29)) return 0;
+    // below about 4e8 multiply-adds the extra launches (expansion, second flavour, gated fall-back) cost more than the
+    // faster kernel gains (measured on MI355X: even at 3e8, 57 against 85 us at 5.4e8)
+    if (!force && (size_t)M * K * N < (3ull << 27)) return 0;
     const size_t n_tiles = (N + kSlabCols - 1) / kSlabCols;
     const size_t k_quads = ((size_t)K + 3) / 4;
     return 256 + n_tiles * k_quads * kSlabChunkBytes;
