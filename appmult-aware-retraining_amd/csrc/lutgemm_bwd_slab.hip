@@ -222,9 +222,14 @@ __global__ __launch_bounds__(1024) void lutgemm_gradB_slab_kernel(
 // undone at the end with the column sums of gC:  sum_m g*(G-offset) + offset * sum_m g (nothing to undo and no
 // column sums for offset 0).
 //
-// LDS layout: byte address = (kk>>1)*32768 + a*256 + (kk&1)*128 + 2*c: the two k of a pair share a 256 B
-// row.  Row slots 1 and 3 of a wave visit the two k of every pair in the other order than slots 0 and 2,
-// so that the 32 lanes of a half-wave always read one 128 B half-row in banks 0-31 and one in banks 32-63.
+// LDS layout: byte address = (kk>>1)*32768 + a*256 + (kk&1)*128 + 2*pos(c): the two k of a pair share a 256 B
+// row; column c of the tile sits at position pos(c) = 8*((c%32)/4) + 4*(c/32) + c%4 of its 128 B half-row, so that the
+// 16 bytes a lane reads (column group cg) hold columns 4cg..4cg+3 and 32+4cg..32+4cg+3 and its two 16-byte loads of
+// a row of gC belong to two instructions that each cover 128 contiguous bytes per row.
+// Lane = (row slot rs of 4, k half kh, column group cg of 8): per row of A it reads the four k of its half with
+// 128-bit reads (one v_perm_b32 per eight multiply-adds).  The LDS serves 16 lanes of such a read together, i.e. the
+// two k halves of one row slot: half 1 visits the two k of every pair in the other order than half 0, so that one
+// reads a 128 B half-row in banks 0-31 and the other one in banks 32-63.
 // Requires K % 8 == 0, N % 64 == 0, row counts that are multiples of the rows per iteration, gC 16-byte
 // aligned and 32-bit offsets (the launcher checks).
 constexpr int kBwdKT16 = 8;
@@ -239,8 +244,8 @@ __global__ __launch_bounds__(1024) void lutgemm_gradB_slab16_kernel(
     const int tid = threadIdx.x;
     const int wave = uniform(tid >> 6);
     const int lane = tid & 63;
-    const int rs = lane >> 4, cg = lane & 15;
-    const uint32_t swap = (uint32_t)(rs & 1);
+    const int rs = lane >> 4, kh = (lane >> 3) & 1, cg = lane & 7;
+    const uint32_t swap = (uint32_t)kh;
     // Workgroups are dealt to the 8 XCDs round-robin by their index; the workgroups of one XCD (same index mod 8) take
     // consecutive k tiles of one (column tile, M split), so that the rows of gC and A they all stream are shared in
     // that XCD's L2 instead of being fetched once per XCD.
@@ -282,7 +287,7 @@ __global__ __launch_bounds__(1024) void lutgemm_gradB_slab16_kernel(
         const _Float16 zero = (_Float16)(-offset);
 #pragma unroll
         for (int kk = 0; kk < KT; ++kk) {
-            unsigned char* s = smem + (kk >> 1) * 32768 + (kk & 1) * 128 + 2 * col;
+            unsigned char* s = smem + (kk >> 1) * 32768 + (kk & 1) * 128 + 2 * (8 * ((col & 31) >> 2) + 4 * (col >> 5) + (col & 3));
             const bool masked = bcode[kk] > 127;           // the masked code of a 7-bit operand: the table's zero column
             const _Float16* t = tab + min(bcode[kk], 127);
 #pragma unroll
@@ -295,42 +300,47 @@ __global__ __launch_bounds__(1024) void lutgemm_gradB_slab16_kernel(
     }
     __syncthreads();
 
-    // address pieces: byte0 = half-row (pair member) and column group, byte1 = code (v_perm), byte2 = pair >> 1
-    const uint32_t lo_even = (swap << 7) | (uint32_t)(cg << 3);          // reads 0,2,4,6
-    const uint32_t lo_odd = ((swap ^ 1u) << 7) | (uint32_t)(cg << 3);    // reads 1,3,5,7
-    uint32_t sel[4];                                                     // code byte of read j: (j & 3) ^ swap
+    // address pieces: byte0 = half-row (pair member) and column group, byte1 = code (v_perm), byte2 = k half
+    const uint32_t lo_even = (swap << 7) | (uint32_t)(cg << 4) | (swap << 16);          // reads 0, 2
+    const uint32_t lo_odd = ((swap ^ 1u) << 7) | (uint32_t)(cg << 4) | (swap << 16);    // reads 1, 3
+    uint32_t sel[4];                                                                     // code byte of read j: j ^ swap
 #pragma unroll
     for (int j = 0; j < 4; ++j) sel[j] = 0x0c020400u + ((uint32_t)(j ^ (int)swap) << 8);
     const int ncol = n0 + 4 * cg;
 
-    typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
-    float acc[KT][4];      // acc[j]: k = k0 + (j ^ swap)
-    float gsum[4] = {0.f, 0.f, 0.f, 0.f};
+    typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+    float acc[4][8];       // acc[j]: k = k0 + 4 kh + (j ^ kh); columns 4cg..4cg+3, 32+4cg..32+4cg+3
+    float gsum[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int j = 0; j < KT; ++j)
+    for (int j = 0; j < 4; ++j)
 #pragma unroll
-        for (int c = 0; c < 4; ++c) acc[j][c] = 0.f;
+        for (int c = 0; c < 8; ++c) acc[j][c] = 0.f;
     uint32_t seen = 0;
 
     constexpr int RU = kBwdRU;
-    auto consume = [&](auto sums_tag, uint32_t alo, uint32_t ahi, const f32x4& gvec) __attribute__((always_inline)) {
-        seen |= alo | ahi;
-        const uint32_t a4[2] = {alo, ahi};
-        f16x4 s[KT];
+    auto consume = [&](auto sums_tag, uint32_t a4, const f32x4& g0, const f32x4& g1) __attribute__((always_inline)) {
+        seen |= a4;
+        f16x8 s[4];
 #pragma unroll
-        for (int j = 0; j < KT; ++j) {
-            const uint32_t base = ((j & 1) ? lo_odd : lo_even) | ((j & 4) ? 0x10000u : 0u);
-            const uint32_t addr = __builtin_amdgcn_perm(a4[j >> 2], base, sel[j & 3]);
-            s[j] = *reinterpret_cast<const f16x4*>(smem + addr + ((j >> 1) & 1) * 32768);
+        for (int j = 0; j < 4; ++j) {
+            const uint32_t addr = __builtin_amdgcn_perm(a4, (j & 1) ? lo_odd : lo_even, sel[j]);
+            s[j] = *reinterpret_cast<const f16x8*>(smem + addr + (j >> 1) * 32768);
         }
 #pragma unroll
-        for (int j = 0; j < KT; ++j) {
-            acc[j][0] = __builtin_fmaf(gvec.x, (float)s[j].x, acc[j][0]);
-            acc[j][1] = __builtin_fmaf(gvec.y, (float)s[j].y, acc[j][1]);
-            acc[j][2] = __builtin_fmaf(gvec.z, (float)s[j].z, acc[j][2]);
-            acc[j][3] = __builtin_fmaf(gvec.w, (float)s[j].w, acc[j][3]);
+        for (int j = 0; j < 4; ++j) {
+            acc[j][0] = __builtin_fmaf(g0.x, (float)s[j][0], acc[j][0]);
+            acc[j][1] = __builtin_fmaf(g0.y, (float)s[j][1], acc[j][1]);
+            acc[j][2] = __builtin_fmaf(g0.z, (float)s[j][2], acc[j][2]);
+            acc[j][3] = __builtin_fmaf(g0.w, (float)s[j][3], acc[j][3]);
+            acc[j][4] = __builtin_fmaf(g1.x, (float)s[j][4], acc[j][4]);
+            acc[j][5] = __builtin_fmaf(g1.y, (float)s[j][5], acc[j][5]);
+            acc[j][6] = __builtin_fmaf(g1.z, (float)s[j][6], acc[j][6]);
+            acc[j][7] = __builtin_fmaf(g1.w, (float)s[j][7], acc[j][7]);
         }
-        if (decltype(sums_tag)::value) { gsum[0] += gvec.x; gsum[1] += gvec.y; gsum[2] += gvec.z; gsum[3] += gvec.w; }
+        if (decltype(sums_tag)::value) {
+            gsum[0] += g0.x; gsum[1] += g0.y; gsum[2] += g0.z; gsum[3] += g0.w;
+            gsum[4] += g1.x; gsum[5] += g1.y; gsum[6] += g1.z; gsum[7] += g1.w;
+        }
     };
 
     auto stream_rows = [&](auto sums_tag) __attribute__((always_inline)) {
@@ -339,25 +349,25 @@ __global__ __launch_bounds__(1024) void lutgemm_gradB_slab16_kernel(
 #pragma unroll
         for (int u = 0; u < RU; ++u) {
             const uint32_t m = (uint32_t)(mb + 4 * (wave * RU + u) + rs);
-            aoff[u] = m * (uint32_t)K + (uint32_t)k0;
+            aoff[u] = m * (uint32_t)K + (uint32_t)(k0 + 4 * kh);
             goff[u] = (m * (uint32_t)N + (uint32_t)ncol) * 4u;
         }
         const uint32_t astep = (uint32_t)(16 * RU * 4) * (uint32_t)K;
         const uint32_t gstep = (uint32_t)(16 * RU * 4) * (uint32_t)N * 4u;
         const unsigned char* gbytes = reinterpret_cast<const unsigned char*>(gC);
-        uint32_t al0[RU], ah0[RU], al1[RU], ah1[RU];
-        f32x4 g0[RU], g1[RU];
+        uint32_t ca[RU], cb[RU];
+        f32x4 ga0[RU], ga1[RU], gb0[RU], gb1[RU];
         // Every load batch is issued unconditionally (beyond the end: the last rows again, nobody consumes them): behind
         // a branch around the loads the compiler's wait in front of the consumer has to cover the path without new
         // loads too, and on the other path it then waits for the first of the loads it has just issued -- no prefetch
         // at all (measured: the waves spent half their time in s_waitcnt).
         int next = 0;
-        auto load = [&](uint32_t (&al)[RU], uint32_t (&ah)[RU], f32x4 (&g)[RU]) {
+        auto load = [&](uint32_t (&c4)[RU], f32x4 (&g0)[RU], f32x4 (&g1)[RU]) {
 #pragma unroll
             for (int u = 0; u < RU; ++u) {
-                al[u] = load_u32_unaligned(A + aoff[u]);
-                ah[u] = load_u32_unaligned(A + aoff[u] + 4);
-                g[u] = *reinterpret_cast<const f32x4*>(gbytes + goff[u]);
+                c4[u] = load_u32_unaligned(A + aoff[u]);
+                g0[u] = *reinterpret_cast<const f32x4*>(gbytes + goff[u]);
+                g1[u] = *reinterpret_cast<const f32x4*>(gbytes + goff[u] + 128);
             }
             ++next;
             const uint32_t as = next < iters ? astep : 0u, gs = next < iters ? gstep : 0u;
@@ -371,19 +381,19 @@ __global__ __launch_bounds__(1024) void lutgemm_gradB_slab16_kernel(
             __builtin_amdgcn_sched_barrier(0);
         };
         if (iters > 0) {
-            load(al0, ah0, g0);
+            load(ca, ga0, ga1);
             int it = 0;
             for (; it + 2 <= iters; it += 2) {
-                load(al1, ah1, g1);
+                load(cb, gb0, gb1);
 #pragma unroll
-                for (int u = 0; u < RU; ++u) consume(sums_tag, al0[u], ah0[u], g0[u]);
-                load(al0, ah0, g0);
+                for (int u = 0; u < RU; ++u) consume(sums_tag, ca[u], ga0[u], ga1[u]);
+                load(ca, ga0, ga1);
 #pragma unroll
-                for (int u = 0; u < RU; ++u) consume(sums_tag, al1[u], ah1[u], g1[u]);
+                for (int u = 0; u < RU; ++u) consume(sums_tag, cb[u], gb0[u], gb1[u]);
             }
             if (it < iters) {
 #pragma unroll
-                for (int u = 0; u < RU; ++u) consume(sums_tag, al0[u], ah0[u], g0[u]);
+                for (int u = 0; u < RU; ++u) consume(sums_tag, ca[u], ga0[u], ga1[u]);
             }
         }
     };
@@ -396,31 +406,39 @@ __global__ __launch_bounds__(1024) void lutgemm_gradB_slab16_kernel(
         if (lane == 0) atomicOr(&flags[1], 1u);
     }
 
-    // row slots 0+2 and 1+3 hold the same k order: add them in registers; the two orders, the 16 waves and
-    // the column sums of gC meet in LDS (the slabs are no longer needed)
+    // the four row slots of a wave are added in registers; the 16 waves and the column sums of gC meet in LDS (the slabs
+    // are no longer needed)
 #pragma unroll
-    for (int j = 0; j < KT; ++j)
+    for (int j = 0; j < 4; ++j)
 #pragma unroll
-        for (int c = 0; c < 4; ++c) acc[j][c] += __shfl_xor(acc[j][c], 32);
+        for (int c = 0; c < 8; ++c) {
+            acc[j][c] += __shfl_xor(acc[j][c], 32);
+            acc[j][c] += __shfl_xor(acc[j][c], 16);
+        }
 #pragma unroll
-    for (int c = 0; c < 4; ++c) gsum[c] += __shfl_xor(gsum[c], 32);
+    for (int c = 0; c < 8; ++c) {
+        gsum[c] += __shfl_xor(gsum[c], 32);
+        gsum[c] += __shfl_xor(gsum[c], 16);
+    }
     __syncthreads();
-    float* red = reinterpret_cast<float*>(smem);   // [wave][slot][KT + 1][64]
-    if (rs < 2) {
-        float* r = red + (size_t)((wave * 2 + rs) * (KT + 1)) * 64 + 4 * cg;
+    float* red = reinterpret_cast<float*>(smem);   // [wave][KT + 1][64]
+    if (rs == 0) {
+        float* r = red + (size_t)(wave * (KT + 1)) * 64 + 4 * cg;
 #pragma unroll
-        for (int j = 0; j < KT; ++j)
+        for (int j = 0; j < 4; ++j)
 #pragma unroll
-            for (int c = 0; c < 4; ++c) r[(j ^ (int)swap) * 64 + c] = acc[j][c];
+            for (int c = 0; c < 8; ++c) r[(4 * kh + (j ^ kh)) * 64 + 32 * (c >> 2) + (c & 3)] = acc[j][c];
+        if (kh == 0) {
 #pragma unroll
-        for (int c = 0; c < 4; ++c) r[KT * 64 + c] = gsum[c];
+            for (int c = 0; c < 8; ++c) r[KT * 64 + 32 * (c >> 2) + (c & 3)] = gsum[c];
+        }
     }
     __syncthreads();
     if (tid < KT * 64) {
         const int kk = tid >> 6, col = tid & 63;
         float v = 0.f, gs = 0.f;
 #pragma unroll
-        for (int w = 0; w < 32; ++w) {
+        for (int w = 0; w < 16; ++w) {
             v += red[(w * (KT + 1) + kk) * 64 + col];
             gs += red[(w * (KT + 1) + KT) * 64 + col];
         }
