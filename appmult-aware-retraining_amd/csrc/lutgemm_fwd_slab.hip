@@ -160,18 +160,26 @@ __device__ __forceinline__ void slab_addr4(uint32_t (&addr)[4], uint32_t codes4,
 }
 
 // One pair of columns (one dword of each of the four reads of a row group) into its two sums.
+// PACKED (4 * max(lut) < 65536): even / odd are the sums of the even and of the odd column.
+// Otherwise: even collects the whole dwords, i.e. sum(even entries) + 65536 * sum(odd entries) modulo 2^32, and odd the odd
+// entries alone; slab_store_tile takes 65536 * odd off again (the sums are defined modulo 2^32 anyway).  That is six
+// instructions per eight entries instead of eight (or twelve with masks and shifts).
 template <bool PACKED>
 __device__ __forceinline__ void slab_add_pair(uint32_t& even, uint32_t& odd, uint32_t x0, uint32_t x1, uint32_t x2, uint32_t x3) {
+    typedef unsigned short us2 __attribute__((ext_vector_type(2)));
     if (PACKED) {
         // (no 16-bit half of these sums overflows, so one 32-bit addition adds both halves and a three-operand
         // addition saves an instruction per pair of columns over packed 16-bit additions)
-        typedef unsigned short us2 __attribute__((ext_vector_type(2)));
         const us2 s = __builtin_bit_cast(us2, (x0 + x1 + x2) + x3);
         even += s.x;
         odd += s.y;
     } else {
-        even += (x0 & 0xffffu) + (x1 & 0xffffu) + (x2 & 0xffffu) + (x3 & 0xffffu);
-        odd += (x0 >> 16) + (x1 >> 16) + (x2 >> 16) + (x3 >> 16);
+        even = (even + x0 + x1) + x2 + x3;
+        const us2 hi = {0, 1};
+        odd = __builtin_amdgcn_udot2(__builtin_bit_cast(us2, x0), hi, odd, false);
+        odd = __builtin_amdgcn_udot2(__builtin_bit_cast(us2, x1), hi, odd, false);
+        odd = __builtin_amdgcn_udot2(__builtin_bit_cast(us2, x2), hi, odd, false);
+        odd = __builtin_amdgcn_udot2(__builtin_bit_cast(us2, x3), hi, odd, false);
     }
 }
 
@@ -238,7 +246,7 @@ __device__ __forceinline__ void slab_read_codes(uint32_t (&a)[4], uint32_t addr)
 // so that every store or atomic instruction of a wave covers two whole 128 B lines of C (straight from the accumulators an
 // instruction would touch 16 rows and four dwords in each; a split K adds its sums with atomics, which pay per line).
 // The caller has waited for its loads towards LDS and passed a workgroup barrier.
-template <int RG>
+template <int RG, bool PACKED>
 __device__ __forceinline__ void slab_store_tile(const uint32_t (&acc)[RG][8], unsigned char* wave_lds, int lane, int rs, int cg,
                                                 uint32_t* __restrict__ C, int m_wave, int m_first, int n0, int N, int atomic_out,
                                                 int out_f32) {
@@ -246,8 +254,11 @@ __device__ __forceinline__ void slab_store_tile(const uint32_t (&acc)[RG][8], un
     for (int i = 0; i < RG; ++i) {
         u32x4* dst = reinterpret_cast<u32x4*>(wave_lds + (16 * i + rs) * 128 + cg * 32);
         u32x4 lo, hi;
-        lo.x = acc[i][0]; lo.y = acc[i][1]; lo.z = acc[i][2]; lo.w = acc[i][3];
-        hi.x = acc[i][4]; hi.y = acc[i][5]; hi.z = acc[i][6]; hi.w = acc[i][7];
+        // (see slab_add_pair for what the even accumulators of the unpacked flavour hold)
+        lo.x = PACKED ? acc[i][0] : acc[i][0] - (acc[i][1] << 16); lo.y = acc[i][1];
+        lo.z = PACKED ? acc[i][2] : acc[i][2] - (acc[i][3] << 16); lo.w = acc[i][3];
+        hi.x = PACKED ? acc[i][4] : acc[i][4] - (acc[i][5] << 16); hi.y = acc[i][5];
+        hi.z = PACKED ? acc[i][6] : acc[i][6] - (acc[i][7] << 16); hi.w = acc[i][7];
         dst[0] = lo;
         dst[1] = hi;
     }
@@ -391,7 +402,7 @@ __global__ __launch_bounds__(WAVES * 64) void lutgemm_fwd_slab_kernel(
     if (__builtin_amdgcn_ballot_w64((seen & 0x80808080u) != 0) != 0) {
         if (lane == 0) atomicOr(&flags[1], 1u);
     }
-    slab_store_tile<RG>(acc, smem + wave * 8192, lane, rs, cg, C, m_wave, m_first, tile_x * kSlabCols, N, atomic_out, out_f32);
+    slab_store_tile<RG, PACKED>(acc, smem + wave * 8192, lane, rs, cg, C, m_wave, m_first, tile_x * kSlabCols, N, atomic_out, out_f32);
 }
 
 // ------------------------------------------------------------------------------------------ 8-bit tables
@@ -481,7 +492,7 @@ __global__ __launch_bounds__(1024) void lutgemm_fwd_slab8_kernel(
     }
     // nothing is left in flight towards LDS and every wave has read its last chunk: the buffers take the sums
     asm volatile("s_waitcnt vmcnt(0)\n s_barrier" ::: "memory");
-    slab_store_tile<RG>(acc, smem + wave * 8192, lane, rs, cg, C, m_wave, m_first, tile_x * kSlabCols, N, atomic_out, out_f32);
+    slab_store_tile<RG, PACKED>(acc, smem + wave * 8192, lane, rs, cg, C, m_wave, m_first, tile_x * kSlabCols, N, atomic_out, out_f32);
 }
 
 hipError_t launch_fwd_gated(const uint8_t* A, const uint8_t* B, uint32_t* C, const uint16_t* lut, const LutGeom& g,
