@@ -26,10 +26,11 @@
 // per-lane constant by ONE v_perm_b32 per eight entries.  That needs a < 128: a 7-bit operand holding
 // the masked code 128 (zero contribution) is detected, flags[1] is raised and the direct kernel, queued
 // behind this one and gated on that flag, recomputes C.
-// Accumulation: when 4 * max(lut) < 65536 (flag written by the expand kernel) the four k of a chunk
-// are first added as packed uint16 pairs (plain 32-bit additions: no half overflows) and widened to 32
-// bit once per chunk: 2.5 vector instructions per four entries (one address, two additions, two widening
-// additions per pair of columns and four k), which is what bounds the kernel.
+// Accumulation: the four k of a chunk are first added as packed uint16 pairs (plain 32-bit additions:
+// no half overflows when 4 * max(lut) < 65536, true of every multiplier table of at most 7 bits) and
+// widened to 32 bit once per chunk: 2.5 vector instructions per four entries (one address, two additions,
+// two widening additions per pair of columns and four k), which is what bounds the kernel.  A table with
+// larger entries (the expand kernel leaves the maximum in flags[0]) is left to the gated direct kernel.
 #include <type_traits>
 
 #include "amr_common.h"
@@ -316,9 +317,13 @@ __global__ __launch_bounds__(WAVES * 64) void lutgemm_fwd_slab_kernel(
     const int c_begin = split_z * chunks_per_split;
     const int c_end = min(k_quads, c_begin + chunks_per_split);
     if (c_begin >= c_end) return;
-    // Two instances of this kernel are queued for every GEMM; the table maximum (written by the
-    // expand kernel) decides which one does the work: 16-bit packed partial sums need 4*max < 65536.
-    if ((flags[0] < 16384u) != PACKED) return;
+    // 16-bit packed partial sums need 4 * max(lut) < 65536 (true of every multiplier table of at most 7 bits: 127 * 127 =
+    // 16129; the expand kernel left the maximum in flags[0]).  A table with larger entries goes to the direct kernel,
+    // which is queued behind this launch and gated on flags[1]; the other accumulation flavour serves 8-bit tables.
+    if (PACKED && flags[0] >= 16384u) {
+        if (tid == 0) atomicOr(&flags[1], 1u);
+        return;
+    }
 
     const u32x4* Eblk = E + ((size_t)tile_x * k_quads) * (kSlabChunkBytes / 16);
 
@@ -432,7 +437,6 @@ __global__ __launch_bounds__(1024) void lutgemm_fwd_slab8_kernel(
     const int c_begin = split_z * chunks_per_split;
     const int c_end = min(k_quads, c_begin + chunks_per_split);
     if (c_begin >= c_end) return;
-    if ((flags[0] < 16384u) != PACKED) return;     // both flavours are queued; the table maximum picks one
 
     const u32x4* Eblk = E + ((size_t)tile_x * k_quads) * (kSlab8ChunkBytes / 16);
     // instruction j of a chunk reads k = 4c + ((j + rot) & 3); byte 2 of the address = chunk buffer
@@ -510,7 +514,7 @@ size_t fwd_slab_workspace_bytes(const LutGeom& g, int M, int K, int N, bool forc
         if (!force && (M < 4096 || (size_t)M * K * N < (3ull << 29))) return 0;
         return 256 + (size_t)((N + kSlabCols - 1) / kSlabCols) * (((size_t)K + 3) / 4) * kSlab8ChunkBytes;
     }
-    // below about 4e8 multiply-adds the extra launches (expansion, second flavour, gated fall-back) cost more than the
+    // below about 4e8 multiply-adds the extra launches (expansion, gated fall-back) cost more than the
     // faster kernel gains (measured on MI355X: even at 3e8, 57 against 85 us at 5.4e8)
     if (!force && (size_t)M * K * N < (3ull << 27)) return 0;
     const size_t n_tiles = (N + kSlabCols - 1) / kSlabCols;
@@ -545,8 +549,6 @@ hipError_t launch_fwd_slab(const uint8_t* A, const uint8_t* B, uint32_t* C, cons
         const int zs8 = (k_quads + cps8 - 1) / cps8;
         if (zs8 > 1 && (e = launch_zero_u32(C, (size_t)M * N, stream)) != hipSuccess) return e;
         const dim3 grid8(n_tiles, row_blocks8, zs8);
-        hipLaunchKernelGGL((lutgemm_fwd_slab8_kernel<true>), grid8, dim3(1024), 0, stream, A, reinterpret_cast<const u32x4*>(E), C, flags,
-                           M, K, N, k_quads, cps8, zs8 > 1 ? 1 : 0, out_f32);
         hipLaunchKernelGGL((lutgemm_fwd_slab8_kernel<false>), grid8, dim3(1024), 0, stream, A, reinterpret_cast<const u32x4*>(E), C, flags,
                            M, K, N, k_quads, cps8, zs8 > 1 ? 1 : 0, out_f32);
         if ((e = hipGetLastError()) != hipSuccess) return e;
@@ -584,10 +586,7 @@ hipError_t launch_fwd_slab(const uint8_t* A, const uint8_t* B, uint32_t* C, cons
         grouped = n_tiles;
         grid = dim3(8 * ((row_blocks + 7) / 8) * n_tiles);
     }
-    // both accumulation flavours are queued; flags[0] (table maximum) decides on the device which one works
     hipLaunchKernelGGL((lutgemm_fwd_slab_kernel<RG, WAVES, true>), grid, dim3(WAVES * 64), 0, stream, A,
-                       reinterpret_cast<const u32x4*>(E), C, flags, M, K, N, k_quads, cps, zs > 1 ? 1 : 0, out_f32, grouped, row_blocks);
-    hipLaunchKernelGGL((lutgemm_fwd_slab_kernel<RG, WAVES, false>), grid, dim3(WAVES * 64), 0, stream, A,
                        reinterpret_cast<const u32x4*>(E), C, flags, M, K, N, k_quads, cps, zs > 1 ? 1 : 0, out_f32, grouped, row_blocks);
     e = hipGetLastError();
     if (e != hipSuccess) return e;
@@ -596,8 +595,8 @@ hipError_t launch_fwd_slab(const uint8_t* A, const uint8_t* B, uint32_t* C, cons
         e = launch_u32_to_f32(C, (size_t)M * N, stream);
         if (e != hipSuccess) return e;
     }
-    if (g.bits == 7) return launch_fwd_gated(A, B, C, lut, g, M, K, N, flags + 1, stream, out_f32);
-    return hipGetLastError();
+    // (the fall-back for the masked code of a 7-bit operand and for tables whose entries do not fit packed sums)
+    return launch_fwd_gated(A, B, C, lut, g, M, K, N, flags + 1, stream, out_f32);
 }
 
 }  // namespace amr
