@@ -50,9 +50,8 @@ VALU_ISSUE_PEAK = N_CU * CLK * 64         # lane-operations/s of unpacked VALU i
 HBM_PEAK = 8.0e12
 
 PROFILES = os.path.join(ROOT, "profiles")
-# the expanded-table kernel that runs the conv2_x launch of each phase (the launch the committed counter tables cover),
-# and how many multiply-adds a lane gets out of one of its wide LDS reads (table entries are 2 bytes in all three)
-CONV2X_KERNEL = {"forward": ("lutgemm_fwd_slab_kernel", 4), "gradA": ("lutgemm_gradA_slab_kernel<32", 8), "gradB": ("lutgemm_gradB_slab16_kernel", 4)}
+# the expanded-table kernel that runs the conv2_x launch of each phase (the launch the committed counter tables cover)
+CONV2X_KERNEL = {"forward": "lutgemm_fwd_slab_kernel", "gradA": "lutgemm_gradA_slab_kernel<32", "gradB": "lutgemm_gradB_slab16_kernel"}
 
 
 def profile_rows(name):
@@ -70,17 +69,18 @@ def profile_rows(name):
 
 
 def conv2x_counters(kind):
-    """From profiles/: (bytes the L2s read + wrote for the conv2_x launch of this phase's kernel, VALU instructions per LDS
-    instruction of that kernel); None for what no committed table holds."""
-    kernel, _ = CONV2X_KERNEL[kind]
-    traffic = valu_per_lds = None
+    """From profiles/: (bytes the L2s read + wrote for the conv2_x launch of this phase's kernel, VALU instructions per
+    multiply-add of that kernel = counted wave instructions x 64 lanes / multiply-adds of the counted launches); None for what
+    no committed table holds."""
+    kernel = CONV2X_KERNEL[kind]
+    traffic = valu_per_mac = None
     for k, cells in profile_rows("conv2x_hbm_traffic.md").items():
         if kernel in k:
             traffic = (int(cells[2]) + int(cells[4])) * 2**20          # scaled FETCH_SIZE + WRITE_SIZE, MiB
     for k, cells in profile_rows("conv2x_lds_counters.md").items():
-        if kernel in k:
-            valu_per_lds = float(cells[7])
-    return traffic, valu_per_lds
+        if kernel in k and len(cells) > 9:
+            valu_per_mac = float(cells[9])
+    return traffic, valu_per_mac
 
 
 def training_step_lut_share():
@@ -346,7 +346,8 @@ def main():
                           gC=torch.randn((M1, N1), dtype=torch.float32, device=dev, generator=gen),
                           gA=torch.empty((M1, K1), dtype=torch.float32, device=dev),
                           gB=torch.empty((K1, N1), dtype=torch.float32, device=dev))
-    t_single = timed(lambda: (fwd("single", M1, K1, N1), bwd("single", M1, K1, N1)), reps=50)
+    # (left out of a run restricted to some layers: a profiler run of such a subset then holds launches of those layers only)
+    t_single = timed(lambda: (fwd("single", M1, K1, N1), bwd("single", M1, K1, N1)), reps=50) if full else float("nan")
 
     out = {
         "metric": "LUT-MAC/s fwd+bwd (ResNet-18 conv shapes, 7-bit)" if headline else "LUT-MAC/s fwd+bwd (VGG-16 conv shapes, 8-bit)",
@@ -384,15 +385,15 @@ def main():
 
     # Limits that bound the expanded-table kernels, for the conv2_x launch of each phase (the launch the committed counter
     # tables cover): bytes the kernel reads from LDS (2 per multiply-add: the table entry) against the LDS read bandwidth, and
-    # VALU instructions (counted by the profiler per LDS read) against the VALU issue rate.
+    # VALU instructions (counted by the profiler) against the VALU issue rate.
     conv2x = [l for l in per_layer if l[0] == "conv2_x"]
     if headline and not f32_tables and conv2x:
         _, _, M2, K2, N2, *times = conv2x[0]
         kb = {"launch": f"conv2_x (M={M2},K={K2},N={N2})", "lds_read_peak_GBps": LDS_READ_PEAK / 1e9, "valu_issue_peak_Gops": VALU_ISSUE_PEAK / 1e9}
         for kind, ms in zip(("forward", "gradA", "gradB"), times):
             mac_rate = M2 * K2 * N2 / (ms * 1e-3)
-            traffic, valu_per_lds = conv2x_counters(kind)
-            entry = {"kernel": CONV2X_KERNEL[kind][0], "ms": round(ms, 4), "lut_mac_per_s": mac_rate,
+            traffic, valu_per_mac = conv2x_counters(kind)
+            entry = {"kernel": CONV2X_KERNEL[kind], "ms": round(ms, 4), "lut_mac_per_s": mac_rate,
                      "lds_read": {"achieved_GBps": 2 * mac_rate / 1e9, "frac": 2 * mac_rate / LDS_READ_PEAK},
                      "gather_equivalent_vs_direct_gather_peak": mac_rate / LDS_GATHER_PEAK,
                      "l2_traffic_bytes": traffic, "algorithmic_bytes": hbm_bytes(kind, M2, K2, N2)}
@@ -408,8 +409,7 @@ def main():
             if direct_bytes:
                 entry["lds_direct_delivery"] = {"achieved_GBps": direct_bytes / (ms * 1e-3) / 1e9, "probe_GBps": probe_delivery / 1e9,
                                                 "frac": direct_bytes / (ms * 1e-3) / probe_delivery}
-            if valu_per_lds is not None:
-                valu_per_mac = valu_per_lds / CONV2X_KERNEL[kind][1]
+            if valu_per_mac is not None:
                 entry["valu_issue"] = {"valu_per_mac": round(valu_per_mac, 3), "frac": mac_rate * valu_per_mac / VALU_ISSUE_PEAK}
                 entry["bounded_by"] = "valu_issue" if entry["valu_issue"]["frac"] > entry["lds_read"]["frac"] else "lds_read"
             kb[kind] = entry
