@@ -510,8 +510,9 @@ size_t fwd_slab_workspace_bytes(const LutGeom& g, int M, int K, int N, bool forc
     if (M < 2048 || K < (force ? 32 : 64) || (K & 3) != 0 || (size_t)M * K >= (1ull << 31)) return 0;
     if (g.bits == 8) {
         // 8-bit tables: 64 KB per (column tile, four k); every block of 1024 rows streams all of it, so the rows have to
-        // outnumber the 256 codes well (measured against the direct kernel on MI355X)
-        if (!force && (M < 4096 || (size_t)M * K * N < (3ull << 29))) return 0;
+        // outnumber the 256 codes well (measured against the direct kernel on MI355X: even at 2048 rows, 157 against 198 us
+        // at 4096 x 1152 x 256)
+        if (!force && (M < 4096 || (size_t)M * K * N < (3ull << 28))) return 0;
         return 256 + (size_t)((N + kSlabCols - 1) / kSlabCols) * (((size_t)K + 3) / 4) * kSlab8ChunkBytes;
     }
     // below about 4e8 multiply-adds the extra launches (expansion, gated fall-back) cost more than the
