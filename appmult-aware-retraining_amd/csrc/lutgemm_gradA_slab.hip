@@ -279,29 +279,34 @@ __global__ __launch_bounds__(kGaWaves * 64) void lutgemm_gradA_slab_kernel(
     // The codes of a tile: A[m][k0 + 4 j + c], one byte per chunk and row, packed four to a register.  Assembly loads:
     // the waiting is explicit (the compiler would wait for everything in flight).
     uint32_t codes[2][(CH + 3) / 4];
-    auto load_codes = [&](const Tile& t, uint32_t (&raw)[2][CH]) {
+    // (16 codes = four chunks per load: one address per row, a quarter of the load instructions of dword loads)
+    static_assert(CH % 4 == 0, "the codes of a row are loaded sixteen at a time");
+    auto load_codes = [&](const Tile& t, u32x4 (&raw)[2][CH / 4]) {
         const int m_base = m_base_of(t);
 #pragma unroll
         for (int r = 0; r < 2; ++r) {
             const uint8_t* arow = A + (size_t)(m_base + 16 * r + quad) * K + t.k0;
 #pragma unroll
-            for (int j = 0; j < CH; ++j) asm volatile("global_load_dword %0, %1, off" : "=v"(raw[r][j]) : "v"(arow + 4 * j) : "memory");
+            for (int h = 0; h < CH / 4; ++h)
+                asm volatile("global_load_dwordx4 %0, %1, off offset:%2" : "=v"(raw[r][h]) : "v"(arow), "n"(16 * h) : "memory");
         }
     };
-    auto pack_codes = [&](uint32_t (&raw)[2][CH]) {
+    // byte c of the four dwords of a load, in their order: two v_perm_b32 pick it from pairs of dwords, a third joins them
+    const uint32_t pick = 0x0c0c0000u | (uint32_t)c | ((uint32_t)(4 + c) << 8);
+    auto pack_codes = [&](u32x4 (&raw)[2][CH / 4]) {
         uint32_t high_bits = 0;
 #pragma unroll
         for (int r = 0; r < 2; ++r) {
 #pragma unroll
-            for (int w = 0; w < (CH + 3) / 4; ++w) codes[r][w] = 0;
-#pragma unroll
-            for (int j = 0; j < CH; ++j) {
-                const uint32_t a = (raw[r][j] >> (8 * c)) & 0xffu;
-                high_bits |= a;
-                codes[r][j >> 2] |= a << (8 * (j & 3));
+            for (int w = 0; w < CH / 4; ++w) {
+                const u32x4 q = raw[r][w];
+                const uint32_t lo = __builtin_amdgcn_perm(q.y, q.x, pick);     // {x.byte c, y.byte c, 0, 0}
+                const uint32_t hi = __builtin_amdgcn_perm(q.w, q.z, pick);     // {z.byte c, w.byte c, 0, 0}
+                codes[r][w] = __builtin_amdgcn_perm(hi, lo, 0x05040100u);
+                high_bits |= codes[r][w];
             }
         }
-        if (__builtin_amdgcn_ballot_w64((high_bits & 0x80u) != 0) != 0) {
+        if (__builtin_amdgcn_ballot_w64((high_bits & 0x80808080u) != 0) != 0) {
             if (lane == 0) atomicOr(&flags[2], 1u);
         }
     };
@@ -333,13 +338,13 @@ __global__ __launch_bounds__(kGaWaves * 64) void lutgemm_gradA_slab_kernel(
 #pragma unroll
     for (int i = 0; i < DIST; ++i) request_chunk(i, i);
     {
-        uint32_t raw[2][CH];
+        u32x4 raw[2][CH / 4];
         load_codes(cur, raw);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 #pragma unroll
         for (int r = 0; r < 2; ++r)
 #pragma unroll
-            for (int j = 0; j < CH; ++j) asm volatile("" : "+v"(raw[r][j]));
+            for (int h = 0; h < CH / 4; ++h) asm volatile("" : "+v"(raw[r][h]));
         pack_codes(raw);
     }
     bool after_stores = false;     // the previous tile's stores may still be on their way (this wave issued all NST of them)
@@ -514,7 +519,7 @@ __global__ __launch_bounds__(kGaWaves * 64) void lutgemm_gradA_slab_kernel(
             asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(d[2]), "+v"(d[3]) : : "memory");
             pair_fma(std::integral_constant<int, CH - 1>{}, std::integral_constant<int, 3>{}, d[2], d[3]);
         }
-        uint32_t raw[2][CH];
+        u32x4 raw[2][CH / 4];
         if (nxt.valid) load_codes(nxt, raw);
         const int m_base = m_base_of(cur);
         const bool whole = m_base == cur.m_wave;             // every lane of the wave stores: NST store instructions, no more, no less
@@ -559,7 +564,7 @@ __global__ __launch_bounds__(kGaWaves * 64) void lutgemm_gradA_slab_kernel(
 #pragma unroll
         for (int r = 0; r < 2; ++r)
 #pragma unroll
-            for (int j = 0; j < CH; ++j) asm volatile("" : "+v"(raw[r][j]));
+            for (int h = 0; h < CH / 4; ++h) asm volatile("" : "+v"(raw[r][h]));
         pack_codes(raw);
         after_stores = whole;
         const bool same_rows = nxt.m_wave == cur.m_wave;
