@@ -96,11 +96,12 @@ def test_forward_bit_exact_random_tables(lib, oracle, bits, shape):
     assert (gpu_forward(lib, A, B, flat) == oracle.forward_c(A, B, flat, bits)).all()
 
 
-# shapes with M >= 2048 and K >= 512 take the expanded-table forward path (tables of at most 7 bits)
-# (K % 4 == 0 and K >= 512 take the expanded-table kernels; K % 16 != 0 moves the last group of codes back; a small
-# M x N grid splits K over workgroups)
+# shapes with M >= 2048, K >= 32 and K % 4 == 0 take the expanded-table forward kernels in the mode the fixture sets
+# (K % 16 != 0 moves the last group of codes back; a small M x N grid splits K over workgroups)
 BIG_M_SHAPES = [(2048, 512, 64), (2081, 515, 65), (2081, 516, 65), (3000, 27, 10), (4096, 640, 300), (2500, 1153, 128),
-                (2500, 1156, 128), (5000, 777, 1), (5000, 776, 1), (2048, 2056, 96), (3100, 520, 33)]
+                (2500, 1156, 128), (5000, 777, 1), (5000, 776, 1), (2048, 2056, 96), (3100, 520, 33),
+                # short K (the expanded-table kernels take K >= 32 when forced, K >= 64 by themselves)
+                (2048, 32, 64), (2500, 36, 33), (4096, 64, 512), (2048, 100, 40), (65536, 64, 128)]
 
 
 @pytest.mark.parametrize("bits", [7, 6, 4, 8])
