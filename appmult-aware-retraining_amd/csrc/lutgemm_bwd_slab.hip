@@ -249,25 +249,14 @@ __global__ __launch_bounds__(1024) void lutgemm_gradB_slab16_kernel(
     // Workgroups are dealt to the 8 XCDs round-robin by their index; the workgroups of one XCD (same index mod 8) take
     // consecutive k tiles of one (column tile, M split), so that the rows of gC and A they all stream are shared in
     // that XCD's L2 instead of being fetched once per XCD.
+    // A workgroup keeps its CU and takes every (gridDim.x / 8)-th unit of its XCD's share: the copy of the table in LDS is made
+    // once per workgroup, not once per unit (a unit of 4096 rows lasts 34 us, 3 of them were that copy and the start-up).
     const int total = n_tiles * k_tiles * splits;
     const int per_xcd = (total + 7) / 8;
-    const int logical = (int)(blockIdx.x % 8) * per_xcd + (int)(blockIdx.x / 8);
-    if (logical >= total) return;
-    const int k_tile = logical % k_tiles;
-    const int n_tile = (logical / k_tiles) % n_tiles;
-    const int split = logical / (k_tiles * n_tiles);
-    const int n0 = n_tile * 64;
-    const int k0 = k_tile * KT;
-    const int mb = split * m_chunk;
-    const int me = min(M, mb + m_chunk);
     if (flags[6] != 0u) return;                  // the table cannot be held as halves (bwd_header_kernel): the direct kernel does it
     const float offset = (float)(int)flags[4];   // bwd_header_kernel
-
-    {   // expansion.  First the table itself goes to LDS, as halves, 128 x 128 without the padding (32 KB behind the
-        // slabs; codes the table does not have read as zero): 16 independent loads per thread, one trip to L2.
-        // The slabs are then gathered from that copy: wave-uniform code a, lanes = columns.  (Gathering them from
-        // the table in global memory took 64 loads per thread in 8 dependent rounds: 5 of the 12 us a workgroup
-        // spends outside its streaming loop, a third of the run time of a layer of 4096 rows.)
+    {   // The table itself goes to LDS, as halves, 128 x 128 without the padding (32 KB behind the slabs; codes the table
+        // does not have read as zero): 16 independent loads per thread, one trip to L2.
         _Float16* tab = reinterpret_cast<_Float16*>(smem + KT * 16384);
         bool inexact = false;
 #pragma unroll
@@ -279,6 +268,22 @@ __global__ __launch_bounds__(1024) void lutgemm_gradB_slab16_kernel(
             tab[idx] = h;
         }
         if (__builtin_amdgcn_ballot_w64(inexact) != 0 && lane == 0) atomicOr(&flags[1], 1u);
+    }
+    for (int slot = (int)(blockIdx.x / 8); slot < per_xcd; slot += (int)(gridDim.x / 8)) {
+    const int logical = (int)(blockIdx.x % 8) * per_xcd + slot;
+    if (logical >= total) break;
+    const int k_tile = logical % k_tiles;
+    const int n_tile = (logical / k_tiles) % n_tiles;
+    const int split = logical / (k_tiles * n_tiles);
+    const int n0 = n_tile * 64;
+    const int k0 = k_tile * KT;
+    const int mb = split * m_chunk;
+    const int me = min(M, mb + m_chunk);
+
+    {   // The slabs are gathered from the copy of the table: wave-uniform code a, lanes = columns.  (Gathering them from
+        // the table in global memory took 64 loads per thread in 8 dependent rounds: 5 of the 12 us a workgroup
+        // spent outside its streaming loop.)
+        const _Float16* tab = reinterpret_cast<const _Float16*>(smem + KT * 16384);
         const int col = lane;
         int bcode[KT];
 #pragma unroll
@@ -444,6 +449,8 @@ __global__ __launch_bounds__(1024) void lutgemm_gradB_slab16_kernel(
         }
         out[((size_t)split * K + k0 + kk) * N + n0 + col] = v * scale;
         if (do_sums && kk == 0) colsum[(size_t)split * N + n0 + col] = gs;
+    }
+    __syncthreads();     // the sums have been read: the slabs of the next unit may be written
     }
 }
 
@@ -623,7 +630,9 @@ hipError_t launch_gradB_slab(const float* gC, const uint8_t* A, const uint8_t* B
         float* part16 = partials + kBwdColsumSplits * (size_t)N;
         out = zs > 1 ? part16 : gB;
         const int total = (int)(grid.x * grid.y * grid.z);
-        hipLaunchKernelGGL(lutgemm_gradB_slab16_kernel, dim3(8 * ((total + 7) / 8)), dim3(1024), 0, stream, gC, A, B, out, lut, g.cols,
+        // (one workgroup per CU at most; the workgroups of an XCD walk their share of the units in steps of that many)
+        const int per_xcd16 = (total + 7) / 8, cus_per_xcd16 = n_cu >= 8 ? n_cu / 8 : 1;
+        hipLaunchKernelGGL(lutgemm_gradB_slab16_kernel, dim3(8 * (per_xcd16 < cus_per_xcd16 ? per_xcd16 : cus_per_xcd16)), dim3(1024), 0, stream, gC, A, B, out, lut, g.cols,
                            1 << g.bits, flags, M, K, N, m_chunk, scale, (int)grid.x, (int)grid.y, (int)grid.z, colsum);
         hipError_t e16 = hipGetLastError();
         if (e16 != hipSuccess) return e16;
