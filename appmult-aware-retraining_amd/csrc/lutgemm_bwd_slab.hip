@@ -269,6 +269,15 @@ __global__ __launch_bounds__(1024) void lutgemm_gradB_slab16_kernel(
         }
         if (__builtin_amdgcn_ballot_w64(inexact) != 0 && lane == 0) atomicOr(&flags[1], 1u);
     }
+    // the codes of B of a unit (lanes = its 64 columns, eight k) are loaded while the previous unit is being finished
+    auto load_b_codes = [&](int logical_u, int (&bc)[KT]) {
+        const int lu = min(logical_u, total - 1);
+        const int kt_u = lu % k_tiles, nt_u = (lu / k_tiles) % n_tiles;
+#pragma unroll
+        for (int kk = 0; kk < KT; ++kk) bc[kk] = (int)B[(size_t)(kt_u * KT + kk) * N + nt_u * 64 + lane];
+    };
+    int bnext[KT];
+    load_b_codes((int)(blockIdx.x % 8) * per_xcd + (int)(blockIdx.x / 8), bnext);
     for (int slot = (int)(blockIdx.x / 8); slot < per_xcd; slot += (int)(gridDim.x / 8)) {
     const int logical = (int)(blockIdx.x % 8) * per_xcd + slot;
     if (logical >= total) break;
@@ -287,7 +296,7 @@ __global__ __launch_bounds__(1024) void lutgemm_gradB_slab16_kernel(
         const int col = lane;
         int bcode[KT];
 #pragma unroll
-        for (int kk = 0; kk < KT; ++kk) bcode[kk] = (int)B[(size_t)(k0 + kk) * N + n0 + col];
+        for (int kk = 0; kk < KT; ++kk) bcode[kk] = bnext[kk];
         __syncthreads();
         const _Float16 zero = (_Float16)(-offset);
 #pragma unroll
@@ -410,6 +419,7 @@ __global__ __launch_bounds__(1024) void lutgemm_gradB_slab16_kernel(
     if (__builtin_amdgcn_ballot_w64((seen & 0x80808080u) != 0) != 0) {
         if (lane == 0) atomicOr(&flags[1], 1u);
     }
+    load_b_codes(logical + (int)(gridDim.x / 8), bnext);       // (beyond the last unit: the last one again, unused)
 
     // the four row slots of a wave are added in registers; the 16 waves and the column sums of gC meet in LDS (the slabs
     // are no longer needed)
