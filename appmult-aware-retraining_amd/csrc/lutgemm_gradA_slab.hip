@@ -170,6 +170,26 @@ __device__ __forceinline__ void ga_read(u32x4& d, uint32_t codeword, uint32_t la
                  : "memory");
 }
 
+// One piece (eight floats) of the two rows of gC a lane works on, from the staging area (the rows are 2 KB apart: 16 rows
+// of 128 B): four 128-bit reads, NOT waited for ...
+__device__ __forceinline__ void ga_issue_piece(u32x4 (&t)[4], uint32_t addr) {
+    asm volatile("ds_read_b128 %0, %4\n ds_read_b128 %1, %4 offset:16\n ds_read_b128 %2, %4 offset:2048\n ds_read_b128 %3, %4 offset:2064"
+                 : "=&v"(t[0]), "=&v"(t[1]), "=&v"(t[2]), "=&v"(t[3])
+                 : "v"(addr)
+                 : "memory");
+}
+// ... and, once they have landed, into piece S of the register copy of the rows.
+template <int S, int COLS>
+__device__ __forceinline__ void ga_take_piece(float (&g0)[COLS], float (&g1)[COLS], const u32x4 (&t)[4]) {
+    static_assert(8 * S + 7 < COLS, "piece index");
+    const f32x4 a0 = __builtin_bit_cast(f32x4, t[0]), a1 = __builtin_bit_cast(f32x4, t[1]);
+    const f32x4 b0 = __builtin_bit_cast(f32x4, t[2]), b1 = __builtin_bit_cast(f32x4, t[3]);
+    g0[8 * S] = a0.x; g0[8 * S + 1] = a0.y; g0[8 * S + 2] = a0.z; g0[8 * S + 3] = a0.w;
+    g0[8 * S + 4] = a1.x; g0[8 * S + 5] = a1.y; g0[8 * S + 6] = a1.z; g0[8 * S + 7] = a1.w;
+    g1[8 * S] = b0.x; g1[8 * S + 1] = b0.y; g1[8 * S + 2] = b0.z; g1[8 * S + 3] = b0.w;
+    g1[8 * S + 4] = b1.x; g1[8 * S + 5] = b1.y; g1[8 * S + 6] = b1.z; g1[8 * S + 7] = b1.w;
+}
+
 // grid: 8 * (workgroups per XCD, at most one per CU) workgroups of 1024 threads; every workgroup walks several tiles
 // (512 rows x KT k) one after the other.  Requires N % 32 == 0, K % KT == 0, M >= 32, M*K < 2^31, gC 16-byte aligned.
 // rows_per_image = 0: gA row-major [M,K]; L > 0: image-major transposed gA[m / L][k][m % L].
@@ -447,56 +467,46 @@ __global__ __launch_bounds__(kGaWaves * 64) void lutgemm_gradA_slab_kernel(
         if (KC != 0 || nt != 0) pair_fma(std::integral_constant<int, KP>{}, std::integral_constant<int, 3>{}, d[2], d[3]);
         ga_read<KC & 3, BUF>(d[2], codes[0][KC >> 2], lane_const[1]);
         ga_read<KC & 3, BUF>(d[3], codes[1][KC >> 2], lane_const[1]);
-        if (KC == 0) {
-            // new column tile: the rows of gC from the staging area, pieces in this lane's rotated order
+        if constexpr (!F32 && KC == 0) {
+            // New column tile: the rows of gC come from the staging area, piece by piece in this lane's rotated order (piece
+            // s = eight floats of both rows = four reads).  Only the first piece is waited for on the spot; the reads of
+            // piece s + 1 travel while the multiply-adds of step s run.
             const uint32_t gbase = (uint32_t)(STAGE_BASE + wave * STAGE_WAVE + quad * (COLS * 4));
+            u32x4 t[4];
+            ga_issue_piece(t, gbase + (uint32_t)(((quad + 0) & 3) << 5));
+            asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(t[0]), "+v"(t[1]), "+v"(t[2]), "+v"(t[3]), "+v"(d[0]), "+v"(d[1]), "+v"(d[2]), "+v"(d[3]) : : "memory");
+            ga_take_piece<0>(g[0], g[1], t);
+            ga_issue_piece(t, gbase + (uint32_t)(((quad + 1) & 3) << 5));
+            __builtin_amdgcn_s_setprio(2);
+            pair_fma(kc_tag, std::integral_constant<int, 0>{}, d[0], d[1]);
+            ga_read<KC & 3, BUF>(d[0], codes[0][KC >> 2], lane_const[2]);
+            ga_read<KC & 3, BUF>(d[1], codes[1][KC >> 2], lane_const[2]);
+            asm volatile("s_waitcnt lgkmcnt(2)" : "+v"(t[0]), "+v"(t[1]), "+v"(t[2]), "+v"(t[3]) : : "memory");
+            ga_take_piece<1>(g[0], g[1], t);
+            ga_issue_piece(t, gbase + (uint32_t)(((quad + 2) & 3) << 5));
+            __builtin_amdgcn_s_setprio(1);
+            pair_fma(kc_tag, std::integral_constant<int, 1>{}, d[2], d[3]);
+            ga_read<KC & 3, BUF>(d[2], codes[0][KC >> 2], lane_const[3]);
+            ga_read<KC & 3, BUF>(d[3], codes[1][KC >> 2], lane_const[3]);
+            asm volatile("s_waitcnt lgkmcnt(2)" : "+v"(t[0]), "+v"(t[1]), "+v"(t[2]), "+v"(t[3]), "+v"(d[0]), "+v"(d[1]) : : "memory");
+            ga_take_piece<2>(g[0], g[1], t);
+            ga_issue_piece(t, gbase + (uint32_t)(((quad + 3) & 3) << 5));
+            __builtin_amdgcn_s_setprio(0);
+            pair_fma(kc_tag, std::integral_constant<int, 2>{}, d[0], d[1]);
+            // (the last pair of table reads of this chunk is consumed behind the next barrier, as in every step; here its
+            // landing is waited for together with the last piece)
+            asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(t[0]), "+v"(t[1]), "+v"(t[2]), "+v"(t[3]), "+v"(d[2]), "+v"(d[3]) : : "memory");
+            ga_take_piece<3>(g[0], g[1], t);
+            if (sum_rows) {
 #pragma unroll
-            for (int r = 0; r < 2; ++r) {
-                if constexpr (F32) {
-                    // a row is 64 B: piece (quad + s) % 4 for step s, one 128-bit read each
-                    u32x4 t[4];
+                for (int r = 0; r < 2; ++r) {
+                    float sr = row_sum[r];
 #pragma unroll
-                    for (int s = 0; s < 4; ++s) {
-                        const uint32_t ga = gbase + (uint32_t)(((quad + s) & 3) << 4);
-                        if (r == 0) asm volatile("ds_read_b128 %0, %1" : "=&v"(t[s]) : "v"(ga) : "memory");
-                        else asm volatile("ds_read_b128 %0, %1 offset:1024" : "=&v"(t[s]) : "v"(ga) : "memory");
-                    }
-                    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(t[0]), "+v"(t[1]), "+v"(t[2]), "+v"(t[3]), "+v"(d[0]), "+v"(d[1]), "+v"(d[2]), "+v"(d[3]) : : "memory");
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        const f32x4 v = __builtin_bit_cast(f32x4, t[i]);
-                        g[r][4 * i] = v.x; g[r][4 * i + 1] = v.y; g[r][4 * i + 2] = v.z; g[r][4 * i + 3] = v.w;
-                    }
-                } else {
-                // (two pieces at a time: eight more registers in flight would not fit)
-#pragma unroll
-                for (int hf = 0; hf < 2; ++hf) {
-                    u32x4 t[4];
-#pragma unroll
-                    for (int s2 = 0; s2 < 2; ++s2) {
-                        const int s = 2 * hf + s2;
-                        const uint32_t ga = gbase + (uint32_t)(((quad + s) & 3) << 5);
-                        if (r == 0) {
-                            asm volatile("ds_read_b128 %0, %2\n ds_read_b128 %1, %2 offset:16" : "=&v"(t[2 * s2]), "=&v"(t[2 * s2 + 1]) : "v"(ga) : "memory");
-                        } else {
-                            asm volatile("ds_read_b128 %0, %2 offset:2048\n ds_read_b128 %1, %2 offset:2064" : "=&v"(t[2 * s2]), "=&v"(t[2 * s2 + 1]) : "v"(ga) : "memory");
-                        }
-                    }
-                    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(t[0]), "+v"(t[1]), "+v"(t[2]), "+v"(t[3]), "+v"(d[0]), "+v"(d[1]), "+v"(d[2]), "+v"(d[3]) : : "memory");
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        const f32x4 v = __builtin_bit_cast(f32x4, t[i]);
-                        g[r][16 * hf + 4 * i] = v.x; g[r][16 * hf + 4 * i + 1] = v.y; g[r][16 * hf + 4 * i + 2] = v.z; g[r][16 * hf + 4 * i + 3] = v.w;
-                    }
-                }
-                if (sum_rows) {
-                    float s = row_sum[r];
-#pragma unroll
-                    for (int i = 0; i < COLS; ++i) s += g[r][i];
-                    row_sum[r] = s;
-                }
+                    for (int i = 0; i < COLS; ++i) sr += g[r][i];
+                    row_sum[r] = sr;
                 }
             }
+            return;
         }
         __builtin_amdgcn_s_setprio(2);
         asm volatile("s_waitcnt lgkmcnt(2)" : "+v"(d[0]), "+v"(d[1]) : : "memory");
