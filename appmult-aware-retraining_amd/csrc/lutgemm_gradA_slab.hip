@@ -190,6 +190,29 @@ __device__ __forceinline__ void ga_take_piece(float (&g0)[COLS], float (&g1)[COL
     g1[8 * S + 4] = b1.x; g1[8 * S + 5] = b1.y; g1[8 * S + 6] = b1.z; g1[8 * S + 7] = b1.w;
 }
 
+// The results of a tile leave through LDS so that a store instruction covers whole 128 B lines (a lane's own results are
+// single floats 16 B apart per row: stored directly, an instruction touches 16 lines in 16 B pieces and the stores of a
+// tile, 64 KB, cost 2.8 us of its 18).  One float into LDS ...
+__device__ __forceinline__ void ga_lds_put(uint32_t addr, float v) {
+    asm volatile("ds_write_b32 %0, %1" : : "v"(addr), "v"(v) : "memory");
+}
+// ... N 16-byte pieces back (STEP bytes apart), waited for, ...
+template <int N, int STEP>
+__device__ __forceinline__ void ga_lds_get(u32x4 (&q)[N], uint32_t addr) {
+    static_assert(N == 1 || N == 2, "one or two reads");
+    if constexpr (N == 2)
+        asm volatile("ds_read_b128 %0, %2\n ds_read_b128 %1, %2 offset:%3\n s_waitcnt lgkmcnt(0)"
+                     : "=&v"(q[0]), "=&v"(q[1]) : "v"(addr), "n"(STEP) : "memory");
+    else
+        asm volatile("ds_read_b128 %0, %1\n s_waitcnt lgkmcnt(0)" : "=&v"(q[0]) : "v"(addr) : "memory");
+}
+// ... and to memory, not waited for.  (A store of more than 64 bits still reads its data registers for two cycles after
+// it is issued; the compiler keeps its own stores apart from a following write to those registers but does not look into
+// assembly blocks, so the two idle cycles are part of the block.)
+__device__ __forceinline__ void ga_store16(float* p, const u32x4& q) {
+    asm volatile("global_store_dwordx4 %0, %1, off\n s_nop 1" : : "v"(p), "v"(q) : "memory");
+}
+
 // grid: 8 * (workgroups per XCD, at most one per CU) workgroups of 1024 threads; every workgroup walks several tiles
 // (512 rows x KT k) one after the other.  Requires N % 32 == 0, K % KT == 0, M >= 32, M*K < 2^31, gC 16-byte aligned.
 // rows_per_image = 0: gA row-major [M,K]; L > 0: image-major transposed gA[m / L][k][m % L].
@@ -210,7 +233,7 @@ __global__ __launch_bounds__(kGaWaves * 64) void lutgemm_gradA_slab_kernel(
     static_assert(STAGE_BASE + kGaRows * (F32 ? kGaColsF32 : kGaCols) * 4 <= kGaStageBase + kGaStageBytes, "LDS budget");
     constexpr int NTU = (CH % BUFS) == 0 ? 1 : BUFS;       // column tiles per unrolled pass: the buffer of a chunk is then static
     static_assert(NTU == 1 || NTU == 3, "the tile loop below unrolls one or three column tiles");
-    constexpr int NST = 2 * CH;                            // stores per lane at the end of a tile
+    constexpr int NST = CH / 2;                            // 16-byte stores per lane at the end of a tile
     constexpr int COLS = F32 ? kGaColsF32 : kGaCols;       // columns per tile
     constexpr int STAGE_WAVE = kGaRowsPerWave * COLS * 4;  // bytes of gC rows a wave stages per column tile (4 KB / 2 KB)
     constexpr int ROWOPS = STAGE_WAVE / 1024;              // wave-wide 16-byte loads of a row request (4 / 2)
@@ -234,6 +257,8 @@ __global__ __launch_bounds__(kGaWaves * 64) void lutgemm_gradA_slab_kernel(
     const int total = n_tiles * CH;                          // chunks of a tile: (column tile, four k)
     if (!F32 && flags[5] != 0u) return;                      // (set before this launch and never changed during it: every wave sees the same)
     const float offset = F32 ? 0.f : (float)(int)flags[3];
+    // 16-byte stores need gA aligned and, image-major, four consecutive rows in one image (same for every wave)
+    const bool wide_stores = ((uintptr_t)gA & 15) == 0 && (rows_per_image & 3) == 0;
     struct Tile { int k0, m_wave; bool valid; };
     auto decode = [&](int pos) {
         Tile t;
@@ -523,43 +548,91 @@ __global__ __launch_bounds__(kGaWaves * 64) void lutgemm_gradA_slab_kernel(
         pair_fma(kc_tag, std::integral_constant<int, 2>{}, d[0], d[1]);
     };
     // End of a tile: last multiply-adds, the codes of the next tile are asked for, gA of this one is stored meanwhile.
+    // FREE = the buffer of the tile's last chunk: once every wave has read it, it is free until the request of the next
+    // step (issued behind that step's barrier); each wave turns its results round in 2 KB of it.
     // Returns false when the workgroup has no further tile.
-    auto finish_tile = [&]() __attribute__((always_inline)) {
+    auto finish_tile = [&](auto free_tag) __attribute__((always_inline)) {
+        constexpr int FREE = decltype(free_tag)::value;
         if constexpr (!F32) {
             asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(d[2]), "+v"(d[3]) : : "memory");
             pair_fma(std::integral_constant<int, CH - 1>{}, std::integral_constant<int, 3>{}, d[2], d[3]);
         }
         u32x4 raw[2][CH / 4];
         if (nxt.valid) load_codes(nxt, raw);
+        if (wide_stores) asm volatile("s_barrier" ::: "memory");   // (the reads of the last chunk have landed in every wave)
         const int m_base = m_base_of(cur);
-        const bool whole = m_base == cur.m_wave;             // every lane of the wave stores: NST store instructions, no more, no less
-        // (k outside, row inside: the two stores of a k then fill the same 128 B lines of the image-major layout)
-        float* o[2];
+        const bool whole = m_base == cur.m_wave;             // every lane of the wave stores
+        const bool fast = whole && wide_stores;              // NST store instructions, no more, no less
         float corr[2];
-        size_t k_stride = 4;
 #pragma unroll
-        for (int r = 0; r < 2; ++r) {
-            const int m = m_base + 16 * r + quad;
-            corr[r] = offset * row_sum[r];
-            if (m < cur.m_wave) {
-                o[r] = nullptr;          // row stored by the wave above
-            } else if (rows_per_image > 0) {
-                const int img = m / rows_per_image, l = m - img * rows_per_image;
-                o[r] = gA + ((size_t)img * K + cur.k0 + c) * rows_per_image + l;
-                k_stride = (size_t)4 * rows_per_image;
-            } else {
-                o[r] = gA + (size_t)m * K + cur.k0 + c;
-            }
-        }
-        if (whole) {
-#pragma unroll
-            for (int j = 0; j < CH; ++j)
+        for (int r = 0; r < 2; ++r) corr[r] = offset * row_sum[r];
+        if (fast) {
+            // (everything below is derived from the lane number afresh: computed ahead of the tile loop, as the compiler
+            // would, these addresses take registers the main loop does not have)
+            int ln = lane;
+            asm volatile("" : "+v"(ln));
+            const int quad = ln >> 2, c = ln & 3;
+            const uint32_t tbase = (uint32_t)(FREE * kGaChunkBytes + wave * 2048);
+            if (rows_per_image == 0) {
+                // row-major: the 16 rows r of the quads at a time, [row][kGaKT k] floats; the 16 B group j of a row sits at
+                // j ^ (row % CH) (the rows are a multiple of 64 B apart).  Back: lane = (row % (64 / CH), group): whole rows.
+                constexpr int PITCH = kGaKT * 4, RPI = 64 / CH;       // bytes per row; rows per read instruction
+                const uint32_t wr = tbase + (uint32_t)(quad * PITCH + c * 4);
+                const int row = ln / CH, grp = ln % CH;
+                const uint32_t rd = tbase + (uint32_t)(row * PITCH + ((grp ^ (row & (CH - 1))) << 4));
+                // (row + RPI has the same low bits as row when RPI is a multiple of CH; with CH = 8, RPI = 8)
+                static_assert(RPI % CH == 0 || CH / 4 == 1, "the second read of a lane keeps its group position");
+                float* out = gA + (size_t)(m_base + row) * K + cur.k0 + 4 * grp;
 #pragma unroll
                 for (int r = 0; r < 2; ++r) {
-                    const float v = (acc[r][j] + corr[r]) * scale;
-                    asm volatile("global_store_dword %0, %1, off" : : "v"(o[r] + j * k_stride), "v"(v) : "memory");
+#pragma unroll
+                    for (int j = 0; j < CH; ++j)
+                        ga_lds_put(wr + (uint32_t)((j ^ (quad & (CH - 1))) << 4), (acc[r][j] + corr[r]) * scale);
+                    u32x4 q[CH / 4];
+                    ga_lds_get<CH / 4, RPI * PITCH>(q, rd);
+#pragma unroll
+                    for (int i = 0; i < CH / 4; ++i) ga_store16(out + (size_t)(16 * r + RPI * i) * K, q[i]);
                 }
+            } else {
+                // image-major: half of the k at a time, [k][32 rows] floats; the rows of k with k % 4 >= 2 swap their halves
+                // (k and k + 2 are 256 B apart).  Back: lane = (k % 8, four consecutive rows): whole lines of gA[img][k][:].
+                constexpr int KH = kGaKT / 2;
+                const int kl0 = ln >> 3, pp = ln & 7;
+                const uint32_t rd = tbase + (uint32_t)(kl0 * 128 + (((4 * pp) ^ (16 * ((kl0 >> 1) & 1))) << 2));
+                const int m4 = m_base + 4 * pp;
+                const int img = m4 / rows_per_image, l = m4 - img * rows_per_image;
+                float* out = gA + ((size_t)img * K + cur.k0 + kl0) * rows_per_image + l;
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+#pragma unroll
+                    for (int r = 0; r < 2; ++r)
+#pragma unroll
+                        for (int jj = 0; jj < CH / 2; ++jj)
+                            ga_lds_put(tbase + (uint32_t)((4 * jj + c) * 128 + (((16 * r + quad) ^ (16 * (c >> 1))) << 2)),
+                                       (acc[r][h * (CH / 2) + jj] + corr[r]) * scale);
+                    u32x4 q[CH / 4];
+                    ga_lds_get<CH / 4, 8 * 128>(q, rd);
+#pragma unroll
+                    for (int i = 0; i < CH / 4; ++i) ga_store16(out + (size_t)(h * KH + 8 * i) * rows_per_image, q[i]);
+                }
+            }
         } else {
+            // (k outside, row inside: the two stores of a k then fill the same 128 B lines of the image-major layout)
+            float* o[2];
+            size_t k_stride = 4;
+#pragma unroll
+            for (int r = 0; r < 2; ++r) {
+                const int m = m_base + 16 * r + quad;
+                if (m < cur.m_wave) {
+                    o[r] = nullptr;          // row stored by the wave above
+                } else if (rows_per_image > 0) {
+                    const int img = m / rows_per_image, l = m - img * rows_per_image;
+                    o[r] = gA + ((size_t)img * K + cur.k0 + c) * rows_per_image + l;
+                    k_stride = (size_t)4 * rows_per_image;
+                } else {
+                    o[r] = gA + (size_t)m * K + cur.k0 + c;
+                }
+            }
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 #pragma unroll
             for (int j = 0; j < CH; ++j)
@@ -570,13 +643,13 @@ __global__ __launch_bounds__(kGaWaves * 64) void lutgemm_gradA_slab_kernel(
         }
         if (!nxt.valid) return false;
         // the codes have arrived (they were asked for before the stores)
-        if (whole) asm volatile("s_waitcnt vmcnt(%0)" : : "n"(NST) : "memory");
+        if (fast) asm volatile("s_waitcnt vmcnt(%0)" : : "n"(NST) : "memory");
 #pragma unroll
         for (int r = 0; r < 2; ++r)
 #pragma unroll
             for (int h = 0; h < CH / 4; ++h) asm volatile("" : "+v"(raw[r][h]));
         pack_codes(raw);
-        after_stores = whole;
+        after_stores = fast;
         const bool same_rows = nxt.m_wave == cur.m_wave;
         sum_rows = offset != 0.f && !same_rows;
 #pragma unroll
@@ -599,7 +672,7 @@ __global__ __launch_bounds__(kGaWaves * 64) void lutgemm_gradA_slab_kernel(
         }(std::make_integer_sequence<int, CH>{});
         if (++nt < n_tiles) return true;
         nt = 0;
-        return finish_tile();
+        return finish_tile(std::integral_constant<int, (J * CH + CH - 1) % BUFS>{});
     };
     for (;;) {
         if (!tile_step(std::integral_constant<int, 0>{})) break;

@@ -215,7 +215,10 @@ def test_im2col_codes_rejects_wrong_shapes(ops):
 
 
 @pytest.mark.parametrize("M,K,N,L", [(192, 40, 24, 64), (150, 33, 10, 25), (4096, 64, 64, 1024), (6, 5, 3, 1),
-                                     (8192, 32, 32, 1024), (9216, 48, 64, 256)])   # the last two: expanded-table gradA
+                                     # expanded-table gradA: 16 k per workgroup; 32 k per workgroup with images of 64, 16 and 4
+                                     # rows, the last with a ragged row block; images of 2 rows (no 16-byte stores)
+                                     (8192, 32, 32, 1024), (9216, 48, 64, 256), (32768, 128, 32, 64), (32768, 128, 64, 16),
+                                     (33012, 128, 32, 4), (33010, 128, 32, 2), (4100, 32, 64, 4)])
 def test_backward_image_major_ga_equals_row_major(ops, oracle, golden_dir, M, K, N, L):
     import approx_ops
     self_ops, P = ops

@@ -58,11 +58,12 @@ def gpu_forward(lib, A, B, flat_u16):
     return c.cpu().numpy().view(np.uint32)
 
 
-def gpu_backward(lib, g, A, B, la, lb, own_workspace=True):
+def gpu_backward(lib, g, A, B, la, lb, own_workspace=True, ga_offset_floats=0):
     M, K = A.shape
     N = B.shape[1]
     gd, a, b, ta, tb = dev(g), dev(A), dev(B), dev(la), dev(lb)
-    ga = torch.full((M, K), float("nan"), device="cuda")
+    # (ga_offset_floats: gA starts that many floats into its allocation, i.e. aligned to 4 bytes only)
+    ga = torch.full((M * K + ga_offset_floats,), float("nan"), device="cuda")[ga_offset_floats:].view(M, K)
     gb = torch.full((K, N), float("nan"), device="cuda")
     need = lib.amr_lut_gemm_backward_workspace_bytes(M, K, N)
     ws = torch.empty(max(need, 1), dtype=torch.uint8, device="cuda") if own_workspace else None
@@ -285,7 +286,9 @@ def test_backward_large_m_masked_codes(lib, oracle):
 # (N % 32 == 0, K % 16 == 0 and M >= 2048: gradA runs on its own expanded table, 16, 32 or 48 k per workgroup and one to
 # six column tiles, also with a ragged last row block)
 HALF_SLAB_SHAPES = [(4096, 8, 64), (4224, 24, 128), (8192, 64, 64), (16384, 16, 192), (8200, 48, 96), (9001, 64, 32),
-                    (4100, 32, 64), (2148, 144, 160), (5000, 80, 128), (1024, 16, 64), (2048, 48, 128), (1280, 64, 192)]
+                    (4100, 32, 64), (2148, 144, 160), (5000, 80, 128), (1024, 16, 64), (2048, 48, 128), (1280, 64, 192),
+                    # enough tiles for 32 k per workgroup in gradA: whole row blocks; a ragged last one
+                    (32768, 128, 64), (33011, 128, 32)]
 
 
 @pytest.mark.parametrize("bits", [7, 6, 4])
@@ -348,6 +351,22 @@ def test_backward_half_tables_whose_offset_would_swamp_small_entries(lib, oracle
     check_backward(oracle, gpu_backward(lib, g, A, B, la, lb), g, A, B, la, lb, 7)
 
 
+@pytest.mark.parametrize("shape", [(4096, 64, 64), (33011, 128, 32), (4100, 32, 64)])
+def test_backward_ga_aligned_to_four_bytes_only(lib, oracle, shape):
+    """gA one, two and three floats into a 16-byte-aligned allocation: the expanded-table kernel stores 16 bytes at a time
+    where it can and must not where it cannot."""
+    print("backward, gA not 16-byte aligned", shape, flush=True)
+    rng, A, B, _ = rand_case(hash((shape, "u")) % 2**32, *shape, 7)
+    la = oracle.pack_table(rng.integers(-1024, 3073, (128, 128)), 7, np.int16)
+    lb = oracle.pack_table(rng.integers(-1024, 3073, (128, 128)), 7, np.int16)
+    g = rng.standard_normal((shape[0], shape[2])).astype(np.float32)
+    want = gpu_backward(lib, g, A, B, la, lb)
+    check_backward(oracle, want, g, A, B, la, lb, 7)
+    for off in (1, 2, 3):
+        got = gpu_backward(lib, g, A, B, la, lb, ga_offset_floats=off)
+        assert np.array_equal(got[0], want[0]) and np.array_equal(got[1], want[1])
+
+
 def test_backward_config2_difference_tables_and_ste(lib, oracle):
     print("backward config2", flush=True)
     A, B, T, g = oracle.synth_gemm(4096, 576, 64, bits=7, err=64, seed=0)
@@ -400,7 +419,8 @@ def gpu_backward_f32tab(lib, g, A, B, la, lb, scale, own_workspace=True, rows_pe
 # with a ragged last row block)
 F32TAB_SHAPES = [(1, 1, 1), (3, 5, 7), (9, 27, 10), (64, 64, 64), (33, 130, 65), (600, 96, 64), (257, 100, 129), (300, 288, 256),
                  (70, 50, 513), (1100, 27, 64), (4096, 8, 64), (4100, 27, 10), (5000, 130, 65), (2048, 48, 128), (1500, 40, 70),
-                 (1024, 16, 16), (5000, 80, 48), (4096, 64, 32), (9001, 64, 16), (2148, 144, 160), (16384, 32, 64), (8192, 576, 64)]
+                 (1024, 16, 16), (5000, 80, 48), (4096, 64, 32), (9001, 64, 16), (2148, 144, 160), (16384, 32, 64), (8192, 576, 64),
+                 (33011, 128, 32)]
 
 
 @pytest.mark.parametrize("bits", [7, 8, 6, 4])

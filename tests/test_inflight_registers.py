@@ -5,7 +5,8 @@ s_waitcnt blocks, so the compiler does not know that the destination registers o
 written.  It is free to copy one of them (at a merge point of the control flow, or in front of an assembly block that
 ties it as an in/out operand): a copy that sits between the load and its wait reads stale data.  This test compiles the
 device code to assembly and walks every kernel: between an asynchronous load and the wait that covers it no instruction
-may name one of its destination registers.
+may name one of its destination registers.  Likewise a 128-bit store written in assembly must be followed by two idle
+cycles before its data registers are written again.
 """
 import os
 import re
@@ -78,6 +79,52 @@ def scan(asm_text):
     return hits
 
 
+def scan_wide_stores(asm_text):
+    """Returns [(line number, store, next instruction)]: a store of more than 64 bits written in an assembly block whose data
+    registers are written within the two cycles that follow it.  The hardware still reads the data then; the compiler
+    inserts the idle cycles after its own stores only."""
+    hits, in_asm, watch = [], False, []          # watch: [data registers, cycles left, line, text]
+    for ln, raw in enumerate(asm_text.split("\n"), 1):
+        t = raw.strip()
+        if "#ASMSTART" in t:
+            in_asm = True
+            continue
+        if "#ASMEND" in t:
+            in_asm = False
+            continue
+        if not t or t[0] in ";.":
+            continue
+        t = t.split(";")[0].strip()
+        if not t or t.endswith(":"):
+            continue
+        op, args = t.split()[0], t[len(t.split()[0]):]
+        if op == "s_nop":
+            idle = int(args.strip(), 0) + 1
+            watch = [[r, left - idle, l0, t0] for r, left, l0, t0 in watch if left - idle > 0]
+            continue
+        written = _vgprs(args.split(",")[0]) if op.startswith("v_") or "load" in op or op.startswith("ds_read") else set()
+        for r, left, l0, t0 in watch:
+            if r & written:
+                hits.append((l0, t0, t))
+        watch = [[r, left - 1, l0, t0] for r, left, l0, t0 in watch if left - 1 > 0]
+        if in_asm and re.match(r"(global|flat|buffer|scratch)_store_dwordx[34]", op):
+            watch.append([_vgprs(args.split(",")[1]), 2, ln, t])
+    return hits
+
+
+def test_scanner_sees_a_write_behind_a_wide_store():
+    bad = """	;;#ASMSTART
+	global_store_dwordx4 v[62:63], v[52:55], off
+	;;#ASMEND
+	v_readlane_b32 s7, v127, 7
+	v_lshl_add_u64 v[52:53], v[62:63], 0, s[6:7]
+"""
+    assert [h[0] for h in scan_wide_stores(bad)] == [2]
+    assert scan_wide_stores(bad.replace("off\n", "off\n s_nop 1\n")) == []
+    assert scan_wide_stores(bad.replace("v[52:53], v[62:63]", "v[56:57], v[62:63]")) == []
+    assert scan_wide_stores(bad.replace("dwordx4 v[62:63], v[52:55]", "dwordx2 v[62:63], v[52:53]")) == []
+
+
 def test_scanner_sees_a_copy_in_front_of_the_wait():
     bad = """_Zkernel:
 	ds_read_b128 v[4:7], v1
@@ -117,3 +164,5 @@ def test_no_instruction_touches_a_register_whose_load_is_in_flight(source, tmp_p
     assert r.returncode == 0, r.stderr[-2000:]
     hits = scan(out.read_text())
     assert not hits, "\n".join(f"{k}: line {ln}: {ins}  <- in flight: {regs}" for k, ln, ins, regs in hits[:20])
+    wide = scan_wide_stores(out.read_text())
+    assert not wide, "\n".join(f"line {ln}: {st}  <- data written by: {ins}" for ln, st, ins in wide[:20])
