@@ -45,6 +45,11 @@ hipError_t launch_col2im_f32(const float* cols, float* x, int B, int C, int H, i
 hipError_t launch_im2col_u8_f32(const float* x, uint8_t* A, int B, int C, int H, int W, int kh, int kw, int stride, int pad,
                                 int dil, int oh, int ow, hipStream_t stream);
 bool bwd_slab_applies(const LutGeom& g, int M, int K, int N);
+bool gradB_slab8_applies(const LutGeom& g, int M, int K, int N, const float* gC, bool force);
+int gradB_slab8_splits(int M, int K, int N, int n_cu);
+hipError_t launch_gradB_slab8(const float* gC, const uint8_t* A, const uint8_t* B, float* gB, const int16_t* lut,
+                              const LutGeom& g, int M, int K, int N, float scale, float* partials, int n_cu,
+                              hipStream_t stream);
 int gradB_slab_splits(int M, int K, int N, int n_cu);
 size_t gradB_slab_colsum_floats(int N);
 hipError_t launch_gradB_slab(const float* gC, const uint8_t* A, const uint8_t* B, float* gB, const int16_t* lut,
@@ -265,7 +270,8 @@ int amr_lut_gemm_forward(const uint8_t* A, const uint8_t* B, uint32_t* C, const 
 // gradient table of gradA]; each part a multiple of 256 bytes.
 static size_t backward_partial_bytes(int M, int K, int N, int n_cu) {
     size_t direct = amr::gradB_workspace_bytes(M, K, N, n_cu);
-    const int s = amr::gradB_slab_splits(M, K, N, n_cu);
+    const int s7 = amr::gradB_slab_splits(M, K, N, n_cu), s8 = amr::gradB_slab8_splits(M, K, N, n_cu);
+    const int s = s7 > s8 ? s7 : s8;
     size_t slab = (s > 1 ? (size_t)s * K * N * sizeof(float) : 0) + amr::gradB_slab_colsum_floats(N) * sizeof(float);
     const size_t b = direct > slab ? direct : slab;
     return (b + 255) & ~(size_t)255;
@@ -407,6 +413,8 @@ static int backward_impl(const float* gC, const uint8_t* A, const uint8_t* B, fl
     if (gB) {     // (queued also when the gradA launch failed: a forked side stream must be joined again either way)
         if (slab) {
             eb = amr::launch_gradB_slab(gC, A, B, gB, lut_grad_b, g, M, K, N, scale, flags, partials, n_cu, sb);
+        } else if (mode && amr::gradB_slab8_applies(g, M, K, N, gC, mode == 2)) {
+            eb = amr::launch_gradB_slab8(gC, A, B, gB, lut_grad_b, g, M, K, N, scale, partials, n_cu, sb);
         } else {
             eb = amr::launch_gradB(gC, A, B, gB, lut_grad_b, g, M, K, N, scale, partials, n_cu, sb);
         }

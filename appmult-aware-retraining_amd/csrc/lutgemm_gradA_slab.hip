@@ -190,6 +190,21 @@ __device__ __forceinline__ void ga_take_piece(float (&g0)[COLS], float (&g1)[COL
     g1[8 * S + 4] = b1.x; g1[8 * S + 5] = b1.y; g1[8 * S + 6] = b1.z; g1[8 * S + 7] = b1.w;
 }
 
+// The value lane SRC of the quad holds, in all four lanes of the quad.
+template <int SRC>
+__device__ __forceinline__ uint32_t ga_quad_bcast(uint32_t v) {
+    return (uint32_t)__builtin_amdgcn_mov_dpp((int)v, SRC * 0x55, 0xf, 0xf, true);
+}
+// Byte c of the four dwords lane SRC of the quad holds, in their order (pick = the v_perm_b32 selector of byte c of a pair
+// of dwords): two v_perm_b32 pick it from pairs of dwords, a third joins them.
+template <int SRC>
+__device__ __forceinline__ uint32_t ga_codes_from(const u32x4& q, uint32_t pick) {
+    const uint32_t x = ga_quad_bcast<SRC>(q.x), y = ga_quad_bcast<SRC>(q.y), z = ga_quad_bcast<SRC>(q.z), w = ga_quad_bcast<SRC>(q.w);
+    const uint32_t lo = __builtin_amdgcn_perm(y, x, pick);     // {x.byte c, y.byte c, 0, 0}
+    const uint32_t hi = __builtin_amdgcn_perm(w, z, pick);     // {z.byte c, w.byte c, 0, 0}
+    return __builtin_amdgcn_perm(hi, lo, 0x05040100u);
+}
+
 // The results of a tile leave through LDS so that a store instruction covers whole 128 B lines (a lane's own results are
 // single floats 16 B apart per row: stored directly, an instruction touches 16 lines in 16 B pieces and the stores of a
 // tile, 64 KB, cost 2.8 us of its 18).  One float into LDS ...
@@ -321,39 +336,51 @@ __global__ __launch_bounds__(kGaWaves * 64) void lutgemm_gradA_slab_kernel(
             __builtin_amdgcn_global_load_lds((gptr_t)(base + (size_t)(RPO * i) * N + glane),
                                              (lptr_t)(smem + STAGE_BASE + wave * STAGE_WAVE + i * 1024), 16, 0, 0);
     };
-    // The codes of a tile: A[m][k0 + 4 j + c], one byte per chunk and row, packed four to a register.  Assembly loads:
-    // the waiting is explicit (the compiler would wait for everything in flight).
-    uint32_t codes[2][(CH + 3) / 4];
-    // (16 codes = four chunks per load: one address per row, a quarter of the load instructions of dword loads)
-    static_assert(CH % 4 == 0, "the codes of a row are loaded sixteen at a time");
-    auto load_codes = [&](const Tile& t, u32x4 (&raw)[2][CH / 4]) {
-        const int m_base = m_base_of(t);
-#pragma unroll
-        for (int r = 0; r < 2; ++r) {
-            const uint8_t* arow = A + (size_t)(m_base + 16 * r + quad) * K + t.k0;
-#pragma unroll
-            for (int h = 0; h < CH / 4; ++h)
-                asm volatile("global_load_dwordx4 %0, %1, off offset:%2" : "=v"(raw[r][h]) : "v"(arow), "n"(16 * h) : "memory");
-        }
+    // The codes of a tile: A[m][k0 + 4 j + c], one byte per chunk and row, packed four to a register.  The 2 x kGaKT bytes of
+    // the two rows of a quad are fetched once, 16 bytes per lane (lane c: 32 k per tile: row c / 2, codes 16 (c % 2) ...;
+    // 16 k per tile: row c % 2), and dealt out inside the quad.  Assembly load: the waiting is explicit (the compiler would
+    // wait for everything in flight).  The codes of the NEXT tile are asked for in the second step of the last column tile,
+    // in front of the other requests of that step, and have landed at the wait of the third step (which lets only those
+    // other requests be outstanding): their way from memory is hidden behind a step of arithmetic.
+    uint32_t codes[2][CH / 4], codes_next[2][CH / 4];
+    static_assert(CH == 4 || CH == 8, "one or two 16-byte pieces of codes per row");
+    u32x4 craw = {0, 0, 0, 0};
+    // (both derive what they need from the lane number afresh: kept from the start of the kernel, as the compiler would,
+    // these values take registers the main loop does not have)
+    auto request_codes = [&](const Tile& t) {
+        int ln = lane;
+        asm volatile("" : "+v"(ln));
+        const int r = CH == 8 ? ((ln >> 1) & 1) : (ln & 1), h = CH == 8 ? (ln & 1) : 0;
+        const uint8_t* p = A + (size_t)(m_base_of(t) + 16 * r + (ln >> 2)) * K + t.k0 + 16 * h;
+        asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(craw) : "v"(p) : "memory");
     };
-    // byte c of the four dwords of a load, in their order: two v_perm_b32 pick it from pairs of dwords, a third joins them
-    const uint32_t pick = 0x0c0c0000u | (uint32_t)c | ((uint32_t)(4 + c) << 8);
-    auto pack_codes = [&](u32x4 (&raw)[2][CH / 4]) {
+    auto unpack_codes = [&]() {
+        int ln = lane;
+        asm volatile("" : "+v"(craw), "+v"(ln));
+        const uint32_t pick = 0x0c0c0000u | (uint32_t)(ln & 3) | ((uint32_t)(4 + (ln & 3)) << 8);
+        if constexpr (CH == 8) {
+            codes_next[0][0] = ga_codes_from<0>(craw, pick);
+            codes_next[0][1] = ga_codes_from<1>(craw, pick);
+            codes_next[1][0] = ga_codes_from<2>(craw, pick);
+            codes_next[1][1] = ga_codes_from<3>(craw, pick);
+        } else {
+            codes_next[0][0] = ga_codes_from<0>(craw, pick);
+            codes_next[1][0] = ga_codes_from<1>(craw, pick);
+        }
         uint32_t high_bits = 0;
 #pragma unroll
-        for (int r = 0; r < 2; ++r) {
+        for (int r = 0; r < 2; ++r)
 #pragma unroll
-            for (int w = 0; w < CH / 4; ++w) {
-                const u32x4 q = raw[r][w];
-                const uint32_t lo = __builtin_amdgcn_perm(q.y, q.x, pick);     // {x.byte c, y.byte c, 0, 0}
-                const uint32_t hi = __builtin_amdgcn_perm(q.w, q.z, pick);     // {z.byte c, w.byte c, 0, 0}
-                codes[r][w] = __builtin_amdgcn_perm(hi, lo, 0x05040100u);
-                high_bits |= codes[r][w];
-            }
-        }
+            for (int w = 0; w < CH / 4; ++w) high_bits |= codes_next[r][w];
         if (__builtin_amdgcn_ballot_w64((high_bits & 0x80808080u) != 0) != 0) {
             if (lane == 0) atomicOr(&flags[2], 1u);
         }
+    };
+    auto take_codes = [&]() {
+#pragma unroll
+        for (int r = 0; r < 2; ++r)
+#pragma unroll
+            for (int w = 0; w < CH / 4; ++w) codes[r][w] = codes_next[r][w];
     };
 
     float acc[2][CH];
@@ -374,24 +401,18 @@ __global__ __launch_bounds__(kGaWaves * 64) void lutgemm_gradA_slab_kernel(
     u32x4 e[4] = {{0, 0, 0, 0}, {0, 0, 0, 0}, {0, 0, 0, 0}, {0, 0, 0, 0}};      // float32 entries: the second half of a chunk's reads
 
     // Operations of a wave towards memory, in issue order (vmcnt counts them in this order):
-    //   rows(0) chunk(0) .. chunk(DIST - 1) codes | step q: chunk(q + DIST); second step of column tile nt also: rows(nt + 1)
-    //   | end of a tile: codes of the next tile, NST stores | ...
-    // (a chunk request is two operations, a row request ROWOPS = four, two with float32 entries).  At the top of step q, chunk q (requested two steps
-    // earlier) must have landed: all but the requests of the previous step may be outstanding; in the first two
-    // steps of a tile the stores of the previous one as well.
+    //   rows(0) chunk(0) .. chunk(DIST - 1) codes | step q: chunk(q + DIST); second step of column tile nt:
+    //   [last column tile: codes(next tile)] chunk(q + DIST) rows(nt + 1) | end of a tile: NST stores | ...
+    // (a chunk request is two operations, a row request ROWOPS = four, two with float32 entries, the codes one).  At the top
+    // of step q, chunk q (requested DIST steps earlier) must have landed: all but the requests of the steps in between may be
+    // outstanding; in the first two steps of a tile the stores of the previous one as well.
     request_rows(0);
 #pragma unroll
     for (int i = 0; i < DIST; ++i) request_chunk(i, i);
-    {
-        u32x4 raw[2][CH / 4];
-        load_codes(cur, raw);
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-#pragma unroll
-        for (int r = 0; r < 2; ++r)
-#pragma unroll
-            for (int h = 0; h < CH / 4; ++h) asm volatile("" : "+v"(raw[r][h]));
-        pack_codes(raw);
-    }
+    request_codes(cur);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    unpack_codes();
+    take_codes();
     bool after_stores = false;     // the previous tile's stores may still be on their way (this wave issued all NST of them)
 
     // Read i of a chunk (i = 0..7): step s = i / 2, row r = i % 2; data in d[i % 4].  Two pairs of reads are in flight;
@@ -435,13 +456,20 @@ __global__ __launch_bounds__(kGaWaves * 64) void lutgemm_gradA_slab_kernel(
         // of those reads as operands, the register allocator may copy them, i.e. read them, in front of the block)
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         if (KC < 2 && nt == 0 && after_stores) {
-            if (KC == 0) asm volatile("s_waitcnt vmcnt(%2)\n s_barrier" : "+v"(d[2]), "+v"(d[3]) : "n"(NST) : "memory");
-            else asm volatile("s_waitcnt vmcnt(%2)\n s_barrier" : "+v"(d[2]), "+v"(d[3]) : "n"(NST + 2) : "memory");
+            asm volatile("s_waitcnt vmcnt(%2)\n s_barrier" : "+v"(d[2]), "+v"(d[3]) : "n"(OUT + NST) : "memory");
+        } else if (KC == 2) {
+            // the youngest operations are the row request and the chunk request of step 1: codes asked for in front of
+            // them have landed
+            asm volatile("s_waitcnt vmcnt(%2)\n s_barrier" : "+v"(d[2]), "+v"(d[3]) : "n"(2 + ROWOPS) : "memory");
         } else if (KC >= 2 && KC <= DIST + 1) {
             // the row request of step 1 was issued after the request of the chunk this step needs
             asm volatile("s_waitcnt vmcnt(%2)\n s_barrier" : "+v"(d[2]), "+v"(d[3]) : "n"(OUT + ROWOPS) : "memory");
         } else {
             asm volatile("s_waitcnt vmcnt(%2)\n s_barrier" : "+v"(d[2]), "+v"(d[3]) : "n"(OUT) : "memory");
+        }
+        if (KC == 1) {
+            if (nt == n_tiles - 1) request_codes(nxt.valid ? nxt : cur);
+            else asm volatile("" : "=v"(craw));      // (no value to keep: the registers are free in the other column tiles)
         }
         request_chunk(q + DIST, (BUF + DIST) % BUFS);
         if (KC == 1) request_rows(nt + 1);
@@ -496,6 +524,10 @@ __global__ __launch_bounds__(kGaWaves * 64) void lutgemm_gradA_slab_kernel(
             // New column tile: the rows of gC come from the staging area, piece by piece in this lane's rotated order (piece
             // s = eight floats of both rows = four reads).  Only the first piece is waited for on the spot; the reads of
             // piece s + 1 travel while the multiply-adds of step s run.
+            // (addresses from the lane number afresh, not kept in registers over the other steps)
+            int ln = lane;
+            asm volatile("" : "+v"(ln));
+            const int quad = ln >> 2;
             const uint32_t gbase = (uint32_t)(STAGE_BASE + wave * STAGE_WAVE + quad * (COLS * 4));
             u32x4 t[4];
             ga_issue_piece(t, gbase + (uint32_t)(((quad + 0) & 3) << 5));
@@ -547,7 +579,7 @@ __global__ __launch_bounds__(kGaWaves * 64) void lutgemm_gradA_slab_kernel(
         asm volatile("s_waitcnt lgkmcnt(2)" : "+v"(d[0]), "+v"(d[1]) : : "memory");
         pair_fma(kc_tag, std::integral_constant<int, 2>{}, d[0], d[1]);
     };
-    // End of a tile: last multiply-adds, the codes of the next tile are asked for, gA of this one is stored meanwhile.
+    // End of a tile: last multiply-adds, gA of the tile is stored; none of it is waited for.
     // FREE = the buffer of the tile's last chunk: once every wave has read it, it is free until the request of the next
     // step (issued behind that step's barrier); each wave turns its results round in 2 KB of it.
     // Returns false when the workgroup has no further tile.
@@ -557,8 +589,6 @@ __global__ __launch_bounds__(kGaWaves * 64) void lutgemm_gradA_slab_kernel(
             asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(d[2]), "+v"(d[3]) : : "memory");
             pair_fma(std::integral_constant<int, CH - 1>{}, std::integral_constant<int, 3>{}, d[2], d[3]);
         }
-        u32x4 raw[2][CH / 4];
-        if (nxt.valid) load_codes(nxt, raw);
         if (wide_stores) asm volatile("s_barrier" ::: "memory");   // (the reads of the last chunk have landed in every wave)
         const int m_base = m_base_of(cur);
         const bool whole = m_base == cur.m_wave;             // every lane of the wave stores
@@ -642,13 +672,8 @@ __global__ __launch_bounds__(kGaWaves * 64) void lutgemm_gradA_slab_kernel(
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         }
         if (!nxt.valid) return false;
-        // the codes have arrived (they were asked for before the stores)
-        if (fast) asm volatile("s_waitcnt vmcnt(%0)" : : "n"(NST) : "memory");
-#pragma unroll
-        for (int r = 0; r < 2; ++r)
-#pragma unroll
-            for (int h = 0; h < CH / 4; ++h) asm volatile("" : "+v"(raw[r][h]));
-        pack_codes(raw);
+        unpack_codes();            // (they arrived during the last column tile)
+        take_codes();
         after_stores = fast;
         const bool same_rows = nxt.m_wave == cur.m_wave;
         sum_rows = offset != 0.f && !same_rows;

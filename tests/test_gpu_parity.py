@@ -267,6 +267,32 @@ def test_backward_within_tolerance_large_m(lib, oracle, bits, shape):
     check_backward(oracle, gpu_backward(lib, g, A, B, la, lb), g, A, B, la, lb, bits)
 
 
+# 8-bit tables, M % 256 == 0, M >= 2048, K % 4 == 0, N % 64 == 0: gradB on the expanded table held as int16
+# (one to three column tiles, one to 144 k tiles, one and several M splits)
+SLAB8_SHAPES = [(2048, 4, 64), (4096, 8, 64), (4096, 64, 128), (8192, 36, 192), (2304, 12, 64), (16384, 576, 64), (32768, 20, 64)]
+
+
+@pytest.mark.parametrize("shape", SLAB8_SHAPES)
+def test_backward_8bit_int16_slab(lib, oracle, shape):
+    print("backward 8-bit int16 slab", shape, flush=True)
+    rng, A, B, _ = rand_case(hash((shape, "s8")) % 2**32, *shape, 8)
+    A[0, :] = 255                                                       # the last code of both operands occurs
+    B[:, 0] = 255
+    la = oracle.pack_table(rng.integers(-32768, 32768, (256, 256)), 8, np.int16)
+    Gb = rng.integers(-32768, 32768, (256, 256))
+    Gb[255, 255], Gb[0, 0], Gb[255, 0], Gb[0, 255] = -32768, 32767, 12345, -12345
+    lb = oracle.pack_table(Gb, 8, np.int16)
+    g = (rng.standard_normal((shape[0], shape[2])) + 0.25).astype(np.float32)
+    got = gpu_backward(lib, g, A, B, la, lb)
+    check_backward(oracle, got, g, A, B, la, lb, 8)
+    old = lib.amr_set_expanded_table_kernels(0)                          # the direct kernels: same sums in another order
+    try:
+        ref = gpu_backward(lib, g, A, B, la, lb)
+    finally:
+        lib.amr_set_expanded_table_kernels(old)
+    assert np.abs(got[1] - ref[1]).max() <= 1e-5 * np.abs(ref[1]).max()
+
+
 def test_backward_large_m_masked_codes(lib, oracle):
     print("backward large M masked", flush=True)
     M, K, N = 4300, 40, 70
