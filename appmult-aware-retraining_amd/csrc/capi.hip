@@ -25,6 +25,10 @@ hipError_t launch_gradA(const float* gC, const uint8_t* A, const uint8_t* B, flo
                         const LutGeom& g, int M, int K, int N, float scale, int n_cu, hipStream_t stream,
                         const uint32_t* gate = nullptr, int rows_per_image = 0);
 size_t gradA_slab_workspace_bytes(const LutGeom& g, int M, int K, int N, bool force);
+size_t gradA_slab_i16_workspace_bytes(const LutGeom& g, int M, int K, int N, bool force);
+hipError_t launch_gradA_slab_i16(const float* gC, const uint8_t* A, const uint8_t* B, float* gA, const int16_t* lut,
+                                 const LutGeom& g, int M, int K, int N, float scale, int n_cu, uint32_t* flags, void* S,
+                                 int rows_per_image, hipStream_t stream);
 hipError_t launch_gradA_slab(const float* gC, const uint8_t* A, const uint8_t* B, float* gA, const int16_t* lut,
                              const LutGeom& g, int M, int K, int N, float scale, int n_cu, uint32_t* flags, void* S,
                              int rows_per_image, hipStream_t stream);
@@ -278,12 +282,15 @@ static size_t backward_partial_bytes(int M, int K, int N, int n_cu) {
 }
 
 // Size of the expanded table of gradA.  bits == 0: the table width is not known (a query by shape alone), so the scratch
-// is sized for 7-bit tables, the widest the expanded-table kernels take.
+// is sized for the larger of the 7-bit and the 8-bit expanded table.
 static size_t backward_gradA_bytes(int mode, int bits, int M, int K, int N) {
     if (!mode) return 0;
-    amr::LutGeom g;
-    amr::lut_geom_from_bits(bits ? bits : 7, &g);
-    return amr::gradA_slab_workspace_bytes(g, M, K, N, mode == 2);
+    amr::LutGeom g7, g8;
+    amr::lut_geom_from_bits(bits && bits < 8 ? bits : 7, &g7);
+    amr::lut_geom_from_bits(8, &g8);
+    const size_t b7 = bits == 8 ? 0 : amr::gradA_slab_workspace_bytes(g7, M, K, N, mode == 2);
+    const size_t b8 = bits == 0 || bits == 8 ? amr::gradA_slab_i16_workspace_bytes(g8, M, K, N, mode == 2) : 0;
+    return b7 > b8 ? b7 : b8;
 }
 
 size_t amr_lut_gemm_backward_workspace_bytes(int M, int K, int N) {
@@ -384,6 +391,8 @@ static int backward_impl(const float* gC, const uint8_t* A, const uint8_t* B, fl
     float* partials = reinterpret_cast<float*>(reinterpret_cast<unsigned char*>(ws) + 256);
     const bool slab = mode && amr::bwd_slab_applies(g, M, K, N);
     const bool slab_a = mode && allow_slab_a && gA && amr::gradA_slab_workspace_bytes(g, M, K, N, mode == 2) != 0 && ((uintptr_t)gC & 15) == 0;
+    // (8-bit tables: the expanded table holds the int16 entries, nothing to decide in a header)
+    const bool slab_a8 = mode && allow_slab_a && gA && amr::gradA_slab_i16_workspace_bytes(g, M, K, N, mode == 2) != 0 && ((uintptr_t)gC & 15) == 0;
     if ((slab && gB) || slab_a) {
         // flags cleared, offsets of the half-precision tables decided from the tables' extremes
         e = amr::launch_bwd_header(slab_a ? lut_grad_a : nullptr, (slab && gB) ? lut_grad_b : nullptr, g, flags, s);
@@ -406,6 +415,9 @@ static int backward_impl(const float* gC, const uint8_t* A, const uint8_t* B, fl
         if (slab_a)
             e = amr::launch_gradA_slab(gC, A, B, gA, lut_grad_a, g, M, K, N, scale, n_cu, flags,
                                        reinterpret_cast<unsigned char*>(ws) + 256 + partial_bytes, ga_rows_per_image, s);
+        else if (slab_a8)
+            e = amr::launch_gradA_slab_i16(gC, A, B, gA, lut_grad_a, g, M, K, N, scale, n_cu, flags,
+                                           reinterpret_cast<unsigned char*>(ws) + 256 + partial_bytes, ga_rows_per_image, s);
         else
             e = amr::launch_gradA(gC, A, B, gA, lut_grad_a, g, M, K, N, scale, n_cu, s, nullptr, ga_rows_per_image);
     }

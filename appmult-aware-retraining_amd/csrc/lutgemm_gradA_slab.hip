@@ -43,6 +43,7 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 
+constexpr int kGaFmtHalf = 0, kGaFmtF32 = 1, kGaFmtI16 = 2;   // how S holds the entries
 constexpr int kGaCols = 32;                               // columns per tile (half entries; 16 for float32 entries)
 constexpr int kGaColsF32 = 16;
 constexpr int kGaChunkK = 4;
@@ -152,6 +153,45 @@ __global__ __launch_bounds__(256) void expand_gradA_f32_kernel(const uint8_t* __
     }
 }
 
+// The same for an 8-bit int16 table held as it is: S[n_tile][k / 4][a (256 rows)][k % 4][16 columns] int16, 32 KB per chunk
+// (every entry exact whatever the table holds: no offset, no flag).  grid (N / 16, ceil(K / 4 / quads_per_wg)), 256
+// threads, the table (rows x cols int16) in dynamic LDS.
+constexpr int kGaI16MaxQuads = 8;
+__global__ __launch_bounds__(256) void expand_gradA_i16_kernel(const uint8_t* __restrict__ B, const uint32_t* __restrict__ lut32,
+                                                               int lut_dwords, int lut_cols, uint32_t* __restrict__ S, int K, int N,
+                                                               int quads_per_wg) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    stage_table_dwords<256>(smem, lut32, lut_dwords);
+    __syncthreads();
+    const uint16_t* s16 = reinterpret_cast<const uint16_t*>(smem);
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    // a wave writes the 128 B rows of two consecutive codes: lane = (code % 2, k % 4, column pair), one dword per lane
+    const int ap = lane >> 5, ks = (lane >> 3) & 3, cp = lane & 7;
+    const int n = blockIdx.x * kGaColsF32 + 2 * cp;
+    // (the codes of B for all k quads of the workgroup first)
+    uint16_t bpair[kGaI16MaxQuads];
+#pragma unroll
+    for (int pp = 0; pp < kGaI16MaxQuads; ++pp) {
+        const int kq = min(blockIdx.y * quads_per_wg + min(pp, quads_per_wg - 1), K / 4 - 1);
+        const uint8_t* bp = B + (size_t)(4 * kq + ks) * N + n;
+        bpair[pp] = (uint16_t)((uint32_t)bp[0] | ((uint32_t)bp[1] << 8));
+    }
+#pragma unroll
+    for (int pp = 0; pp < kGaI16MaxQuads; ++pp) {
+        if (pp >= quads_per_wg) break;
+        const int kq = blockIdx.y * quads_per_wg + pp;
+        if (4 * kq >= K) break;
+        const uint16_t* p0 = s16 + (int)(bpair[pp] & 0xffu);
+        const uint16_t* p1 = s16 + (int)(bpair[pp] >> 8);
+        uint32_t* chunk = S + ((size_t)blockIdx.x * (K / 4) + kq) * (kGaChunkBytes / 4) + (lane & 31);
+#pragma unroll 8
+        for (int a2 = wave; a2 < 128; a2 += 4) {
+            const int a = 2 * a2 + ap, row = a * lut_cols;
+            chunk[a * 32] = (uint32_t)p0[row] | ((uint32_t)p1[row] << 16);
+        }
+    }
+}
+
 // ------------------------------------------------------------------------------------------ consume
 // One 128-bit LDS read of a chunk, issued and NOT waited for.  The address comes out of ONE v_perm_b32:
 // byte 0 = the lane's constant (window and piece), byte 1 = the code (BYTE of codeword; < 128), byte 2 = 1 for
@@ -167,6 +207,19 @@ __device__ __forceinline__ void ga_read(u32x4& d, uint32_t codeword, uint32_t la
     asm volatile("v_perm_b32 %1, %2, %3, %4\n ds_read_b128 %0, %1 offset:%5"
                  : "=v"(d), "=&v"(addr)
                  : "v"(codeword), "v"(lane_const), "s"(sel), "n"((BUF & 1) ? kGaChunkBytes : 0)
+                 : "memory");
+}
+
+// The same for chunks of int16 entries of an 8-bit table: 256 rows of 128 B (window c 32 B, two pieces), four buffers of
+// 32 KB.  v_perm_b32 assembles twice the address -- byte 0 = twice the lane's offset, byte 1 = the code, byte 2 = the
+// buffer number (byte BUF of the lane's constant; none for buffer 0) -- and a shift halves it.
+template <int BYTE, int BUF>
+__device__ __forceinline__ void ga_read_i16(u32x4& d, uint32_t codeword, uint32_t lane_const) {
+    constexpr uint32_t sel = 0x0c000000u | ((BUF == 0 ? 0x0cu : (uint32_t)BUF) << 16) | ((4u + BYTE) << 8);
+    uint32_t addr;
+    asm volatile("v_perm_b32 %1, %2, %3, %4\n v_lshrrev_b32 %1, 1, %1\n ds_read_b128 %0, %1"
+                 : "=v"(d), "=&v"(addr)
+                 : "v"(codeword), "v"(lane_const), "s"(sel)
                  : "memory");
 }
 
@@ -233,23 +286,25 @@ __device__ __forceinline__ void ga_store16(float* p, const u32x4& q) {
 // rows_per_image = 0: gA row-major [M,K]; L > 0: image-major transposed gA[m / L][k][m % L].
 // F32: S holds float32 entries, 16 columns per tile (a 64 B window is 16 floats, a 128-bit read feeds four v_fma_f32 instead
 // of eight v_fma_mix_f32); no offset.
-template <int kGaKT, bool F32>
+template <int kGaKT, int FMT>
 __global__ __launch_bounds__(kGaWaves * 64) void lutgemm_gradA_slab_kernel(
     const float* __restrict__ gC, const uint8_t* __restrict__ A, const u32x4* __restrict__ S, float* __restrict__ gA,
     uint32_t* __restrict__ flags, int M, int K, int N, float scale, int rows_per_image, int row_blocks, int band_rows_max) {
     __shared__ __align__(16) unsigned char smem[kGaStageBase + kGaStageBytes];
+    constexpr bool F32 = FMT == kGaFmtF32, I16 = FMT == kGaFmtI16, HALF = FMT == kGaFmtHalf;
+    constexpr bool WIDE = !HALF;                           // 4 bytes of S per multiply-add of a row: 16 columns per tile
     constexpr int CH = kGaKT / kGaChunkK;                  // chunks per column tile
     // Chunk buffers: three, requested two chunks ahead; with float32 entries the staging area is half the size and a fourth
     // buffer fits: three chunks ahead (the loop is bound by the delivery of the chunks, 36 KB per 32 K multiply-adds).
-    constexpr int BUFS = F32 ? 4 : kGaBufs;
+    constexpr int BUFS = WIDE ? 4 : kGaBufs;
     constexpr int DIST = BUFS - 1;                         // chunks between a request and its use
     constexpr int OUT = 2 * (DIST - 1);                    // chunk operations issued after the request of the chunk a step needs
     constexpr int STAGE_BASE = BUFS * kGaChunkBytes;
-    static_assert(STAGE_BASE + kGaRows * (F32 ? kGaColsF32 : kGaCols) * 4 <= kGaStageBase + kGaStageBytes, "LDS budget");
+    static_assert(STAGE_BASE + kGaRows * (WIDE ? kGaColsF32 : kGaCols) * 4 <= kGaStageBase + kGaStageBytes, "LDS budget");
     constexpr int NTU = (CH % BUFS) == 0 ? 1 : BUFS;       // column tiles per unrolled pass: the buffer of a chunk is then static
     static_assert(NTU == 1 || NTU == 3, "the tile loop below unrolls one or three column tiles");
     constexpr int NST = CH / 2;                            // 16-byte stores per lane at the end of a tile
-    constexpr int COLS = F32 ? kGaColsF32 : kGaCols;       // columns per tile
+    constexpr int COLS = WIDE ? kGaColsF32 : kGaCols;      // columns per tile
     constexpr int STAGE_WAVE = kGaRowsPerWave * COLS * 4;  // bytes of gC rows a wave stages per column tile (4 KB / 2 KB)
     constexpr int ROWOPS = STAGE_WAVE / 1024;              // wave-wide 16-byte loads of a row request (4 / 2)
     static_assert(CH >= 4, "the bookkeeping of outstanding loads assumes at least four chunks per column tile");
@@ -270,8 +325,8 @@ __global__ __launch_bounds__(kGaWaves * 64) void lutgemm_gradA_slab_kernel(
     const int xcd = (int)(blockIdx.x % 8), pos_stride = (int)(gridDim.x / 8);
     const int n_tiles = N / COLS;
     const int total = n_tiles * CH;                          // chunks of a tile: (column tile, four k)
-    if (!F32 && flags[5] != 0u) return;                      // (set before this launch and never changed during it: every wave sees the same)
-    const float offset = F32 ? 0.f : (float)(int)flags[3];
+    if (HALF && flags[5] != 0u) return;                      // (set before this launch and never changed during it: every wave sees the same)
+    const float offset = HALF ? (float)(int)flags[3] : 0.f;
     // 16-byte stores need gA aligned and, image-major, four consecutive rows in one image (same for every wave)
     const bool wide_stores = ((uintptr_t)gA & 15) == 0 && (rows_per_image & 3) == 0;
     struct Tile { int k0, m_wave; bool valid; };
@@ -295,9 +350,13 @@ __global__ __launch_bounds__(kGaWaves * 64) void lutgemm_gradA_slab_kernel(
     Tile nxt = decode(pos + pos_stride);
 
     // per-lane address constants: window c, piece (quad + s) % 4 at step s; byte 3 = 1 (see ga_read)
+    // (int16 entries: a code's row is 128 B, window c 32 B, two pieces; the constant holds TWICE the offset, the bytes 1, 2, 3
+    // for the buffer number, and ga_read_i16 halves the assembled address)
     uint32_t lane_const[4];
 #pragma unroll
-    for (int s = 0; s < 4; ++s) lane_const[s] = (uint32_t)(c << 6) | (uint32_t)(((quad + s) & 3) << 4) | 0x01000000u;
+    for (int s = 0; s < 4; ++s)
+        lane_const[s] = I16 ? ((uint32_t)(c << 6) | (uint32_t)(((quad + s) & 1) << 5) | 0x03020100u)
+                            : ((uint32_t)(c << 6) | (uint32_t)(((quad + s) & 3) << 4) | 0x01000000u);
 
     typedef const __attribute__((address_space(1))) void* gptr_t;
     typedef __attribute__((address_space(3))) void* lptr_t;
@@ -372,7 +431,8 @@ __global__ __launch_bounds__(kGaWaves * 64) void lutgemm_gradA_slab_kernel(
         for (int r = 0; r < 2; ++r)
 #pragma unroll
             for (int w = 0; w < CH / 4; ++w) high_bits |= codes_next[r][w];
-        if (__builtin_amdgcn_ballot_w64((high_bits & 0x80808080u) != 0) != 0) {
+        // (a masked code 128 of a 7-bit operand; an 8-bit table has a row for every value of a byte)
+        if (!I16 && __builtin_amdgcn_ballot_w64((high_bits & 0x80808080u) != 0) != 0) {
             if (lane == 0) atomicOr(&flags[2], 1u);
         }
     };
@@ -430,6 +490,16 @@ __global__ __launch_bounds__(kGaWaves * 64) void lutgemm_gradA_slab_kernel(
                 s0 = __builtin_fmaf(g[0][S4 + e], f0[e], s0);
                 s1 = __builtin_fmaf(g[1][S4 + e], f1[e], s1);
             }
+        } else if constexpr (I16) {
+            // (entries 2 q and 2 q + 1 are the halves of dword q; the conversion sign-extends the half it selects)
+            constexpr int S8 = 8 * decltype(s_tag)::value;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                s0 = __builtin_fmaf(g[0][S8 + 2 * q], (float)(int16_t)(d0[q] & 0xffffu), s0);
+                s1 = __builtin_fmaf(g[1][S8 + 2 * q], (float)(int16_t)(d1[q] & 0xffffu), s1);
+                s0 = __builtin_fmaf(g[0][S8 + 2 * q + 1], (float)((int32_t)d0[q] >> 16), s0);
+                s1 = __builtin_fmaf(g[1][S8 + 2 * q + 1], (float)((int32_t)d1[q] >> 16), s1);
+            }
         } else {
             constexpr int S8 = 8 * decltype(s_tag)::value;
             const f16x8 h0 = __builtin_bit_cast(f16x8, d0), h1 = __builtin_bit_cast(f16x8, d1);
@@ -473,10 +543,10 @@ __global__ __launch_bounds__(kGaWaves * 64) void lutgemm_gradA_slab_kernel(
         }
         request_chunk(q + DIST, (BUF + DIST) % BUFS);
         if (KC == 1) request_rows(nt + 1);
-        if constexpr (F32) {
+        if constexpr (WIDE) {
             // float32 entries: a read feeds four multiply-adds only, so the loop is bound by the latency of the LDS, not by
             // arithmetic: all eight reads of the chunk are issued at once (the registers are there: 16 values of gC per row
-            // instead of 32) and consumed in order; nothing is carried over the barrier.
+            // instead of 32) and consumed in order; nothing is carried over the barrier.  int16 entries: four reads.
             if (KC == 0) {
                 const uint32_t gbase = (uint32_t)(STAGE_BASE + wave * STAGE_WAVE + quad * (COLS * 4));
 #pragma unroll
@@ -484,7 +554,10 @@ __global__ __launch_bounds__(kGaWaves * 64) void lutgemm_gradA_slab_kernel(
                     u32x4 t[4];
 #pragma unroll
                     for (int s4 = 0; s4 < 4; ++s4) {
-                        const uint32_t ga = gbase + (uint32_t)(((quad + s4) & 3) << 4);
+                        // the rows of gC in the order the entries are read in: 16-byte pieces (quad + s) % 4 of the window
+                        // (int16 entries: 32-byte pieces (quad + s) % 2, i.e. floats 8 ((quad + s4 / 2) % 2) + 4 (s4 % 2) ...)
+                        const uint32_t ga = gbase + (I16 ? (uint32_t)((((quad + (s4 >> 1)) & 1) << 5) | ((s4 & 1) << 4))
+                                                         : (uint32_t)(((quad + s4) & 3) << 4));
                         if (r == 0) asm volatile("ds_read_b128 %0, %1" : "=&v"(t[s4]) : "v"(ga) : "memory");
                         else asm volatile("ds_read_b128 %0, %1 offset:1024" : "=&v"(t[s4]) : "v"(ga) : "memory");
                     }
@@ -495,6 +568,17 @@ __global__ __launch_bounds__(kGaWaves * 64) void lutgemm_gradA_slab_kernel(
                         g[r][4 * i] = v.x; g[r][4 * i + 1] = v.y; g[r][4 * i + 2] = v.z; g[r][4 * i + 3] = v.w;
                     }
                 }
+            }
+            if constexpr (I16) {
+                ga_read_i16<KC & 3, BUF>(d[0], codes[0][KC >> 2], lane_const[0]);
+                ga_read_i16<KC & 3, BUF>(d[1], codes[1][KC >> 2], lane_const[0]);
+                ga_read_i16<KC & 3, BUF>(d[2], codes[0][KC >> 2], lane_const[1]);
+                ga_read_i16<KC & 3, BUF>(d[3], codes[1][KC >> 2], lane_const[1]);
+                asm volatile("s_waitcnt lgkmcnt(2)" : "+v"(d[0]), "+v"(d[1]) : : "memory");
+                pair_fma(kc_tag, std::integral_constant<int, 0>{}, d[0], d[1]);
+                asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(d[2]), "+v"(d[3]) : : "memory");
+                pair_fma(kc_tag, std::integral_constant<int, 1>{}, d[2], d[3]);
+                return;
             }
             ga_read<KC & 3, BUF>(d[0], codes[0][KC >> 2], lane_const[0]);
             ga_read<KC & 3, BUF>(d[1], codes[1][KC >> 2], lane_const[0]);
@@ -520,7 +604,7 @@ __global__ __launch_bounds__(kGaWaves * 64) void lutgemm_gradA_slab_kernel(
         if (KC != 0 || nt != 0) pair_fma(std::integral_constant<int, KP>{}, std::integral_constant<int, 3>{}, d[2], d[3]);
         ga_read<KC & 3, BUF>(d[2], codes[0][KC >> 2], lane_const[1]);
         ga_read<KC & 3, BUF>(d[3], codes[1][KC >> 2], lane_const[1]);
-        if constexpr (!F32 && KC == 0) {
+        if constexpr (HALF && KC == 0) {
             // New column tile: the rows of gC come from the staging area, piece by piece in this lane's rotated order (piece
             // s = eight floats of both rows = four reads).  Only the first piece is waited for on the spot; the reads of
             // piece s + 1 travel while the multiply-adds of step s run.
@@ -585,7 +669,7 @@ __global__ __launch_bounds__(kGaWaves * 64) void lutgemm_gradA_slab_kernel(
     // Returns false when the workgroup has no further tile.
     auto finish_tile = [&](auto free_tag) __attribute__((always_inline)) {
         constexpr int FREE = decltype(free_tag)::value;
-        if constexpr (!F32) {
+        if constexpr (HALF) {
             asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(d[2]), "+v"(d[3]) : : "memory");
             pair_fma(std::integral_constant<int, CH - 1>{}, std::integral_constant<int, 3>{}, d[2], d[3]);
         }
@@ -748,15 +832,58 @@ hipError_t launch_gradA_slab(const float* gC, const uint8_t* A, const uint8_t* B
     const int per_xcd = (tiles + 7) / 8, cus_per_xcd = n_cu >= 8 ? n_cu / 8 : 1;
     const dim3 grid(8 * (per_xcd < cus_per_xcd ? per_xcd : cus_per_xcd));
     if (kt == 32)
-        hipLaunchKernelGGL((lutgemm_gradA_slab_kernel<32, false>), grid, block, 0, stream, gC, A, S4, gA, flags, M, K, N, scale,
+        hipLaunchKernelGGL((lutgemm_gradA_slab_kernel<32, kGaFmtHalf>), grid, block, 0, stream, gC, A, S4, gA, flags, M, K, N, scale,
                            rows_per_image, row_blocks, band_rows);
     else
-        hipLaunchKernelGGL((lutgemm_gradA_slab_kernel<16, false>), grid, block, 0, stream, gC, A, S4, gA, flags, M, K, N, scale,
+        hipLaunchKernelGGL((lutgemm_gradA_slab_kernel<16, kGaFmtHalf>), grid, block, 0, stream, gC, A, S4, gA, flags, M, K, N, scale,
                            rows_per_image, row_blocks, band_rows);
     e = hipGetLastError();
     if (e != hipSuccess) return e;
     // masked codes in A or table entries a half cannot hold: the gated direct kernel recomputes gA
     return launch_gradA(gC, A, B, gA, lut, g, M, K, N, scale, n_cu, stream, flags + 2, rows_per_image);
+}
+
+// ------------------------------------------------------------------------------------------ 8-bit tables
+// Bytes of the int16 expanded table of an 8-bit gradient table, or 0 when that kernel does not apply.  It is twice the size
+// of the half one of a 7-bit table (256 code rows); every block of 512 rows streams all of it.
+size_t gradA_slab_i16_workspace_bytes(const LutGeom& g, int M, int K, int N, bool force) {
+    if (!force && (M < 4096 || (double)M * K * N < 2e8)) return 0;
+    if (g.bits != 8 || M < 512 || (N % kGaColsF32) != 0 || (K % 16) != 0 || (size_t)M * K >= (1ull << 31)) return 0;
+    return (size_t)(N / kGaColsF32) * (K / kGaChunkK) * kGaChunkBytes;
+}
+
+// No flag is read or written: 8-bit operands have no masked code and every int16 entry is held exactly.
+hipError_t launch_gradA_slab_i16(const float* gC, const uint8_t* A, const uint8_t* B, float* gA, const int16_t* lut,
+                                 const LutGeom& g, int M, int K, int N, float scale, int n_cu, uint32_t* flags, void* S,
+                                 int rows_per_image, hipStream_t stream) {
+    if (((uintptr_t)gC & 15) != 0) return hipErrorInvalidValue;   // callers check: rows of gC are fetched 16 bytes at a time
+    const int lut_dwords = g.rows * g.cols / 2;
+    static std::atomic<uint64_t> attr_done{0};
+    if (hipError_t ea = allow_full_lds(reinterpret_cast<const void*>(expand_gradA_i16_kernel), attr_done); ea != hipSuccess) return ea;
+    // every workgroup copies the table (130 KB) into its LDS: as many chunks per workgroup as still leave one workgroup per CU
+    const long chunks = (long)(N / kGaColsF32) * (K / 4);
+    long qpw = chunks / (n_cu > 0 ? n_cu : 1);
+    qpw = qpw < 1 ? 1 : (qpw > kGaI16MaxQuads ? kGaI16MaxQuads : qpw);
+    hipLaunchKernelGGL(expand_gradA_i16_kernel, dim3(N / kGaColsF32, (unsigned)((K / 4 + qpw - 1) / qpw)), dim3(256),
+                       (size_t)lut_dwords * 4, stream, B, reinterpret_cast<const uint32_t*>(lut), lut_dwords, g.cols,
+                       reinterpret_cast<uint32_t*>(S), K, N, (int)qpw);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    const u32x4* S4 = reinterpret_cast<const u32x4*>(S);
+    const dim3 block(kGaWaves * 64);
+    const int row_blocks = (M + kGaRows - 1) / kGaRows;
+    const int band_rows = 16;
+    const int kt = ((K % 32) == 0 && row_blocks * (K / 32) >= n_cu) ? 32 : 16;
+    const int tiles = row_blocks * (K / kt);
+    const int per_xcd = (tiles + 7) / 8, cus_per_xcd = n_cu >= 8 ? n_cu / 8 : 1;
+    const dim3 grid(8 * (per_xcd < cus_per_xcd ? per_xcd : cus_per_xcd));
+    if (kt == 32)
+        hipLaunchKernelGGL((lutgemm_gradA_slab_kernel<32, kGaFmtI16>), grid, block, 0, stream, gC, A, S4, gA, flags, M, K, N, scale,
+                           rows_per_image, row_blocks, band_rows);
+    else
+        hipLaunchKernelGGL((lutgemm_gradA_slab_kernel<16, kGaFmtI16>), grid, block, 0, stream, gC, A, S4, gA, flags, M, K, N, scale,
+                           rows_per_image, row_blocks, band_rows);
+    return hipGetLastError();
 }
 
 // ------------------------------------------------------------------------------------------ float32 tables
@@ -795,10 +922,10 @@ hipError_t launch_gradA_slab_f32tab(const float* gC, const uint8_t* A, const uin
     const int per_xcd = (tiles + 7) / 8, cus_per_xcd = n_cu >= 8 ? n_cu / 8 : 1;
     const dim3 grid(8 * (per_xcd < cus_per_xcd ? per_xcd : cus_per_xcd));
     if (kt == 32)
-        hipLaunchKernelGGL((lutgemm_gradA_slab_kernel<32, true>), grid, block, 0, stream, gC, A, S4, gA, flags, M, K, N, scale,
+        hipLaunchKernelGGL((lutgemm_gradA_slab_kernel<32, kGaFmtF32>), grid, block, 0, stream, gC, A, S4, gA, flags, M, K, N, scale,
                            rows_per_image, row_blocks, band_rows);
     else
-        hipLaunchKernelGGL((lutgemm_gradA_slab_kernel<16, true>), grid, block, 0, stream, gC, A, S4, gA, flags, M, K, N, scale,
+        hipLaunchKernelGGL((lutgemm_gradA_slab_kernel<16, kGaFmtF32>), grid, block, 0, stream, gC, A, S4, gA, flags, M, K, N, scale,
                            rows_per_image, row_blocks, band_rows);
     e = hipGetLastError();
     if (e != hipSuccess) return e;

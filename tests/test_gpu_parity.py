@@ -35,6 +35,8 @@ def lib():
     L.amr_lut_gemm_backward_f32tab_workspace_bytes.restype = sz
     L.amr_lut_gemm_backward_workspace_bytes.argtypes = [i, i, i]
     L.amr_lut_gemm_backward_workspace_bytes.restype = sz
+    L.amr_lut_gemm_backward_workspace_bytes_for.argtypes = [i64, i, i, i]
+    L.amr_lut_gemm_backward_workspace_bytes_for.restype = sz
     L.amr_acc_gemm_forward_fp32.argtypes = [vp, vp, vp, i, i, i, vp]
     # mode 2: the expanded-table kernels wherever the shape allows, so that the test sizes (small next to the sizes
     # at which the library would pick them by itself) exercise them; mode 0 / 1 have tests of their own below
@@ -291,6 +293,31 @@ def test_backward_8bit_int16_slab(lib, oracle, shape):
     finally:
         lib.amr_set_expanded_table_kernels(old)
     assert np.abs(got[1] - ref[1]).max() <= 1e-5 * np.abs(ref[1]).max()
+
+
+# 8-bit tables, M >= 512 (forced; 4096 by itself), K % 16 == 0, N % 16 == 0: gradA on the expanded table held as int16, 16 or
+# 32 k per tile, one to twelve column tiles, ragged last row block
+SLAB8_GA_SHAPES = [(4096, 16, 16), (4096, 64, 64), (4100, 32, 48), (9001, 64, 16), (2148, 144, 160), (33011, 128, 32), (32768, 128, 192),
+                   (1024, 16, 64)]
+
+
+@pytest.mark.parametrize("shape", SLAB8_GA_SHAPES)
+def test_backward_8bit_int16_expanded_table_gradA(lib, oracle, shape):
+    print("backward 8-bit int16 expanded table, gradA", shape, flush=True)
+    rng, A, B, _ = rand_case(hash((shape, "a8")) % 2**32, *shape, 8)
+    A[0, :] = 255                                                       # the last code of both operands occurs
+    A[-1, :] = 128
+    B[:, 0] = 255
+    Ga = rng.integers(-32768, 32768, (256, 256))
+    Ga[255, 255], Ga[0, 0], Ga[255, 0], Ga[0, 255] = -32768, 32767, 12345, -12345
+    la = oracle.pack_table(Ga, 8, np.int16)
+    lb = oracle.pack_table(rng.integers(-32768, 32768, (256, 256)), 8, np.int16)
+    g = (rng.standard_normal((shape[0], shape[2])) + 0.25).astype(np.float32)
+    got = gpu_backward(lib, g, A, B, la, lb)
+    check_backward(oracle, got, g, A, B, la, lb, 8)
+    for off in (0, 1):                                                  # gA aligned to 16 and to 4 bytes
+        again = gpu_backward(lib, g, A, B, la, lb, ga_offset_floats=off)
+        assert np.array_equal(again[0], got[0])
 
 
 def test_backward_large_m_masked_codes(lib, oracle):
@@ -572,7 +599,10 @@ def test_backward_float_tables_expanded_gradA_masked_codes(lib, oracle):
     la = oracle.pack_table(rng.standard_normal((128, 128)) * 10, 7, np.float32)
     lb = oracle.pack_table(rng.standard_normal((128, 128)) * 10, 7, np.float32)
     g = rng.standard_normal((M, N)).astype(np.float32)
-    assert lib.amr_lut_gemm_backward_f32tab_workspace_bytes(M, K, N) > lib.amr_lut_gemm_backward_workspace_bytes(M, K, N) > 0
+    # (queried by shape alone the int16 scratch is sized for an 8-bit table as well, whose expanded table is as large as
+    # the float32 one of a 7-bit table; with the table's size given it is half of that)
+    assert lib.amr_lut_gemm_backward_f32tab_workspace_bytes(M, K, N) >= lib.amr_lut_gemm_backward_workspace_bytes(M, K, N) > 0
+    assert lib.amr_lut_gemm_backward_f32tab_workspace_bytes(M, K, N) > lib.amr_lut_gemm_backward_workspace_bytes_for(129 * 130 + 638, M, K, N) > 0
     check_backward(oracle, gpu_backward_f32tab(lib, g, A, B, la, lb, 1.0), g, A, B, la, lb, 7, factor=1.0)
     A2, B2 = A.copy(), B.copy()
     A2[::7, 3] = 128
