@@ -421,44 +421,55 @@ __global__ __launch_bounds__(1024) void lutgemm_gradB_slab16_kernel(
     }
     load_b_codes(logical + (int)(gridDim.x / 8), bnext);       // (beyond the last unit: the last one again, unused)
 
-    // the four row slots of a wave are added in registers; the 16 waves and the column sums of gC meet in LDS (the slabs
-    // are no longer needed)
+    // The 4 row slots x 16 waves meet in LDS (the slabs are no longer needed; the copy of the table behind them stays):
+    // every lane leaves its 32 sums there with eight 16-byte writes, red[wave][rs][k][64 columns] (128 KB), and the sums
+    // over (wave, rs) are formed in a fixed order: two partial sums of 32 terms per output by all 1024 threads, then their
+    // sum.  (Adding the row slots in registers first took 64 cross-lane operations per wave and unit.)  The lanes of k half
+    // 1 keep the two halves of a row of 64 the other way round: the 16 lanes the LDS serves together then write 64
+    // different banks.
+    __syncthreads();
+    float* red = reinterpret_cast<float*>(smem);
+    {
+        float* r = red + (size_t)((wave * 4 + rs) * KT) * 64 + 4 * cg;
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
-#pragma unroll
-        for (int c = 0; c < 8; ++c) {
-            acc[j][c] += __shfl_xor(acc[j][c], 32);
-            acc[j][c] += __shfl_xor(acc[j][c], 16);
+        for (int j = 0; j < 4; ++j) {
+            const int kk = 4 * kh + (j ^ kh);
+            const f32x4 lo = {acc[j][0], acc[j][1], acc[j][2], acc[j][3]}, hi = {acc[j][4], acc[j][5], acc[j][6], acc[j][7]};
+            *reinterpret_cast<f32x4*>(r + kk * 64 + 32 * kh) = lo;
+            *reinterpret_cast<f32x4*>(r + kk * 64 + 32 * (kh ^ 1)) = hi;
         }
-#pragma unroll
-    for (int c = 0; c < 8; ++c) {
-        gsum[c] += __shfl_xor(gsum[c], 32);
-        gsum[c] += __shfl_xor(gsum[c], 16);
     }
     __syncthreads();
-    float* red = reinterpret_cast<float*>(smem);   // [wave][KT + 1][64]
-    if (rs == 0) {
-        float* r = red + (size_t)(wave * (KT + 1)) * 64 + 4 * cg;
+    float part = 0.f;
+    {
+        const int o = tid & 511, p = tid >> 9;          // output (k, column) and half of the (wave, rs) pairs
+        const float* r = red + (size_t)(p * 32 * KT) * 64 + (o ^ (((o >> 8) & 1) << 5));      // (o >> 8 = k half of the output)
+#pragma unroll 8
+        for (int t = 0; t < 32; ++t) part += r[t * KT * 64];
+    }
+    __syncthreads();
+    red[tid] = part;
+    if (do_sums) {      // (same for every thread) the column sums of gC: row slots in registers, waves through LDS
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+        for (int c = 0; c < 8; ++c) {
+            gsum[c] += __shfl_xor(gsum[c], 32);
+            gsum[c] += __shfl_xor(gsum[c], 16);
+        }
+        if (rs == 0 && kh == 0) {
 #pragma unroll
-            for (int c = 0; c < 8; ++c) r[(4 * kh + (j ^ kh)) * 64 + 32 * (c >> 2) + (c & 3)] = acc[j][c];
-        if (kh == 0) {
-#pragma unroll
-            for (int c = 0; c < 8; ++c) r[KT * 64 + 32 * (c >> 2) + (c & 3)] = gsum[c];
+            for (int c = 0; c < 8; ++c) red[1024 + wave * 64 + 32 * (c >> 2) + 4 * cg + (c & 3)] = gsum[c];
         }
     }
     __syncthreads();
     if (tid < KT * 64) {
         const int kk = tid >> 6, col = tid & 63;
-        float v = 0.f, gs = 0.f;
+        out[((size_t)split * K + k0 + kk) * N + n0 + col] = (red[tid] + red[512 + tid]) * scale;
+        if (do_sums && kk == 0) {
+            float gs = 0.f;
 #pragma unroll
-        for (int w = 0; w < 16; ++w) {
-            v += red[(w * (KT + 1) + kk) * 64 + col];
-            gs += red[(w * (KT + 1) + KT) * 64 + col];
+            for (int w = 0; w < 16; ++w) gs += red[1024 + w * 64 + col];
+            colsum[(size_t)split * N + n0 + col] = gs;
         }
-        out[((size_t)split * K + k0 + kk) * N + n0 + col] = v * scale;
-        if (do_sums && kk == 0) colsum[(size_t)split * N + n0 + col] = gs;
     }
     __syncthreads();     // the sums have been read: the slabs of the next unit may be written
     }

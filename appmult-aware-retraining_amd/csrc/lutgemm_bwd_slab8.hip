@@ -71,18 +71,22 @@ __global__ __launch_bounds__(1024) void lutgemm_gradB_slab8_kernel(
         const int me = min(M, mb + m_chunk);
 
         {   // The slabs are gathered from the table in global memory (132 KB: it stays in the L2): wave-uniform code a,
-            // lanes = columns; the 16 loads of a k are issued before the first is stored.
+            // lanes = columns; all 64 loads of a thread are issued before the first is stored (one trip to the L2 per
+            // unit instead of one per k: at 2048 rows per unit the gather is a quarter of the unit's time otherwise).
             const int col = lane;
             __syncthreads();
+            int16_t e[KT][16];
+#pragma unroll
+            for (int kk = 0; kk < KT; ++kk) {
+                const int16_t* t = G + bnext[kk];
+#pragma unroll
+                for (int i = 0; i < 16; ++i) e[kk][i] = t[(wave + 16 * i) * lut_cols];
+            }
 #pragma unroll
             for (int kk = 0; kk < KT; ++kk) {
                 unsigned char* s = smem + (kk >> 1) * 65536 + (kk & 1) * 128 + 2 * (8 * ((col & 31) >> 2) + 4 * (col >> 5) + (col & 3));
-                const int16_t* t = G + bnext[kk];
-                int16_t e[16];
 #pragma unroll
-                for (int i = 0; i < 16; ++i) e[i] = t[(wave + 16 * i) * lut_cols];
-#pragma unroll
-                for (int i = 0; i < 16; ++i) *reinterpret_cast<int16_t*>(s + (wave + 16 * i) * 256) = e[i];
+                for (int i = 0; i < 16; ++i) *reinterpret_cast<int16_t*>(s + (wave + 16 * i) * 256) = e[kk][i];
             }
         }
         __syncthreads();
@@ -179,35 +183,38 @@ __global__ __launch_bounds__(1024) void lutgemm_gradB_slab8_kernel(
         }
         load_b_codes(logical + (int)(gridDim.x / 8), bnext);       // (beyond the last unit: the last one again, unused)
 
-        // The eight row slots of a wave are added in registers: slots of the same parity hold the same k in acc[j]; a slot
-        // of the other parity holds it in acc[j ^ 1].  The 16 waves meet in LDS (the slabs are no longer needed).
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-#pragma unroll
-            for (int c = 0; c < 8; ++c) {
-                acc[j][c] += __shfl_xor(acc[j][c], 32);
-                acc[j][c] += __shfl_xor(acc[j][c], 16);
-            }
-        float tot[4][8];
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-#pragma unroll
-            for (int c = 0; c < 8; ++c) tot[j][c] = acc[j][c] + __shfl_xor(acc[j ^ 1][c], 8);
+        // The 8 row slots x 16 waves meet in LDS (the slabs are no longer needed): every lane leaves its 32 sums there with
+        // eight 16-byte writes, red[wave][rs][k][64 columns] (128 KB), and the sums over (wave, rs) are formed in a fixed
+        // order: four partial sums of 32 terms per output by all 1024 threads, then their sum.  (Adding the row slots in
+        // registers first took 96 cross-lane operations per wave and unit.)
         __syncthreads();
-        float* red = reinterpret_cast<float*>(smem);   // [wave][KT][64]
-        if (rs == 0) {      // (swap == 0: tot[j] is k0 + j)
-            float* r = red + (size_t)(wave * KT) * 64 + 4 * cg;
+        float* red = reinterpret_cast<float*>(smem);
+        {
+            float* r = red + (size_t)((wave * 8 + rs) * KT) * 64 + 4 * cg;
 #pragma unroll
-            for (int j = 0; j < 4; ++j)
-#pragma unroll
-                for (int c = 0; c < 8; ++c) r[j * 64 + 32 * (c >> 2) + (c & 3)] = tot[j][c];
+            for (int j = 0; j < 4; ++j) {
+                const int kk = j ^ (int)swap;
+                const f32x4 lo = {acc[j][0], acc[j][1], acc[j][2], acc[j][3]}, hi = {acc[j][4], acc[j][5], acc[j][6], acc[j][7]};
+                // (odd row slots keep their two halves of a row of 64 the other way round: the 16 lanes the LDS serves
+                // together then write 64 different banks)
+                *reinterpret_cast<f32x4*>(r + kk * 64 + 32 * (int)swap) = lo;
+                *reinterpret_cast<f32x4*>(r + kk * 64 + 32 * (int)(swap ^ 1u)) = hi;
+            }
         }
+        __syncthreads();
+        float part = 0.f;
+        {
+            const int o = tid & 255, p = tid >> 8;          // output (k, column) and quarter of the (wave, rs) pairs
+            const float* r = red + (size_t)(p * 32 * KT) * 64;
+#pragma unroll 8
+            for (int t = 0; t < 32; ++t) part += r[t * KT * 64 + (o ^ ((t & 1) << 5))];      // (t % 2 = parity of the row slot)
+        }
+        __syncthreads();
+        red[tid] = part;
         __syncthreads();
         if (tid < KT * 64) {
             const int kk = tid >> 6, col = tid & 63;
-            float v = 0.f;
-#pragma unroll
-            for (int w = 0; w < 16; ++w) v += red[(w * KT + kk) * 64 + col];
+            const float v = ((red[tid] + red[256 + tid]) + red[512 + tid]) + red[768 + tid];
             out[((size_t)split * K + k0 + kk) * N + n0 + col] = v * scale;
         }
         // (the barrier at the top of the next unit's slab build keeps these reads ahead of its writes)

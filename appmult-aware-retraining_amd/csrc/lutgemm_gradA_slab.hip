@@ -846,8 +846,9 @@ hipError_t launch_gradA_slab(const float* gC, const uint8_t* A, const uint8_t* B
 // ------------------------------------------------------------------------------------------ 8-bit tables
 // Bytes of the int16 expanded table of an 8-bit gradient table, or 0 when that kernel does not apply.  It is twice the size
 // of the half one of a 7-bit table (256 code rows); every block of 512 rows streams all of it.
+// (measured on MI355X against the direct kernel: 1.6-1.9 x faster from 8192 rows on, 1.3 x at 2048 rows, 0.65 x at 512)
 size_t gradA_slab_i16_workspace_bytes(const LutGeom& g, int M, int K, int N, bool force) {
-    if (!force && (M < 4096 || (double)M * K * N < 2e8)) return 0;
+    if (!force && (M < 2048 || (double)M * K * N < 2e8)) return 0;
     if (g.bits != 8 || M < 512 || (N % kGaColsF32) != 0 || (K % 16) != 0 || (size_t)M * K >= (1ull << 31)) return 0;
     return (size_t)(N / kGaColsF32) * (K / kGaChunkK) * kGaChunkBytes;
 }
