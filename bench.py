@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the LUT-GEMM hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--layers] [--grad-tables f32] [--workload vgg16_b128_8bit] [--codes captured]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-train-step] [--no-8bit] [--layers] [--grad-tables f32] [--workload vgg16_b128_8bit] [--codes captured]
 
 One "step" = forward + backward (gradA and gradB) LUT-GEMM of every conv layer and the fc layer of a
 CIFAR-style ResNet-18 at batch 256, 7-bit tables (BASELINE.json configs[2]: 21 GEMMs,
@@ -152,6 +152,62 @@ def training_step(torch, dev, tables, bits, batch=512, steps=10):
             "lut_gemm_share_of_gpu_time": share, "share_source": "profiles/resnet18_b512_training_step_kernels.md (rocprofv3 --kernel-trace)"}
 
 
+def eight_bit_step(torch, np, dev, lib, O, stream, steps=5):
+    """The 8-bit stress configuration (BASELINE.json configs[3]: VGG-16 conv shapes at batch 128, 8-bit int16 tables) as a
+    secondary record of the default run: the same forward + backward GEMM step as the headline, timed over `steps` steps after
+    two untimed ones.  (`--workload vgg16_b128_8bit` runs it as the main workload, with the per-kernel break-down.)"""
+    bits, err, half_ws = 8, 256, 16
+    rng = np.random.default_rng(0)
+    T = O.synth_lut(bits, err, rng)
+    Gx, Gy = O.gen_bp_lut(T, half_ws)
+    lut = torch.from_numpy(O.pack_table(T, bits, np.uint16)).to(dev)
+    lga = torch.from_numpy(O.pack_table(Gx, bits, np.int16)).to(dev)
+    lgb = torch.from_numpy(O.pack_table(Gy, bits, np.int16)).to(dev)
+    L = lut.numel()
+    gen = torch.Generator(device=dev).manual_seed(0)
+    bufs, ws_need = {}, 0
+    for name, cnt, M, K, N in VGG16_B128:
+        bufs[name] = (torch.randint(0, 256, (M, K), dtype=torch.uint8, device=dev, generator=gen),
+                      torch.randint(0, 256, (K, N), dtype=torch.uint8, device=dev, generator=gen),
+                      torch.empty((M, N), dtype=torch.int32, device=dev),
+                      torch.randn((M, N), dtype=torch.float32, device=dev, generator=gen),
+                      torch.empty((M, K), dtype=torch.float32, device=dev), torch.empty((K, N), dtype=torch.float32, device=dev))
+        ws_need = max(ws_need, lib.amr_lut_gemm_backward_workspace_bytes(M, K, N))
+    ws = torch.empty(max(ws_need, 256), dtype=torch.uint8, device=dev)
+
+    def step():
+        for name, cnt, M, K, N in VGG16_B128:
+            A, B, C = bufs[name][:3]
+            for _ in range(cnt):
+                assert lib.amr_lut_gemm_forward(A.data_ptr(), B.data_ptr(), C.data_ptr(), lut.data_ptr(), L, M, K, N, stream) == 0, lib.amr_last_error()
+        for name, cnt, M, K, N in reversed(VGG16_B128):
+            A, B, C, gC, gA, gB = bufs[name]
+            for _ in range(cnt):
+                assert lib.amr_lut_gemm_backward(gC.data_ptr(), A.data_ptr(), B.data_ptr(), gA.data_ptr(), gB.data_ptr(), lga.data_ptr(),
+                                                 lgb.data_ptr(), L, M, K, N, ws.data_ptr(), ws.numel(), stream) == 0, lib.amr_last_error()
+
+    # parity guard on a row sample of one layer that takes the expanded int16 tables (the parity suite proper is tests/ -m gpu)
+    name, _, M, K, N = VGG16_B128[2]
+    A, B, C, gC, gA, gB = bufs[name]
+    step()
+    torch.cuda.synchronize()
+    rows = slice(100, 132)
+    want_a, _ = O.backward_c_f32(gC[rows].cpu().numpy(), A[rows].cpu().numpy(), B.cpu().numpy(), lga.cpu().numpy(), lgb.cpu().numpy(), bits)
+    got_a = gA[rows].cpu().numpy()
+    assert np.abs(got_a - want_a).max() <= 1e-4 * np.abs(want_a).max(), "8-bit gradA parity guard failed"
+    step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    macs = 3 * sum(c * M * K * N for _, c, M, K, N in VGG16_B128)
+    return {"workload": "vgg16_cifar_b128_8bit_lutgemm_fwd_bwd (BASELINE.json configs[3]: 13 conv + 1 fc GEMMs), int16 gradient tables",
+            "steps": steps, "ms_per_step": dt / steps * 1e3, "lut_mac_per_s": macs * steps / dt,
+            "frac_of_lds_gather_roofline": macs * steps / dt / LDS_GATHER_PEAK}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -159,6 +215,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-train-step", action="store_true", help="skip the full training step leg (ResNet-18, batch 512)")
+    ap.add_argument("--no-8bit", action="store_true", help="skip the secondary 8-bit leg (VGG-16 conv shapes, batch 128)")
     ap.add_argument("--layers", action="store_true", help="also print a per-layer table to stderr")
     ap.add_argument("--calib", action="store_true", help="also run three plain 256 MiB device copies (reference for scaling FETCH_SIZE/WRITE_SIZE counters)")
     ap.add_argument("--only", default="", help="comma-separated layer names: restrict the step to them (profiling aid; the JSON line then describes that subset)")
@@ -414,6 +471,12 @@ def main():
                 entry["bounded_by"] = "valu_issue" if entry["valu_issue"]["frac"] > entry["lds_read"]["frac"] else "lds_read"
             kb[kind] = entry
         out["kernel_bounds"] = kb
+
+    # The 8-bit configuration (BASELINE.json configs[3]) as a secondary record, outside the headline's timed region
+    if headline and full and not args.no_8bit and not f32_tables and args.codes == "uniform":
+        del bufs, ws
+        torch.cuda.empty_cache()
+        out["vgg16_b128_8bit"] = eight_bit_step(torch, np, dev, lib, O, stream)
 
     # The full training step (BASELINE.json configs[4]): ResNet-18, batch 512, SGD, outside the headline's timed region
     if headline and full and not args.no_train_step and args.codes == "uniform":
