@@ -27,12 +27,18 @@
 // instead of 4.)  gC is kept in registers in the same rotated order.
 //
 // A workgroup (16 waves, one per CU, all 160 KB of LDS) owns 512 rows and KT = 16 or 32 consecutive k and walks
-// all column tiles.  The chunks go from L2 to LDS by LDS-direct loads, three buffers, requested two chunks ahead
-// by waves 0-7; the rows of gC take the same road (64 KB staging area, requested a column tile ahead by waves
-// 8-15), so no load of the main loop has a register destination and all waiting is explicit.
-// Measured on MI355X: no LDS bank-conflict cycles (4.0 LDS clocks per 128-bit read); about 1.0 us per chunk and
-// CU against 0.5 us of v_fma_mix_f32 issue (72 VALU instructions per wave and chunk, 4.25 clocks each, four waves
-// per SIMD); without the LDS-direct loads of the loop 0.8 us.
+// all column tiles.  The chunks go from L2 to LDS by LDS-direct loads, three buffers, requested two chunks ahead, two
+// wave-wide loads per wave and chunk; the rows of gC take the same road (64 KB staging area, every wave its own rows,
+// requested a column tile ahead).  The only loads with a register destination are the codes of the next tile (one
+// 16-byte load per lane and tile); all waiting is explicit.  The results of a tile leave through LDS as 16-byte
+// stores of whole 128 B lines.
+// Measured on MI355X: no LDS bank-conflict cycles (4.0 LDS clocks per 128-bit read); 0.77-0.80 us per chunk and
+// CU against 0.5 us of v_fma_mix_f32 issue (72 VALU instructions per wave and chunk, four waves per SIMD), plus
+// 4 us per tile.
+//
+// The same kernel serves two more table formats, 16 columns per tile and four chunk buffers each: float32 entries
+// (7-bit float tables; a 128-bit read feeds four v_fma_f32) and the int16 entries of an 8-bit table (256 code rows of
+// 128 B; a conversion in front of every multiply-add; exact for any table, no offset and no fall-back).
 #include <type_traits>
 
 #include "amr_common.h"
