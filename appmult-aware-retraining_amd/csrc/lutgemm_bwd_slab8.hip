@@ -39,7 +39,7 @@ __global__ __launch_bounds__(1024) void lutgemm_gradB_slab8_kernel(
     const int16_t* __restrict__ G, int lut_cols, int M, int K, int N, int m_chunk, float scale, int n_tiles, int k_tiles,
     int splits) {
     constexpr int KT = kB8KT;
-    __shared__ __align__(16) unsigned char smem[2 * 65536];
+    __shared__ __align__(16) unsigned char smem[2 * 65536 + 16 * 1024];   // slabs + 1 KB per wave for the slab build
     const int tid = threadIdx.x;
     const int wave = uniform(tid >> 6);
     const int lane = tid & 63;
@@ -70,23 +70,39 @@ __global__ __launch_bounds__(1024) void lutgemm_gradB_slab8_kernel(
         const int mb = split * m_chunk;
         const int me = min(M, mb + m_chunk);
 
-        {   // The slabs are gathered from the table in global memory (132 KB: it stays in the L2): wave-uniform code a,
-            // lanes = columns; all 64 loads of a thread are issued before the first is stored (one trip to the L2 per
-            // unit instead of one per k: at 2048 rows per unit the gather is a quarter of the unit's time otherwise).
+        {   // The slabs are gathered from the table in global memory (132 KB: it stays in the L2), a table row (code a, 256
+            // entries = 512 B) per wave at a time: the row comes in with two coalesced dword loads per lane, goes to a
+            // 512 B spot of LDS that only this wave uses, and every lane (= column) picks the entries of its four codes of B
+            // from there.  (Gathering from global memory itself, 64 two-byte loads per thread whose lanes scatter over a row,
+            // took 14 us per unit: more than streaming 2048 rows.)
             const int col = lane;
             __syncthreads();
-            int16_t e[KT][16];
+            const unsigned char* gbytes8 = reinterpret_cast<const unsigned char*>(G);
+            uint32_t* stage = reinterpret_cast<uint32_t*>(smem + 2 * 65536 + wave * 1024);
+            unsigned char* s_col = smem + 2 * (8 * ((col & 31) >> 2) + 4 * (col >> 5) + (col & 3));
+#pragma unroll 1
+            for (int half = 0; half < 2; ++half) {             // (eight rows = 16 loads of a thread in flight at a time)
+                uint32_t r0[8], r1[8];
 #pragma unroll
-            for (int kk = 0; kk < KT; ++kk) {
-                const int16_t* t = G + bnext[kk];
+                for (int i = 0; i < 8; ++i) {
+                    const unsigned char* row = gbytes8 + (size_t)(wave + 16 * (8 * half + i)) * (size_t)lut_cols * 2 + 4 * lane;
+                    r0[i] = load_u32_unaligned(row);
+                    r1[i] = load_u32_unaligned(row + 256);
+                }
 #pragma unroll
-                for (int i = 0; i < 16; ++i) e[kk][i] = t[(wave + 16 * i) * lut_cols];
-            }
+                for (int i = 0; i < 8; ++i) {
+                    uint32_t* st = stage + (i & 1) * 128;      // (two spots in turn: the next row is written while this one is read)
+                    st[lane] = r0[i];
+                    st[64 + lane] = r1[i];
+                    // (read back as 16-bit entries through a type that may alias the dwords just written: with plain uint16_t
+                    // the compiler is free to move these reads in front of those writes)
+                    typedef uint16_t __attribute__((may_alias)) u16_alias;
+                    const u16_alias* s16 = reinterpret_cast<const u16_alias*>(st);
+                    const int a = wave + 16 * (8 * half + i);
 #pragma unroll
-            for (int kk = 0; kk < KT; ++kk) {
-                unsigned char* s = smem + (kk >> 1) * 65536 + (kk & 1) * 128 + 2 * (8 * ((col & 31) >> 2) + 4 * (col >> 5) + (col & 3));
-#pragma unroll
-                for (int i = 0; i < 16; ++i) *reinterpret_cast<int16_t*>(s + (wave + 16 * i) * 256) = e[kk][i];
+                    for (int kk = 0; kk < KT; ++kk)
+                        *reinterpret_cast<uint16_t*>(s_col + (kk >> 1) * 65536 + (kk & 1) * 128 + a * 256) = s16[bnext[kk]];
+                }
             }
         }
         __syncthreads();
@@ -224,17 +240,16 @@ __global__ __launch_bounds__(1024) void lutgemm_gradB_slab8_kernel(
 // ------------------------------------------------------------------------------------------ host
 __global__ void reduce_partials_kernel(const float* __restrict__ partial, float* __restrict__ out, size_t count, int splits);
 
-// (measured on MI355X against the direct kernel: 2.7 x faster at 131072 rows, 1.7 x at 8192, 5 % slower at 2048, where the
-// gather of the slabs, 64 loads per thread and unit, is no longer small next to the streaming; `force`: every shape
-// the kernel can do)
+// (measured on MI355X against the direct kernel: 2.9 x faster at 131072 rows, 2.1 x at 8192, 1.45 x at 2048; at 512 rows
+// the build of the slabs outweighs the streaming; `force`: from 1024 rows)
 bool gradB_slab8_applies(const LutGeom& g, int M, int K, int N, const float* gC, bool force) {
     const bool small = (size_t)M * K < (1ull << 31) && (size_t)M * N * 4 < (1ull << 31);
-    return g.bits == 8 && M >= (force ? 2048 : 4096) && (M % kB8RowsPerIter) == 0 && (K & 3) == 0 && (N & 63) == 0 && small &&
+    return g.bits == 8 && M >= (force ? 1024 : 2048) && (M % kB8RowsPerIter) == 0 && (K & 3) == 0 && (N & 63) == 0 && small &&
            ((uintptr_t)gC & 15) == 0;
 }
 
-// M splits: as many as keep every CU busy, at least 2048 rows per workgroup (the slab gather of a unit costs about as much
-// as streaming 700 rows).
+// M splits: as many as keep every CU busy, at least 2048 rows per workgroup (building the slabs of a unit costs about as
+// much as streaming 700 rows).
 int gradB_slab8_splits(int M, int K, int N, int n_cu) {
     const long per_split = (long)(N / 64) * (K / kB8KT);
     long max_s = M / 2048;

@@ -269,9 +269,10 @@ def test_backward_within_tolerance_large_m(lib, oracle, bits, shape):
     check_backward(oracle, gpu_backward(lib, g, A, B, la, lb), g, A, B, la, lb, bits)
 
 
-# 8-bit tables, M % 256 == 0, M >= 2048, K % 4 == 0, N % 64 == 0: gradB on the expanded table held as int16
+# 8-bit tables, M % 256 == 0, M >= 1024 (forced; 2048 by itself), K % 4 == 0, N % 64 == 0: gradB on the expanded table held as int16
 # (one to three column tiles, one to 144 k tiles, one and several M splits)
-SLAB8_SHAPES = [(2048, 4, 64), (4096, 8, 64), (4096, 64, 128), (8192, 36, 192), (2304, 12, 64), (16384, 576, 64), (32768, 20, 64)]
+SLAB8_SHAPES = [(2048, 4, 64), (4096, 8, 64), (4096, 64, 128), (8192, 36, 192), (2304, 12, 64), (16384, 576, 64), (32768, 20, 64),
+                (1024, 16, 128), (1280, 8, 64)]
 
 
 @pytest.mark.parametrize("shape", SLAB8_SHAPES)
