@@ -54,6 +54,11 @@ int gradB_slab8_splits(int M, int K, int N, int n_cu);
 hipError_t launch_gradB_slab8(const float* gC, const uint8_t* A, const uint8_t* B, float* gB, const int16_t* lut,
                               const LutGeom& g, int M, int K, int N, float scale, float* partials, int n_cu,
                               hipStream_t stream);
+bool gradB_slab8f_applies(const LutGeom& g, int M, int K, int N, const float* gC, bool force);
+int gradB_slab8f_splits(int M, int K, int N, int n_cu);
+hipError_t launch_gradB_slab8f(const float* gC, const uint8_t* A, const uint8_t* B, float* gB, const float* lut,
+                               const LutGeom& g, int M, int K, int N, float scale, float* partials, int n_cu,
+                               hipStream_t stream);
 int gradB_slab_splits(int M, int K, int N, int n_cu);
 size_t gradB_slab_colsum_floats(int N);
 hipError_t launch_gradB_slab(const float* gC, const uint8_t* A, const uint8_t* B, float* gB, const int16_t* lut,
@@ -274,8 +279,9 @@ int amr_lut_gemm_forward(const uint8_t* A, const uint8_t* B, uint32_t* C, const 
 // gradient table of gradA]; each part a multiple of 256 bytes.
 static size_t backward_partial_bytes(int M, int K, int N, int n_cu) {
     size_t direct = amr::gradB_workspace_bytes(M, K, N, n_cu);
-    const int s7 = amr::gradB_slab_splits(M, K, N, n_cu), s8 = amr::gradB_slab8_splits(M, K, N, n_cu);
-    const int s = s7 > s8 ? s7 : s8;
+    const int s7 = amr::gradB_slab_splits(M, K, N, n_cu), s8 = amr::gradB_slab8_splits(M, K, N, n_cu),
+              s8f = amr::gradB_slab8f_splits(M, K, N, n_cu);
+    const int s = s7 > s8 ? (s7 > s8f ? s7 : s8f) : (s8 > s8f ? s8 : s8f);
     size_t slab = (s > 1 ? (size_t)s * K * N * sizeof(float) : 0) + amr::gradB_slab_colsum_floats(N) * sizeof(float);
     const size_t b = direct > slab ? direct : slab;
     return (b + 255) & ~(size_t)255;
@@ -534,6 +540,8 @@ int amr_lut_gemm_backward_f32tab(const float* gC, const uint8_t* A, const uint8_
     if (gB) {
         if (slab_b) {
             e = amr::launch_gradB_slab_f32tab(gC, A, B, gB, lut_grad_b, g, M, K, N, scale, flags, partials, n_cu, s);
+        } else if (mode && amr::gradB_slab8f_applies(g, M, K, N, gC, mode == 2)) {
+            e = amr::launch_gradB_slab8f(gC, A, B, gB, lut_grad_b, g, M, K, N, scale, partials, n_cu, s);
         } else {
             e = amr::launch_gradB_f32tab(gC, A, B, gB, lut_grad_b, g, M, K, N, scale, partials, n_cu, s, nullptr);
         }

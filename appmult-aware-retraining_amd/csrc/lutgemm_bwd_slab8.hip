@@ -237,6 +237,196 @@ __global__ __launch_bounds__(1024) void lutgemm_gradB_slab8_kernel(
     }
 }
 
+// ------------------------------------------------------------------------------------------ float32 tables, 8 bits
+// The same for an 8-bit table of float32 entries (the direct kernel needs two passes over every gather there: the table,
+// 258 KB, does not fit the LDS).  The slab keeps the entries themselves, S[kk][a][c] = G[a][B[k0+kk, n0+c]] as float32,
+// 256 B per code and k in the natural column order, two k in 128 KB, and a multiply-add is one v_fma_f32 (no conversion);
+// a 128-bit read brings four entries.  Lane = (row slot rs of 8, column group cg of 8): per row of A it reads columns
+// 4cg..4cg+3 and 32+4cg..32+4cg+3 of both k; odd row slots take the two halves of a 256 B row in the other order (and
+// load their two pieces of gC in that order), so that the 16 lanes the LDS serves together read 64 different banks.
+// Requires K % 4 == 0, N % 64 == 0, M % 256 == 0, gC 16-byte aligned and 32-bit offsets (the launcher checks).
+constexpr int kB8fKT = 2;
+
+__global__ __launch_bounds__(1024) void lutgemm_gradB_slab8f_kernel(
+    const float* __restrict__ gC, const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, float* __restrict__ out,
+    const float* __restrict__ G, int lut_cols, int M, int K, int N, int m_chunk, float scale, int n_tiles, int k_tiles,
+    int splits) {
+    constexpr int KT = kB8fKT;
+    __shared__ __align__(16) unsigned char smem[2 * 65536 + 16 * 1024];   // slabs + 1 KB per wave for the slab build
+    const int tid = threadIdx.x;
+    const int wave = uniform(tid >> 6);
+    const int lane = tid & 63;
+    const int rs = lane >> 3, cg = lane & 7;
+    const uint32_t swap = (uint32_t)(rs & 1);
+    const int total = n_tiles * k_tiles * splits;
+    const int per_xcd = (total + 7) / 8;
+    auto load_b_codes = [&](int logical_u, int (&bc)[KT]) {
+        const int lu = min(logical_u, total - 1);
+        const int kt_u = lu % k_tiles, nt_u = (lu / k_tiles) % n_tiles;
+#pragma unroll
+        for (int kk = 0; kk < KT; ++kk) bc[kk] = (int)B[(size_t)(kt_u * KT + kk) * N + nt_u * 64 + lane];
+    };
+    int bnext[KT];
+    load_b_codes((int)(blockIdx.x % 8) * per_xcd + (int)(blockIdx.x / 8), bnext);
+    for (int slot = (int)(blockIdx.x / 8); slot < per_xcd; slot += (int)(gridDim.x / 8)) {
+        const int logical = (int)(blockIdx.x % 8) * per_xcd + slot;
+        if (logical >= total) break;
+        const int k_tile = logical % k_tiles;
+        const int n_tile = (logical / k_tiles) % n_tiles;
+        const int split = logical / (k_tiles * n_tiles);
+        const int n0 = n_tile * 64;
+        const int k0 = k_tile * KT;
+        const int mb = split * m_chunk;
+        const int me = min(M, mb + m_chunk);
+
+        {   // Slab build: a table row (code a, 256 entries = 1 KB) per wave at a time comes in with four coalesced dword
+            // loads per lane, goes to 1 KB of LDS that only this wave uses, and every lane (= column) picks the entries of
+            // its two codes of B from there.  Eight rows = 32 loads of a thread are in flight at a time.
+            const int col = lane;
+            __syncthreads();
+            float* stage = reinterpret_cast<float*>(smem + 2 * 65536 + wave * 1024);
+            float* s_col = reinterpret_cast<float*>(smem) + col;
+#pragma unroll 1
+            for (int half = 0; half < 2; ++half) {
+                float r[8][4];
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    const float* row = G + (size_t)(wave + 16 * (8 * half + i)) * (size_t)lut_cols + lane;
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) r[i][q] = row[64 * q];
+                }
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) stage[64 * q + lane] = r[i][q];
+                    const int a = wave + 16 * (8 * half + i);
+#pragma unroll
+                    for (int kk = 0; kk < KT; ++kk) s_col[kk * 16384 + a * 64] = stage[bnext[kk]];
+                }
+            }
+        }
+        __syncthreads();
+
+        // address pieces: byte0 = half of the row and column group, byte1 = code (v_perm), byte2 = k (byte 3 of the lane's
+        // constant holds the 1 the second k needs)
+        const uint32_t lo_first = (swap << 7) | (uint32_t)(cg << 4) | 0x01000000u;          // reads 0, 2
+        const uint32_t lo_second = ((swap ^ 1u) << 7) | (uint32_t)(cg << 4) | 0x01000000u;  // reads 1, 3
+        const int ncol = n0 + 4 * cg;
+
+        float acc[4][4];       // acc[j]: k = k0 + j / 2; columns 32 ((j % 2) ^ swap) + 4cg .. + 3
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int c = 0; c < 4; ++c) acc[j][c] = 0.f;
+
+        constexpr int RU = kB8RU;
+        // a2: the codes of the two k in bytes 0 and 1; gf / gs: the lane's first and second piece of the row of gC
+        auto consume = [&](uint32_t a2, const f32x4& gf, const f32x4& gs) __attribute__((always_inline)) {
+            f32x4 s[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const uint32_t sel = (j >= 2 ? 0x0c030400u : 0x0c0c0400u) + ((uint32_t)(j >> 1) << 8);
+                const uint32_t addr = __builtin_amdgcn_perm(a2, (j & 1) ? lo_second : lo_first, sel);
+                s[j] = *reinterpret_cast<const f32x4*>(smem + addr);
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const f32x4& gv = (j & 1) ? gs : gf;
+                acc[j][0] = __builtin_fmaf(gv.x, s[j].x, acc[j][0]);
+                acc[j][1] = __builtin_fmaf(gv.y, s[j].y, acc[j][1]);
+                acc[j][2] = __builtin_fmaf(gv.z, s[j].z, acc[j][2]);
+                acc[j][3] = __builtin_fmaf(gv.w, s[j].w, acc[j][3]);
+            }
+        };
+
+        {
+            const int iters = (me - mb) / kB8RowsPerIter;
+            uint32_t aoff[RU], goff[RU];
+#pragma unroll
+            for (int u = 0; u < RU; ++u) {
+                const uint32_t m = (uint32_t)(mb + 8 * (wave * RU + u) + rs);
+                aoff[u] = m * (uint32_t)K + (uint32_t)k0;
+                goff[u] = (m * (uint32_t)N + (uint32_t)ncol) * 4u;
+            }
+            const uint32_t astep = (uint32_t)kB8RowsPerIter * (uint32_t)K;
+            const uint32_t gstep = (uint32_t)kB8RowsPerIter * (uint32_t)N * 4u;
+            const uint32_t first = 128u * swap, second = 128u * (swap ^ 1u);      // byte offsets of the lane's two pieces of a row of gC
+            const unsigned char* gbytes = reinterpret_cast<const unsigned char*>(gC);
+            uint32_t ca[RU], cb[RU];
+            f32x4 ga0[RU], ga1[RU], gb0[RU], gb1[RU];
+            int next = 0;
+            // (every load batch is issued unconditionally, beyond the end the last rows again: see the int16 kernel)
+            auto load = [&](uint32_t (&c2)[RU], f32x4 (&g0)[RU], f32x4 (&g1)[RU]) {
+#pragma unroll
+                for (int u = 0; u < RU; ++u) {
+                    uint16_t two;
+                    __builtin_memcpy(&two, A + aoff[u], 2);
+                    c2[u] = two;
+                    g0[u] = *reinterpret_cast<const f32x4*>(gbytes + goff[u] + first);
+                    g1[u] = *reinterpret_cast<const f32x4*>(gbytes + goff[u] + second);
+                }
+                ++next;
+                const uint32_t as = next < iters ? astep : 0u, gs = next < iters ? gstep : 0u;
+#pragma unroll
+                for (int u = 0; u < RU; ++u) {
+                    aoff[u] += as;
+                    goff[u] += gs;
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            };
+            if (iters > 0) {
+                load(ca, ga0, ga1);
+                int it = 0;
+                for (; it + 2 <= iters; it += 2) {
+                    load(cb, gb0, gb1);
+#pragma unroll
+                    for (int u = 0; u < RU; ++u) consume(ca[u], ga0[u], ga1[u]);
+                    load(ca, ga0, ga1);
+#pragma unroll
+                    for (int u = 0; u < RU; ++u) consume(cb[u], gb0[u], gb1[u]);
+                }
+                if (it < iters) {
+#pragma unroll
+                    for (int u = 0; u < RU; ++u) consume(ca[u], ga0[u], ga1[u]);
+                }
+            }
+        }
+        load_b_codes(logical + (int)(gridDim.x / 8), bnext);       // (beyond the last unit: the last one again, unused)
+
+        // The 8 row slots x 16 waves meet in LDS, red[wave][rs][k][64 columns] (64 KB): 16 partial sums of 8 terms per
+        // output by all 1024 threads (2 k x 64 columns x 8 parts), then their sum, in a fixed order.
+        __syncthreads();
+        float* red = reinterpret_cast<float*>(smem);
+        {
+            float* r = red + (size_t)((wave * 8 + rs) * KT) * 64 + 4 * cg;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const f32x4 v = {acc[j][0], acc[j][1], acc[j][2], acc[j][3]};
+                *reinterpret_cast<f32x4*>(r + (j >> 1) * 64 + 32 * ((j & 1) ^ (int)swap)) = v;
+            }
+        }
+        __syncthreads();
+        float part = 0.f;
+        {
+            const int o = tid & 127, p = tid >> 7;          // output (k, column) and eighth of the (wave, rs) pairs
+            const float* r = red + (size_t)(p * 16 * KT) * 64 + o;
+#pragma unroll
+            for (int t = 0; t < 16; ++t) part += r[t * KT * 64];
+        }
+        __syncthreads();
+        red[tid] = part;
+        __syncthreads();
+        if (tid < KT * 64) {
+            const int kk = tid >> 6, col = tid & 63;
+            float v = 0.f;
+#pragma unroll
+            for (int p = 0; p < 8; ++p) v += red[128 * p + tid];
+            out[((size_t)split * K + k0 + kk) * N + n0 + col] = v * scale;
+        }
+        // (the barrier at the top of the next unit's slab build keeps these reads ahead of its writes)
+    }
+}
+
 // ------------------------------------------------------------------------------------------ host
 __global__ void reduce_partials_kernel(const float* __restrict__ partial, float* __restrict__ out, size_t count, int splits);
 
@@ -280,6 +470,55 @@ hipError_t launch_gradB_slab8(const float* gC, const uint8_t* A, const uint8_t* 
     const int total = n_tiles * k_tiles * zs;
     const int per_xcd = (total + 7) / 8, cus_per_xcd = n_cu >= 8 ? n_cu / 8 : 1;
     hipLaunchKernelGGL(lutgemm_gradB_slab8_kernel, dim3(8 * (per_xcd < cus_per_xcd ? per_xcd : cus_per_xcd)), dim3(1024), 0,
+                       stream, gC, A, B, out, lut, g.cols, M, K, N, m_chunk, scale, n_tiles, k_tiles, zs);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    if (zs > 1) {
+        const size_t count = (size_t)K * N;
+        hipLaunchKernelGGL(reduce_partials_kernel, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, stream, partials, gB,
+                           count, zs);
+        e = hipGetLastError();
+    }
+    return e;
+}
+
+bool gradB_slab8f_applies(const LutGeom& g, int M, int K, int N, const float* gC, bool force) {
+    const bool small = (size_t)M * K < (1ull << 31) && (size_t)M * N * 4 < (1ull << 31);
+    return g.bits == 8 && M >= (force ? 1024 : 2048) && (M % kB8RowsPerIter) == 0 && (K & 3) == 0 && (N & 63) == 0 && small &&
+           ((uintptr_t)gC & 15) == 0;
+}
+
+// M splits of the float32 variant (two k per unit).
+int gradB_slab8f_splits(int M, int K, int N, int n_cu) {
+    const long per_split = (long)(N / 64) * (K / kB8fKT);
+    long max_s = M / 2048;
+    if (max_s > 64) max_s = 64;
+    if (max_s < 1) max_s = 1;
+    long best_s = 1, best_cost = -1;
+    for (long sp = 1; sp <= max_s; ++sp) {
+        long chunk = (M + sp - 1) / sp;
+        chunk = (chunk + kB8RowsPerIter - 1) / kB8RowsPerIter * kB8RowsPerIter;
+        const long zs = (M + chunk - 1) / chunk;
+        const long rounds = (per_split * zs + n_cu - 1) / n_cu;
+        const long cost = rounds * (chunk + 1400);
+        if (best_cost < 0 || cost < best_cost) { best_cost = cost; best_s = sp; }
+    }
+    return (int)best_s;
+}
+
+// partials: room for gradB_slab8f_splits(...) x K x N floats when that is more than one.
+hipError_t launch_gradB_slab8f(const float* gC, const uint8_t* A, const uint8_t* B, float* gB, const float* lut,
+                               const LutGeom& g, int M, int K, int N, float scale, float* partials, int n_cu,
+                               hipStream_t stream) {
+    const int splits = gradB_slab8f_splits(M, K, N, n_cu);
+    int m_chunk = (M + splits - 1) / splits;
+    m_chunk = (m_chunk + kB8RowsPerIter - 1) / kB8RowsPerIter * kB8RowsPerIter;
+    const int zs = (M + m_chunk - 1) / m_chunk;
+    float* out = zs > 1 ? partials : gB;
+    const int n_tiles = N / 64, k_tiles = K / kB8fKT;
+    const int total = n_tiles * k_tiles * zs;
+    const int per_xcd = (total + 7) / 8, cus_per_xcd = n_cu >= 8 ? n_cu / 8 : 1;
+    hipLaunchKernelGGL(lutgemm_gradB_slab8f_kernel, dim3(8 * (per_xcd < cus_per_xcd ? per_xcd : cus_per_xcd)), dim3(1024), 0,
                        stream, gC, A, B, out, lut, g.cols, M, K, N, m_chunk, scale, n_tiles, k_tiles, zs);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;

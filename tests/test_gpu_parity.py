@@ -477,6 +477,31 @@ F32TAB_SHAPES = [(1, 1, 1), (3, 5, 7), (9, 27, 10), (64, 64, 64), (33, 130, 65),
                  (33011, 128, 32)]
 
 
+# 8-bit float32 tables, M % 256 == 0, M >= 1024 (forced; 2048 by itself), K % 4 == 0, N % 64 == 0: gradB on the expanded float32
+# table (two k per workgroup; one to three column tiles, one and several M splits)
+SLAB8F_SHAPES = [(2048, 4, 64), (4096, 64, 128), (8192, 36, 192), (2304, 12, 64), (1024, 16, 128), (16384, 576, 64), (32768, 20, 64)]
+
+
+@pytest.mark.parametrize("shape", SLAB8F_SHAPES)
+def test_backward_8bit_float_table_slab(lib, oracle, shape):
+    print("backward 8-bit float32 slab", shape, flush=True)
+    rng, A, B, _ = rand_case(hash((shape, "s8f")) % 2**32, *shape, 8)
+    A[0, :] = 255                                                       # the last code of both operands occurs
+    B[:, 0] = 255
+    Ga, Gb = rng.standard_normal((256, 256)) * 40 + 3, rng.standard_normal((256, 256)) * 40 - 5
+    Gb[255, 255], Gb[0, 0], Gb[255, 0], Gb[0, 255] = -1234.5, 4321.25, 0.125, -0.375
+    la, lb = oracle.pack_table(Ga, 8, np.float32), oracle.pack_table(Gb, 8, np.float32)
+    g = (rng.standard_normal((shape[0], shape[2])) + 0.25).astype(np.float32)
+    got = gpu_backward_f32tab(lib, g, A, B, la, lb, 0.5)
+    check_backward(oracle, got, g, A, B, la, lb, 8, factor=np.float32(0.5))
+    old = lib.amr_set_expanded_table_kernels(0)                          # the direct kernels: same sums in another order
+    try:
+        ref = gpu_backward_f32tab(lib, g, A, B, la, lb, 0.5)
+    finally:
+        lib.amr_set_expanded_table_kernels(old)
+    assert np.abs(got[1] - ref[1]).max() <= 1e-5 * np.abs(ref[1]).max()
+
+
 @pytest.mark.parametrize("bits", [7, 8, 6, 4])
 @pytest.mark.parametrize("shape", F32TAB_SHAPES)
 def test_backward_float_tables_within_tolerance(lib, oracle, bits, shape):
