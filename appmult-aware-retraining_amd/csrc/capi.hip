@@ -74,6 +74,10 @@ hipError_t launch_gradB_slab_f32tab(const float* gC, const uint8_t* A, const uin
                                     const LutGeom& g, int M, int K, int N, float scale, uint32_t* flags, float* partials,
                                     int n_cu, hipStream_t stream);
 size_t gradA_slab_f32_workspace_bytes(const LutGeom& g, int M, int K, int N, bool force);
+size_t gradA_slab_f32w_workspace_bytes(const LutGeom& g, int M, int K, int N, bool force);
+hipError_t launch_gradA_slab_f32w(const float* gC, const uint8_t* A, const uint8_t* B, float* gA, const float* lut,
+                                  const LutGeom& g, int M, int K, int N, float scale, int n_cu, uint32_t* flags, void* S,
+                                  int rows_per_image, hipStream_t stream);
 hipError_t launch_gradA_slab_f32tab(const float* gC, const uint8_t* A, const uint8_t* B, float* gA, const float* lut,
                                     const LutGeom& g, int M, int K, int N, float scale, int n_cu, uint32_t* flags, void* S,
                                     int rows_per_image, hipStream_t stream);
@@ -466,9 +470,13 @@ int amr_lut_gemm_backward_static(const float* gC, const uint8_t* A, const uint8_
 // Scratch of the float-table backward pass: [256 B of flags][partial sums of gB][float32 expanded table of gradA].
 static size_t backward_gradA_f32_bytes(int mode, int bits, int M, int K, int N) {
     if (!mode) return 0;
-    amr::LutGeom g;
-    amr::lut_geom_from_bits(bits ? bits : 7, &g);
-    return amr::gradA_slab_f32_workspace_bytes(g, M, K, N, mode == 2);
+    // (bits == 0: a query by shape alone, answered for the larger of the 7-bit and the 8-bit expanded table)
+    amr::LutGeom g7, g8;
+    amr::lut_geom_from_bits(bits && bits < 8 ? bits : 7, &g7);
+    amr::lut_geom_from_bits(8, &g8);
+    const size_t b7 = bits == 8 ? 0 : amr::gradA_slab_f32_workspace_bytes(g7, M, K, N, mode == 2);
+    const size_t b8 = bits == 0 || bits == 8 ? amr::gradA_slab_f32w_workspace_bytes(g8, M, K, N, mode == 2) : 0;
+    return b7 > b8 ? b7 : b8;
 }
 
 size_t amr_lut_gemm_backward_f32tab_workspace_bytes(int M, int K, int N) {
@@ -525,6 +533,8 @@ int amr_lut_gemm_backward_f32tab(const float* gC, const uint8_t* A, const uint8_
     const bool slab_b = mode && gB && amr::bwd_slab_applies(g, M, K, N);
     const bool slab_a = mode && gA && amr::gradA_slab_f32_workspace_bytes(g, M, K, N, mode == 2) != 0 &&
                         ((uintptr_t)gC & 15) == 0;
+    const bool slab_a8 = mode && gA && amr::gradA_slab_f32w_workspace_bytes(g, M, K, N, mode == 2) != 0 &&
+                         ((uintptr_t)gC & 15) == 0;
     if (slab_a || slab_b) {
         e = amr::launch_zero_u32(flags, 64, s);
         if (e != hipSuccess) return hip_fail(e, "scratch header launch");
@@ -533,6 +543,9 @@ int amr_lut_gemm_backward_f32tab(const float* gC, const uint8_t* A, const uint8_
         if (slab_a)
             e = amr::launch_gradA_slab_f32tab(gC, A, B, gA, lut_grad_a, g, M, K, N, scale, n_cu, flags,
                                               reinterpret_cast<unsigned char*>(ws) + 256 + partial_bytes, ga_rows_per_image, s);
+        else if (slab_a8)
+            e = amr::launch_gradA_slab_f32w(gC, A, B, gA, lut_grad_a, g, M, K, N, scale, n_cu, flags,
+                                            reinterpret_cast<unsigned char*>(ws) + 256 + partial_bytes, ga_rows_per_image, s);
         else
             e = amr::launch_gradA_f32tab(gC, A, B, gA, lut_grad_a, g, M, K, N, scale, n_cu, s, nullptr, ga_rows_per_image);
         if (e != hipSuccess) return hip_fail(e, "gradA launch");

@@ -49,9 +49,10 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 
-constexpr int kGaFmtHalf = 0, kGaFmtF32 = 1, kGaFmtI16 = 2;   // how S holds the entries
+constexpr int kGaFmtHalf = 0, kGaFmtF32 = 1, kGaFmtI16 = 2, kGaFmtF32W = 3;   // how S holds the entries (W: float32 entries of an 8-bit table)
 constexpr int kGaCols = 32;                               // columns per tile (half entries; 16 for float32 entries)
 constexpr int kGaColsF32 = 16;
+constexpr int kGaColsF32W = 8;                            // float32 entries of an 8-bit table: 256 code rows of 128 B in a 32 KB chunk
 constexpr int kGaChunkK = 4;
 constexpr int kGaChunkBytes = 128 * kGaChunkK * 2 * kGaCols;   // 32 KB (= 128 codes x 4 k x 16 columns x 4 bytes as well)
 constexpr int kGaBufs = 3;
@@ -198,6 +199,28 @@ __global__ __launch_bounds__(256) void expand_gradA_i16_kernel(const uint8_t* __
     }
 }
 
+// The same for an 8-bit table of float32 entries: S[n_tile][k / 4][a (256 rows)][k % 4][8 columns] float32, 32 KB per chunk.
+// The table (258 KB) does not fit the LDS: the entries are gathered from global memory (it stays in the L2; the expansion
+// is 256 / M of the multiply-adds).  grid (N / 8, ceil(K / 4 / quads_per_wg)), 256 threads.
+__global__ __launch_bounds__(256) void expand_gradA_f32w_kernel(const uint8_t* __restrict__ B, const float* __restrict__ lut, int lut_cols,
+                                                                float* __restrict__ S, int K, int N, int quads_per_wg) {
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    // a wave writes the 128 B rows of two consecutive codes: lane = (code % 2, k % 4, column), one float per lane
+    const int ap = lane >> 5, ks = (lane >> 3) & 3, col = lane & 7;
+    const int n = blockIdx.x * kGaColsF32W + col;
+    for (int pp = 0; pp < quads_per_wg; ++pp) {
+        const int kq = blockIdx.y * quads_per_wg + pp;
+        if (4 * kq >= K) break;
+        const float* p0 = lut + (int)B[(size_t)(4 * kq + ks) * N + n];
+        float* chunk = S + ((size_t)blockIdx.x * (K / 4) + kq) * (kGaChunkBytes / 4) + (lane & 31);
+#pragma unroll 8
+        for (int a2 = wave; a2 < 128; a2 += 4) {
+            const int a = 2 * a2 + ap;
+            chunk[a * 32] = p0[a * lut_cols];
+        }
+    }
+}
+
 // ------------------------------------------------------------------------------------------ consume
 // One 128-bit LDS read of a chunk, issued and NOT waited for.  The address comes out of ONE v_perm_b32:
 // byte 0 = the lane's constant (window and piece), byte 1 = the code (BYTE of codeword; < 128), byte 2 = 1 for
@@ -297,8 +320,9 @@ __global__ __launch_bounds__(kGaWaves * 64) void lutgemm_gradA_slab_kernel(
     const float* __restrict__ gC, const uint8_t* __restrict__ A, const u32x4* __restrict__ S, float* __restrict__ gA,
     uint32_t* __restrict__ flags, int M, int K, int N, float scale, int rows_per_image, int row_blocks, int band_rows_max) {
     __shared__ __align__(16) unsigned char smem[kGaStageBase + kGaStageBytes];
-    constexpr bool F32 = FMT == kGaFmtF32, I16 = FMT == kGaFmtI16, HALF = FMT == kGaFmtHalf;
-    constexpr bool WIDE = !HALF;                           // 4 bytes of S per multiply-add of a row: 16 columns per tile
+    constexpr bool F32 = FMT == kGaFmtF32, I16 = FMT == kGaFmtI16, HALF = FMT == kGaFmtHalf, F32W = FMT == kGaFmtF32W;
+    constexpr bool WIDE = !HALF;                           // 16 (8) columns per tile, four chunk buffers
+    constexpr bool ROWS128 = I16 || F32W;                  // 8-bit tables: 256 code rows of 128 B per chunk
     constexpr int CH = kGaKT / kGaChunkK;                  // chunks per column tile
     // Chunk buffers: three, requested two chunks ahead; with float32 entries the staging area is half the size and a fourth
     // buffer fits: three chunks ahead (the loop is bound by the delivery of the chunks, 36 KB per 32 K multiply-adds).
@@ -306,11 +330,11 @@ __global__ __launch_bounds__(kGaWaves * 64) void lutgemm_gradA_slab_kernel(
     constexpr int DIST = BUFS - 1;                         // chunks between a request and its use
     constexpr int OUT = 2 * (DIST - 1);                    // chunk operations issued after the request of the chunk a step needs
     constexpr int STAGE_BASE = BUFS * kGaChunkBytes;
-    static_assert(STAGE_BASE + kGaRows * (WIDE ? kGaColsF32 : kGaCols) * 4 <= kGaStageBase + kGaStageBytes, "LDS budget");
+    static_assert(STAGE_BASE + kGaRows * (F32W ? kGaColsF32W : WIDE ? kGaColsF32 : kGaCols) * 4 <= kGaStageBase + kGaStageBytes, "LDS budget");
     constexpr int NTU = (CH % BUFS) == 0 ? 1 : BUFS;       // column tiles per unrolled pass: the buffer of a chunk is then static
     static_assert(NTU == 1 || NTU == 3, "the tile loop below unrolls one or three column tiles");
     constexpr int NST = CH / 2;                            // 16-byte stores per lane at the end of a tile
-    constexpr int COLS = WIDE ? kGaColsF32 : kGaCols;      // columns per tile
+    constexpr int COLS = F32W ? kGaColsF32W : WIDE ? kGaColsF32 : kGaCols;      // columns per tile
     constexpr int STAGE_WAVE = kGaRowsPerWave * COLS * 4;  // bytes of gC rows a wave stages per column tile (4 KB / 2 KB)
     constexpr int ROWOPS = STAGE_WAVE / 1024;              // wave-wide 16-byte loads of a row request (4 / 2)
     static_assert(CH >= 4, "the bookkeeping of outstanding loads assumes at least four chunks per column tile");
@@ -361,7 +385,7 @@ __global__ __launch_bounds__(kGaWaves * 64) void lutgemm_gradA_slab_kernel(
     uint32_t lane_const[4];
 #pragma unroll
     for (int s = 0; s < 4; ++s)
-        lane_const[s] = I16 ? ((uint32_t)(c << 6) | (uint32_t)(((quad + s) & 1) << 5) | 0x03020100u)
+        lane_const[s] = ROWS128 ? ((uint32_t)(c << 6) | (uint32_t)(((quad + s) & 1) << 5) | 0x03020100u)
                             : ((uint32_t)(c << 6) | (uint32_t)(((quad + s) & 3) << 4) | 0x01000000u);
 
     typedef const __attribute__((address_space(1))) void* gptr_t;
@@ -438,7 +462,7 @@ __global__ __launch_bounds__(kGaWaves * 64) void lutgemm_gradA_slab_kernel(
 #pragma unroll
             for (int w = 0; w < CH / 4; ++w) high_bits |= codes_next[r][w];
         // (a masked code 128 of a 7-bit operand; an 8-bit table has a row for every value of a byte)
-        if (!I16 && __builtin_amdgcn_ballot_w64((high_bits & 0x80808080u) != 0) != 0) {
+        if (!ROWS128 && __builtin_amdgcn_ballot_w64((high_bits & 0x80808080u) != 0) != 0) {
             if (lane == 0) atomicOr(&flags[2], 1u);
         }
     };
@@ -488,7 +512,7 @@ __global__ __launch_bounds__(kGaWaves * 64) void lutgemm_gradA_slab_kernel(
     auto pair_fma = [&](auto kc_tag, auto s_tag, const u32x4& d0, const u32x4& d1) {
         constexpr int KC = decltype(kc_tag)::value;
         float s0 = acc[0][KC], s1 = acc[1][KC];
-        if constexpr (F32) {
+        if constexpr (F32 || F32W) {
             constexpr int S4 = 4 * decltype(s_tag)::value;
             const f32x4 f0 = __builtin_bit_cast(f32x4, d0), f1 = __builtin_bit_cast(f32x4, d1);
 #pragma unroll
@@ -557,25 +581,29 @@ __global__ __launch_bounds__(kGaWaves * 64) void lutgemm_gradA_slab_kernel(
                 const uint32_t gbase = (uint32_t)(STAGE_BASE + wave * STAGE_WAVE + quad * (COLS * 4));
 #pragma unroll
                 for (int r = 0; r < 2; ++r) {
-                    u32x4 t[4];
+                    constexpr int NP = COLS / 4;             // 16-byte pieces of a row of the tile
+                    u32x4 t[NP];
 #pragma unroll
-                    for (int s4 = 0; s4 < 4; ++s4) {
+                    for (int s4 = 0; s4 < NP; ++s4) {
                         // the rows of gC in the order the entries are read in: 16-byte pieces (quad + s) % 4 of the window
-                        // (int16 entries: 32-byte pieces (quad + s) % 2, i.e. floats 8 ((quad + s4 / 2) % 2) + 4 (s4 % 2) ...)
+                        // (int16 entries: 32-byte pieces (quad + s) % 2, i.e. floats 8 ((quad + s4 / 2) % 2) + 4 (s4 % 2) ...;
+                        // float32 entries of an 8-bit table: 16-byte pieces (quad + s) % 2)
                         const uint32_t ga = gbase + (I16 ? (uint32_t)((((quad + (s4 >> 1)) & 1) << 5) | ((s4 & 1) << 4))
-                                                         : (uint32_t)(((quad + s4) & 3) << 4));
+                                                         : (uint32_t)(((quad + s4) & (NP - 1)) << 4));
+                        // (the second row of the lane is 16 rows further on)
                         if (r == 0) asm volatile("ds_read_b128 %0, %1" : "=&v"(t[s4]) : "v"(ga) : "memory");
-                        else asm volatile("ds_read_b128 %0, %1 offset:1024" : "=&v"(t[s4]) : "v"(ga) : "memory");
+                        else asm volatile("ds_read_b128 %0, %1 offset:%2" : "=&v"(t[s4]) : "v"(ga), "n"(16 * COLS * 4) : "memory");
                     }
-                    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(t[0]), "+v"(t[1]), "+v"(t[2]), "+v"(t[3]) : : "memory");
+                    if constexpr (NP == 4) asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(t[0]), "+v"(t[1]), "+v"(t[2]), "+v"(t[3]) : : "memory");
+                    else asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(t[0]), "+v"(t[1]) : : "memory");
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) {
+                    for (int i = 0; i < NP; ++i) {
                         const f32x4 v = __builtin_bit_cast(f32x4, t[i]);
                         g[r][4 * i] = v.x; g[r][4 * i + 1] = v.y; g[r][4 * i + 2] = v.z; g[r][4 * i + 3] = v.w;
                     }
                 }
             }
-            if constexpr (I16) {
+            if constexpr (ROWS128) {
                 ga_read_i16<KC & 3, BUF>(d[0], codes[0][KC >> 2], lane_const[0]);
                 ga_read_i16<KC & 3, BUF>(d[1], codes[1][KC >> 2], lane_const[0]);
                 ga_read_i16<KC & 3, BUF>(d[2], codes[0][KC >> 2], lane_const[1]);
@@ -889,6 +917,43 @@ hipError_t launch_gradA_slab_i16(const float* gC, const uint8_t* A, const uint8_
                            rows_per_image, row_blocks, band_rows);
     else
         hipLaunchKernelGGL((lutgemm_gradA_slab_kernel<16, kGaFmtI16>), grid, block, 0, stream, gC, A, S4, gA, flags, M, K, N, scale,
+                           rows_per_image, row_blocks, band_rows);
+    return hipGetLastError();
+}
+
+// ------------------------------------------------------------------------------------------ 8-bit float32 tables
+// Bytes of the float32 expanded table of an 8-bit float table, or 0 when that kernel does not apply: K*N*1 KB, four times the
+// half table of a 7-bit one, and every block of 512 rows streams all of it: from 8192 rows on (measured on MI355X
+// against the two-band direct kernel; VGG-16 conv3_x: 604 MB).
+size_t gradA_slab_f32w_workspace_bytes(const LutGeom& g, int M, int K, int N, bool force) {
+    if (!force && (M < 8192 || (double)M * K * N < 2e8)) return 0;
+    if (g.bits != 8 || M < 512 || (N % kGaColsF32W) != 0 || (K % 16) != 0 || (size_t)M * K >= (1ull << 31)) return 0;
+    return (size_t)(N / kGaColsF32W) * (K / kGaChunkK) * kGaChunkBytes;
+}
+
+// No flag is read or written (8-bit operands have no masked code).
+hipError_t launch_gradA_slab_f32w(const float* gC, const uint8_t* A, const uint8_t* B, float* gA, const float* lut,
+                                  const LutGeom& g, int M, int K, int N, float scale, int n_cu, uint32_t* flags, void* S,
+                                  int rows_per_image, hipStream_t stream) {
+    if (((uintptr_t)gC & 15) != 0) return hipErrorInvalidValue;   // callers check: rows of gC are fetched 16 bytes at a time
+    const int qpw = 4;
+    hipLaunchKernelGGL(expand_gradA_f32w_kernel, dim3(N / kGaColsF32W, (K / 4 + qpw - 1) / qpw), dim3(256), 0, stream, B, lut, g.cols,
+                       reinterpret_cast<float*>(S), K, N, qpw);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    const u32x4* S4 = reinterpret_cast<const u32x4*>(S);
+    const dim3 block(kGaWaves * 64);
+    const int row_blocks = (M + kGaRows - 1) / kGaRows;
+    const int band_rows = 16;
+    const int kt = ((K % 32) == 0 && row_blocks * (K / 32) >= n_cu) ? 32 : 16;
+    const int tiles = row_blocks * (K / kt);
+    const int per_xcd = (tiles + 7) / 8, cus_per_xcd = n_cu >= 8 ? n_cu / 8 : 1;
+    const dim3 grid(8 * (per_xcd < cus_per_xcd ? per_xcd : cus_per_xcd));
+    if (kt == 32)
+        hipLaunchKernelGGL((lutgemm_gradA_slab_kernel<32, kGaFmtF32W>), grid, block, 0, stream, gC, A, S4, gA, flags, M, K, N, scale,
+                           rows_per_image, row_blocks, band_rows);
+    else
+        hipLaunchKernelGGL((lutgemm_gradA_slab_kernel<16, kGaFmtF32W>), grid, block, 0, stream, gC, A, S4, gA, flags, M, K, N, scale,
                            rows_per_image, row_blocks, band_rows);
     return hipGetLastError();
 }
