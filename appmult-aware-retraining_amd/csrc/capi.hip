@@ -26,6 +26,11 @@ hipError_t launch_gradA(const float* gC, const uint8_t* A, const uint8_t* B, flo
                         const uint32_t* gate = nullptr, int rows_per_image = 0);
 size_t gradA_slab_workspace_bytes(const LutGeom& g, int M, int K, int N, bool force);
 size_t gradA_slab_i16_workspace_bytes(const LutGeom& g, int M, int K, int N, bool force);
+bool gradA_rows8_applies(const LutGeom& g, int M, int K, int N, const float* gC, bool force);
+size_t gradA_rows8_workspace_bytes(const LutGeom& g, int M, int K, int N, bool force);
+hipError_t launch_gradA_rows8(const float* gC, const uint8_t* A, const uint8_t* B, float* gA, const int16_t* lut,
+                              const LutGeom& g, int M, int K, int N, float scale, int n_cu, void* P, size_t p_bytes,
+                              int rows_per_image, hipStream_t stream);
 hipError_t launch_gradA_slab_i16(const float* gC, const uint8_t* A, const uint8_t* B, float* gA, const int16_t* lut,
                                  const LutGeom& g, int M, int K, int N, float scale, int n_cu, uint32_t* flags, void* S,
                                  int rows_per_image, hipStream_t stream);
@@ -299,7 +304,12 @@ static size_t backward_gradA_bytes(int mode, int bits, int M, int K, int N) {
     amr::lut_geom_from_bits(bits && bits < 8 ? bits : 7, &g7);
     amr::lut_geom_from_bits(8, &g8);
     const size_t b7 = bits == 8 ? 0 : amr::gradA_slab_workspace_bytes(g7, M, K, N, mode == 2);
-    const size_t b8 = bits == 0 || bits == 8 ? amr::gradA_slab_i16_workspace_bytes(g8, M, K, N, mode == 2) : 0;
+    size_t b8 = 0;
+    if (bits == 0 || bits == 8) {
+        // (a layer takes one of the two: partial results of the kernel with the table in LDS, or the expanded table)
+        const size_t rows8 = amr::gradA_rows8_workspace_bytes(g8, M, K, N, mode == 2);
+        b8 = rows8 ? rows8 : amr::gradA_slab_i16_workspace_bytes(g8, M, K, N, mode == 2);
+    }
     return b7 > b8 ? b7 : b8;
 }
 
@@ -402,7 +412,9 @@ static int backward_impl(const float* gC, const uint8_t* A, const uint8_t* B, fl
     const bool slab = mode && amr::bwd_slab_applies(g, M, K, N);
     const bool slab_a = mode && allow_slab_a && gA && amr::gradA_slab_workspace_bytes(g, M, K, N, mode == 2) != 0 && ((uintptr_t)gC & 15) == 0;
     // (8-bit tables: the expanded table holds the int16 entries, nothing to decide in a header)
-    const bool slab_a8 = mode && allow_slab_a && gA && amr::gradA_slab_i16_workspace_bytes(g, M, K, N, mode == 2) != 0 && ((uintptr_t)gC & 15) == 0;
+    // (or, for layers of a few thousand rows, none at all: the table is expanded in LDS and the scratch holds partial results)
+    const bool rows_a8 = mode && allow_slab_a && gA && amr::gradA_rows8_applies(g, M, K, N, gC, mode == 2);
+    const bool slab_a8 = !rows_a8 && mode && allow_slab_a && gA && amr::gradA_slab_i16_workspace_bytes(g, M, K, N, mode == 2) != 0 && ((uintptr_t)gC & 15) == 0;
     if ((slab && gB) || slab_a) {
         // flags cleared, offsets of the half-precision tables decided from the tables' extremes
         e = amr::launch_bwd_header(slab_a ? lut_grad_a : nullptr, (slab && gB) ? lut_grad_b : nullptr, g, flags, s);
@@ -425,6 +437,9 @@ static int backward_impl(const float* gC, const uint8_t* A, const uint8_t* B, fl
         if (slab_a)
             e = amr::launch_gradA_slab(gC, A, B, gA, lut_grad_a, g, M, K, N, scale, n_cu, flags,
                                        reinterpret_cast<unsigned char*>(ws) + 256 + partial_bytes, ga_rows_per_image, s);
+        else if (rows_a8)
+            e = amr::launch_gradA_rows8(gC, A, B, gA, lut_grad_a, g, M, K, N, scale, n_cu,
+                                        reinterpret_cast<unsigned char*>(ws) + 256 + partial_bytes, gradA_bytes, ga_rows_per_image, s);
         else if (slab_a8)
             e = amr::launch_gradA_slab_i16(gC, A, B, gA, lut_grad_a, g, M, K, N, scale, n_cu, flags,
                                            reinterpret_cast<unsigned char*>(ws) + 256 + partial_bytes, ga_rows_per_image, s);

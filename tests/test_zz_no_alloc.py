@@ -82,6 +82,10 @@ def test_static_scratch_backward_two_calls_in_a_row(lib, oracle):
     both_ways(lib, oracle, 3, 1500, 40, 70, 8)
     both_ways(lib, oracle, 4, 4096, 48, 64, 6, rows_per_image=256, lo=-2048, hi=2049)
     both_ways(lib, oracle, 5, 300, 27, 10, 7)
+    # 8-bit table, 2048 rows: gradA with the table expanded in LDS (scratch: partial results per column tile), gradB on the
+    # int16 slab; row-major and image-major gA
+    both_ways(lib, oracle, 7, 2048, 16, 128, 8, lo=-32768, hi=32768)
+    both_ways(lib, oracle, 8, 2048, 12, 64, 8, rows_per_image=256, lo=-32768, hi=32768)
 
 
 def test_static_scratch_backward_steps_aside_or_rejects_beyond_its_size(lib, oracle):
