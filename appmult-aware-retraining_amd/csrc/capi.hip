@@ -80,6 +80,11 @@ hipError_t launch_gradB_slab_f32tab(const float* gC, const uint8_t* A, const uin
                                     int n_cu, hipStream_t stream);
 size_t gradA_slab_f32_workspace_bytes(const LutGeom& g, int M, int K, int N, bool force);
 size_t gradA_slab_f32w_workspace_bytes(const LutGeom& g, int M, int K, int N, bool force);
+bool gradA_rows8f_applies(const LutGeom& g, int M, int K, int N, const float* gC, bool force);
+size_t gradA_rows8f_workspace_bytes(const LutGeom& g, int M, int K, int N, bool force);
+hipError_t launch_gradA_rows8f(const float* gC, const uint8_t* A, const uint8_t* B, float* gA, const float* lut,
+                               const LutGeom& g, int M, int K, int N, float scale, int n_cu, void* P, size_t p_bytes,
+                               int rows_per_image, hipStream_t stream);
 hipError_t launch_gradA_slab_f32w(const float* gC, const uint8_t* A, const uint8_t* B, float* gA, const float* lut,
                                   const LutGeom& g, int M, int K, int N, float scale, int n_cu, uint32_t* flags, void* S,
                                   int rows_per_image, hipStream_t stream);
@@ -490,7 +495,11 @@ static size_t backward_gradA_f32_bytes(int mode, int bits, int M, int K, int N) 
     amr::lut_geom_from_bits(bits && bits < 8 ? bits : 7, &g7);
     amr::lut_geom_from_bits(8, &g8);
     const size_t b7 = bits == 8 ? 0 : amr::gradA_slab_f32_workspace_bytes(g7, M, K, N, mode == 2);
-    const size_t b8 = bits == 0 || bits == 8 ? amr::gradA_slab_f32w_workspace_bytes(g8, M, K, N, mode == 2) : 0;
+    size_t b8 = 0;
+    if (bits == 0 || bits == 8) {
+        const size_t rows8 = amr::gradA_rows8f_workspace_bytes(g8, M, K, N, mode == 2);
+        b8 = rows8 ? rows8 : amr::gradA_slab_f32w_workspace_bytes(g8, M, K, N, mode == 2);
+    }
     return b7 > b8 ? b7 : b8;
 }
 
@@ -548,7 +557,8 @@ int amr_lut_gemm_backward_f32tab(const float* gC, const uint8_t* A, const uint8_
     const bool slab_b = mode && gB && amr::bwd_slab_applies(g, M, K, N);
     const bool slab_a = mode && gA && amr::gradA_slab_f32_workspace_bytes(g, M, K, N, mode == 2) != 0 &&
                         ((uintptr_t)gC & 15) == 0;
-    const bool slab_a8 = mode && gA && amr::gradA_slab_f32w_workspace_bytes(g, M, K, N, mode == 2) != 0 &&
+    const bool rows_a8 = mode && gA && amr::gradA_rows8f_applies(g, M, K, N, gC, mode == 2);
+    const bool slab_a8 = !rows_a8 && mode && gA && amr::gradA_slab_f32w_workspace_bytes(g, M, K, N, mode == 2) != 0 &&
                          ((uintptr_t)gC & 15) == 0;
     if (slab_a || slab_b) {
         e = amr::launch_zero_u32(flags, 64, s);
@@ -558,6 +568,10 @@ int amr_lut_gemm_backward_f32tab(const float* gC, const uint8_t* A, const uint8_
         if (slab_a)
             e = amr::launch_gradA_slab_f32tab(gC, A, B, gA, lut_grad_a, g, M, K, N, scale, n_cu, flags,
                                               reinterpret_cast<unsigned char*>(ws) + 256 + partial_bytes, ga_rows_per_image, s);
+        else if (rows_a8)
+            e = amr::launch_gradA_rows8f(gC, A, B, gA, lut_grad_a, g, M, K, N, scale, n_cu,
+                                         reinterpret_cast<unsigned char*>(ws) + 256 + partial_bytes,
+                                         backward_gradA_f32_bytes(mode, g.bits, M, K, N), ga_rows_per_image, s);
         else if (slab_a8)
             e = amr::launch_gradA_slab_f32w(gC, A, B, gA, lut_grad_a, g, M, K, N, scale, n_cu, flags,
                                             reinterpret_cast<unsigned char*>(ws) + 256 + partial_bytes, ga_rows_per_image, s);

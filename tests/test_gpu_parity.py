@@ -500,6 +500,11 @@ def test_backward_8bit_float_table_slab(lib, oracle, shape):
     finally:
         lib.amr_set_expanded_table_kernels(old)
     assert np.abs(got[1] - ref[1]).max() <= 1e-5 * np.abs(ref[1]).max()
+    # image-major gA (1024 to 8191 rows: gradA with the table expanded in LDS and a kernel of its own that writes gA)
+    M, K, N = shape
+    L = 256
+    gat = gpu_backward_f32tab(lib, g, A, B, la, lb, 0.5, rows_per_image=L)[0]
+    assert np.array_equal(gat.reshape(M // L, K, L).transpose(0, 2, 1).reshape(M, K), got[0])
 
 
 @pytest.mark.parametrize("bits", [7, 8, 6, 4])
