@@ -1,4 +1,4 @@
-// Backward LUT-GEMM, gradient of A, 8-bit int16 tables, for layers of a few thousand rows on gfx950.
+// Backward LUT-GEMM, gradient of A, 8-bit tables (int16 or float32), for layers of 2048 to 8192 rows on gfx950.
 //
 // Same result (to fp32 summation order) as lutgemm_gradA_kernel and as the reference's
 // ApproxGemmBackwardKernelForGA (self_ops/src/approx_gemm_backward.cu:44-267):
@@ -381,13 +381,14 @@ __global__ __launch_bounds__(1024) void lutgemm_gradA_rows8f_kernel(
 }
 
 // ------------------------------------------------------------------------------------------ host
-// (measured on MI355X: between 2048 and 8192 rows this kernel beats both the direct kernel and the expanded-table kernel,
-// whose table, written to memory, weighs most there; from 8192 rows on the expanded-table kernel is faster; `force`
-// lowers the floor to 1024 rows and keeps the ceiling)
+// (measured on MI355X: from 2048 to 8192 rows this kernel beats both the direct kernel and the expanded-table kernel,
+// whose table, written to memory, weighs most there -- 1.2 x at 2048 rows, level at 8192 with int16 tables, 1.35 x at 8192
+// with float32 ones; at 32768 rows the expanded-table kernel is 1.2 x faster; `force` lowers the floor to 1024 rows and
+// keeps the ceiling)
 bool gradA_rows8_applies(const LutGeom& g, int M, int K, int N, const float* gC, bool force) {
     const bool small = (size_t)M * K < (1ull << 31) && (size_t)M * N * 4 < (1ull << 31) &&
                        (size_t)(N / 64) * (size_t)M * (size_t)K < (1ull << 32);
-    return g.bits == 8 && M >= (force ? 1024 : 2048) && M < 8192 && (M % kR8RowsPerIter) == 0 && (K & 3) == 0 && (N & 63) == 0 &&
+    return g.bits == 8 && M >= (force ? 1024 : 2048) && M < 16384 && (M % kR8RowsPerIter) == 0 && (K & 3) == 0 && (N & 63) == 0 &&
            small && ((uintptr_t)gC & 15) == 0;
 }
 

@@ -923,10 +923,10 @@ hipError_t launch_gradA_slab_i16(const float* gC, const uint8_t* A, const uint8_
 
 // ------------------------------------------------------------------------------------------ 8-bit float32 tables
 // Bytes of the float32 expanded table of an 8-bit float table, or 0 when that kernel does not apply: K*N*1 KB, four times the
-// half table of a 7-bit one, and every block of 512 rows streams all of it: from 8192 rows on (measured on MI355X
-// against the two-band direct kernel; VGG-16 conv3_x: 604 MB).
+// half table of a 7-bit one, and every block of 512 rows streams all of it: from 16384 rows on (measured on MI355X:
+// 3 x the two-band direct kernel at 32768 rows; up to 8192 rows the kernel that expands the table in LDS is faster).
 size_t gradA_slab_f32w_workspace_bytes(const LutGeom& g, int M, int K, int N, bool force) {
-    if (!force && (M < 8192 || (double)M * K * N < 2e8)) return 0;
+    if (!force && (M < 16384 || (double)M * K * N < 2e8)) return 0;
     if (g.bits != 8 || M < 512 || (N % kGaColsF32W) != 0 || (K % 16) != 0 || (size_t)M * K >= (1ull << 31)) return 0;
     return (size_t)(N / kGaColsF32W) * (K / kGaChunkK) * kGaChunkBytes;
 }
