@@ -349,6 +349,23 @@ hipError_t launch_gradA(const float* gC, const uint8_t* A, const uint8_t* B, flo
     constexpr int KT = 16;
     const bool vec = ((N & 3) == 0) && (((uintptr_t)gC & 15) == 0);   // rows of gC are read 16 bytes at a time
     const int ktiles = (K + KT - 1) / KT;
+    if (g.bits == 8 && M <= 1024) {
+        // One block of rows: the k tiles are the only workgroups, one per CU at a time, and a launch lasts (rounds of n_cu
+        // workgroups) x (k per tile).  4608 k in tiles of 16 are 288 workgroups, two rounds on 256 CUs with the second one
+        // nearly empty; in tiles of 20 they are 231 workgroups, one round (measured: 0.36 -> 0.2 ms at 512 x 4608 x 512).
+        auto cost = [&](int kt) { return ((long)((K + kt - 1) / kt) + n_cu - 1) / n_cu * kt; };
+        int kt = 16;
+        if (cost(20) < cost(kt)) kt = 20;
+        if (cost(24) < cost(kt)) kt = 24;
+#define AMR_GA8_CASE(t)                                                                                                  \
+    if (kt == t)                                                                                                         \
+        return vec ? launch_gradA_t<t, 1, 16, true>(gC, A, B, gA, lut, g, M, K, N, scale, stream, gate, rows_per_image)  \
+                   : launch_gradA_t<t, 1, 16, false>(gC, A, B, gA, lut, g, M, K, N, scale, stream, gate, rows_per_image);
+        AMR_GA8_CASE(20)
+        AMR_GA8_CASE(24)
+        AMR_GA8_CASE(16)
+#undef AMR_GA8_CASE
+    }
     if (g.bits == 8) {
         // one 1024-thread workgroup per CU; two rows per lane (half the scalar work per gather) unless one row per lane
         // needs fewer (rounds of n_cu workgroups) x (rows per workgroup)

@@ -319,7 +319,25 @@ hipError_t launch_gradA_f32tab(const float* gC, const uint8_t* A, const uint8_t*
     f32tab_bands(g, &rows_pp, &passes);
     const bool vec = ((N & 3) == 0) && (((uintptr_t)gC & 15) == 0);   // rows of gC are read 16 bytes at a time
     const int ktiles = (K + KT - 1) / KT;
-    if (passes > 1 || (size_t)rows_pp * g.cols * 4 > 80 * 1024) {
+    const bool wide = passes > 1 || (size_t)rows_pp * g.cols * 4 > 80 * 1024;
+    if (wide && M <= 1024) {
+        // One block of rows: the k tiles are the only workgroups, one per CU at a time, and a launch lasts (rounds of n_cu
+        // workgroups) x (k per tile): 16, 20 or 24 k per tile, whichever makes that smallest (4608 k: 231 tiles of 20 are one
+        // round on 256 CUs, 288 tiles of 16 two).
+        auto cost = [&](int kt) { return ((long)((K + kt - 1) / kt) + n_cu - 1) / n_cu * kt; };
+        int kt = 16;
+        if (cost(20) < cost(kt)) kt = 20;
+        if (cost(24) < cost(kt)) kt = 24;
+#define AMR_GA8F_CASE(t)                                                                                                                            \
+    if (kt == t)                                                                                                                                    \
+        return vec ? launch_gradA_f32tab_t<t, 1, 16, true, true>(gC, A, B, gA, lut, g, rows_pp, passes, M, K, N, scale, stream, gate, rows_per_image)  \
+                   : launch_gradA_f32tab_t<t, 1, 16, false, true>(gC, A, B, gA, lut, g, rows_pp, passes, M, K, N, scale, stream, gate, rows_per_image);
+        AMR_GA8F_CASE(20)
+        AMR_GA8F_CASE(24)
+        AMR_GA8F_CASE(16)
+#undef AMR_GA8F_CASE
+    }
+    if (wide) {
         // one 1024-thread workgroup per CU shares the staged band; two rows per lane (half the scalar work per gather) unless
         // one row per lane needs fewer (rounds of n_cu workgroups) x (rows per workgroup)
         const long cost2 = (((long)ktiles * ((M + 2047) / 2048) + n_cu - 1) / n_cu) * 2048;

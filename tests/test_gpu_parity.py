@@ -30,6 +30,7 @@ def lib():
     L.amr_lut_gemm_forward_workspace_bytes.argtypes = [i64, i, i, i]
     L.amr_lut_gemm_forward_workspace_bytes.restype = sz
     L.amr_lut_gemm_backward.argtypes = [vp, vp, vp, vp, vp, vp, vp, i64, i, i, i, vp, sz, vp]
+    L.amr_lut_gemm_backward_ex.argtypes = [vp, vp, vp, vp, vp, vp, vp, i64, i, i, i, i, vp, sz, vp]
     L.amr_lut_gemm_backward_f32tab.argtypes = [vp, vp, vp, vp, vp, vp, vp, i64, ctypes.c_float, i, i, i, i, vp, sz, vp]
     L.amr_lut_gemm_backward_f32tab_workspace_bytes.argtypes = [i, i, i]
     L.amr_lut_gemm_backward_f32tab_workspace_bytes.restype = sz
@@ -319,6 +320,41 @@ def test_backward_8bit_int16_expanded_table_gradA(lib, oracle, shape):
     for off in (0, 1):                                                  # gA aligned to 16 and to 4 bytes
         again = gpu_backward(lib, g, A, B, la, lb, ga_offset_floats=off)
         assert np.array_equal(again[0], got[0])
+
+
+# 8-bit tables, at most 1024 rows: the k tiles of the direct gradA kernel are its only workgroups, so their depth (16, 20 or 24 k)
+# follows the count that fills the CUs in the fewest rounds (256 CUs: K = 4612 -> 20, K = 6142 -> 24); K % 4 != 0 takes the
+# scalar stores, a last tile sticking out of K the clamped loads
+@pytest.mark.parametrize("kind", ["i16", "f32"])
+@pytest.mark.parametrize("shape,L", [((300, 4612, 40), 4), ((130, 6142, 24), 10), ((1024, 4608, 16), 64), ((512, 9220, 8), 0)])
+def test_backward_8bit_one_row_block_deep_k_tiles(lib, oracle, kind, shape, L):
+    print("backward 8-bit, one row block, deep k tiles", kind, shape, flush=True)
+    M, K, N = shape
+    rng, A, B, _ = rand_case(hash((shape, "deep")) % 2**32, *shape, 8)
+    g = rng.standard_normal((M, N)).astype(np.float32)
+    if kind == "f32":
+        la = oracle.pack_table(rng.standard_normal((256, 256)) * 40 + 3, 8, np.float32)
+        lb = oracle.pack_table(rng.standard_normal((256, 256)) * 40 - 5, 8, np.float32)
+        got = gpu_backward_f32tab(lib, g, A, B, la, lb, 0.5)
+        check_backward(oracle, got, g, A, B, la, lb, 8, factor=np.float32(0.5))
+        if L:
+            gat = gpu_backward_f32tab(lib, g, A, B, la, lb, 0.5, rows_per_image=L)[0]
+            assert np.array_equal(gat.reshape(M // L, K, L).transpose(0, 2, 1).reshape(M, K), got[0])
+        return
+    la = oracle.pack_table(rng.integers(-32768, 32768, (256, 256)), 8, np.int16)
+    lb = oracle.pack_table(rng.integers(-32768, 32768, (256, 256)), 8, np.int16)
+    got = gpu_backward(lib, g, A, B, la, lb)
+    check_backward(oracle, got, g, A, B, la, lb, 8)
+    if L:
+        gd, a, b, ta, tb = dev(g), dev(A), dev(B), dev(la), dev(lb)
+        gat = torch.full((M * K,), float("nan"), device="cuda")
+        need = lib.amr_lut_gemm_backward_workspace_bytes(M, K, N)
+        ws = torch.empty(max(need, 1), dtype=torch.uint8, device="cuda")
+        rc = lib.amr_lut_gemm_backward_ex(gd.data_ptr(), a.data_ptr(), b.data_ptr(), gat.data_ptr(), None, ta.data_ptr(), tb.data_ptr(),
+                                          ta.numel(), M, K, N, L, ws.data_ptr(), need, None)
+        assert rc == 0, lib.amr_last_error()
+        torch.cuda.synchronize()
+        assert np.array_equal(gat.cpu().numpy().reshape(M // L, K, L).transpose(0, 2, 1).reshape(M, K), got[0])
 
 
 def test_backward_large_m_masked_codes(lib, oracle):
