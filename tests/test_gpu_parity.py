@@ -972,12 +972,12 @@ def test_two_host_threads_on_two_streams_equal_the_serial_results(lib, oracle):
     import threading
     print("two threads, two streams", flush=True)
     problems = []
-    for seed, (M, K, N) in ((41, (8192, 576, 64)), (42, (4096, 1152, 128))):
-        rng, A, B, T = rand_case(seed, M, K, N, 7)
-        T = oracle.synth_lut(7, 64, rng)
+    for seed, (M, K, N), bits in ((41, (8192, 576, 64), 7), (42, (4096, 1152, 128), 8)):       # (one 7-bit and one 8-bit problem)
+        rng, A, B, T = rand_case(seed, M, K, N, bits)
+        T = oracle.synth_lut(bits, 64, rng)
         Gx, Gy = oracle.gen_bp_lut(T, 8)
-        t = dict(M=M, K=K, N=N, a=dev(A), b=dev(B), l=dev(oracle.pack_table(T, 7, np.uint16)), ta=dev(oracle.pack_table(Gx, 7, np.int16)),
-                 tb=dev(oracle.pack_table(Gy, 7, np.int16)), g=dev(rng.standard_normal((M, N)).astype(np.float32)),
+        t = dict(M=M, K=K, N=N, a=dev(A), b=dev(B), l=dev(oracle.pack_table(T, bits, np.uint16)), ta=dev(oracle.pack_table(Gx, bits, np.int16)),
+                 tb=dev(oracle.pack_table(Gy, bits, np.int16)), g=dev(rng.standard_normal((M, N)).astype(np.float32)),
                  c=torch.zeros((M, N), dtype=torch.int32, device="cuda"), ga=torch.zeros((M, K), device="cuda"),
                  gb=torch.zeros((K, N), device="cuda"), stream=torch.cuda.Stream())
         problems.append(t)
