@@ -1,7 +1,7 @@
 // Backward LUT-GEMM, gradient of A, 8-bit tables (int16 or float32), for layers of 2048 to 8192 rows on gfx950.
 //
 // Same result (to fp32 summation order) as lutgemm_gradA_kernel and as the reference's
-// ApproxGemmBackwardKernelForGA (self_ops/src/approx_gemm_backward.cu:44-267):
+// ApproxGemmBackwardKernelForGA (self_ops/src/approx_gemm_backward.cu:21-258):
 //       gA[m,k] = 1/16 * sum_n gC[m,n] * G[A[m,k]][B[k,n]]
 //
 // The expanded-table kernel of lutgemm_gradA_slab.hip writes K*N*512 B of table to memory whatever M is: with 2048 rows

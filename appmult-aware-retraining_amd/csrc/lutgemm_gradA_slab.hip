@@ -2,7 +2,7 @@
 // narrower).
 //
 // Same result (to fp32 summation order) as lutgemm_gradA_kernel and as the reference's
-// ApproxGemmBackwardKernelForGA (self_ops/src/approx_gemm_backward.cu:44-267):
+// ApproxGemmBackwardKernelForGA (self_ops/src/approx_gemm_backward.cu:21-258):
 //       gA[m,k] = 1/16 * sum_n gC[m,n] * G[A[m,k]][B[k,n]]
 //
 //   step 1  expand_gradA_kernel:  S[k][a][n] = half(G[a][B[k,n]] - offset) for every code a
