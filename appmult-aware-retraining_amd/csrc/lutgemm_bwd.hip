@@ -118,6 +118,17 @@ __global__ void reduce_partials_kernel(const float* __restrict__ partial, float*
     out[i] = s;
 }
 
+// The same behind a gated kernel: nothing is written unless *gate != 0.
+__global__ void reduce_partials_gated_kernel(const float* __restrict__ partial, float* __restrict__ out, size_t count, int splits,
+                                             const uint32_t* __restrict__ gate) {
+    if (*gate == 0u) return;
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= count) return;
+    float s = partial[i];
+    for (int p = 1; p < splits; ++p) s += partial[(size_t)p * count + i];
+    out[i] = s;
+}
+
 // ------------------------------------------------------------------------------------------ gradA
 // VEC: N % 4 == 0 and gC 16-byte aligned, so the per-lane rows of gC are read 16 bytes at a time; vec_store: K % 4 == 0
 // and gA 16-byte aligned, so the per-lane rows of gA are written 16 bytes at a time (a lane owns a row, so every scalar access would
@@ -321,8 +332,12 @@ hipError_t launch_gradB(const float* gC, const uint8_t* A, const uint8_t* B, flo
     if (e != hipSuccess) return e;
     if (zs > 1) {
         const size_t count = (size_t)K * N;
-        hipLaunchKernelGGL(reduce_partials_kernel, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, stream,
-                           reinterpret_cast<const float*>(workspace), gB, count, zs);
+        if (gate)
+            hipLaunchKernelGGL(reduce_partials_gated_kernel, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, stream,
+                               reinterpret_cast<const float*>(workspace), gB, count, zs, gate);
+        else
+            hipLaunchKernelGGL(reduce_partials_kernel, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, stream,
+                               reinterpret_cast<const float*>(workspace), gB, count, zs);
         e = hipGetLastError();
     }
     return e;
@@ -388,10 +403,13 @@ hipError_t launch_gradA(const float* gC, const uint8_t* A, const uint8_t* B, flo
 }
 
 // Direct kernel queued behind the expanded-table kernel; it runs only when *gate != 0 (an operand
-// held a masked code) and then overwrites the whole result (no M split: no scratch).
+// held a masked code) and then overwrites the whole result.  workspace: the scratch for partial sums (the kernel in front
+// has finished with it), so that the sum over M is split as in an ungated launch: one workgroup per k tile adding all
+// rows in turn would be slow and, over tens of thousands of rows, lose digits; nullptr: no split.
 hipError_t launch_gradB_gated(const float* gC, const uint8_t* A, const uint8_t* B, float* gB, const int16_t* lut,
-                              const LutGeom& g, int M, int K, int N, float scale, const uint32_t* gate, hipStream_t stream) {
-    return launch_gradB(gC, A, B, gB, lut, g, M, K, N, scale, nullptr, 0, stream, gate);
+                              const LutGeom& g, int M, int K, int N, float scale, const uint32_t* gate, void* workspace,
+                              int n_cu, hipStream_t stream) {
+    return launch_gradB(gC, A, B, gB, lut, g, M, K, N, scale, workspace, n_cu, stream, gate);
 }
 
 }  // namespace amr

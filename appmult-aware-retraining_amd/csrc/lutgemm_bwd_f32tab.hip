@@ -23,6 +23,8 @@
 namespace amr {
 
 __global__ void reduce_partials_kernel(const float* __restrict__ partial, float* __restrict__ out, size_t count, int splits);
+__global__ void reduce_partials_gated_kernel(const float* __restrict__ partial, float* __restrict__ out, size_t count, int splits,
+                                             const uint32_t* __restrict__ gate);
 
 // ------------------------------------------------------------------------------------------ gradB
 // Lanes own columns n, the uniform operand is a = A[m,k]; band p holds table rows a in [p*rows_pp, (p+1)*rows_pp).
@@ -288,8 +290,12 @@ hipError_t launch_gradB_f32tab(const float* gC, const uint8_t* A, const uint8_t*
     if (e != hipSuccess) return e;
     if (zs > 1) {
         const size_t count = (size_t)K * N;
-        hipLaunchKernelGGL(reduce_partials_kernel, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, stream,
-                           reinterpret_cast<const float*>(workspace), gB, count, zs);
+        if (gate)      // (behind a gated kernel: nothing may be written unless the gate is raised)
+            hipLaunchKernelGGL(reduce_partials_gated_kernel, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, stream,
+                               reinterpret_cast<const float*>(workspace), gB, count, zs, gate);
+        else
+            hipLaunchKernelGGL(reduce_partials_kernel, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, stream,
+                               reinterpret_cast<const float*>(workspace), gB, count, zs);
         e = hipGetLastError();
     }
     return e;

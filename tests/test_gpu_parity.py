@@ -78,6 +78,12 @@ def gpu_backward(lib, g, A, B, la, lb, own_workspace=True, ga_offset_floats=0):
     return ga.cpu().numpy(), gb.cpu().numpy()
 
 
+def seed_of(*key):
+    """Seed of a test case from its parameters: the same in every process (hash() of a str is not)."""
+    import zlib
+    return zlib.crc32(repr(key).encode())
+
+
 def rand_case(seed, M, K, N, bits):
     rng = np.random.default_rng(seed)
     n = 1 << bits
@@ -95,7 +101,7 @@ FWD_SHAPES = [(1, 1, 1), (3, 5, 7), (9, 27, 10), (64, 64, 64), (33, 130, 65), (1
 @pytest.mark.parametrize("shape", FWD_SHAPES)
 def test_forward_bit_exact_random_tables(lib, oracle, bits, shape):
     print("forward", bits, shape, flush=True)
-    _, A, B, T = rand_case(hash((bits, shape)) % 2**32, *shape, bits)
+    _, A, B, T = rand_case(seed_of(bits, shape), *shape, bits)
     flat = oracle.pack_table(T, bits, np.uint16)
     assert (gpu_forward(lib, A, B, flat) == oracle.forward_c(A, B, flat, bits)).all()
 
@@ -112,7 +118,7 @@ BIG_M_SHAPES = [(2048, 512, 64), (2081, 515, 65), (2081, 516, 65), (3000, 27, 10
 @pytest.mark.parametrize("shape", BIG_M_SHAPES)
 def test_forward_bit_exact_large_m(lib, oracle, bits, shape):
     print("forward large M", bits, shape, flush=True)
-    _, A, B, T = rand_case(hash((bits, shape, "L")) % 2**32, *shape, bits)
+    _, A, B, T = rand_case(seed_of(bits, shape, "L"), *shape, bits)
     flat = oracle.pack_table(T, bits, np.uint16)
     assert (gpu_forward(lib, A, B, flat) == oracle.forward_c(A, B, flat, bits)).all()
 
@@ -196,7 +202,7 @@ def test_forward_golden_shipped_tables(lib, oracle, golden_dir):
 def test_forward_float_output_is_the_converted_integer_sum(lib, oracle, bits, shape, big):
     print("forward f32", bits, shape, big, flush=True)
     M, K, N = shape
-    rng, A, B, _ = rand_case(hash((bits, shape, "f32")) % 2**32, M, K, N, bits)
+    rng, A, B, _ = rand_case(seed_of(bits, shape, "f32"), M, K, N, bits)
     n = 1 << bits
     T = rng.integers(60000, 65536, (n, n)) if big else rng.integers(0, 300, (n, n))      # big: sums pass 2^24 (and 2^32 for long K)
     flat = oracle.pack_table(T, bits, np.uint16)
@@ -245,7 +251,7 @@ BWD_SHAPES = [(1, 1, 1), (3, 5, 7), (9, 27, 10), (64, 64, 64), (33, 130, 65), (6
 @pytest.mark.parametrize("shape", BWD_SHAPES)
 def test_backward_within_tolerance_random_tables(lib, oracle, bits, shape):
     print("backward", bits, shape, flush=True)
-    rng, A, B, _ = rand_case(hash((bits, shape, "b")) % 2**32, *shape, bits)
+    rng, A, B, _ = rand_case(seed_of(bits, shape, "b"), *shape, bits)
     n = 1 << bits
     la = oracle.pack_table(rng.integers(-32768, 32768, (n, n)), bits, np.int16)
     lb = oracle.pack_table(rng.integers(-32768, 32768, (n, n)), bits, np.int16)
@@ -262,7 +268,7 @@ BWD_BIG_M_SHAPES = [(4096, 8, 64), (4100, 27, 10), (5000, 130, 65), (4096, 64, 3
 @pytest.mark.parametrize("shape", BWD_BIG_M_SHAPES)
 def test_backward_within_tolerance_large_m(lib, oracle, bits, shape):
     print("backward large M", bits, shape, flush=True)
-    rng, A, B, _ = rand_case(hash((bits, shape, "bL")) % 2**32, *shape, bits)
+    rng, A, B, _ = rand_case(seed_of(bits, shape, "bL"), *shape, bits)
     n = 1 << bits
     la = oracle.pack_table(rng.integers(-32768, 32768, (n, n)), bits, np.int16)
     lb = oracle.pack_table(rng.integers(-32768, 32768, (n, n)), bits, np.int16)
@@ -279,7 +285,7 @@ SLAB8_SHAPES = [(2048, 4, 64), (4096, 8, 64), (4096, 64, 128), (8192, 36, 192), 
 @pytest.mark.parametrize("shape", SLAB8_SHAPES)
 def test_backward_8bit_int16_slab(lib, oracle, shape):
     print("backward 8-bit int16 slab", shape, flush=True)
-    rng, A, B, _ = rand_case(hash((shape, "s8")) % 2**32, *shape, 8)
+    rng, A, B, _ = rand_case(seed_of(shape, "s8"), *shape, 8)
     A[0, :] = 255                                                       # the last code of both operands occurs
     B[:, 0] = 255
     la = oracle.pack_table(rng.integers(-32768, 32768, (256, 256)), 8, np.int16)
@@ -306,7 +312,7 @@ SLAB8_GA_SHAPES = [(4096, 16, 16), (4096, 64, 64), (4100, 32, 48), (9001, 64, 16
 @pytest.mark.parametrize("shape", SLAB8_GA_SHAPES)
 def test_backward_8bit_int16_expanded_table_gradA(lib, oracle, shape):
     print("backward 8-bit int16 expanded table, gradA", shape, flush=True)
-    rng, A, B, _ = rand_case(hash((shape, "a8")) % 2**32, *shape, 8)
+    rng, A, B, _ = rand_case(seed_of(shape, "a8"), *shape, 8)
     A[0, :] = 255                                                       # the last code of both operands occurs
     A[-1, :] = 128
     B[:, 0] = 255
@@ -330,7 +336,7 @@ def test_backward_8bit_int16_expanded_table_gradA(lib, oracle, shape):
 def test_backward_8bit_one_row_block_deep_k_tiles(lib, oracle, kind, shape, L):
     print("backward 8-bit, one row block, deep k tiles", kind, shape, flush=True)
     M, K, N = shape
-    rng, A, B, _ = rand_case(hash((shape, "deep")) % 2**32, *shape, 8)
+    rng, A, B, _ = rand_case(seed_of(shape, "deep"), *shape, 8)
     g = rng.standard_normal((M, N)).astype(np.float32)
     if kind == "f32":
         la = oracle.pack_table(rng.standard_normal((256, 256)) * 40 + 3, 8, np.float32)
@@ -372,6 +378,31 @@ def test_backward_large_m_masked_codes(lib, oracle):
     check_backward(oracle, gpu_backward(lib, g, A, B, la, lb), g, A, B, la, lb, 7)
 
 
+@pytest.mark.parametrize("kind", ["i16", "f32"])
+def test_backward_masked_code_fallback_splits_the_sum_over_rows(lib, oracle, kind):
+    """A masked code sends the whole result to the direct kernels queued behind the expanded-table ones.  Their sum over
+    tens of thousands of rows is split like an ungated launch's (over the scratch the kernel in front has finished with): the
+    result stays within 3e-6 of the float64 one norm-wise, where one accumulator per output walking all rows comes to 1e-5
+    on gradients with a non-zero mean."""
+    print("masked-code fallback at 32768 rows", kind, flush=True)
+    M, K, N = 32768, 128, 64
+    rng, A, B, _ = rand_case(seed_of("mask", kind), M, K, N, 7)
+    A[-1, :] = 128
+    A[::7, 3] = 128
+    Ga, Gb = rng.integers(-1024, 3073, (128, 128)), rng.integers(-1024, 3073, (128, 128))
+    g = (rng.standard_normal((M, N)) + 0.25).astype(np.float32)
+    if kind == "i16":
+        la, lb = oracle.pack_table(Ga, 7, np.int16), oracle.pack_table(Gb, 7, np.int16)
+        got = gpu_backward(lib, g, A, B, la, lb)
+    else:
+        la, lb = oracle.pack_table(Ga, 7, np.float32), oracle.pack_table(Gb, 7, np.float32)
+        got = gpu_backward_f32tab(lib, g, A, B, la, lb, 1.0 / 16)
+    check_backward(oracle, got, g, A, B, la, lb, 7)
+    a64, b64 = oracle.backward_c_f64(g, A, B, la, lb, 7, factor=1.0 / 16)
+    for x, r in ((got[0], a64), (got[1], b64)):
+        assert np.abs(x - r).max() <= 3e-6 * np.abs(r).max()
+
+
 # K % 8 == 0, N % 64 == 0, M % 128 == 0 and M >= 4096: gradB runs on the expanded table held as halves (entries - 1024)
 # (N % 32 == 0, K % 16 == 0 and M >= 2048: gradA runs on its own expanded table, 16, 32 or 48 k per workgroup and one to
 # six column tiles, also with a ragged last row block)
@@ -386,7 +417,7 @@ HALF_SLAB_SHAPES = [(4096, 8, 64), (4224, 24, 128), (8192, 64, 64), (16384, 16, 
 @pytest.mark.parametrize("shape", HALF_SLAB_SHAPES)
 def test_backward_half_slab_tables_inside_the_exact_range(lib, oracle, bits, shape, low):
     print("backward half slab", bits, shape, low, flush=True)
-    rng, A, B, _ = rand_case(hash((bits, shape, "h")) % 2**32, *shape, bits)
+    rng, A, B, _ = rand_case(seed_of(bits, shape, "h"), *shape, bits)
     n = 1 << bits
     # [-1024, 3072]: halves of the entries - 1024; [-2048, 2048]: gradA holds the entries themselves
     Ga, Gb = rng.integers(low, low + 4097, (n, n)), rng.integers(-1024, 3073, (n, n))
@@ -430,7 +461,7 @@ def test_backward_half_tables_whose_offset_would_swamp_small_entries(lib, oracle
     for every output, for both gradients, whether the library stores such a table with an offset or steps aside."""
     print("backward, offset against small entries", shape, small, big, flush=True)
     M, K, N = shape
-    rng, A, B, _ = rand_case(hash((shape, small, big)) % 2**32, M, K, N, 7)
+    rng, A, B, _ = rand_case(seed_of(shape, small, big), M, K, N, 7)
     Ga, Gb = rng.integers(small[0], small[1], (128, 128)), rng.integers(small[0], small[1], (128, 128))
     Ga[77, 13] = big
     Gb[13, 77] = big
@@ -446,7 +477,7 @@ def test_backward_ga_aligned_to_four_bytes_only(lib, oracle, shape):
     """gA one, two and three floats into a 16-byte-aligned allocation: the expanded-table kernel stores 16 bytes at a time
     where it can and must not where it cannot."""
     print("backward, gA not 16-byte aligned", shape, flush=True)
-    rng, A, B, _ = rand_case(hash((shape, "u")) % 2**32, *shape, 7)
+    rng, A, B, _ = rand_case(seed_of(shape, "u"), *shape, 7)
     la = oracle.pack_table(rng.integers(-1024, 3073, (128, 128)), 7, np.int16)
     lb = oracle.pack_table(rng.integers(-1024, 3073, (128, 128)), 7, np.int16)
     g = rng.standard_normal((shape[0], shape[2])).astype(np.float32)
@@ -521,7 +552,7 @@ SLAB8F_SHAPES = [(2048, 4, 64), (4096, 64, 128), (8192, 36, 192), (2304, 12, 64)
 @pytest.mark.parametrize("shape", SLAB8F_SHAPES)
 def test_backward_8bit_float_table_slab(lib, oracle, shape):
     print("backward 8-bit float32 slab", shape, flush=True)
-    rng, A, B, _ = rand_case(hash((shape, "s8f")) % 2**32, *shape, 8)
+    rng, A, B, _ = rand_case(seed_of(shape, "s8f"), *shape, 8)
     A[0, :] = 255                                                       # the last code of both operands occurs
     B[:, 0] = 255
     Ga, Gb = rng.standard_normal((256, 256)) * 40 + 3, rng.standard_normal((256, 256)) * 40 - 5
@@ -547,7 +578,7 @@ def test_backward_8bit_float_table_slab(lib, oracle, shape):
 @pytest.mark.parametrize("shape", F32TAB_SHAPES)
 def test_backward_float_tables_within_tolerance(lib, oracle, bits, shape):
     print("backward float tables", bits, shape, flush=True)
-    rng, A, B, _ = rand_case(hash((bits, shape, "f")) % 2**32, *shape, bits)
+    rng, A, B, _ = rand_case(seed_of(bits, shape, "f"), *shape, bits)
     n = 1 << bits
     la = oracle.pack_table(rng.standard_normal((n, n)) * 40 + 3, bits, np.float32)
     lb = oracle.pack_table(rng.standard_normal((n, n)) * 40 - 5, bits, np.float32)
@@ -757,7 +788,7 @@ def test_direct_kernels_at_large_m(lib, oracle, shape):
     """Mode 0: the direct gather kernels on shapes that otherwise take the expanded-table kernels."""
     print("direct kernels, large M", shape, flush=True)
     M, K, N = shape
-    rng, A, B, T = rand_case(hash((shape, "d")) % 2**32, M, K, N, 7)
+    rng, A, B, T = rand_case(seed_of(shape, "d"), M, K, N, 7)
     flat = oracle.pack_table(T, 7, np.uint16)
     la = oracle.pack_table(rng.integers(-1024, 3073, (128, 128)), 7, np.int16)
     lb = oracle.pack_table(rng.integers(-1024, 3073, (128, 128)), 7, np.int16)
