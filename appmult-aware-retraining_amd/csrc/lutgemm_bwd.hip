@@ -118,15 +118,17 @@ __global__ void reduce_partials_kernel(const float* __restrict__ partial, float*
     out[i] = s;
 }
 
-// The same behind a gated kernel: nothing is written unless *gate != 0.
+// The same behind a gated kernel: nothing is written unless *gate != 0.  Launched with a small grid whatever `count` is
+// (the usual case is a raised gate nowhere: the launch should cost no more than a launch); the threads stride over the outputs.
 __global__ void reduce_partials_gated_kernel(const float* __restrict__ partial, float* __restrict__ out, size_t count, int splits,
                                              const uint32_t* __restrict__ gate) {
     if (*gate == 0u) return;
-    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= count) return;
-    float s = partial[i];
-    for (int p = 1; p < splits; ++p) s += partial[(size_t)p * count + i];
-    out[i] = s;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < count; i += stride) {
+        float s = partial[i];
+        for (int p = 1; p < splits; ++p) s += partial[(size_t)p * count + i];
+        out[i] = s;
+    }
 }
 
 // ------------------------------------------------------------------------------------------ gradA
@@ -333,7 +335,7 @@ hipError_t launch_gradB(const float* gC, const uint8_t* A, const uint8_t* B, flo
     if (zs > 1) {
         const size_t count = (size_t)K * N;
         if (gate)
-            hipLaunchKernelGGL(reduce_partials_gated_kernel, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, stream,
+            hipLaunchKernelGGL(reduce_partials_gated_kernel, dim3((unsigned)std::min<size_t>((count + 255) / 256, 256)), dim3(256), 0, stream,
                                reinterpret_cast<const float*>(workspace), gB, count, zs, gate);
         else
             hipLaunchKernelGGL(reduce_partials_kernel, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, stream,

@@ -291,7 +291,7 @@ hipError_t launch_gradB_f32tab(const float* gC, const uint8_t* A, const uint8_t*
     if (zs > 1) {
         const size_t count = (size_t)K * N;
         if (gate)      // (behind a gated kernel: nothing may be written unless the gate is raised)
-            hipLaunchKernelGGL(reduce_partials_gated_kernel, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, stream,
+            hipLaunchKernelGGL(reduce_partials_gated_kernel, dim3((unsigned)std::min<size_t>((count + 255) / 256, 256)), dim3(256), 0, stream,
                                reinterpret_cast<const float*>(workspace), gB, count, zs, gate);
         else
             hipLaunchKernelGGL(reduce_partials_kernel, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, stream,
