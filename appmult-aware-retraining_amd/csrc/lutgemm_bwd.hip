@@ -86,10 +86,16 @@ __global__ __launch_bounds__(WAVES * 64) void lutgemm_gradB_kernel(
             __builtin_amdgcn_sched_barrier(0);
         }
     };
+    // Sums of blocks of kBlockTrips * 2 * RPL rows are added to a second set of accumulators: a chunk of tens of thousands of
+    // rows (the gated launch behind an expanded-table kernel has no M split) then loses no more digits than a split sum.
+    constexpr int kBlockTrips = 8;
+    float tot[KT];
+#pragma unroll
+    for (int kk = 0; kk < KT; ++kk) tot[kk] = 0.f;
     {
         uint32_t a4x, a4y;
         float gx[RPL], gy[RPL];
-        int m = mb;
+        int m = mb, trips = 0;
         if (m < me) load_rows(m, a4x, gx);
         while (m < me) {
             if (m + RPL < me) load_rows(m + RPL, a4y, gy);
@@ -99,13 +105,21 @@ __global__ __launch_bounds__(WAVES * 64) void lutgemm_gradB_kernel(
             if (m + RPL < me) load_rows(m + RPL, a4x, gx);
             consume_rows(a4y, gy);
             m += RPL;
+            if (++trips == kBlockTrips) {     // (wave-uniform)
+                trips = 0;
+#pragma unroll
+                for (int kk = 0; kk < KT; ++kk) {
+                    tot[kk] += acc[kk];
+                    acc[kk] = 0.f;
+                }
+            }
         }
     }
     if (n < N) {
         float* o = out + (size_t)blockIdx.z * K * N;
 #pragma unroll
         for (int kk = 0; kk < KT; ++kk)
-            if (k0 + kk < K) o[(size_t)(k0 + kk) * N + n] = acc[kk] * scale;
+            if (k0 + kk < K) o[(size_t)(k0 + kk) * N + n] = (tot[kk] + acc[kk]) * scale;
     }
 }
 
@@ -116,19 +130,6 @@ __global__ void reduce_partials_kernel(const float* __restrict__ partial, float*
     float s = partial[i];
     for (int p = 1; p < splits; ++p) s += partial[(size_t)p * count + i];
     out[i] = s;
-}
-
-// The same behind a gated kernel: nothing is written unless *gate != 0.  Launched with a small grid whatever `count` is
-// (the usual case is a raised gate nowhere: the launch should cost no more than a launch); the threads stride over the outputs.
-__global__ void reduce_partials_gated_kernel(const float* __restrict__ partial, float* __restrict__ out, size_t count, int splits,
-                                             const uint32_t* __restrict__ gate) {
-    if (*gate == 0u) return;
-    const size_t stride = (size_t)gridDim.x * blockDim.x;
-    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < count; i += stride) {
-        float s = partial[i];
-        for (int p = 1; p < splits; ++p) s += partial[(size_t)p * count + i];
-        out[i] = s;
-    }
 }
 
 // ------------------------------------------------------------------------------------------ gradA
@@ -334,12 +335,8 @@ hipError_t launch_gradB(const float* gC, const uint8_t* A, const uint8_t* B, flo
     if (e != hipSuccess) return e;
     if (zs > 1) {
         const size_t count = (size_t)K * N;
-        if (gate)
-            hipLaunchKernelGGL(reduce_partials_gated_kernel, dim3((unsigned)std::min<size_t>((count + 255) / 256, 256)), dim3(256), 0, stream,
-                               reinterpret_cast<const float*>(workspace), gB, count, zs, gate);
-        else
-            hipLaunchKernelGGL(reduce_partials_kernel, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, stream,
-                               reinterpret_cast<const float*>(workspace), gB, count, zs);
+        hipLaunchKernelGGL(reduce_partials_kernel, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, stream,
+                           reinterpret_cast<const float*>(workspace), gB, count, zs);
         e = hipGetLastError();
     }
     return e;
@@ -405,13 +402,11 @@ hipError_t launch_gradA(const float* gC, const uint8_t* A, const uint8_t* B, flo
 }
 
 // Direct kernel queued behind the expanded-table kernel; it runs only when *gate != 0 (an operand
-// held a masked code) and then overwrites the whole result.  workspace: the scratch for partial sums (the kernel in front
-// has finished with it), so that the sum over M is split as in an ungated launch: one workgroup per k tile adding all
-// rows in turn would be slow and, over tens of thousands of rows, lose digits; nullptr: no split.
+// held a masked code) and then overwrites the whole result (no M split: no scratch and no second launch; the kernel adds
+// its rows in blocks, so the long sum keeps its digits).
 hipError_t launch_gradB_gated(const float* gC, const uint8_t* A, const uint8_t* B, float* gB, const int16_t* lut,
-                              const LutGeom& g, int M, int K, int N, float scale, const uint32_t* gate, void* workspace,
-                              int n_cu, hipStream_t stream) {
-    return launch_gradB(gC, A, B, gB, lut, g, M, K, N, scale, workspace, n_cu, stream, gate);
+                              const LutGeom& g, int M, int K, int N, float scale, const uint32_t* gate, hipStream_t stream) {
+    return launch_gradB(gC, A, B, gB, lut, g, M, K, N, scale, nullptr, 0, stream, gate);
 }
 
 }  // namespace amr

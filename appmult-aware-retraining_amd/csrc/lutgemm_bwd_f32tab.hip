@@ -23,8 +23,6 @@
 namespace amr {
 
 __global__ void reduce_partials_kernel(const float* __restrict__ partial, float* __restrict__ out, size_t count, int splits);
-__global__ void reduce_partials_gated_kernel(const float* __restrict__ partial, float* __restrict__ out, size_t count, int splits,
-                                             const uint32_t* __restrict__ gate);
 
 // ------------------------------------------------------------------------------------------ gradB
 // Lanes own columns n, the uniform operand is a = A[m,k]; band p holds table rows a in [p*rows_pp, (p+1)*rows_pp).
@@ -53,9 +51,12 @@ __global__ __launch_bounds__(WAVES * 64) void lutgemm_gradB_f32tab_kernel(
     uint32_t boff[KT];
 #pragma unroll
     for (int kk = 0; kk < KT; ++kk) boff[kk] = 4u * (uint32_t)B[(size_t)min(k0 + kk, K - 1) * N + nc];
-    float acc[KT];
+    // Sums of blocks of kBlockTrips * RPL rows are added to a second set of accumulators: a chunk of tens of thousands of rows
+    // (the gated launch behind an expanded-table kernel has no M split) then loses no more digits than a split sum.
+    constexpr int kBlockTrips = 16;
+    float acc[KT], tot[KT];
 #pragma unroll
-    for (int kk = 0; kk < KT; ++kk) acc[kk] = 0.f;
+    for (int kk = 0; kk < KT; ++kk) acc[kk] = tot[kk] = 0.f;
 
     for (int p = 0; p < passes; ++p) {
         const int lo = p * rows_pp;
@@ -71,6 +72,7 @@ __global__ __launch_bounds__(WAVES * 64) void lutgemm_gradB_f32tab_kernel(
         }
         __syncthreads();
         if (!active) continue;
+        int trips = 0;
         for (int m = mb; m < me; m += RPL) {
             const int r = min(m + lrow, me - 1);
             const uint32_t a4 = load_codes4_clamped(A + (size_t)r * K, k0 + 4 * ldw, K);
@@ -95,13 +97,21 @@ __global__ __launch_bounds__(WAVES * 64) void lutgemm_gradB_f32tab_kernel(
                 for (int kk = 0; kk < KT; ++kk) acc[kk] = __builtin_fmaf(t[kk], g[i], acc[kk]);
                 __builtin_amdgcn_sched_barrier(0);
             }
+            if (++trips == kBlockTrips) {     // (wave-uniform) a block of rows is done: its sums join the totals
+                trips = 0;
+#pragma unroll
+                for (int kk = 0; kk < KT; ++kk) {
+                    tot[kk] += acc[kk];
+                    acc[kk] = 0.f;
+                }
+            }
         }
     }
     if (active && n < N) {
         float* o = out + (size_t)blockIdx.z * K * N;
 #pragma unroll
         for (int kk = 0; kk < KT; ++kk)
-            if (k0 + kk < K) o[(size_t)(k0 + kk) * N + n] = acc[kk] * scale;
+            if (k0 + kk < K) o[(size_t)(k0 + kk) * N + n] = (tot[kk] + acc[kk]) * scale;
     }
 }
 
@@ -290,12 +300,8 @@ hipError_t launch_gradB_f32tab(const float* gC, const uint8_t* A, const uint8_t*
     if (e != hipSuccess) return e;
     if (zs > 1) {
         const size_t count = (size_t)K * N;
-        if (gate)      // (behind a gated kernel: nothing may be written unless the gate is raised)
-            hipLaunchKernelGGL(reduce_partials_gated_kernel, dim3((unsigned)std::min<size_t>((count + 255) / 256, 256)), dim3(256), 0, stream,
-                               reinterpret_cast<const float*>(workspace), gB, count, zs, gate);
-        else
-            hipLaunchKernelGGL(reduce_partials_kernel, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, stream,
-                               reinterpret_cast<const float*>(workspace), gB, count, zs);
+        hipLaunchKernelGGL(reduce_partials_kernel, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, stream,
+                           reinterpret_cast<const float*>(workspace), gB, count, zs);
         e = hipGetLastError();
     }
     return e;

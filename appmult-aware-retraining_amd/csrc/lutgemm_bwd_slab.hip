@@ -592,8 +592,7 @@ hipError_t launch_bwd_header(const int16_t* lut_a, const int16_t* lut_b, const L
 
 // ------------------------------------------------------------------------------------------ host
 hipError_t launch_gradB_gated(const float* gC, const uint8_t* A, const uint8_t* B, float* gB, const int16_t* lut,
-                              const LutGeom& g, int M, int K, int N, float scale, const uint32_t* gate, void* workspace,
-                              int n_cu, hipStream_t stream);
+                              const LutGeom& g, int M, int K, int N, float scale, const uint32_t* gate, hipStream_t stream);
 __global__ void reduce_partials_kernel(const float* __restrict__ partial, float* __restrict__ out, size_t count, int splits);
 
 // Floats of scratch the half-slab kernel keeps in front of its partial results (column sums of gC per M split).
@@ -663,7 +662,7 @@ hipError_t launch_gradB_slab(const float* gC, const uint8_t* A, const uint8_t* B
                            zs > 1 ? (const float*)part16 : (const float*)nullptr, gB, colsum, flags, K, N, zs, scale);
         e16 = hipGetLastError();
         if (e16 != hipSuccess) return e16;
-        return launch_gradB_gated(gC, A, B, gB, lut, g, M, K, N, scale, flags + 1, partials, n_cu, stream);
+        return launch_gradB_gated(gC, A, B, gB, lut, g, M, K, N, scale, flags + 1, stream);
     }
     else if (regular && (K & 3) == 0)
         hipLaunchKernelGGL((lutgemm_gradB_slab_kernel<true, int16_t>), grid, dim3(1024), 0, stream, gC, A, B, out, lut, g.cols, 1 << g.bits,
@@ -682,7 +681,7 @@ hipError_t launch_gradB_slab(const float* gC, const uint8_t* A, const uint8_t* B
     }
     // 7-bit operands can hold the masked code 128, and any table can hold an entry a half cannot: the gated
     // direct kernel covers both (for narrower tables a code 2^b is an ordinary slab row of zeros)
-    if (g.bits == 7 || half_slab) return launch_gradB_gated(gC, A, B, gB, lut, g, M, K, N, scale, flags + 1, partials, n_cu, stream);
+    if (g.bits == 7 || half_slab) return launch_gradB_gated(gC, A, B, gB, lut, g, M, K, N, scale, flags + 1, stream);
     return hipSuccess;
 }
 
@@ -720,8 +719,7 @@ hipError_t launch_gradB_slab_f32tab(const float* gC, const uint8_t* A, const uin
         e = hipGetLastError();
         if (e != hipSuccess) return e;
     }
-    // (the gated direct kernel splits M over the scratch of partial sums, free again by then)
-    if (g.bits == 7) return launch_gradB_f32tab(gC, A, B, gB, lut, g, M, K, N, scale, partials, n_cu, stream, flags + 1);
+    if (g.bits == 7) return launch_gradB_f32tab(gC, A, B, gB, lut, g, M, K, N, scale, nullptr, n_cu, stream, flags + 1);
     return hipSuccess;
 }
 

@@ -379,11 +379,10 @@ def test_backward_large_m_masked_codes(lib, oracle):
 
 
 @pytest.mark.parametrize("kind", ["i16", "f32"])
-def test_backward_masked_code_fallback_splits_the_sum_over_rows(lib, oracle, kind):
-    """A masked code sends the whole result to the direct kernels queued behind the expanded-table ones.  Their sum over
-    tens of thousands of rows is split like an ungated launch's (over the scratch the kernel in front has finished with): the
-    result stays within 3e-6 of the float64 one norm-wise, where one accumulator per output walking all rows comes to 1e-5
-    on gradients with a non-zero mean."""
+def test_backward_masked_code_fallback_keeps_the_digits_of_a_long_sum(lib, oracle, kind):
+    """A masked code sends the whole result to the direct kernels queued behind the expanded-table ones, where one wave adds
+    all rows of a k tile.  It adds them in blocks (block sums into a second accumulator), so the result stays within 3e-6 of
+    the float64 one norm-wise; one running sum over 32768 rows comes to 1e-5 on gradients with a non-zero mean."""
     print("masked-code fallback at 32768 rows", kind, flush=True)
     M, K, N = 32768, 128, 64
     rng, A, B, _ = rand_case(seed_of("mask", kind), M, K, N, 7)
