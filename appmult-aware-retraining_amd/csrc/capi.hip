@@ -20,7 +20,8 @@ hipError_t launch_fwd_slab(const uint8_t* A, const uint8_t* B, uint32_t* C, cons
 size_t gradB_workspace_bytes(int M, int K, int N, int n_cu);
 hipError_t launch_gradB(const float* gC, const uint8_t* A, const uint8_t* B, float* gB, const int16_t* lut,
                         const LutGeom& g, int M, int K, int N, float scale, void* workspace, int n_cu,
-                        hipStream_t stream, const uint32_t* gate = nullptr);
+                        hipStream_t stream, const uint32_t* gate = nullptr, int split_cap = 0);
+int gradB_direct_splits_for(const LutGeom& g, int M, int K, int N, int n_cu);
 hipError_t launch_gradA(const float* gC, const uint8_t* A, const uint8_t* B, float* gA, const int16_t* lut,
                         const LutGeom& g, int M, int K, int N, float scale, int n_cu, hipStream_t stream,
                         const uint32_t* gate = nullptr, int rows_per_image = 0);
@@ -58,7 +59,7 @@ bool gradB_slab8_applies(const LutGeom& g, int M, int K, int N, const float* gC,
 int gradB_slab8_splits(int M, int K, int N, int n_cu);
 hipError_t launch_gradB_slab8(const float* gC, const uint8_t* A, const uint8_t* B, float* gB, const int16_t* lut,
                               const LutGeom& g, int M, int K, int N, float scale, float* partials, int n_cu,
-                              hipStream_t stream);
+                              hipStream_t stream, int split_cap = 0);
 bool gradB_slab8f_applies(const LutGeom& g, int M, int K, int N, const float* gC, bool force);
 int gradB_slab8f_splits(int M, int K, int N, int n_cu);
 hipError_t launch_gradB_slab8f(const float* gC, const uint8_t* A, const uint8_t* B, float* gB, const float* lut,
@@ -68,7 +69,7 @@ int gradB_slab_splits(int M, int K, int N, int n_cu);
 size_t gradB_slab_colsum_floats(int N);
 hipError_t launch_gradB_slab(const float* gC, const uint8_t* A, const uint8_t* B, float* gB, const int16_t* lut,
                              const LutGeom& g, int M, int K, int N, float scale, uint32_t* flags, float* partials,
-                             int n_cu, hipStream_t stream);
+                             int n_cu, hipStream_t stream, int split_cap = 0);
 hipError_t launch_gradB_f32tab(const float* gC, const uint8_t* A, const uint8_t* B, float* gB, const float* lut, const LutGeom& g,
                                int M, int K, int N, float scale, void* workspace, int n_cu, hipStream_t stream,
                                const uint32_t* gate);
@@ -140,6 +141,9 @@ struct DeviceState {
 };
 DeviceState g_dev[kMaxDevices];
 std::mutex g_mu;
+// what the library itself has taken from the runtime so far (amr_library_resources)
+size_t g_allocated_bytes = 0;
+int g_side_streams = 0;
 
 // Number of compute units of the current device (cached).
 int current_device_cus(int* dev_out) {
@@ -171,6 +175,7 @@ void* internal_workspace(int dev, hipStream_t stream, size_t bytes, hipError_t* 
     void* p = nullptr;
     *err = hipMalloc(&p, want);
     if (*err != hipSuccess) return nullptr;
+    g_allocated_bytes += want;
     if (slot) { slot->ptr = p; slot->bytes = want; }               // the old buffer stays allocated (see above)
     else d.scratch.push_back({stream, p, want});
     return p;
@@ -190,6 +195,7 @@ bool stream_fork(int dev, hipStream_t stream, StreamFork* out) {
         return false;
     }
     d.forks.push_back(f);
+    ++g_side_streams;
     *out = f;
     return true;
 }
@@ -222,6 +228,12 @@ int amr_set_expanded_table_kernels(int mode) {
 }
 
 int amr_set_backward_fork(int on) { return g_fork_small.exchange(on ? 1 : 0); }
+
+void amr_library_resources(size_t* scratch_bytes, int* side_streams) {
+    std::lock_guard<std::mutex> lk(g_mu);
+    if (scratch_bytes) *scratch_bytes = g_allocated_bytes;
+    if (side_streams) *side_streams = g_side_streams;
+}
 
 int amr_bits_from_lut_elems(int64_t lut_elems) {
     amr::LutGeom g;
@@ -388,19 +400,37 @@ static int backward_impl(const float* gC, const uint8_t* A, const uint8_t* B, fl
     if (n_cu <= 0) return fail(AMR_EINVAL, "no HIP device available");
     hipError_t e;
     const int mode = g_expanded_kernels.load();
-    const size_t partial_bytes = backward_partial_bytes(M, K, N, n_cu);
+    size_t partial_bytes = backward_partial_bytes(M, K, N, n_cu);
     // (what this table width needs: never more than the shape-only query answers)
     size_t gradA_bytes = backward_gradA_bytes(mode, g.bits, M, K, N);
     bool allow_slab_a = true;
+    int split_cap = 0;
     void* ws = workspace;
+    const bool slab = mode && amr::bwd_slab_applies(g, M, K, N);
+    const bool slab_b8 = !slab && mode && amr::gradB_slab8_applies(g, M, K, N, gC, mode == 2);
     if (from == ScratchFrom::Static) {
-        if (256 + partial_bytes + gradA_bytes > kStaticScratchBytes) {   // without the expanded table of gradA (direct kernel) it may still fit
+        // The array is sized for the kernels this call will launch, not for the largest any width could take: gradB splits
+        // M as far as the array has room for partial sums (down to no split at all, which needs none), gradA keeps its
+        // expanded table if that still fits behind them and runs on the direct kernel otherwise.
+        const size_t per_split = (size_t)K * N * sizeof(float);
+        const size_t colsum = (gB && slab) ? amr::gradB_slab_colsum_floats(N) * sizeof(float) : 0;
+        if (256 + colsum + 256 > kStaticScratchBytes)
+            return fail(AMR_EWORKSPACE, "N = %d needs %zu bytes of column sums, the static scratch holds %zu: use amr_lut_gemm_backward with a workspace",
+                        N, colsum, kStaticScratchBytes);
+        int want = !gB ? 1 : slab ? amr::gradB_slab_splits(M, K, N, n_cu) : slab_b8 ? amr::gradB_slab8_splits(M, K, N, n_cu)
+                                                                                   : amr::gradB_direct_splits_for(g, M, K, N, n_cu);
+        const size_t room = kStaticScratchBytes - 256 - colsum - 256;
+        // (half the array at most for partial sums while gradA has an expanded table to place behind them)
+        size_t cap = room / per_split;
+        if (gA && gradA_bytes && gradA_bytes < room && (room - gradA_bytes) / per_split >= 2) cap = (room - gradA_bytes) / per_split;
+        if (cap < 1) cap = 1;
+        if ((size_t)want > cap) want = (int)cap;
+        split_cap = (int)cap;
+        partial_bytes = (colsum + (want > 1 ? (size_t)want * per_split : 0) + 255) & ~(size_t)255;
+        if (256 + partial_bytes + gradA_bytes > kStaticScratchBytes) {   // gradA without its expanded table (direct kernel)
             gradA_bytes = 0;
             allow_slab_a = false;
         }
-        if (256 + partial_bytes > kStaticScratchBytes)
-            return fail(AMR_EWORKSPACE, "this shape needs %zu bytes of scratch, the static scratch holds %zu: use amr_lut_gemm_backward with a workspace",
-                        256 + partial_bytes, kStaticScratchBytes);
         ws = static_scratch_ptr(dev, &e);
         if (!ws) return hip_fail(e, "hipGetSymbolAddress(scratch)");
     }
@@ -414,7 +444,6 @@ static int backward_impl(const float* gC, const uint8_t* A, const uint8_t* B, fl
     }
     uint32_t* flags = reinterpret_cast<uint32_t*>(ws);
     float* partials = reinterpret_cast<float*>(reinterpret_cast<unsigned char*>(ws) + 256);
-    const bool slab = mode && amr::bwd_slab_applies(g, M, K, N);
     const bool slab_a = mode && allow_slab_a && gA && amr::gradA_slab_workspace_bytes(g, M, K, N, mode == 2) != 0 && ((uintptr_t)gC & 15) == 0;
     // (8-bit tables: the expanded table holds the int16 entries, nothing to decide in a header)
     // (or, for layers of a few thousand rows, none at all: the table is expanded in LDS and the scratch holds partial results)
@@ -454,11 +483,11 @@ static int backward_impl(const float* gC, const uint8_t* A, const uint8_t* B, fl
     hipError_t eb = hipSuccess;
     if (gB) {     // (queued also when the gradA launch failed: a forked side stream must be joined again either way)
         if (slab) {
-            eb = amr::launch_gradB_slab(gC, A, B, gB, lut_grad_b, g, M, K, N, scale, flags, partials, n_cu, sb);
-        } else if (mode && amr::gradB_slab8_applies(g, M, K, N, gC, mode == 2)) {
-            eb = amr::launch_gradB_slab8(gC, A, B, gB, lut_grad_b, g, M, K, N, scale, partials, n_cu, sb);
+            eb = amr::launch_gradB_slab(gC, A, B, gB, lut_grad_b, g, M, K, N, scale, flags, partials, n_cu, sb, split_cap);
+        } else if (slab_b8) {
+            eb = amr::launch_gradB_slab8(gC, A, B, gB, lut_grad_b, g, M, K, N, scale, partials, n_cu, sb, split_cap);
         } else {
-            eb = amr::launch_gradB(gC, A, B, gB, lut_grad_b, g, M, K, N, scale, partials, n_cu, sb);
+            eb = amr::launch_gradB(gC, A, B, gB, lut_grad_b, g, M, K, N, scale, partials, n_cu, sb, nullptr, split_cap);
         }
     }
     if (forked) {

@@ -301,15 +301,23 @@ size_t gradB_workspace_bytes(int M, int K, int N, int n_cu) {
     return s > 1 ? (size_t)s * K * N * sizeof(float) : 0;
 }
 
+// M splits the direct gradB launch of a table of this width picks (launch_gradB below).
+int gradB_direct_splits_for(const LutGeom& g, int M, int K, int N, int n_cu) {
+    const bool big = g.bits == 8;
+    return gradB_direct_splits(M, K, N, n_cu, big ? 16 : 4, big ? 1 : 4);
+}
+
 // workspace: room for the partial sums (gradB_workspace_bytes), or nullptr: no split over M.
 hipError_t launch_gradB(const float* gC, const uint8_t* A, const uint8_t* B, float* gB, const int16_t* lut,
                         const LutGeom& g, int M, int K, int N, float scale, void* workspace, int n_cu,
-                        hipStream_t stream, const uint32_t* gate = nullptr) {
+                        hipStream_t stream, const uint32_t* gate = nullptr, int split_cap = 0) {
     constexpr int KT = 16;
     const int lut_dwords = g.rows * g.cols / 2;
     const size_t lds = (size_t)lut_dwords * 4;
     const bool big = g.bits == 8;
-    const int splits = workspace ? gradB_direct_splits(M, K, N, n_cu, big ? 16 : 4, big ? 1 : 4) : 1;
+    // split_cap > 0: the most M splits the caller's scratch has room for
+    int splits = workspace ? gradB_direct_splits(M, K, N, n_cu, big ? 16 : 4, big ? 1 : 4) : 1;
+    if (split_cap > 0 && splits > split_cap) splits = split_cap;
     int m_chunk = (M + splits - 1) / splits;
     m_chunk = (m_chunk + 15) & ~15;
     const int zs = (M + m_chunk - 1) / m_chunk;

@@ -509,9 +509,9 @@ __global__ __launch_bounds__(256) void gradB_finish_kernel(const float* __restri
 __global__ __launch_bounds__(1024) void bwd_header_kernel(const uint32_t* __restrict__ lut_a, const uint32_t* __restrict__ lut_b,
                                                           int lut_dwords, int n_entries, uint32_t* __restrict__ flags) {
     __shared__ int extremes[4];
-    __shared__ float magnitude[2];
+    __shared__ unsigned int magnitude[2];      // sum of |entry|: at most 65536 x 32768 < 2^32, added as integers (any order, same sum)
     if (threadIdx.x < 4) extremes[threadIdx.x] = 0;
-    if (threadIdx.x < 2) magnitude[threadIdx.x] = 0.f;
+    if (threadIdx.x < 2) magnitude[threadIdx.x] = 0u;
     __syncthreads();
     // all loads of both tables are issued before the first is used (one dependent load at a time would pay the
     // memory latency 66 times: 19 us instead of 5)
@@ -546,7 +546,7 @@ __global__ __launch_bounds__(1024) void bwd_header_kernel(const uint32_t* __rest
             if ((threadIdx.x & 63) == 0) {
                 atomicMin(&extremes[2 * t], lo);
                 atomicMax(&extremes[2 * t + 1], hi);
-                atomicAdd(&magnitude[t], (float)mag);
+                atomicAdd(&magnitude[t], (unsigned int)mag);
             }
         }
     }
@@ -570,7 +570,7 @@ __global__ __launch_bounds__(1024) void bwd_header_kernel(const uint32_t* __rest
                     const int mag_off = p <= room ? p : need;
                     off[t] = hi > 2048 ? mag_off : -mag_off;
                 }
-                if ((float)abs(off[t]) * (float)n_entries > 8.f * magnitude[t]) unusable[t] = 1;
+                if ((unsigned long long)abs(off[t]) * (unsigned long long)n_entries > 8ull * magnitude[t]) unusable[t] = 1;
             }
             if (unusable[t]) off[t] = 0;
         }
@@ -633,13 +633,15 @@ int gradB_slab_splits(int M, int K, int N, int n_cu) {
 
 hipError_t launch_gradB_slab(const float* gC, const uint8_t* A, const uint8_t* B, float* gB, const int16_t* lut,
                              const LutGeom& g, int M, int K, int N, float scale, uint32_t* flags, float* partials,
-                             int n_cu, hipStream_t stream) {
+                             int n_cu, hipStream_t stream, int split_cap) {
     const int vec_ok = ((N & 3) == 0) && (((uintptr_t)gC & 15) == 0);
     const bool small = (size_t)M * K < (1ull << 31) && (size_t)M * N * 4 < (1ull << 31);
     const bool regular = vec_ok && small && (N & 63) == 0 && (M % kBwdRowsPerIter) == 0;
     const bool half_slab = regular && (K & 7) == 0;
     const int kt = half_slab ? kBwdKT16 : kBwdKT;
-    const int splits = gradB_slab_splits_kt(M, K, N, n_cu, kt);
+    // split_cap > 0: the most M splits the caller's scratch has room for
+    int splits = gradB_slab_splits_kt(M, K, N, n_cu, kt);
+    if (split_cap > 0 && splits > split_cap) splits = split_cap;
     int m_chunk = (M + splits - 1) / splits;
     m_chunk = (m_chunk + 255) & ~255;
     const int zs = (M + m_chunk - 1) / m_chunk;

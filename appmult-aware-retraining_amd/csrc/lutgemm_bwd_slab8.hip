@@ -460,8 +460,10 @@ int gradB_slab8_splits(int M, int K, int N, int n_cu) {
 // partials: room for gradB_slab8_splits(...) x K x N floats when that is more than one.
 hipError_t launch_gradB_slab8(const float* gC, const uint8_t* A, const uint8_t* B, float* gB, const int16_t* lut,
                               const LutGeom& g, int M, int K, int N, float scale, float* partials, int n_cu,
-                              hipStream_t stream) {
-    const int splits = gradB_slab8_splits(M, K, N, n_cu);
+                              hipStream_t stream, int split_cap) {
+    // split_cap > 0: the most M splits the caller's scratch has room for
+    int splits = gradB_slab8_splits(M, K, N, n_cu);
+    if (split_cap > 0 && splits > split_cap) splits = split_cap;
     int m_chunk = (M + splits - 1) / splits;
     m_chunk = (m_chunk + kB8RowsPerIter - 1) / kB8RowsPerIter * kB8RowsPerIter;
     const int zs = (M + m_chunk - 1) / m_chunk;

@@ -388,8 +388,9 @@ __global__ __launch_bounds__(1024) void lutgemm_gradA_rows8f_kernel(
 bool gradA_rows8_applies(const LutGeom& g, int M, int K, int N, const float* gC, bool force) {
     const bool small = (size_t)M * K < (1ull << 31) && (size_t)M * N * 4 < (1ull << 31) &&
                        (size_t)(N / 64) * (size_t)M * (size_t)K < (1ull << 32);
+    // (the k tiles are gridDim.y of the second kernel: at most 65535 of the float variant's two k)
     return g.bits == 8 && M >= (force ? 1024 : 2048) && M < 16384 && (M % kR8RowsPerIter) == 0 && (K & 3) == 0 && (N & 63) == 0 &&
-           small && ((uintptr_t)gC & 15) == 0;
+           K / kR8fKT <= 65535 && small && ((uintptr_t)gC & 15) == 0;
 }
 
 // Bytes of the partial results, or 0 when the kernel does not apply (gC's alignment is the caller's to check).

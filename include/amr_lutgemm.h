@@ -101,8 +101,10 @@ int amr_lut_gemm_forward_f32_ws(const uint8_t *A, const uint8_t *B, float *C, co
  *   or through amr_lut_gemm_backward_static.
  */
 size_t amr_lut_gemm_backward_workspace_bytes(int M, int K, int N);
-/* The same for a known table width (lut_elems as passed to the call): 8-bit tables never use the expanded table of gradA,
- * so this answer can be much smaller; the shape-only query above is an upper bound over all widths. */
+/* The same for a known table width (lut_elems as passed to the call); the shape-only query above is an upper bound over all
+ * widths.  What gradA adds to the partial sums of gB: tables of at most 7 bits K*N*256 B of expanded table (large M only);
+ * 8-bit tables (N/64)*M*K*4 B of partial results for 2048 <= M < 16384, or K*N*512 B of int16 expanded table beyond that
+ * (K*N*1 KB for float tables) -- e.g. 302 MB for 2048 x 4608 x 512, more than the 7-bit answer for that shape. */
 size_t amr_lut_gemm_backward_workspace_bytes_for(int64_t lut_elems, int M, int K, int N);
 int amr_lut_gemm_backward(const float *gC, const uint8_t *A, const uint8_t *B, float *gA, float *gB,
                           const int16_t *lut_grad_a, const int16_t *lut_grad_b, int64_t lut_elems,
@@ -124,10 +126,12 @@ int amr_lut_gemm_backward_ex(const float *gC, const uint8_t *A, const uint8_t *B
  * amr_lut_gemm_backward_ex for callers that cannot allocate: code under HIP graph capture, tight serving loops, harnesses
  * that forbid hipMalloc.  It has no counterpart in the reference.  Same arguments, results and kernels; the scratch
  * (flags, partial sums of gB, expanded table of gradA) is a file-scope device array of AMR_STATIC_SCRATCH_BYTES inside the
- * library, one copy per GPU, held until the process ends.  The call allocates and frees nothing.  A shape whose expanded
- * table of gradA does not fit runs gradA on the direct kernel instead; a shape whose partial sums of gB alone exceed the
- * array is rejected with AMR_EWORKSPACE.  All calls on one GPU share that array: calls that overlap in time on one
- * GPU (two streams, two threads) race; calls queued on one stream do not.
+ * library, one copy per GPU, held until the process ends.  The call allocates and frees nothing.  The array is sized for
+ * the kernels the call launches: gradB splits M only as far as the array has room for partial sums (K*N*4 B each; with
+ * room for fewer than two it does not split, which needs none), and a shape whose expanded table of gradA does not fit
+ * behind them runs gradA on the direct kernel -- same results up to summation order, slower.  Only a shape whose column sums
+ * of gC alone (64*N*4 B, N beyond 131 000) exceed the array is rejected with AMR_EWORKSPACE.  All calls on one GPU share
+ * that array: calls that overlap in time on one GPU (two streams, two threads) race; calls queued on one stream do not.
  */
 #define AMR_STATIC_SCRATCH_BYTES (32u << 20)
 size_t amr_static_scratch_bytes(void);
@@ -193,6 +197,14 @@ int amr_set_expanded_table_kernels(int mode);
  * (self_ops/src/approx_gemm_backward.cu:560-608).
  */
 int amr_set_backward_fork(int on);
+
+/*
+ * What the library has taken from the HIP runtime since it was loaded, over all devices: bytes of scratch it allocated for
+ * callers that passed no workspace (never freed), and side streams it created (amr_set_backward_fork).  Either pointer may
+ * be NULL.  A call with a caller workspace on a problem that does not fork, and amr_lut_gemm_backward_static, change neither.
+ * Diagnostics; no counterpart in the reference.
+ */
+void amr_library_resources(size_t *scratch_bytes, int *side_streams);
 
 /*
  * Dequantisation behind the LUT convolution, from the GEMM's row layout to the NCHW activation in one pass:
