@@ -34,6 +34,18 @@ def lut_geometry(quantization_bit):
     return rows, cols, rows * cols + _TAIL[quantization_bit]
 
 
+def pad_table(table2d, quantization_bit, dtype):
+    """A (2^b, 2^b) table as the padded 1-D array of the boundary: entry (a, b) at a * cols + b, zeros elsewhere
+    (reference ``approx_ops.py:21-41,70-77``)."""
+    rows, cols, elems = lut_geometry(quantization_bit)
+    n = 1 << quantization_bit
+    t = np.asarray(table2d)
+    assert t.shape == (n, n), f"table must be {n} x {n}"
+    flat = np.zeros(elems, dtype)
+    flat[:rows * cols].reshape(rows, cols)[:n, :n] = t.astype(dtype)
+    return flat
+
+
 def read_lut_file(file_name, quantization_bit):
     """Parse a table file into three padded 1-D NumPy arrays (uint16, int16, int16).
 

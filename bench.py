@@ -69,9 +69,10 @@ def profile_rows(name):
 
 
 def conv2x_counters(kind):
-    """From profiles/: (bytes the L2s read + wrote for the conv2_x launch of this phase's kernel, VALU instructions per
-    multiply-add of that kernel = counted wave instructions x 64 lanes / multiply-adds of the counted launches); None for what
-    no committed table holds."""
+    """From the committed counter tables in profiles/ (NOT measured in this run; every field taken from them is labelled
+    "source": "committed profile"): (bytes the L2s read + wrote for the conv2_x launch of this phase's kernel, VALU
+    instructions per multiply-add of that kernel = counted wave instructions x 64 lanes / multiply-adds of the counted
+    launches); None, with a warning on stderr, for what no committed table holds."""
     kernel = CONV2X_KERNEL[kind]
     traffic = valu_per_mac = None
     for k, cells in profile_rows("conv2x_hbm_traffic.md").items():
@@ -80,25 +81,25 @@ def conv2x_counters(kind):
     for k, cells in profile_rows("conv2x_lds_counters.md").items():
         if kernel in k and len(cells) > 9:
             valu_per_mac = float(cells[9])
+    if traffic is None or valu_per_mac is None:
+        print(f"bench.py: no row for kernel '{kernel}' in profiles/conv2x_hbm_traffic.md / conv2x_lds_counters.md: "
+              "counter-derived fields of this phase are null", file=sys.stderr)
     return traffic, valu_per_mac
 
 
-def training_step_lut_share():
-    """Share of the LUT GEMM kernels (forward, gradA, gradB, table expansions, gated fall-backs) in the GPU time of a training
-    step, from the committed kernel trace of app_train.py (profiles/resnet18_b512_training_step_kernels.md)."""
-    lut = total = 0.0
-    try:
-        with open(os.path.join(PROFILES, "resnet18_b512_training_step_kernels.md")) as f:
-            for line in f:
-                parts = line.split()
-                if len(parts) >= 6 and parts[-1] == "%" and parts[-3] == "ms" and "calls" in parts:
-                    ms = float(parts[-4])
-                    total += ms
-                    if any(t in line for t in ("amr::lutgemm_", "amr::expand_", "amr::gradB_finish", "amr::bwd_header", "amr::reduce_partials")):
-                        lut += ms
-    except OSError:
-        return None
-    return lut / total if total > 0 else None
+def synth_tables(np, bits, err, half_ws, float_slopes=False):
+    """The benchmark's tables from the package's own generator: forward table a*b + seeded error in [-err, err] clipped to
+    uint16 (BASELINE.json configs[0]), gradient tables = its difference-based slopes (gen_bp_lut.gradient_tables), all three
+    as the padded 1-D arrays of the boundary.  Returns (forward u16, grad_a, grad_b, 2-D forward table)."""
+    import gen_bp_lut
+    from self_ops.ops_py import approx_ops as ops
+    rng = np.random.default_rng(0)
+    n = 1 << bits
+    a = np.arange(n, dtype=np.int64)
+    T = np.clip(a[:, None] * a[None, :] + rng.integers(-err, err + 1, size=(n, n)), 0, 65535)
+    gx, gy = gen_bp_lut.gradient_tables(T, half_ws, rounded=not float_slopes)
+    gdt = np.float32 if float_slopes else np.int16
+    return ops.pad_table(T, bits, np.uint16), ops.pad_table(gx, bits, gdt), ops.pad_table(gy, bits, gdt), T
 
 
 def capture_codes(torch, dev, bits, tables, arch, batch):
@@ -129,50 +130,81 @@ def capture_codes(torch, dev, bits, tables, arch, batch):
 
 def training_step(torch, dev, tables, bits, batch=512, steps=10):
     """Forward + cross-entropy + backward + SGD update of this package's quantised ResNet-18 (LUT convolutions) on synthetic
-    CIFAR-shaped data, after one calibration pass and one untimed step: wall-clock ms per step and images per second, and
-    the LUT kernels' share of a step's GPU time from the committed kernel trace of the same loop."""
+    CIFAR-shaped data, after one calibration pass and one untimed step: wall-clock ms per step and images per second.
+    The LUT GEMM's share of a step's GPU time is measured in this run, on three further steps outside the timed ones: HIP
+    events on the launch stream around every call of the library's forward and backward GEMM entry points (table expansion,
+    header, finish and gated launches included), summed, over the events around the whole steps."""
     import app_train
+    import approx_ops as native
     from self_ops.ops_py import approx_ops as ops
     ops.set_lookup_tables(dev, *(t.cpu().numpy() for t in tables))
     torch.manual_seed(0)
     model = app_train.build_model("resnet18", bits, False, dev)
-    xs, ys = app_train.synthetic_batches(steps + 2, batch, dev)
+    share_steps = 3
+    xs, ys = app_train.synthetic_batches(steps + 2 + share_steps, batch, dev)
     app_train.calibrate(model, xs[:1])
     opt = torch.optim.SGD(model.parameters(), lr=1e-2, momentum=0.9)
     app_train.train_steps(model, opt, xs[1:2], ys[1:2])
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    losses = app_train.train_steps(model, opt, xs[2:], ys[2:])
+    losses = app_train.train_steps(model, opt, xs[2:2 + steps], ys[2:2 + steps])
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
-    share = training_step_lut_share()
+
+    spans = []
+    names = [n for n in ("approx_gemm_forward", "approx_gemm_backward", "approx_conv_forward_dequant") if hasattr(native, n)]
+    originals = {n: getattr(native, n) for n in names}
+
+    def timed_call(fn):
+        def call(*a, **k):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            r = fn(*a, **k)
+            e1.record()
+            spans.append((e0, e1))
+            return r
+        return call
+
+    for n in names:
+        setattr(native, n, timed_call(originals[n]))
+    try:
+        s0, s1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        s0.record()
+        app_train.train_steps(model, opt, xs[2 + steps:], ys[2 + steps:])
+        s1.record()
+        torch.cuda.synchronize()
+    finally:
+        for n in names:
+            setattr(native, n, originals[n])
+    lut_ms = sum(a.elapsed_time(b) for a, b in spans)
     return {"workload": f"resnet18_cifar_b{batch}_{bits}bit full step: forward, cross-entropy, backward, SGD (BASELINE.json configs[4])",
             "steps": steps, "ms_per_step": dt / steps * 1e3, "images_per_s": batch * steps / dt,
             "loss_first_last": [float(losses[0]), float(losses[-1])],
-            "lut_gemm_share_of_gpu_time": share, "share_source": "profiles/resnet18_b512_training_step_kernels.md (rocprofv3 --kernel-trace)"}
+            "lut_gemm_share_of_gpu_time": lut_ms / s0.elapsed_time(s1),
+            "lut_gemm_ms_per_step": lut_ms / share_steps,
+            "share_source": f"measured in this run: HIP events around the {len(spans) // share_steps} library GEMM calls of a step, {share_steps} steps"}
 
 
-def eight_bit_step(torch, np, dev, lib, O, stream, steps=5):
-    """The 8-bit stress configuration (BASELINE.json configs[3]: VGG-16 conv shapes at batch 128, 8-bit int16 tables) as a
-    secondary record of the default run: the same forward + backward GEMM step as the headline, timed over `steps` steps after
-    two untimed ones.  (`--workload vgg16_b128_8bit` runs it as the main workload, with the per-kernel break-down.)"""
-    bits, err, half_ws = 8, 256, 16
-    rng = np.random.default_rng(0)
-    T = O.synth_lut(bits, err, rng)
-    Gx, Gy = O.gen_bp_lut(T, half_ws)
-    lut = torch.from_numpy(O.pack_table(T, bits, np.uint16)).to(dev)
-    lga = torch.from_numpy(O.pack_table(Gx, bits, np.int16)).to(dev)
-    lgb = torch.from_numpy(O.pack_table(Gy, bits, np.int16)).to(dev)
+def eight_bit_step(torch, np, dev, lib, O, stream, float_tables, steps=5):
+    """The 8-bit stress configuration (BASELINE.json configs[3]: VGG-16 conv shapes at batch 128, forward error +-256, half
+    window 16) as a secondary record of the default run, with the reference's int16 x16 gradient tables or with the float32
+    slopes the configuration names: the same forward + backward GEMM step as the headline, timed over `steps` steps after two
+    untimed ones.  (`--workload vgg16_b128_8bit [--grad-tables f32]` runs it as the main workload, with the per-kernel
+    break-down.)"""
+    bits = 8
+    f16, ga_t, gb_t, _ = synth_tables(np, bits, 256, 16, float_slopes=float_tables)
+    lut, lga, lgb = (torch.from_numpy(t).to(dev) for t in (f16, ga_t, gb_t))
     L = lut.numel()
     gen = torch.Generator(device=dev).manual_seed(0)
     bufs, ws_need = {}, 0
+    ws_query = lib.amr_lut_gemm_backward_f32tab_workspace_bytes if float_tables else lib.amr_lut_gemm_backward_workspace_bytes
     for name, cnt, M, K, N in VGG16_B128:
         bufs[name] = (torch.randint(0, 256, (M, K), dtype=torch.uint8, device=dev, generator=gen),
                       torch.randint(0, 256, (K, N), dtype=torch.uint8, device=dev, generator=gen),
                       torch.empty((M, N), dtype=torch.int32, device=dev),
                       torch.randn((M, N), dtype=torch.float32, device=dev, generator=gen),
                       torch.empty((M, K), dtype=torch.float32, device=dev), torch.empty((K, N), dtype=torch.float32, device=dev))
-        ws_need = max(ws_need, lib.amr_lut_gemm_backward_workspace_bytes(M, K, N))
+        ws_need = max(ws_need, ws_query(M, K, N))
     ws = torch.empty(max(ws_need, 256), dtype=torch.uint8, device=dev)
 
     def step():
@@ -183,16 +215,25 @@ def eight_bit_step(torch, np, dev, lib, O, stream, steps=5):
         for name, cnt, M, K, N in reversed(VGG16_B128):
             A, B, C, gC, gA, gB = bufs[name]
             for _ in range(cnt):
-                assert lib.amr_lut_gemm_backward(gC.data_ptr(), A.data_ptr(), B.data_ptr(), gA.data_ptr(), gB.data_ptr(), lga.data_ptr(),
-                                                 lgb.data_ptr(), L, M, K, N, ws.data_ptr(), ws.numel(), stream) == 0, lib.amr_last_error()
+                if float_tables:
+                    rc = lib.amr_lut_gemm_backward_f32tab(gC.data_ptr(), A.data_ptr(), B.data_ptr(), gA.data_ptr(), gB.data_ptr(), lga.data_ptr(),
+                                                          lgb.data_ptr(), L, 1.0, M, K, N, 0, ws.data_ptr(), ws.numel(), stream)
+                else:
+                    rc = lib.amr_lut_gemm_backward(gC.data_ptr(), A.data_ptr(), B.data_ptr(), gA.data_ptr(), gB.data_ptr(), lga.data_ptr(),
+                                                   lgb.data_ptr(), L, M, K, N, ws.data_ptr(), ws.numel(), stream)
+                assert rc == 0, lib.amr_last_error()
 
-    # parity guard on a row sample of one layer that takes the expanded int16 tables (the parity suite proper is tests/ -m gpu)
+    # parity guard on a row sample of one layer that takes the expanded tables (the parity suite proper is tests/ -m gpu)
     name, _, M, K, N = VGG16_B128[2]
     A, B, C, gC, gA, gB = bufs[name]
     step()
     torch.cuda.synchronize()
     rows = slice(100, 132)
-    want_a, _ = O.backward_c_f32(gC[rows].cpu().numpy(), A[rows].cpu().numpy(), B.cpu().numpy(), lga.cpu().numpy(), lgb.cpu().numpy(), bits)
+    if float_tables:
+        want_a, _ = O.backward_np(gC[rows].cpu().numpy(), A[rows].cpu().numpy(), B.cpu().numpy(), O.unpack_table(ga_t, bits),
+                                  O.unpack_table(gb_t, bits), factor=1.0)
+    else:
+        want_a, _ = O.backward_c_f32(gC[rows].cpu().numpy(), A[rows].cpu().numpy(), B.cpu().numpy(), ga_t, gb_t, bits)
     got_a = gA[rows].cpu().numpy()
     assert np.abs(got_a - want_a).max() <= 1e-4 * np.abs(want_a).max(), "8-bit gradA parity guard failed"
     step()
@@ -203,9 +244,17 @@ def eight_bit_step(torch, np, dev, lib, O, stream, steps=5):
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
     macs = 3 * sum(c * M * K * N for _, c, M, K, N in VGG16_B128)
-    return {"workload": "vgg16_cifar_b128_8bit_lutgemm_fwd_bwd (BASELINE.json configs[3]: 13 conv + 1 fc GEMMs), int16 gradient tables",
+    # floors of this step: VALU issue, one multiply-add per backward LUT-MAC and half an addition per forward entry; LDS read
+    # bandwidth, 2 bytes per table entry (4 for float32 gradient tables)
+    floor_valu = (0.5 + 2.0) * (macs / 3) / VALU_ISSUE_PEAK
+    floor_lds = (2 + (8 if float_tables else 4)) * (macs / 3) / LDS_READ_PEAK
+    floor = max(floor_valu, floor_lds)
+    return {"workload": "vgg16_cifar_b128_8bit_lutgemm_fwd_bwd (BASELINE.json configs[3]: 13 conv + 1 fc GEMMs), " +
+                        ("float32 gradient tables (unrounded slopes)" if float_tables else "int16 x16 gradient tables"),
             "steps": steps, "ms_per_step": dt / steps * 1e3, "lut_mac_per_s": macs * steps / dt,
-            "frac_of_lds_gather_roofline": macs * steps / dt / LDS_GATHER_PEAK}
+            "frac_of_lds_gather_roofline": macs * steps / dt / LDS_GATHER_PEAK,
+            "own_bound": {"floor_ms": floor * 1e3, "binds": "valu_issue" if floor_valu >= floor_lds else "lds_read",
+                          "frac": floor / (dt / steps)}}
 
 
 def main():
@@ -249,7 +298,7 @@ def main():
         assert RESNET18_B256, "no such layer"
 
     import approx_ops  # loads libamr_lutgemm.so, fails loudly when it is missing
-    from oracle import lutgemm_oracle as O   # checker + CPU baseline only
+    from oracle import lutgemm_oracle as O   # the parity guards and the CPU baseline leg only: every input comes from the package
 
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = torch.device("cuda:0")
@@ -257,17 +306,10 @@ def main():
     lib = approx_ops._lib
     stream = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
 
-    # tables (config 1 recipe) -------------------------------------------------------------------
-    rng = np.random.default_rng(0)
-    T = O.synth_lut(BITS, ERR, rng)
-    Gx, Gy = O.gen_bp_lut(T, HALF_WS)
-    lut = torch.from_numpy(O.pack_table(T, BITS, np.uint16)).to(dev)
+    # tables (config 1 recipe), built by the package's own generator --------------------------------
     f32_tables = args.grad_tables == "f32"
-    if f32_tables:
-        Gx, Gy = O.gen_bp_lut(T, HALF_WS, rounded=False)
-    gdt = np.float32 if f32_tables else np.int16
-    lga = torch.from_numpy(O.pack_table(Gx, BITS, gdt)).to(dev)
-    lgb = torch.from_numpy(O.pack_table(Gy, BITS, gdt)).to(dev)
+    f16_np, ga_np, gb_np, _ = synth_tables(np, BITS, ERR, HALF_WS, float_slopes=f32_tables)
+    lut, lga, lgb = (torch.from_numpy(t).to(dev) for t in (f16_np, ga_np, gb_np))
     L = lut.numel()
 
     # operands, resident in HBM --------------------------------------------------------------------
@@ -286,7 +328,7 @@ def main():
     ws = torch.empty(max(ws_need, 256), dtype=torch.uint8, device=dev)
 
     if args.codes == "captured":
-        seen = capture_codes(torch, dev, BITS, (lut.cpu().numpy(), lga.cpu().numpy(), lgb.cpu().numpy()),
+        seen = capture_codes(torch, dev, BITS, (f16_np, ga_np, gb_np),
                              "resnet18" if headline else "vgg16", BATCH)
         for name, cnt, M, K, N in RESNET18_B256:
             assert (M, K, N) in seen, f"the network's forward pass ran no LUT GEMM of shape {(M, K, N)} ({name})"
@@ -406,6 +448,23 @@ def main():
     # (left out of a run restricted to some layers: a profiler run of such a subset then holds launches of those layers only)
     t_single = timed(lambda: (fwd("single", M1, K1, N1), bwd("single", M1, K1, N1)), reps=50) if full else float("nan")
 
+    # Limits that are ceilings of this hardware for the work itself, whatever the formulation (no fraction of them can pass 1):
+    # vector issue -- one multiply-add instruction lane per backward LUT-MAC, half an addition per forward table entry (two
+    # 16-bit entries per 32-bit add), 64 lanes per clock and CU; LDS read bandwidth -- the table entry of every LUT-MAC (2 B;
+    # 4 B from float32 gradient tables) at 256 B per clock and CU.
+    entry_b = 4 if f32_tables else 2
+    own = {"valu_issue_peak_lane_ops_per_s": VALU_ISSUE_PEAK, "lds_read_peak_Bps": LDS_READ_PEAK,
+           "definition": "floor time = max(VALU-issue floor: 1 multiply-add per backward LUT-MAC, 0.5 additions per forward entry, 64 lanes/clk/CU; "
+                         "LDS-read floor: one table entry per LUT-MAC at 256 B/clk/CU), 256 CU x 2.4 GHz; frac = floor time / measured time",
+           "per_phase": {}}
+    floor_step = 0.0
+    for kind, ops_per_mac, bytes_per_mac in (("forward", 0.5, 2), ("gradA", 1.0, entry_b), ("gradB", 1.0, entry_b)):
+        fv, fl = macs_fwd * ops_per_mac / VALU_ISSUE_PEAK * 1e3, macs_fwd * bytes_per_mac / LDS_READ_PEAK * 1e3
+        floor_step += max(fv, fl)
+        own["per_phase"][kind] = {"valu_floor_ms": fv, "lds_read_floor_ms": fl, "binds": "valu_issue" if fv >= fl else "lds_read",
+                                  "measured_ms": kernels[kind], "frac": max(fv, fl) / kernels[kind]}
+    own["step"] = {"floor_ms": floor_step, "measured_ms": ms_step, "frac": floor_step / ms_step}
+
     out = {
         "metric": "LUT-MAC/s fwd+bwd (ResNet-18 conv shapes, 7-bit)" if headline else "LUT-MAC/s fwd+bwd (VGG-16 conv shapes, 8-bit)",
         "value": rate, "unit": "LUT-MAC/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -417,6 +476,8 @@ def main():
                    "vgg16_cifar_b128_8bit_lutgemm_fwd_bwd (BASELINE.json configs[3]: 13 conv + 1 fc GEMMs)",
                    "batch": BATCH, "lut_macs_per_step": macs_step, "codes": "uniform random" if args.codes == "uniform" else "captured from one forward pass of the network (N(0,1) images, random-init weights, min/max quantisation)", "grad_tables": (f"float32 unrounded difference slopes, half window {HALF_WS}" if f32_tables else f"int16 x16 difference-based, half window {HALF_WS}")},
         "images_per_s": BATCH * args.steps / dt,
+        # gather-equivalent: one table entry per LUT-MAC against the direct-gather peak; the expanded-table kernels read 8
+        # entries per LDS instruction, so this figure can pass 1 -- `roofline.own_bound.step.frac` is the one that cannot
         "frac_of_lds_gather_roofline": rate / LDS_GATHER_PEAK,
         "kernel_ms_per_step": {k: round(v, 4) for k, v in kernels.items()},
         # The contract's roofline of this path: one LDS gather per LUT-MAC, 32 conflict-free lanes per clock and CU.  It is the
@@ -429,7 +490,9 @@ def main():
                      # bytes the L2s fetched + wrote for the conv2_x launch of that kernel (rocprofv3 FETCH_SIZE / WRITE_SIZE scaled
                      # against plain copies), read from the committed table profiles/conv2x_hbm_traffic.md
                      "traffic": conv2x_counters(dominant)[0] if headline and not f32_tables else None,
+                     "traffic_source": "committed profile profiles/conv2x_hbm_traffic.md (rocprofv3 --pmc, not measured in this run)",
                      "traffic_launch": "conv2_x (M=262144,K=576,N=64)", "traffic_algorithmic": hbm_bytes(dominant, 262144, 576, 64),
+                     "own_bound": own,
                      "avg_launch_ms": dom_ms / launches,
                      "hbm": {"achieved": dom_bytes / (dom_ms * 1e-3) / 1e9, "peak": HBM_PEAK / 1e9, "unit": "GB/s",
                              "frac": dom_bytes / (dom_ms * 1e-3) / HBM_PEAK},
@@ -466,8 +529,12 @@ def main():
             if direct_bytes:
                 entry["lds_direct_delivery"] = {"achieved_GBps": direct_bytes / (ms * 1e-3) / 1e9, "probe_GBps": probe_delivery / 1e9,
                                                 "frac": direct_bytes / (ms * 1e-3) / probe_delivery}
+            entry["l2_traffic_source"] = "committed profile profiles/conv2x_hbm_traffic.md"
             if valu_per_mac is not None:
-                entry["valu_issue"] = {"valu_per_mac": round(valu_per_mac, 3), "frac": mac_rate * valu_per_mac / VALU_ISSUE_PEAK}
+                # utilisation of the issue slots by the instructions the kernel executes (counted: committed profile), not a
+                # fraction of an algorithmic bound -- that is roofline.own_bound
+                entry["valu_issue"] = {"valu_per_mac": round(valu_per_mac, 3), "frac": mac_rate * valu_per_mac / VALU_ISSUE_PEAK,
+                                       "source": "committed profile profiles/conv2x_lds_counters.md"}
                 entry["bounded_by"] = "valu_issue" if entry["valu_issue"]["frac"] > entry["lds_read"]["frac"] else "lds_read"
             kb[kind] = entry
         out["kernel_bounds"] = kb
@@ -476,7 +543,10 @@ def main():
     if headline and full and not args.no_8bit and not f32_tables and args.codes == "uniform":
         del bufs, ws
         torch.cuda.empty_cache()
-        out["vgg16_b128_8bit"] = eight_bit_step(torch, np, dev, lib, O, stream)
+        out["vgg16_b128_8bit"] = eight_bit_step(torch, np, dev, lib, O, stream, float_tables=False)
+        torch.cuda.empty_cache()
+        out["vgg16_b128_8bit_f32tab"] = eight_bit_step(torch, np, dev, lib, O, stream, float_tables=True)
+        torch.cuda.empty_cache()
 
     # The full training step (BASELINE.json configs[4]): ResNet-18, batch 512, SGD, outside the headline's timed region
     if headline and full and not args.no_train_step and args.codes == "uniform":
@@ -484,9 +554,8 @@ def main():
 
     # CPU baseline: the C oracle (port of the reference formulation) on the host cores ----------------------
     if not args.no_cpu:
-        A, B, Tc, g = O.synth_gemm(M1, K1, N1, bits=BITS, err=ERR, seed=0)
-        Gx16, Gy16 = O.gen_bp_lut(Tc, HALF_WS)
-        f16, a16, b16 = O.pack_table(Tc, BITS, np.uint16), O.pack_table(Gx16, BITS, np.int16), O.pack_table(Gy16, BITS, np.int16)
+        A, B, _, g = O.synth_gemm(M1, K1, N1, bits=BITS, err=ERR, seed=0)
+        f16, a16, b16, _ = synth_tables(np, BITS, ERR, HALF_WS)
         O.forward_c(A, B, f16, BITS)
         reps, t0 = 0, time.perf_counter()
         while time.perf_counter() - t0 < 10.0:

@@ -148,3 +148,22 @@ def test_init_lookup_tables_on_cpu_device_and_errors(golden_dir, tmp_path):
     bad.write_text("LUT for approximate multiplier:\n0 0\n")
     with pytest.raises(ValueError):
         P.read_lut_file(str(bad), 7)
+
+
+@pytest.mark.parametrize("bits", [4, 6, 7, 8])
+def test_pad_table_places_entries_like_the_reader_and_the_oracle(oracle, bits):
+    """The padded layout written by the package's pad_table: entry (a, b) at a * cols + b and zeros everywhere else, i.e.
+    what the table reader produces for a file that lists every entry, and what the oracle packs."""
+    from self_ops.ops_py import approx_ops as P
+    n = 1 << bits
+    rng = np.random.default_rng(bits)
+    t = rng.integers(0, 65536, (n, n))
+    flat = P.pad_table(t, bits, np.uint16)
+    rows, cols, elems = P.lut_geometry(bits)
+    assert flat.shape == (elems,) and flat.dtype == np.uint16
+    for a, b in ((0, 0), (n - 1, n - 1), (3, n - 2), (n - 1, 0)):
+        assert flat[a * cols + b] == t[a, b]
+    assert flat.astype(np.int64).sum() == t.sum()                       # nothing but the entries is non-zero
+    assert (flat == oracle.pack_table(t, bits, np.uint16)).all()
+    g = rng.standard_normal((n, n)).astype(np.float32)
+    assert (P.pad_table(g, bits, np.float32) == oracle.pack_table(g, bits, np.float32)).all()
