@@ -179,6 +179,93 @@ class _ConvDequantFn(torch.autograd.Function):
         return g_rows, g_xs, g_wr, None, None, None, None, None, g_bias, None
 
 
+def _box_sum(xs, kernel, stride, padding, dilation):
+    """Sum of a one-channel tensor over every convolution window (zero padding): conv2d with an all-ones kernel."""
+    kh, kw = kernel
+    if tuple(dilation) == (1, 1) and 2 * padding[0] <= kh and 2 * padding[1] <= kw:
+        # (no single-channel convolution: the library runs those image by image)
+        return F.avg_pool2d(xs, (kh, kw), stride=stride, padding=padding, divisor_override=1)
+    return F.conv2d(xs, torch.ones(1, 1, kh, kw, dtype=xs.dtype, device=xs.device), bias=None, stride=stride, padding=padding,
+                    dilation=dilation)
+
+
+class _ApproxConvLayerFn(torch.autograd.Function):
+    """The activation side of ApproxConv2d.forward as one operator on uint8 codes (reference ``app_layers.py:172-183`` with
+    ``approx_ops.py:556-571`` inlined): quantiser -> pixel-major uint8 codes, in-range mask and channel sums in one pass;
+    uint8 im2col; LUT GEMM; zero-point terms, scaling and bias from the GEMM's rows to the NCHW activation.  Backward: the
+    output gradient to GEMM rows (with its row sums) in one pass, the two LUT gradient GEMMs, then col2im + gradient of the
+    zero-point term + straight-through backward of the quantiser in one pass.  No float32 code tensor exists on this path.
+
+    ``w_codes`` (float32 integer codes [N,C,kh,kw]) and ``w_resp`` come from the weight side, which stays in torch
+    operators; their gradients are returned for it."""
+
+    @staticmethod
+    def forward(ctx, x, w_codes, w_resp, taps, a_scale, a_zp, w_scale, w_zp, bias, a_qmax, stride, padding, dilation):
+        import approx_ops
+        from self_ops.ops_py import approx_ops as ops
+        one = lambda t: t.detach().reshape(1).contiguous()
+        s_a, z_a, s_w, z_w = one(a_scale), one(a_zp), one(w_scale), one(w_zp)
+        xc = x.detach().contiguous()
+        bn, cin, h, w = xc.shape
+        cout, _, kh, kw = w_codes.shape
+        s, p, d = stride[0], padding[0], dilation[0]
+        oh = (h + 2 * p - d * (kh - 1) - 1) // s + 1
+        ow = (w + 2 * p - d * (kw - 1) - 1) // s + 1
+        dev = xc.device
+        codes = torch.empty((bn * h * w, cin), dtype=torch.uint8, device=dev)
+        inside = torch.empty((bn, cin, h, w), dtype=torch.uint8, device=dev)
+        xs = torch.empty((bn, 1, h, w), dtype=torch.float32, device=dev)
+        approx_ops.quantize_codes_nhwc(xc, s_a, z_a, a_qmax, codes, inside, xs)
+        if (kh, kw, s, p) == (1, 1, 1, 0):
+            a_mat = codes                                           # a 1x1 window is the pixel itself
+        else:
+            a_mat = torch.empty((bn * oh * ow, kh * kw * cin), dtype=torch.uint8, device=dev)
+            approx_ops.im2col_nhwc(codes, a_mat, (bn, cin, h, w), (kh, kw), s, p, d)
+        # rows of B in the order of A's columns: (tap, channel)
+        b_mat = w_codes.detach().permute(2, 3, 1, 0).reshape(kh * kw * cin, cout).to(torch.uint8).contiguous()
+        x_sum = _box_sum(xs, (kh, kw), stride, padding, dilation)
+        c_rows = torch.empty((bn * oh * ow, cout), dtype=torch.float32, device=dev)
+        approx_ops.approx_gemm_forward(a_mat, b_mat, c_rows, ops.lut_appmult)
+        out = torch.empty((bn, cout, oh, ow), dtype=torch.float32, device=dev)
+        approx_ops.conv_dequant(c_rows, x_sum.contiguous(), w_resp.detach().contiguous(), taps.contiguous(), z_a, z_w, s_a, s_w,
+                                None if bias is None else bias.detach().contiguous(), out)
+        ctx.save_for_backward(a_mat, b_mat, inside, s_a, z_a, s_w, z_w)
+        ctx.geo = (bn, cin, h, w, cout, kh, kw, s, p, d, oh, ow)
+        ctx.aux = (w_resp.shape, bias is not None, x.dtype)
+        return out
+
+    @staticmethod
+    def backward(ctx, g):
+        import approx_ops
+        from self_ops.ops_py import approx_ops as ops
+        a_mat, b_mat, inside, s_a, z_a, s_w, z_w = ctx.saved_tensors
+        bn, cin, h, w, cout, kh, kw, s, p, d, oh, ow = ctx.geo
+        wr_shape, has_bias, x_dtype = ctx.aux
+        need_x, need_w, need_wr = ctx.needs_input_grad[0], ctx.needs_input_grad[1], ctx.needs_input_grad[2]
+        g = g.contiguous()
+        dev = g.device
+        g_x = g_w = g_wr = g_bias = None
+        if need_x or need_w:
+            g_rows = torch.empty((bn * oh * ow, cout), dtype=torch.float32, device=dev)
+            t = torch.empty(bn * oh * ow, dtype=torch.float32, device=dev)
+            approx_ops.conv_dequant_backward_rowsum(g, s_a, s_w, g_rows, t)
+            # (a gradient nobody asked for -- the images in front of the first layer -- is not computed)
+            g_a = torch.empty((bn, kh * kw * cin, oh * ow), dtype=torch.float32, device=dev) if need_x else None
+            g_b = torch.empty(b_mat.shape, dtype=torch.float32, device=dev) if need_w else None
+            approx_ops.approx_gemm_backward(g_rows, a_mat, b_mat, g_a, g_b, ops.lut_grad_a, ops.lut_grad_b, ga_rows_per_image=oh * ow)
+            if need_x:
+                g_x = torch.empty((bn, cin, h, w), dtype=torch.float32, device=dev)
+                approx_ops.conv_input_grad(g_a, t, z_w, inside, s_a, g_x, (kh, kw), s, p, d)
+                g_x = g_x.to(x_dtype)
+            if need_w:
+                g_w = g_b.view(kh, kw, cin, cout).permute(3, 2, 0, 1)
+        if need_wr:
+            g_wr = ((z_a * (s_a * s_w)) * g.sum(dim=0, keepdim=True)).reshape(wr_shape)
+        if has_bias and ctx.needs_input_grad[8]:
+            g_bias = g.sum(dim=(0, 2, 3))
+        return g_x, g_w, g_wr, None, None, None, None, None, g_bias, None, None, None, None
+
+
 # ------------------------------------------------------------------------------------------ quantiser module
 class AsymmetricQuantizer(nn.Module):
     """Fake quantiser used in front of the pooling layers (reference ``app_layers.py:56-74``; note that its
@@ -277,6 +364,7 @@ class ApproxConv2d(nn.Conv2d, _QuantParamsMixin):
         self.conv2d_op = self_ops.approx_conv2d_baseline_op if use_ste_gradient else self_ops.approx_conv2d_op
         self.reference_zero_point_terms = False     # True: evaluate the three correction terms as full convolutions
         self.fused_dequant = True                   # False: zero-point terms and scaling as torch operators
+        self.fused_layer = True                     # False: float32 code tensors between quantiser, convolution and dequantisation
 
     def quantize_v2(self, x, s, zpn, qmax):
         return _to_codes(x, s, zpn, qmax)
@@ -288,21 +376,22 @@ class ApproxConv2d(nn.Conv2d, _QuantParamsMixin):
         conv(Za*1, Zw*1) = Za*Zw*C * (number of taps inside the image).  All quantities are integer valued,
         so as long as they stay below 2^24 the result is bit-identical to the literal form; autograd sees
         ordinary torch ops and yields the same gradients for the codes."""
-        _, cin, h, w = x_codes.shape
+        kh, kw = w_codes.shape[2], w_codes.shape[3]
+        x_sum = _box_sum(x_codes.sum(dim=1, keepdim=True), (kh, kw), conv_args["stride"], conv_args["padding"], conv_args["dilation"])
+        w_resp, taps = self._weight_zero_point_parts(w_codes, x_codes.shape[1:], conv_args, x_codes.dtype, x_codes.device)
+        return x_sum, w_resp, taps
+
+    def _weight_zero_point_parts(self, w_codes, chw, conv_args, dtype, device):
+        """w_resp [1,N,oh,ow] = conv(all-ones image, W) and taps [1,1,oh,ow] = C * (taps inside the image)."""
+        cin, h, w = chw
         cout, kh, kw = w_codes.shape[0], w_codes.shape[2], w_codes.shape[3]
         s, p, d = conv_args["stride"], conv_args["padding"], conv_args["dilation"]
-        mask = self._tap_mask(h, w, kh, kw, s, p, d, x_codes.dtype, x_codes.device)               # [kh*kw, oh*ow]
+        mask = self._tap_mask(h, w, kh, kw, s, p, d, dtype, device)                                  # [kh*kw, oh*ow]
         oh = (h + 2 * p[0] - d[0] * (kh - 1) - 1) // s[0] + 1
         ow = mask.shape[1] // oh
-        xs = x_codes.sum(dim=1, keepdim=True)
-        if tuple(d) == (1, 1) and 2 * p[0] <= kh and 2 * p[1] <= kw:
-            # box sum with zero padding (no single-channel convolution: the library runs those image by image)
-            x_sum = F.avg_pool2d(xs, (kh, kw), stride=s, padding=p, divisor_override=1)              # [B,1,oh,ow]
-        else:
-            x_sum = F.conv2d(xs, torch.ones(1, 1, kh, kw, dtype=xs.dtype, device=xs.device), **conv_args)
         w_resp = (w_codes.sum(dim=1).reshape(cout, kh * kw) @ mask).view(1, cout, oh, ow)           # [1,N,oh,ow]
         taps = (mask.sum(dim=0) * float(cin)).view(1, 1, oh, ow)
-        return x_sum, w_resp, taps
+        return w_resp, taps
 
     def _tap_mask(self, h, w, kh, kw, stride, padding, dilation, dtype, device):
         """mask[i*kw+j, l] = 1 where tap (i,j) of output position l lies inside the h x w image (constant per
@@ -314,11 +403,25 @@ class ApproxConv2d(nn.Conv2d, _QuantParamsMixin):
             cache[key] = F.unfold(ones, (kh, kw), dilation=dilation, padding=padding, stride=stride)[0]
         return cache[key]
 
+    def _takes_uint8_path(self, input):
+        """The one-operator path on uint8 codes serves the LUT-gradient convolution of float32 CUDA tensors with square
+        geometry (the reference's operator reads element 0 of stride / padding / dilation, ``approx_ops.py:545-547``)."""
+        square = all(len(set(t)) == 1 for t in (self.stride, self.padding, self.dilation)) and not isinstance(self.padding, str)
+        return (self.fused_layer and self.fused_dequant and not self.reference_zero_point_terms and square and self.groups == 1
+                and self.conv2d_op is self_ops.approx_conv2d_op and input.is_cuda and input.dtype == torch.float32
+                and self.weight.dtype == torch.float32 and float(self.activation_quant_max) <= 255
+                and self.activation_scale.is_cuda and self.weight_scale.is_cuda)
+
     def forward(self, input):
         self._update_ranges(input)
         conv_args = dict(bias=None, stride=self.stride, padding=self.padding, dilation=self.dilation, groups=self.groups)
-        x_codes = self.quantize_v2(input, self.activation_scale, self.activation_zp_neg, self.activation_quant_max)
         w_codes = self.quantize_v2(self.weight, self.weight_scale, self.weight_zp_neg, self.weight_quant_max)
+        if self._takes_uint8_path(input):
+            w_resp, taps = self._weight_zero_point_parts(w_codes, input.shape[1:], conv_args, torch.float32, input.device)
+            return _ApproxConvLayerFn.apply(input, w_codes, w_resp, taps, self.activation_scale, self.activation_zp_neg,
+                                            self.weight_scale, self.weight_zp_neg, self.bias, float(self.activation_quant_max),
+                                            tuple(self.stride), tuple(self.padding), tuple(self.dilation))
+        x_codes = self.quantize_v2(input, self.activation_scale, self.activation_zp_neg, self.activation_quant_max)
         total = self.conv2d_op(x_codes, w_codes, **conv_args)       # approximate products of the codes
         if self.reference_zero_point_terms:
             # the reference's literal form: three full convolutions with constant operands

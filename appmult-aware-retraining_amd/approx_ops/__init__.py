@@ -51,6 +51,10 @@ _lib.amr_conv_dequant_backward_f32.argtypes = [_vp, _vp, _vp, _vp, _i, _i, _i, _
 _lib.amr_observer_update_f32.argtypes = [_vp] * 6 + [_i] + [ctypes.c_float] * 5 + [_vp]
 _lib.amr_quantize_codes_f32.argtypes = [_vp, _vp, _vp, ctypes.c_float, _vp, _i64, _vp]
 _lib.amr_quantize_codes_backward_f32.argtypes = [_vp, _vp, _vp, _vp, ctypes.c_float, _vp, _i64, _vp]
+_lib.amr_quantize_codes_nhwc_u8.argtypes = [_vp, _vp, _vp, ctypes.c_float, _vp, _vp, _vp, _i, _i, _i, _vp]
+_lib.amr_im2col_nhwc_u8.argtypes = [_vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp]
+_lib.amr_conv_input_grad_f32.argtypes = [_vp] * 6 + [_i] * 9 + [_vp]
+_lib.amr_conv_dequant_backward_rowsum_f32.argtypes = [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp]
 _lib.amr_lut_gemm_backward_workspace_bytes.argtypes = [_i, _i, _i]
 _lib.amr_lut_gemm_backward_workspace_bytes.restype = _sz
 _lib.amr_lut_gemm_backward_workspace_bytes_for.argtypes = [_i64, _i, _i, _i]
@@ -331,6 +335,94 @@ def quantize_codes_backward(g_tensor, x_tensor, scale_tensor, zp_neg_tensor, qua
                                                   zp_neg_tensor.data_ptr(), float(quant_max), gx_tensor.data_ptr(), x_tensor.numel(),
                                                   _stream_ptr(dev))
     _raise_for(rc, "quantize_codes_backward")
+
+
+def _conv_out_size(H, W, kh, kw, stride, padding, dilation):
+    oh = (H + 2 * padding - dilation * (kh - 1) - 1) // stride + 1
+    ow = (W + 2 * padding - dilation * (kw - 1) - 1) // stride + 1
+    _check(oh > 0 and ow > 0, "empty convolution output")
+    return oh, ow
+
+
+def quantize_codes_nhwc(x_tensor, scale_tensor, zp_neg_tensor, quant_max, codes_tensor, inside_tensor, xsum_tensor):
+    """The quantiser of the reference's quantize_v2 (micronet+/app_layers.py:147-160) writing what the LUT convolution
+    consumes: codes uint8 [B*H*W, C] (a pixel's channel codes adjacent), inside uint8 [B,C,H,W] (the mask of the
+    straight-through backward) and xsum float32 [B*H*W] (a pixel's codes summed over the channels), from x float32 [B,C,H,W]."""
+    for t, name, dt in ((x_tensor, "x_tensor", torch.float32), (scale_tensor, "scale_tensor", torch.float32),
+                        (zp_neg_tensor, "zp_neg_tensor", torch.float32), (codes_tensor, "codes_tensor", torch.uint8),
+                        (inside_tensor, "inside_tensor", torch.uint8), (xsum_tensor, "xsum_tensor", torch.float32)):
+        _check_input(t, dt, name)
+    _check(x_tensor.dim() == 4, "x must be 4-D")
+    Bn, C, H, W = x_tensor.shape
+    _check(scale_tensor.numel() == 1 and zp_neg_tensor.numel() == 1, "scale and zp_neg must hold one element")
+    _check(tuple(codes_tensor.shape) == (Bn * H * W, C), f"codes_tensor's shape should be {Bn * H * W} x {C}")
+    _check(inside_tensor.shape == x_tensor.shape, "inside_tensor must have the shape of x_tensor")
+    _check(xsum_tensor.numel() == Bn * H * W, f"xsum_tensor should have {Bn * H * W} elements")
+    _check(0 <= quant_max <= 255, "quant_max must fit a byte")
+    dev = x_tensor.device
+    _check(all(t.device == dev for t in (scale_tensor, zp_neg_tensor, codes_tensor, inside_tensor, xsum_tensor)), "All tensors should be on the same device")
+    with torch.cuda.device(dev):
+        rc = _lib.amr_quantize_codes_nhwc_u8(x_tensor.data_ptr(), scale_tensor.data_ptr(), zp_neg_tensor.data_ptr(), float(quant_max),
+                                             codes_tensor.data_ptr(), inside_tensor.data_ptr(), xsum_tensor.data_ptr(), Bn, C, H * W,
+                                             _stream_ptr(dev))
+    _raise_for(rc, "quantize_codes_nhwc")
+
+
+def im2col_nhwc(codes_tensor, a_tensor, image_shape, kernel_size, stride, padding, dilation):
+    """a[(b,oy,ox), (i*kw+j)*C + c] = codes[(b, oy*s-p+i*d, ox*s-p+j*d), c] (0 outside the image); codes uint8 [B*H*W, C],
+    image_shape = (B, C, H, W), a uint8 [B*oh*ow, kh*kw*C]."""
+    _check_input(codes_tensor, torch.uint8, "codes_tensor")
+    _check_input(a_tensor, torch.uint8, "a_tensor")
+    Bn, C, H, W = image_shape
+    kh, kw = kernel_size
+    oh, ow = _conv_out_size(H, W, kh, kw, stride, padding, dilation)
+    _check(tuple(codes_tensor.shape) == (Bn * H * W, C), f"codes_tensor's shape should be {Bn * H * W} x {C}")
+    _check(tuple(a_tensor.shape) == (Bn * oh * ow, kh * kw * C), f"a_tensor's shape should be {Bn * oh * ow} x {kh * kw * C}")
+    dev = codes_tensor.device
+    _check(dev == a_tensor.device, "device id not match")
+    with torch.cuda.device(dev):
+        rc = _lib.amr_im2col_nhwc_u8(codes_tensor.data_ptr(), a_tensor.data_ptr(), Bn, C, H, W, kh, kw, stride, padding, dilation,
+                                     _stream_ptr(dev))
+    _raise_for(rc, "im2col_nhwc")
+
+
+def conv_input_grad(cols_tensor, t_tensor, z_w, inside_tensor, scale_tensor, gx_tensor, kernel_size, stride, padding, dilation):
+    """gx = inside ? (col2im(cols) + z_w * window sums of t) / scale : 0 for a tap-major cols float32 [B, kh*kw*C, oh*ow] (None:
+    gx already holds col2im(cols)); t float32 [B*oh*ow]; inside uint8 and gx float32 [B,C,H,W]."""
+    for t, name, dt in ((t_tensor, "t_tensor", torch.float32), (z_w, "z_w", torch.float32), (inside_tensor, "inside_tensor", torch.uint8),
+                        (scale_tensor, "scale_tensor", torch.float32), (gx_tensor, "gx_tensor", torch.float32)):
+        _check_input(t, dt, name)
+    _check(gx_tensor.dim() == 4 and inside_tensor.shape == gx_tensor.shape, "gx must be 4-D and inside of its shape")
+    Bn, C, H, W = gx_tensor.shape
+    kh, kw = kernel_size
+    oh, ow = _conv_out_size(H, W, kh, kw, stride, padding, dilation)
+    if cols_tensor is not None:
+        _check_input(cols_tensor, torch.float32, "cols_tensor")
+        _check(tuple(cols_tensor.shape) == (Bn, kh * kw * C, oh * ow), f"cols_tensor's shape should be {Bn} x {kh * kw * C} x {oh * ow}")
+    _check(t_tensor.numel() == Bn * oh * ow, f"t_tensor should have {Bn * oh * ow} elements")
+    _check(z_w.numel() == 1 and scale_tensor.numel() == 1, "z_w and scale must hold one element")
+    dev = gx_tensor.device
+    with torch.cuda.device(dev):
+        rc = _lib.amr_conv_input_grad_f32(cols_tensor.data_ptr() if cols_tensor is not None else None, t_tensor.data_ptr(), z_w.data_ptr(),
+                                          inside_tensor.data_ptr(), scale_tensor.data_ptr(), gx_tensor.data_ptr(), Bn, C, H, W, kh, kw,
+                                          stride, padding, dilation, _stream_ptr(dev))
+    _raise_for(rc, "conv_input_grad")
+
+
+def conv_dequant_backward_rowsum(g_tensor, s_a, s_w, gc_rows, t_tensor):
+    """conv_dequant_backward that also leaves t[m] = sum over n of gc_rows[m, n] (float32 [B*L])."""
+    for t, name in ((g_tensor, "g_tensor"), (s_a, "s_a"), (s_w, "s_w"), (gc_rows, "gc_rows"), (t_tensor, "t_tensor")):
+        _check_input(t, torch.float32, name)
+    _check(g_tensor.dim() == 4 and gc_rows.dim() == 2, "g must be 4-D and gc_rows 2-D")
+    Bn, N = g_tensor.size(0), g_tensor.size(1)
+    L = g_tensor.size(2) * g_tensor.size(3)
+    _check(tuple(gc_rows.shape) == (Bn * L, N), f"gc_rows's shape should be {Bn * L} x {N}")
+    _check(t_tensor.numel() == Bn * L, f"t_tensor should have {Bn * L} elements")
+    dev = g_tensor.device
+    with torch.cuda.device(dev):
+        rc = _lib.amr_conv_dequant_backward_rowsum_f32(g_tensor.data_ptr(), s_a.data_ptr(), s_w.data_ptr(), gc_rows.data_ptr(),
+                                                       t_tensor.data_ptr(), Bn, N, L, _stream_ptr(dev))
+    _raise_for(rc, "conv_dequant_backward_rowsum")
 
 
 def lds_gather_probe(pattern=0, waves_per_cu=16, iters=4000):

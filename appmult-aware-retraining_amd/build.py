@@ -14,7 +14,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "libamr_lutgemm.so")
-SOURCES = ["lutgemm_fwd.hip", "lutgemm_fwd_slab.hip", "lutgemm_bwd.hip", "lutgemm_bwd_f32tab.hip", "lutgemm_bwd_slab.hip", "lutgemm_bwd_slab8.hip", "lutgemm_gradA_slab.hip", "lutgemm_gradA_rows8.hip", "accgemm.hip", "im2col.hip", "quantize.hip", "fill.hip", "dequant.hip", "lds_probe.hip", "capi.hip"]
+SOURCES = ["lutgemm_fwd.hip", "lutgemm_fwd_slab.hip", "lutgemm_bwd.hip", "lutgemm_bwd_f32tab.hip", "lutgemm_bwd_slab.hip", "lutgemm_bwd_slab8.hip", "lutgemm_gradA_slab.hip", "lutgemm_gradA_rows8.hip", "accgemm.hip", "im2col.hip", "quantize.hip", "fill.hip", "dequant.hip", "conv_glue.hip", "lds_probe.hip", "capi.hip"]
 HEADERS = [os.path.join(CSRC, "amr_common.h"), os.path.join(HERE, "..", "include", "amr_lutgemm.h")]
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++20", "-fPIC", "-Wall",
          # packed-fp32 VALU forms are switched off for every device translation unit

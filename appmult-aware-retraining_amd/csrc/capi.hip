@@ -92,6 +92,15 @@ hipError_t launch_gradA_slab_f32w(const float* gC, const uint8_t* A, const uint8
 hipError_t launch_gradA_slab_f32tab(const float* gC, const uint8_t* A, const uint8_t* B, float* gA, const float* lut,
                                     const LutGeom& g, int M, int K, int N, float scale, int n_cu, uint32_t* flags, void* S,
                                     int rows_per_image, hipStream_t stream);
+hipError_t launch_quantize_nhwc(const float* x, const float* scale, const float* zp_neg, float qmax, uint8_t* codes, uint8_t* inside,
+                                float* xs, long B, int C, int L, hipStream_t stream);
+hipError_t launch_im2col_nhwc(const uint8_t* codes, uint8_t* A, long B, int C, int H, int W, int kh, int kw, int stride, int pad,
+                              int dil, int oh, int ow, hipStream_t stream);
+hipError_t launch_conv_input_grad(const float* cols, const float* t, const float* zw, const uint8_t* inside, const float* scale,
+                                  float* gx, long B, int C, int H, int W, int kh, int kw, int stride, int pad, int dil, int oh, int ow,
+                                  hipStream_t stream);
+hipError_t launch_dequant_grad_rowsum(const float* g, const float* sa, const float* sw, float* gc, float* t, int M, int N, int L,
+                                      hipStream_t stream);
 hipError_t launch_accgemm(const float* A, const float* B, float* C, int M, int K, int N, hipStream_t stream);
 hipError_t run_lds_probe(int pattern, int waves_per_cu, int iters, int n_cu, float* ms_out, double* gathers_out,
                          hipStream_t stream);
@@ -699,6 +708,57 @@ int amr_quantize_codes_backward_f32(const float* g, const float* x, const float*
     if (!g || !x || !scale || !zp_neg || !gx) return fail(AMR_EINVAL, "null pointer argument");
     hipError_t e = amr::launch_quantize_codes_backward(g, x, scale, zp_neg, qmax, gx, (size_t)n, reinterpret_cast<hipStream_t>(stream));
     return e == hipSuccess ? AMR_OK : hip_fail(e, "quantize backward launch");
+}
+
+static bool conv_geometry(int C, int H, int W, int kh, int kw, int stride, int pad, int dil, int* oh, int* ow) {
+    if (C <= 0 || H <= 0 || W <= 0 || kh <= 0 || kw <= 0 || stride <= 0 || pad < 0 || dil <= 0) return false;
+    *oh = (H + 2 * pad - dil * (kh - 1) - 1) / stride + 1;
+    *ow = (W + 2 * pad - dil * (kw - 1) - 1) / stride + 1;
+    return *oh > 0 && *ow > 0;
+}
+
+int amr_quantize_codes_nhwc_u8(const float* x, const float* scale, const float* zp_neg, float qmax, uint8_t* codes, uint8_t* inside,
+                               float* x_sum, int B, int C, int L, void* stream) {
+    if (B < 0 || C <= 0 || L <= 0 || !(qmax >= 0.f) || qmax > 255.f) return fail(AMR_EINVAL, "bad shape or code range");
+    if (B == 0) return AMR_OK;
+    if ((long)B * L >= (1L << 31)) return fail(AMR_EUNSUPPORTED, "more than 2^31 pixels");
+    if (!x || !scale || !zp_neg || !codes || !inside || !x_sum) return fail(AMR_EINVAL, "null pointer argument");
+    hipError_t e = amr::launch_quantize_nhwc(x, scale, zp_neg, qmax, codes, inside, x_sum, B, C, L, reinterpret_cast<hipStream_t>(stream));
+    return e == hipSuccess ? AMR_OK : hip_fail(e, "quantize launch");
+}
+
+int amr_im2col_nhwc_u8(const uint8_t* codes, uint8_t* A, int B, int C, int H, int W, int kh, int kw, int stride, int pad, int dil,
+                       void* stream) {
+    int oh, ow;
+    if (B < 0 || !conv_geometry(C, H, W, kh, kw, stride, pad, dil, &oh, &ow)) return fail(AMR_EINVAL, "bad convolution geometry");
+    if (B == 0) return AMR_OK;
+    if ((long)B * oh * ow >= (1L << 31)) return fail(AMR_EUNSUPPORTED, "more than 2^31 output positions");
+    if (!codes || !A) return fail(AMR_EINVAL, "null pointer argument");
+    hipError_t e = amr::launch_im2col_nhwc(codes, A, B, C, H, W, kh, kw, stride, pad, dil, oh, ow, reinterpret_cast<hipStream_t>(stream));
+    return e == hipSuccess ? AMR_OK : hip_fail(e, "im2col launch");
+}
+
+int amr_conv_input_grad_f32(const float* cols, const float* t, const float* z_w, const uint8_t* inside, const float* scale, float* gx,
+                            int B, int C, int H, int W, int kh, int kw, int stride, int pad, int dil, void* stream) {
+    int oh, ow;
+    if (B < 0 || !conv_geometry(C, H, W, kh, kw, stride, pad, dil, &oh, &ow)) return fail(AMR_EINVAL, "bad convolution geometry");
+    if (B == 0) return AMR_OK;
+    if ((size_t)B * C * H * W >= ((size_t)1 << 40)) return fail(AMR_EUNSUPPORTED, "more than 2^40 pixels");
+    if (!t || !z_w || !inside || !scale || !gx) return fail(AMR_EINVAL, "null pointer argument");
+    hipError_t e = amr::launch_conv_input_grad(cols, t, z_w, inside, scale, gx, B, C, H, W, kh, kw, stride, pad, dil, oh, ow,
+                                               reinterpret_cast<hipStream_t>(stream));
+    return e == hipSuccess ? AMR_OK : hip_fail(e, "input gradient launch");
+}
+
+int amr_conv_dequant_backward_rowsum_f32(const float* g, const float* s_a, const float* s_w, float* g_c, float* t, int batch,
+                                         int out_channels, int positions, void* stream) {
+    if (batch < 0 || out_channels <= 0 || positions <= 0) return fail(AMR_EINVAL, "bad shape");
+    if (batch == 0) return AMR_OK;
+    if ((long)batch * positions >= (1L << 31)) return fail(AMR_EUNSUPPORTED, "more than 2^31 output positions");
+    if (!g || !s_a || !s_w || !g_c || !t) return fail(AMR_EINVAL, "null pointer argument");
+    hipError_t e = amr::launch_dequant_grad_rowsum(g, s_a, s_w, g_c, t, batch * positions, out_channels, positions,
+                                                   reinterpret_cast<hipStream_t>(stream));
+    return e == hipSuccess ? AMR_OK : hip_fail(e, "dequant backward launch");
 }
 
 int amr_acc_gemm_forward_fp32(const float* A, const float* B, float* C, int M, int K, int N, void* stream) {

@@ -244,6 +244,42 @@ int amr_quantize_codes_backward_f32(const float *g, const float *x, const float 
                                     float qmax, float *gx, int64_t n, void *stream);
 
 /*
+ * The same quantiser producing what the LUT convolution consumes, with no float32 code tensor in between (the reference
+ * keeps the codes as float32 and casts them in front of the GEMM, micronet+/app_layers.py:172-173 ->
+ * self_ops/ops_py/approx_ops.py:161-164):
+ *   codes  [B*L, C] uint8, "pixel-major": the C codes of pixel m = b*L + pix are adjacent (L = H*W)
+ *   inside [B, C, L] uint8: 1 where the rounded value lay in [0, qmax] -- all the straight-through backward of the clamp
+ *          needs (amr_conv_input_grad_f32), so that x is not read again
+ *   x_sum  [B*L] float32: sum of a pixel's codes over the channels, the operand of the zero-point term conv(X, Zw)
+ * x is [B, C, L] float32; qmax <= 255.  A NaN input gives code 0, inside 0.
+ */
+int amr_quantize_codes_nhwc_u8(const float *x, const float *scale, const float *zp_neg, float qmax, uint8_t *codes,
+                               uint8_t *inside, float *x_sum, int B, int C, int L, void *stream);
+
+/*
+ * im2col of pixel-major codes: A [B*oh*ow, kh*kw*C] uint8, row (b,oy,ox), column (i*kw + j)*C + c ("tap-major": the
+ * order of the GEMM's k index is free as long as the rows of B follow it; the reference's is c*kh*kw + i*kw + j,
+ * self_ops/ops_py/approx_ops.py:556-563), padding positions = code 0.  A window row is kh*kw runs of C adjacent bytes.
+ */
+int amr_im2col_nhwc_u8(const uint8_t *codes, uint8_t *A, int B, int C, int H, int W, int kh, int kw, int stride, int pad,
+                       int dil, void *stream);
+
+/*
+ * Input gradient of the quantised LUT convolution in one pass: the adjoint of amr_im2col_nhwc_u8, the gradient of the
+ * zero-point term conv(X, Zw) and the quantiser's straight-through backward (micronet+/app_layers.py:147-160,175-181):
+ *   gx[b,c,y,x] = inside[b,c,y,x] ? (sum over taps of cols[b][tap*C + c][pos(tap)] + *z_w * sum over taps of t[b][pos(tap)]) / *scale : 0
+ * cols [B][kh*kw*C][oh*ow] float32 is what amr_lut_gemm_backward_ex writes with ga_rows_per_image = oh*ow for a tap-major A;
+ * cols = NULL: gx already holds the sum over the taps and is finished in place.  t [B][oh*ow] = the row sums of the
+ * GEMM's output gradient (amr_conv_dequant_backward_rowsum_f32); z_w, scale: device scalars.  Fixed summation order.
+ */
+int amr_conv_input_grad_f32(const float *cols, const float *t, const float *z_w, const uint8_t *inside, const float *scale,
+                            float *gx, int B, int C, int H, int W, int kh, int kw, int stride, int pad, int dil, void *stream);
+
+/* amr_conv_dequant_backward_f32 that also leaves t[m] = sum over n of g_c[m, n] (ascending n), in the same pass. */
+int amr_conv_dequant_backward_rowsum_f32(const float *g, const float *s_a, const float *s_w, float *g_c, float *t, int batch,
+                                         int out_channels, int positions, void *stream);
+
+/*
  * Accurate fp32 GEMM  C = A . B  (row-major), kept for API parity only.
  * Replaces acc_gemm_forward_fp32_gpu (self_ops/src/approx_gemm_forward.cu:494-571), bound as
  * approx_ops.acc_gemm_forward_fp32 (self_ops/src/op_register.cpp:18).

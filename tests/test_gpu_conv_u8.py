@@ -1,0 +1,182 @@
+"""GPU tests of the quantised LUT convolution on uint8 codes: the pixel-major quantiser, the tap-major im2col, the fused
+input-gradient pass, the output-gradient pass with row sums and the layer operator built from them, each against the
+unfused composition (float32 code tensors and torch operators) and against the CPU oracle."""
+import os
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ops(golden_dir):
+    import self_ops
+    from self_ops.ops_py import approx_ops as P
+    P.init_lookup_tables(torch.device("cuda"), os.path.join(golden_dir, "lut7_resub_63_bp8.txt.gz"), 7)
+    return self_ops, P
+
+
+def out_size(h, w, k, s, p, d):
+    return (h + 2 * p - d * (k - 1) - 1) // s + 1, (w + 2 * p - d * (k - 1) - 1) // s + 1
+
+
+@pytest.mark.parametrize("shape", [(4, 3, 5, 5), (2, 16, 8, 8), (3, 64, 32, 32), (2, 528, 4, 4), (1, 20, 3, 7), (130, 32, 1, 1)])
+def test_pixel_major_quantiser_equals_float_quantiser(ops, shape):
+    """Codes, in-range mask and channel sums of the uint8 quantiser against the float32 quantiser and its backward
+    (themselves pinned against the torch expression of the reference's quantize_v2): same codes at every element, the mask
+    is where the straight-through gradient passes, the sums are the codes added over the channels."""
+    import app_layers
+    import approx_ops
+    print("quantiser nhwc", shape, flush=True)
+    g = torch.Generator(device="cuda").manual_seed(5)
+    x = torch.randn(shape, device="cuda", generator=g) * 3
+    x.view(-1)[::5] = (torch.arange(x.numel(), device="cuda")[::5] % 200 - 30).float() * 0.05 + 0.025      # ties after scaling
+    x.view(-1)[1], x.view(-1)[x.numel() // 2], x.view(-1)[-2] = float("nan"), float("inf"), float("-inf")
+    scale, zp = torch.tensor([0.05], device="cuda"), torch.tensor([-17.0], device="cuda")
+    bn, c, h, w = shape
+    codes = torch.full((bn * h * w, c), 255, dtype=torch.uint8, device="cuda")
+    inside = torch.full(shape, 7, dtype=torch.uint8, device="cuda")
+    xs = torch.full((bn * h * w,), float("nan"), device="cuda")
+    approx_ops.quantize_codes_nhwc(x, scale, zp, 127.0, codes, inside, xs)
+    xr = x.clone().requires_grad_()
+    want = app_layers._to_codes(xr, scale, zp, 127.0)
+    want.backward(torch.ones_like(want))
+    finite = ~torch.isnan(want.detach())
+    want_u8 = torch.where(finite, want.detach(), torch.zeros_like(want)).to(torch.uint8)       # a NaN: code 0 (documented)
+    got = codes.view(bn, h, w, c).permute(0, 3, 1, 2)
+    assert torch.equal(got, want_u8)
+    passes = torch.nan_to_num(xr.grad, nan=0.0) != 0
+    assert torch.equal(inside.bool(), passes)
+    assert int((~finite).sum()) == 3 and not inside.bool()[~finite].any()
+    assert torch.equal(xs.view(bn, h, w), want_u8.float().sum(dim=1))
+
+
+@pytest.mark.parametrize("shape,k,stride,padding,dilation", [
+    ((3, 5, 10, 10), 3, 1, 1, 1), ((2, 4, 9, 7), 3, 2, 1, 1), ((2, 16, 12, 12), 1, 2, 0, 1), ((1, 3, 16, 16), 7, 2, 3, 1),
+    ((2, 6, 11, 11), 3, 1, 2, 2), ((2, 64, 8, 8), 3, 1, 1, 1), ((3, 32, 16, 16), 3, 2, 1, 1), ((2, 48, 5, 5), 1, 1, 0, 1)])
+def test_tap_major_im2col_against_oracle(ops, oracle, shape, k, stride, padding, dilation):
+    """The uint8 im2col of pixel-major codes against the oracle's window matrix (reference column order c*kh*kw + tap),
+    columns permuted to the tap-major order."""
+    import approx_ops
+    print("im2col nhwc", shape, k, stride, padding, dilation, flush=True)
+    rng = np.random.default_rng(12)
+    x = rng.integers(0, 256, shape).astype(np.uint8)
+    bn, c, h, w = shape
+    want, oh, ow = oracle.im2col_np(x, k, k, stride, padding, dilation)
+    want = want.reshape(-1, c, k * k).transpose(0, 2, 1).reshape(-1, k * k * c)
+    codes = torch.tensor(x, device="cuda").permute(0, 2, 3, 1).reshape(bn * h * w, c).contiguous()
+    a = torch.full(want.shape, 77, dtype=torch.uint8, device="cuda")
+    approx_ops.im2col_nhwc(codes, a, shape, (k, k), stride, padding, dilation)
+    assert (a.cpu().numpy() == want).all()
+
+
+@pytest.mark.parametrize("shape,k,stride,padding,dilation", [
+    ((3, 5, 10, 10), 3, 1, 1, 1), ((2, 4, 9, 7), 3, 2, 1, 1), ((2, 8, 12, 12), 1, 2, 0, 1), ((1, 3, 16, 16), 7, 2, 3, 1),
+    ((2, 6, 11, 11), 3, 1, 2, 2), ((2, 64, 8, 8), 3, 1, 1, 1), ((4, 16, 32, 32), 3, 1, 1, 1), ((2, 32, 6, 6), 1, 1, 0, 1)])
+def test_fused_input_gradient_equals_fold_plus_torch_operators(ops, shape, k, stride, padding, dilation):
+    """gx = inside ? (fold(cols) + z_w * fold of the row sums spread over the taps) / scale : 0 against torch's fold in
+    float64; with cols = None the kernel finishes a tensor that already holds fold(cols)."""
+    import approx_ops
+    print("input gradient", shape, k, stride, padding, dilation, flush=True)
+    bn, c, h, w = shape
+    oh, ow = out_size(h, w, k, stride, padding, dilation)
+    g = torch.Generator(device="cuda").manual_seed(2)
+    cols_tap = torch.randn(bn, k * k * c, oh * ow, device="cuda", generator=g)               # tap-major k
+    t = torch.randn(bn * oh * ow, device="cuda", generator=g)
+    inside = (torch.rand(shape, device="cuda", generator=g) < 0.8).to(torch.uint8)
+    zw, scale = torch.tensor([-61.0], device="cuda"), torch.tensor([0.037], device="cuda")
+    gx = torch.full(shape, float("nan"), device="cuda")
+    approx_ops.conv_input_grad(cols_tap, t, zw, inside, scale, gx, (k, k), stride, padding, dilation)
+    cols_ref = cols_tap.view(bn, k * k, c, oh * ow).transpose(1, 2).reshape(bn, c * k * k, oh * ow).double()
+    fold = lambda cc: F.fold(cc, (h, w), (k, k), dilation=dilation, padding=padding, stride=stride)
+    t_cols = t.double().view(bn, 1, oh * ow).expand(bn, k * k, oh * ow)
+    want = (fold(cols_ref) + zw.double() * fold(t_cols)) / scale.double() * inside.double()
+    torch.testing.assert_close(gx.double(), want, rtol=0, atol=2e-6 * float(want.abs().max()))
+    assert (gx[inside == 0] == 0).all()
+    # finishing in place what a convolution-shaped gradA left
+    raw = fold(cols_ref).float().contiguous()
+    approx_ops.conv_input_grad(None, t, zw, inside, scale, raw, (k, k), stride, padding, dilation)
+    torch.testing.assert_close(raw.double(), want, rtol=0, atol=2e-6 * float(want.abs().max()))
+
+
+@pytest.mark.parametrize("bn,n,hw", [(3, 40, (5, 7)), (2, 64, (16, 16)), (130, 10, (1, 1)), (1, 33, (9, 9)), (4, 128, (8, 8))])
+def test_output_gradient_rows_with_row_sums(ops, bn, n, hw):
+    import approx_ops
+    print("dequant backward rowsum", bn, n, hw, flush=True)
+    g = torch.randn(bn, n, *hw, device="cuda")
+    sa, sw = torch.tensor([0.031], device="cuda"), torch.tensor([0.0077], device="cuda")
+    L = hw[0] * hw[1]
+    rows = torch.full((bn * L, n), float("nan"), device="cuda")
+    rows2 = torch.full((bn * L, n), float("nan"), device="cuda")
+    t = torch.full((bn * L,), float("nan"), device="cuda")
+    approx_ops.conv_dequant_backward_rowsum(g, sa, sw, rows, t)
+    approx_ops.conv_dequant_backward(g, sa, sw, rows2)
+    assert torch.equal(rows, rows2)
+    assert torch.equal(rows, ((sa * sw) * g).permute(0, 2, 3, 1).reshape(bn * L, n))
+    want = rows.double().sum(dim=1)
+    torch.testing.assert_close(t.double(), want, rtol=0, atol=1e-6 * float(rows.abs().sum(dim=1).max()))
+
+
+@pytest.mark.parametrize("cin,cout,k,stride,padding,dilation,hw,bias", [
+    (16, 24, 3, 1, 1, 1, 12, True),        # 3x3 same-size convolution, 16-byte code runs
+    (5, 7, 3, 1, 1, 1, 9, True),           # channel count that takes the byte path
+    (32, 40, 1, 1, 0, 1, 8, False),        # 1x1: the codes are the operand matrix
+    (16, 33, 1, 2, 0, 1, 8, False),        # 1x1 stride-2 shortcut
+    (6, 40, 3, 2, 1, 1, 9, True),          # 3x3 stride 2
+    (8, 12, 3, 1, 2, 2, 10, True),         # dilation
+    (3, 64, 3, 1, 1, 1, 32, True),         # first layer of the network
+])
+def test_uint8_layer_path_equals_float_code_path_and_oracle(ops, oracle, golden_dir, cin, cout, k, stride, padding, dilation, hw, bias):
+    """ApproxConv2d on the uint8 path (one operator, no float32 code tensor) against the same layer on float32 code
+    tensors and torch operators: identical outputs, gradients to summation order; and the output against the four-term
+    expression of the reference (app_layers.py:175-183) evaluated with the oracle's LUT convolution in float64."""
+    import app_layers as L
+    self_ops, P = ops
+    print("uint8 layer path", cin, cout, k, stride, padding, dilation, hw, flush=True)
+    torch.manual_seed(7)
+    layer = L.ApproxConv2d(cin, cout, k, stride=stride, padding=padding, dilation=dilation, bias=bias, a_bits=7, w_bits=7).cuda().train()
+    x = torch.randn(4, cin, hw, hw, device="cuda") * 2 + 0.3
+    layer(x)                                          # one training pass sets the ranges
+    layer.eval()                                      # frozen observers: both paths see the same scales
+    gy = None
+    res = []
+    for fused in (True, False):
+        layer.fused_layer = fused
+        xi = x.clone().requires_grad_()
+        layer.zero_grad()
+        y = layer(xi)
+        if gy is None:
+            gy = torch.randn_like(y)
+        y.backward(gy)
+        res.append((y.detach(), xi.grad, layer.weight.grad.clone(), layer.bias.grad.clone() if bias else None))
+    assert layer._takes_uint8_path(x) is False
+    layer.fused_layer = True
+    assert layer._takes_uint8_path(x) is True
+    assert res[0][0].is_contiguous() and torch.equal(res[0][0], res[1][0])
+    for a, b in zip(res[0][1:], res[1][1:]):
+        if a is not None:
+            torch.testing.assert_close(a, b, rtol=1e-5, atol=2e-6 * float(b.abs().max()))
+    # the reference's expression with the oracle's LUT convolution
+    s_a, z_a, s_w, z_w = (float(t) for t in (layer.activation_scale, layer.activation_zp_neg, layer.weight_scale, layer.weight_zp_neg))
+    xc = L._to_codes_torch(x, layer.activation_scale, layer.activation_zp_neg, 127.0)
+    wc = L._to_codes_torch(layer.weight.detach(), layer.weight_scale, layer.weight_zp_neg, 127.0)
+    fwd2d = oracle.unpack_table(P.lut_appmult.cpu().numpy(), 7)
+    am = oracle.conv2d_lut_np(xc.cpu().numpy().astype(np.uint8), wc.cpu().numpy().astype(np.uint8), fwd2d, stride, padding, dilation)
+    conv = lambda a, b: F.conv2d(a.double(), b.double(), stride=stride, padding=padding, dilation=dilation)
+    total = (torch.tensor(am.astype(np.float64), device="cuda") + conv(xc, torch.full_like(wc, z_w)) + conv(torch.full_like(xc, z_a), wc)
+             + conv(torch.full_like(xc, z_a), torch.full_like(wc, z_w)))
+    want = s_a * s_w * total + (layer.bias.detach().double().view(1, -1, 1, 1) if bias else 0.0)
+    torch.testing.assert_close(res[0][0].double(), want, rtol=1e-5, atol=1e-5 * float(want.abs().max()))
+
+
+def test_uint8_layer_path_first_layer_needs_no_input_gradient(ops):
+    import app_layers as L
+    torch.manual_seed(1)
+    layer = L.ApproxConv2d(3, 16, 3, padding=1, bias=False, a_bits=7, w_bits=7).cuda().train()
+    x = torch.randn(2, 3, 8, 8, device="cuda")
+    y = layer(x)
+    y.square().mean().backward()
+    assert layer.weight.grad is not None and torch.isfinite(layer.weight.grad).all()
