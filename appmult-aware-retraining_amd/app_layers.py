@@ -224,11 +224,11 @@ class _ApproxConvLayerFn(torch.autograd.Function):
         # rows of B in the order of A's columns: (tap, channel)
         b_mat = w_codes.detach().permute(2, 3, 1, 0).reshape(kh * kw * cin, cout).to(torch.uint8).contiguous()
         x_sum = _box_sum(xs, (kh, kw), stride, padding, dilation)
-        c_rows = torch.empty((bn * oh * ow, cout), dtype=torch.float32, device=dev)
-        approx_ops.approx_gemm_forward(a_mat, b_mat, c_rows, ops.lut_appmult)
         out = torch.empty((bn, cout, oh, ow), dtype=torch.float32, device=dev)
-        approx_ops.conv_dequant(c_rows, x_sum.contiguous(), w_resp.detach().contiguous(), taps.contiguous(), z_a, z_w, s_a, s_w,
-                                None if bias is None else bias.detach().contiguous(), out)
+        # (LUT GEMM whose store applies the zero-point terms, the scaling and the bias and writes NCHW)
+        approx_ops.approx_conv_forward_dequant(a_mat, b_mat, ops.lut_appmult, x_sum.contiguous(), w_resp.detach().contiguous(),
+                                               taps.contiguous(), z_a, z_w, s_a, s_w,
+                                               None if bias is None else bias.detach().contiguous(), out)
         ctx.save_for_backward(a_mat, b_mat, inside, s_a, z_a, s_w, z_w)
         ctx.geo = (bn, cin, h, w, cout, kh, kw, s, p, d, oh, ow)
         ctx.aux = (w_resp.shape, bias is not None, x.dtype)

@@ -51,6 +51,9 @@ _lib.amr_conv_dequant_backward_f32.argtypes = [_vp, _vp, _vp, _vp, _i, _i, _i, _
 _lib.amr_observer_update_f32.argtypes = [_vp] * 6 + [_i] + [ctypes.c_float] * 5 + [_vp]
 _lib.amr_quantize_codes_f32.argtypes = [_vp, _vp, _vp, ctypes.c_float, _vp, _i64, _vp]
 _lib.amr_quantize_codes_backward_f32.argtypes = [_vp, _vp, _vp, _vp, ctypes.c_float, _vp, _i64, _vp]
+_lib.amr_lut_conv_forward_dequant_workspace_bytes.argtypes = [_i64, _i, _i, _i]
+_lib.amr_lut_conv_forward_dequant_workspace_bytes.restype = _sz
+_lib.amr_lut_conv_forward_dequant_f32.argtypes = [_vp, _vp, _vp, _i64, _i, _i, _i, _i] + [_vp] * 9 + [_vp, _sz, _vp]
 _lib.amr_quantize_codes_nhwc_u8.argtypes = [_vp, _vp, _vp, ctypes.c_float, _vp, _vp, _vp, _i, _i, _i, _vp]
 _lib.amr_im2col_nhwc_u8.argtypes = [_vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp]
 _lib.amr_conv_input_grad_f32.argtypes = [_vp] * 6 + [_i] * 9 + [_vp]
@@ -273,6 +276,39 @@ def conv_dequant(c_rows, x_sum, w_resp, taps, z_a, z_w, s_a, s_w, bias, out_tens
                                        z_w.data_ptr(), s_a.data_ptr(), s_w.data_ptr(), bias.data_ptr() if bias is not None else None,
                                        out_tensor.data_ptr(), Bn, N, L, _stream_ptr(dev))
     _raise_for(rc, "conv_dequant")
+
+
+def approx_conv_forward_dequant(a_tensor, b_tensor, lut_appmult_tensor, x_sum, w_resp, taps, z_a, z_w, s_a, s_w, bias, out_tensor):
+    """approx_gemm_forward followed by conv_dequant without the sums going to memory: out float32 [B, N, oh, ow] from the uint8
+    operand matrices a [B*L, K], b [K, N] (any common order of k) and the operands of conv_dequant."""
+    _check_input(a_tensor, torch.uint8, "a_tensor")
+    _check_input(b_tensor, torch.uint8, "b_tensor")
+    _check_input(lut_appmult_tensor, torch.uint16, "lut_appmult_tensor")
+    tensors = [(x_sum, "x_sum"), (w_resp, "w_resp"), (taps, "taps"), (z_a, "z_a"), (z_w, "z_w"), (s_a, "s_a"), (s_w, "s_w"),
+               (out_tensor, "out_tensor")] + ([(bias, "bias")] if bias is not None else [])
+    for t, name in tensors:
+        _check_input(t, torch.float32, name)
+    _check(a_tensor.dim() == 2 and b_tensor.dim() == 2 and out_tensor.dim() == 4, "a and b must be 2-D, out 4-D")
+    M, K = a_tensor.shape
+    N = b_tensor.size(1)
+    Bn, L = out_tensor.size(0), out_tensor.size(2) * out_tensor.size(3)
+    _check(K == b_tensor.size(0), f"b_tensor's shape should be {K} x {N}")
+    _check(out_tensor.size(1) == N and Bn * L == M, f"out_tensor should hold {M} positions of {N} channels")
+    _check(x_sum.numel() == M and w_resp.numel() == N * L and taps.numel() == L, "x_sum, w_resp or taps has the wrong size")
+    _check(all(t.numel() == 1 for t in (z_a, z_w, s_a, s_w)), "z_a, z_w, s_a and s_w must hold one element")
+    _check(bias is None or bias.numel() == N, f"bias should have {N} elements")
+    _lut_len_check(lut_appmult_tensor, "lut_appmult_tensor")
+    dev = a_tensor.device
+    _check(all(t.device == dev for t, _ in tensors) and b_tensor.device == dev and lut_appmult_tensor.device == dev, "device id not match")
+    with torch.cuda.device(dev):
+        need = _lib.amr_lut_conv_forward_dequant_workspace_bytes(lut_appmult_tensor.size(0), M, K, N)
+        ws = torch.empty(max(need, 256), dtype=torch.uint8, device=dev)
+        rc = _lib.amr_lut_conv_forward_dequant_f32(a_tensor.data_ptr(), b_tensor.data_ptr(), lut_appmult_tensor.data_ptr(),
+                                                   lut_appmult_tensor.size(0), M, K, N, L, x_sum.data_ptr(), w_resp.data_ptr(),
+                                                   taps.data_ptr(), z_a.data_ptr(), z_w.data_ptr(), s_a.data_ptr(), s_w.data_ptr(),
+                                                   bias.data_ptr() if bias is not None else None, out_tensor.data_ptr(), ws.data_ptr(),
+                                                   ws.numel(), _stream_ptr(dev))
+    _raise_for(rc, "approx_conv_forward_dequant")
 
 
 def conv_dequant_backward(g_tensor, s_a, s_w, gc_rows):

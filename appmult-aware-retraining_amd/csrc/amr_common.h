@@ -58,6 +58,21 @@ inline hipError_t allow_full_lds(const void* kernel, std::atomic<uint64_t>& done
     return e;
 }
 
+// Operands of the dequantising store (the zero-point terms, scaling and bias of the reference's ApproxConv2d.forward,
+// micronet+/app_layers.py:175-183, see dequant.hip): out == nullptr selects the plain store.
+struct SlabDequant {
+    const float* xs;      // [M] box sums of the input codes
+    const float* wr;      // [N][L] response of the weight codes to an all-ones image
+    const float* tp;      // [L] taps inside the image x input channels
+    const float* za;      // device scalars
+    const float* zw;
+    const float* sa;
+    const float* sw;
+    const float* bias;    // [N] or nullptr
+    float* out;           // [M / L][N][L]
+    int L;                // positions per image
+};
+
 __device__ __forceinline__ int uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
 
 // Four consecutive bytes starting at an arbitrary byte address (global memory accepts unaligned

@@ -16,7 +16,9 @@ hipError_t launch_fwd(const uint8_t* A, const uint8_t* B, uint32_t* C, const uin
                       int K, int N, int n_cu, hipStream_t stream, int out_f32);
 size_t fwd_slab_workspace_bytes(const LutGeom& g, int M, int K, int N, bool force);
 hipError_t launch_fwd_slab(const uint8_t* A, const uint8_t* B, uint32_t* C, const uint16_t* lut, const LutGeom& g,
-                           int M, int K, int N, int n_cu, void* workspace, hipStream_t stream, int out_f32);
+                           int M, int K, int N, int n_cu, void* workspace, hipStream_t stream, int out_f32,
+                           const SlabDequant* dq = nullptr);
+bool fwd_slab_can_dequant(const LutGeom& g, int M, int K, int N, int n_cu, bool force);
 size_t gradB_workspace_bytes(int M, int K, int N, int n_cu);
 hipError_t launch_gradB(const float* gC, const uint8_t* A, const uint8_t* B, float* gB, const int16_t* lut,
                         const LutGeom& g, int M, int K, int N, float scale, void* workspace, int n_cu,
@@ -292,6 +294,51 @@ static int forward_impl(const uint8_t* A, const uint8_t* B, uint32_t* C, const u
         e = amr::launch_fwd(A, B, C, lut, g, M, K, N, n_cu, s, out_f32);
     }
     return e == hipSuccess ? AMR_OK : hip_fail(e, "forward launch");
+}
+
+size_t amr_lut_conv_forward_dequant_workspace_bytes(int64_t lut_elems, int M, int K, int N) {
+    if (M <= 0 || N <= 0) return 0;
+    // [the expanded table of the forward pass, if this shape takes it][float32 sums, M x N]
+    const size_t e = (amr_lut_gemm_forward_workspace_bytes(lut_elems, M, K, N) + 255) & ~(size_t)255;
+    return e + (size_t)M * N * sizeof(float);
+}
+
+int amr_lut_conv_forward_dequant_f32(const uint8_t* A, const uint8_t* B, const uint16_t* lut, int64_t lut_elems, int M, int K, int N,
+                                     int positions, const float* x_sum, const float* w_resp, const float* taps, const float* z_a,
+                                     const float* z_w, const float* s_a, const float* s_w, const float* bias, float* out,
+                                     void* workspace, size_t workspace_bytes, void* stream) {
+    if (M < 0 || K < 0 || N < 0) return fail(AMR_EINVAL, "negative dimension M=%d K=%d N=%d", M, K, N);
+    if (positions <= 0 || M % positions != 0) return fail(AMR_EINVAL, "positions=%d must divide M=%d", positions, M);
+    amr::LutGeom g;
+    if (!amr::lut_geom_from_elems(lut_elems, &g))
+        return fail(AMR_ELUTLEN, "lut size should be one of 1024/5120/17408/66306, got %lld", (long long)lut_elems);
+    if (M == 0 || N == 0) return AMR_OK;
+    if (!lut || (K > 0 && (!A || !B)) || !x_sum || !w_resp || !taps || !z_a || !z_w || !s_a || !s_w || !out)
+        return fail(AMR_EINVAL, "null pointer argument");
+    if ((uintptr_t)lut & 3) return fail(AMR_EINVAL, "lut must be 4-byte aligned");
+    const size_t need = amr_lut_conv_forward_dequant_workspace_bytes(lut_elems, M, K, N);
+    if (!workspace || workspace_bytes < need)
+        return fail(AMR_EWORKSPACE, "workspace of %zu bytes is smaller than the %zu required", workspace ? workspace_bytes : (size_t)0, need);
+    if ((uintptr_t)workspace & 255) return fail(AMR_EINVAL, "workspace must be 256-byte aligned");
+    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    int dev = 0;
+    const int n_cu = current_device_cus(&dev);
+    if (n_cu <= 0) return fail(AMR_EINVAL, "no HIP device available");
+    const size_t e_bytes = need - (size_t)M * N * sizeof(float);
+    float* sums = reinterpret_cast<float*>(reinterpret_cast<unsigned char*>(workspace) + e_bytes);
+    const int mode = g_expanded_kernels.load();
+    hipError_t e;
+    if (K > 0 && mode && e_bytes && amr::fwd_slab_can_dequant(g, M, K, N, n_cu, mode == 2)) {
+        // one launch stores the activation; `sums` is touched by the gated fall-back only
+        const amr::SlabDequant dq{x_sum, w_resp, taps, z_a, z_w, s_a, s_w, bias, out, positions};
+        e = amr::launch_fwd_slab(A, B, reinterpret_cast<uint32_t*>(sums), lut, g, M, K, N, n_cu, workspace, s, 1, &dq);
+        return e == hipSuccess ? AMR_OK : hip_fail(e, "forward launch");
+    }
+    // K split over workgroups, small problems, direct kernels: the sums meet in memory first, a second pass dequantises them
+    const int rc = forward_impl(A, B, reinterpret_cast<uint32_t*>(sums), lut, lut_elems, M, K, N, e_bytes ? workspace : nullptr, e_bytes, stream, 1);
+    if (rc != AMR_OK) return rc;
+    e = amr::launch_dequant(sums, x_sum, w_resp, taps, z_a, z_w, s_a, s_w, bias, out, M, N, positions, s);
+    return e == hipSuccess ? AMR_OK : hip_fail(e, "dequant launch");
 }
 
 int amr_lut_gemm_forward_ws(const uint8_t* A, const uint8_t* B, uint32_t* C, const uint16_t* lut, int64_t lut_elems,

@@ -17,8 +17,9 @@ namespace amr {
 __global__ __launch_bounds__(256) void dequant_rows_to_nchw_kernel(
     const float* __restrict__ c, const float* __restrict__ xs, const float* __restrict__ wr, const float* __restrict__ tp,
     const float* __restrict__ za_p, const float* __restrict__ zw_p, const float* __restrict__ sa_p, const float* __restrict__ sw_p,
-    const float* __restrict__ bias, float* __restrict__ out, int M, int N, int L) {
+    const float* __restrict__ bias, float* __restrict__ out, int M, int N, int L, const uint32_t* __restrict__ gate) {
     __shared__ float tile[4][32][33];
+    if (gate != nullptr && *gate == 0u) return;       // queued behind a kernel that usually has done this work already
     const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
     const int m0 = blockIdx.x * 128, n0 = blockIdx.y * 32;
     const float za = *za_p, zw = *zw_p;
@@ -95,7 +96,16 @@ __global__ __launch_bounds__(256) void dequant_grad_nchw_to_rows_kernel(const fl
 hipError_t launch_dequant(const float* c, const float* xs, const float* wr, const float* tp, const float* za, const float* zw,
                           const float* sa, const float* sw, const float* bias, float* out, int M, int N, int L, hipStream_t stream) {
     hipLaunchKernelGGL(dequant_rows_to_nchw_kernel, dim3((M + 127) / 128, (N + 31) / 32), dim3(256), 0, stream, c, xs, wr, tp, za, zw, sa,
-                       sw, bias, out, M, N, L);
+                       sw, bias, out, M, N, L, (const uint32_t*)nullptr);
+    return hipGetLastError();
+}
+
+// The same pass queued behind a kernel that normally produced `out` itself: it runs only when *gate != 0.
+hipError_t launch_dequant_gated(const float* c, const float* xs, const float* wr, const float* tp, const float* za, const float* zw,
+                                const float* sa, const float* sw, const float* bias, float* out, int M, int N, int L,
+                                const uint32_t* gate, hipStream_t stream) {
+    hipLaunchKernelGGL(dequant_rows_to_nchw_kernel, dim3((M + 127) / 128, (N + 31) / 32), dim3(256), 0, stream, c, xs, wr, tp, za, zw, sa,
+                       sw, bias, out, M, N, L, gate);
     return hipGetLastError();
 }
 

@@ -282,11 +282,52 @@ __device__ __forceinline__ void slab_store_tile(const uint32_t (&acc)[RG][8], un
     }
 }
 
-template <int RG, int WAVES, bool PACKED>
+// The same tile, dequantised on its way out and stored as the NCHW activation:
+//   out[b,n,pos] = (s_a*s_w) * ((float)sum + ((z_w*xs[m] + z_a*wr[n,pos]) + (z_a*z_w)*tp[pos])) + bias[n],   m = b*L + pos
+// every operation rounded on its own in that order (the bits of dequant_rows_to_nchw_kernel on the float32 sums).  The sums
+// go to LDS column-major ([32 columns][64 rows]); afterwards lane = row, so that a store instruction writes 64 consecutive
+// positions of one output channel (256 B) and reads 64 different banks.
+template <int RG, bool PACKED>
+__device__ __forceinline__ void slab_store_tile_dequant(const uint32_t (&acc)[RG][8], unsigned char* wave_lds, int lane, int rs, int cg,
+                                                        const SlabDequant& dq, int m_wave, int m_first, int n0, int N) {
+    float* w = reinterpret_cast<float*>(wave_lds);
+#pragma unroll
+    for (int i = 0; i < RG; ++i) {
+        const int row = 16 * i + rs;
+#pragma unroll
+        for (int c = 0; c < 8; c += 2) {
+            const uint32_t even = PACKED ? acc[i][c] : acc[i][c] - (acc[i][c + 1] << 16);
+            w[(cg * 8 + c) * 64 + row] = (float)even;
+            w[(cg * 8 + c + 1) * 64 + row] = (float)acc[i][c + 1];
+        }
+    }
+    const int m = m_wave + lane;
+    const int L = dq.L;
+    const int b = m / L, pos = m - b * L;
+    const float za = *dq.za, zw = *dq.zw;
+    const float s = __fmul_rn(*dq.sa, *dq.sw), zz = __fmul_rn(za, zw);
+    const float x_term = __fmul_rn(zw, dq.xs[m]);
+    const float t_term = __fmul_rn(zz, dq.tp[pos]);
+    const float* wr = dq.wr + pos;
+    float* out = dq.out + (size_t)b * N * L + pos;
+    const bool live = m >= m_first;
+#pragma unroll 8
+    for (int col = 0; col < 32; ++col) {
+        const int n = n0 + col;
+        if (n < N && live) {
+            const float terms = __fadd_rn(__fadd_rn(x_term, __fmul_rn(za, wr[(size_t)n * L])), t_term);
+            float v = __fmul_rn(s, __fadd_rn(w[col * 64 + lane], terms));
+            if (dq.bias != nullptr) v = __fadd_rn(v, dq.bias[n]);
+            out[(size_t)n * L] = v;
+        }
+    }
+}
+
+template <int RG, int WAVES, bool PACKED, bool DEQ = false>
 __global__ __launch_bounds__(WAVES * 64) void lutgemm_fwd_slab_kernel(
     const uint8_t* __restrict__ A, const u32x4* __restrict__ E, uint32_t* __restrict__ C,
     uint32_t* __restrict__ flags, int M, int K, int N, int k_quads, int chunks_per_split, int atomic_out, int out_f32,
-    int n_tiles_grouped, int row_blocks) {
+    int n_tiles_grouped, int row_blocks, SlabDequant dq) {
     // static: lets the compiler fold the base address (chunk buffers first: their addresses come out of v_perm)
     __shared__ __align__(16) unsigned char smem[kSlabBuffers * kSlabChunkBytes + 2 * kSlabCodeBytes];
     constexpr int THREADS = WAVES * 64;
@@ -407,7 +448,10 @@ __global__ __launch_bounds__(WAVES * 64) void lutgemm_fwd_slab_kernel(
     if (__builtin_amdgcn_ballot_w64((seen & 0x80808080u) != 0) != 0) {
         if (lane == 0) atomicOr(&flags[1], 1u);
     }
-    slab_store_tile<RG, PACKED>(acc, smem + wave * 8192, lane, rs, cg, C, m_wave, m_first, tile_x * kSlabCols, N, atomic_out, out_f32);
+    if constexpr (DEQ)
+        slab_store_tile_dequant<RG, PACKED>(acc, smem + wave * 8192, lane, rs, cg, dq, m_wave, m_first, tile_x * kSlabCols, N);
+    else
+        slab_store_tile<RG, PACKED>(acc, smem + wave * 8192, lane, rs, cg, C, m_wave, m_first, tile_x * kSlabCols, N, atomic_out, out_f32);
 }
 
 // ------------------------------------------------------------------------------------------ 8-bit tables
@@ -419,10 +463,11 @@ __global__ __launch_bounds__(WAVES * 64) void lutgemm_fwd_slab_kernel(
 constexpr int kSlab8Rows = 256;
 constexpr int kSlab8ChunkBytes = kSlab8Rows * 256;   // 64 KB
 
-template <bool PACKED>
+template <bool PACKED, bool DEQ = false>
 __global__ __launch_bounds__(1024) void lutgemm_fwd_slab8_kernel(
     const uint8_t* __restrict__ A, const u32x4* __restrict__ E, uint32_t* __restrict__ C,
-    const uint32_t* __restrict__ flags, int M, int K, int N, int k_quads, int chunks_per_split, int atomic_out, int out_f32) {
+    const uint32_t* __restrict__ flags, int M, int K, int N, int k_quads, int chunks_per_split, int atomic_out, int out_f32,
+    SlabDequant dq) {
     __shared__ __align__(16) unsigned char smem[2 * kSlab8ChunkBytes + 2 * kSlabCodeBytes];
     constexpr int RG = 4, WAVES = 16, THREADS = WAVES * 64, ROWS_PER_WAVE = 16 * RG;
     static_assert(2 * kSlab8ChunkBytes + 2 * kSlabCodeBytes == 160 * 1024, "the workgroup uses the whole LDS of a CU");
@@ -496,7 +541,10 @@ __global__ __launch_bounds__(1024) void lutgemm_fwd_slab8_kernel(
     }
     // nothing is left in flight towards LDS and every wave has read its last chunk: the buffers take the sums
     asm volatile("s_waitcnt vmcnt(0)\n s_barrier" ::: "memory");
-    slab_store_tile<RG, PACKED>(acc, smem + wave * 8192, lane, rs, cg, C, m_wave, m_first, tile_x * kSlabCols, N, atomic_out, out_f32);
+    if constexpr (DEQ)
+        slab_store_tile_dequant<RG, PACKED>(acc, smem + wave * 8192, lane, rs, cg, dq, m_wave, m_first, tile_x * kSlabCols, N);
+    else
+        slab_store_tile<RG, PACKED>(acc, smem + wave * 8192, lane, rs, cg, C, m_wave, m_first, tile_x * kSlabCols, N, atomic_out, out_f32);
 }
 
 hipError_t launch_fwd_gated(const uint8_t* A, const uint8_t* B, uint32_t* C, const uint16_t* lut, const LutGeom& g,
@@ -523,10 +571,37 @@ size_t fwd_slab_workspace_bytes(const LutGeom& g, int M, int K, int N, bool forc
     return 256 + n_tiles * k_quads * kSlabChunkBytes;
 }
 
+hipError_t launch_dequant_gated(const float* c, const float* xs, const float* wr, const float* tp, const float* za, const float* zw,
+                                const float* sa, const float* sw, const float* bias, float* out, int M, int N, int L,
+                                const uint32_t* gate, hipStream_t stream);
+
+// K splits of the expanded-table forward launch for this shape (1: every workgroup owns whole sums).
+static int fwd_slab_ksplit(int M, int K, int N, int n_cu) {
+    const int n_tiles = (N + kSlabCols - 1) / kSlabCols, k_quads = (K + 3) / 4;
+    const long wgs = (long)n_tiles * ((M + 1023) / 1024);
+    int ksplit = 1;
+    if (wgs < n_cu) {
+        ksplit = (int)((n_cu + wgs - 1) / wgs);
+        const int max_split = k_quads / 8 > 0 ? k_quads / 8 : 1;     // at least 32 k per workgroup
+        if (ksplit > max_split) ksplit = max_split;
+    }
+    const int cps = (k_quads + ksplit - 1) / ksplit;
+    return (k_quads + cps - 1) / cps;
+}
+
+// The expanded-table forward pass can dequantise in its store when no K split adds partial sums in memory.
+bool fwd_slab_can_dequant(const LutGeom& g, int M, int K, int N, int n_cu, bool force) {
+    return fwd_slab_workspace_bytes(g, M, K, N, force) != 0 && fwd_slab_ksplit(M, K, N, n_cu) == 1;
+}
+
+// dq != nullptr (only with fwd_slab_can_dequant): the kernel stores the dequantised NCHW activation dq->out instead of C; C
+// (float32 [M,N]) is then scratch that only the gated fall-back touches, followed by a dequantisation pass under the same gate.
 hipError_t launch_fwd_slab(const uint8_t* A, const uint8_t* B, uint32_t* C, const uint16_t* lut, const LutGeom& g,
-                           int M, int K, int N, int n_cu, void* workspace, hipStream_t stream, int out_f32) {
+                           int M, int K, int N, int n_cu, void* workspace, hipStream_t stream, int out_f32,
+                           const SlabDequant* dq = nullptr) {
     const int n_tiles = (N + kSlabCols - 1) / kSlabCols;
     const int k_quads = (K + 3) / 4;
+    const SlabDequant none{};
     uint32_t* flags = reinterpret_cast<uint32_t*>(workspace);
     uint32_t* E = reinterpret_cast<uint32_t*>(reinterpret_cast<unsigned char*>(workspace) + 256);
     hipError_t e;
@@ -550,8 +625,14 @@ hipError_t launch_fwd_slab(const uint8_t* A, const uint8_t* B, uint32_t* C, cons
         const int zs8 = (k_quads + cps8 - 1) / cps8;
         if (zs8 > 1 && (e = launch_zero_u32(C, (size_t)M * N, stream)) != hipSuccess) return e;
         const dim3 grid8(n_tiles, row_blocks8, zs8);
+        if (dq) {
+            if (zs8 != 1) return hipErrorInvalidValue;
+            hipLaunchKernelGGL((lutgemm_fwd_slab8_kernel<false, true>), grid8, dim3(1024), 0, stream, A, reinterpret_cast<const u32x4*>(E), C,
+                               flags, M, K, N, k_quads, cps8, 0, 1, *dq);
+            return hipGetLastError();
+        }
         hipLaunchKernelGGL((lutgemm_fwd_slab8_kernel<false>), grid8, dim3(1024), 0, stream, A, reinterpret_cast<const u32x4*>(E), C, flags,
-                           M, K, N, k_quads, cps8, zs8 > 1 ? 1 : 0, out_f32);
+                           M, K, N, k_quads, cps8, zs8 > 1 ? 1 : 0, out_f32, none);
         if ((e = hipGetLastError()) != hipSuccess) return e;
         if (zs8 > 1 && out_f32) return launch_u32_to_f32(C, (size_t)M * N, stream);
         return hipSuccess;
@@ -587,8 +668,19 @@ hipError_t launch_fwd_slab(const uint8_t* A, const uint8_t* B, uint32_t* C, cons
         grouped = n_tiles;
         grid = dim3(8 * ((row_blocks + 7) / 8) * n_tiles);
     }
+    if (dq) {
+        if (zs != 1) return hipErrorInvalidValue;
+        hipLaunchKernelGGL((lutgemm_fwd_slab_kernel<RG, WAVES, true, true>), grid, dim3(WAVES * 64), 0, stream, A,
+                           reinterpret_cast<const u32x4*>(E), C, flags, M, K, N, k_quads, cps, 0, 1, grouped, row_blocks, *dq);
+        if ((e = hipGetLastError()) != hipSuccess) return e;
+        // masked codes / entries too large for packed sums: the direct kernel recomputes the sums into C, a pass under the
+        // same gate dequantises them
+        if ((e = launch_fwd_gated(A, B, C, lut, g, M, K, N, flags + 1, stream, 1)) != hipSuccess) return e;
+        return launch_dequant_gated(reinterpret_cast<const float*>(C), dq->xs, dq->wr, dq->tp, dq->za, dq->zw, dq->sa, dq->sw, dq->bias,
+                                    dq->out, M, N, dq->L, flags + 1, stream);
+    }
     hipLaunchKernelGGL((lutgemm_fwd_slab_kernel<RG, WAVES, true>), grid, dim3(WAVES * 64), 0, stream, A,
-                       reinterpret_cast<const u32x4*>(E), C, flags, M, K, N, k_quads, cps, zs > 1 ? 1 : 0, out_f32, grouped, row_blocks);
+                       reinterpret_cast<const u32x4*>(E), C, flags, M, K, N, k_quads, cps, zs > 1 ? 1 : 0, out_f32, grouped, row_blocks, none);
     e = hipGetLastError();
     if (e != hipSuccess) return e;
     // (partial sums over a split K met as integers: converted before the fall-back, which stores floats itself)

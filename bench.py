@@ -112,19 +112,25 @@ def capture_codes(torch, dev, bits, tables, arch, batch):
     model = app_train.build_model(arch, bits, False, dev, approx_linear=True)
     x = torch.randn(batch, 3, 32, 32, device=dev, generator=torch.Generator(device=dev).manual_seed(1))
     seen = {}
-    native = ops.approx_ops.approx_gemm_forward
+    # (the layers call the LUT GEMM through either of the native module's two forward functions; both take a, b first)
+    names = ("approx_gemm_forward", "approx_conv_forward_dequant")
+    natives = {n: getattr(ops.approx_ops, n) for n in names}
 
-    def spy(a, b, c, lut):
-        seen.setdefault((a.shape[0], a.shape[1], b.shape[1]), (a.clone(), b.clone()))
-        return native(a, b, c, lut)
+    def spy_on(fn):
+        def spy(a, b, *rest):
+            seen.setdefault((a.shape[0], a.shape[1], b.shape[1]), (a.clone(), b.clone()))
+            return fn(a, b, *rest)
+        return spy
 
-    ops.approx_ops.approx_gemm_forward = spy
+    for n in names:
+        setattr(ops.approx_ops, n, spy_on(natives[n]))
     try:
         model.train()
         with torch.no_grad():
             model(x)
     finally:
-        ops.approx_ops.approx_gemm_forward = native
+        for n in names:
+            setattr(ops.approx_ops, n, natives[n])
     return seen
 
 

@@ -221,6 +221,23 @@ int amr_conv_dequant_backward_f32(const float *g, const float *s_a, const float 
                                   int out_channels, int positions, void *stream);
 
 /*
+ * Forward LUT GEMM of a convolution with the dequantisation in the kernel's store: the sums of amr_lut_gemm_forward never
+ * go to memory, the kernel writes the NCHW activation of amr_conv_dequant_f32 directly (same operations in the same order
+ * on the float32 sums: the same bits),
+ *   out[b,n,pos] = (*s_a * *s_w) * ((float)C[b*L+pos, n] + ((*z_w * x_sum[b*L+pos] + *z_a * w_resp[n*L+pos]) + (*z_a * *z_w) * taps[pos])) + bias[n]
+ * with L = positions (must divide M); A [M,K], B [K,N] uint8 in any common order of k.  Replaces the LUT GEMM plus the
+ * zero-point terms and scaling of the reference's ApproxConv2d.forward (self_ops/src/approx_gemm_forward.cu:241-314 called
+ * from micronet+/app_layers.py:175-183).  Shapes the expanded-table kernel does not take whole (small problems, a K split
+ * over workgroups) run the GEMM into the workspace and dequantise in a second pass.  workspace: at least
+ * amr_lut_conv_forward_dequant_workspace_bytes(...) bytes, 256-byte aligned, required.
+ */
+size_t amr_lut_conv_forward_dequant_workspace_bytes(int64_t lut_elems, int M, int K, int N);
+int amr_lut_conv_forward_dequant_f32(const uint8_t *A, const uint8_t *B, const uint16_t *lut, int64_t lut_elems, int M, int K,
+                                     int N, int positions, const float *x_sum, const float *w_resp, const float *taps,
+                                     const float *z_a, const float *z_w, const float *s_a, const float *s_w, const float *bias,
+                                     float *out, void *workspace, size_t workspace_bytes, void *stream);
+
+/*
  * Range tracking and quantisation parameters of one tensor in one launch (all pointers: one float in device memory).
  * mode 0: min_val/max_val := cur_min/cur_max (first batch); 1: running extremes; 2: keep * old + momentum * current;
  * then *scale = max((max - min) / quant_max, eps) -- or (max - min) * inv_quant_max when inv_quant_max != 0, which is

@@ -180,3 +180,53 @@ def test_uint8_layer_path_first_layer_needs_no_input_gradient(ops):
     y = layer(x)
     y.square().mean().backward()
     assert layer.weight.grad is not None and torch.isfinite(layer.weight.grad).all()
+
+
+@pytest.mark.parametrize("bits,bn,L,K,N,masked,bias", [
+    (7, 8, 1024, 576, 64, False, True),      # expanded-table kernel stores the activation itself
+    (7, 8, 1024, 576, 64, True, True),       # a masked code 128: the gated direct kernel and the gated dequantisation do the work
+    (7, 32, 64, 64, 40, False, False),       # ragged column tile
+    (7, 16, 256, 2304, 256, False, True),    # K split over workgroups: sums meet in memory, second pass
+    (7, 3, 25, 45, 10, False, True),         # small: direct kernel + second pass
+    (7, 2050, 1, 64, 32, False, True),       # one position per image, rows not a multiple of the wave's 64
+    (8, 8, 1024, 288, 64, False, True),      # 8-bit expanded-table kernel
+    (6, 4, 1024, 72, 32, False, False),      # narrower table
+])
+def test_forward_with_dequantising_store_equals_gemm_then_dequantisation(ops, oracle, bits, bn, L, K, N, masked, bias):
+    """amr_lut_conv_forward_dequant_f32 through the module function, against approx_gemm_forward (float32 sums, themselves
+    checked bit-exact against the oracle here) followed by conv_dequant: identical bits for every shape and kernel choice."""
+    import approx_ops
+    print("forward + dequant", bits, bn, L, K, N, masked, flush=True)
+    rng = np.random.default_rng(21)
+    n = 1 << bits
+    M = bn * L
+    A = rng.integers(0, n, (M, K)).astype(np.uint8)
+    B = rng.integers(0, n, (K, N)).astype(np.uint8)
+    if masked:
+        A[M // 2, 3] = n
+    T = oracle.synth_lut(bits, 64, rng)
+    flat = oracle.pack_table(T, bits, np.uint16)
+    a, b, lut = (torch.tensor(v, device="cuda") for v in (A, B, flat))
+    g = torch.Generator(device="cuda").manual_seed(4)
+    x_sum = torch.randint(0, 9 * 64 * 127, (M,), device="cuda", generator=g).float()
+    w_resp = torch.randint(0, 9 * 64 * 127, (N, L), device="cuda", generator=g).float()
+    taps = torch.randint(1, 577, (L,), device="cuda", generator=g).float()
+    z_a, z_w = torch.tensor([-3.0], device="cuda"), torch.tensor([-61.0], device="cuda")
+    s_a, s_w = torch.tensor([0.0213], device="cuda"), torch.tensor([0.0037], device="cuda")
+    bvec = torch.randn(N, device="cuda", generator=g) if bias else None
+    side = int(round(L ** 0.5))
+    hw = (side, side) if side * side == L else (1, L)
+    # mode 2: the expanded-table kernels wherever the shape allows (the test sizes are below the sizes the library picks them at)
+    old = approx_ops._lib.amr_set_expanded_table_kernels(2)
+    try:
+        c = torch.empty((M, N), dtype=torch.float32, device="cuda")
+        approx_ops.approx_gemm_forward(a, b, c, lut)
+        want = torch.full((bn, N, *hw), float("nan"), device="cuda")
+        approx_ops.conv_dequant(c, x_sum, w_resp, taps, z_a, z_w, s_a, s_w, bvec, want)
+        got = torch.full((bn, N, *hw), float("nan"), device="cuda")
+        approx_ops.approx_conv_forward_dequant(a, b, lut, x_sum, w_resp, taps, z_a, z_w, s_a, s_w, bvec, got)
+    finally:
+        approx_ops._lib.amr_set_expanded_table_kernels(old)
+    rows = slice(0, min(M, 2048))
+    assert (c[rows].cpu().numpy() == oracle.forward_c(A[rows], B, flat, bits).astype(np.float32)).all()
+    assert torch.equal(got, want)
