@@ -229,7 +229,11 @@ class _ApproxConvLayerFn(torch.autograd.Function):
         approx_ops.approx_conv_forward_dequant(a_mat, b_mat, ops.lut_appmult, x_sum.contiguous(), w_resp.detach().contiguous(),
                                                taps.contiguous(), z_a, z_w, s_a, s_w,
                                                None if bias is None else bias.detach().contiguous(), out)
-        ctx.save_for_backward(a_mat, b_mat, inside, s_a, z_a, s_w, z_w)
+        # a 3x3 / stride 1 / padding 1 layer takes its input gradient from one implicit GEMM over the input pixels (no
+        # [M][9C] gradient matrix, no col2im) where the library serves the shape and the gradient table fits halves
+        conv_shaped = ((kh, kw, s, p, d) == (3, 3, 1, 1, 1) and ops.lut_grad_a_fits_halves
+                       and approx_ops.conv_input_grad_supported(ops.lut_grad_a, (bn, cin, h, w), cout))
+        ctx.save_for_backward(a_mat, b_mat, inside, s_a, z_a, s_w, z_w, codes if conv_shaped else None)
         ctx.geo = (bn, cin, h, w, cout, kh, kw, s, p, d, oh, ow)
         ctx.aux = (w_resp.shape, bias is not None, x.dtype)
         return out
@@ -238,7 +242,7 @@ class _ApproxConvLayerFn(torch.autograd.Function):
     def backward(ctx, g):
         import approx_ops
         from self_ops.ops_py import approx_ops as ops
-        a_mat, b_mat, inside, s_a, z_a, s_w, z_w = ctx.saved_tensors
+        a_mat, b_mat, inside, s_a, z_a, s_w, z_w, codes = ctx.saved_tensors
         bn, cin, h, w, cout, kh, kw, s, p, d, oh, ow = ctx.geo
         wr_shape, has_bias, x_dtype = ctx.aux
         need_x, need_w, need_wr = ctx.needs_input_grad[0], ctx.needs_input_grad[1], ctx.needs_input_grad[2]
@@ -250,12 +254,17 @@ class _ApproxConvLayerFn(torch.autograd.Function):
             t = torch.empty(bn * oh * ow, dtype=torch.float32, device=dev)
             approx_ops.conv_dequant_backward_rowsum(g, s_a, s_w, g_rows, t)
             # (a gradient nobody asked for -- the images in front of the first layer -- is not computed)
-            g_a = torch.empty((bn, kh * kw * cin, oh * ow), dtype=torch.float32, device=dev) if need_x else None
+            conv_shaped = codes is not None and need_x
+            g_a = torch.empty((bn, kh * kw * cin, oh * ow), dtype=torch.float32, device=dev) if need_x and not conv_shaped else None
             g_b = torch.empty(b_mat.shape, dtype=torch.float32, device=dev) if need_w else None
-            approx_ops.approx_gemm_backward(g_rows, a_mat, b_mat, g_a, g_b, ops.lut_grad_a, ops.lut_grad_b, ga_rows_per_image=oh * ow)
+            if g_a is not None or g_b is not None:
+                approx_ops.approx_gemm_backward(g_rows, a_mat, b_mat, g_a, g_b, ops.lut_grad_a, ops.lut_grad_b, ga_rows_per_image=oh * ow)
             if need_x:
                 g_x = torch.empty((bn, cin, h, w), dtype=torch.float32, device=dev)
-                approx_ops.conv_input_grad(g_a, t, z_w, inside, s_a, g_x, (kh, kw), s, p, d)
+                if conv_shaped:
+                    approx_ops.approx_conv_input_grad(g_rows, codes, b_mat, ops.lut_grad_a, t, z_w, inside, s_a, g_x)
+                else:
+                    approx_ops.conv_input_grad(g_a, t, z_w, inside, s_a, g_x, (kh, kw), s, p, d)
                 g_x = g_x.to(x_dtype)
             if need_w:
                 g_w = g_b.view(kh, kw, cin, cout).permute(3, 2, 0, 1)

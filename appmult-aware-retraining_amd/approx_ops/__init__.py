@@ -54,6 +54,11 @@ _lib.amr_quantize_codes_backward_f32.argtypes = [_vp, _vp, _vp, _vp, ctypes.c_fl
 _lib.amr_lut_conv_forward_dequant_workspace_bytes.argtypes = [_i64, _i, _i, _i]
 _lib.amr_lut_conv_forward_dequant_workspace_bytes.restype = _sz
 _lib.amr_lut_conv_forward_dequant_f32.argtypes = [_vp, _vp, _vp, _i64, _i, _i, _i, _i] + [_vp] * 9 + [_vp, _sz, _vp]
+_lib.amr_lut_conv_input_grad_supported.argtypes = [_i64, _i, _i, _i, _i, _i]
+_lib.amr_lut_conv_input_grad_workspace_bytes.argtypes = [_i64, _i, _i, _i, _i, _i]
+_lib.amr_lut_conv_input_grad_workspace_bytes.restype = _sz
+_lib.amr_grad_table_fits_halves.argtypes = [_vp, _i64]
+_lib.amr_lut_conv_input_grad_f32.argtypes = [_vp] * 4 + [_i64] + [_vp] * 5 + [_i] * 5 + [_vp, _vp, _vp, _sz, _vp]
 _lib.amr_quantize_codes_nhwc_u8.argtypes = [_vp, _vp, _vp, ctypes.c_float, _vp, _vp, _vp, _i, _i, _i, _vp]
 _lib.amr_im2col_nhwc_u8.argtypes = [_vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp]
 _lib.amr_conv_input_grad_f32.argtypes = [_vp] * 6 + [_i] * 9 + [_vp]
@@ -443,6 +448,63 @@ def conv_input_grad(cols_tensor, t_tensor, z_w, inside_tensor, scale_tensor, gx_
                                           inside_tensor.data_ptr(), scale_tensor.data_ptr(), gx_tensor.data_ptr(), Bn, C, H, W, kh, kw,
                                           stride, padding, dilation, _stream_ptr(dev))
     _raise_for(rc, "conv_input_grad")
+
+
+def grad_table_fits_halves(table_i16):
+    """Whether the expanded-table backward kernels can hold this int16 gradient table (a NumPy array, padded layout) as
+    halves; the decision the library takes on the device for every backward call."""
+    import numpy as np
+    arr = np.ascontiguousarray(table_i16, np.int16)
+    rc = _lib.amr_grad_table_fits_halves(arr.ctypes.data, arr.size)
+    _check(rc >= 0, f"grad_table_fits_halves failed ({rc}): {_lib.amr_last_error().decode()}")
+    return bool(rc)
+
+
+def conv_input_grad_supported(lut_grad_a_tensor, image_shape, out_channels):
+    """Whether approx_conv_input_grad serves this shape (3x3, stride 1, padding 1 is the caller's to check)."""
+    Bn, C, H, W = image_shape
+    return (lut_grad_a_tensor.dtype == torch.int16 and
+            bool(_lib.amr_lut_conv_input_grad_supported(lut_grad_a_tensor.numel(), Bn, C, H, W, out_channels)))
+
+
+def approx_conv_input_grad(gc_rows, codes_tensor, bt_tensor, lut_grad_a_tensor, t_tensor, z_w, inside_tensor, scale_tensor, gx_tensor,
+                           a_fallback=None):
+    """Input gradient of the quantised 3x3 / stride 1 / padding 1 LUT convolution as one implicit GEMM over the input pixels
+    (amr_lut_conv_input_grad_f32): gc_rows float32 [B*H*W, N], codes uint8 [B*H*W, C], bt uint8 [9*C, N] tap-major, gx float32
+    [B,C,H,W].  a_fallback: the window matrix uint8 [B*H*W, 9*C]; given, tables that do not fit halves and masked codes are
+    served too (through a scratch of 9*C*B*H*W floats), else such a call yields NaN."""
+    _check_input(gc_rows, torch.float32, "gc_rows")
+    _check_input(codes_tensor, torch.uint8, "codes_tensor")
+    _check_input(bt_tensor, torch.uint8, "bt_tensor")
+    _check_input(lut_grad_a_tensor, torch.int16, "lut_grad_a_tensor")
+    for t, name, dt in ((t_tensor, "t_tensor", torch.float32), (z_w, "z_w", torch.float32), (inside_tensor, "inside_tensor", torch.uint8),
+                        (scale_tensor, "scale_tensor", torch.float32), (gx_tensor, "gx_tensor", torch.float32)):
+        _check_input(t, dt, name)
+    _check(gx_tensor.dim() == 4 and inside_tensor.shape == gx_tensor.shape, "gx must be 4-D and inside of its shape")
+    Bn, C, H, W = gx_tensor.shape
+    M = Bn * H * W
+    N = bt_tensor.size(1)
+    _check(tuple(gc_rows.shape) == (M, N), f"gc_rows's shape should be {M} x {N}")
+    _check(tuple(codes_tensor.shape) == (M, C), f"codes_tensor's shape should be {M} x {C}")
+    _check(tuple(bt_tensor.shape) == (9 * C, N), f"bt_tensor's shape should be {9 * C} x {N}")
+    _check(t_tensor.numel() == M and z_w.numel() == 1 and scale_tensor.numel() == 1, "t, z_w or scale has the wrong size")
+    _lut_len_check(lut_grad_a_tensor, "lut_grad_a_tensor")
+    dev = gx_tensor.device
+    cols = None
+    if a_fallback is not None:
+        _check_input(a_fallback, torch.uint8, "a_fallback")
+        _check(tuple(a_fallback.shape) == (M, 9 * C), f"a_fallback's shape should be {M} x {9 * C}")
+    with torch.cuda.device(dev):
+        if a_fallback is not None:
+            cols = torch.empty((Bn, 9 * C, H * W), dtype=torch.float32, device=dev)
+        need = _lib.amr_lut_conv_input_grad_workspace_bytes(lut_grad_a_tensor.numel(), Bn, C, H, W, N)
+        ws = torch.empty(max(need, 256), dtype=torch.uint8, device=dev)
+        rc = _lib.amr_lut_conv_input_grad_f32(gc_rows.data_ptr(), codes_tensor.data_ptr(), bt_tensor.data_ptr(), lut_grad_a_tensor.data_ptr(),
+                                              lut_grad_a_tensor.numel(), t_tensor.data_ptr(), z_w.data_ptr(), inside_tensor.data_ptr(),
+                                              scale_tensor.data_ptr(), gx_tensor.data_ptr(), Bn, C, H, W, N,
+                                              a_fallback.data_ptr() if a_fallback is not None else None,
+                                              cols.data_ptr() if cols is not None else None, ws.data_ptr(), ws.numel(), _stream_ptr(dev))
+    _raise_for(rc, "approx_conv_input_grad")
 
 
 def conv_dequant_backward_rowsum(g_tensor, s_a, s_w, gc_rows, t_tensor):

@@ -100,7 +100,12 @@ hipError_t launch_im2col_nhwc(const uint8_t* codes, uint8_t* A, long B, int C, i
                               int dil, int oh, int ow, hipStream_t stream);
 hipError_t launch_conv_input_grad(const float* cols, const float* t, const float* zw, const uint8_t* inside, const float* scale,
                                   float* gx, long B, int C, int H, int W, int kh, int kw, int stride, int pad, int dil, int oh, int ow,
-                                  hipStream_t stream);
+                                  hipStream_t stream, const uint32_t* gate = nullptr, int gate_mode = 0);
+bool gradA_slab_conv_applies(const LutGeom& g, long M, int C, int N, const float* gC, bool force);
+size_t gradA_slab_conv_workspace_bytes(int C, int N);
+hipError_t launch_gradA_slab_conv(const float* gC, const uint8_t* codes, const uint8_t* Bt, float* g_in, const int16_t* lut,
+                                  const LutGeom& g, int Bn, int C, int H, int W, int N, float scale, int n_cu, uint32_t* flags,
+                                  void* S, const float* zero_line, hipStream_t stream);
 hipError_t launch_dequant_grad_rowsum(const float* g, const float* sa, const float* sw, float* gc, float* t, int M, int N, int L,
                                       hipStream_t stream);
 hipError_t launch_accgemm(const float* A, const float* B, float* C, int M, int K, int N, hipStream_t stream);
@@ -795,6 +800,83 @@ int amr_conv_input_grad_f32(const float* cols, const float* t, const float* z_w,
     hipError_t e = amr::launch_conv_input_grad(cols, t, z_w, inside, scale, gx, B, C, H, W, kh, kw, stride, pad, dil, oh, ow,
                                                reinterpret_cast<hipStream_t>(stream));
     return e == hipSuccess ? AMR_OK : hip_fail(e, "input gradient launch");
+}
+
+int amr_lut_conv_input_grad_supported(int64_t lut_elems, int B, int C, int H, int W, int N) {
+    amr::LutGeom g;
+    if (B <= 0 || C <= 0 || H <= 0 || W <= 0 || N <= 0 || !amr::lut_geom_from_elems(lut_elems, &g)) return 0;
+    const int mode = g_expanded_kernels.load();
+    return mode && amr::gradA_slab_conv_applies(g, (long)B * H * W, C, N, nullptr, mode == 2) ? 1 : 0;
+}
+
+size_t amr_lut_conv_input_grad_workspace_bytes(int64_t lut_elems, int B, int C, int H, int W, int N) {
+    if (!amr_lut_conv_input_grad_supported(lut_elems, B, C, H, W, N)) return 0;
+    return 256 + amr::gradA_slab_conv_workspace_bytes(C, N);
+}
+
+// The decision bwd_header_kernel takes on the device (lutgemm_bwd_slab.hip), for a table in host memory.
+int amr_grad_table_fits_halves(const int16_t* host_table, int64_t lut_elems) {
+    amr::LutGeom g;
+    if (!host_table || !amr::lut_geom_from_elems(lut_elems, &g)) return fail(AMR_ELUTLEN, "bad table");
+    int lo = 0, hi = 0;
+    unsigned long long mag = 0;
+    for (int64_t i = 0; i < (int64_t)g.rows * g.cols; ++i) {
+        const int v = host_table[i];
+        lo = v < lo ? v : lo;
+        hi = v > hi ? v : hi;
+        mag += (unsigned long long)(v < 0 ? -v : v);
+    }
+    if (lo >= -2048 && hi <= 2048) return 1;
+    if (hi - lo > 4096) return 0;
+    const int need = hi > 2048 ? hi - 2048 : -(lo + 2048), room = hi > 2048 ? lo + 2048 : -(hi - 2048);
+    int p = 1;
+    while (p < need) p <<= 1;
+    const int off = p <= room ? p : need;
+    const unsigned long long n_entries = (unsigned long long)(1 << g.bits) * (1 << g.bits);
+    return (unsigned long long)off * n_entries > 8ull * mag ? 0 : 1;
+}
+
+int amr_lut_conv_input_grad_f32(const float* gC, const uint8_t* codes, const uint8_t* Bt, const int16_t* lut_grad_a, int64_t lut_elems,
+                                const float* t, const float* z_w, const uint8_t* inside, const float* scale, float* gx, int B, int C,
+                                int H, int W, int N, const uint8_t* A_fallback, float* cols_fallback, void* workspace,
+                                size_t workspace_bytes, void* stream) {
+    amr::LutGeom g;
+    if (!amr::lut_geom_from_elems(lut_elems, &g))
+        return fail(AMR_ELUTLEN, "lut size should be one of 1024/5120/17408/66306, got %lld", (long long)lut_elems);
+    if (B <= 0 || C <= 0 || H <= 0 || W <= 0 || N <= 0) return fail(AMR_EINVAL, "bad shape");
+    if (!gC || !codes || !Bt || !lut_grad_a || !t || !z_w || !inside || !scale || !gx) return fail(AMR_EINVAL, "null pointer argument");
+    if ((uintptr_t)lut_grad_a & 3) return fail(AMR_EINVAL, "gradient tables must be 4-byte aligned");
+    if ((A_fallback == nullptr) != (cols_fallback == nullptr)) return fail(AMR_EINVAL, "A_fallback and cols_fallback go together");
+    const int mode = g_expanded_kernels.load();
+    const long M = (long)B * H * W;
+    if (!mode || !amr::gradA_slab_conv_applies(g, M, C, N, gC, mode == 2))
+        return fail(AMR_EUNSUPPORTED, "shape, alignment or mode not served by the convolution-shaped gradA (ask amr_lut_conv_input_grad_supported)");
+    const size_t need = 256 + amr::gradA_slab_conv_workspace_bytes(C, N);
+    if (!workspace || workspace_bytes < need)
+        return fail(AMR_EWORKSPACE, "workspace of %zu bytes is smaller than the %zu required", workspace ? workspace_bytes : (size_t)0, need);
+    if ((uintptr_t)workspace & 255) return fail(AMR_EINVAL, "workspace must be 256-byte aligned");
+    int dev = 0;
+    const int n_cu = current_device_cus(&dev);
+    if (n_cu <= 0) return fail(AMR_EINVAL, "no HIP device available");
+    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    const float factor = 1.0f / 16.0f;  // FACTOR, self_ops/src/approx_mult.h:41
+    uint32_t* flags = reinterpret_cast<uint32_t*>(workspace);
+    hipError_t e = amr::launch_bwd_header(lut_grad_a, nullptr, g, flags, s);      // clears the 64 flag words: words 32..63 stay zero
+    if (e != hipSuccess) return hip_fail(e, "scratch header launch");
+    e = amr::launch_gradA_slab_conv(gC, codes, Bt, gx, lut_grad_a, g, B, C, H, W, N, factor, n_cu, flags,
+                                    reinterpret_cast<unsigned char*>(workspace) + 256, reinterpret_cast<const float*>(flags + 32), s);
+    if (e != hipSuccess) return hip_fail(e, "gradA launch");
+    // flags[2]: a masked code, an entry a half cannot hold, or a table that cannot be held as halves at all
+    const bool fallback = A_fallback != nullptr;
+    e = amr::launch_conv_input_grad(nullptr, t, z_w, inside, scale, gx, B, C, H, W, 3, 3, 1, 1, 1, H, W, s, flags + 2, fallback ? 1 : 3);
+    if (e != hipSuccess) return hip_fail(e, "input gradient launch");
+    if (fallback) {
+        e = amr::launch_gradA(gC, A_fallback, Bt, cols_fallback, lut_grad_a, g, (int)M, 9 * C, N, factor, n_cu, s, flags + 2, H * W);
+        if (e != hipSuccess) return hip_fail(e, "gradA fall-back launch");
+        e = amr::launch_conv_input_grad(cols_fallback, t, z_w, inside, scale, gx, B, C, H, W, 3, 3, 1, 1, 1, H, W, s, flags + 2, 2);
+        if (e != hipSuccess) return hip_fail(e, "input gradient fall-back launch");
+    }
+    return AMR_OK;
 }
 
 int amr_conv_dequant_backward_rowsum_f32(const float* g, const float* s_a, const float* s_w, float* g_c, float* t, int batch,

@@ -165,9 +165,19 @@ __global__ __launch_bounds__(256) void conv_input_grad_kernel(const float* __res
                                                               const float* __restrict__ zw_p, const uint8_t* __restrict__ inside,
                                                               const float* __restrict__ scale_p, float* __restrict__ gx, int C,
                                                               int H, int W, int kh_rt, int kw_rt, int stride_rt, int pad, int dil,
-                                                              int oh, int ow, size_t total) {
+                                                              int oh, int ow, size_t total, const uint32_t* __restrict__ gate,
+                                                              int gate_mode) {
     const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
     if (idx >= total) return;
+    // gate_mode 1: the pass behind a kernel that left the tap sums in gx -- when *gate says that kernel could not do its work,
+    // this pass leaves gx alone (a recomputation is queued behind, gate_mode 2) or, gate_mode 3, marks every element NaN;
+    // gate_mode 2: runs only when *gate is set.
+    if (gate_mode != 0) {
+        const bool raised = *gate != 0u;
+        if (gate_mode == 2 && !raised) return;
+        if (gate_mode == 1 && raised) return;
+        if (gate_mode == 3 && raised) { gx[idx] = __builtin_nanf(""); return; }
+    }
     const int kh = KH ? KH : kh_rt, kw = KW ? KW : kw_rt, stride = STRIDE ? STRIDE : stride_rt;
     const int xx = (int)(idx % W);
     size_t r = idx / W;
@@ -227,13 +237,13 @@ __global__ __launch_bounds__(256) void conv_input_grad_kernel(const float* __res
 
 hipError_t launch_conv_input_grad(const float* cols, const float* t, const float* zw, const uint8_t* inside, const float* scale,
                                   float* gx, long B, int C, int H, int W, int kh, int kw, int stride, int pad, int dil, int oh, int ow,
-                                  hipStream_t stream) {
+                                  hipStream_t stream, const uint32_t* gate = nullptr, int gate_mode = 0) {
     const size_t total = (size_t)B * C * H * W;
     if (total == 0) return hipSuccess;
     const dim3 grid((unsigned)((total + 255) / 256));
 #define AMR_CIG(KH, KW, S)                                                                                                        \
     hipLaunchKernelGGL((conv_input_grad_kernel<KH, KW, S>), grid, dim3(256), 0, stream, cols, t, zw, inside, scale, gx, C, H, W, kh, kw, \
-                       stride, pad, dil, oh, ow, total)
+                       stride, pad, dil, oh, ow, total, gate, gate_mode)
     if (kh == 3 && kw == 3 && stride == 1) AMR_CIG(3, 3, 1);
     else if (kh == 3 && kw == 3 && stride == 2) AMR_CIG(3, 3, 2);
     else if (kh == 1 && kw == 1 && stride == 1) AMR_CIG(1, 1, 1);

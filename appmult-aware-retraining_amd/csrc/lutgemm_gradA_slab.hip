@@ -315,10 +315,18 @@ __device__ __forceinline__ void ga_store16(float* p, const u32x4& q) {
 // rows_per_image = 0: gA row-major [M,K]; L > 0: image-major transposed gA[m / L][k][m % L].
 // F32: S holds float32 entries, 16 columns per tile (a 64 B window is 16 floats, a 128-bit read feeds four v_fma_f32 instead
 // of eight v_fma_mix_f32); no offset.
-template <int kGaKT, int FMT>
+//
+// CONV (input gradient of a 3x3 convolution of stride 1 and padding 1, as one implicit GEMM): the rows are the B*H*W INPUT
+// pixels, A holds their pixel-major codes [M][C] (K = C here), S the expanded table of the kh*kw*C rows of B in tap-major
+// order, and a tile (512 pixels x KT channels) adds, tap after tap, the products with the rows of gC of the output
+// positions that tap connects the pixel to: row m + (1 - ti) * W + (1 - tj), or a line of zeros where that position lies
+// outside the image.  The sums over taps and columns stay in the accumulators, so neither the [M][9C] gradient matrix
+// nor its col2im pass exists; gA receives [B][C][H*W] (rows_per_image = H*W).  A tile lasts nine times as many chunk steps.
+template <int kGaKT, int FMT, bool CONV = false>
 __global__ __launch_bounds__(kGaWaves * 64) void lutgemm_gradA_slab_kernel(
     const float* __restrict__ gC, const uint8_t* __restrict__ A, const u32x4* __restrict__ S, float* __restrict__ gA,
-    uint32_t* __restrict__ flags, int M, int K, int N, float scale, int rows_per_image, int row_blocks, int band_rows_max) {
+    uint32_t* __restrict__ flags, int M, int K, int N, float scale, int rows_per_image, int row_blocks, int band_rows_max,
+    int conv_h, int conv_w, const float* __restrict__ zero_line) {
     __shared__ __align__(16) unsigned char smem[kGaStageBase + kGaStageBytes];
     constexpr bool F32 = FMT == kGaFmtF32, I16 = FMT == kGaFmtI16, HALF = FMT == kGaFmtHalf, F32W = FMT == kGaFmtF32W;
     constexpr bool WIDE = !HALF;                           // 16 (8) columns per tile, four chunk buffers
@@ -353,8 +361,12 @@ __global__ __launch_bounds__(kGaWaves * 64) void lutgemm_gradA_slab_kernel(
     const int total_tiles = row_blocks * k_groups;
     const int per_xcd = (total_tiles + 7) / 8;
     const int xcd = (int)(blockIdx.x % 8), pos_stride = (int)(gridDim.x / 8);
-    const int n_tiles = N / COLS;
+    // column tiles of a tile; CONV: (column tile of gC, tap) pairs, the nine taps of a column tile one after the other (their rows
+    // of gC are the same lines of memory shifted by a pixel or an image row)
+    constexpr int TAPS = CONV ? 9 : 1;
+    const int n_tiles = (N / COLS) * TAPS;
     const int total = n_tiles * CH;                          // chunks of a tile: (column tile, four k)
+    static_assert(!CONV || FMT == kGaFmtHalf, "the convolution-shaped walk is written for the half tables");
     if (HALF && flags[5] != 0u) return;                      // (set before this launch and never changed during it: every wave sees the same)
     const float offset = HALF ? (float)(int)flags[3] : 0.f;
     // 16-byte stores need gA aligned and, image-major, four consecutive rows in one image (same for every wave)
@@ -402,8 +414,16 @@ __global__ __launch_bounds__(kGaWaves * 64) void lutgemm_gradA_slab_kernel(
         if (q >= total) {
             if (nxt.valid) { q -= total; k0 = nxt.k0; } else q = total - 1;
         }
-        const int nt = q / CH, kc = q - nt * CH;
-        const u32x4* src = S + ((size_t)nt * (K / kGaChunkK) + k0 / kGaChunkK + kc) * (kGaChunkBytes / 16);
+        int nt = q / CH;
+        const int kc = q - nt * CH;
+        int k_quads = K / kGaChunkK;
+        if constexpr (CONV) {       // S covers the 9 C rows of B: tap-major, channel k0 of tap t is row t * C + k0
+            const int ct = nt;
+            nt = ct / TAPS;
+            k0 += (ct - nt * TAPS) * K;
+            k_quads *= TAPS;
+        }
+        const u32x4* src = S + ((size_t)nt * k_quads + k0 / kGaChunkK + kc) * (kGaChunkBytes / 16);
 #pragma unroll
         for (int i = 0; i < 2; ++i)
             __builtin_amdgcn_global_load_lds((gptr_t)(src + (wave + kGaWaves * i) * 64 + lane),
@@ -414,10 +434,52 @@ __global__ __launch_bounds__(kGaWaves * 64) void lutgemm_gradA_slab_kernel(
     // beyond the last column tile: the first one of the next tile
     constexpr int RPO = 64 * 16 / (COLS * 4);                // rows per wave-wide load (8 / 16)
     const uint32_t glane = (uint32_t)(lane / (64 / RPO)) * (uint32_t)N + 4u * (uint32_t)(lane % (64 / RPO));
+    // CONV: which neighbours of a pixel exist, for the four rows this lane requests (row 8 i + lane / 8 of the wave): bits
+    // 4 i .. 4 i + 3 = (row below exists, row above exists, pixel to the right exists, pixel to the left exists)
+    auto conv_neighbours = [&](int m_base) {
+        uint32_t vm = 0;
+        if constexpr (CONV) {
+            int ln = lane;
+            asm volatile("" : "+v"(ln));
+            const float inv_l = 1.0f / (float)rows_per_image, inv_w = 1.0f / (float)conv_w;
+#pragma unroll
+            for (int i = 0; i < ROWOPS; ++i) {
+                const int m = m_base + RPO * i + (ln >> 3);
+                const int pix = m - div_small(m, rows_per_image, inv_l) * rows_per_image;
+                const int y = div_small(pix, conv_w, inv_w), x = pix - y * conv_w;
+                vm |= (uint32_t)((y + 1 < conv_h) | ((y >= 1) << 1) | ((x + 1 < conv_w) << 2) | ((x >= 1) << 3)) << (4 * i);
+            }
+        }
+        return vm;
+    };
+    uint32_t neighbours = conv_neighbours(m_base_of(cur));
     auto request_rows = [&](int nt) {
         int m_base = m_base_of(cur);
+        bool of_next = false;
         if (nt >= n_tiles) {
-            if (nxt.valid) { nt = 0; m_base = m_base_of(nxt); } else nt = n_tiles - 1;
+            if (nxt.valid) { nt = 0; m_base = m_base_of(nxt); of_next = true; } else nt = n_tiles - 1;
+        }
+        if constexpr (CONV) {
+            const int ct = nt;
+            nt = ct / TAPS;
+            const int tap = ct - nt * TAPS;
+            const int ti = tap / 3, tj = tap - 3 * ti;
+            // the output position tap (ti, tj) connects pixel (y, x) to is (y + 1 - ti, x + 1 - tj)
+            const int shift = (1 - ti) * conv_w + (1 - tj);
+            const uint32_t need = (ti == 0 ? 1u : 0u) | (ti == 2 ? 2u : 0u) | (tj == 0 ? 4u : 0u) | (tj == 2 ? 8u : 0u);
+            // (the first rows of the next tile: its neighbour bits are worked out here, once, and again when it becomes current)
+            const uint32_t vm = of_next ? conv_neighbours(m_base) : neighbours;
+            const float* base = gC + ((size_t)m_base + shift) * N + nt * COLS;     // (shift < 0 never reaches below the rows that exist: see `need`)
+            int ln = lane;
+            asm volatile("" : "+v"(ln));
+            const float* zero = zero_line + 4 * (ln & 7);
+#pragma unroll
+            for (int i = 0; i < ROWOPS; ++i) {
+                const bool ok = ((vm >> (4 * i)) & need) == need;
+                const float* p = ok ? base + (size_t)(RPO * i) * N + glane : zero;
+                __builtin_amdgcn_global_load_lds((gptr_t)p, (lptr_t)(smem + STAGE_BASE + wave * STAGE_WAVE + i * 1024), 16, 0, 0);
+            }
+            return;
         }
         const float* base = gC + (size_t)m_base * N + nt * COLS;
 #pragma unroll
@@ -804,6 +866,7 @@ __global__ __launch_bounds__(kGaWaves * 64) void lutgemm_gradA_slab_kernel(
         cur = nxt;
         pos += pos_stride;
         nxt = decode(pos + pos_stride);
+        if constexpr (CONV) neighbours = conv_neighbours(m_base_of(cur));
         return true;
     };
     int nt = 0;
@@ -867,14 +930,54 @@ hipError_t launch_gradA_slab(const float* gC, const uint8_t* A, const uint8_t* B
     const dim3 grid(8 * (per_xcd < cus_per_xcd ? per_xcd : cus_per_xcd));
     if (kt == 32)
         hipLaunchKernelGGL((lutgemm_gradA_slab_kernel<32, kGaFmtHalf>), grid, block, 0, stream, gC, A, S4, gA, flags, M, K, N, scale,
-                           rows_per_image, row_blocks, band_rows);
+                           rows_per_image, row_blocks, band_rows, 0, 0, (const float*)nullptr);
     else
         hipLaunchKernelGGL((lutgemm_gradA_slab_kernel<16, kGaFmtHalf>), grid, block, 0, stream, gC, A, S4, gA, flags, M, K, N, scale,
-                           rows_per_image, row_blocks, band_rows);
+                           rows_per_image, row_blocks, band_rows, 0, 0, (const float*)nullptr);
     e = hipGetLastError();
     if (e != hipSuccess) return e;
     // masked codes in A or table entries a half cannot hold: the gated direct kernel recomputes gA
     return launch_gradA(gC, A, B, gA, lut, g, M, K, N, scale, n_cu, stream, flags + 2, rows_per_image);
+}
+
+// ------------------------------------------------------------------------------------------ convolution-shaped gradA
+// Input gradient of a 3x3 / stride 1 / padding 1 convolution as one implicit GEMM over the B*H*W input pixels (see CONV
+// above).  codes [B*H*W][C] pixel-major, Bt [9*C][N] tap-major, g_in [B][C][H*W].  Same conditions on the table as the
+// GEMM-shaped kernel (flags[5] set by bwd_header_kernel: the kernel returns at once; a masked code or an entry a half
+// cannot hold raises flags[2]); what the caller queues behind for those cases is its business.
+bool gradA_slab_conv_applies(const LutGeom& g, long M, int C, int N, const float* gC, bool force) {
+    if (!force && (M < 1024 || (double)M * C * 9 * N < 1e8)) return false;
+    return g.bits <= 7 && M >= 512 && (N % kGaCols) == 0 && (C % 16) == 0 && (size_t)M * C < (1ull << 31) && M < (1L << 23) &&
+           ((uintptr_t)gC & 15) == 0;
+}
+size_t gradA_slab_conv_workspace_bytes(int C, int N) { return (size_t)(N / kGaCols) * (9 * C / kGaChunkK) * kGaChunkBytes; }
+
+hipError_t launch_gradA_slab_conv(const float* gC, const uint8_t* codes, const uint8_t* Bt, float* g_in, const int16_t* lut,
+                                  const LutGeom& g, int Bn, int C, int H, int W, int N, float scale, int n_cu, uint32_t* flags,
+                                  void* S, const float* zero_line, hipStream_t stream) {
+    const int lut_dwords = g.rows * g.cols / 2;
+    const int K = 9 * C, M = Bn * H * W;
+    const int qpw = (long)(N / kGaCols) * ((K / 4 + 3) / 4) >= n_cu ? 4 : 1;
+    hipLaunchKernelGGL(expand_gradA_kernel, dim3(N / kGaCols, (K / 4 + qpw - 1) / qpw), dim3(256), (size_t)lut_dwords * 4, stream, Bt,
+                       reinterpret_cast<const uint32_t*>(lut), lut_dwords, g.cols, 1 << g.bits, reinterpret_cast<uint32_t*>(S),
+                       flags, K, N, qpw);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    const u32x4* S4 = reinterpret_cast<const u32x4*>(S);
+    const dim3 block(kGaWaves * 64);
+    const int row_blocks = (M + kGaRows - 1) / kGaRows;
+    const int band_rows = 16;
+    const int kt = ((C % 32) == 0 && row_blocks * (C / 32) >= n_cu) ? 32 : 16;
+    const int tiles = row_blocks * (C / kt);
+    const int per_xcd = (tiles + 7) / 8, cus_per_xcd = n_cu >= 8 ? n_cu / 8 : 1;
+    const dim3 grid(8 * (per_xcd < cus_per_xcd ? per_xcd : cus_per_xcd));
+    if (kt == 32)
+        hipLaunchKernelGGL((lutgemm_gradA_slab_kernel<32, kGaFmtHalf, true>), grid, block, 0, stream, gC, codes, S4, g_in, flags, M, C, N,
+                           scale, H * W, row_blocks, band_rows, H, W, zero_line);
+    else
+        hipLaunchKernelGGL((lutgemm_gradA_slab_kernel<16, kGaFmtHalf, true>), grid, block, 0, stream, gC, codes, S4, g_in, flags, M, C, N,
+                           scale, H * W, row_blocks, band_rows, H, W, zero_line);
+    return hipGetLastError();
 }
 
 // ------------------------------------------------------------------------------------------ 8-bit tables
@@ -914,10 +1017,10 @@ hipError_t launch_gradA_slab_i16(const float* gC, const uint8_t* A, const uint8_
     const dim3 grid(8 * (per_xcd < cus_per_xcd ? per_xcd : cus_per_xcd));
     if (kt == 32)
         hipLaunchKernelGGL((lutgemm_gradA_slab_kernel<32, kGaFmtI16>), grid, block, 0, stream, gC, A, S4, gA, flags, M, K, N, scale,
-                           rows_per_image, row_blocks, band_rows);
+                           rows_per_image, row_blocks, band_rows, 0, 0, (const float*)nullptr);
     else
         hipLaunchKernelGGL((lutgemm_gradA_slab_kernel<16, kGaFmtI16>), grid, block, 0, stream, gC, A, S4, gA, flags, M, K, N, scale,
-                           rows_per_image, row_blocks, band_rows);
+                           rows_per_image, row_blocks, band_rows, 0, 0, (const float*)nullptr);
     return hipGetLastError();
 }
 
@@ -951,10 +1054,10 @@ hipError_t launch_gradA_slab_f32w(const float* gC, const uint8_t* A, const uint8
     const dim3 grid(8 * (per_xcd < cus_per_xcd ? per_xcd : cus_per_xcd));
     if (kt == 32)
         hipLaunchKernelGGL((lutgemm_gradA_slab_kernel<32, kGaFmtF32W>), grid, block, 0, stream, gC, A, S4, gA, flags, M, K, N, scale,
-                           rows_per_image, row_blocks, band_rows);
+                           rows_per_image, row_blocks, band_rows, 0, 0, (const float*)nullptr);
     else
         hipLaunchKernelGGL((lutgemm_gradA_slab_kernel<16, kGaFmtF32W>), grid, block, 0, stream, gC, A, S4, gA, flags, M, K, N, scale,
-                           rows_per_image, row_blocks, band_rows);
+                           rows_per_image, row_blocks, band_rows, 0, 0, (const float*)nullptr);
     return hipGetLastError();
 }
 
@@ -995,10 +1098,10 @@ hipError_t launch_gradA_slab_f32tab(const float* gC, const uint8_t* A, const uin
     const dim3 grid(8 * (per_xcd < cus_per_xcd ? per_xcd : cus_per_xcd));
     if (kt == 32)
         hipLaunchKernelGGL((lutgemm_gradA_slab_kernel<32, kGaFmtF32>), grid, block, 0, stream, gC, A, S4, gA, flags, M, K, N, scale,
-                           rows_per_image, row_blocks, band_rows);
+                           rows_per_image, row_blocks, band_rows, 0, 0, (const float*)nullptr);
     else
         hipLaunchKernelGGL((lutgemm_gradA_slab_kernel<16, kGaFmtF32>), grid, block, 0, stream, gC, A, S4, gA, flags, M, K, N, scale,
-                           rows_per_image, row_blocks, band_rows);
+                           rows_per_image, row_blocks, band_rows, 0, 0, (const float*)nullptr);
     e = hipGetLastError();
     if (e != hipSuccess) return e;
     return launch_gradA_f32tab(gC, A, B, gA, lut, g, M, K, N, scale, n_cu, stream, flags + 2, rows_per_image);

@@ -292,6 +292,31 @@ int amr_im2col_nhwc_u8(const uint8_t *codes, uint8_t *A, int B, int C, int H, in
 int amr_conv_input_grad_f32(const float *cols, const float *t, const float *z_w, const uint8_t *inside, const float *scale,
                             float *gx, int B, int C, int H, int W, int kh, int kw, int stride, int pad, int dil, void *stream);
 
+/*
+ * Input gradient of a quantised 3x3 LUT convolution of stride 1 and padding 1 WITHOUT the [M][9C] gradient matrix: gradA of
+ * amr_lut_gemm_backward_ex, amr_col2im_f32 and amr_conv_input_grad_f32 as one implicit GEMM over the B*H*W input pixels,
+ *   gx[b,c,y,x] = inside[b,c,y,x] ? ((1/16) * sum over taps (ti,tj) and n of gC[(b, y+1-ti, x+1-tj), n] *
+ *                 (float)lut_grad_a[codes[(b,y,x), c] * cols + Bt[(ti*3+tj)*C + c, n]] + *z_w * sum over taps of t[(b, y+1-ti, x+1-tj)]) / *scale : 0
+ * (positions outside the image contribute nothing).  gC [B*H*W, N] float32 (the GEMM rows of the output gradient), codes
+ * [B*H*W, C] uint8 pixel-major (amr_quantize_codes_nhwc_u8), Bt [9*C, N] uint8 tap-major, t / z_w / inside / scale as in
+ * amr_conv_input_grad_f32.  What the reference obtains from approx_gemm_backward_gpu
+ * (self_ops/src/approx_gemm_backward.cu:506-624) followed by autograd's fold (self_ops/ops_py/approx_ops.py:558) and the
+ * quantiser's backward (micronet+/app_layers.py:147-160); sums in another order, results to fp32 summation-order tolerance.
+ * Served shapes: amr_lut_conv_input_grad_supported(...) != 0 (tables of at most 7 bits, C % 16 == 0, N % 32 == 0, at least
+ * 1024 pixels, gC 16-byte aligned), else AMR_EUNSUPPORTED and nothing is launched.
+ * A gradient table that cannot be held as halves (amr_grad_table_fits_halves(host copy) == 0) or an operand holding the masked
+ * code 2^b needs the GEMM-shaped path: pass A_fallback [B*H*W, 9*C] (amr_im2col_nhwc_u8 of codes) and cols_fallback (scratch,
+ * B*9*C*H*W floats) and the library queues it, gated on the device-side flag; with both NULL such a call fills gx with NaN.
+ * workspace: amr_lut_conv_input_grad_workspace_bytes(...) bytes, 256-byte aligned, required.
+ */
+int amr_lut_conv_input_grad_supported(int64_t lut_elems, int B, int C, int H, int W, int N);
+size_t amr_lut_conv_input_grad_workspace_bytes(int64_t lut_elems, int B, int C, int H, int W, int N);
+int amr_grad_table_fits_halves(const int16_t *host_table, int64_t lut_elems);      /* host pointer; 1, 0 or a negative AMR_E* */
+int amr_lut_conv_input_grad_f32(const float *gC, const uint8_t *codes, const uint8_t *Bt, const int16_t *lut_grad_a,
+                                int64_t lut_elems, const float *t, const float *z_w, const uint8_t *inside, const float *scale,
+                                float *gx, int B, int C, int H, int W, int N, const uint8_t *A_fallback, float *cols_fallback,
+                                void *workspace, size_t workspace_bytes, void *stream);
+
 /* amr_conv_dequant_backward_f32 that also leaves t[m] = sum over n of g_c[m, n] (ascending n), in the same pass. */
 int amr_conv_dequant_backward_rowsum_f32(const float *g, const float *s_a, const float *s_w, float *g_c, float *t, int batch,
                                          int out_channels, int positions, void *stream);

@@ -230,3 +230,132 @@ def test_forward_with_dequantising_store_equals_gemm_then_dequantisation(ops, or
     rows = slice(0, min(M, 2048))
     assert (c[rows].cpu().numpy() == oracle.forward_c(A[rows], B, flat, bits).astype(np.float32)).all()
     assert torch.equal(got, want)
+
+
+def _conv_grad_case(oracle, seed, bn, c, h, w, n, lo=-1024, hi=3073, masked=False):
+    """Operands of one input-gradient problem of a 3x3 / stride 1 / padding 1 convolution and its float64 answer."""
+    rng = np.random.default_rng(seed)
+    x_codes = rng.integers(0, 128, (bn, c, h, w)).astype(np.uint8)
+    if masked:
+        x_codes[bn // 2, 3, h // 2, w // 2] = 128
+    bt = rng.integers(0, 128, (9 * c, n)).astype(np.uint8)                              # rows (tap, channel)
+    la = oracle.pack_table(rng.integers(lo, hi, (128, 128)), 7, np.int16)
+    g_rows = rng.standard_normal((bn * h * w, n)).astype(np.float32)
+    t = g_rows.sum(axis=1)
+    inside = (rng.random((bn, c, h, w)) < 0.85).astype(np.uint8)
+    zw, scale = -61.0, 0.037
+    a_ref, _, _ = oracle.im2col_np(x_codes, 3, 3, 1, 1, 1)                              # columns (channel, tap)
+    a_tap = a_ref.reshape(-1, c, 9).transpose(0, 2, 1).reshape(-1, 9 * c)
+    ga64, _ = oracle.backward_c_f64(g_rows, a_tap, bt, la, la, 7)
+    cols = torch.tensor(ga64).view(bn, h * w, 9, c).permute(0, 3, 2, 1).reshape(bn, c * 9, h * w)      # fold's (channel, tap) order
+    fold = lambda cc: F.fold(cc, (h, w), (3, 3), padding=1)
+    t_cols = torch.tensor(t, dtype=torch.float64).view(bn, 1, h * w).expand(bn, 9, h * w)
+    want = (fold(cols) + zw * fold(t_cols)) / scale * torch.tensor(inside, dtype=torch.float64)
+    codes = np.ascontiguousarray(x_codes.transpose(0, 2, 3, 1).reshape(bn * h * w, c))
+    return dict(codes=codes, a_tap=a_tap, bt=bt, la=la, g_rows=g_rows, t=t, inside=inside, zw=zw, scale=scale, want=want)
+
+
+@pytest.mark.parametrize("bn,c,h,w,n", [
+    (2, 16, 16, 16, 32),        # one block of 512 pixels, 16 channels per tile
+    (8, 64, 32, 32, 64),        # conv2_x of the benchmark network: 32 channels per tile, half an image per tile
+    (3, 48, 16, 16, 96),        # channels and columns that are multiples of 16 / 32 only
+    (40, 16, 4, 4, 32),         # 4x4 images: most pixels sit on a border
+    (3, 16, 15, 17, 32),        # sizes that are no powers of two, pixel count no multiple of 32, 255 positions per image
+    (10, 32, 8, 8, 128),        # four column tiles
+])
+def test_convolution_shaped_input_gradient_against_oracle_and_gemm_shaped_path(ops, oracle, bn, c, h, w, n):
+    """amr_lut_conv_input_grad_f32 (implicit GEMM over the input pixels) against the float64 oracle (LUT gradient GEMM, fold,
+    zero-point term, straight-through mask) and against the library's GEMM-shaped composition of the same steps."""
+    import approx_ops
+    print("conv-shaped gradA", bn, c, h, w, n, flush=True)
+    k = _conv_grad_case(oracle, 31, bn, c, h, w, n)
+    dev = lambda v, dt=None: torch.tensor(v, device="cuda", dtype=dt)
+    codes, a_tap, bt, la, g_rows, t, inside = (dev(k[x]) for x in ("codes", "a_tap", "bt", "la", "g_rows", "t", "inside"))
+    zw, scale = dev([k["zw"]], torch.float32), dev([k["scale"]], torch.float32)
+    old = approx_ops._lib.amr_set_expanded_table_kernels(2)
+    try:
+        assert approx_ops.conv_input_grad_supported(la, (bn, c, h, w), n)
+        gx = torch.full((bn, c, h, w), float("nan"), device="cuda")
+        approx_ops.approx_conv_input_grad(g_rows, codes, bt, la, t, zw, inside, scale, gx)
+        cols = torch.empty((bn, 9 * c, h * w), device="cuda")
+        approx_ops.approx_gemm_backward(g_rows, a_tap, bt, cols, None, la, la, ga_rows_per_image=h * w)
+        gx2 = torch.full((bn, c, h, w), float("nan"), device="cuda")
+        approx_ops.conv_input_grad(cols, t, zw, inside, scale, gx2, (3, 3), 1, 1, 1)
+    finally:
+        approx_ops._lib.amr_set_expanded_table_kernels(old)
+    want = k["want"].cuda()
+    tol = 1e-5 * float(want.abs().max())
+    torch.testing.assert_close(gx.double(), want, rtol=0, atol=tol)
+    torch.testing.assert_close(gx2.double(), want, rtol=0, atol=tol)
+    assert (gx[inside == 0] == 0).all()
+
+
+def test_convolution_shaped_input_gradient_fall_backs(ops, oracle):
+    """A gradient table that cannot be held as halves, and a masked code among the operand codes: with the window matrix as
+    fall-back operand the GEMM-shaped kernels queued behind give the oracle's answer; without it the result is NaN, not a
+    silently wrong gradient.  Shapes the kernel does not serve are refused before anything is launched."""
+    import approx_ops
+    print("conv-shaped gradA fall-backs", flush=True)
+    bn, c, h, w, n = 4, 32, 16, 16, 64
+    dev = lambda v, dt=None: torch.tensor(v, device="cuda", dtype=dt)
+    old = approx_ops._lib.amr_set_expanded_table_kernels(2)
+    try:
+        for name, kw in (("wide table", dict(lo=-20000, hi=20000)), ("masked code", dict(masked=True))):
+            k = _conv_grad_case(oracle, 32, bn, c, h, w, n, **kw)
+            assert approx_ops.grad_table_fits_halves(k["la"]) == (name == "masked code")
+            codes, a_tap, bt, la, g_rows, t, inside = (dev(k[x]) for x in ("codes", "a_tap", "bt", "la", "g_rows", "t", "inside"))
+            zw, scale = dev([k["zw"]], torch.float32), dev([k["scale"]], torch.float32)
+            gx = torch.full((bn, c, h, w), 5.0, device="cuda")
+            approx_ops.approx_conv_input_grad(g_rows, codes, bt, la, t, zw, inside, scale, gx, a_fallback=a_tap)
+            want = k["want"].cuda()
+            torch.testing.assert_close(gx.double(), want, rtol=0, atol=1e-5 * float(want.abs().max()), msg=name)
+            gx.fill_(5.0)
+            approx_ops.approx_conv_input_grad(g_rows, codes, bt, la, t, zw, inside, scale, gx)
+            assert torch.isnan(gx).all(), name
+        # refused: fewer than 512 pixels; channels no multiple of 16; 8-bit table
+        la7 = dev(oracle.pack_table(np.zeros((128, 128), np.int64), 7, np.int16))
+        la8 = dev(oracle.pack_table(np.zeros((256, 256), np.int64), 8, np.int16))
+        assert not approx_ops.conv_input_grad_supported(la7, (1, 16, 16, 16), 32)
+        assert not approx_ops.conv_input_grad_supported(la7, (4, 24, 16, 16), 32)
+        assert not approx_ops.conv_input_grad_supported(la8, (4, 32, 16, 16), 32)
+        assert approx_ops.conv_input_grad_supported(la7, (4, 32, 16, 16), 32)
+        with pytest.raises(RuntimeError, match="not served"):
+            approx_ops.approx_conv_input_grad(torch.zeros(256, 32, device="cuda"), torch.zeros((256, 16), dtype=torch.uint8, device="cuda"),
+                                              torch.zeros((144, 32), dtype=torch.uint8, device="cuda"), la7, torch.zeros(256, device="cuda"),
+                                              zw, torch.zeros((1, 16, 16, 16), dtype=torch.uint8, device="cuda"), scale,
+                                              torch.zeros(1, 16, 16, 16, device="cuda"))
+    finally:
+        approx_ops._lib.amr_set_expanded_table_kernels(old)
+
+
+def test_uint8_layer_takes_the_convolution_shaped_input_gradient(ops):
+    """A layer of the benchmark network's size (32 -> 64 channels, 32 x 32, batch 8) takes the implicit-GEMM input gradient
+    by itself; its gradients agree with the float-code path."""
+    import app_layers as L
+    import approx_ops
+    print("layer, conv-shaped gradA", flush=True)
+    torch.manual_seed(9)
+    layer = L.ApproxConv2d(32, 64, 3, stride=1, padding=1, bias=False, a_bits=7, w_bits=7).cuda().train()
+    x = torch.randn(8, 32, 32, 32, device="cuda")
+    layer(x)
+    layer.eval()
+    calls = []
+    native = approx_ops.approx_conv_input_grad
+    approx_ops.approx_conv_input_grad = lambda *a, **k: (calls.append(1), native(*a, **k))[1]
+    try:
+        res = []
+        gy = None
+        for fused in (True, False):
+            layer.fused_layer = fused
+            xi = x.clone().requires_grad_()
+            layer.zero_grad()
+            y = layer(xi)
+            gy = torch.randn_like(y) if gy is None else gy
+            y.backward(gy)
+            res.append((y.detach(), xi.grad, layer.weight.grad.clone()))
+    finally:
+        approx_ops.approx_conv_input_grad = native
+    assert len(calls) == 1
+    assert torch.equal(res[0][0], res[1][0])
+    for a, b in zip(res[0][1:], res[1][1:]):
+        torch.testing.assert_close(a, b, rtol=0, atol=1e-5 * float(b.abs().max()))
