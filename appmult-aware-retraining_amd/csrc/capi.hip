@@ -105,7 +105,10 @@ bool gradA_slab_conv_applies(const LutGeom& g, long M, int C, int N, const float
 size_t gradA_slab_conv_workspace_bytes(int C, int N);
 hipError_t launch_gradA_slab_conv(const float* gC, const uint8_t* codes, const uint8_t* Bt, float* g_in, const int16_t* lut,
                                   const LutGeom& g, int Bn, int C, int H, int W, int N, float scale, int n_cu, uint32_t* flags,
-                                  void* S, const float* zero_line, hipStream_t stream);
+                                  void* S, const float* zero_line, hipStream_t stream, const float* zt, const float* zw,
+                                  const float* qscale, const uint8_t* inside);
+bool gradA_slab_conv_can_finish(int Bn, int H, int W, const float* g_in);
+hipError_t launch_window_sums_3x3(const float* t, float* zt, long B, int H, int W, hipStream_t stream);
 hipError_t launch_dequant_grad_rowsum(const float* g, const float* sa, const float* sw, float* gc, float* t, int M, int N, int L,
                                       hipStream_t stream);
 hipError_t launch_accgemm(const float* A, const float* B, float* C, int M, int K, int N, hipStream_t stream);
@@ -809,9 +812,12 @@ int amr_lut_conv_input_grad_supported(int64_t lut_elems, int B, int C, int H, in
     return mode && amr::gradA_slab_conv_applies(g, (long)B * H * W, C, N, nullptr, mode == 2) ? 1 : 0;
 }
 
+// scratch of the convolution-shaped gradA: [256 B of flags][window sums of t, B*H*W floats][expanded table]
+static size_t conv_grad_zt_bytes(int B, int H, int W) { return ((size_t)B * H * W * sizeof(float) + 255) & ~(size_t)255; }
+
 size_t amr_lut_conv_input_grad_workspace_bytes(int64_t lut_elems, int B, int C, int H, int W, int N) {
     if (!amr_lut_conv_input_grad_supported(lut_elems, B, C, H, W, N)) return 0;
-    return 256 + amr::gradA_slab_conv_workspace_bytes(C, N);
+    return 256 + conv_grad_zt_bytes(B, H, W) + amr::gradA_slab_conv_workspace_bytes(C, N);
 }
 
 // The decision bwd_header_kernel takes on the device (lutgemm_bwd_slab.hip), for a table in host memory.
@@ -851,7 +857,8 @@ int amr_lut_conv_input_grad_f32(const float* gC, const uint8_t* codes, const uin
     const long M = (long)B * H * W;
     if (!mode || !amr::gradA_slab_conv_applies(g, M, C, N, gC, mode == 2))
         return fail(AMR_EUNSUPPORTED, "shape, alignment or mode not served by the convolution-shaped gradA (ask amr_lut_conv_input_grad_supported)");
-    const size_t need = 256 + amr::gradA_slab_conv_workspace_bytes(C, N);
+    const size_t zt_bytes = conv_grad_zt_bytes(B, H, W);
+    const size_t need = 256 + zt_bytes + amr::gradA_slab_conv_workspace_bytes(C, N);
     if (!workspace || workspace_bytes < need)
         return fail(AMR_EWORKSPACE, "workspace of %zu bytes is smaller than the %zu required", workspace ? workspace_bytes : (size_t)0, need);
     if ((uintptr_t)workspace & 255) return fail(AMR_EINVAL, "workspace must be 256-byte aligned");
@@ -863,12 +870,21 @@ int amr_lut_conv_input_grad_f32(const float* gC, const uint8_t* codes, const uin
     uint32_t* flags = reinterpret_cast<uint32_t*>(workspace);
     hipError_t e = amr::launch_bwd_header(lut_grad_a, nullptr, g, flags, s);      // clears the 64 flag words: words 32..63 stay zero
     if (e != hipSuccess) return hip_fail(e, "scratch header launch");
+    // Where every wave stores whole 16-byte pieces the kernel finishes the gradient in its store (mask, zero-point term,
+    // quantiser scale); the channel-independent window sums of t it needs for that are formed first.
+    const bool finish = amr::gradA_slab_conv_can_finish(B, H, W, gx);
+    float* zt = reinterpret_cast<float*>(reinterpret_cast<unsigned char*>(workspace) + 256);
+    if (finish && (e = amr::launch_window_sums_3x3(t, zt, B, H, W, s)) != hipSuccess) return hip_fail(e, "window sums launch");
     e = amr::launch_gradA_slab_conv(gC, codes, Bt, gx, lut_grad_a, g, B, C, H, W, N, factor, n_cu, flags,
-                                    reinterpret_cast<unsigned char*>(workspace) + 256, reinterpret_cast<const float*>(flags + 32), s);
+                                    reinterpret_cast<unsigned char*>(workspace) + 256 + zt_bytes, reinterpret_cast<const float*>(flags + 32), s,
+                                    finish ? zt : nullptr, z_w, scale, inside);
     if (e != hipSuccess) return hip_fail(e, "gradA launch");
     // flags[2]: a masked code, an entry a half cannot hold, or a table that cannot be held as halves at all
     const bool fallback = A_fallback != nullptr;
-    e = amr::launch_conv_input_grad(nullptr, t, z_w, inside, scale, gx, B, C, H, W, 3, 3, 1, 1, 1, H, W, s, flags + 2, fallback ? 1 : 3);
+    if (!finish)
+        e = amr::launch_conv_input_grad(nullptr, t, z_w, inside, scale, gx, B, C, H, W, 3, 3, 1, 1, 1, H, W, s, flags + 2, fallback ? 1 : 3);
+    else if (!fallback)
+        e = amr::launch_conv_input_grad(nullptr, t, z_w, inside, scale, gx, B, C, H, W, 3, 3, 1, 1, 1, H, W, s, flags + 2, 4);
     if (e != hipSuccess) return hip_fail(e, "input gradient launch");
     if (fallback) {
         e = amr::launch_gradA(gC, A_fallback, Bt, cols_fallback, lut_grad_a, g, (int)M, 9 * C, N, factor, n_cu, s, flags + 2, H * W);

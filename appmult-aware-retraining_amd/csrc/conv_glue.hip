@@ -171,12 +171,16 @@ __global__ __launch_bounds__(256) void conv_input_grad_kernel(const float* __res
     if (idx >= total) return;
     // gate_mode 1: the pass behind a kernel that left the tap sums in gx -- when *gate says that kernel could not do its work,
     // this pass leaves gx alone (a recomputation is queued behind, gate_mode 2) or, gate_mode 3, marks every element NaN;
-    // gate_mode 2: runs only when *gate is set.
+    // gate_mode 2: runs only when *gate is set; gate_mode 4: marks every element NaN when *gate is set and does nothing else.
     if (gate_mode != 0) {
         const bool raised = *gate != 0u;
         if (gate_mode == 2 && !raised) return;
         if (gate_mode == 1 && raised) return;
         if (gate_mode == 3 && raised) { gx[idx] = __builtin_nanf(""); return; }
+        if (gate_mode == 4) {      // behind a kernel that finished gx itself: only the NaN marking is left to do
+            if (raised) gx[idx] = __builtin_nanf("");
+            return;
+        }
     }
     const int kh = KH ? KH : kh_rt, kw = KW ? KW : kw_rt, stride = STRIDE ? STRIDE : stride_rt;
     const int xx = (int)(idx % W);
@@ -250,6 +254,34 @@ hipError_t launch_conv_input_grad(const float* cols, const float* t, const float
     else if (kh == 1 && kw == 1 && stride == 2) AMR_CIG(1, 1, 2);
     else AMR_CIG(0, 0, 0);
 #undef AMR_CIG
+    return hipGetLastError();
+}
+
+// zt[b][y][x] = sum of t[b][pos] over the output positions a 3x3 / stride 1 / padding 1 window connects pixel (y, x) to
+// (ascending tap order): the channel-independent part of the input gradient, for the kernel that finishes the gradient in
+// its own store.
+__global__ __launch_bounds__(256) void window_sums_3x3_kernel(const float* __restrict__ t, float* __restrict__ zt, int H, int W, size_t total) {
+    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= total) return;
+    const int x = (int)(idx % W);
+    const int y = (int)((idx / W) % H);
+    float acc = 0.f;
+#pragma unroll
+    for (int i = 0; i < 3; ++i)
+#pragma unroll
+        for (int j = 0; j < 3; ++j) {
+            const int oy = y + 1 - i, ox = x + 1 - j;
+            const bool ok = oy >= 0 && oy < H && ox >= 0 && ox < W;
+            const float v = t[ok ? idx + (size_t)((1 - i) * W + (1 - j)) : idx];
+            acc += ok ? v : 0.f;
+        }
+    zt[idx] = acc;
+}
+
+hipError_t launch_window_sums_3x3(const float* t, float* zt, long B, int H, int W, hipStream_t stream) {
+    const size_t total = (size_t)B * H * W;
+    if (total == 0) return hipSuccess;
+    hipLaunchKernelGGL(window_sums_3x3_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, t, zt, H, W, total);
     return hipGetLastError();
 }
 

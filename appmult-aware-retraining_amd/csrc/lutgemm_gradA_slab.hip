@@ -322,11 +322,20 @@ __device__ __forceinline__ void ga_store16(float* p, const u32x4& q) {
 // positions that tap connects the pixel to: row m + (1 - ti) * W + (1 - tj), or a line of zeros where that position lies
 // outside the image.  The sums over taps and columns stay in the accumulators, so neither the [M][9C] gradient matrix
 // nor its col2im pass exists; gA receives [B][C][H*W] (rows_per_image = H*W).  A tile lasts nine times as many chunk steps.
+// CONV only: what the store needs to finish the input gradient of the quantised layer on the spot,
+//   gx = inside ? (tap sums + *zw * zt[pixel]) / *scale : 0     (zt == nullptr: the tap sums are stored as they are)
+struct GaFinish {
+    const float* zt;          // [B*H*W] window sums of the output gradient's row sums
+    const float* zw;          // device scalars
+    const float* scale;
+    const uint8_t* inside;    // [B][C][H*W]
+};
+
 template <int kGaKT, int FMT, bool CONV = false>
 __global__ __launch_bounds__(kGaWaves * 64) void lutgemm_gradA_slab_kernel(
     const float* __restrict__ gC, const uint8_t* __restrict__ A, const u32x4* __restrict__ S, float* __restrict__ gA,
     uint32_t* __restrict__ flags, int M, int K, int N, float scale, int rows_per_image, int row_blocks, int band_rows_max,
-    int conv_h, int conv_w, const float* __restrict__ zero_line) {
+    int conv_h, int conv_w, const float* __restrict__ zero_line, GaFinish fin) {
     __shared__ __align__(16) unsigned char smem[kGaStageBase + kGaStageBytes];
     constexpr bool F32 = FMT == kGaFmtF32, I16 = FMT == kGaFmtI16, HALF = FMT == kGaFmtHalf, F32W = FMT == kGaFmtF32W;
     constexpr bool WIDE = !HALF;                           // 16 (8) columns per tile, four chunk buffers
@@ -811,7 +820,18 @@ __global__ __launch_bounds__(kGaWaves * 64) void lutgemm_gradA_slab_kernel(
                 const uint32_t rd = tbase + (uint32_t)(kl0 * 128 + (((4 * pp) ^ (16 * ((kl0 >> 1) & 1))) << 2));
                 const int m4 = m_base + 4 * pp;
                 const int img = m4 / rows_per_image, l = m4 - img * rows_per_image;
-                float* out = gA + ((size_t)img * K + cur.k0 + kl0) * rows_per_image + l;
+                const size_t out_off = ((size_t)img * K + cur.k0 + kl0) * rows_per_image + l;
+                float* out = gA + out_off;
+                // (CONV with a finishing store: the host only asks for it where every wave takes this branch)
+                const bool finish = CONV && fin.zt != nullptr;
+                f32x4 zt4 = {0.f, 0.f, 0.f, 0.f};
+                float inv_den = 1.f;
+                if (finish) {
+                    zt4 = *reinterpret_cast<const f32x4*>(fin.zt + m4);
+                    const float zw = *fin.zw;
+                    zt4 = zt4 * zw;
+                    inv_den = *fin.scale;
+                }
 #pragma unroll
                 for (int h = 0; h < 2; ++h) {
 #pragma unroll
@@ -823,7 +843,20 @@ __global__ __launch_bounds__(kGaWaves * 64) void lutgemm_gradA_slab_kernel(
                     u32x4 q[CH / 4];
                     ga_lds_get<CH / 4, 8 * 128>(q, rd);
 #pragma unroll
-                    for (int i = 0; i < CH / 4; ++i) ga_store16(out + (size_t)(h * KH + 8 * i) * rows_per_image, q[i]);
+                    for (int i = 0; i < CH / 4; ++i) {
+                        const size_t ko = (size_t)(h * KH + 8 * i) * rows_per_image;
+                        if (finish) {
+                            const uint32_t in4 = *reinterpret_cast<const uint32_t*>(fin.inside + out_off + ko);
+                            f32x4 v = __builtin_bit_cast(f32x4, q[i]);
+                            v = v + zt4;
+                            v.x = (in4 & 0xffu) ? v.x / inv_den : 0.f;
+                            v.y = (in4 & 0xff00u) ? v.y / inv_den : 0.f;
+                            v.z = (in4 & 0xff0000u) ? v.z / inv_den : 0.f;
+                            v.w = (in4 & 0xff000000u) ? v.w / inv_den : 0.f;
+                            q[i] = __builtin_bit_cast(u32x4, v);
+                        }
+                        ga_store16(out + ko, q[i]);
+                    }
                 }
             }
         } else {
@@ -930,10 +963,10 @@ hipError_t launch_gradA_slab(const float* gC, const uint8_t* A, const uint8_t* B
     const dim3 grid(8 * (per_xcd < cus_per_xcd ? per_xcd : cus_per_xcd));
     if (kt == 32)
         hipLaunchKernelGGL((lutgemm_gradA_slab_kernel<32, kGaFmtHalf>), grid, block, 0, stream, gC, A, S4, gA, flags, M, K, N, scale,
-                           rows_per_image, row_blocks, band_rows, 0, 0, (const float*)nullptr);
+                           rows_per_image, row_blocks, band_rows, 0, 0, (const float*)nullptr, GaFinish{});
     else
         hipLaunchKernelGGL((lutgemm_gradA_slab_kernel<16, kGaFmtHalf>), grid, block, 0, stream, gC, A, S4, gA, flags, M, K, N, scale,
-                           rows_per_image, row_blocks, band_rows, 0, 0, (const float*)nullptr);
+                           rows_per_image, row_blocks, band_rows, 0, 0, (const float*)nullptr, GaFinish{});
     e = hipGetLastError();
     if (e != hipSuccess) return e;
     // masked codes in A or table entries a half cannot hold: the gated direct kernel recomputes gA
@@ -952,9 +985,17 @@ bool gradA_slab_conv_applies(const LutGeom& g, long M, int C, int N, const float
 }
 size_t gradA_slab_conv_workspace_bytes(int C, int N) { return (size_t)(N / kGaCols) * (9 * C / kGaChunkK) * kGaChunkBytes; }
 
+// Whether the kernel's store can finish the gradient (mask, zero-point term, quantiser scale) for this geometry: every
+// wave must take the branch of 16-byte image-major stores.
+bool gradA_slab_conv_can_finish(int Bn, int H, int W, const float* g_in) {
+    return ((long)Bn * H * W) % kGaRowsPerWave == 0 && ((H * W) & 3) == 0 && ((uintptr_t)g_in & 15) == 0;
+}
+
 hipError_t launch_gradA_slab_conv(const float* gC, const uint8_t* codes, const uint8_t* Bt, float* g_in, const int16_t* lut,
                                   const LutGeom& g, int Bn, int C, int H, int W, int N, float scale, int n_cu, uint32_t* flags,
-                                  void* S, const float* zero_line, hipStream_t stream) {
+                                  void* S, const float* zero_line, hipStream_t stream, const float* zt, const float* zw,
+                                  const float* qscale, const uint8_t* inside) {
+    const GaFinish fin{zt, zw, qscale, inside};
     const int lut_dwords = g.rows * g.cols / 2;
     const int K = 9 * C, M = Bn * H * W;
     const int qpw = (long)(N / kGaCols) * ((K / 4 + 3) / 4) >= n_cu ? 4 : 1;
@@ -973,10 +1014,10 @@ hipError_t launch_gradA_slab_conv(const float* gC, const uint8_t* codes, const u
     const dim3 grid(8 * (per_xcd < cus_per_xcd ? per_xcd : cus_per_xcd));
     if (kt == 32)
         hipLaunchKernelGGL((lutgemm_gradA_slab_kernel<32, kGaFmtHalf, true>), grid, block, 0, stream, gC, codes, S4, g_in, flags, M, C, N,
-                           scale, H * W, row_blocks, band_rows, H, W, zero_line);
+                           scale, H * W, row_blocks, band_rows, H, W, zero_line, fin);
     else
         hipLaunchKernelGGL((lutgemm_gradA_slab_kernel<16, kGaFmtHalf, true>), grid, block, 0, stream, gC, codes, S4, g_in, flags, M, C, N,
-                           scale, H * W, row_blocks, band_rows, H, W, zero_line);
+                           scale, H * W, row_blocks, band_rows, H, W, zero_line, fin);
     return hipGetLastError();
 }
 
@@ -1017,10 +1058,10 @@ hipError_t launch_gradA_slab_i16(const float* gC, const uint8_t* A, const uint8_
     const dim3 grid(8 * (per_xcd < cus_per_xcd ? per_xcd : cus_per_xcd));
     if (kt == 32)
         hipLaunchKernelGGL((lutgemm_gradA_slab_kernel<32, kGaFmtI16>), grid, block, 0, stream, gC, A, S4, gA, flags, M, K, N, scale,
-                           rows_per_image, row_blocks, band_rows, 0, 0, (const float*)nullptr);
+                           rows_per_image, row_blocks, band_rows, 0, 0, (const float*)nullptr, GaFinish{});
     else
         hipLaunchKernelGGL((lutgemm_gradA_slab_kernel<16, kGaFmtI16>), grid, block, 0, stream, gC, A, S4, gA, flags, M, K, N, scale,
-                           rows_per_image, row_blocks, band_rows, 0, 0, (const float*)nullptr);
+                           rows_per_image, row_blocks, band_rows, 0, 0, (const float*)nullptr, GaFinish{});
     return hipGetLastError();
 }
 
@@ -1054,10 +1095,10 @@ hipError_t launch_gradA_slab_f32w(const float* gC, const uint8_t* A, const uint8
     const dim3 grid(8 * (per_xcd < cus_per_xcd ? per_xcd : cus_per_xcd));
     if (kt == 32)
         hipLaunchKernelGGL((lutgemm_gradA_slab_kernel<32, kGaFmtF32W>), grid, block, 0, stream, gC, A, S4, gA, flags, M, K, N, scale,
-                           rows_per_image, row_blocks, band_rows, 0, 0, (const float*)nullptr);
+                           rows_per_image, row_blocks, band_rows, 0, 0, (const float*)nullptr, GaFinish{});
     else
         hipLaunchKernelGGL((lutgemm_gradA_slab_kernel<16, kGaFmtF32W>), grid, block, 0, stream, gC, A, S4, gA, flags, M, K, N, scale,
-                           rows_per_image, row_blocks, band_rows, 0, 0, (const float*)nullptr);
+                           rows_per_image, row_blocks, band_rows, 0, 0, (const float*)nullptr, GaFinish{});
     return hipGetLastError();
 }
 
@@ -1098,10 +1139,10 @@ hipError_t launch_gradA_slab_f32tab(const float* gC, const uint8_t* A, const uin
     const dim3 grid(8 * (per_xcd < cus_per_xcd ? per_xcd : cus_per_xcd));
     if (kt == 32)
         hipLaunchKernelGGL((lutgemm_gradA_slab_kernel<32, kGaFmtF32>), grid, block, 0, stream, gC, A, S4, gA, flags, M, K, N, scale,
-                           rows_per_image, row_blocks, band_rows, 0, 0, (const float*)nullptr);
+                           rows_per_image, row_blocks, band_rows, 0, 0, (const float*)nullptr, GaFinish{});
     else
         hipLaunchKernelGGL((lutgemm_gradA_slab_kernel<16, kGaFmtF32>), grid, block, 0, stream, gC, A, S4, gA, flags, M, K, N, scale,
-                           rows_per_image, row_blocks, band_rows, 0, 0, (const float*)nullptr);
+                           rows_per_image, row_blocks, band_rows, 0, 0, (const float*)nullptr, GaFinish{});
     e = hipGetLastError();
     if (e != hipSuccess) return e;
     return launch_gradA_f32tab(gC, A, B, gA, lut, g, M, K, N, scale, n_cu, stream, flags + 2, rows_per_image);
