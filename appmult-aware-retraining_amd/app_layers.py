@@ -92,15 +92,25 @@ def _observe(observer, x, quant_max, eps, scale, zp_neg):
         return _scale_and_zero_point(observer, quant_max, eps)
     import approx_ops
     with torch.no_grad():
-        lo, hi = torch.aminmax(x)
         mode = 0 if observer.num_flag == 0 else fused_mode
         observer.num_flag = 1
         fresh = torch.empty(2, dtype=torch.float32, device=x.device)
         new_scale, new_zp = fresh[0:1], fresh[1:2]
-        approx_ops.observer_update(lo.reshape(1), hi.reshape(1), observer.min_val, observer.max_val, new_scale, new_zp, mode,
-                                   getattr(observer, "momentum", 0.0), float(quant_max), float(eps),
-                                   # torch divides by a host-side scalar through its reciprocal rounded to float32
-                                   0.0 if quant_max.is_cuda else float(torch.tensor(1.0, dtype=torch.float32) / quant_max.to(torch.float32)))
+        # torch divides by a host-side scalar through its reciprocal rounded to float32
+        inv_qmax = 0.0 if quant_max.is_cuda else float(torch.tensor(1.0, dtype=torch.float32) / quant_max.to(torch.float32))
+        momentum = getattr(observer, "momentum", 0.0)
+        if x.is_contiguous() and x.numel() > 0:
+            # extremes of x and the scalar update in one launch (the workgroups meet in four words owned by this observer)
+            state = observer.__dict__.get("_minmax_state")
+            if state is None or state.device != x.device:
+                state = torch.zeros(approx_ops.MINMAX_STATE_WORDS, dtype=torch.int32, device=x.device)
+                observer.__dict__["_minmax_state"] = state
+            approx_ops.observe_minmax(x.detach(), state, observer.min_val, observer.max_val, new_scale, new_zp, mode, momentum,
+                                      float(quant_max), float(eps), inv_qmax)
+        else:
+            lo, hi = torch.aminmax(x)
+            approx_ops.observer_update(lo.reshape(1), hi.reshape(1), observer.min_val, observer.max_val, new_scale, new_zp, mode,
+                                       momentum, float(quant_max), float(eps), inv_qmax)
     return new_scale, new_zp
 
 

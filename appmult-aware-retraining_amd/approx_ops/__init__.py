@@ -49,6 +49,7 @@ _lib.amr_col2im_f32.argtypes = [_vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _v
 _lib.amr_conv_dequant_f32.argtypes = [_vp] * 10 + [_i, _i, _i, _vp]
 _lib.amr_conv_dequant_backward_f32.argtypes = [_vp, _vp, _vp, _vp, _i, _i, _i, _vp]
 _lib.amr_observer_update_f32.argtypes = [_vp] * 6 + [_i] + [ctypes.c_float] * 5 + [_vp]
+_lib.amr_observe_minmax_f32.argtypes = [_vp, _i64, _vp, _vp, _vp, _vp, _vp, _i] + [ctypes.c_float] * 5 + [_vp]
 _lib.amr_quantize_codes_f32.argtypes = [_vp, _vp, _vp, ctypes.c_float, _vp, _i64, _vp]
 _lib.amr_quantize_codes_backward_f32.argtypes = [_vp, _vp, _vp, _vp, ctypes.c_float, _vp, _i64, _vp]
 _lib.amr_lut_conv_forward_dequant_workspace_bytes.argtypes = [_i64, _i, _i, _i]
@@ -345,6 +346,27 @@ def observer_update(cur_min, cur_max, min_val, max_val, scale, zp_neg, mode, mom
                                           scale.data_ptr(), zp_neg.data_ptr(), int(mode), float(1 - momentum), float(momentum),
                                           float(quant_max), float(inv_quant_max), float(eps), _stream_ptr(dev))
     _raise_for(rc, "observer_update")
+
+
+MINMAX_STATE_WORDS = 4 + 3 * 1024     # AMR_OBSERVE_STATE_WORDS: int32 words of an observer's state, all zero before the first call
+
+
+def observe_minmax(x_tensor, state_tensor, min_val, max_val, scale, zp_neg, mode, momentum, quant_max, eps, inv_quant_max=0.0):
+    """observer_update on the extremes of x_tensor, which the same launch finds (x float32, contiguous; state int32
+    [MINMAX_STATE_WORDS] on the device, zeros before the first call)."""
+    _check_input(x_tensor, torch.float32, "x_tensor")
+    _check_input(state_tensor, torch.int32, "state_tensor")
+    _check(state_tensor.numel() >= MINMAX_STATE_WORDS and x_tensor.numel() > 0, "state too small, or x empty")
+    for t, name in ((min_val, "min_val"), (max_val, "max_val"), (scale, "scale"), (zp_neg, "zp_neg")):
+        _check_input(t, torch.float32, name)
+        _check(t.numel() == 1, f"{name} must hold one element")
+    dev = x_tensor.device
+    _check(all(t.device == dev for t in (state_tensor, min_val, max_val, scale, zp_neg)), "All tensors should be on the same device")
+    with torch.cuda.device(dev):
+        rc = _lib.amr_observe_minmax_f32(x_tensor.data_ptr(), x_tensor.numel(), state_tensor.data_ptr(), min_val.data_ptr(),
+                                         max_val.data_ptr(), scale.data_ptr(), zp_neg.data_ptr(), int(mode), float(1 - momentum),
+                                         float(momentum), float(quant_max), float(inv_quant_max), float(eps), _stream_ptr(dev))
+    _raise_for(rc, "observe_minmax")
 
 
 def quantize_codes(x_tensor, scale_tensor, zp_neg_tensor, quant_max, codes_tensor):

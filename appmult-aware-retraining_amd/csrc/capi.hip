@@ -43,6 +43,8 @@ hipError_t launch_gradA_slab(const float* gC, const uint8_t* A, const uint8_t* B
 hipError_t launch_observer_update(const float* cur_min, const float* cur_max, float* min_val, float* max_val, float* scale,
                                   float* zp_neg, int mode, float keep, float momentum, float qmax, float inv_qmax, float eps,
                                   hipStream_t stream);
+hipError_t launch_observe_minmax(const float* x, size_t n, uint32_t* state, float* min_val, float* max_val, float* scale, float* zp_neg,
+                                 int mode, float keep, float momentum, float qmax, float inv_qmax, float eps, int n_cu, hipStream_t stream);
 hipError_t launch_quantize_codes(const float* x, const float* scale, const float* zp_neg, float qmax, float* codes, size_t n,
                                  hipStream_t stream);
 hipError_t launch_quantize_codes_backward(const float* g, const float* x, const float* scale, const float* zp_neg, float qmax,
@@ -743,6 +745,18 @@ int amr_observer_update_f32(const float* cur_min, const float* cur_max, float* m
     hipError_t e = amr::launch_observer_update(cur_min, cur_max, min_val, max_val, scale, zp_neg, mode, keep, momentum, quant_max, inv_quant_max, eps,
                                                reinterpret_cast<hipStream_t>(stream));
     return e == hipSuccess ? AMR_OK : hip_fail(e, "observer update launch");
+}
+
+int amr_observe_minmax_f32(const float* x, int64_t n, uint32_t* state, float* min_val, float* max_val, float* scale, float* zp_neg,
+                           int mode, float keep, float momentum, float quant_max, float inv_quant_max, float eps, void* stream) {
+    if (mode < 0 || mode > 2 || !(quant_max > 0.f) || n <= 0) return fail(AMR_EINVAL, "bad observer mode, code range or element count");
+    if (!x || !state || !min_val || !max_val || !scale || !zp_neg) return fail(AMR_EINVAL, "null pointer argument");
+    if ((uintptr_t)state & 3) return fail(AMR_EINVAL, "state must be 4-byte aligned");
+    const int n_cu = current_device_cus(nullptr);
+    if (n_cu <= 0) return fail(AMR_EINVAL, "no HIP device available");
+    hipError_t e = amr::launch_observe_minmax(x, (size_t)n, state, min_val, max_val, scale, zp_neg, mode, keep, momentum, quant_max,
+                                              inv_quant_max, eps, n_cu, reinterpret_cast<hipStream_t>(stream));
+    return e == hipSuccess ? AMR_OK : hip_fail(e, "observer launch");
 }
 
 int amr_quantize_codes_f32(const float* x, const float* scale, const float* zp_neg, float qmax, float* codes, int64_t n,

@@ -73,11 +73,12 @@ __global__ __launch_bounds__(256) void quantize_codes_backward_kernel(const floa
 //   (keep = 1 - momentum, rounded by the caller the way the tensor expression rounds it)
 //   scale = max((max - min) / qmax, eps)  [or (max - min) * inv_qmax when inv_qmax != 0];  zp_neg = round(min / scale)
 // Same operations in the same order as the tensor expressions, each rounded on its own.
-__global__ void observer_update_kernel(const float* __restrict__ cur_min, const float* __restrict__ cur_max, float* __restrict__ min_val,
-                                       float* __restrict__ max_val, float* __restrict__ scale, float* __restrict__ zp_neg, int mode,
-                                       float keep, float momentum, float qmax, float inv_qmax, float eps) {
-    if (threadIdx.x != 0 || blockIdx.x != 0) return;
-    float lo = *cur_min, hi = *cur_max;
+// The scalar part of an observer step: range update (mode 0 first batch, 1 running extremes, 2 moving average), then
+// scale = max((max - min) / qmax, eps) [or (max - min) * inv_qmax], zp_neg = round(min / scale); every operation rounded on
+// its own, in the order of the tensor expressions (micronet+/app_layers.py:21-53, :154-160).
+__device__ __forceinline__ void observer_update_scalars(float lo, float hi, float* __restrict__ min_val, float* __restrict__ max_val,
+                                                        float* __restrict__ scale, float* __restrict__ zp_neg, int mode, float keep,
+                                                        float momentum, float qmax, float inv_qmax, float eps) {
     if (mode == 1) {
         // torch.min / torch.max hand a NaN on; fminf / fmaxf would drop it
         const float old_lo = *min_val, old_hi = *max_val;
@@ -95,6 +96,117 @@ __global__ void observer_update_kernel(const float* __restrict__ cur_min, const 
     const float s = raw != raw ? raw : fmaxf(raw, eps);
     *scale = s;
     *zp_neg = rintf(__fdiv_rn(lo, s));
+}
+
+// Extremes of a tensor and the observer step that follows, in ONE launch (the reference: torch.min, torch.max and a dozen
+// one-element tensor operations per layer and step).  Every workgroup folds its share (eight 16-byte loads in flight per
+// thread, grid-stride) and leaves its three results -- smallest, largest, "saw a NaN" -- in a slot of its own in `state`
+// (plain stores), then draws a ticket from state[0], the only atomic; the workgroup that draws the last ticket folds the
+// slots, does the scalar update and puts the ticket counter back to 0 for the next call.  torch.aminmax hands a NaN on:
+// so does this.  state: 4 + 3 * kObserveMaxBlocks words, all zero before the first call.
+constexpr int kObserveMaxBlocks = 1024;
+
+__global__ __launch_bounds__(256) void observe_minmax_kernel(const float* __restrict__ x, size_t n, uint32_t* __restrict__ state,
+                                                             float* __restrict__ min_val, float* __restrict__ max_val,
+                                                             float* __restrict__ scale, float* __restrict__ zp_neg, int mode, float keep,
+                                                             float momentum, float qmax, float inv_qmax, float eps, int vec) {
+    __shared__ float s_lo[4], s_hi[4];
+    __shared__ uint32_t s_nan[4], s_last;
+    float lo = __builtin_inff(), hi = -__builtin_inff();
+    bool nan = false;
+    const size_t stride = (size_t)gridDim.x * 256, tid = (size_t)blockIdx.x * 256 + threadIdx.x;
+    auto take = [&](float v) {
+        nan |= v != v;
+        lo = fminf(lo, v);          // (fminf / fmaxf drop a NaN: it is carried by `nan`)
+        hi = fmaxf(hi, v);
+    };
+    if (vec) {
+        const size_t n4 = n >> 2;
+        const f32x4* x4 = reinterpret_cast<const f32x4*>(x);
+        size_t i = tid;
+        for (; i + 7 * stride < n4; i += 8 * stride) {
+            f32x4 v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) v[u] = x4[i + u * stride];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) { take(v[u].x); take(v[u].y); take(v[u].z); take(v[u].w); }
+        }
+        for (; i < n4; i += stride) {
+            const f32x4 v = x4[i];
+            take(v.x); take(v.y); take(v.z); take(v.w);
+        }
+        for (size_t j = (n4 << 2) + tid; j < n; j += stride) take(x[j]);
+    } else {
+        for (size_t i = tid; i < n; i += stride) take(x[i]);
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        lo = fminf(lo, __shfl_xor(lo, o));
+        hi = fmaxf(hi, __shfl_xor(hi, o));
+    }
+    const bool wave_nan = __builtin_amdgcn_ballot_w64(nan) != 0;
+    const int wave = threadIdx.x >> 6;
+    if ((threadIdx.x & 63) == 0) { s_lo[wave] = lo; s_hi[wave] = hi; s_nan[wave] = wave_nan; }
+    __syncthreads();
+    uint32_t* slots = state + 4;
+    if (threadIdx.x == 0) {
+        lo = fminf(fminf(s_lo[0], s_lo[1]), fminf(s_lo[2], s_lo[3]));
+        hi = fmaxf(fmaxf(s_hi[0], s_hi[1]), fmaxf(s_hi[2], s_hi[3]));
+        // (atomic exchanges instead of plain stores: they are performed in the L2, where the last workgroup reads them)
+        atomicExch(&slots[3 * blockIdx.x], __float_as_uint(lo));
+        atomicExch(&slots[3 * blockIdx.x + 1], __float_as_uint(hi));
+        atomicExch(&slots[3 * blockIdx.x + 2], s_nan[0] | s_nan[1] | s_nan[2] | s_nan[3]);
+        __threadfence();
+        s_last = atomicAdd(&state[0], 1u) == gridDim.x - 1 ? 1u : 0u;
+    }
+    __syncthreads();
+    if (!s_last) return;
+    __threadfence();
+    lo = __builtin_inff(), hi = -__builtin_inff();
+    uint32_t any_nan = 0;
+    for (int b = threadIdx.x; b < (int)gridDim.x; b += 256) {
+        lo = fminf(lo, __uint_as_float(atomicOr(&slots[3 * b], 0u)));
+        hi = fmaxf(hi, __uint_as_float(atomicOr(&slots[3 * b + 1], 0u)));
+        any_nan |= atomicOr(&slots[3 * b + 2], 0u);
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        lo = fminf(lo, __shfl_xor(lo, o));
+        hi = fmaxf(hi, __shfl_xor(hi, o));
+    }
+    const bool nan2 = __builtin_amdgcn_ballot_w64(any_nan != 0) != 0;
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) { s_lo[wave] = lo; s_hi[wave] = hi; s_nan[wave] = nan2; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        float t_lo = fminf(fminf(s_lo[0], s_lo[1]), fminf(s_lo[2], s_lo[3]));
+        float t_hi = fmaxf(fmaxf(s_hi[0], s_hi[1]), fmaxf(s_hi[2], s_hi[3]));
+        if (s_nan[0] | s_nan[1] | s_nan[2] | s_nan[3]) t_lo = t_hi = __builtin_nanf("");
+        observer_update_scalars(t_lo, t_hi, min_val, max_val, scale, zp_neg, mode, keep, momentum, qmax, inv_qmax, eps);
+        atomicExch(&state[0], 0u);
+    }
+}
+
+hipError_t launch_observe_minmax(const float* x, size_t n, uint32_t* state, float* min_val, float* max_val, float* scale, float* zp_neg,
+                                 int mode, float keep, float momentum, float qmax, float inv_qmax, float eps, int n_cu, hipStream_t stream) {
+    const int vec = (((uintptr_t)x) & 15) == 0;
+    size_t blocks = (n + 256 * 32 - 1) / (256 * 32);         // at least 32 values per thread
+    // one workgroup per CU at most (measured on MI355X for 134 MB: 28 us with 256 workgroups, 37 with 512, 57 with 1024 -- the
+    // tickets and the slots cost more than the extra loads in flight gain)
+    size_t cap = (size_t)(n_cu > 0 ? n_cu : 256);
+    if (cap > kObserveMaxBlocks) cap = kObserveMaxBlocks;
+    if (blocks > cap) blocks = cap;
+    if (blocks < 1) blocks = 1;
+    hipLaunchKernelGGL(observe_minmax_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, x, n, state, min_val, max_val, scale, zp_neg,
+                       mode, keep, momentum, qmax, inv_qmax, eps, vec);
+    return hipGetLastError();
+}
+
+__global__ void observer_update_kernel(const float* __restrict__ cur_min, const float* __restrict__ cur_max, float* __restrict__ min_val,
+                                       float* __restrict__ max_val, float* __restrict__ scale, float* __restrict__ zp_neg, int mode,
+                                       float keep, float momentum, float qmax, float inv_qmax, float eps) {
+    if (threadIdx.x != 0 || blockIdx.x != 0) return;
+    observer_update_scalars(*cur_min, *cur_max, min_val, max_val, scale, zp_neg, mode, keep, momentum, qmax, inv_qmax, eps);
 }
 
 hipError_t launch_observer_update(const float* cur_min, const float* cur_max, float* min_val, float* max_val, float* scale,

@@ -249,6 +249,18 @@ int amr_observer_update_f32(const float *cur_min, const float *cur_max, float *m
                             float eps, void *stream);
 
 /*
+ * The extremes of x (n float32 values; what torch.min / torch.max give the reference's observers, micronet+/app_layers.py:41-46)
+ * and amr_observer_update_f32 on them, in one launch.  A NaN in x makes both extremes NaN, as in the tensor library.
+ * state: AMR_OBSERVE_STATE_WORDS 32-bit words of device memory owned by the caller, one set per observer, all zero before the
+ * first call (word 0 counts the workgroups that have finished and is back at zero when the call ends; the others hold their
+ * partial results).  Calls that share a state must not overlap in time.
+ */
+#define AMR_OBSERVE_STATE_WORDS (4 + 3 * 1024)
+int amr_observe_minmax_f32(const float *x, int64_t n, uint32_t *state, float *min_val, float *max_val, float *scale,
+                           float *zp_neg, int mode, float keep, float momentum, float quant_max, float inv_quant_max, float eps,
+                           void *stream);
+
+/*
  * Quantiser in front of the LUT GEMM: codes[i] = clamp(round(x[i] / *scale - *zp_neg), 0, qmax) as float32,
  * round half to even; scale and zp_neg are device pointers to one float each.  One pass instead of the
  * divide / subtract / round / straight-through / clamp chain of the reference's quantize_v2

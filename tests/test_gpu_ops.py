@@ -599,6 +599,34 @@ def test_one_launch_observer_update_equals_tensor_expressions(ops, kind, qmax_on
     assert torch.equal(s1.reshape(1), s2.reshape(1)) and torch.equal(z1.reshape(1), z2.reshape(1))
 
 
+@pytest.mark.parametrize("n", [1, 5, 4097, 3 * 64 * 32 * 32 + 3, 33554432 + 17])
+def test_one_launch_extremes_and_observer_update(ops, n):
+    """amr_observe_minmax_f32 against torch.aminmax + the observer's tensor expressions: every workgroup count, ragged tails,
+    unaligned data, a NaN in the last element, three calls in a row on one state (the last ticket puts the counter back)."""
+    import approx_ops
+    print("observe minmax", n, flush=True)
+    g = torch.Generator(device="cuda").manual_seed(6)
+    base = torch.randn(n + 1, device="cuda", generator=g)
+    state = torch.zeros(approx_ops.MINMAX_STATE_WORDS, dtype=torch.int32, device="cuda")
+    lo, hi, sc, zp = (torch.zeros(1, device="cuda") for _ in range(4))
+    lo2, hi2, sc2, zp2 = (torch.zeros(1, device="cuda") for _ in range(4))
+    eps = float(torch.finfo(torch.float32).eps)
+    for call, (x, mode) in enumerate(((base[:n], 0), (base[1:] * 3 - 1, 2), (base[:n] * 0.5 + 2, 1))):
+        x = x if call != 1 else x.clone()[:n]                     # (call 0: 16-byte aligned view; call 1: a fresh tensor)
+        if call == 0 and n > 1:
+            x = base[1:n + 1]                                     # 4-byte aligned only
+        approx_ops.observe_minmax(x.contiguous(), state, lo, hi, sc, zp, mode, 0.1, 127.0, eps)
+        want_lo, want_hi = torch.aminmax(x)
+        approx_ops.observer_update(want_lo.reshape(1), want_hi.reshape(1), lo2, hi2, sc2, zp2, mode, 0.1, 127.0, eps)
+        for a, b in ((lo, lo2), (hi, hi2), (sc, sc2), (zp, zp2)):
+            assert torch.equal(a, b), (call, float(a), float(b))
+        assert int(state[0]) == 0
+    x = base[:n].clone()
+    x[-1] = float("nan")
+    approx_ops.observe_minmax(x, state, lo, hi, sc, zp, 0, 0.1, 127.0, eps)
+    assert all(bool(torch.isnan(t).all()) for t in (lo, hi, sc, zp)) and int(state[0]) == 0
+
+
 def test_bench_captured_codes_cover_every_benchmark_layer(ops):
     """bench.py --codes captured: one forward pass of the package's ResNet-18 yields operand codes for each of the 12
     benchmark GEMM shapes (here at batch 4), uint8 below 2^7, and post-ReLU activations pile up on one code."""
