@@ -110,6 +110,7 @@ hipError_t launch_gradA_slab_conv(const float* gC, const uint8_t* codes, const u
                                   void* S, const float* zero_line, hipStream_t stream, const float* zt, const float* zw,
                                   const float* qscale, const uint8_t* inside);
 bool gradA_slab_conv_can_finish(int Bn, int H, int W, const float* g_in);
+hipError_t launch_poison_if_raised(float* gx, size_t total, const uint32_t* gate, hipStream_t stream);
 hipError_t launch_window_sums_3x3(const float* t, float* zt, long B, int H, int W, hipStream_t stream);
 hipError_t launch_dequant_grad_rowsum(const float* g, const float* sa, const float* sw, float* gc, float* t, int M, int N, int L,
                                       hipStream_t stream);
@@ -898,7 +899,7 @@ int amr_lut_conv_input_grad_f32(const float* gC, const uint8_t* codes, const uin
     if (!finish)
         e = amr::launch_conv_input_grad(nullptr, t, z_w, inside, scale, gx, B, C, H, W, 3, 3, 1, 1, 1, H, W, s, flags + 2, fallback ? 1 : 3);
     else if (!fallback)
-        e = amr::launch_conv_input_grad(nullptr, t, z_w, inside, scale, gx, B, C, H, W, 3, 3, 1, 1, 1, H, W, s, flags + 2, 4);
+        e = amr::launch_poison_if_raised(gx, (size_t)B * C * H * W, flags + 2, s);
     if (e != hipSuccess) return hip_fail(e, "input gradient launch");
     if (fallback) {
         e = amr::launch_gradA(gC, A_fallback, Bt, cols_fallback, lut_grad_a, g, (int)M, 9 * C, N, factor, n_cu, s, flags + 2, H * W);

@@ -171,16 +171,12 @@ __global__ __launch_bounds__(256) void conv_input_grad_kernel(const float* __res
     if (idx >= total) return;
     // gate_mode 1: the pass behind a kernel that left the tap sums in gx -- when *gate says that kernel could not do its work,
     // this pass leaves gx alone (a recomputation is queued behind, gate_mode 2) or, gate_mode 3, marks every element NaN;
-    // gate_mode 2: runs only when *gate is set; gate_mode 4: marks every element NaN when *gate is set and does nothing else.
+    // gate_mode 2: runs only when *gate is set.
     if (gate_mode != 0) {
         const bool raised = *gate != 0u;
         if (gate_mode == 2 && !raised) return;
         if (gate_mode == 1 && raised) return;
         if (gate_mode == 3 && raised) { gx[idx] = __builtin_nanf(""); return; }
-        if (gate_mode == 4) {      // behind a kernel that finished gx itself: only the NaN marking is left to do
-            if (raised) gx[idx] = __builtin_nanf("");
-            return;
-        }
     }
     const int kh = KH ? KH : kh_rt, kw = KW ? KW : kw_rt, stride = STRIDE ? STRIDE : stride_rt;
     const int xx = (int)(idx % W);
@@ -282,6 +278,19 @@ hipError_t launch_window_sums_3x3(const float* t, float* zt, long B, int H, int 
     const size_t total = (size_t)B * H * W;
     if (total == 0) return hipSuccess;
     hipLaunchKernelGGL(window_sums_3x3_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, t, zt, H, W, total);
+    return hipGetLastError();
+}
+
+// Queued behind a kernel that finished gx itself: marks every element NaN when *gate says that kernel met what it cannot
+// serve (and nobody queued a recomputation); otherwise its few workgroups leave at once.
+__global__ __launch_bounds__(256) void poison_if_raised_kernel(float* __restrict__ gx, size_t total, const uint32_t* __restrict__ gate) {
+    if (*gate == 0u) return;
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (size_t)gridDim.x * 256) gx[i] = __builtin_nanf("");
+}
+
+hipError_t launch_poison_if_raised(float* gx, size_t total, const uint32_t* gate, hipStream_t stream) {
+    if (total == 0) return hipSuccess;
+    hipLaunchKernelGGL(poison_if_raised_kernel, dim3(256), dim3(256), 0, stream, gx, total, gate);
     return hipGetLastError();
 }
 
