@@ -210,7 +210,7 @@ class _ApproxConvLayerFn(torch.autograd.Function):
     operators; their gradients are returned for it."""
 
     @staticmethod
-    def forward(ctx, x, w_codes, w_resp, taps, a_scale, a_zp, w_scale, w_zp, bias, a_qmax, stride, padding, dilation):
+    def forward(ctx, x, w_codes, w_resp, taps, a_scale, a_zp, w_scale, w_zp, bias, a_qmax, stride, padding, dilation, fwd_cache=None):
         import approx_ops
         from self_ops.ops_py import approx_ops as ops
         one = lambda t: t.detach().reshape(1).contiguous()
@@ -238,7 +238,8 @@ class _ApproxConvLayerFn(torch.autograd.Function):
         # (LUT GEMM whose store applies the zero-point terms, the scaling and the bias and writes NCHW)
         approx_ops.approx_conv_forward_dequant(a_mat, b_mat, ops.lut_appmult, x_sum.contiguous(), w_resp.detach().contiguous(),
                                                taps.contiguous(), z_a, z_w, s_a, s_w,
-                                               None if bias is None else bias.detach().contiguous(), out)
+                                               None if bias is None else bias.detach().contiguous(), out,
+                                               cache=fwd_cache[0] if fwd_cache else None, b_version=fwd_cache[1] if fwd_cache else 0)
         # a 3x3 / stride 1 / padding 1 layer takes its input gradient from one implicit GEMM over the input pixels (no
         # [M][9C] gradient matrix, no col2im) where the library serves the shape and the gradient table fits halves
         conv_shaped = ((kh, kw, s, p, d) == (3, 3, 1, 1, 1) and ops.lut_grad_a_fits_halves
@@ -282,7 +283,7 @@ class _ApproxConvLayerFn(torch.autograd.Function):
             g_wr = ((z_a * (s_a * s_w)) * g.sum(dim=0, keepdim=True)).reshape(wr_shape)
         if has_bias and ctx.needs_input_grad[8]:
             g_bias = g.sum(dim=(0, 2, 3))
-        return g_x, g_w, g_wr, None, None, None, None, None, g_bias, None, None, None, None
+        return g_x, g_w, g_wr, None, None, None, None, None, g_bias, None, None, None, None, None
 
 
 # ------------------------------------------------------------------------------------------ quantiser module
@@ -323,6 +324,7 @@ class _QuantParamsMixin:
 
     def _update_ranges(self, input):
         if self.training:
+            self.__dict__["_range_epoch"] = self.__dict__.get("_range_epoch", 0) + 1     # (the quantisation parameters may move)
             self.activation_scale, self.activation_zp_neg = _observe(
                 self.activation_observer, input, self.activation_quant_max, self.eps, self.activation_scale, self.activation_zp_neg)
             self.weight_scale, self.weight_zp_neg = _observe(
@@ -384,6 +386,7 @@ class ApproxConv2d(nn.Conv2d, _QuantParamsMixin):
         self.reference_zero_point_terms = False     # True: evaluate the three correction terms as full convolutions
         self.fused_dequant = True                   # False: zero-point terms and scaling as torch operators
         self.fused_layer = True                     # False: float32 code tensors between quantiser, convolution and dequantisation
+        self.keep_expansion_in_eval = True          # evaluation mode: the forward table expanded along the weight codes stays on the device
 
     def quantize_v2(self, x, s, zpn, qmax):
         return _to_codes(x, s, zpn, qmax)
@@ -422,6 +425,21 @@ class ApproxConv2d(nn.Conv2d, _QuantParamsMixin):
             cache[key] = F.unfold(ones, (kh, kw), dilation=dilation, padding=padding, stride=stride)[0]
         return cache[key]
 
+    def _frozen_weight_cache(self):
+        """In evaluation mode the weight codes only change when the weights, their quantisation parameters or the tables do:
+        the expansion of the forward table along them is then kept on the device between calls (approx_ops.ForwardCache) under a
+        number made of everything that could change them.  Training mode: None (the weights move every step)."""
+        if self.training or not self.keep_expansion_in_eval:
+            return None
+        import approx_ops
+        from self_ops.ops_py import approx_ops as ops
+        cache = self.__dict__.get("_fwd_cache")
+        if cache is None:
+            cache = self.__dict__["_fwd_cache"] = approx_ops.ForwardCache()
+        token = hash((self.weight._version, self.weight.data_ptr(), self.weight_scale._version, self.weight_scale.data_ptr(),
+                      self.weight_zp_neg._version, self.weight_zp_neg.data_ptr(), self.__dict__.get("_range_epoch", 0), ops.table_generation))
+        return cache, token & 0xFFFFFFFFFFFFFFFF
+
     def _takes_uint8_path(self, input):
         """The one-operator path on uint8 codes serves the LUT-gradient convolution of float32 CUDA tensors with square
         geometry (the reference's operator reads element 0 of stride / padding / dilation, ``approx_ops.py:545-547``)."""
@@ -439,7 +457,7 @@ class ApproxConv2d(nn.Conv2d, _QuantParamsMixin):
             w_resp, taps = self._weight_zero_point_parts(w_codes, input.shape[1:], conv_args, torch.float32, input.device)
             return _ApproxConvLayerFn.apply(input, w_codes, w_resp, taps, self.activation_scale, self.activation_zp_neg,
                                             self.weight_scale, self.weight_zp_neg, self.bias, float(self.activation_quant_max),
-                                            tuple(self.stride), tuple(self.padding), tuple(self.dilation))
+                                            tuple(self.stride), tuple(self.padding), tuple(self.dilation), self._frozen_weight_cache())
         x_codes = self.quantize_v2(input, self.activation_scale, self.activation_zp_neg, self.activation_quant_max)
         total = self.conv2d_op(x_codes, w_codes, **conv_args)       # approximate products of the codes
         if self.reference_zero_point_terms:

@@ -60,6 +60,12 @@ _lib.amr_lut_conv_input_grad_workspace_bytes.argtypes = [_i64, _i, _i, _i, _i, _
 _lib.amr_lut_conv_input_grad_workspace_bytes.restype = _sz
 _lib.amr_grad_table_fits_halves.argtypes = [_vp, _i64]
 _lib.amr_lut_conv_input_grad_f32.argtypes = [_vp] * 4 + [_i64] + [_vp] * 5 + [_i] * 5 + [_vp, _vp, _vp, _sz, _vp]
+_u64 = ctypes.c_uint64
+_lib.amr_fwd_cache_create.argtypes = [ctypes.POINTER(_vp)]
+_lib.amr_fwd_cache_destroy.argtypes = [_vp]
+_lib.amr_fwd_cache_stats.argtypes = [_vp, ctypes.POINTER(_u64), ctypes.POINTER(_u64), ctypes.POINTER(_sz)]
+_lib.amr_lut_gemm_forward_cached.argtypes = [_vp, _u64, _vp, _vp, _vp, _i, _vp, _i64, _i, _i, _i, _vp]
+_lib.amr_lut_conv_forward_dequant_cached_f32.argtypes = [_vp, _u64, _vp, _vp, _vp, _i64, _i, _i, _i, _i] + [_vp] * 9 + [_vp, _sz, _vp]
 _lib.amr_quantize_codes_nhwc_u8.argtypes = [_vp, _vp, _vp, ctypes.c_float, _vp, _vp, _vp, _i, _i, _i, _vp]
 _lib.amr_im2col_nhwc_u8.argtypes = [_vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp]
 _lib.amr_conv_input_grad_f32.argtypes = [_vp] * 6 + [_i] * 9 + [_vp]
@@ -110,7 +116,37 @@ def _stream_ptr(device):
     return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
 
 
-def approx_gemm_forward(a_tensor, b_tensor, c_tensor, lut_appmult_tensor):
+class ForwardCache:
+    """The expansion of the forward table along one weight matrix, kept on the device between forward calls whose B does not
+    change (amr_fwd_cache): pass it, with a number that changes whenever B's contents do, to approx_gemm_forward or
+    approx_conv_forward_dequant.  Calls sharing a cache must be stream-ordered."""
+
+    def __init__(self):
+        self._h = _vp()
+        _raise_for(_lib.amr_fwd_cache_create(ctypes.byref(self._h)), "amr_fwd_cache_create")
+
+    def stats(self):
+        """(hits, misses, bytes of device memory held)."""
+        h, m, b = _u64(0), _u64(0), _sz(0)
+        _raise_for(_lib.amr_fwd_cache_stats(self._h, ctypes.byref(h), ctypes.byref(m), ctypes.byref(b)), "amr_fwd_cache_stats")
+        return h.value, m.value, b.value
+
+    def close(self):
+        if self._h:
+            _lib.amr_fwd_cache_destroy(self._h)
+            self._h = _vp()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def __deepcopy__(self, memo):
+        return ForwardCache()         # a copied layer expands for itself
+
+
+def approx_gemm_forward(a_tensor, b_tensor, c_tensor, lut_appmult_tensor, cache=None, b_version=0):
     """c[m,n] = sum_k lut[a[m,k]][b[k,n]]; a u8 [M,K], b u8 [K,N], c u32 [M,N] (out), lut u16 padded table.
     Contract of approx_gemm_forward_gpu (self_ops/src/approx_gemm_forward.cu:241-259).
     A float32 c_tensor receives the same sums converted to float32 (what the reference's callers do with the uint32
@@ -131,6 +167,13 @@ def approx_gemm_forward(a_tensor, b_tensor, c_tensor, lut_appmult_tensor):
     with torch.cuda.device(dev):
         # scratch (the expanded table of large problems) comes from torch's caching allocator, so that it is
         # ordered with the stream like any other tensor and freed with the process' other device memory
+        if cache is not None:
+            # (an extension: the expansion of the table along b is kept in `cache` while b_version stays the same)
+            rc = _lib.amr_lut_gemm_forward_cached(cache._h, int(b_version) & 0xFFFFFFFFFFFFFFFF, a_tensor.data_ptr(), b_tensor.data_ptr(),
+                                                  c_tensor.data_ptr(), 1 if as_float else 0, lut_appmult_tensor.data_ptr(),
+                                                  lut_appmult_tensor.size(0), M, K, N, _stream_ptr(dev))
+            _raise_for(rc, "approx_gemm_forward")
+            return
         need = _lib.amr_lut_gemm_forward_workspace_bytes(lut_appmult_tensor.size(0), M, K, N)
         ws = torch.empty(need, dtype=torch.uint8, device=dev) if need else None
         entry = _lib.amr_lut_gemm_forward_f32_ws if as_float else _lib.amr_lut_gemm_forward_ws
@@ -284,7 +327,8 @@ def conv_dequant(c_rows, x_sum, w_resp, taps, z_a, z_w, s_a, s_w, bias, out_tens
     _raise_for(rc, "conv_dequant")
 
 
-def approx_conv_forward_dequant(a_tensor, b_tensor, lut_appmult_tensor, x_sum, w_resp, taps, z_a, z_w, s_a, s_w, bias, out_tensor):
+def approx_conv_forward_dequant(a_tensor, b_tensor, lut_appmult_tensor, x_sum, w_resp, taps, z_a, z_w, s_a, s_w, bias, out_tensor,
+                                cache=None, b_version=0):
     """approx_gemm_forward followed by conv_dequant without the sums going to memory: out float32 [B, N, oh, ow] from the uint8
     operand matrices a [B*L, K], b [K, N] (any common order of k) and the operands of conv_dequant."""
     _check_input(a_tensor, torch.uint8, "a_tensor")
@@ -309,7 +353,8 @@ def approx_conv_forward_dequant(a_tensor, b_tensor, lut_appmult_tensor, x_sum, w
     with torch.cuda.device(dev):
         need = _lib.amr_lut_conv_forward_dequant_workspace_bytes(lut_appmult_tensor.size(0), M, K, N)
         ws = torch.empty(max(need, 256), dtype=torch.uint8, device=dev)
-        rc = _lib.amr_lut_conv_forward_dequant_f32(a_tensor.data_ptr(), b_tensor.data_ptr(), lut_appmult_tensor.data_ptr(),
+        rc = _lib.amr_lut_conv_forward_dequant_cached_f32(cache._h if cache is not None else None, int(b_version) & 0xFFFFFFFFFFFFFFFF,
+                                                   a_tensor.data_ptr(), b_tensor.data_ptr(), lut_appmult_tensor.data_ptr(),
                                                    lut_appmult_tensor.size(0), M, K, N, L, x_sum.data_ptr(), w_resp.data_ptr(),
                                                    taps.data_ptr(), z_a.data_ptr(), z_w.data_ptr(), s_a.data_ptr(), s_w.data_ptr(),
                                                    bias.data_ptr() if bias is not None else None, out_tensor.data_ptr(), ws.data_ptr(),

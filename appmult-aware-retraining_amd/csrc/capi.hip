@@ -4,6 +4,7 @@
 
 #include <atomic>
 #include <mutex>
+#include <new>
 #include <vector>
 #include <stdarg.h>
 #include <stdio.h>
@@ -17,7 +18,7 @@ hipError_t launch_fwd(const uint8_t* A, const uint8_t* B, uint32_t* C, const uin
 size_t fwd_slab_workspace_bytes(const LutGeom& g, int M, int K, int N, bool force);
 hipError_t launch_fwd_slab(const uint8_t* A, const uint8_t* B, uint32_t* C, const uint16_t* lut, const LutGeom& g,
                            int M, int K, int N, int n_cu, void* workspace, hipStream_t stream, int out_f32,
-                           const SlabDequant* dq = nullptr);
+                           const SlabDequant* dq = nullptr, int expanded = 0);
 bool fwd_slab_can_dequant(const LutGeom& g, int M, int K, int N, int n_cu, bool force);
 size_t gradB_workspace_bytes(int M, int K, int N, int n_cu);
 hipError_t launch_gradB(const float* gC, const uint8_t* A, const uint8_t* B, float* gB, const int16_t* lut,
@@ -271,8 +272,72 @@ size_t amr_lut_gemm_forward_workspace_bytes(int64_t lut_elems, int M, int K, int
     return mode ? amr::fwd_slab_workspace_bytes(g, M, K, N, mode == 2) : 0;
 }
 
+}  // extern "C"
+
+// Expansion of the forward table along one weight matrix, kept between calls (amr_fwd_cache_* in the header).
+struct amr_fwd_cache {
+    std::mutex mu;
+    int dev = -1;
+    void* buf = nullptr;        // [256 B header][E], as the forward workspace
+    size_t bytes = 0;
+    bool valid = false;
+    uint64_t version = 0;
+    const void* lut = nullptr;
+    int64_t lut_elems = 0;
+    int K = 0, N = 0;
+    uint64_t hits = 0, misses = 0;
+};
+
+// Buffer of `need` bytes for the expansion of (version, lut, K, N); *hit says whether it already holds it.  A miss leaves the
+// cache claiming the new contents: the caller expands into the buffer on its stream right away.
+static void* fwd_cache_lookup(amr_fwd_cache* c, int dev, size_t need, uint64_t version, const void* lut, int64_t lut_elems, int K, int N,
+                              bool* hit, hipError_t* err) {
+    std::lock_guard<std::mutex> lk(c->mu);
+    *err = hipSuccess;
+    *hit = c->valid && c->dev == dev && c->bytes >= need && c->version == version && c->lut == lut && c->lut_elems == lut_elems &&
+           c->K == K && c->N == N;
+    if (*hit) { ++c->hits; return c->buf; }
+    ++c->misses;
+    if (c->dev != dev || c->bytes < need) {
+        // (hipFree waits for the device: work queued on the old buffer has finished before it goes)
+        if (c->buf) (void)hipFree(c->buf);
+        c->buf = nullptr; c->bytes = 0; c->valid = false;
+        *err = hipMalloc(&c->buf, need);
+        if (*err != hipSuccess) { c->buf = nullptr; return nullptr; }
+        c->bytes = need;
+        c->dev = dev;
+    }
+    c->valid = true; c->version = version; c->lut = lut; c->lut_elems = lut_elems; c->K = K; c->N = N;
+    return c->buf;
+}
+
+extern "C" {
+
+int amr_fwd_cache_create(amr_fwd_cache** out) {
+    if (!out) return fail(AMR_EINVAL, "null pointer argument");
+    *out = new (std::nothrow) amr_fwd_cache();
+    return *out ? AMR_OK : fail(AMR_EINVAL, "out of host memory");
+}
+
+int amr_fwd_cache_destroy(amr_fwd_cache* c) {
+    if (!c) return AMR_OK;
+    if (c->buf) (void)hipFree(c->buf);
+    delete c;
+    return AMR_OK;
+}
+
+int amr_fwd_cache_stats(amr_fwd_cache* c, uint64_t* hits, uint64_t* misses, size_t* device_bytes) {
+    if (!c) return fail(AMR_EINVAL, "null pointer argument");
+    std::lock_guard<std::mutex> lk(c->mu);
+    if (hits) *hits = c->hits;
+    if (misses) *misses = c->misses;
+    if (device_bytes) *device_bytes = c->bytes;
+    return AMR_OK;
+}
+
 static int forward_impl(const uint8_t* A, const uint8_t* B, uint32_t* C, const uint16_t* lut, int64_t lut_elems, int M, int K, int N,
-                        void* workspace, size_t workspace_bytes, void* stream, int out_f32) {
+                        void* workspace, size_t workspace_bytes, void* stream, int out_f32, amr_fwd_cache* cache = nullptr,
+                        uint64_t b_version = 0) {
     if (M < 0 || K < 0 || N < 0) return fail(AMR_EINVAL, "negative dimension M=%d K=%d N=%d", M, K, N);
     amr::LutGeom g;
     if (!amr::lut_geom_from_elems(lut_elems, &g))
@@ -293,14 +358,18 @@ static int forward_impl(const uint8_t* A, const uint8_t* B, uint32_t* C, const u
     hipError_t e;
     if (need > 0) {
         void* ws = workspace;
-        if (ws) {
+        bool hit = false;
+        if (cache) {
+            ws = fwd_cache_lookup(cache, dev, need, b_version, lut, lut_elems, K, N, &hit, &e);
+            if (!ws) return hip_fail(e, "cache hipMalloc");
+        } else if (ws) {
             if (workspace_bytes < need) return fail(AMR_EWORKSPACE, "workspace of %zu bytes is smaller than the %zu required", workspace_bytes, need);
             if ((uintptr_t)ws & 255) return fail(AMR_EINVAL, "workspace must be 256-byte aligned");
         } else {
             ws = internal_workspace(dev, s, need, &e);
             if (!ws) return hip_fail(e, "workspace hipMalloc");
         }
-        e = amr::launch_fwd_slab(A, B, C, lut, g, M, K, N, n_cu, ws, s, out_f32);
+        e = amr::launch_fwd_slab(A, B, C, lut, g, M, K, N, n_cu, ws, s, out_f32, nullptr, hit ? 1 : 0);
     } else {
         e = amr::launch_fwd(A, B, C, lut, g, M, K, N, n_cu, s, out_f32);
     }
@@ -318,6 +387,15 @@ int amr_lut_conv_forward_dequant_f32(const uint8_t* A, const uint8_t* B, const u
                                      int positions, const float* x_sum, const float* w_resp, const float* taps, const float* z_a,
                                      const float* z_w, const float* s_a, const float* s_w, const float* bias, float* out,
                                      void* workspace, size_t workspace_bytes, void* stream) {
+    return amr_lut_conv_forward_dequant_cached_f32(nullptr, 0, A, B, lut, lut_elems, M, K, N, positions, x_sum, w_resp, taps, z_a, z_w, s_a,
+                                                   s_w, bias, out, workspace, workspace_bytes, stream);
+}
+
+int amr_lut_conv_forward_dequant_cached_f32(amr_fwd_cache* cache, uint64_t b_version, const uint8_t* A, const uint8_t* B,
+                                            const uint16_t* lut, int64_t lut_elems, int M, int K, int N, int positions,
+                                            const float* x_sum, const float* w_resp, const float* taps, const float* z_a,
+                                            const float* z_w, const float* s_a, const float* s_w, const float* bias, float* out,
+                                            void* workspace, size_t workspace_bytes, void* stream) {
     if (M < 0 || K < 0 || N < 0) return fail(AMR_EINVAL, "negative dimension M=%d K=%d N=%d", M, K, N);
     if (positions <= 0 || M % positions != 0) return fail(AMR_EINVAL, "positions=%d must divide M=%d", positions, M);
     amr::LutGeom g;
@@ -342,11 +420,18 @@ int amr_lut_conv_forward_dequant_f32(const uint8_t* A, const uint8_t* B, const u
     if (K > 0 && mode && e_bytes && amr::fwd_slab_can_dequant(g, M, K, N, n_cu, mode == 2)) {
         // one launch stores the activation; `sums` is touched by the gated fall-back only
         const amr::SlabDequant dq{x_sum, w_resp, taps, z_a, z_w, s_a, s_w, bias, out, positions};
-        e = amr::launch_fwd_slab(A, B, reinterpret_cast<uint32_t*>(sums), lut, g, M, K, N, n_cu, workspace, s, 1, &dq);
+        void* e_buf = workspace;
+        bool hit = false;
+        if (cache) {
+            e_buf = fwd_cache_lookup(cache, dev, amr::fwd_slab_workspace_bytes(g, M, K, N, mode == 2), b_version, lut, lut_elems, K, N, &hit, &e);
+            if (!e_buf) return hip_fail(e, "cache hipMalloc");
+        }
+        e = amr::launch_fwd_slab(A, B, reinterpret_cast<uint32_t*>(sums), lut, g, M, K, N, n_cu, e_buf, s, 1, &dq, hit ? 1 : 0);
         return e == hipSuccess ? AMR_OK : hip_fail(e, "forward launch");
     }
     // K split over workgroups, small problems, direct kernels: the sums meet in memory first, a second pass dequantises them
-    const int rc = forward_impl(A, B, reinterpret_cast<uint32_t*>(sums), lut, lut_elems, M, K, N, e_bytes ? workspace : nullptr, e_bytes, stream, 1);
+    const int rc = forward_impl(A, B, reinterpret_cast<uint32_t*>(sums), lut, lut_elems, M, K, N, e_bytes ? workspace : nullptr, e_bytes, stream, 1,
+                                cache, b_version);
     if (rc != AMR_OK) return rc;
     e = amr::launch_dequant(sums, x_sum, w_resp, taps, z_a, z_w, s_a, s_w, bias, out, M, N, positions, s);
     return e == hipSuccess ? AMR_OK : hip_fail(e, "dequant launch");
@@ -361,6 +446,12 @@ int amr_lut_gemm_forward_f32_ws(const uint8_t* A, const uint8_t* B, float* C, co
                                 int M, int K, int N, void* workspace, size_t workspace_bytes, void* stream) {
     // (a zero of either type has the same bits: the empty sums of K == 0 need no conversion)
     return forward_impl(A, B, reinterpret_cast<uint32_t*>(C), lut, lut_elems, M, K, N, workspace, workspace_bytes, stream, 1);
+}
+
+int amr_lut_gemm_forward_cached(amr_fwd_cache* cache, uint64_t b_version, const uint8_t* A, const uint8_t* B, void* C, int c_is_f32,
+                                const uint16_t* lut, int64_t lut_elems, int M, int K, int N, void* stream) {
+    if (!cache) return fail(AMR_EINVAL, "null cache");
+    return forward_impl(A, B, reinterpret_cast<uint32_t*>(C), lut, lut_elems, M, K, N, nullptr, 0, stream, c_is_f32 ? 1 : 0, cache, b_version);
 }
 
 int amr_lut_gemm_forward(const uint8_t* A, const uint8_t* B, uint32_t* C, const uint16_t* lut, int64_t lut_elems,

@@ -596,9 +596,11 @@ bool fwd_slab_can_dequant(const LutGeom& g, int M, int K, int N, int n_cu, bool 
 
 // dq != nullptr (only with fwd_slab_can_dequant): the kernel stores the dequantised NCHW activation dq->out instead of C; C
 // (float32 [M,N]) is then scratch that only the gated fall-back touches, followed by a dequantisation pass under the same gate.
+// expanded != 0: `workspace` already holds the expansion of this B and table (a caller's cache); only the fall-back request
+// in its header is cleared, by a one-word fill, in place of the expansion launch.
 hipError_t launch_fwd_slab(const uint8_t* A, const uint8_t* B, uint32_t* C, const uint16_t* lut, const LutGeom& g,
                            int M, int K, int N, int n_cu, void* workspace, hipStream_t stream, int out_f32,
-                           const SlabDequant* dq = nullptr) {
+                           const SlabDequant* dq = nullptr, int expanded = 0) {
     const int n_tiles = (N + kSlabCols - 1) / kSlabCols;
     const int k_quads = (K + 3) / 4;
     const SlabDequant none{};
@@ -606,12 +608,14 @@ hipError_t launch_fwd_slab(const uint8_t* A, const uint8_t* B, uint32_t* C, cons
     uint32_t* E = reinterpret_cast<uint32_t*>(reinterpret_cast<unsigned char*>(workspace) + 256);
     hipError_t e;
     const int lut_dwords = g.rows * g.cols / 2;
+    if (expanded && (e = launch_zero_u32(flags + 1, 1, stream)) != hipSuccess) return e;
     if (g.bits == 8) {
         static std::atomic<uint64_t> attr_done{0};
         if ((e = allow_full_lds(reinterpret_cast<const void*>(expand_fwd_kernel), attr_done)) != hipSuccess) return e;
-        hipLaunchKernelGGL(expand_fwd_kernel, dim3(n_tiles, (k_quads + kExpandQuadsPerWg - 1) / kExpandQuadsPerWg), dim3(256),
-                           (size_t)lut_dwords * 4 + 16, stream, B, reinterpret_cast<const uint32_t*>(lut), lut_dwords, g.cols,
-                           1 << g.bits, E, flags, K, N, k_quads, kSlab8Rows);
+        if (!expanded)
+            hipLaunchKernelGGL(expand_fwd_kernel, dim3(n_tiles, (k_quads + kExpandQuadsPerWg - 1) / kExpandQuadsPerWg), dim3(256),
+                               (size_t)lut_dwords * 4 + 16, stream, B, reinterpret_cast<const uint32_t*>(lut), lut_dwords, g.cols,
+                               1 << g.bits, E, flags, K, N, k_quads, kSlab8Rows);
         if ((e = hipGetLastError()) != hipSuccess) return e;
         const int row_blocks8 = (M + 1023) / 1024;
         const long wgs8 = (long)n_tiles * row_blocks8;
@@ -637,9 +641,10 @@ hipError_t launch_fwd_slab(const uint8_t* A, const uint8_t* B, uint32_t* C, cons
         if (zs8 > 1 && out_f32) return launch_u32_to_f32(C, (size_t)M * N, stream);
         return hipSuccess;
     }
-    hipLaunchKernelGGL(expand_fwd_kernel, dim3(n_tiles, (k_quads + kExpandQuadsPerWg - 1) / kExpandQuadsPerWg), dim3(256),
-                       (size_t)lut_dwords * 4 + 16, stream, B, reinterpret_cast<const uint32_t*>(lut), lut_dwords, g.cols,
-                       1 << g.bits, E, flags, K, N, k_quads, kSlabRows);
+    if (!expanded)
+        hipLaunchKernelGGL(expand_fwd_kernel, dim3(n_tiles, (k_quads + kExpandQuadsPerWg - 1) / kExpandQuadsPerWg), dim3(256),
+                           (size_t)lut_dwords * 4 + 16, stream, B, reinterpret_cast<const uint32_t*>(lut), lut_dwords, g.cols,
+                           1 << g.bits, E, flags, K, N, k_quads, kSlabRows);
     e = hipGetLastError();
     if (e != hipSuccess) return e;
 

@@ -16,6 +16,7 @@ import approx_ops  # native module: approx_gemm_forward / acc_gemm_forward_fp32 
 lut_appmult = None   # uint16 padded table of the approximate products
 lut_grad_a = None    # int16 padded table, 16 x d(product)/d(first operand)
 lut_grad_b = None    # int16 padded table, 16 x d(product)/d(second operand)
+table_generation = 0             # counts set_lookup_tables calls: part of what identifies an expansion kept between calls
 lut_grad_a_fits_halves = False   # whether the expanded-table backward kernels can hold lut_grad_a as halves (int16 tables)
 
 _SECTION_HEADERS = (
@@ -88,7 +89,8 @@ def set_lookup_tables(device, appmult, grad_a, grad_b):
 
     Gradient tables of a floating dtype are installed as float32 and taken as the slopes themselves (no factor 1/16):
     the backward pass then runs on the native float-table entry point."""
-    global lut_appmult, lut_grad_a, lut_grad_b, lut_grad_a_fits_halves
+    global lut_appmult, lut_grad_a, lut_grad_b, lut_grad_a_fits_halves, table_generation
+    table_generation += 1
     lut_appmult = torch.as_tensor(np.ascontiguousarray(appmult, np.uint16)).to(device)
     as_float = np.issubdtype(np.asarray(grad_a).dtype, np.floating) and np.issubdtype(np.asarray(grad_b).dtype, np.floating)
     gdt = np.float32 if as_float else np.int16

@@ -72,6 +72,24 @@ int amr_lut_gemm_forward_ws(const uint8_t *A, const uint8_t *B, uint32_t *C, con
                             void *stream);
 
 /*
+ * The expansion of the forward table along B (K*N*256 B for tables of at most 7 bits: 604 MB for a 4608 x 512 layer) depends
+ * on B and the table only, not on A: a caller whose B stays put between calls -- inference, evaluation, calibration
+ * passes -- keeps it in an amr_fwd_cache, one per weight matrix, and the forward pass skips the expansion launch while the
+ * caller's b_version (any number that changes whenever the contents of B change), the table pointer, K and N stay the
+ * same.  The cache owns its device memory (hipMalloc on the first call and when a larger shape arrives; hipFree, which
+ * waits for the device, on replacement and on destroy).  Calls that share a cache must be ordered with each other (one
+ * stream, or events); results are those of amr_lut_gemm_forward.  Shapes that do not take the expanded-table kernels
+ * ignore the cache.  No counterpart in the reference.
+ *   amr_lut_gemm_forward_cached: C is uint32 [M,N], or float32 when c_is_f32 != 0 (amr_lut_gemm_forward_f32_ws).
+ */
+typedef struct amr_fwd_cache amr_fwd_cache;
+int amr_fwd_cache_create(amr_fwd_cache **out);
+int amr_fwd_cache_destroy(amr_fwd_cache *cache);
+int amr_fwd_cache_stats(amr_fwd_cache *cache, uint64_t *hits, uint64_t *misses, size_t *device_bytes);   /* any pointer may be NULL */
+int amr_lut_gemm_forward_cached(amr_fwd_cache *cache, uint64_t b_version, const uint8_t *A, const uint8_t *B, void *C,
+                                int c_is_f32, const uint16_t *lut, int64_t lut_elems, int M, int K, int N, void *stream);
+
+/*
  * Same sums, stored as float32: C[m,n] = (float)(uint32 sum), rounded to nearest even above 2^24, i.e. the
  * bits of the `.to(torch.float32)` the reference's callers apply to the result at once
  * (self_ops/ops_py/approx_ops.py:569, :165) without the pass over C that conversion costs.
@@ -236,6 +254,12 @@ int amr_lut_conv_forward_dequant_f32(const uint8_t *A, const uint8_t *B, const u
                                      int N, int positions, const float *x_sum, const float *w_resp, const float *taps,
                                      const float *z_a, const float *z_w, const float *s_a, const float *s_w, const float *bias,
                                      float *out, void *workspace, size_t workspace_bytes, void *stream);
+/* The same with the expansion kept in an amr_fwd_cache (cache = NULL: as above). */
+int amr_lut_conv_forward_dequant_cached_f32(amr_fwd_cache *cache, uint64_t b_version, const uint8_t *A, const uint8_t *B,
+                                            const uint16_t *lut, int64_t lut_elems, int M, int K, int N, int positions,
+                                            const float *x_sum, const float *w_resp, const float *taps, const float *z_a,
+                                            const float *z_w, const float *s_a, const float *s_w, const float *bias, float *out,
+                                            void *workspace, size_t workspace_bytes, void *stream);
 
 /*
  * Range tracking and quantisation parameters of one tensor in one launch (all pointers: one float in device memory).

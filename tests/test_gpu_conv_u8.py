@@ -359,3 +359,85 @@ def test_uint8_layer_takes_the_convolution_shaped_input_gradient(ops):
     assert torch.equal(res[0][0], res[1][0])
     for a, b in zip(res[0][1:], res[1][1:]):
         torch.testing.assert_close(a, b, rtol=0, atol=1e-5 * float(b.abs().max()))
+
+
+def test_forward_expansion_cache_hits_and_invalidates(ops, oracle):
+    """amr_lut_gemm_forward_cached through the module function: the first call expands, calls with the same version reuse the
+    expansion (also with other rows A, also after a call whose A held a masked code), a changed B under an unchanged version
+    gives the OLD B's sums -- the expansion really was reused -- and a new version gives the new ones; every result checked
+    against the oracle."""
+    import approx_ops
+    print("forward cache", flush=True)
+    rng = np.random.default_rng(41)
+    M, K, N, bits = 4096, 256, 64, 7
+    T = oracle.synth_lut(bits, 64, rng)
+    flat = oracle.pack_table(T, bits, np.uint16)
+    lut = torch.tensor(flat, device="cuda")
+    A1, A2 = (rng.integers(0, 128, (M, K)).astype(np.uint8) for _ in range(2))
+    A2[7, 5] = 128                                             # a masked code: the gated direct kernel serves this call
+    B1, B2 = (rng.integers(0, 128, (K, N)).astype(np.uint8) for _ in range(2))
+    a1, a2, b = torch.tensor(A1, device="cuda"), torch.tensor(A2, device="cuda"), torch.tensor(B1, device="cuda")
+    c = torch.empty((M, N), dtype=torch.uint32, device="cuda")
+    want = lambda A, B: oracle.forward_c(A, B, flat, bits)
+    got = lambda: c.cpu().numpy().view(np.uint32)
+    cache = approx_ops.ForwardCache()
+    old = approx_ops._lib.amr_set_expanded_table_kernels(2)
+    try:
+        approx_ops.approx_gemm_forward(a1, b, c, lut, cache=cache, b_version=1)
+        assert (got() == want(A1, B1)).all() and cache.stats()[:2] == (0, 1) and cache.stats()[2] >= K * N * 256
+        approx_ops.approx_gemm_forward(a2, b, c, lut, cache=cache, b_version=1)
+        assert (got() == want(A2, B1)).all() and cache.stats()[:2] == (1, 1)
+        approx_ops.approx_gemm_forward(a1, b, c, lut, cache=cache, b_version=1)       # (the fall-back request of the call before is gone)
+        assert (got() == want(A1, B1)).all() and cache.stats()[:2] == (2, 1)
+        b.copy_(torch.tensor(B2))
+        approx_ops.approx_gemm_forward(a1, b, c, lut, cache=cache, b_version=1)       # stale on purpose: same version, other contents
+        assert (got() == want(A1, B1)).all() and cache.stats()[:2] == (3, 1)
+        approx_ops.approx_gemm_forward(a1, b, c, lut, cache=cache, b_version=2)
+        assert (got() == want(A1, B2)).all() and cache.stats()[:2] == (3, 2)
+        cf = torch.empty((M, N), dtype=torch.float32, device="cuda")
+        approx_ops.approx_gemm_forward(a1, b, cf, lut, cache=cache, b_version=2)
+        assert (cf.cpu().numpy() == want(A1, B2).astype(np.float32)).all() and cache.stats()[:2] == (4, 2)
+        # a larger shape replaces the buffer; a shape the expanded-table kernels do not take leaves the cache alone
+        b_big = torch.tensor(rng.integers(0, 128, (2 * K, N)).astype(np.uint8), device="cuda")
+        a_big = torch.tensor(rng.integers(0, 128, (M, 2 * K)).astype(np.uint8), device="cuda")
+        approx_ops.approx_gemm_forward(a_big, b_big, c, lut, cache=cache, b_version=2)
+        assert (got() == want(a_big.cpu().numpy(), b_big.cpu().numpy())).all() and cache.stats()[:2] == (4, 3)
+        small_a, small_c = a1[:100].contiguous(), torch.empty((100, N), dtype=torch.uint32, device="cuda")
+        approx_ops.approx_gemm_forward(small_a, b, small_c, lut, cache=cache, b_version=9)
+        assert (small_c.cpu().numpy().view(np.uint32) == want(A1[:100], B2)).all() and cache.stats()[:2] == (4, 3)
+    finally:
+        approx_ops._lib.amr_set_expanded_table_kernels(old)
+        cache.close()
+
+
+def test_layer_keeps_its_expansion_in_evaluation_mode(ops):
+    """An ApproxConv2d in evaluation mode expands the forward table once for its frozen weights; an in-place weight update, a
+    training-mode pass or new tables make it expand again; outputs equal those of a layer without the cache throughout."""
+    import app_layers as L
+    import copy
+    self_ops, P = ops
+    print("layer forward cache", flush=True)
+    torch.manual_seed(11)
+    layer = L.ApproxConv2d(64, 64, 3, padding=1, bias=False, a_bits=7, w_bits=7).cuda().train()
+    x = torch.randn(16, 64, 32, 32, device="cuda")           # 16384 x 576 x 64: a shape the library expands the table for by itself
+    layer(x)
+    plain = copy.deepcopy(layer)
+    plain.keep_expansion_in_eval = False
+    layer.eval(); plain.eval()
+    with torch.no_grad():
+        for _ in range(3):
+            assert torch.equal(layer(x), plain(x))
+        assert layer._fwd_cache.stats()[:2] == (2, 1)
+        layer.weight.mul_(1.01); plain.weight.mul_(1.01)                       # in place: the version counter moves
+        assert torch.equal(layer(x), plain(x)) and layer._fwd_cache.stats()[:2] == (2, 2)
+        assert torch.equal(layer(x * 0.5), plain(x * 0.5)) and layer._fwd_cache.stats()[:2] == (3, 2)
+        layer.train(); plain.train()
+        assert torch.equal(layer(x * 2), plain(x * 2)) and layer._fwd_cache.stats()[:2] == (3, 2)   # training mode: no cache
+        layer.eval(); plain.eval()
+        assert torch.equal(layer(x), plain(x)) and layer._fwd_cache.stats()[:2] == (3, 3)            # the ranges may have moved
+        keep = (P.lut_appmult, P.lut_grad_a, P.lut_grad_b)
+        try:
+            P.set_lookup_tables("cuda", keep[0].cpu().numpy(), keep[1].cpu().numpy(), keep[2].cpu().numpy())
+            assert torch.equal(layer(x), plain(x)) and layer._fwd_cache.stats()[:2] == (3, 4)        # new tables: expanded again
+        finally:
+            P.lut_appmult, P.lut_grad_a, P.lut_grad_b = keep
