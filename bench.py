@@ -138,8 +138,9 @@ def training_step(torch, dev, tables, bits, batch=512, steps=10):
     """Forward + cross-entropy + backward + SGD update of this package's quantised ResNet-18 (LUT convolutions) on synthetic
     CIFAR-shaped data, after one calibration pass and one untimed step: wall-clock ms per step and images per second.
     The LUT GEMM's share of a step's GPU time is measured in this run, on three further steps outside the timed ones: HIP
-    events on the launch stream around every call of the library's forward and backward GEMM entry points (table expansion,
-    header, finish and gated launches included), summed, over the events around the whole steps."""
+    events on the launch stream around every call of the library's forward and backward LUT entry points (table expansion,
+    header, finish and gated launches included; the forward call includes the dequantising store, the convolution-shaped
+    gradA the finishing of the input gradient), summed, over the events around the whole steps."""
     import app_train
     import approx_ops as native
     from self_ops.ops_py import approx_ops as ops
@@ -158,7 +159,9 @@ def training_step(torch, dev, tables, bits, batch=512, steps=10):
     dt = time.perf_counter() - t0
 
     spans = []
-    names = [n for n in ("approx_gemm_forward", "approx_gemm_backward", "approx_conv_forward_dequant") if hasattr(native, n)]
+    # (the layers reach the LUT kernels through these four functions of the native module; the last one, the convolution-shaped
+    # gradA, finishes the input gradient of the quantiser in the same kernel)
+    names = [n for n in ("approx_gemm_forward", "approx_gemm_backward", "approx_conv_forward_dequant", "approx_conv_input_grad") if hasattr(native, n)]
     originals = {n: getattr(native, n) for n in names}
 
     def timed_call(fn):
