@@ -311,6 +311,11 @@ static void* fwd_cache_lookup(amr_fwd_cache* c, int dev, size_t need, uint64_t v
     return c->buf;
 }
 
+static void fwd_cache_forget(amr_fwd_cache* c) {
+    std::lock_guard<std::mutex> lk(c->mu);
+    c->valid = false;
+}
+
 extern "C" {
 
 int amr_fwd_cache_create(amr_fwd_cache** out) {
@@ -370,6 +375,7 @@ static int forward_impl(const uint8_t* A, const uint8_t* B, uint32_t* C, const u
             if (!ws) return hip_fail(e, "workspace hipMalloc");
         }
         e = amr::launch_fwd_slab(A, B, C, lut, g, M, K, N, n_cu, ws, s, out_f32, nullptr, hit ? 1 : 0);
+        if (cache && e != hipSuccess) fwd_cache_forget(cache);      // (whether the expansion got there is unknown)
     } else {
         e = amr::launch_fwd(A, B, C, lut, g, M, K, N, n_cu, s, out_f32);
     }
@@ -427,6 +433,7 @@ int amr_lut_conv_forward_dequant_cached_f32(amr_fwd_cache* cache, uint64_t b_ver
             if (!e_buf) return hip_fail(e, "cache hipMalloc");
         }
         e = amr::launch_fwd_slab(A, B, reinterpret_cast<uint32_t*>(sums), lut, g, M, K, N, n_cu, e_buf, s, 1, &dq, hit ? 1 : 0);
+        if (cache && e != hipSuccess) fwd_cache_forget(cache);
         return e == hipSuccess ? AMR_OK : hip_fail(e, "forward launch");
     }
     // K split over workgroups, small problems, direct kernels: the sums meet in memory first, a second pass dequantises them

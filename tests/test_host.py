@@ -167,3 +167,60 @@ def test_pad_table_places_entries_like_the_reader_and_the_oracle(oracle, bits):
     assert (flat == oracle.pack_table(t, bits, np.uint16)).all()
     g = rng.standard_normal((n, n)).astype(np.float32)
     assert (P.pad_table(g, bits, np.float32) == oracle.pack_table(g, bits, np.float32)).all()
+
+
+def test_layer_level_entry_points_check_arguments_without_touching_a_device():
+    """The entry points of the quantised layer on uint8 codes reject bad shapes, null pointers and unknown table lengths
+    with an AMR_E* code before anything is launched; the size queries answer 0 for what the kernels do not serve."""
+    lib = _lib()
+    lib.amr_last_error.restype = ctypes.c_char_p
+    vp, i64, i, sz, f = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_size_t, ctypes.c_float
+    lib.amr_quantize_codes_nhwc_u8.argtypes = [vp, vp, vp, f, vp, vp, vp, i, i, i, vp]
+    assert lib.amr_quantize_codes_nhwc_u8(None, None, None, 127.0, None, None, None, 2, 0, 4, None) == -1      # no channels
+    assert lib.amr_quantize_codes_nhwc_u8(None, None, None, 300.0, None, None, None, 2, 3, 4, None) == -1      # codes must fit a byte
+    assert lib.amr_quantize_codes_nhwc_u8(None, None, None, 127.0, None, None, None, 0, 3, 4, None) == 0       # empty batch
+    assert lib.amr_quantize_codes_nhwc_u8(None, None, None, 127.0, None, None, None, 2, 3, 4, None) == -1      # null pointers
+    lib.amr_im2col_nhwc_u8.argtypes = [vp, vp, i, i, i, i, i, i, i, i, i, vp]
+    assert lib.amr_im2col_nhwc_u8(None, None, 2, 3, 4, 4, 5, 5, 1, 0, 1, None) == -1                            # window larger than the image
+    assert lib.amr_im2col_nhwc_u8(None, None, 2, 3, 4, 4, 3, 3, 1, 1, 1, None) == -1                            # null pointers
+    lib.amr_lut_conv_forward_dequant_f32.argtypes = [vp, vp, vp, i64, i, i, i, i] + [vp] * 9 + [vp, sz, vp]
+    call = lambda elems, M, K, N, L: lib.amr_lut_conv_forward_dequant_f32(None, None, None, elems, M, K, N, L, *([None] * 9), None, 0, None)
+    assert call(17408, 10, 4, 4, 3) == -1          # positions must divide M
+    assert call(17000, 12, 4, 4, 3) == -2          # not a padded table length
+    assert call(17408, 0, 4, 4, 3) == 0            # empty problem
+    assert call(17408, 12, 4, 4, 3) == -1          # null pointers
+    lib.amr_lut_conv_forward_dequant_workspace_bytes.argtypes = [i64, i, i, i]
+    lib.amr_lut_conv_forward_dequant_workspace_bytes.restype = sz
+    assert lib.amr_lut_conv_forward_dequant_workspace_bytes(17408, 100, 27, 10) == 100 * 10 * 4
+    lib.amr_lut_conv_input_grad_supported.argtypes = [i64, i, i, i, i, i]
+    lib.amr_lut_conv_input_grad_workspace_bytes.argtypes = [i64, i, i, i, i, i]
+    lib.amr_lut_conv_input_grad_workspace_bytes.restype = sz
+    assert lib.amr_lut_conv_input_grad_supported(17408, 512, 64, 32, 32, 64) == 1
+    assert lib.amr_lut_conv_input_grad_supported(66306, 512, 64, 32, 32, 64) == 0      # 8-bit table
+    assert lib.amr_lut_conv_input_grad_supported(17408, 512, 24, 32, 32, 64) == 0      # channels no multiple of 16
+    assert lib.amr_lut_conv_input_grad_workspace_bytes(17408, 512, 24, 32, 32, 64) == 0
+    assert lib.amr_lut_conv_input_grad_workspace_bytes(17408, 512, 64, 32, 32, 64) == 256 + 512 * 1024 * 4 + 9 * 64 * 64 * 256
+    lib.amr_lut_conv_input_grad_f32.argtypes = [vp] * 4 + [i64] + [vp] * 5 + [i] * 5 + [vp, vp, vp, sz, vp]
+    assert lib.amr_lut_conv_input_grad_f32(*([None] * 4), 17408, *([None] * 5), 512, 64, 32, 32, 64, None, None, None, 0, None) == -1
+    lib.amr_observe_minmax_f32.argtypes = [vp, i64, vp, vp, vp, vp, vp, i] + [f] * 5 + [vp]
+    assert lib.amr_observe_minmax_f32(None, 10, None, None, None, None, None, 3, 0.9, 0.1, 127.0, 0.0, 1e-7, None) == -1   # mode
+    assert lib.amr_observe_minmax_f32(None, 10, None, None, None, None, None, 2, 0.9, 0.1, 127.0, 0.0, 1e-7, None) == -1   # null pointers
+    # the decision on a gradient table in host memory
+    lib.amr_grad_table_fits_halves.argtypes = [vp, i64]
+    small = np.zeros(17408, np.int16); small[:100] = 2048; small[200:300] = -2048
+    wide = small.copy(); wide[5] = 6000
+    shifted = np.zeros(17408, np.int16); shifted[:129 * 130] = 1500; shifted[7] = 3000; shifted[9] = -500
+    assert lib.amr_grad_table_fits_halves(small.ctypes.data, small.size) == 1
+    assert lib.amr_grad_table_fits_halves(wide.ctypes.data, wide.size) == 0            # spans more than 4096
+    assert lib.amr_grad_table_fits_halves(shifted.ctypes.data, shifted.size) == 1      # fits with an offset that does not swamp the entries
+    assert lib.amr_grad_table_fits_halves(small.ctypes.data, 17000) < 0
+    # the cache object lives on the host until it is used
+    h = vp()
+    lib.amr_fwd_cache_create.argtypes = [ctypes.POINTER(vp)]
+    lib.amr_fwd_cache_destroy.argtypes = [vp]
+    lib.amr_fwd_cache_stats.argtypes = [vp, ctypes.POINTER(ctypes.c_uint64), ctypes.POINTER(ctypes.c_uint64), ctypes.POINTER(sz)]
+    assert lib.amr_fwd_cache_create(ctypes.byref(h)) == 0 and h.value
+    hits, misses, held = ctypes.c_uint64(9), ctypes.c_uint64(9), sz(9)
+    assert lib.amr_fwd_cache_stats(h, ctypes.byref(hits), ctypes.byref(misses), ctypes.byref(held)) == 0
+    assert (hits.value, misses.value, held.value) == (0, 0, 0)
+    assert lib.amr_fwd_cache_destroy(h) == 0
