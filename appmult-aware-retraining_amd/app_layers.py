@@ -206,33 +206,41 @@ class _ApproxConvLayerFn(torch.autograd.Function):
     output gradient to GEMM rows (with its row sums) in one pass, the two LUT gradient GEMMs, then col2im + gradient of the
     zero-point term + straight-through backward of the quantiser in one pass.  No float32 code tensor exists on this path.
 
-    ``w_codes`` (float32 integer codes [N,C,kh,kw]) and ``w_resp`` come from the weight side, which stays in torch
-    operators; their gradients are returned for it."""
+    The weight side comes in one of two forms.  ``prepared`` = (b_mat uint8 [kh*kw*C, N], inside_w uint8 [N,C,kh,kw],
+    w_resp float32 [N, L], tapmask float32 [kh*kw, L]) from ``approx_ops.conv_weight_prepare``: then ``w`` is the layer's real
+    weight, ``w_resp`` is None and backward finishes the weight gradient itself (LUT gradient + zero-point term + the
+    quantiser's straight-through backward in one launch).  Without it ``w`` holds float32 integer codes [N,C,kh,kw] and
+    ``w_resp`` their response to an all-ones image, both from torch operators, which receive their gradients."""
 
     @staticmethod
-    def forward(ctx, x, w_codes, w_resp, taps, a_scale, a_zp, w_scale, w_zp, bias, a_qmax, stride, padding, dilation, fwd_cache=None):
+    def forward(ctx, x, w, w_resp, taps, a_scale, a_zp, w_scale, w_zp, bias, a_qmax, stride, padding, dilation, fwd_cache=None,
+                prepared=None):
         import approx_ops
         from self_ops.ops_py import approx_ops as ops
         one = lambda t: t.detach().reshape(1).contiguous()
         s_a, z_a, s_w, z_w = one(a_scale), one(a_zp), one(w_scale), one(w_zp)
         xc = x.detach().contiguous()
-        bn, cin, h, w = xc.shape
-        cout, _, kh, kw = w_codes.shape
+        bn, cin, h, w_in = xc.shape
+        cout, _, kh, kw = w.shape
         s, p, d = stride[0], padding[0], dilation[0]
         oh = (h + 2 * p - d * (kh - 1) - 1) // s + 1
-        ow = (w + 2 * p - d * (kw - 1) - 1) // s + 1
+        ow = (w_in + 2 * p - d * (kw - 1) - 1) // s + 1
         dev = xc.device
-        codes = torch.empty((bn * h * w, cin), dtype=torch.uint8, device=dev)
-        inside = torch.empty((bn, cin, h, w), dtype=torch.uint8, device=dev)
-        xs = torch.empty((bn, 1, h, w), dtype=torch.float32, device=dev)
+        codes = torch.empty((bn * h * w_in, cin), dtype=torch.uint8, device=dev)
+        inside = torch.empty((bn, cin, h, w_in), dtype=torch.uint8, device=dev)
+        xs = torch.empty((bn, 1, h, w_in), dtype=torch.float32, device=dev)
         approx_ops.quantize_codes_nhwc(xc, s_a, z_a, a_qmax, codes, inside, xs)
         if (kh, kw, s, p) == (1, 1, 1, 0):
             a_mat = codes                                           # a 1x1 window is the pixel itself
         else:
             a_mat = torch.empty((bn * oh * ow, kh * kw * cin), dtype=torch.uint8, device=dev)
-            approx_ops.im2col_nhwc(codes, a_mat, (bn, cin, h, w), (kh, kw), s, p, d)
+            approx_ops.im2col_nhwc(codes, a_mat, (bn, cin, h, w_in), (kh, kw), s, p, d)
         # rows of B in the order of A's columns: (tap, channel)
-        b_mat = w_codes.detach().permute(2, 3, 1, 0).reshape(kh * kw * cin, cout).to(torch.uint8).contiguous()
+        if prepared is not None:
+            b_mat, inside_w, w_resp, tapmask = prepared
+        else:
+            b_mat = w.detach().permute(2, 3, 1, 0).reshape(kh * kw * cin, cout).to(torch.uint8).contiguous()
+            inside_w = tapmask = None
         x_sum = _box_sum(xs, (kh, kw), stride, padding, dilation)
         out = torch.empty((bn, cout, oh, ow), dtype=torch.float32, device=dev)
         # (LUT GEMM whose store applies the zero-point terms, the scaling and the bias and writes NCHW)
@@ -243,9 +251,9 @@ class _ApproxConvLayerFn(torch.autograd.Function):
         # a 3x3 / stride 1 / padding 1 layer takes its input gradient from one implicit GEMM over the input pixels (no
         # [M][9C] gradient matrix, no col2im) where the library serves the shape and the gradient table fits halves
         conv_shaped = ((kh, kw, s, p, d) == (3, 3, 1, 1, 1) and ops.lut_grad_a_fits_halves
-                       and approx_ops.conv_input_grad_supported(ops.lut_grad_a, (bn, cin, h, w), cout))
-        ctx.save_for_backward(a_mat, b_mat, inside, s_a, z_a, s_w, z_w, codes if conv_shaped else None)
-        ctx.geo = (bn, cin, h, w, cout, kh, kw, s, p, d, oh, ow)
+                       and approx_ops.conv_input_grad_supported(ops.lut_grad_a, (bn, cin, h, w_in), cout))
+        ctx.save_for_backward(a_mat, b_mat, inside, s_a, z_a, s_w, z_w, codes if conv_shaped else None, inside_w, tapmask)
+        ctx.geo = (bn, cin, h, w_in, cout, kh, kw, s, p, d, oh, ow)
         ctx.aux = (w_resp.shape, bias is not None, x.dtype)
         return out
 
@@ -253,10 +261,12 @@ class _ApproxConvLayerFn(torch.autograd.Function):
     def backward(ctx, g):
         import approx_ops
         from self_ops.ops_py import approx_ops as ops
-        a_mat, b_mat, inside, s_a, z_a, s_w, z_w, codes = ctx.saved_tensors
+        a_mat, b_mat, inside, s_a, z_a, s_w, z_w, codes, inside_w, tapmask = ctx.saved_tensors
         bn, cin, h, w, cout, kh, kw, s, p, d, oh, ow = ctx.geo
         wr_shape, has_bias, x_dtype = ctx.aux
-        need_x, need_w, need_wr = ctx.needs_input_grad[0], ctx.needs_input_grad[1], ctx.needs_input_grad[2]
+        fused_w = inside_w is not None
+        need_x, need_w = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
+        need_wr = need_w if fused_w else ctx.needs_input_grad[2]
         g = g.contiguous()
         dev = g.device
         g_x = g_w = g_wr = g_bias = None
@@ -277,13 +287,20 @@ class _ApproxConvLayerFn(torch.autograd.Function):
                 else:
                     approx_ops.conv_input_grad(g_a, t, z_w, inside, s_a, g_x, (kh, kw), s, p, d)
                 g_x = g_x.to(x_dtype)
-            if need_w:
+            if need_w and not fused_w:
                 g_w = g_b.view(kh, kw, cin, cout).permute(3, 2, 0, 1)
-        if need_wr:
+        if need_wr and fused_w:
+            # gradient of the zero-point term Za * w_resp, then everything that ends in the real weight in one launch
+            g_wr = torch.empty((cout, oh * ow), dtype=torch.float32, device=dev)
+            approx_ops.conv_batch_sum_scaled(g, z_a, s_a, s_w, g_wr)
+            g_w = torch.empty((cout, cin, kh, kw), dtype=torch.float32, device=dev)
+            approx_ops.conv_weight_grad(g_b, g_wr, tapmask, inside_w, s_w, g_w)
+            g_wr = None
+        elif need_wr:
             g_wr = ((z_a * (s_a * s_w)) * g.sum(dim=0, keepdim=True)).reshape(wr_shape)
         if has_bias and ctx.needs_input_grad[8]:
             g_bias = g.sum(dim=(0, 2, 3))
-        return g_x, g_w, g_wr, None, None, None, None, None, g_bias, None, None, None, None, None
+        return g_x, g_w, g_wr, None, None, None, None, None, g_bias, None, None, None, None, None, None
 
 
 # ------------------------------------------------------------------------------------------ quantiser module
@@ -387,6 +404,7 @@ class ApproxConv2d(nn.Conv2d, _QuantParamsMixin):
         self.fused_dequant = True                   # False: zero-point terms and scaling as torch operators
         self.fused_layer = True                     # False: float32 code tensors between quantiser, convolution and dequantisation
         self.keep_expansion_in_eval = True          # evaluation mode: the forward table expanded along the weight codes stays on the device
+        self.fused_weight_side = True               # False: weight codes, their all-ones response and their gradients as torch operators
 
     def quantize_v2(self, x, s, zpn, qmax):
         return _to_codes(x, s, zpn, qmax)
@@ -449,9 +467,46 @@ class ApproxConv2d(nn.Conv2d, _QuantParamsMixin):
                 and self.weight.dtype == torch.float32 and float(self.activation_quant_max) <= 255
                 and self.activation_scale.is_cuda and self.weight_scale.is_cuda)
 
+    def _prepared_weight_side(self, input, frozen):
+        """(b_mat, inside_w, w_resp, tapmask) and taps of ``_ApproxConvLayerFn`` from the real weight in one launch (reference
+        ``app_layers.py:173,179``: quantize_v2 on the weights and conv(Za, W)).  In evaluation mode the result is kept under the
+        number of ``_frozen_weight_cache`` and the geometry."""
+        import approx_ops
+        cin, h, w = input.shape[1:]
+        kh, kw = self.kernel_size
+        key = (frozen[1], h, w) if frozen else None
+        kept = self.__dict__.get("_prepared")
+        if key is not None and kept is not None and kept[0] == key:
+            return kept[1], kept[2]
+        dev = input.device
+        tapmask = self._tap_mask(h, w, kh, kw, self.stride, self.padding, self.dilation, torch.float32, dev)
+        positions = tapmask.shape[1]
+        oh = (h + 2 * self.padding[0] - self.dilation[0] * (kh - 1) - 1) // self.stride[0] + 1
+        tkey = ("taps", h, w, cin, str(dev))
+        masks = self.__dict__["_tap_masks"]
+        if tkey not in masks:
+            masks[tkey] = (tapmask.sum(dim=0) * float(cin)).view(1, 1, oh, positions // oh)
+        cout = self.out_channels
+        b_mat = torch.empty((kh * kw * cin, cout), dtype=torch.uint8, device=dev)
+        inside_w = torch.empty((cout, cin, kh, kw), dtype=torch.uint8, device=dev)
+        w_resp = torch.empty((cout, positions), dtype=torch.float32, device=dev)
+        one = lambda t: t.detach().reshape(1).contiguous()
+        approx_ops.conv_weight_prepare(self.weight.detach().contiguous(), one(self.weight_scale), one(self.weight_zp_neg),
+                                       float(self.weight_quant_max), tapmask, b_mat, inside_w, w_resp)
+        prepared = (b_mat, inside_w, w_resp, tapmask)
+        self.__dict__["_prepared"] = (key, prepared, masks[tkey]) if key is not None else None
+        return prepared, masks[tkey]
+
     def forward(self, input):
         self._update_ranges(input)
         conv_args = dict(bias=None, stride=self.stride, padding=self.padding, dilation=self.dilation, groups=self.groups)
+        if (self.fused_weight_side and self._takes_uint8_path(input) and float(self.weight_quant_max) <= 255
+                and self.kernel_size[0] * self.kernel_size[1] <= 64):
+            frozen = self._frozen_weight_cache()
+            prepared, taps = self._prepared_weight_side(input, frozen)
+            return _ApproxConvLayerFn.apply(input, self.weight, None, taps, self.activation_scale, self.activation_zp_neg,
+                                            self.weight_scale, self.weight_zp_neg, self.bias, float(self.activation_quant_max),
+                                            tuple(self.stride), tuple(self.padding), tuple(self.dilation), frozen, prepared)
         w_codes = self.quantize_v2(self.weight, self.weight_scale, self.weight_zp_neg, self.weight_quant_max)
         if self._takes_uint8_path(input):
             w_resp, taps = self._weight_zero_point_parts(w_codes, input.shape[1:], conv_args, torch.float32, input.device)

@@ -66,6 +66,11 @@ _lib.amr_fwd_cache_destroy.argtypes = [_vp]
 _lib.amr_fwd_cache_stats.argtypes = [_vp, ctypes.POINTER(_u64), ctypes.POINTER(_u64), ctypes.POINTER(_sz)]
 _lib.amr_lut_gemm_forward_cached.argtypes = [_vp, _u64, _vp, _vp, _vp, _i, _vp, _i64, _i, _i, _i, _vp]
 _lib.amr_lut_conv_forward_dequant_cached_f32.argtypes = [_vp, _u64, _vp, _vp, _vp, _i64, _i, _i, _i, _i] + [_vp] * 9 + [_vp, _sz, _vp]
+_lib.amr_conv_weight_prepare_f32.argtypes = [_vp, _vp, _vp, ctypes.c_float, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]
+_lib.amr_conv_batch_sum_workspace_bytes.argtypes = [_i, _i64]
+_lib.amr_conv_batch_sum_workspace_bytes.restype = _sz
+_lib.amr_conv_batch_sum_scaled_f32.argtypes = [_vp, _vp, _vp, _vp, _vp, _i, _i64, _vp, _sz, _vp]
+_lib.amr_conv_weight_grad_f32.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]
 _lib.amr_quantize_codes_nhwc_u8.argtypes = [_vp, _vp, _vp, ctypes.c_float, _vp, _vp, _vp, _i, _i, _i, _vp]
 _lib.amr_im2col_nhwc_u8.argtypes = [_vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp]
 _lib.amr_conv_input_grad_f32.argtypes = [_vp] * 6 + [_i] * 9 + [_vp]
@@ -515,6 +520,67 @@ def conv_input_grad(cols_tensor, t_tensor, z_w, inside_tensor, scale_tensor, gx_
                                           inside_tensor.data_ptr(), scale_tensor.data_ptr(), gx_tensor.data_ptr(), Bn, C, H, W, kh, kw,
                                           stride, padding, dilation, _stream_ptr(dev))
     _raise_for(rc, "conv_input_grad")
+
+
+def conv_weight_prepare(w_tensor, scale_tensor, zp_neg_tensor, quant_max, tapmask, bt_tensor, inside_tensor, wresp_tensor):
+    """Weight operand of the quantised LUT convolution in one launch: bt uint8 [taps*C, N] (codes, tap-major rows), inside
+    uint8 [N,C,kh,kw] (mask of the straight-through backward), wresp float32 [N, L] (response of the codes to an all-ones
+    image) from w float32 [N,C,kh,kw] and tapmask float32 [taps, L]."""
+    for t, name, dt in ((w_tensor, "w_tensor", torch.float32), (scale_tensor, "scale_tensor", torch.float32),
+                        (zp_neg_tensor, "zp_neg_tensor", torch.float32), (tapmask, "tapmask", torch.float32),
+                        (bt_tensor, "bt_tensor", torch.uint8), (inside_tensor, "inside_tensor", torch.uint8),
+                        (wresp_tensor, "wresp_tensor", torch.float32)):
+        _check_input(t, dt, name)
+    _check(w_tensor.dim() == 4 and tapmask.dim() == 2, "w must be 4-D and tapmask 2-D")
+    N, C, kh, kw = w_tensor.shape
+    T, L = kh * kw, tapmask.size(1)
+    _check(tapmask.size(0) == T and T <= 64, f"tapmask should have {T} rows (at most 64 taps)")
+    _check(tuple(bt_tensor.shape) == (T * C, N), f"bt_tensor's shape should be {T * C} x {N}")
+    _check(inside_tensor.shape == w_tensor.shape and wresp_tensor.numel() == N * L, "inside or wresp has the wrong size")
+    _check(scale_tensor.numel() == 1 and zp_neg_tensor.numel() == 1 and 0 <= quant_max <= 255, "bad scale, zero point or code range")
+    dev = w_tensor.device
+    _check(all(t.device == dev for t in (scale_tensor, zp_neg_tensor, tapmask, bt_tensor, inside_tensor, wresp_tensor)), "All tensors should be on the same device")
+    with torch.cuda.device(dev):
+        rc = _lib.amr_conv_weight_prepare_f32(w_tensor.data_ptr(), scale_tensor.data_ptr(), zp_neg_tensor.data_ptr(), float(quant_max),
+                                              tapmask.data_ptr(), bt_tensor.data_ptr(), inside_tensor.data_ptr(), wresp_tensor.data_ptr(),
+                                              N, C, T, L, _stream_ptr(dev))
+    _raise_for(rc, "conv_weight_prepare")
+
+
+def conv_batch_sum_scaled(g_tensor, z_a, s_a, s_w, out_tensor):
+    """out[j] = (z_a * (s_a * s_w)) * sum over the batch of g[b].flatten()[j]; g float32 [B, ...] contiguous, out float32 with the
+    elements of one batch entry; scalars one-element device tensors.  Fixed summation order."""
+    for t, name in ((g_tensor, "g_tensor"), (z_a, "z_a"), (s_a, "s_a"), (s_w, "s_w"), (out_tensor, "out_tensor")):
+        _check_input(t, torch.float32, name)
+    Bn = g_tensor.size(0)
+    inner = g_tensor.numel() // max(Bn, 1)
+    _check(Bn > 0 and inner > 0 and out_tensor.numel() == inner, "out must hold the elements of one batch entry")
+    _check(all(t.numel() == 1 for t in (z_a, s_a, s_w)), "z_a, s_a and s_w must hold one element")
+    dev = g_tensor.device
+    with torch.cuda.device(dev):
+        need = _lib.amr_conv_batch_sum_workspace_bytes(Bn, inner)
+        ws = torch.empty(max(need, 16), dtype=torch.uint8, device=dev)
+        rc = _lib.amr_conv_batch_sum_scaled_f32(g_tensor.data_ptr(), z_a.data_ptr(), s_a.data_ptr(), s_w.data_ptr(), out_tensor.data_ptr(), Bn,
+                                                inner, ws.data_ptr(), ws.numel(), _stream_ptr(dev))
+    _raise_for(rc, "conv_batch_sum_scaled")
+
+
+def conv_weight_grad(gbt_tensor, gwr_tensor, tapmask, inside_tensor, scale_tensor, gw_tensor):
+    """gw[n,c,tap] = inside ? (gbt[tap*C + c, n] + sum over pos of gwr[n, pos] * tapmask[tap, pos]) / scale : 0; gbt float32
+    [taps*C, N], gwr float32 [N, L], gw float32 [N,C,kh,kw]."""
+    for t, name, dt in ((gbt_tensor, "gbt_tensor", torch.float32), (gwr_tensor, "gwr_tensor", torch.float32), (tapmask, "tapmask", torch.float32),
+                        (inside_tensor, "inside_tensor", torch.uint8), (scale_tensor, "scale_tensor", torch.float32), (gw_tensor, "gw_tensor", torch.float32)):
+        _check_input(t, dt, name)
+    _check(gw_tensor.dim() == 4 and inside_tensor.shape == gw_tensor.shape, "gw must be 4-D and inside of its shape")
+    N, C, kh, kw = gw_tensor.shape
+    T, L = kh * kw, tapmask.size(1)
+    _check(tuple(tapmask.shape) == (T, L) and T <= 64, f"tapmask should have {T} rows (at most 64 taps)")
+    _check(tuple(gbt_tensor.shape) == (T * C, N) and gwr_tensor.numel() == N * L and scale_tensor.numel() == 1, "gbt, gwr or scale has the wrong size")
+    dev = gw_tensor.device
+    with torch.cuda.device(dev):
+        rc = _lib.amr_conv_weight_grad_f32(gbt_tensor.data_ptr(), gwr_tensor.data_ptr(), tapmask.data_ptr(), inside_tensor.data_ptr(),
+                                           scale_tensor.data_ptr(), gw_tensor.data_ptr(), N, C, T, L, _stream_ptr(dev))
+    _raise_for(rc, "conv_weight_grad")
 
 
 def grad_table_fits_halves(table_i16):

@@ -281,6 +281,148 @@ hipError_t launch_window_sums_3x3(const float* t, float* zt, long B, int H, int 
     return hipGetLastError();
 }
 
+// ------------------------------------------------------------------------------------------ weight side of the layer
+// Weight operand of the quantised LUT convolution in one launch (the reference: quantize_v2 on the weights, the cast and the
+// transposes in front of the GEMM, and the zero-point convolution conv(Za, W); micronet+/app_layers.py:173,179 and
+// self_ops/ops_py/approx_ops.py:560-561):
+//   Bt[(tap*C + c)*N + n] = code of w[n][c][tap]            (uint8, rows in tap-major order)
+//   inside[n][c][tap]     = the rounded value lay in [0, qmax] (mask of the straight-through backward)
+//   w_resp[n][pos]        = sum over taps of (sum over c of the codes) * tapmask[tap][pos]
+// One workgroup per output channel n.  The sums are integers below 2^24: exact in float32 in any order.
+constexpr int kWpMaxTaps = 64;
+__global__ __launch_bounds__(256) void conv_weight_prepare_kernel(const float* __restrict__ w, const float* __restrict__ scale,
+                                                                  const float* __restrict__ zp_neg, float qmax,
+                                                                  const float* __restrict__ tapmask, uint8_t* __restrict__ Bt,
+                                                                  uint8_t* __restrict__ inside, float* __restrict__ w_resp, int N, int C,
+                                                                  int T, int L) {
+    __shared__ float wsum[kWpMaxTaps];
+    const int n = blockIdx.x;
+    const float s = *scale, zp = *zp_neg;
+    if (threadIdx.x < kWpMaxTaps) wsum[threadIdx.x] = 0.f;
+    __syncthreads();
+    const int per_n = C * T;
+    const float* wn = w + (size_t)n * per_n;
+    for (int idx = threadIdx.x; idx < per_n; idx += 256) {
+        const int c = idx / T, tap = idx - c * T;
+        uint32_t in;
+        const uint32_t code = quant_code_u8(wn[idx], s, zp, qmax, &in);
+        Bt[((size_t)tap * C + c) * N + n] = (uint8_t)code;
+        inside[(size_t)n * per_n + idx] = (uint8_t)in;
+        atomicAdd(&wsum[tap], (float)code);         // (LDS; integer-valued: any order gives the same float)
+    }
+    __syncthreads();
+    for (int pos = threadIdx.x; pos < L; pos += 256) {
+        float acc = 0.f;
+        for (int tap = 0; tap < T; ++tap) acc += wsum[tap] * tapmask[(size_t)tap * L + pos];
+        w_resp[(size_t)n * L + pos] = acc;
+    }
+}
+
+hipError_t launch_conv_weight_prepare(const float* w, const float* scale, const float* zp_neg, float qmax, const float* tapmask,
+                                      uint8_t* Bt, uint8_t* inside, float* w_resp, int N, int C, int T, int L, hipStream_t stream) {
+    hipLaunchKernelGGL(conv_weight_prepare_kernel, dim3(N), dim3(256), 0, stream, w, scale, zp_neg, qmax, tapmask, Bt, inside, w_resp, N, C,
+                       T, L);
+    return hipGetLastError();
+}
+
+// out[j] = (*z_a * (*s_a * *s_w)) * sum over b of g[b][j], j < inner: the gradient of the zero-point term conv(Za, W) with
+// respect to w_resp, summed over the batch.  Two launches: S segments of the batch into partial sums (a thread owns four
+// neighbouring j and walks its segment with four loads in flight), then the segments in ascending order.  Fixed order.
+__global__ __launch_bounds__(256) void batch_sum_partial_kernel(const float* __restrict__ g, float* __restrict__ partial, int B, size_t inner,
+                                                                int seg_len) {
+    const size_t j4 = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (j4 >= inner) return;
+    const int b0 = blockIdx.y * seg_len, b1 = min(B, b0 + seg_len);
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    const bool vec = j4 + 3 < inner && (inner & 3) == 0;
+    if (vec) {
+        int b = b0;
+        for (; b + 3 < b1; b += 4) {
+            f32x4 v[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) v[u] = *reinterpret_cast<const f32x4*>(g + (size_t)(b + u) * inner + j4);
+#pragma unroll
+            for (int u = 0; u < 4; ++u) acc = acc + v[u];
+        }
+        for (; b < b1; ++b) acc = acc + *reinterpret_cast<const f32x4*>(g + (size_t)b * inner + j4);
+        *reinterpret_cast<f32x4*>(partial + (size_t)blockIdx.y * inner + j4) = acc;
+    } else {
+        for (int e = 0; e < 4 && j4 + e < inner; ++e) {
+            float a = 0.f;
+            for (int b = b0; b < b1; ++b) a += g[(size_t)b * inner + j4 + e];
+            partial[(size_t)blockIdx.y * inner + j4 + e] = a;
+        }
+    }
+}
+
+__global__ __launch_bounds__(256) void batch_sum_finish_kernel(const float* __restrict__ partial, const float* __restrict__ za_p,
+                                                               const float* __restrict__ sa_p, const float* __restrict__ sw_p,
+                                                               float* __restrict__ out, size_t inner, int segs) {
+    const size_t j = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (j >= inner) return;
+    float acc = partial[j];
+    for (int s = 1; s < segs; ++s) acc += partial[(size_t)s * inner + j];
+    out[j] = __fmul_rn(__fmul_rn(*za_p, __fmul_rn(*sa_p, *sw_p)), acc);
+}
+
+int batch_sum_segments(int B, size_t inner, int n_cu) {
+    // enough workgroups to fill the device, at least 8 images per segment
+    const size_t wg_per_seg = (inner / 4 + 255) / 256;
+    int segs = (int)((4 * (size_t)n_cu + wg_per_seg - 1) / (wg_per_seg ? wg_per_seg : 1));
+    if (segs > B / 8) segs = B / 8;
+    if (segs > 64) segs = 64;
+    return segs < 1 ? 1 : segs;
+}
+
+hipError_t launch_batch_sum_scaled(const float* g, const float* za, const float* sa, const float* sw, float* out, float* partial, int B,
+                                   size_t inner, int n_cu, hipStream_t stream) {
+    const int segs = batch_sum_segments(B, inner, n_cu);
+    const int seg_len = (B + segs - 1) / segs;
+    const int used = (B + seg_len - 1) / seg_len;
+    hipLaunchKernelGGL(batch_sum_partial_kernel, dim3((unsigned)((inner / 4 + 256) / 256), used), dim3(256), 0, stream, g, partial, B, inner,
+                       seg_len);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(batch_sum_finish_kernel, dim3((unsigned)((inner + 255) / 256)), dim3(256), 0, stream, partial, za, sa, sw, out, inner,
+                       used);
+    return hipGetLastError();
+}
+
+// Weight gradient of the layer, finished in one launch: the LUT gradient gBt [T*C][N] (tap-major rows, what gradB wrote), the
+// zero-point term -- g_wr [N][L] spread over the taps a position has, gz[tap] = sum over pos of g_wr[n][pos] * tapmask[tap][pos]
+// (fixed order) -- and the quantiser's straight-through backward:  gw[n][c][tap] = inside ? (gBt + gz[tap]) / *scale : 0.
+__global__ __launch_bounds__(256) void conv_weight_grad_kernel(const float* __restrict__ gBt, const float* __restrict__ g_wr,
+                                                               const float* __restrict__ tapmask, const uint8_t* __restrict__ inside,
+                                                               const float* __restrict__ scale, float* __restrict__ gw, int N, int C, int T,
+                                                               int L) {
+    __shared__ float red[4][kWpMaxTaps];
+    __shared__ float gz[kWpMaxTaps];
+    const int n = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    for (int tap = 0; tap < T; ++tap) {
+        float acc = 0.f;
+        for (int pos = threadIdx.x; pos < L; pos += 256) acc += g_wr[(size_t)n * L + pos] * tapmask[(size_t)tap * L + pos];
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) acc += __shfl_xor(acc, o);
+        if (lane == 0) red[wave][tap] = acc;
+    }
+    __syncthreads();
+    if (threadIdx.x < T) gz[threadIdx.x] = (red[0][threadIdx.x] + red[1][threadIdx.x]) + (red[2][threadIdx.x] + red[3][threadIdx.x]);
+    __syncthreads();
+    const float s = *scale;
+    const int per_n = C * T;
+    for (int idx = threadIdx.x; idx < per_n; idx += 256) {
+        const int c = idx / T, tap = idx - c * T;
+        const float v = gBt[((size_t)tap * C + c) * N + n] + gz[tap];
+        gw[(size_t)n * per_n + idx] = inside[(size_t)n * per_n + idx] ? v / s : 0.f;
+    }
+}
+
+hipError_t launch_conv_weight_grad(const float* gBt, const float* g_wr, const float* tapmask, const uint8_t* inside, const float* scale,
+                                   float* gw, int N, int C, int T, int L, hipStream_t stream) {
+    hipLaunchKernelGGL(conv_weight_grad_kernel, dim3(N), dim3(256), 0, stream, gBt, g_wr, tapmask, inside, scale, gw, N, C, T, L);
+    return hipGetLastError();
+}
+
 // Queued behind a kernel that finished gx itself: marks every element NaN when *gate says that kernel met what it cannot
 // serve (and nobody queued a recomputation); otherwise its few workgroups leave at once.
 __global__ __launch_bounds__(256) void poison_if_raised_kernel(float* __restrict__ gx, size_t total, const uint32_t* __restrict__ gate) {

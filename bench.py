@@ -117,9 +117,9 @@ def capture_codes(torch, dev, bits, tables, arch, batch):
     natives = {n: getattr(ops.approx_ops, n) for n in names}
 
     def spy_on(fn):
-        def spy(a, b, *rest):
+        def spy(a, b, *rest, **kw):
             seen.setdefault((a.shape[0], a.shape[1], b.shape[1]), (a.clone(), b.clone()))
-            return fn(a, b, *rest)
+            return fn(a, b, *rest, **kw)
         return spy
 
     for n in names:

@@ -329,6 +329,27 @@ int amr_conv_input_grad_f32(const float *cols, const float *t, const float *z_w,
                             float *gx, int B, int C, int H, int W, int kh, int kw, int stride, int pad, int dil, void *stream);
 
 /*
+ * Weight side of the quantised LUT convolution, one launch each way (the reference: quantize_v2 on the weights, the cast and
+ * transposes in front of the GEMM and the zero-point convolution conv(Za, W), micronet+/app_layers.py:173,179 with
+ * self_ops/ops_py/approx_ops.py:560-561, and their autograd graph):
+ *   prepare:  Bt[(tap*C + c)*N + n] = code of w[n][c][tap] (uint8, the GEMM's B with tap-major rows); inside[n][c][tap] = 1 where
+ *             the rounded value lay in [0, qmax]; w_resp[n][pos] = sum over taps of (sum over c of the codes) * tapmask[tap][pos]
+ *             -- the response of the weight codes to an all-ones image, tapmask[tap][pos] = 1 where tap `tap` of output position
+ *             `pos` lies inside the image.  w [N][C][taps] float32; scale, zp_neg device scalars; at most 64 taps.
+ *   batch sum: out[j] = (*z_a * (*s_a * *s_w)) * sum over b of g[b][j] (fixed order; workspace of
+ *             amr_conv_batch_sum_workspace_bytes bytes): with g the output gradient [B][N*L] this is the gradient with respect to w_resp.
+ *   grad:     gw[n][c][tap] = inside ? (gBt[(tap*C + c)*N + n] + sum over pos of g_wr[n][pos] * tapmask[tap][pos]) / *scale : 0,
+ *             gBt the gB of amr_lut_gemm_backward_ex for the tap-major operands.
+ */
+int amr_conv_weight_prepare_f32(const float *w, const float *scale, const float *zp_neg, float qmax, const float *tapmask,
+                                uint8_t *Bt, uint8_t *inside, float *w_resp, int N, int C, int taps, int positions, void *stream);
+size_t amr_conv_batch_sum_workspace_bytes(int batch, int64_t inner);
+int amr_conv_batch_sum_scaled_f32(const float *g, const float *z_a, const float *s_a, const float *s_w, float *out, int batch,
+                                  int64_t inner, void *workspace, size_t workspace_bytes, void *stream);
+int amr_conv_weight_grad_f32(const float *gBt, const float *g_wr, const float *tapmask, const uint8_t *inside, const float *scale,
+                             float *gw, int N, int C, int taps, int positions, void *stream);
+
+/*
  * Input gradient of a quantised 3x3 LUT convolution of stride 1 and padding 1 WITHOUT the [M][9C] gradient matrix: gradA of
  * amr_lut_gemm_backward_ex, amr_col2im_f32 and amr_conv_input_grad_f32 as one implicit GEMM over the B*H*W input pixels,
  *   gx[b,c,y,x] = inside[b,c,y,x] ? ((1/16) * sum over taps (ti,tj) and n of gC[(b, y+1-ti, x+1-tj), n] *

@@ -143,8 +143,8 @@ def test_uint8_layer_path_equals_float_code_path_and_oracle(ops, oracle, golden_
     layer.eval()                                      # frozen observers: both paths see the same scales
     gy = None
     res = []
-    for fused in (True, False):
-        layer.fused_layer = fused
+    for fused, fused_w in ((True, True), (False, True), (True, False)):
+        layer.fused_layer, layer.fused_weight_side = fused, fused_w
         xi = x.clone().requires_grad_()
         layer.zero_grad()
         y = layer(xi)
@@ -152,13 +152,16 @@ def test_uint8_layer_path_equals_float_code_path_and_oracle(ops, oracle, golden_
             gy = torch.randn_like(y)
         y.backward(gy)
         res.append((y.detach(), xi.grad, layer.weight.grad.clone(), layer.bias.grad.clone() if bias else None))
+    layer.fused_layer = False
     assert layer._takes_uint8_path(x) is False
     layer.fused_layer = True
     assert layer._takes_uint8_path(x) is True
-    assert res[0][0].is_contiguous() and torch.equal(res[0][0], res[1][0])
-    for a, b in zip(res[0][1:], res[1][1:]):
-        if a is not None:
-            torch.testing.assert_close(a, b, rtol=1e-5, atol=2e-6 * float(b.abs().max()))
+    # (weight side in one launch each way, weight side in torch operators) against the float32 code path
+    for other in (res[0], res[2]):
+        assert other[0].is_contiguous() and torch.equal(other[0], res[1][0])
+        for a, b in zip(other[1:], res[1][1:]):
+            if a is not None:
+                torch.testing.assert_close(a, b, rtol=1e-5, atol=2e-6 * float(b.abs().max()))
     # the reference's expression with the oracle's LUT convolution
     s_a, z_a, s_w, z_w = (float(t) for t in (layer.activation_scale, layer.activation_zp_neg, layer.weight_scale, layer.weight_zp_neg))
     xc = L._to_codes_torch(x, layer.activation_scale, layer.activation_zp_neg, 127.0)
@@ -170,6 +173,73 @@ def test_uint8_layer_path_equals_float_code_path_and_oracle(ops, oracle, golden_
              + conv(torch.full_like(xc, z_a), torch.full_like(wc, z_w)))
     want = s_a * s_w * total + (layer.bias.detach().double().view(1, -1, 1, 1) if bias else 0.0)
     torch.testing.assert_close(res[0][0].double(), want, rtol=1e-5, atol=1e-5 * float(want.abs().max()))
+
+
+@pytest.mark.parametrize("n,c,k,hw,stride,padding,dilation", [
+    (24, 16, 3, (12, 12), 1, 1, 1), (7, 5, 3, (9, 7), 2, 1, 1), (40, 32, 1, (8, 8), 1, 0, 1), (64, 3, 7, (20, 20), 2, 3, 1),
+    (12, 300, 3, (6, 6), 1, 2, 2), (512, 512, 3, (4, 4), 1, 1, 1)])
+def test_weight_side_in_one_launch_each_way(ops, n, c, k, hw, stride, padding, dilation):
+    """conv_weight_prepare against the torch operators it replaces (codes, tap-major operand, in-range mask, response to an
+    all-ones image: integer valued, so exact), conv_batch_sum_scaled against a float64 sum, and conv_weight_grad against
+    autograd through those operators in float64."""
+    import approx_ops
+    import app_layers as L
+    print("weight side", n, c, k, hw, stride, padding, dilation, flush=True)
+    g = torch.Generator(device="cuda").manual_seed(n * 131 + c)
+    w = torch.randn(n, c, k, k, device="cuda", generator=g) * 0.2
+    scale = torch.tensor([0.0041], device="cuda")
+    zpn = torch.tensor([-57.0], device="cuda")                  # some weights fall outside the code range on both sides
+    qmax = 127.0
+    ones = torch.ones(1, 1, *hw, device="cuda")
+    tapmask = F.unfold(ones, (k, k), dilation=dilation, padding=padding, stride=stride)[0].contiguous()
+    T, Lp = tapmask.shape
+    bt = torch.empty(T * c, n, dtype=torch.uint8, device="cuda")
+    inside = torch.empty(n, c, k, k, dtype=torch.uint8, device="cuda")
+    wresp = torch.empty(n, Lp, device="cuda")
+    approx_ops.conv_weight_prepare(w, scale, zpn, qmax, tapmask, bt, inside, wresp)
+    q = w / scale - zpn
+    codes = torch.clamp(torch.round(q), 0, qmax)
+    assert torch.equal(codes, L._to_codes_torch(w, scale, zpn, torch.tensor(qmax, device="cuda")))
+    assert torch.equal(bt, codes.permute(2, 3, 1, 0).reshape(T * c, n).to(torch.uint8))
+    r = torch.round(q)
+    assert torch.equal(inside.bool(), (r >= 0) & (r <= qmax))
+    assert 0 < int(inside.sum()) < inside.numel()
+    want_resp = F.conv2d(torch.ones(1, c, *hw, device="cuda", dtype=torch.float64), codes.double(), stride=stride, padding=padding, dilation=dilation)
+    assert torch.equal(wresp.double().view(-1), want_resp.view(-1))
+    # batch sum with the three scalars
+    bn = 37
+    gout = torch.randn(bn, n, Lp, device="cuda", generator=g)
+    z_a, s_a, s_w = (torch.tensor([v], device="cuda") for v in (-3.0, 0.013, 0.0041))
+    gwr = torch.empty(n, Lp, device="cuda")
+    approx_ops.conv_batch_sum_scaled(gout, z_a, s_a, s_w, gwr)
+    want = (z_a * (s_a * s_w)).double() * gout.double().sum(dim=0)
+    torch.testing.assert_close(gwr.double(), want, rtol=1e-5, atol=1e-6 * float(want.abs().max()))
+    # weight gradient: autograd through codes -> (operand gradient, response) in float64
+    gbt = torch.randn(T * c, n, device="cuda", generator=g)
+    gw = torch.empty_like(w)
+    approx_ops.conv_weight_grad(gbt, gwr, tapmask, inside, scale, gw)
+    wd = w.double().requires_grad_()
+    qd = wd / scale.double() - zpn.double()
+    cd = torch.clamp(qd - qd.detach() + torch.round(q).double(), 0, qmax)
+    resp = cd.sum(dim=1).reshape(n, T) @ tapmask.double()
+    loss = (cd.permute(2, 3, 1, 0).reshape(T * c, n) * gbt.double()).sum() + (resp * gwr.double()).sum()
+    loss.backward()
+    torch.testing.assert_close(gw.double(), wd.grad, rtol=1e-5, atol=2e-6 * float(wd.grad.abs().max()))
+
+
+def test_batch_sum_of_a_large_gradient_and_ragged_sizes(ops):
+    import approx_ops
+    g = torch.Generator(device="cuda").manual_seed(5)
+    one = lambda v: torch.tensor([v], device="cuda")
+    for bn, inner in ((512, 64 * 1024), (3, 10), (130, 4098), (9, 7), (64, 512 * 16)):
+        x = torch.randn(bn, inner, device="cuda", generator=g)
+        out = torch.empty(inner, device="cuda")
+        approx_ops.conv_batch_sum_scaled(x, one(2.0), one(0.5), one(3.0), out)
+        want = 3.0 * x.double().sum(dim=0)
+        torch.testing.assert_close(out.double(), want, rtol=1e-5, atol=1e-6 * float(want.abs().max()))
+        again = torch.empty(inner, device="cuda")
+        approx_ops.conv_batch_sum_scaled(x, one(2.0), one(0.5), one(3.0), again)
+        assert torch.equal(out, again)                      # fixed summation order
 
 
 def test_uint8_layer_path_first_layer_needs_no_input_gradient(ops):
