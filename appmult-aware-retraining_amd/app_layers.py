@@ -291,11 +291,10 @@ class _ApproxConvLayerFn(torch.autograd.Function):
                 g_w = g_b.view(kh, kw, cin, cout).permute(3, 2, 0, 1)
         if need_wr and fused_w:
             # gradient of the zero-point term Za * w_resp, then everything that ends in the real weight in one launch
-            g_wr = torch.empty((cout, oh * ow), dtype=torch.float32, device=dev)
-            approx_ops.conv_batch_sum_scaled(g, z_a, s_a, s_w, g_wr)
+            g_z = torch.empty((approx_ops.conv_zero_point_grad_parts(oh * ow), cout, kh * kw), dtype=torch.float32, device=dev)
+            approx_ops.conv_zero_point_grad(g, z_a, s_a, s_w, tapmask, g_z)
             g_w = torch.empty((cout, cin, kh, kw), dtype=torch.float32, device=dev)
-            approx_ops.conv_weight_grad(g_b, g_wr, tapmask, inside_w, s_w, g_w)
-            g_wr = None
+            approx_ops.conv_weight_grad(g_b, g_z, inside_w, s_w, g_w)
         elif need_wr:
             g_wr = ((z_a * (s_a * s_w)) * g.sum(dim=0, keepdim=True)).reshape(wr_shape)
         if has_bias and ctx.needs_input_grad[8]:

@@ -67,10 +67,11 @@ _lib.amr_fwd_cache_stats.argtypes = [_vp, ctypes.POINTER(_u64), ctypes.POINTER(_
 _lib.amr_lut_gemm_forward_cached.argtypes = [_vp, _u64, _vp, _vp, _vp, _i, _vp, _i64, _i, _i, _i, _vp]
 _lib.amr_lut_conv_forward_dequant_cached_f32.argtypes = [_vp, _u64, _vp, _vp, _vp, _i64, _i, _i, _i, _i] + [_vp] * 9 + [_vp, _sz, _vp]
 _lib.amr_conv_weight_prepare_f32.argtypes = [_vp, _vp, _vp, ctypes.c_float, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]
-_lib.amr_conv_batch_sum_workspace_bytes.argtypes = [_i, _i64]
-_lib.amr_conv_batch_sum_workspace_bytes.restype = _sz
-_lib.amr_conv_batch_sum_scaled_f32.argtypes = [_vp, _vp, _vp, _vp, _vp, _i, _i64, _vp, _sz, _vp]
-_lib.amr_conv_weight_grad_f32.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]
+_lib.amr_conv_zero_point_grad_workspace_bytes.argtypes = [_i, _i, _i]
+_lib.amr_conv_zero_point_grad_workspace_bytes.restype = _sz
+_lib.amr_conv_zero_point_grad_f32.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _sz, _vp]
+_lib.amr_conv_zero_point_grad_parts.argtypes = [_i]
+_lib.amr_conv_weight_grad_f32.argtypes = [_vp, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _vp]
 _lib.amr_quantize_codes_nhwc_u8.argtypes = [_vp, _vp, _vp, ctypes.c_float, _vp, _vp, _vp, _i, _i, _i, _vp]
 _lib.amr_im2col_nhwc_u8.argtypes = [_vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp]
 _lib.amr_conv_input_grad_f32.argtypes = [_vp] * 6 + [_i] * 9 + [_vp]
@@ -547,39 +548,57 @@ def conv_weight_prepare(w_tensor, scale_tensor, zp_neg_tensor, quant_max, tapmas
     _raise_for(rc, "conv_weight_prepare")
 
 
-def conv_batch_sum_scaled(g_tensor, z_a, s_a, s_w, out_tensor):
-    """out[j] = (z_a * (s_a * s_w)) * sum over the batch of g[b].flatten()[j]; g float32 [B, ...] contiguous, out float32 with the
-    elements of one batch entry; scalars one-element device tensors.  Fixed summation order."""
-    for t, name in ((g_tensor, "g_tensor"), (z_a, "z_a"), (s_a, "s_a"), (s_w, "s_w"), (out_tensor, "out_tensor")):
+def conv_zero_point_grad(g_tensor, z_a, s_a, s_w, tapmask, gz_tensor, gwr_tensor=None):
+    """Gradient of the zero-point term Za * w_resp: gwr[n, pos] = (z_a * (s_a * s_w)) * sum over the batch of g[b, n, pos]
+    (optional output) and gz[p, n, tap] = sum over the positions pos of block p of gwr[n, pos] * tapmask[tap, pos], in
+    ``conv_zero_point_grad_parts(L)`` blocks of positions (``conv_weight_grad`` adds the blocks; gz.sum(0) is the whole sum).
+    g float32 [B, N, ...] contiguous, tapmask float32 [taps, L], gz float32 [parts, N, taps]; scalars one-element device
+    tensors.  Fixed summation order."""
+    tensors = [(g_tensor, "g_tensor"), (z_a, "z_a"), (s_a, "s_a"), (s_w, "s_w"), (tapmask, "tapmask"), (gz_tensor, "gz_tensor")]
+    if gwr_tensor is not None:
+        tensors.append((gwr_tensor, "gwr_tensor"))
+    for t, name in tensors:
         _check_input(t, torch.float32, name)
-    Bn = g_tensor.size(0)
-    inner = g_tensor.numel() // max(Bn, 1)
-    _check(Bn > 0 and inner > 0 and out_tensor.numel() == inner, "out must hold the elements of one batch entry")
+    _check(g_tensor.dim() >= 2 and tapmask.dim() == 2, "g must be [B, N, ...] and tapmask [taps, L]")
+    Bn, N = g_tensor.size(0), g_tensor.size(1)
+    T, L = tapmask.shape
+    _check(Bn > 0 and N > 0 and g_tensor.numel() == Bn * N * L, "g does not hold N x L elements per batch entry")
+    parts = _lib.amr_conv_zero_point_grad_parts(L)
+    _check(tuple(gz_tensor.shape) == (parts, N, T) and T <= 64, f"gz_tensor's shape should be {parts} x {N} x {T} (at most 64 taps)")
+    _check(gwr_tensor is None or gwr_tensor.numel() == N * L, "gwr_tensor has the wrong size")
     _check(all(t.numel() == 1 for t in (z_a, s_a, s_w)), "z_a, s_a and s_w must hold one element")
     dev = g_tensor.device
+    _check(all(t.device == dev for t, _ in tensors), "All tensors should be on the same device")
     with torch.cuda.device(dev):
-        need = _lib.amr_conv_batch_sum_workspace_bytes(Bn, inner)
+        need = _lib.amr_conv_zero_point_grad_workspace_bytes(Bn, N, L)
         ws = torch.empty(max(need, 16), dtype=torch.uint8, device=dev)
-        rc = _lib.amr_conv_batch_sum_scaled_f32(g_tensor.data_ptr(), z_a.data_ptr(), s_a.data_ptr(), s_w.data_ptr(), out_tensor.data_ptr(), Bn,
-                                                inner, ws.data_ptr(), ws.numel(), _stream_ptr(dev))
-    _raise_for(rc, "conv_batch_sum_scaled")
+        rc = _lib.amr_conv_zero_point_grad_f32(g_tensor.data_ptr(), z_a.data_ptr(), s_a.data_ptr(), s_w.data_ptr(), tapmask.data_ptr(),
+                                               gwr_tensor.data_ptr() if gwr_tensor is not None else None, gz_tensor.data_ptr(), Bn, N, L, T,
+                                               ws.data_ptr(), ws.numel(), _stream_ptr(dev))
+    _raise_for(rc, "conv_zero_point_grad")
 
 
-def conv_weight_grad(gbt_tensor, gwr_tensor, tapmask, inside_tensor, scale_tensor, gw_tensor):
-    """gw[n,c,tap] = inside ? (gbt[tap*C + c, n] + sum over pos of gwr[n, pos] * tapmask[tap, pos]) / scale : 0; gbt float32
-    [taps*C, N], gwr float32 [N, L], gw float32 [N,C,kh,kw]."""
-    for t, name, dt in ((gbt_tensor, "gbt_tensor", torch.float32), (gwr_tensor, "gwr_tensor", torch.float32), (tapmask, "tapmask", torch.float32),
+def conv_zero_point_grad_parts(positions):
+    """Blocks of positions ``conv_zero_point_grad`` folds separately."""
+    return _lib.amr_conv_zero_point_grad_parts(int(positions))
+
+
+def conv_weight_grad(gbt_tensor, gz_tensor, inside_tensor, scale_tensor, gw_tensor):
+    """gw[n,c,tap] = inside ? (gbt[tap*C + c, n] + sum over p of gz[p, n, tap]) / scale : 0; gbt float32 [taps*C, N], gz
+    float32 [parts, N, taps], inside uint8 and gw float32 [N,C,kh,kw]."""
+    for t, name, dt in ((gbt_tensor, "gbt_tensor", torch.float32), (gz_tensor, "gz_tensor", torch.float32),
                         (inside_tensor, "inside_tensor", torch.uint8), (scale_tensor, "scale_tensor", torch.float32), (gw_tensor, "gw_tensor", torch.float32)):
         _check_input(t, dt, name)
     _check(gw_tensor.dim() == 4 and inside_tensor.shape == gw_tensor.shape, "gw must be 4-D and inside of its shape")
     N, C, kh, kw = gw_tensor.shape
-    T, L = kh * kw, tapmask.size(1)
-    _check(tuple(tapmask.shape) == (T, L) and T <= 64, f"tapmask should have {T} rows (at most 64 taps)")
-    _check(tuple(gbt_tensor.shape) == (T * C, N) and gwr_tensor.numel() == N * L and scale_tensor.numel() == 1, "gbt, gwr or scale has the wrong size")
+    T = kh * kw
+    _check(T <= 64 and tuple(gbt_tensor.shape) == (T * C, N) and gz_tensor.dim() == 3 and tuple(gz_tensor.shape[1:]) == (N, T)
+           and gz_tensor.size(0) > 0 and scale_tensor.numel() == 1, "gbt, gz or scale has the wrong size (at most 64 taps)")
     dev = gw_tensor.device
+    _check(all(t.device == dev for t in (gbt_tensor, gz_tensor, inside_tensor, scale_tensor)), "All tensors should be on the same device")
     with torch.cuda.device(dev):
-        rc = _lib.amr_conv_weight_grad_f32(gbt_tensor.data_ptr(), gwr_tensor.data_ptr(), tapmask.data_ptr(), inside_tensor.data_ptr(),
-                                           scale_tensor.data_ptr(), gw_tensor.data_ptr(), N, C, T, L, _stream_ptr(dev))
+        rc = _lib.amr_conv_weight_grad_f32(gbt_tensor.data_ptr(), gz_tensor.data_ptr(), gz_tensor.size(0), inside_tensor.data_ptr(), scale_tensor.data_ptr(),
+                                           gw_tensor.data_ptr(), N, C, T, _stream_ptr(dev))
     _raise_for(rc, "conv_weight_grad")
 
 

@@ -114,10 +114,11 @@ bool gradA_slab_conv_can_finish(int Bn, int H, int W, const float* g_in);
 hipError_t launch_conv_weight_prepare(const float* w, const float* scale, const float* zp_neg, float qmax, const float* tapmask,
                                       uint8_t* Bt, uint8_t* inside, float* w_resp, int N, int C, int T, int L, hipStream_t stream);
 int batch_sum_segments(int B, size_t inner, int n_cu);
-hipError_t launch_batch_sum_scaled(const float* g, const float* za, const float* sa, const float* sw, float* out, float* partial, int B,
-                                   size_t inner, int n_cu, hipStream_t stream);
-hipError_t launch_conv_weight_grad(const float* gBt, const float* g_wr, const float* tapmask, const uint8_t* inside, const float* scale,
-                                   float* gw, int N, int C, int T, int L, hipStream_t stream);
+hipError_t launch_batch_sum_taps(const float* g, const float* za, const float* sa, const float* sw, const float* tapmask, float* g_wr,
+                                 float* gz, float* partial, int B, int N, int L, int T, int n_cu, hipStream_t stream);
+int batch_sum_parts(int L);
+hipError_t launch_conv_weight_grad(const float* gBt, const float* gz, int parts, const uint8_t* inside, const float* scale, float* gw,
+                                   int N, int C, int T, int n_cu, hipStream_t stream);
 hipError_t launch_poison_if_raised(float* gx, size_t total, const uint32_t* gate, hipStream_t stream);
 hipError_t launch_window_sums_3x3(const float* t, float* zt, long B, int H, int W, hipStream_t stream);
 hipError_t launch_dequant_grad_rowsum(const float* g, const float* sa, const float* sw, float* gc, float* t, int M, int N, int L,
@@ -919,6 +920,7 @@ int amr_conv_input_grad_f32(const float* cols, const float* t, const float* z_w,
     if (B < 0 || !conv_geometry(C, H, W, kh, kw, stride, pad, dil, &oh, &ow)) return fail(AMR_EINVAL, "bad convolution geometry");
     if (B == 0) return AMR_OK;
     if ((size_t)B * C * H * W >= ((size_t)1 << 40)) return fail(AMR_EUNSUPPORTED, "more than 2^40 pixels");
+    if ((size_t)C * H * W > 0x7fffffffull) return fail(AMR_EUNSUPPORTED, "more than 2^31 pixels in one image");
     if (!t || !z_w || !inside || !scale || !gx) return fail(AMR_EINVAL, "null pointer argument");
     hipError_t e = amr::launch_conv_input_grad(cols, t, z_w, inside, scale, gx, B, C, H, W, kh, kw, stride, pad, dil, oh, ow,
                                                reinterpret_cast<hipStream_t>(stream));
@@ -1025,32 +1027,38 @@ int amr_conv_weight_prepare_f32(const float* w, const float* scale, const float*
     return e == hipSuccess ? AMR_OK : hip_fail(e, "weight prepare launch");
 }
 
-size_t amr_conv_batch_sum_workspace_bytes(int batch, int64_t inner) {
-    if (batch <= 0 || inner <= 0) return 0;
+size_t amr_conv_zero_point_grad_workspace_bytes(int batch, int N, int positions) {
+    if (batch <= 0 || N <= 0 || positions <= 0) return 0;
     const int n_cu = current_device_cus(nullptr);
-    return (size_t)amr::batch_sum_segments(batch, (size_t)inner, n_cu > 0 ? n_cu : 256) * (size_t)inner * sizeof(float);
+    const size_t inner = (size_t)N * positions;
+    return (size_t)amr::batch_sum_segments(batch, inner, n_cu > 0 ? n_cu : 256) * inner * sizeof(float);
 }
 
-int amr_conv_batch_sum_scaled_f32(const float* g, const float* z_a, const float* s_a, const float* s_w, float* out, int batch,
-                                  int64_t inner, void* workspace, size_t workspace_bytes, void* stream) {
-    if (batch <= 0 || inner <= 0) return fail(AMR_EINVAL, "bad shape");
-    if (!g || !z_a || !s_a || !s_w || !out) return fail(AMR_EINVAL, "null pointer argument");
+int amr_conv_zero_point_grad_parts(int positions) { return positions > 0 ? amr::batch_sum_parts(positions) : 0; }
+
+int amr_conv_zero_point_grad_f32(const float* g, const float* z_a, const float* s_a, const float* s_w, const float* tapmask, float* g_wr,
+                                 float* gz, int batch, int N, int positions, int taps, void* workspace, size_t workspace_bytes,
+                                 void* stream) {
+    if (batch <= 0 || N <= 0 || positions <= 0 || taps <= 0 || taps > 64) return fail(AMR_EINVAL, "bad shape (at most 64 taps)");
+    if (!g || !z_a || !s_a || !s_w || !tapmask || !gz) return fail(AMR_EINVAL, "null pointer argument");
     const int n_cu = current_device_cus(nullptr);
     if (n_cu <= 0) return fail(AMR_EINVAL, "no HIP device available");
-    const size_t need = (size_t)amr::batch_sum_segments(batch, (size_t)inner, n_cu) * (size_t)inner * sizeof(float);
+    const size_t inner = (size_t)N * positions;
+    const size_t need = (size_t)amr::batch_sum_segments(batch, inner, n_cu) * inner * sizeof(float);
     if (!workspace || workspace_bytes < need)
         return fail(AMR_EWORKSPACE, "workspace of %zu bytes is smaller than the %zu required", workspace ? workspace_bytes : (size_t)0, need);
-    if ((uintptr_t)workspace & 15) return fail(AMR_EINVAL, "workspace must be 16-byte aligned");
-    hipError_t e = amr::launch_batch_sum_scaled(g, z_a, s_a, s_w, out, reinterpret_cast<float*>(workspace), batch, (size_t)inner, n_cu,
-                                                reinterpret_cast<hipStream_t>(stream));
-    return e == hipSuccess ? AMR_OK : hip_fail(e, "batch sum launch");
+    if (((uintptr_t)workspace | (uintptr_t)g) & 15) return fail(AMR_EINVAL, "g and workspace must be 16-byte aligned");
+    hipError_t e = amr::launch_batch_sum_taps(g, z_a, s_a, s_w, tapmask, g_wr, gz, reinterpret_cast<float*>(workspace), batch, N, positions,
+                                              taps, n_cu, reinterpret_cast<hipStream_t>(stream));
+    return e == hipSuccess ? AMR_OK : hip_fail(e, "zero-point gradient launch");
 }
 
-int amr_conv_weight_grad_f32(const float* gBt, const float* g_wr, const float* tapmask, const uint8_t* inside, const float* scale, float* gw,
-                             int N, int C, int taps, int positions, void* stream) {
-    if (N <= 0 || C <= 0 || taps <= 0 || taps > 64 || positions <= 0) return fail(AMR_EINVAL, "bad shape (at most 64 taps)");
-    if (!gBt || !g_wr || !tapmask || !inside || !scale || !gw) return fail(AMR_EINVAL, "null pointer argument");
-    hipError_t e = amr::launch_conv_weight_grad(gBt, g_wr, tapmask, inside, scale, gw, N, C, taps, positions, reinterpret_cast<hipStream_t>(stream));
+int amr_conv_weight_grad_f32(const float* gBt, const float* gz, int gz_parts, const uint8_t* inside, const float* scale, float* gw, int N,
+                             int C, int taps, void* stream) {
+    if (N <= 0 || C <= 0 || taps <= 0 || taps > 64 || gz_parts <= 0) return fail(AMR_EINVAL, "bad shape (at most 64 taps)");
+    if (!gBt || !gz || !inside || !scale || !gw) return fail(AMR_EINVAL, "null pointer argument");
+    hipError_t e = amr::launch_conv_weight_grad(gBt, gz, gz_parts, inside, scale, gw, N, C, taps, current_device_cus(nullptr),
+                                                reinterpret_cast<hipStream_t>(stream));
     return e == hipSuccess ? AMR_OK : hip_fail(e, "weight gradient launch");
 }
 

@@ -167,8 +167,18 @@ __global__ __launch_bounds__(256) void conv_input_grad_kernel(const float* __res
                                                               int H, int W, int kh_rt, int kw_rt, int stride_rt, int pad, int dil,
                                                               int oh, int ow, size_t total, const uint32_t* __restrict__ gate,
                                                               int gate_mode) {
-    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
-    if (idx >= total) return;
+    // (32-bit index arithmetic inside an image; the images of the batch on blockIdx.y, strided when there are more than the grid holds)
+    const uint32_t per_image = (uint32_t)C * (uint32_t)H * (uint32_t)W;
+    const uint32_t e = blockIdx.x * 256u + threadIdx.x;
+    if (e >= per_image) return;
+    const int kh = KH ? KH : kh_rt, kw = KW ? KW : kw_rt, stride = STRIDE ? STRIDE : stride_rt;
+    const int xx = (int)(e % (uint32_t)W);
+    const uint32_t r = e / (uint32_t)W;
+    const int yy = (int)(r % (uint32_t)H);
+    const int c = (int)(r / (uint32_t)H);
+    const size_t L = (size_t)oh * ow;
+    for (size_t b = blockIdx.y; b * per_image < total; b += gridDim.y) {
+    const size_t idx = b * per_image + e;
     // gate_mode 1: the pass behind a kernel that left the tap sums in gx -- when *gate says that kernel could not do its work,
     // this pass leaves gx alone (a recomputation is queued behind, gate_mode 2) or, gate_mode 3, marks every element NaN;
     // gate_mode 2: runs only when *gate is set.
@@ -176,16 +186,8 @@ __global__ __launch_bounds__(256) void conv_input_grad_kernel(const float* __res
         const bool raised = *gate != 0u;
         if (gate_mode == 2 && !raised) return;
         if (gate_mode == 1 && raised) return;
-        if (gate_mode == 3 && raised) { gx[idx] = __builtin_nanf(""); return; }
+        if (gate_mode == 3 && raised) { gx[idx] = __builtin_nanf(""); continue; }
     }
-    const int kh = KH ? KH : kh_rt, kw = KW ? KW : kw_rt, stride = STRIDE ? STRIDE : stride_rt;
-    const int xx = (int)(idx % W);
-    size_t r = idx / W;
-    const int yy = (int)(r % H);
-    r /= H;                                   // = b * C + c
-    const int c = (int)(r % C);
-    const size_t b = r / C;
-    const size_t L = (size_t)oh * ow;
     const float* base = cols ? cols + (b * (size_t)(kh * kw) * C + c) * L : nullptr;
     const float* tb = t + b * L;
     float acc = 0.f, tsum = 0.f;
@@ -233,6 +235,65 @@ __global__ __launch_bounds__(256) void conv_input_grad_kernel(const float* __res
     if (!cols) acc = gx[idx];
     const float total_g = acc + *zw_p * tsum;
     gx[idx] = inside[idx] ? total_g / *scale_p : 0.f;
+    }
+}
+
+// Stride 2 with an even image (3x3 / padding 1 or 1x1 / padding 0, no dilation): a thread owns one output position of one
+// channel and the 2 x 2 input pixels it maps to.  Every tap's column is loaded exactly once (nine loads for the four
+// pixels: the even/even pixel has one tap, the mixed ones two, the odd/odd one four), the pixels leave as two 8-byte
+// stores.  Taps are added in ascending order like the general kernel.
+template <int K>
+__global__ __launch_bounds__(256) void conv_input_grad_s2_kernel(const float* __restrict__ cols, const float* __restrict__ t,
+                                                                 const float* __restrict__ zw_p, const uint8_t* __restrict__ inside,
+                                                                 const float* __restrict__ scale_p, float* __restrict__ gx, int C,
+                                                                 int oh, int ow, long B) {
+    typedef float f32x2 __attribute__((ext_vector_type(2)));
+    const uint32_t per_image = (uint32_t)C * (uint32_t)oh * (uint32_t)ow;
+    const uint32_t e = blockIdx.x * 256u + threadIdx.x;
+    if (e >= per_image) return;
+    const int ox = (int)(e % (uint32_t)ow);
+    const uint32_t r = e / (uint32_t)ow;
+    const int oy = (int)(r % (uint32_t)oh);
+    const int c = (int)(r / (uint32_t)oh);
+    const size_t L = (size_t)oh * ow, CL = (size_t)C * L;
+    const int W = 2 * ow;
+    const float zw = *zw_p, scale = *scale_p;
+    const bool right = ox + 1 < ow, down = oy + 1 < oh;
+    const size_t p00 = (size_t)oy * ow + ox;
+    const size_t p01 = right ? p00 + 1 : p00, p10 = down ? p00 + ow : p00, p11 = p10 + (right ? 1 : 0);
+    for (long b = blockIdx.y; b < B; b += gridDim.y) {
+        const float* base = cols + ((size_t)b * (K * K) * C + c) * L;
+        const float* tb = t + (size_t)b * L;
+        float a00, a01, a10, a11, s00, s01, s10, s11;
+        if constexpr (K == 1) {
+            a00 = base[p00];
+            s00 = tb[p00];
+            a01 = a10 = a11 = s01 = s10 = s11 = 0.f;
+        } else {
+            // tap (i, j) reaches pixel (2*oy' + i - 1, 2*ox' + j - 1) from output position (oy', ox')
+            const float v0 = base[0 * CL + p11], v1 = base[1 * CL + p10], v2 = base[2 * CL + p10];
+            const float v3 = base[3 * CL + p01], v4 = base[4 * CL + p00], v5 = base[5 * CL + p00];
+            const float v6 = base[6 * CL + p01], v7 = base[7 * CL + p00], v8 = base[8 * CL + p00];
+            const float t00 = tb[p00], t01 = right ? tb[p01] : 0.f, t10 = down ? tb[p10] : 0.f, t11 = right && down ? tb[p11] : 0.f;
+            a00 = v4;
+            s00 = t00;
+            a01 = (right ? v3 : 0.f) + v5;                      // pixel (2oy, 2ox+1): taps (1,0) from ox+1 and (1,2) from ox
+            s01 = t01 + t00;
+            a10 = (down ? v1 : 0.f) + v7;                       // pixel (2oy+1, 2ox): taps (0,1) from oy+1 and (2,1) from oy
+            s10 = t10 + t00;
+            a11 = (((right && down ? v0 : 0.f) + (down ? v2 : 0.f)) + (right ? v6 : 0.f)) + v8;
+            s11 = ((t11 + t10) + t01) + t00;
+        }
+        const size_t o = (((size_t)b * C + c) * (2 * oh) + 2 * oy) * W + 2 * ox;
+        const uint16_t in0 = *reinterpret_cast<const uint16_t*>(inside + o), in1 = *reinterpret_cast<const uint16_t*>(inside + o + W);
+        f32x2 r0, r1;
+        r0.x = (in0 & 0xff) ? (a00 + zw * s00) / scale : 0.f;
+        r0.y = (in0 >> 8) ? (a01 + zw * s01) / scale : 0.f;
+        r1.x = (in1 & 0xff) ? (a10 + zw * s10) / scale : 0.f;
+        r1.y = (in1 >> 8) ? (a11 + zw * s11) / scale : 0.f;
+        *reinterpret_cast<f32x2*>(gx + o) = r0;
+        *reinterpret_cast<f32x2*>(gx + o + W) = r1;
+    }
 }
 
 hipError_t launch_conv_input_grad(const float* cols, const float* t, const float* zw, const uint8_t* inside, const float* scale,
@@ -240,7 +301,16 @@ hipError_t launch_conv_input_grad(const float* cols, const float* t, const float
                                   hipStream_t stream, const uint32_t* gate = nullptr, int gate_mode = 0) {
     const size_t total = (size_t)B * C * H * W;
     if (total == 0) return hipSuccess;
-    const dim3 grid((unsigned)((total + 255) / 256));
+    const unsigned rows = (unsigned)(B < 32768 ? B : 32768);
+    if ((size_t)C * H * W > 0x7fffffffull) return hipErrorInvalidValue;      // (32-bit index inside an image)
+    if (cols && gate_mode == 0 && stride == 2 && dil == 1 && H == 2 * oh && W == 2 * ow && kh == kw &&
+        ((kh == 3 && pad == 1) || (kh == 1 && pad == 0)) && ((uintptr_t)gx & 7) == 0 && ((uintptr_t)inside & 1) == 0) {
+        const dim3 g2((unsigned)(((size_t)C * oh * ow + 255) / 256), rows);
+        if (kh == 3) hipLaunchKernelGGL((conv_input_grad_s2_kernel<3>), g2, dim3(256), 0, stream, cols, t, zw, inside, scale, gx, C, oh, ow, B);
+        else hipLaunchKernelGGL((conv_input_grad_s2_kernel<1>), g2, dim3(256), 0, stream, cols, t, zw, inside, scale, gx, C, oh, ow, B);
+        return hipGetLastError();
+    }
+    const dim3 grid((unsigned)(((size_t)C * H * W + 255) / 256), rows);
 #define AMR_CIG(KH, KW, S)                                                                                                        \
     hipLaunchKernelGGL((conv_input_grad_kernel<KH, KW, S>), grid, dim3(256), 0, stream, cols, t, zw, inside, scale, gx, C, H, W, kh, kw, \
                        stride, pad, dil, oh, ow, total, gate, gate_mode)
@@ -325,9 +395,13 @@ hipError_t launch_conv_weight_prepare(const float* w, const float* scale, const 
     return hipGetLastError();
 }
 
-// out[j] = (*z_a * (*s_a * *s_w)) * sum over b of g[b][j], j < inner: the gradient of the zero-point term conv(Za, W) with
-// respect to w_resp, summed over the batch.  Two launches: S segments of the batch into partial sums (a thread owns four
-// neighbouring j and walks its segment with four loads in flight), then the segments in ascending order.  Fixed order.
+// Gradient of the zero-point term Za * w_resp, summed over the batch and folded onto the taps:
+//   g_wr[n][pos] = (*z_a * (*s_a * *s_w)) * sum over b of g[b][n][pos]
+//   gz[p][n][tap] = sum over the positions pos of block p (256 positions each) of g_wr[n][pos] * tapmask[tap][pos]
+// (the consumer, the weight-gradient kernel below, adds the blocks in ascending order).  Two launches, fixed summation order.  First S segments of the batch into partial sums (a thread owns four neighbouring
+// elements and walks its segment with four loads in flight); then one workgroup per output channel n and block of positions adds the
+// segments in ascending order (threads side by side along the positions, segment lanes beside them when the block is
+// short), scales, and reduces against the tap masks, one tap per wave at a time.
 __global__ __launch_bounds__(256) void batch_sum_partial_kernel(const float* __restrict__ g, float* __restrict__ partial, int B, size_t inner,
                                                                 int seg_len) {
     const size_t j4 = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4;
@@ -355,27 +429,68 @@ __global__ __launch_bounds__(256) void batch_sum_partial_kernel(const float* __r
     }
 }
 
-__global__ __launch_bounds__(256) void batch_sum_finish_kernel(const float* __restrict__ partial, const float* __restrict__ za_p,
-                                                               const float* __restrict__ sa_p, const float* __restrict__ sw_p,
-                                                               float* __restrict__ out, size_t inner, int segs) {
-    const size_t j = (size_t)blockIdx.x * 256 + threadIdx.x;
-    if (j >= inner) return;
-    float acc = partial[j];
-    for (int s = 1; s < segs; ++s) acc += partial[(size_t)s * inner + j];
-    out[j] = __fmul_rn(__fmul_rn(*za_p, __fmul_rn(*sa_p, *sw_p)), acc);
+constexpr int kBsChunk = 256;       // positions of one channel per workgroup of the folding kernel
+__global__ __launch_bounds__(256) void batch_sum_taps_kernel(const float* __restrict__ partial, const float* __restrict__ za_p,
+                                                             const float* __restrict__ sa_p, const float* __restrict__ sw_p,
+                                                             const float* __restrict__ tapmask, float* __restrict__ g_wr,
+                                                             float* __restrict__ gz_parts, size_t inner, int N, int L, int T, int segs) {
+    __shared__ float part[256];
+    __shared__ float v[kBsChunk];
+    const int n = blockIdx.x, lane = threadIdx.x & 63, wave = uniform(threadIdx.x >> 6);
+    const int p0 = blockIdx.y * kBsChunk;
+    const int cn = min(kBsChunk, L - p0);
+    const float scale = __fmul_rn(*za_p, __fmul_rn(*sa_p, *sw_p));
+    // P threads along the positions (a power of two, 16..256), SP = 256 / P lanes of segments beside them
+    int P = 16;
+    while (P < cn) P <<= 1;
+    const int SP = 256 / P;
+    const int pp = threadIdx.x & (P - 1), sp = threadIdx.x / P;
+    {
+        float acc = 0.f;
+        if (pp < cn) {
+            const float* src = partial + (size_t)n * L + p0 + pp;
+            int sgm = sp;
+            for (; sgm + 3 * SP < segs; sgm += 4 * SP) {
+                const float a0 = src[(size_t)sgm * inner], a1 = src[(size_t)(sgm + SP) * inner];
+                const float a2 = src[(size_t)(sgm + 2 * SP) * inner], a3 = src[(size_t)(sgm + 3 * SP) * inner];
+                acc = (((acc + a0) + a1) + a2) + a3;
+            }
+            for (; sgm < segs; sgm += SP) acc += src[(size_t)sgm * inner];
+        }
+        part[threadIdx.x] = acc;                                    // = part[sp * P + pp]
+    }
+    __syncthreads();
+    if (threadIdx.x < cn) {
+        float acc = part[threadIdx.x];
+        for (int q = 1; q < SP; ++q) acc += part[q * P + threadIdx.x];
+        acc = __fmul_rn(scale, acc);
+        v[threadIdx.x] = acc;
+        if (g_wr) g_wr[(size_t)n * L + p0 + threadIdx.x] = acc;
+    }
+    __syncthreads();
+    for (int tap = wave; tap < T; tap += 4) {
+        float acc = 0.f;
+        for (int pos = lane; pos < cn; pos += 64) acc += v[pos] * tapmask[(size_t)tap * L + p0 + pos];
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) acc += __shfl_xor(acc, o);
+        if (lane == 0) gz_parts[((size_t)blockIdx.y * N + n) * T + tap] = acc;
+    }
 }
 
+int batch_sum_parts(int L) { return (L + kBsChunk - 1) / kBsChunk; }
+
 int batch_sum_segments(int B, size_t inner, int n_cu) {
-    // enough workgroups to fill the device, at least 8 images per segment
+    // enough workgroups to fill the device, at least 8 images per segment, at most 32 segments
     const size_t wg_per_seg = (inner / 4 + 255) / 256;
     int segs = (int)((4 * (size_t)n_cu + wg_per_seg - 1) / (wg_per_seg ? wg_per_seg : 1));
     if (segs > B / 8) segs = B / 8;
-    if (segs > 64) segs = 64;
+    if (segs > 32) segs = 32;
     return segs < 1 ? 1 : segs;
 }
 
-hipError_t launch_batch_sum_scaled(const float* g, const float* za, const float* sa, const float* sw, float* out, float* partial, int B,
-                                   size_t inner, int n_cu, hipStream_t stream) {
+hipError_t launch_batch_sum_taps(const float* g, const float* za, const float* sa, const float* sw, const float* tapmask, float* g_wr,
+                                 float* gz, float* partial, int B, int N, int L, int T, int n_cu, hipStream_t stream) {
+    const size_t inner = (size_t)N * L;
     const int segs = batch_sum_segments(B, inner, n_cu);
     const int seg_len = (B + segs - 1) / segs;
     const int used = (B + seg_len - 1) / seg_len;
@@ -383,43 +498,60 @@ hipError_t launch_batch_sum_scaled(const float* g, const float* za, const float*
                        seg_len);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(batch_sum_finish_kernel, dim3((unsigned)((inner + 255) / 256)), dim3(256), 0, stream, partial, za, sa, sw, out, inner,
-                       used);
+    hipLaunchKernelGGL(batch_sum_taps_kernel, dim3(N, batch_sum_parts(L)), dim3(256), 0, stream, partial, za, sa, sw, tapmask, g_wr, gz, inner,
+                       N, L, T, used);
     return hipGetLastError();
 }
 
 // Weight gradient of the layer, finished in one launch: the LUT gradient gBt [T*C][N] (tap-major rows, what gradB wrote), the
-// zero-point term -- g_wr [N][L] spread over the taps a position has, gz[tap] = sum over pos of g_wr[n][pos] * tapmask[tap][pos]
-// (fixed order) -- and the quantiser's straight-through backward:  gw[n][c][tap] = inside ? (gBt + gz[tap]) / *scale : 0.
-__global__ __launch_bounds__(256) void conv_weight_grad_kernel(const float* __restrict__ gBt, const float* __restrict__ g_wr,
-                                                               const float* __restrict__ tapmask, const uint8_t* __restrict__ inside,
-                                                               const float* __restrict__ scale, float* __restrict__ gw, int N, int C, int T,
-                                                               int L) {
-    __shared__ float red[4][kWpMaxTaps];
-    __shared__ float gz[kWpMaxTaps];
-    const int n = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    for (int tap = 0; tap < T; ++tap) {
-        float acc = 0.f;
-        for (int pos = threadIdx.x; pos < L; pos += 256) acc += g_wr[(size_t)n * L + pos] * tapmask[(size_t)tap * L + pos];
-#pragma unroll
-        for (int o = 32; o > 0; o >>= 1) acc += __shfl_xor(acc, o);
-        if (lane == 0) red[wave][tap] = acc;
+// zero-point term gz [parts][N][T] (blocks of positions, added here in ascending order) and the quantiser's straight-through
+// backward:   gw[n][c][tap] = inside[n][c][tap] ? (gBt[(tap*C + c)*N + n] + sum over p of gz[p][n][tap]) / *scale : 0.
+// A workgroup transposes a tile of all T taps x cb channels x 16 output channels through LDS: reads run along n (64 B per
+// row of gBt), writes along (c, tap), T*cb adjacent floats per output channel.  cb shrinks until the grid fills the device.
+constexpr int kWgRows = 128, kWgCols = 16;
+__global__ __launch_bounds__(256) void conv_weight_grad_kernel(const float* __restrict__ gBt, const float* __restrict__ gz, int parts,
+                                                               const uint8_t* __restrict__ inside, const float* __restrict__ scale,
+                                                               float* __restrict__ gw, int N, int C, int T, int cb) {
+    __shared__ float tile[kWgRows][kWgCols + 1];
+    __shared__ float gzs[kWgCols][kWpMaxTaps];
+    const int lane = threadIdx.x & 63, wave = uniform(threadIdx.x >> 6);
+    const int n0 = blockIdx.x * kWgCols, c0 = blockIdx.y * cb;
+    const int cn = min(cb, C - c0), rows = T * cn;
+    const int n_here = min(kWgCols, N - n0);
+    {
+        const int nl = threadIdx.x & (kWgCols - 1);
+        for (int rr = threadIdx.x / kWgCols; rr < rows; rr += 256 / kWgCols) {
+            const int tap = rr / cn, cc = rr - tap * cn;
+            tile[rr][nl] = nl < n_here ? gBt[((size_t)tap * C + c0 + cc) * N + n0 + nl] : 0.f;
+        }
+        for (int e = threadIdx.x; e < n_here * T; e += 256) {
+            const int q = e / T, tap = e - q * T;
+            float acc = gz[(size_t)(n0 + q) * T + tap];
+            for (int p = 1; p < parts; ++p) acc += gz[((size_t)p * N + n0 + q) * T + tap];
+            gzs[q][tap] = acc;
+        }
     }
     __syncthreads();
-    if (threadIdx.x < T) gz[threadIdx.x] = (red[0][threadIdx.x] + red[1][threadIdx.x]) + (red[2][threadIdx.x] + red[3][threadIdx.x]);
-    __syncthreads();
     const float s = *scale;
-    const int per_n = C * T;
-    for (int idx = threadIdx.x; idx < per_n; idx += 256) {
-        const int c = idx / T, tap = idx - c * T;
-        const float v = gBt[((size_t)tap * C + c) * N + n] + gz[tap];
-        gw[(size_t)n * per_n + idx] = inside[(size_t)n * per_n + idx] ? v / s : 0.f;
+    for (int nl = wave; nl < n_here; nl += 4) {
+        const size_t row = ((size_t)(n0 + nl) * C + c0) * T;
+        for (int j = lane; j < rows; j += 64) {
+            const int cc = j / T, tap = j - cc * T;
+            const float val = tile[tap * cn + cc][nl] + gzs[nl][tap];
+            gw[row + j] = inside[row + j] ? val / s : 0.f;
+        }
     }
 }
 
-hipError_t launch_conv_weight_grad(const float* gBt, const float* g_wr, const float* tapmask, const uint8_t* inside, const float* scale,
-                                   float* gw, int N, int C, int T, int L, hipStream_t stream) {
-    hipLaunchKernelGGL(conv_weight_grad_kernel, dim3(N), dim3(256), 0, stream, gBt, g_wr, tapmask, inside, scale, gw, N, C, T, L);
+hipError_t launch_conv_weight_grad(const float* gBt, const float* gz, int parts, const uint8_t* inside, const float* scale, float* gw,
+                                   int N, int C, int T, int n_cu, hipStream_t stream) {
+    const int n_tiles = (N + kWgCols - 1) / kWgCols;
+    int cb = T >= kWgRows ? 1 : kWgRows / T;
+    const long fill = (long)C * n_tiles / (n_cu > 0 ? n_cu : 256);           // channels per workgroup that still give one workgroup per CU
+    if (cb > fill) cb = (int)(fill < 1 ? 1 : fill);
+    if (cb > C) cb = C;
+    hipLaunchKernelGGL(conv_weight_grad_kernel, dim3(n_tiles, (C + cb - 1) / cb), dim3(256), 0, stream, gBt, gz, parts, inside, scale, gw, N,
+                       C, T, cb);
     return hipGetLastError();
 }
 

@@ -336,18 +336,24 @@ int amr_conv_input_grad_f32(const float *cols, const float *t, const float *z_w,
  *             the rounded value lay in [0, qmax]; w_resp[n][pos] = sum over taps of (sum over c of the codes) * tapmask[tap][pos]
  *             -- the response of the weight codes to an all-ones image, tapmask[tap][pos] = 1 where tap `tap` of output position
  *             `pos` lies inside the image.  w [N][C][taps] float32; scale, zp_neg device scalars; at most 64 taps.
- *   batch sum: out[j] = (*z_a * (*s_a * *s_w)) * sum over b of g[b][j] (fixed order; workspace of
- *             amr_conv_batch_sum_workspace_bytes bytes): with g the output gradient [B][N*L] this is the gradient with respect to w_resp.
- *   grad:     gw[n][c][tap] = inside ? (gBt[(tap*C + c)*N + n] + sum over pos of g_wr[n][pos] * tapmask[tap][pos]) / *scale : 0,
- *             gBt the gB of amr_lut_gemm_backward_ex for the tap-major operands.
+ *   zero-point gradient: g_wr[n][pos] = (*z_a * (*s_a * *s_w)) * sum over b of g[b][n][pos] (g the output gradient [B][N][L],
+ *             16-byte aligned; g_wr may be null): the gradient of the term Za * w_resp with respect to w_resp; and the same folded
+ *             onto the taps, gz[p][n][tap] = sum over the positions pos of block p of g_wr[n][pos] * tapmask[tap][pos], in
+ *             P = amr_conv_zero_point_grad_parts(positions) blocks of positions (gz holds P*N*taps floats; the weight-gradient
+ *             call adds the blocks).  Fixed summation order; workspace of amr_conv_zero_point_grad_workspace_bytes bytes, 16-byte
+ *             aligned.
+ *   grad:     gw[n][c][tap] = inside ? (gBt[(tap*C + c)*N + n] + sum over p < gz_parts of gz[p][n][tap]) / *scale : 0, gBt the
+ *             gB of amr_lut_gemm_backward_ex for the tap-major operands.
  */
 int amr_conv_weight_prepare_f32(const float *w, const float *scale, const float *zp_neg, float qmax, const float *tapmask,
                                 uint8_t *Bt, uint8_t *inside, float *w_resp, int N, int C, int taps, int positions, void *stream);
-size_t amr_conv_batch_sum_workspace_bytes(int batch, int64_t inner);
-int amr_conv_batch_sum_scaled_f32(const float *g, const float *z_a, const float *s_a, const float *s_w, float *out, int batch,
-                                  int64_t inner, void *workspace, size_t workspace_bytes, void *stream);
-int amr_conv_weight_grad_f32(const float *gBt, const float *g_wr, const float *tapmask, const uint8_t *inside, const float *scale,
-                             float *gw, int N, int C, int taps, int positions, void *stream);
+size_t amr_conv_zero_point_grad_workspace_bytes(int batch, int N, int positions);
+int amr_conv_zero_point_grad_parts(int positions);
+int amr_conv_zero_point_grad_f32(const float *g, const float *z_a, const float *s_a, const float *s_w, const float *tapmask,
+                                 float *g_wr, float *gz, int batch, int N, int positions, int taps, void *workspace,
+                                 size_t workspace_bytes, void *stream);
+int amr_conv_weight_grad_f32(const float *gBt, const float *gz, int gz_parts, const uint8_t *inside, const float *scale, float *gw,
+                             int N, int C, int taps, void *stream);
 
 /*
  * Input gradient of a quantised 3x3 LUT convolution of stride 1 and padding 1 WITHOUT the [M][9C] gradient matrix: gradA of

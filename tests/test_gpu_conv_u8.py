@@ -75,7 +75,10 @@ def test_tap_major_im2col_against_oracle(ops, oracle, shape, k, stride, padding,
 
 @pytest.mark.parametrize("shape,k,stride,padding,dilation", [
     ((3, 5, 10, 10), 3, 1, 1, 1), ((2, 4, 9, 7), 3, 2, 1, 1), ((2, 8, 12, 12), 1, 2, 0, 1), ((1, 3, 16, 16), 7, 2, 3, 1),
-    ((2, 6, 11, 11), 3, 1, 2, 2), ((2, 64, 8, 8), 3, 1, 1, 1), ((4, 16, 32, 32), 3, 1, 1, 1), ((2, 32, 6, 6), 1, 1, 0, 1)])
+    ((2, 6, 11, 11), 3, 1, 2, 2), ((2, 64, 8, 8), 3, 1, 1, 1), ((4, 16, 32, 32), 3, 1, 1, 1), ((2, 32, 6, 6), 1, 1, 0, 1),
+    # stride 2 on even images: the kernel that owns the 2 x 2 pixels of an output position
+    ((3, 5, 10, 6), 3, 2, 1, 1), ((2, 64, 32, 32), 3, 2, 1, 1), ((5, 7, 2, 2), 3, 2, 1, 1), ((3, 64, 32, 32), 1, 2, 0, 1),
+    ((2, 3, 2, 4), 1, 2, 0, 1), ((2, 4, 8, 8), 3, 2, 1, 2)])
 def test_fused_input_gradient_equals_fold_plus_torch_operators(ops, shape, k, stride, padding, dilation):
     """gx = inside ? (fold(cols) + z_w * fold of the row sums spread over the taps) / scale : 0 against torch's fold in
     float64; with cols = None the kernel finishes a tensor that already holds fold(cols)."""
@@ -206,18 +209,24 @@ def test_weight_side_in_one_launch_each_way(ops, n, c, k, hw, stride, padding, d
     assert 0 < int(inside.sum()) < inside.numel()
     want_resp = F.conv2d(torch.ones(1, c, *hw, device="cuda", dtype=torch.float64), codes.double(), stride=stride, padding=padding, dilation=dilation)
     assert torch.equal(wresp.double().view(-1), want_resp.view(-1))
-    # batch sum with the three scalars
+    # gradient of the zero-point term: batch sum with the three scalars, folded onto the taps
     bn = 37
     gout = torch.randn(bn, n, Lp, device="cuda", generator=g)
     z_a, s_a, s_w = (torch.tensor([v], device="cuda") for v in (-3.0, 0.013, 0.0041))
     gwr = torch.empty(n, Lp, device="cuda")
-    approx_ops.conv_batch_sum_scaled(gout, z_a, s_a, s_w, gwr)
+    gz = torch.empty(approx_ops.conv_zero_point_grad_parts(Lp), n, T, device="cuda")
+    approx_ops.conv_zero_point_grad(gout, z_a, s_a, s_w, tapmask, gz, gwr)
     want = (z_a * (s_a * s_w)).double() * gout.double().sum(dim=0)
     torch.testing.assert_close(gwr.double(), want, rtol=1e-5, atol=1e-6 * float(want.abs().max()))
+    want_z = want @ tapmask.double().t()
+    torch.testing.assert_close(gz.double().sum(dim=0), want_z, rtol=1e-5, atol=1e-6 * float(want.abs().sum(dim=1).max()))
+    gz2 = torch.empty_like(gz)
+    approx_ops.conv_zero_point_grad(gout, z_a, s_a, s_w, tapmask, gz2)          # (without the optional output)
+    assert torch.equal(gz, gz2)
     # weight gradient: autograd through codes -> (operand gradient, response) in float64
     gbt = torch.randn(T * c, n, device="cuda", generator=g)
     gw = torch.empty_like(w)
-    approx_ops.conv_weight_grad(gbt, gwr, tapmask, inside, scale, gw)
+    approx_ops.conv_weight_grad(gbt, gz, inside, scale, gw)
     wd = w.double().requires_grad_()
     qd = wd / scale.double() - zpn.double()
     cd = torch.clamp(qd - qd.detach() + torch.round(q).double(), 0, qmax)
@@ -227,19 +236,25 @@ def test_weight_side_in_one_launch_each_way(ops, n, c, k, hw, stride, padding, d
     torch.testing.assert_close(gw.double(), wd.grad, rtol=1e-5, atol=2e-6 * float(wd.grad.abs().max()))
 
 
-def test_batch_sum_of_a_large_gradient_and_ragged_sizes(ops):
+def test_zero_point_gradient_of_a_large_batch_and_ragged_sizes(ops):
     import approx_ops
     g = torch.Generator(device="cuda").manual_seed(5)
     one = lambda v: torch.tensor([v], device="cuda")
-    for bn, inner in ((512, 64 * 1024), (3, 10), (130, 4098), (9, 7), (64, 512 * 16)):
-        x = torch.randn(bn, inner, device="cuda", generator=g)
-        out = torch.empty(inner, device="cuda")
-        approx_ops.conv_batch_sum_scaled(x, one(2.0), one(0.5), one(3.0), out)
+    for bn, n, L, T in ((512, 64, 1024, 9), (3, 2, 5, 1), (130, 6, 683, 4), (9, 1, 7, 64), (64, 512, 16, 9), (40, 3, 2500, 49)):
+        print("zero-point gradient", bn, n, L, T, flush=True)
+        x = torch.randn(bn, n, L, device="cuda", generator=g)
+        mask = (torch.rand(T, L, device="cuda", generator=g) < 0.8).float()
+        gwr = torch.empty(n, L, device="cuda")
+        parts = approx_ops.conv_zero_point_grad_parts(L)
+        assert parts == (L + 255) // 256
+        gz = torch.empty(parts, n, T, device="cuda")
+        approx_ops.conv_zero_point_grad(x, one(2.0), one(0.5), one(3.0), mask, gz, gwr)
         want = 3.0 * x.double().sum(dim=0)
-        torch.testing.assert_close(out.double(), want, rtol=1e-5, atol=1e-6 * float(want.abs().max()))
-        again = torch.empty(inner, device="cuda")
-        approx_ops.conv_batch_sum_scaled(x, one(2.0), one(0.5), one(3.0), again)
-        assert torch.equal(out, again)                      # fixed summation order
+        torch.testing.assert_close(gwr.double(), want, rtol=1e-5, atol=1e-6 * float(want.abs().max()))
+        torch.testing.assert_close(gz.double().sum(dim=0), want @ mask.double().t(), rtol=1e-5, atol=1e-6 * float(want.abs().sum(dim=1).max()))
+        again = torch.empty_like(gz)
+        approx_ops.conv_zero_point_grad(x, one(2.0), one(0.5), one(3.0), mask, again)
+        assert torch.equal(gz, again)                       # fixed summation order
 
 
 def test_uint8_layer_path_first_layer_needs_no_input_gradient(ops):

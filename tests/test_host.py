@@ -209,17 +209,20 @@ def test_layer_level_entry_points_check_arguments_without_touching_a_device():
     assert lib.amr_conv_weight_prepare_f32(*([None] * 3), 127.0, *([None] * 4), 8, 4, 81, 16, None) == -1     # more than 64 taps
     assert lib.amr_conv_weight_prepare_f32(*([None] * 3), 300.0, *([None] * 4), 8, 4, 9, 16, None) == -1      # codes must fit a byte
     assert lib.amr_conv_weight_prepare_f32(*([None] * 3), 127.0, *([None] * 4), 8, 4, 9, 16, None) == -1      # null pointers
-    lib.amr_conv_batch_sum_workspace_bytes.argtypes = [i, i64]
-    lib.amr_conv_batch_sum_workspace_bytes.restype = sz
-    assert lib.amr_conv_batch_sum_workspace_bytes(0, 100) == 0
-    assert lib.amr_conv_batch_sum_workspace_bytes(4, 100) == 100 * 4                                         # few images: one segment
-    assert lib.amr_conv_batch_sum_workspace_bytes(512, 65536) % (65536 * 4) == 0
-    lib.amr_conv_batch_sum_scaled_f32.argtypes = [vp] * 5 + [i, i64, vp, sz, vp]
-    assert lib.amr_conv_batch_sum_scaled_f32(*([None] * 5), 0, 10, None, 0, None) == -1
-    assert lib.amr_conv_batch_sum_scaled_f32(*([None] * 5), 4, 10, None, 0, None) == -1                       # null pointers
-    lib.amr_conv_weight_grad_f32.argtypes = [vp] * 6 + [i, i, i, i, vp]
-    assert lib.amr_conv_weight_grad_f32(*([None] * 6), 8, 4, 9, 0, None) == -1
-    assert lib.amr_conv_weight_grad_f32(*([None] * 6), 8, 4, 9, 16, None) == -1                               # null pointers
+    lib.amr_conv_zero_point_grad_workspace_bytes.argtypes = [i, i, i]
+    lib.amr_conv_zero_point_grad_workspace_bytes.restype = sz
+    assert lib.amr_conv_zero_point_grad_workspace_bytes(0, 10, 10) == 0
+    assert lib.amr_conv_zero_point_grad_workspace_bytes(4, 10, 10) == 100 * 4                                 # few images: one segment
+    assert lib.amr_conv_zero_point_grad_workspace_bytes(512, 64, 1024) % (65536 * 4) == 0
+    lib.amr_conv_zero_point_grad_f32.argtypes = [vp] * 7 + [i, i, i, i, vp, sz, vp]
+    assert lib.amr_conv_zero_point_grad_f32(*([None] * 7), 0, 4, 10, 9, None, 0, None) == -1
+    assert lib.amr_conv_zero_point_grad_f32(*([None] * 7), 4, 4, 10, 65, None, 0, None) == -1                 # more than 64 taps
+    assert lib.amr_conv_zero_point_grad_f32(*([None] * 7), 4, 4, 10, 9, None, 0, None) == -1                  # null pointers
+    assert lib.amr_conv_zero_point_grad_parts(1024) == 4 and lib.amr_conv_zero_point_grad_parts(16) == 1 and lib.amr_conv_zero_point_grad_parts(0) == 0
+    lib.amr_conv_weight_grad_f32.argtypes = [vp, vp, i, vp, vp, vp, i, i, i, vp]
+    assert lib.amr_conv_weight_grad_f32(None, None, 1, None, None, None, 8, 0, 9, None) == -1
+    assert lib.amr_conv_weight_grad_f32(None, None, 0, None, None, None, 8, 4, 9, None) == -1                 # no block of positions
+    assert lib.amr_conv_weight_grad_f32(None, None, 1, None, None, None, 8, 4, 9, None) == -1                 # null pointers
     # the decision on a gradient table in host memory
     lib.amr_grad_table_fits_halves.argtypes = [vp, i64]
     small = np.zeros(17408, np.int16); small[:100] = 2048; small[200:300] = -2048
