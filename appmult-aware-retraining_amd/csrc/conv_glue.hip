@@ -109,47 +109,69 @@ hipError_t launch_quantize_nhwc(const float* x, const float* scale, const float*
 // One thread per 16 bytes of A (C % 16 == 0) or per byte: row m = (b, oy, ox), run `tap`, bytes c..c+15 = the codes of input
 // pixel (oy*stride - pad + i*dil, ox*stride - pad + j*dil), zeros outside the image (code 0, as F.pad(value=0) gives the
 // reference, self_ops/ops_py/approx_ops.py:556).  Consecutive threads write consecutive pieces of A.
+// blockIdx.y = a slab of `slab_rows` rows holding fewer than 2^23 pieces, so that every division of the index arithmetic
+// runs on a small number through a reciprocal (the 64-bit divisions of a flat index cost more than the copy).
 template <int VEC>
 __global__ __launch_bounds__(256) void im2col_nhwc_kernel(const uint8_t* __restrict__ codes, uint8_t* __restrict__ A, int C, int H,
                                                           int W, int kh, int kw, int stride, int pad, int dil, int oh, int ow,
-                                                          size_t total) {
-    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
-    if (idx >= total) return;
+                                                          long M, int slab_rows) {
     const int cpp = C / VEC;                               // pieces per run
-    const int taps = kh * kw;
-    const int piece = (int)(idx % cpp);
-    size_t r = idx / cpp;
-    const int tap = (int)(r % taps);
-    r /= taps;                                             // = m
-    const int ox = (int)(r % ow);
-    size_t r2 = r / ow;
-    const int oy = (int)(r2 % oh);
-    const size_t b = r2 / oh;
-    const int i = tap / kw, j = tap - i * kw;
+    const int ppr = kh * kw * cpp;                         // pieces per row of A
+    const long m0 = (long)blockIdx.y * slab_rows;          // first row of the slab (uniform: scalar arithmetic)
+    const int rows = (int)min((long)slab_rows, M - m0);
+    const int e = (int)(blockIdx.x * 256u + threadIdx.x);
+    if (e >= rows * ppr) return;
+    const long line0 = m0 / ow;                            // (b, oy) of the slab's first row
+    const int ox0 = (int)(m0 - line0 * ow);
+    const long b0 = line0 / oh;
+    const int oy0 = (int)(line0 - b0 * oh);
+    const float inv_ppr = 1.0f / (float)ppr, inv_cpp = 1.0f / (float)cpp, inv_kw = 1.0f / (float)kw, inv_ow = 1.0f / (float)ow,
+                inv_oh = 1.0f / (float)oh;
+    const int ml = div_small(e, ppr, inv_ppr);
+    const int p = e - ml * ppr;
+    const int tap = div_small(p, cpp, inv_cpp);
+    const int piece = p - tap * cpp;
+    const int i = div_small(tap, kw, inv_kw), j = tap - i * kw;
+    const int xs = ox0 + ml;                               // < 2^23 + ow
+    const int dl = div_small(xs, ow, inv_ow);
+    const int ox = xs - dl * ow;
+    const int ys = oy0 + dl;
+    const int db = div_small(ys, oh, inv_oh);
+    const int oy = ys - db * oh;
+    const size_t b = (size_t)(b0 + db);
     const int y = oy * stride - pad + i * dil, xx = ox * stride - pad + j * dil;
     const bool in = y >= 0 && y < H && xx >= 0 && xx < W;
     const size_t src = ((b * H + (in ? y : 0)) * W + (in ? xx : 0)) * C + (size_t)piece * VEC;
+    const size_t dst = ((size_t)m0 * ppr + (size_t)e) * VEC;
     if constexpr (VEC == 16) {
         u32x4 v = *reinterpret_cast<const u32x4*>(codes + src);
         if (!in) v = u32x4{0, 0, 0, 0};
-        *reinterpret_cast<u32x4*>(A + idx * 16) = v;
+        *reinterpret_cast<u32x4*>(A + dst) = v;
     } else {
-        A[idx] = in ? codes[src] : (uint8_t)0;
+        A[dst] = in ? codes[src] : (uint8_t)0;
     }
 }
 
 hipError_t launch_im2col_nhwc(const uint8_t* codes, uint8_t* A, long B, int C, int H, int W, int kh, int kw, int stride, int pad,
                               int dil, int oh, int ow, hipStream_t stream) {
     const size_t bytes = (size_t)B * oh * ow * kh * kw * C;
+    const long M = B * oh * ow;
     if (bytes == 0) return hipSuccess;
-    if ((C & 15) == 0 && (((uintptr_t)codes | (uintptr_t)A) & 15) == 0) {
-        const size_t total = bytes / 16;
-        hipLaunchKernelGGL((im2col_nhwc_kernel<16>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, codes, A, C, H, W, kh,
-                           kw, stride, pad, dil, oh, ow, total);
-    } else {
-        hipLaunchKernelGGL((im2col_nhwc_kernel<1>), dim3((unsigned)((bytes + 255) / 256)), dim3(256), 0, stream, codes, A, C, H, W, kh,
-                           kw, stride, pad, dil, oh, ow, bytes);
-    }
+    // slabs of rows with at most 2^22 pieces each (the reciprocal divisions are exact below 2^23; ox0 + row stays below it)
+    const bool vec = (C & 15) == 0 && (((uintptr_t)codes | (uintptr_t)A) & 15) == 0;
+    const long ppr = (long)kh * kw * (vec ? C / 16 : C);
+    if (ppr > (1L << 22) || ow > (1 << 20) || oh > (1 << 20)) return hipErrorInvalidValue;
+    long slab_rows = (1L << 22) / ppr;
+    if (slab_rows > M) slab_rows = M;
+    const long slabs = (M + slab_rows - 1) / slab_rows;
+    if (slabs > 65535) return hipErrorInvalidValue;
+    const dim3 grid((unsigned)((slab_rows * ppr + 255) / 256), (unsigned)slabs);
+    if (vec)
+        hipLaunchKernelGGL((im2col_nhwc_kernel<16>), grid, dim3(256), 0, stream, codes, A, C, H, W, kh, kw, stride, pad, dil, oh, ow, M,
+                           (int)slab_rows);
+    else
+        hipLaunchKernelGGL((im2col_nhwc_kernel<1>), grid, dim3(256), 0, stream, codes, A, C, H, W, kh, kw, stride, pad, dil, oh, ow, M,
+                           (int)slab_rows);
     return hipGetLastError();
 }
 

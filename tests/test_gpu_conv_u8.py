@@ -73,6 +73,26 @@ def test_tap_major_im2col_against_oracle(ops, oracle, shape, k, stride, padding,
     assert (a.cpu().numpy() == want).all()
 
 
+@pytest.mark.parametrize("shape,k,stride,padding,dilation", [((200, 32, 61, 67), 3, 1, 1, 1), ((9, 3, 260, 300), 5, 1, 2, 1), ((300, 16, 131, 127), 3, 2, 1, 1)])
+def test_tap_major_im2col_over_several_slabs_of_rows(ops, shape, k, stride, padding, dilation):
+    """Window matrices of more than 2^22 pieces are written slab by slab (slab borders in the middle of an image line and of
+    an image): against torch's unfold of the same codes, columns permuted to the tap-major order."""
+    import approx_ops
+    print("im2col nhwc, several slabs", shape, k, stride, padding, dilation, flush=True)
+    bn, c, h, w = shape
+    oh, ow = out_size(h, w, k, stride, padding, dilation)
+    g = torch.Generator(device="cuda").manual_seed(3)
+    x = torch.randint(0, 256, shape, device="cuda", generator=g, dtype=torch.int32)
+    pieces = bn * oh * ow * k * k * (c // 16 if c % 16 == 0 else c)
+    assert pieces > 2 * (1 << 22)
+    codes = x.permute(0, 2, 3, 1).reshape(bn * h * w, c).to(torch.uint8).contiguous()
+    a = torch.full((bn * oh * ow, k * k * c), 77, dtype=torch.uint8, device="cuda")
+    approx_ops.im2col_nhwc(codes, a, shape, (k, k), stride, padding, dilation)
+    cols = F.unfold(x.float(), (k, k), dilation=dilation, padding=padding, stride=stride)          # [B, c*k*k, L]
+    want = cols.view(bn, c, k * k, oh * ow).permute(0, 3, 2, 1).reshape(bn * oh * ow, k * k * c).to(torch.uint8)
+    assert torch.equal(a, want)
+
+
 @pytest.mark.parametrize("shape,k,stride,padding,dilation", [
     ((3, 5, 10, 10), 3, 1, 1, 1), ((2, 4, 9, 7), 3, 2, 1, 1), ((2, 8, 12, 12), 1, 2, 0, 1), ((1, 3, 16, 16), 7, 2, 3, 1),
     ((2, 6, 11, 11), 3, 1, 2, 2), ((2, 64, 8, 8), 3, 1, 1, 1), ((4, 16, 32, 32), 3, 1, 1, 1), ((2, 32, 6, 6), 1, 1, 0, 1),
