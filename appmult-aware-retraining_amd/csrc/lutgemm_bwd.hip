@@ -128,7 +128,15 @@ __global__ void reduce_partials_kernel(const float* __restrict__ partial, float*
     size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= count) return;
     float s = partial[i];
-    for (int p = 1; p < splits; ++p) s += partial[(size_t)p * count + i];
+    int p = 1;
+    for (; p + 8 <= splits; p += 8) {      // (eight loads in flight, added in the order of the splits)
+        float t[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) t[u] = partial[(size_t)(p + u) * count + i];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) s += t[u];
+    }
+    for (; p < splits; ++p) s += partial[(size_t)p * count + i];
     out[i] = s;
 }
 

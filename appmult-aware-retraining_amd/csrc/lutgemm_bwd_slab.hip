@@ -487,10 +487,29 @@ __global__ __launch_bounds__(256) void gradB_finish_kernel(const float* __restri
     if (i >= count) return;
     const int n = (int)(i % (size_t)N);
     float v = partial ? partial[i] : gB[i];
-    for (int p = 1; p < splits && partial; ++p) v += partial[(size_t)p * count + i];
+    if (partial) {
+        // (eight loads in flight, added in the order of the splits: a load-add chain pays the memory latency once per split)
+        int p = 1;
+        for (; p + 8 <= splits; p += 8) {
+            float t[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) t[u] = partial[(size_t)(p + u) * count + i];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) v += t[u];
+        }
+        for (; p < splits; ++p) v += partial[(size_t)p * count + i];
+    }
     if (offset != 0.f) {
         float cs = colsum[n];
-        for (int p = 1; p < splits; ++p) cs += colsum[(size_t)p * N + n];
+        int p = 1;
+        for (; p + 8 <= splits; p += 8) {
+            float t[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) t[u] = colsum[(size_t)(p + u) * N + n];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) cs += t[u];
+        }
+        for (; p < splits; ++p) cs += colsum[(size_t)p * N + n];
         v += scale * offset * cs;
     }
     gB[i] = v;
