@@ -199,6 +199,9 @@ def _box_sum(xs, kernel, stride, padding, dilation):
                     dilation=dilation)
 
 
+IMPLICIT_FORWARD = True      # False: every forward pass of the uint8 layer path builds its window matrix
+
+
 class _ApproxConvLayerFn(torch.autograd.Function):
     """The activation side of ApproxConv2d.forward as one operator on uint8 codes (reference ``app_layers.py:172-183`` with
     ``approx_ops.py:556-571`` inlined): quantiser -> pixel-major uint8 codes, in-range mask and channel sums in one pass;
@@ -214,7 +217,7 @@ class _ApproxConvLayerFn(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, x, w, w_resp, taps, a_scale, a_zp, w_scale, w_zp, bias, a_qmax, stride, padding, dilation, fwd_cache=None,
-                prepared=None):
+                prepared=None, grad_mode=True):
         import approx_ops
         from self_ops.ops_py import approx_ops as ops
         one = lambda t: t.detach().reshape(1).contiguous()
@@ -230,8 +233,21 @@ class _ApproxConvLayerFn(torch.autograd.Function):
         inside = torch.empty((bn, cin, h, w_in), dtype=torch.uint8, device=dev)
         xs = torch.empty((bn, 1, h, w_in), dtype=torch.float32, device=dev)
         approx_ops.quantize_codes_nhwc(xc, s_a, z_a, a_qmax, codes, inside, xs)
+        # a 3x3 / stride 1 / padding 1 layer takes its input gradient from one implicit GEMM over the input pixels (no
+        # [M][9C] gradient matrix, no col2im) where the library serves the shape and the gradient table fits halves
+        same3x3 = (kh, kw, s, p, d) == (3, 3, 1, 1, 1)
+        # (grad_mode: whether the caller records a graph at all -- inside forward the mode is always off)
+        need_x, need_w = grad_mode and ctx.needs_input_grad[0], grad_mode and ctx.needs_input_grad[1]
+        conv_shaped = (same3x3 and need_x and ops.lut_grad_a_fits_halves
+                       and approx_ops.conv_input_grad_supported(ops.lut_grad_a, (bn, cin, h, w_in), cout))
+        # The window matrix is the operand of the weight gradient (and of a GEMM-shaped input gradient).  Where nobody will ask
+        # for those (evaluation, frozen weights) the forward pass of such a layer reads the pixel-major codes itself.
+        implicit = (IMPLICIT_FORWARD and same3x3 and not need_w and (conv_shaped or not need_x) and ops.lut_appmult_fits_packed
+                    and approx_ops.conv_forward_implicit_supported(ops.lut_appmult, (bn, cin, h, w_in), cout))
         if (kh, kw, s, p) == (1, 1, 1, 0):
             a_mat = codes                                           # a 1x1 window is the pixel itself
+        elif implicit:
+            a_mat = None
         else:
             a_mat = torch.empty((bn * oh * ow, kh * kw * cin), dtype=torch.uint8, device=dev)
             approx_ops.im2col_nhwc(codes, a_mat, (bn, cin, h, w_in), (kh, kw), s, p, d)
@@ -244,14 +260,13 @@ class _ApproxConvLayerFn(torch.autograd.Function):
         x_sum = _box_sum(xs, (kh, kw), stride, padding, dilation)
         out = torch.empty((bn, cout, oh, ow), dtype=torch.float32, device=dev)
         # (LUT GEMM whose store applies the zero-point terms, the scaling and the bias and writes NCHW)
-        approx_ops.approx_conv_forward_dequant(a_mat, b_mat, ops.lut_appmult, x_sum.contiguous(), w_resp.detach().contiguous(),
-                                               taps.contiguous(), z_a, z_w, s_a, s_w,
-                                               None if bias is None else bias.detach().contiguous(), out,
-                                               cache=fwd_cache[0] if fwd_cache else None, b_version=fwd_cache[1] if fwd_cache else 0)
-        # a 3x3 / stride 1 / padding 1 layer takes its input gradient from one implicit GEMM over the input pixels (no
-        # [M][9C] gradient matrix, no col2im) where the library serves the shape and the gradient table fits halves
-        conv_shaped = ((kh, kw, s, p, d) == (3, 3, 1, 1, 1) and ops.lut_grad_a_fits_halves
-                       and approx_ops.conv_input_grad_supported(ops.lut_grad_a, (bn, cin, h, w_in), cout))
+        dq_args = (ops.lut_appmult, x_sum.contiguous(), w_resp.detach().contiguous(), taps.contiguous(), z_a, z_w, s_a, s_w,
+                   None if bias is None else bias.detach().contiguous(), out)
+        cache_args = dict(cache=fwd_cache[0] if fwd_cache else None, b_version=fwd_cache[1] if fwd_cache else 0)
+        if implicit:
+            approx_ops.approx_conv_forward_implicit(codes, b_mat, *dq_args, (bn, cin, h, w_in), **cache_args)
+        else:
+            approx_ops.approx_conv_forward_dequant(a_mat, b_mat, *dq_args, **cache_args)
         ctx.save_for_backward(a_mat, b_mat, inside, s_a, z_a, s_w, z_w, codes if conv_shaped else None, inside_w, tapmask)
         ctx.geo = (bn, cin, h, w_in, cout, kh, kw, s, p, d, oh, ow)
         ctx.aux = (w_resp.shape, bias is not None, x.dtype)
@@ -299,7 +314,7 @@ class _ApproxConvLayerFn(torch.autograd.Function):
             g_wr = ((z_a * (s_a * s_w)) * g.sum(dim=0, keepdim=True)).reshape(wr_shape)
         if has_bias and ctx.needs_input_grad[8]:
             g_bias = g.sum(dim=(0, 2, 3))
-        return g_x, g_w, g_wr, None, None, None, None, None, g_bias, None, None, None, None, None, None
+        return g_x, g_w, g_wr, None, None, None, None, None, g_bias, None, None, None, None, None, None, None
 
 
 # ------------------------------------------------------------------------------------------ quantiser module
@@ -505,13 +520,15 @@ class ApproxConv2d(nn.Conv2d, _QuantParamsMixin):
             prepared, taps = self._prepared_weight_side(input, frozen)
             return _ApproxConvLayerFn.apply(input, self.weight, None, taps, self.activation_scale, self.activation_zp_neg,
                                             self.weight_scale, self.weight_zp_neg, self.bias, float(self.activation_quant_max),
-                                            tuple(self.stride), tuple(self.padding), tuple(self.dilation), frozen, prepared)
+                                            tuple(self.stride), tuple(self.padding), tuple(self.dilation), frozen, prepared,
+                                            torch.is_grad_enabled())
         w_codes = self.quantize_v2(self.weight, self.weight_scale, self.weight_zp_neg, self.weight_quant_max)
         if self._takes_uint8_path(input):
             w_resp, taps = self._weight_zero_point_parts(w_codes, input.shape[1:], conv_args, torch.float32, input.device)
             return _ApproxConvLayerFn.apply(input, w_codes, w_resp, taps, self.activation_scale, self.activation_zp_neg,
                                             self.weight_scale, self.weight_zp_neg, self.bias, float(self.activation_quant_max),
-                                            tuple(self.stride), tuple(self.padding), tuple(self.dilation), self._frozen_weight_cache())
+                                            tuple(self.stride), tuple(self.padding), tuple(self.dilation), self._frozen_weight_cache(),
+                                            None, torch.is_grad_enabled())
         x_codes = self.quantize_v2(input, self.activation_scale, self.activation_zp_neg, self.activation_quant_max)
         total = self.conv2d_op(x_codes, w_codes, **conv_args)       # approximate products of the codes
         if self.reference_zero_point_terms:

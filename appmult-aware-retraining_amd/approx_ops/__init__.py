@@ -66,6 +66,10 @@ _lib.amr_fwd_cache_destroy.argtypes = [_vp]
 _lib.amr_fwd_cache_stats.argtypes = [_vp, ctypes.POINTER(_u64), ctypes.POINTER(_u64), ctypes.POINTER(_sz)]
 _lib.amr_lut_gemm_forward_cached.argtypes = [_vp, _u64, _vp, _vp, _vp, _i, _vp, _i64, _i, _i, _i, _vp]
 _lib.amr_lut_conv_forward_dequant_cached_f32.argtypes = [_vp, _u64, _vp, _vp, _vp, _i64, _i, _i, _i, _i] + [_vp] * 9 + [_vp, _sz, _vp]
+_lib.amr_lut_conv_forward_implicit_supported.argtypes = [_i64, _i, _i, _i, _i, _i]
+_lib.amr_lut_conv_forward_implicit_workspace_bytes.argtypes = [_i64, _i, _i, _i, _i, _i, _i, _i]
+_lib.amr_lut_conv_forward_implicit_workspace_bytes.restype = _sz
+_lib.amr_lut_conv_forward_implicit_f32.argtypes = [_vp, ctypes.c_uint64, _vp, _vp, _vp, _i64, _i, _i, _i, _i, _i] + [_vp] * 10 + [_vp, _sz, _vp]
 _lib.amr_conv_weight_prepare_f32.argtypes = [_vp, _vp, _vp, ctypes.c_float, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]
 _lib.amr_conv_zero_point_grad_workspace_bytes.argtypes = [_i, _i, _i]
 _lib.amr_conv_zero_point_grad_workspace_bytes.restype = _sz
@@ -366,6 +370,60 @@ def approx_conv_forward_dequant(a_tensor, b_tensor, lut_appmult_tensor, x_sum, w
                                                    bias.data_ptr() if bias is not None else None, out_tensor.data_ptr(), ws.data_ptr(),
                                                    ws.numel(), _stream_ptr(dev))
     _raise_for(rc, "approx_conv_forward_dequant")
+
+
+def conv_forward_implicit_supported(lut_appmult_tensor, x_shape, out_channels):
+    """Whether approx_conv_forward_implicit serves a 3x3 / stride 1 / padding 1 convolution of an input of shape
+    x_shape = (B, C, H, W) with this table (asks the library)."""
+    Bn, C, H, W = (int(v) for v in x_shape)
+    dev = lut_appmult_tensor.device
+    if not lut_appmult_tensor.is_cuda:
+        return False
+    with torch.cuda.device(dev):
+        return bool(_lib.amr_lut_conv_forward_implicit_supported(lut_appmult_tensor.numel(), Bn, C, H, W, int(out_channels)))
+
+
+def approx_conv_forward_implicit(codes, bt_tensor, lut_appmult_tensor, x_sum, w_resp, taps, z_a, z_w, s_a, s_w, bias, out_tensor, x_shape,
+                                 a_fallback=None, cache=None, b_version=0):
+    """approx_conv_forward_dequant of a 3x3 / stride 1 / padding 1 convolution without its window matrix: codes uint8
+    [B*H*W, C] pixel-major (quantize_codes_nhwc), bt uint8 [9*C, N] tap-major weight codes, out float32 [B, N, H, W].
+    a_fallback (optional): the window matrix [B*H*W, 9*C]; without it a masked code or a table the packed sums cannot hold
+    leaves NaN in out."""
+    _check_input(codes, torch.uint8, "codes")
+    _check_input(bt_tensor, torch.uint8, "bt_tensor")
+    _check_input(lut_appmult_tensor, torch.uint16, "lut_appmult_tensor")
+    tensors = [(x_sum, "x_sum"), (w_resp, "w_resp"), (taps, "taps"), (z_a, "z_a"), (z_w, "z_w"), (s_a, "s_a"), (s_w, "s_w"),
+               (out_tensor, "out_tensor")] + ([(bias, "bias")] if bias is not None else [])
+    for t, name in tensors:
+        _check_input(t, torch.float32, name)
+    Bn, C, H, W = (int(v) for v in x_shape)
+    M, L = Bn * H * W, H * W
+    _check(codes.dim() == 2 and tuple(codes.shape) == (M, C), f"codes' shape should be {M} x {C}")
+    _check(bt_tensor.dim() == 2 and bt_tensor.size(0) == 9 * C, f"bt_tensor should have {9 * C} rows")
+    N = bt_tensor.size(1)
+    _check(tuple(out_tensor.shape) == (Bn, N, H, W), f"out_tensor's shape should be {(Bn, N, H, W)}")
+    _check(x_sum.numel() == M and w_resp.numel() == N * L and taps.numel() == L, "x_sum, w_resp or taps has the wrong size")
+    _check(all(t.numel() == 1 for t in (z_a, z_w, s_a, s_w)), "z_a, z_w, s_a and s_w must hold one element")
+    _check(bias is None or bias.numel() == N, f"bias should have {N} elements")
+    if a_fallback is not None:
+        _check_input(a_fallback, torch.uint8, "a_fallback")
+        _check(tuple(a_fallback.shape) == (M, 9 * C), f"a_fallback's shape should be {M} x {9 * C}")
+    _lut_len_check(lut_appmult_tensor, "lut_appmult_tensor")
+    dev = codes.device
+    _check(all(t.device == dev for t, _ in tensors) and bt_tensor.device == dev and lut_appmult_tensor.device == dev
+           and (a_fallback is None or a_fallback.device == dev), "device id not match")
+    with torch.cuda.device(dev):
+        need = _lib.amr_lut_conv_forward_implicit_workspace_bytes(lut_appmult_tensor.size(0), Bn, C, H, W, N, 1 if cache is not None else 0,
+                                                                  1 if a_fallback is not None else 0)
+        ws = torch.empty(need, dtype=torch.uint8, device=dev) if need else None
+        rc = _lib.amr_lut_conv_forward_implicit_f32(cache._h if cache is not None else None, int(b_version) & 0xFFFFFFFFFFFFFFFF,
+                                                    codes.data_ptr(), bt_tensor.data_ptr(), lut_appmult_tensor.data_ptr(),
+                                                    lut_appmult_tensor.size(0), Bn, C, H, W, N, x_sum.data_ptr(), w_resp.data_ptr(),
+                                                    taps.data_ptr(), z_a.data_ptr(), z_w.data_ptr(), s_a.data_ptr(), s_w.data_ptr(),
+                                                    bias.data_ptr() if bias is not None else None, out_tensor.data_ptr(),
+                                                    a_fallback.data_ptr() if a_fallback is not None else None,
+                                                    ws.data_ptr() if ws is not None else None, need, _stream_ptr(dev))
+    _raise_for(rc, "approx_conv_forward_implicit")
 
 
 def conv_dequant_backward(g_tensor, s_a, s_w, gc_rows):

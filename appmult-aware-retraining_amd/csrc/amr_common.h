@@ -73,6 +73,14 @@ struct SlabDequant {
     int L;                // positions per image
 };
 
+// Convolution-shaped forward pass (3x3, stride 1, padding 1): the rows of the GEMM are the pixels of pixel-major codes
+// [B*H*W][C]; column k = tap*C + c of row m is the code of channel c of the pixel tap (ti, tj) reaches from pixel m, or the
+// code 0 of the padding (zero: 16 zero bytes, 16-byte aligned).
+struct SlabConv {
+    const uint8_t* zero;
+    int C, H, W;
+};
+
 __device__ __forceinline__ int uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
 
 // Four consecutive bytes starting at an arbitrary byte address (global memory accepts unaligned

@@ -18,8 +18,10 @@ hipError_t launch_fwd(const uint8_t* A, const uint8_t* B, uint32_t* C, const uin
 size_t fwd_slab_workspace_bytes(const LutGeom& g, int M, int K, int N, bool force);
 hipError_t launch_fwd_slab(const uint8_t* A, const uint8_t* B, uint32_t* C, const uint16_t* lut, const LutGeom& g,
                            int M, int K, int N, int n_cu, void* workspace, hipStream_t stream, int out_f32,
-                           const SlabDequant* dq = nullptr, int expanded = 0);
+                           const SlabDequant* dq = nullptr, int expanded = 0, const SlabConv* cv = nullptr,
+                           const uint8_t* a_fallback = nullptr);
 bool fwd_slab_can_dequant(const LutGeom& g, int M, int K, int N, int n_cu, bool force);
+bool fwd_slab_conv_applies(const LutGeom& g, long M, int C, int N, int n_cu, bool force);
 size_t gradB_workspace_bytes(int M, int K, int N, int n_cu);
 hipError_t launch_gradB(const float* gC, const uint8_t* A, const uint8_t* B, float* gB, const int16_t* lut,
                         const LutGeom& g, int M, int K, int N, float scale, void* workspace, int n_cu,
@@ -450,6 +452,62 @@ int amr_lut_conv_forward_dequant_cached_f32(amr_fwd_cache* cache, uint64_t b_ver
     if (rc != AMR_OK) return rc;
     e = amr::launch_dequant(sums, x_sum, w_resp, taps, z_a, z_w, s_a, s_w, bias, out, M, N, positions, s);
     return e == hipSuccess ? AMR_OK : hip_fail(e, "dequant launch");
+}
+
+int amr_lut_conv_forward_implicit_supported(int64_t lut_elems, int B, int C, int H, int W, int N) {
+    amr::LutGeom g;
+    if (B <= 0 || C <= 0 || H <= 0 || W <= 0 || N <= 0 || !amr::lut_geom_from_elems(lut_elems, &g)) return 0;
+    const int mode = g_expanded_kernels.load();
+    const int n_cu = current_device_cus(nullptr);
+    const long M = (long)B * H * W;
+    if (!mode || (double)M * 9 * C >= 2147483648.0) return 0;
+    return amr::fwd_slab_conv_applies(g, M, C, N, n_cu > 0 ? n_cu : 256, mode == 2) ? 1 : 0;
+}
+
+size_t amr_lut_conv_forward_implicit_workspace_bytes(int64_t lut_elems, int B, int C, int H, int W, int N, int cached, int with_fallback) {
+    if (!amr_lut_conv_forward_implicit_supported(lut_elems, B, C, H, W, N)) return 0;
+    const int M = B * H * W;
+    const size_t e = cached ? 0 : (amr_lut_gemm_forward_workspace_bytes(lut_elems, M, 9 * C, N) + 255) & ~(size_t)255;
+    return e + (with_fallback ? (size_t)M * N * sizeof(float) : 0);
+}
+
+int amr_lut_conv_forward_implicit_f32(amr_fwd_cache* cache, uint64_t b_version, const uint8_t* codes, const uint8_t* Bt,
+                                      const uint16_t* lut, int64_t lut_elems, int B, int C, int H, int W, int N, const float* x_sum,
+                                      const float* w_resp, const float* taps, const float* z_a, const float* z_w, const float* s_a,
+                                      const float* s_w, const float* bias, float* out, const uint8_t* A_fallback, void* workspace,
+                                      size_t workspace_bytes, void* stream) {
+    amr::LutGeom g;
+    if (!amr::lut_geom_from_elems(lut_elems, &g))
+        return fail(AMR_ELUTLEN, "lut size should be one of 1024/5120/17408/66306, got %lld", (long long)lut_elems);
+    if (B <= 0 || C <= 0 || H <= 0 || W <= 0 || N <= 0) return fail(AMR_EINVAL, "bad shape B=%d C=%d H=%d W=%d N=%d", B, C, H, W, N);
+    if (!amr_lut_conv_forward_implicit_supported(lut_elems, B, C, H, W, N))
+        return fail(AMR_EUNSUPPORTED, "shape or table not served by the convolution-shaped forward kernel (ask amr_lut_conv_forward_implicit_supported)");
+    if (!codes || !Bt || !lut || !x_sum || !w_resp || !taps || !z_a || !z_w || !s_a || !s_w || !out) return fail(AMR_EINVAL, "null pointer argument");
+    if (((uintptr_t)lut & 3) || ((uintptr_t)codes & 15)) return fail(AMR_EINVAL, "lut must be 4-byte and codes 16-byte aligned");
+    const size_t need = amr_lut_conv_forward_implicit_workspace_bytes(lut_elems, B, C, H, W, N, cache ? 1 : 0, A_fallback ? 1 : 0);
+    if (need && (!workspace || workspace_bytes < need))
+        return fail(AMR_EWORKSPACE, "workspace of %zu bytes is smaller than the %zu required", workspace ? workspace_bytes : (size_t)0, need);
+    if (need && ((uintptr_t)workspace & 255)) return fail(AMR_EINVAL, "workspace must be 256-byte aligned");
+    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    int dev = 0;
+    const int n_cu = current_device_cus(&dev);
+    if (n_cu <= 0) return fail(AMR_EINVAL, "no HIP device available");
+    const int M = B * H * W, K = 9 * C;
+    const int mode = g_expanded_kernels.load();
+    const size_t e_bytes = cache ? 0 : (amr_lut_gemm_forward_workspace_bytes(lut_elems, M, K, N) + 255) & ~(size_t)255;
+    float* sums = A_fallback ? reinterpret_cast<float*>(reinterpret_cast<unsigned char*>(workspace) + e_bytes) : nullptr;
+    const amr::SlabDequant dq{x_sum, w_resp, taps, z_a, z_w, s_a, s_w, bias, out, H * W};
+    const amr::SlabConv cv{nullptr, C, H, W};
+    void* e_buf = workspace;
+    bool hit = false;
+    hipError_t e;
+    if (cache) {
+        e_buf = fwd_cache_lookup(cache, dev, amr::fwd_slab_workspace_bytes(g, M, K, N, mode == 2), b_version, lut, lut_elems, K, N, &hit, &e);
+        if (!e_buf) return hip_fail(e, "cache hipMalloc");
+    }
+    e = amr::launch_fwd_slab(codes, Bt, reinterpret_cast<uint32_t*>(sums), lut, g, M, K, N, n_cu, e_buf, s, 1, &dq, hit ? 1 : 0, &cv, A_fallback);
+    if (cache && e != hipSuccess) fwd_cache_forget(cache);
+    return e == hipSuccess ? AMR_OK : hip_fail(e, "forward launch");
 }
 
 int amr_lut_gemm_forward_ws(const uint8_t* A, const uint8_t* B, uint32_t* C, const uint16_t* lut, int64_t lut_elems,

@@ -84,6 +84,7 @@ __global__ __launch_bounds__(256) void expand_fwd_kernel(const uint8_t* __restri
     if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) {
         flags[0] = max(max(wave_max[0], wave_max[1]), max(wave_max[2], wave_max[3]));
         flags[1] = 0u;
+        flags[32] = flags[33] = flags[34] = flags[35] = 0u;      // the 16 zero codes the convolution-shaped kernel reads for padding
     }
     const uint16_t* s16 = reinterpret_cast<const uint16_t*>(smem);
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -323,11 +324,14 @@ __device__ __forceinline__ void slab_store_tile_dequant(const uint32_t (&acc)[RG
     }
 }
 
-template <int RG, int WAVES, bool PACKED, bool DEQ = false>
+// CONV: A holds pixel-major codes [M][cv.C] and K = 9 * cv.C: the 16 codes a lane fetches per group are 16 adjacent
+// channels of ONE tap (cv.C % 16 == 0, no K split), i.e. 16 adjacent bytes of a neighbouring pixel, or of the zero line
+// where that neighbour is padding -- no window matrix is read.
+template <int RG, int WAVES, bool PACKED, bool DEQ = false, bool CONV = false>
 __global__ __launch_bounds__(WAVES * 64) void lutgemm_fwd_slab_kernel(
     const uint8_t* __restrict__ A, const u32x4* __restrict__ E, uint32_t* __restrict__ C,
     uint32_t* __restrict__ flags, int M, int K, int N, int k_quads, int chunks_per_split, int atomic_out, int out_f32,
-    int n_tiles_grouped, int row_blocks, SlabDequant dq) {
+    int n_tiles_grouped, int row_blocks, SlabDequant dq, SlabConv cv) {
     // static: lets the compiler fold the base address (chunk buffers first: their addresses come out of v_perm)
     __shared__ __align__(16) unsigned char smem[kSlabBuffers * kSlabChunkBytes + 2 * kSlabCodeBytes];
     constexpr int THREADS = WAVES * 64;
@@ -388,7 +392,16 @@ __global__ __launch_bounds__(WAVES * 64) void lutgemm_fwd_slab_kernel(
     // which land at staging position l (16 B each): the four dword reads of a chunk are 256 B apart and the
     // eight row slots that one pass of a read serves are 16 B apart, in eight different banks.
     // 32-bit offsets: the host only takes this path when M*K < 2^31.
-    const uint32_t code_off = (uint32_t)(m_wave + lane) * (uint32_t)K;
+    const uint32_t code_off = (uint32_t)(m_wave + lane) * (uint32_t)(CONV ? cv.C : K);
+    // CONV: which neighbours of this lane's pixel exist: bit 0 the row below, 1 the row above, 2 the pixel to the right, 3 the
+    // pixel to the left
+    uint32_t neighbours = 0;
+    if constexpr (CONV) {
+        const int m = m_wave + lane;
+        const int pix = m % (cv.H * cv.W);
+        const int y = pix / cv.W, x = pix - y * cv.W;
+        neighbours = (uint32_t)((y + 1 < cv.H) | ((y >= 1) << 1) | ((x + 1 < cv.W) << 2) | ((x >= 1) << 3));
+    }
     unsigned char* code_stage = smem + kSlabBuffers * kSlabChunkBytes + wave * 1024;      // + (group & 1) * kSlabCodeBytes
     const uint32_t code_read = (uint32_t)(kSlabBuffers * kSlabChunkBytes + wave * 1024 + rs * 16);
 
@@ -400,6 +413,17 @@ __global__ __launch_bounds__(WAVES * 64) void lutgemm_fwd_slab_kernel(
     const int g_last = (c_end - 1 - c_begin) >> 2;
     auto group_koff = [&](int g) { return min(4 * (c_begin + 4 * min(g, g_last)), K - 16); };
     auto request_codes = [&](int g) {
+        if constexpr (CONV) {
+            // tap (ti, tj) of output pixel (y, x) reads input pixel (y + ti - 1, x + tj - 1)
+            const int koff = group_koff(g);
+            const int tap = koff / cv.C, c0 = koff - tap * cv.C;
+            const int ti = tap / 3, tj = tap - 3 * ti;
+            const uint32_t need = (ti == 0 ? 2u : 0u) | (ti == 2 ? 1u : 0u) | (tj == 0 ? 8u : 0u) | (tj == 2 ? 4u : 0u);
+            const int off = (int)code_off + ((ti - 1) * cv.W + (tj - 1)) * cv.C + c0;
+            const uint8_t* p = (neighbours & need) == need ? A + off : cv.zero;
+            __builtin_amdgcn_global_load_lds((gptr_t)p, (lptr_t)(code_stage + (g & 1) * kSlabCodeBytes), 16, 0, 0);
+            return;
+        }
         __builtin_amdgcn_global_load_lds((gptr_t)(A + (code_off + (uint32_t)group_koff(g))),
                                          (lptr_t)(code_stage + (g & 1) * kSlabCodeBytes), 16, 0, 0);
     };
@@ -598,12 +622,26 @@ bool fwd_slab_can_dequant(const LutGeom& g, int M, int K, int N, int n_cu, bool 
 // (float32 [M,N]) is then scratch that only the gated fall-back touches, followed by a dequantisation pass under the same gate.
 // expanded != 0: `workspace` already holds the expansion of this B and table (a caller's cache); only the fall-back request
 // in its header is cleared, by a one-word fill, in place of the expansion launch.
+hipError_t launch_poison_if_raised(float* gx, size_t total, const uint32_t* gate, hipStream_t stream);
+
+// Whether the convolution-shaped forward launch serves this geometry (then with a dequantising store and no K split).
+bool fwd_slab_conv_applies(const LutGeom& g, long M, int C, int N, int n_cu, bool force) {
+    if (g.bits > 7 || (C & 15) != 0 || M > (1L << 30) || 9L * C > (1L << 24)) return false;
+    return fwd_slab_can_dequant(g, (int)M, 9 * C, N, n_cu, force);
+}
+
+// cv != nullptr (only with fwd_slab_conv_applies and dq): A holds the pixel-major codes of the layer's input, B the
+// tap-major weight codes [9 C][N]; a_fallback (optional) the window matrix [M][9 C] for the gated direct kernel -- without
+// it a masked code or a table that does not fit packed sums leaves NaN in dq->out.
 hipError_t launch_fwd_slab(const uint8_t* A, const uint8_t* B, uint32_t* C, const uint16_t* lut, const LutGeom& g,
                            int M, int K, int N, int n_cu, void* workspace, hipStream_t stream, int out_f32,
-                           const SlabDequant* dq = nullptr, int expanded = 0) {
+                           const SlabDequant* dq = nullptr, int expanded = 0, const SlabConv* cv = nullptr,
+                           const uint8_t* a_fallback = nullptr) {
     const int n_tiles = (N + kSlabCols - 1) / kSlabCols;
     const int k_quads = (K + 3) / 4;
     const SlabDequant none{};
+    const SlabConv no_conv{};
+    if (cv && (!dq || g.bits == 8)) return hipErrorInvalidValue;
     uint32_t* flags = reinterpret_cast<uint32_t*>(workspace);
     uint32_t* E = reinterpret_cast<uint32_t*>(reinterpret_cast<unsigned char*>(workspace) + 256);
     hipError_t e;
@@ -673,10 +711,22 @@ hipError_t launch_fwd_slab(const uint8_t* A, const uint8_t* B, uint32_t* C, cons
         grouped = n_tiles;
         grid = dim3(8 * ((row_blocks + 7) / 8) * n_tiles);
     }
+    if (cv) {
+        if (zs != 1) return hipErrorInvalidValue;
+        SlabConv c = *cv;
+        c.zero = reinterpret_cast<const uint8_t*>(flags + 32);
+        hipLaunchKernelGGL((lutgemm_fwd_slab_kernel<RG, WAVES, true, true, true>), grid, dim3(WAVES * 64), 0, stream, A,
+                           reinterpret_cast<const u32x4*>(E), C, flags, M, K, N, k_quads, cps, 0, 1, grouped, row_blocks, *dq, c);
+        if ((e = hipGetLastError()) != hipSuccess) return e;
+        if (!a_fallback) return launch_poison_if_raised(dq->out, (size_t)M * N, flags + 1, stream);
+        if ((e = launch_fwd_gated(a_fallback, B, C, lut, g, M, K, N, flags + 1, stream, 1)) != hipSuccess) return e;
+        return launch_dequant_gated(reinterpret_cast<const float*>(C), dq->xs, dq->wr, dq->tp, dq->za, dq->zw, dq->sa, dq->sw, dq->bias,
+                                    dq->out, M, N, dq->L, flags + 1, stream);
+    }
     if (dq) {
         if (zs != 1) return hipErrorInvalidValue;
         hipLaunchKernelGGL((lutgemm_fwd_slab_kernel<RG, WAVES, true, true>), grid, dim3(WAVES * 64), 0, stream, A,
-                           reinterpret_cast<const u32x4*>(E), C, flags, M, K, N, k_quads, cps, 0, 1, grouped, row_blocks, *dq);
+                           reinterpret_cast<const u32x4*>(E), C, flags, M, K, N, k_quads, cps, 0, 1, grouped, row_blocks, *dq, no_conv);
         if ((e = hipGetLastError()) != hipSuccess) return e;
         // masked codes / entries too large for packed sums: the direct kernel recomputes the sums into C, a pass under the
         // same gate dequantises them
@@ -685,7 +735,8 @@ hipError_t launch_fwd_slab(const uint8_t* A, const uint8_t* B, uint32_t* C, cons
                                     dq->out, M, N, dq->L, flags + 1, stream);
     }
     hipLaunchKernelGGL((lutgemm_fwd_slab_kernel<RG, WAVES, true>), grid, dim3(WAVES * 64), 0, stream, A,
-                       reinterpret_cast<const u32x4*>(E), C, flags, M, K, N, k_quads, cps, zs > 1 ? 1 : 0, out_f32, grouped, row_blocks, none);
+                       reinterpret_cast<const u32x4*>(E), C, flags, M, K, N, k_quads, cps, zs > 1 ? 1 : 0, out_f32, grouped, row_blocks, none,
+                       no_conv);
     e = hipGetLastError();
     if (e != hipSuccess) return e;
     // (partial sums over a split K met as integers: converted before the fall-back, which stores floats itself)

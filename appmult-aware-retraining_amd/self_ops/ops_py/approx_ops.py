@@ -18,6 +18,7 @@ lut_grad_a = None    # int16 padded table, 16 x d(product)/d(first operand)
 lut_grad_b = None    # int16 padded table, 16 x d(product)/d(second operand)
 table_generation = 0             # counts set_lookup_tables calls: part of what identifies an expansion kept between calls
 lut_grad_a_fits_halves = False   # whether the expanded-table backward kernels can hold lut_grad_a as halves (int16 tables)
+lut_appmult_fits_packed = False  # whether four entries of lut_appmult add up in 16 bits (the expanded-table forward kernel's packed sums)
 
 _SECTION_HEADERS = (
     ("LUT for approximate multiplier:", 0),
@@ -89,8 +90,9 @@ def set_lookup_tables(device, appmult, grad_a, grad_b):
 
     Gradient tables of a floating dtype are installed as float32 and taken as the slopes themselves (no factor 1/16):
     the backward pass then runs on the native float-table entry point."""
-    global lut_appmult, lut_grad_a, lut_grad_b, lut_grad_a_fits_halves, table_generation
+    global lut_appmult, lut_grad_a, lut_grad_b, lut_grad_a_fits_halves, lut_appmult_fits_packed, table_generation
     table_generation += 1
+    lut_appmult_fits_packed = int(np.max(np.asarray(appmult), initial=0)) < 16384
     lut_appmult = torch.as_tensor(np.ascontiguousarray(appmult, np.uint16)).to(device)
     as_float = np.issubdtype(np.asarray(grad_a).dtype, np.floating) and np.issubdtype(np.asarray(grad_b).dtype, np.floating)
     gdt = np.float32 if as_float else np.int16

@@ -122,13 +122,16 @@ def capture_codes(torch, dev, bits, tables, arch, batch):
             return fn(a, b, *rest, **kw)
         return spy
 
+    import app_layers
     for n in names:
         setattr(ops.approx_ops, n, spy_on(natives[n]))
+    implicit, app_layers.IMPLICIT_FORWARD = app_layers.IMPLICIT_FORWARD, False      # (the GEMM operands are what is captured)
     try:
         model.train()
         with torch.no_grad():
             model(x)
     finally:
+        app_layers.IMPLICIT_FORWARD = implicit
         for n in names:
             setattr(ops.approx_ops, n, natives[n])
     return seen

@@ -262,6 +262,28 @@ int amr_lut_conv_forward_dequant_cached_f32(amr_fwd_cache *cache, uint64_t b_ver
                                             void *workspace, size_t workspace_bytes, void *stream);
 
 /*
+ * The same forward pass of a 3x3 convolution of stride 1 and padding 1 WITHOUT its window matrix (the reference builds it with
+ * F.pad + F.unfold, self_ops/ops_py/approx_ops.py:556-563, and feeds it to self_ops/src/approx_gemm_forward.cu:241-314): the
+ * rows of the GEMM are the B*H*W pixels of `codes` (pixel-major uint8 [B*H*W][C], what amr_quantize_codes_nhwc_u8 writes, 16-byte
+ * aligned), column tap*C + c of a row is read from the neighbouring pixel the tap reaches, or as code 0 where that pixel is
+ * padding; Bt [9*C][N] tap-major weight codes.  out and the dequantisation operands as above with positions = H*W.
+ *   amr_lut_conv_forward_implicit_supported: 1 where the kernel serves the geometry and table width (tables of at most 7 bits,
+ *     C a multiple of 16, the shapes the expanded-table kernel takes without a K split), else 0.
+ *   A_fallback (optional): the window matrix [B*H*W][9*C]; with it a masked code in the operands or a table whose entries do not
+ *     fit the packed sums is recomputed by the gated direct kernel as in the calls above; without it such a case leaves NaN in out.
+ *   cache (optional) as in the _cached call.  workspace: amr_lut_conv_forward_implicit_workspace_bytes(..., cache != NULL,
+ *     A_fallback != NULL) bytes, 256-byte aligned (0 bytes with a cache and no fall-back: workspace may then be NULL).
+ */
+int amr_lut_conv_forward_implicit_supported(int64_t lut_elems, int B, int C, int H, int W, int N);
+size_t amr_lut_conv_forward_implicit_workspace_bytes(int64_t lut_elems, int B, int C, int H, int W, int N, int cached,
+                                                     int with_fallback);
+int amr_lut_conv_forward_implicit_f32(amr_fwd_cache *cache, uint64_t b_version, const uint8_t *codes, const uint8_t *Bt,
+                                      const uint16_t *lut, int64_t lut_elems, int B, int C, int H, int W, int N,
+                                      const float *x_sum, const float *w_resp, const float *taps, const float *z_a,
+                                      const float *z_w, const float *s_a, const float *s_w, const float *bias, float *out,
+                                      const uint8_t *A_fallback, void *workspace, size_t workspace_bytes, void *stream);
+
+/*
  * Range tracking and quantisation parameters of one tensor in one launch (all pointers: one float in device memory).
  * mode 0: min_val/max_val := cur_min/cur_max (first batch); 1: running extremes; 2: keep * old + momentum * current;
  * then *scale = max((max - min) / quant_max, eps) -- or (max - min) * inv_quant_max when inv_quant_max != 0, which is

@@ -337,6 +337,108 @@ def test_forward_with_dequantising_store_equals_gemm_then_dequantisation(ops, or
     assert torch.equal(got, want)
 
 
+@pytest.mark.parametrize("bits,bn,c,h,w,n,masked,bias", [
+    # (the kernel serves shapes that fill the device without a K split: column tiles x blocks of 1024 rows >= compute units)
+    (7, 128, 64, 32, 32, 64, False, True),     # conv2_x
+    (7, 2100, 16, 7, 9, 40, False, False),     # image sides that are no powers of two, ragged column tile
+    (7, 16400, 32, 4, 4, 32, False, True),     # 4x4 images: most pixels touch the border
+    (7, 146, 16, 31, 29, 64, False, True),     # rows not a multiple of a wave's 64
+    (6, 128, 32, 32, 32, 64, False, True),     # narrower table
+    (7, 128, 64, 32, 32, 64, True, True),      # a masked code: fall-back with the window matrix, NaN without
+])
+def test_convolution_shaped_forward_equals_the_forward_pass_on_the_window_matrix(ops, oracle, bits, bn, c, h, w, n, masked, bias):
+    """approx_conv_forward_implicit (no window matrix: the kernel reads the neighbouring pixels' codes, code 0 for padding)
+    against approx_conv_forward_dequant on the window matrix of the same codes: identical bits; the sums of the first rows
+    against the oracle's LUT GEMM on that window matrix."""
+    import approx_ops
+    print("implicit forward", bits, bn, c, h, w, n, masked, flush=True)
+    rng = np.random.default_rng(31)
+    nc = 1 << bits
+    M, L, K = bn * h * w, h * w, 9 * c
+    X = rng.integers(0, nc, (bn, c, h, w)).astype(np.uint8)
+    B = rng.integers(0, nc, (K, n)).astype(np.uint8)
+    if masked:
+        X[bn // 2, 3, h // 2, 1] = nc
+    T = oracle.synth_lut(bits, 64, rng)
+    flat = oracle.pack_table(T, bits, np.uint16)
+    x, bt, lut = (torch.tensor(v, device="cuda") for v in (X, B, flat))
+    codes = x.permute(0, 2, 3, 1).reshape(M, c).contiguous()
+    a = torch.empty((M, K), dtype=torch.uint8, device="cuda")
+    approx_ops.im2col_nhwc(codes, a, (bn, c, h, w), (3, 3), 1, 1, 1)
+    g = torch.Generator(device="cuda").manual_seed(4)
+    x_sum = torch.randint(0, 9 * 64 * 127, (M,), device="cuda", generator=g).float()
+    w_resp = torch.randint(0, 9 * 64 * 127, (n, L), device="cuda", generator=g).float()
+    taps = torch.randint(1, 577, (L,), device="cuda", generator=g).float()
+    z_a, z_w = torch.tensor([-3.0], device="cuda"), torch.tensor([-61.0], device="cuda")
+    s_a, s_w = torch.tensor([0.0213], device="cuda"), torch.tensor([0.0037], device="cuda")
+    bvec = torch.randn(n, device="cuda", generator=g) if bias else None
+    old = approx_ops._lib.amr_set_expanded_table_kernels(2)
+    try:
+        assert approx_ops.conv_forward_implicit_supported(lut, (bn, c, h, w), n)
+        want = torch.full((bn, n, h, w), float("nan"), device="cuda")
+        approx_ops.approx_conv_forward_dequant(a, bt, lut, x_sum, w_resp, taps, z_a, z_w, s_a, s_w, bvec, want)
+        got = torch.full((bn, n, h, w), float("nan"), device="cuda")
+        approx_ops.approx_conv_forward_implicit(codes, bt, lut, x_sum, w_resp, taps, z_a, z_w, s_a, s_w, bvec, got, (bn, c, h, w),
+                                                a_fallback=a if masked else None)
+        assert torch.equal(got, want)
+        if masked:
+            lost = torch.zeros((bn, n, h, w), device="cuda")
+            approx_ops.approx_conv_forward_implicit(codes, bt, lut, x_sum, w_resp, taps, z_a, z_w, s_a, s_w, bvec, lost, (bn, c, h, w))
+            assert torch.isnan(lost).all()
+        # with the expansion kept between calls: a miss, then a hit, same bits
+        cache = approx_ops.ForwardCache()
+        for _ in range(2):
+            again = torch.full((bn, n, h, w), float("nan"), device="cuda")
+            approx_ops.approx_conv_forward_implicit(codes, bt, lut, x_sum, w_resp, taps, z_a, z_w, s_a, s_w, bvec, again, (bn, c, h, w),
+                                                    a_fallback=a if masked else None, cache=cache, b_version=5)
+            assert torch.equal(again, want)
+        assert cache.stats()[:2] == (1, 1)
+        # refused: channels no multiple of 16, 8-bit tables
+        assert not approx_ops.conv_forward_implicit_supported(lut, (bn, c + 8, h, w), n)
+        assert not approx_ops.conv_forward_implicit_supported(torch.zeros(66306, dtype=torch.uint16, device="cuda"), (bn, c, h, w), n)
+    finally:
+        approx_ops._lib.amr_set_expanded_table_kernels(old)
+    # the sums behind the activation, against the oracle on the window matrix (first rows)
+    rows = slice(0, min(M, 1024))
+    csum = torch.empty((M, n), dtype=torch.float32, device="cuda")
+    approx_ops.approx_gemm_forward(a, bt, csum, lut)
+    assert (csum[rows].cpu().numpy() == oracle.forward_c(a[rows].cpu().numpy(), B, flat, bits).astype(np.float32)).all()
+    plain = torch.empty_like(want)
+    approx_ops.conv_dequant(csum, x_sum, w_resp, taps, z_a, z_w, s_a, s_w, bvec, plain)
+    assert torch.equal(plain, want)
+
+
+def test_layer_reads_the_codes_itself_where_no_window_matrix_is_needed(ops):
+    """ApproxConv2d (3x3, stride 1, padding 1): under no_grad, and with frozen weights, the forward pass takes the
+    convolution-shaped kernel (no im2col call); outputs and the input gradient equal those of the pass on the window matrix."""
+    import approx_ops
+    import app_layers as L
+    torch.manual_seed(3)
+    layer = L.ApproxConv2d(64, 64, 3, padding=1, bias=False, a_bits=7, w_bits=7).cuda().train()
+    x = torch.randn(512, 64, 16, 16, device="cuda") * 2 + 0.3
+    layer(x)
+    layer.eval()
+    calls = []
+    native = approx_ops.im2col_nhwc
+    approx_ops.im2col_nhwc = lambda *a, **k: (calls.append(1), native(*a, **k))[1]
+    try:
+        xi = x.clone().requires_grad_()
+        y_train = layer(xi)                               # weights require a gradient: window matrix
+        assert len(calls) == 1
+        y_train.square().mean().backward()
+        with torch.no_grad():
+            y_eval = layer(x)
+        assert len(calls) == 1 and torch.equal(y_eval, y_train.detach())
+        layer.weight.requires_grad_(False)
+        xj = x.clone().requires_grad_()
+        y_frozen = layer(xj)                              # only the input gradient is asked for: convolution-shaped both ways
+        assert len(calls) == 1 and torch.equal(y_frozen.detach(), y_train.detach())
+        y_frozen.square().mean().backward()
+        torch.testing.assert_close(xj.grad, xi.grad, rtol=1e-5, atol=1e-6 * float(xi.grad.abs().max()))
+    finally:
+        approx_ops.im2col_nhwc = native
+
+
 def _conv_grad_case(oracle, seed, bn, c, h, w, n, lo=-1024, hi=3073, masked=False):
     """Operands of one input-gradient problem of a 3x3 / stride 1 / padding 1 convolution and its float64 answer."""
     rng = np.random.default_rng(seed)

@@ -205,6 +205,24 @@ def test_layer_level_entry_points_check_arguments_without_touching_a_device():
     lib.amr_observe_minmax_f32.argtypes = [vp, i64, vp, vp, vp, vp, vp, i] + [f] * 5 + [vp]
     assert lib.amr_observe_minmax_f32(None, 10, None, None, None, None, None, 3, 0.9, 0.1, 127.0, 0.0, 1e-7, None) == -1   # mode
     assert lib.amr_observe_minmax_f32(None, 10, None, None, None, None, None, 2, 0.9, 0.1, 127.0, 0.0, 1e-7, None) == -1   # null pointers
+    lib.amr_lut_conv_forward_implicit_supported.argtypes = [i64, i, i, i, i, i]
+    lib.amr_lut_conv_forward_implicit_workspace_bytes.argtypes = [i64, i, i, i, i, i, i, i]
+    lib.amr_lut_conv_forward_implicit_workspace_bytes.restype = sz
+    assert lib.amr_lut_conv_forward_implicit_supported(17408, 512, 64, 32, 32, 64) == 1
+    assert lib.amr_lut_conv_forward_implicit_supported(17408, 512, 24, 32, 32, 64) == 0      # channels no multiple of 16
+    assert lib.amr_lut_conv_forward_implicit_supported(66306, 512, 64, 32, 32, 64) == 0      # 8-bit table
+    assert lib.amr_lut_conv_forward_implicit_supported(17408, 4, 64, 32, 32, 64) == 0        # too few rows to fill the device without a K split
+    assert lib.amr_lut_conv_forward_implicit_supported(17000, 512, 64, 32, 32, 64) == 0      # not a padded table length
+    e_bytes = 256 + 2 * 144 * 32768
+    assert lib.amr_lut_conv_forward_implicit_workspace_bytes(17408, 512, 64, 32, 32, 64, 0, 0) == e_bytes
+    assert lib.amr_lut_conv_forward_implicit_workspace_bytes(17408, 512, 64, 32, 32, 64, 1, 0) == 0
+    assert lib.amr_lut_conv_forward_implicit_workspace_bytes(17408, 512, 64, 32, 32, 64, 1, 1) == 512 * 1024 * 64 * 4
+    lib.amr_lut_conv_forward_implicit_f32.argtypes = [vp, ctypes.c_uint64, vp, vp, vp, i64, i, i, i, i, i] + [vp] * 10 + [vp, sz, vp]
+    icall = lambda elems, B, C: lib.amr_lut_conv_forward_implicit_f32(None, 0, None, None, None, elems, B, C, 32, 32, 64, *([None] * 10), None, 0, None)
+    assert icall(17000, 512, 64) == -2             # not a padded table length
+    assert icall(17408, 0, 64) == -1               # empty batch is a bad shape here
+    assert icall(17408, 512, 24) == -4             # unsupported geometry
+    assert icall(17408, 512, 64) == -1             # null pointers
     lib.amr_conv_weight_prepare_f32.argtypes = [vp, vp, vp, f, vp, vp, vp, vp, i, i, i, i, vp]
     assert lib.amr_conv_weight_prepare_f32(*([None] * 3), 127.0, *([None] * 4), 8, 4, 81, 16, None) == -1     # more than 64 taps
     assert lib.amr_conv_weight_prepare_f32(*([None] * 3), 300.0, *([None] * 4), 8, 4, 9, 16, None) == -1      # codes must fit a byte
