@@ -143,7 +143,7 @@ def training_step(torch, dev, tables, bits, batch=512, steps=10):
     The LUT GEMM's share of a step's GPU time is measured in this run, on three further steps outside the timed ones: HIP
     events on the launch stream around every call of the library's forward and backward LUT entry points (table expansion,
     header, finish and gated launches included; the forward call includes the dequantising store, the convolution-shaped
-    gradA the finishing of the input gradient), summed, over the events around the whole steps."""
+    gradA the finishing of the input gradient), summed, over the wall-clock time of a timed step (GPU-bound)."""
     import app_train
     import approx_ops as native
     from self_ops.ops_py import approx_ops as ops
@@ -189,12 +189,27 @@ def training_step(torch, dev, tables, bits, batch=512, steps=10):
         for n in names:
             setattr(native, n, originals[n])
     lut_ms = sum(a.elapsed_time(b) for a, b in spans)
+    # the same network in evaluation mode (frozen ranges and weights, no graph): forward passes of one batch, wall clock
+    model.eval()
+    with torch.no_grad():
+        for _ in range(2):
+            model(xs[0])
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            model(xs[0])
+        torch.cuda.synchronize()
+        eval_dt = time.perf_counter() - t0
     return {"workload": f"resnet18_cifar_b{batch}_{bits}bit full step: forward, cross-entropy, backward, SGD (BASELINE.json configs[4])",
             "steps": steps, "ms_per_step": dt / steps * 1e3, "images_per_s": batch * steps / dt,
             "loss_first_last": [float(losses[0]), float(losses[-1])],
-            "lut_gemm_share_of_gpu_time": lut_ms / s0.elapsed_time(s1),
+            "lut_gemm_share_of_gpu_time": (lut_ms / share_steps) / (dt / steps * 1e3),
             "lut_gemm_ms_per_step": lut_ms / share_steps,
-            "share_source": f"measured in this run: HIP events around the {len(spans) // share_steps} library GEMM calls of a step, {share_steps} steps"}
+            "share_source": f"measured in this run: HIP events around the {len(spans) // share_steps} library GEMM calls of a step, {share_steps} steps, "
+                            "over the wall-clock time of the timed steps (the step is bound by the GPU; the steps that carry the events run "
+                            f"{s0.elapsed_time(s1) / share_steps:.1f} ms each, stretched by the event records, and are not the denominator)",
+            "eval_forward": {"ms_per_batch": eval_dt / steps * 1e3, "images_per_s": batch * steps / eval_dt,
+                             "note": "evaluation mode, no graph: expansions kept per layer, 3x3 layers without a window matrix"}}
 
 
 def eight_bit_step(torch, np, dev, lib, O, stream, float_tables, steps=5):
