@@ -285,10 +285,16 @@ class _ApproxConvLayerFn(torch.autograd.Function):
         g = g.contiguous()
         dev = g.device
         g_x = g_w = g_wr = g_bias = None
+        g_z = None
         if need_x or need_w:
             g_rows = torch.empty((bn * oh * ow, cout), dtype=torch.float32, device=dev)
             t = torch.empty(bn * oh * ow, dtype=torch.float32, device=dev)
-            approx_ops.conv_dequant_backward_rowsum(g, s_a, s_w, g_rows, t)
+            if need_wr and fused_w:
+                # (with the gradient of the zero-point term Za * w_resp folded onto the taps, from the same pass over g where it can be)
+                g_z = torch.empty((approx_ops.conv_zero_point_grad_parts(oh * ow), cout, kh * kw), dtype=torch.float32, device=dev)
+                approx_ops.conv_output_grad(g, z_a, s_a, s_w, tapmask, g_rows, t, g_z)
+            else:
+                approx_ops.conv_dequant_backward_rowsum(g, s_a, s_w, g_rows, t)
             # (a gradient nobody asked for -- the images in front of the first layer -- is not computed)
             conv_shaped = codes is not None and need_x
             g_a = torch.empty((bn, kh * kw * cin, oh * ow), dtype=torch.float32, device=dev) if need_x and not conv_shaped else None
@@ -305,9 +311,7 @@ class _ApproxConvLayerFn(torch.autograd.Function):
             if need_w and not fused_w:
                 g_w = g_b.view(kh, kw, cin, cout).permute(3, 2, 0, 1)
         if need_wr and fused_w:
-            # gradient of the zero-point term Za * w_resp, then everything that ends in the real weight in one launch
-            g_z = torch.empty((approx_ops.conv_zero_point_grad_parts(oh * ow), cout, kh * kw), dtype=torch.float32, device=dev)
-            approx_ops.conv_zero_point_grad(g, z_a, s_a, s_w, tapmask, g_z)
+            # everything that ends in the real weight in one launch: LUT gradient + zero-point term, mask, weight scale
             g_w = torch.empty((cout, cin, kh, kw), dtype=torch.float32, device=dev)
             approx_ops.conv_weight_grad(g_b, g_z, inside_w, s_w, g_w)
         elif need_wr:

@@ -75,6 +75,9 @@ _lib.amr_conv_zero_point_grad_workspace_bytes.argtypes = [_i, _i, _i]
 _lib.amr_conv_zero_point_grad_workspace_bytes.restype = _sz
 _lib.amr_conv_zero_point_grad_f32.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _sz, _vp]
 _lib.amr_conv_zero_point_grad_parts.argtypes = [_i]
+_lib.amr_conv_output_grad_workspace_bytes.argtypes = [_i, _i, _i]
+_lib.amr_conv_output_grad_workspace_bytes.restype = _sz
+_lib.amr_conv_output_grad_f32.argtypes = [_vp] * 8 + [_i, _i, _i, _i, _vp, _sz, _vp]
 _lib.amr_conv_weight_grad_f32.argtypes = [_vp, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _vp]
 _lib.amr_quantize_codes_nhwc_u8.argtypes = [_vp, _vp, _vp, ctypes.c_float, _vp, _vp, _vp, _i, _i, _i, _vp]
 _lib.amr_im2col_nhwc_u8.argtypes = [_vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp]
@@ -731,6 +734,39 @@ def conv_dequant_backward_rowsum(g_tensor, s_a, s_w, gc_rows, t_tensor):
         rc = _lib.amr_conv_dequant_backward_rowsum_f32(g_tensor.data_ptr(), s_a.data_ptr(), s_w.data_ptr(), gc_rows.data_ptr(),
                                                        t_tensor.data_ptr(), Bn, N, L, _stream_ptr(dev))
     _raise_for(rc, "conv_dequant_backward_rowsum")
+
+
+def conv_output_grad(g_tensor, z_a, s_a, s_w, tapmask, gc_rows, t_tensor, gz_tensor):
+    """conv_dequant_backward_rowsum and conv_zero_point_grad (without its optional output) in one call: the output gradient
+    is read once where the geometry allows.  tapmask and gz_tensor may both be None (then only gc_rows and t are written)."""
+    tensors = [(g_tensor, "g_tensor"), (s_a, "s_a"), (s_w, "s_w"), (gc_rows, "gc_rows"), (t_tensor, "t_tensor")]
+    _check((tapmask is None) == (gz_tensor is None), "tapmask and gz_tensor go together")
+    if tapmask is not None:
+        tensors += [(z_a, "z_a"), (tapmask, "tapmask"), (gz_tensor, "gz_tensor")]
+    for t, name in tensors:
+        _check_input(t, torch.float32, name)
+    _check(g_tensor.dim() == 4 and gc_rows.dim() == 2, "g must be 4-D and gc_rows 2-D")
+    Bn, N = g_tensor.size(0), g_tensor.size(1)
+    L = g_tensor.size(2) * g_tensor.size(3)
+    _check(tuple(gc_rows.shape) == (Bn * L, N), f"gc_rows's shape should be {Bn * L} x {N}")
+    _check(t_tensor.numel() == Bn * L, f"t_tensor should have {Bn * L} elements")
+    T = 0
+    if tapmask is not None:
+        T = tapmask.size(0)
+        parts = _lib.amr_conv_zero_point_grad_parts(L)
+        _check(tapmask.dim() == 2 and tapmask.size(1) == L and T <= 64, f"tapmask should be [taps <= 64, {L}]")
+        _check(tuple(gz_tensor.shape) == (parts, N, T), f"gz_tensor's shape should be {parts} x {N} x {T}")
+        _check(all(t.numel() == 1 for t in (z_a, s_a, s_w)), "z_a, s_a and s_w must hold one element")
+    dev = g_tensor.device
+    _check(all(t.device == dev for t, _ in tensors), "All tensors should be on the same device")
+    with torch.cuda.device(dev):
+        need = _lib.amr_conv_output_grad_workspace_bytes(Bn, N, L) if tapmask is not None else 0
+        ws = torch.empty(max(need, 16), dtype=torch.uint8, device=dev) if need else None
+        rc = _lib.amr_conv_output_grad_f32(g_tensor.data_ptr(), z_a.data_ptr() if tapmask is not None else None, s_a.data_ptr(), s_w.data_ptr(),
+                                           tapmask.data_ptr() if tapmask is not None else None, gc_rows.data_ptr(), t_tensor.data_ptr(),
+                                           gz_tensor.data_ptr() if gz_tensor is not None else None, Bn, N, L, T,
+                                           ws.data_ptr() if ws is not None else None, need, _stream_ptr(dev))
+    _raise_for(rc, "conv_output_grad")
 
 
 def lds_gather_probe(pattern=0, waves_per_cu=16, iters=4000):

@@ -119,6 +119,9 @@ int batch_sum_segments(int B, size_t inner, int n_cu);
 hipError_t launch_batch_sum_taps(const float* g, const float* za, const float* sa, const float* sw, const float* tapmask, float* g_wr,
                                  float* gz, float* partial, int B, int N, int L, int T, int n_cu, hipStream_t stream);
 int batch_sum_parts(int L);
+int output_grad_segments(int B, int N, int L, int n_cu, bool* fused);
+hipError_t launch_output_grad(const float* g, const float* za, const float* sa, const float* sw, const float* tapmask, float* gc, float* t,
+                              float* gz, float* partial, int B, int N, int L, int T, int n_cu, hipStream_t stream);
 hipError_t launch_conv_weight_grad(const float* gBt, const float* gz, int parts, const uint8_t* inside, const float* scale, float* gw,
                                    int N, int C, int T, int n_cu, hipStream_t stream);
 hipError_t launch_poison_if_raised(float* gx, size_t total, const uint32_t* gate, hipStream_t stream);
@@ -1129,6 +1132,35 @@ int amr_conv_dequant_backward_rowsum_f32(const float* g, const float* s_a, const
     hipError_t e = amr::launch_dequant_grad_rowsum(g, s_a, s_w, g_c, t, batch * positions, out_channels, positions,
                                                    reinterpret_cast<hipStream_t>(stream));
     return e == hipSuccess ? AMR_OK : hip_fail(e, "dequant backward launch");
+}
+
+size_t amr_conv_output_grad_workspace_bytes(int batch, int out_channels, int positions) {
+    if (batch <= 0 || out_channels <= 0 || positions <= 0) return 0;
+    const int n_cu = current_device_cus(nullptr);
+    bool fused = false;
+    const int segs = amr::output_grad_segments(batch, out_channels, positions, n_cu > 0 ? n_cu : 256, &fused);
+    return (size_t)segs * out_channels * positions * sizeof(float);
+}
+
+int amr_conv_output_grad_f32(const float* g, const float* z_a, const float* s_a, const float* s_w, const float* tapmask, float* g_c, float* t,
+                             float* gz, int batch, int out_channels, int positions, int taps, void* workspace, size_t workspace_bytes,
+                             void* stream) {
+    if (batch <= 0 || out_channels <= 0 || positions <= 0) return fail(AMR_EINVAL, "bad shape");
+    if ((long)batch * positions >= (1L << 31)) return fail(AMR_EUNSUPPORTED, "more than 2^31 output positions");
+    if (!g || !s_a || !s_w || !g_c || !t) return fail(AMR_EINVAL, "null pointer argument");
+    if ((tapmask != nullptr) != (gz != nullptr)) return fail(AMR_EINVAL, "tapmask and gz go together");
+    const int n_cu = current_device_cus(nullptr);
+    if (n_cu <= 0) return fail(AMR_EINVAL, "no HIP device available");
+    if (tapmask) {
+        if (taps <= 0 || taps > 64 || !z_a) return fail(AMR_EINVAL, "bad tap count (at most 64) or null z_a");
+        const size_t need = amr_conv_output_grad_workspace_bytes(batch, out_channels, positions);
+        if (!workspace || workspace_bytes < need)
+            return fail(AMR_EWORKSPACE, "workspace of %zu bytes is smaller than the %zu required", workspace ? workspace_bytes : (size_t)0, need);
+        if (((uintptr_t)workspace | (uintptr_t)g) & 15) return fail(AMR_EINVAL, "g and workspace must be 16-byte aligned");
+    }
+    hipError_t e = amr::launch_output_grad(g, z_a, s_a, s_w, tapmask, g_c, t, gz, reinterpret_cast<float*>(workspace), batch, out_channels,
+                                           positions, taps, n_cu, reinterpret_cast<hipStream_t>(stream));
+    return e == hipSuccess ? AMR_OK : hip_fail(e, "output gradient launch");
 }
 
 int amr_acc_gemm_forward_fp32(const float* A, const float* B, float* C, int M, int K, int N, void* stream) {

@@ -419,7 +419,7 @@ hipError_t launch_conv_weight_prepare(const float* w, const float* scale, const 
 
 // Gradient of the zero-point term Za * w_resp, summed over the batch and folded onto the taps:
 //   g_wr[n][pos] = (*z_a * (*s_a * *s_w)) * sum over b of g[b][n][pos]
-//   gz[p][n][tap] = sum over the positions pos of block p (256 positions each) of g_wr[n][pos] * tapmask[tap][pos]
+//   gz[p][n][tap] = sum over the positions pos of block p (64 positions each) of g_wr[n][pos] * tapmask[tap][pos]
 // (the consumer, the weight-gradient kernel below, adds the blocks in ascending order).  Two launches, fixed summation order.  First S segments of the batch into partial sums (a thread owns four neighbouring
 // elements and walks its segment with four loads in flight); then one workgroup per output channel n and block of positions adds the
 // segments in ascending order (threads side by side along the positions, segment lanes beside them when the block is
@@ -451,7 +451,7 @@ __global__ __launch_bounds__(256) void batch_sum_partial_kernel(const float* __r
     }
 }
 
-constexpr int kBsChunk = 256;       // positions of one channel per workgroup of the folding kernel
+constexpr int kBsChunk = 64;        // positions of one channel per workgroup of the folding kernel (four lanes of segments beside them)
 __global__ __launch_bounds__(256) void batch_sum_taps_kernel(const float* __restrict__ partial, const float* __restrict__ za_p,
                                                              const float* __restrict__ sa_p, const float* __restrict__ sw_p,
                                                              const float* __restrict__ tapmask, float* __restrict__ g_wr,
@@ -462,7 +462,7 @@ __global__ __launch_bounds__(256) void batch_sum_taps_kernel(const float* __rest
     const int p0 = blockIdx.y * kBsChunk;
     const int cn = min(kBsChunk, L - p0);
     const float scale = __fmul_rn(*za_p, __fmul_rn(*sa_p, *sw_p));
-    // P threads along the positions (a power of two, 16..256), SP = 256 / P lanes of segments beside them
+    // P threads along the positions (a power of two, 16..64), SP = 256 / P lanes of segments beside them
     int P = 16;
     while (P < cn) P <<= 1;
     const int SP = 256 / P;
@@ -638,6 +638,116 @@ __global__ __launch_bounds__(256) void dequant_grad_rowsum_kernel(const float* _
     }
     __syncthreads();
     if (threadIdx.x < 128 && m0 + (int)threadIdx.x < M) t[m0 + threadIdx.x] = rsum[threadIdx.x];
+}
+
+// The same with the batch sums of the zero-point gradient formed on the way (L % 128 == 0, N <= 32 NB): a workgroup owns 128
+// positions and a segment of the batch, walks its images one after the other and keeps, per thread, the sums over those
+// images of the 16 NB elements it loads per image; partial[seg][n][pos] is what batch_sum_partial_kernel would have written
+// (raw sums of g, images in ascending order), so that the output gradient is read once instead of twice.
+template <int NB>
+__global__ __launch_bounds__(256) void dequant_grad_rowsum_batch_kernel(const float* __restrict__ g, const float* __restrict__ sa_p,
+                                                                        const float* __restrict__ sw_p, float* __restrict__ gc,
+                                                                        float* __restrict__ t, float* __restrict__ partial, int B, int N,
+                                                                        int L, int seg_len) {
+    __shared__ float tile[4][32][33];
+    __shared__ float rsum[128];
+    const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+    const int p0 = blockIdx.x * 128;
+    const int b0 = blockIdx.y * seg_len, b1 = min(B, b0 + seg_len);
+    const float s = __fmul_rn(*sa_p, *sw_p);
+    float acc[NB][4][4];
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int tt = 0; tt < 4; ++tt)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) acc[nb][tt][r] = 0.f;
+    for (int b = b0; b < b1; ++b) {
+        const size_t m0 = (size_t)b * L + p0;
+        if (threadIdx.x < 128) rsum[threadIdx.x] = 0.f;
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+            const int n0 = 32 * nb;
+            float v[4][4];
+#pragma unroll
+            for (int tt = 0; tt < 4; ++tt)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int n = min(n0 + ty + 8 * r, N - 1);
+                    v[tt][r] = g[((size_t)b * N + n) * L + p0 + 32 * tt + tx];
+                }
+            __syncthreads();                      // the previous block's tiles have been read
+#pragma unroll
+            for (int tt = 0; tt < 4; ++tt)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    acc[nb][tt][r] += v[tt][r];
+                    tile[tt][tx][ty + 8 * r] = __fmul_rn(s, v[tt][r]);
+                }
+            __syncthreads();
+#pragma unroll
+            for (int tt = 0; tt < 4; ++tt)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int n = n0 + tx;
+                    if (n < N) gc[(m0 + 32 * tt + ty + 8 * r) * N + n] = tile[tt][ty + 8 * r][tx];
+                }
+            if (threadIdx.x < 128) {
+                const int tt = threadIdx.x >> 5, row = threadIdx.x & 31;
+                float a = rsum[threadIdx.x];
+                const int nn = min(32, N - n0);
+                for (int e = 0; e < nn; ++e) a += tile[tt][row][e];
+                rsum[threadIdx.x] = a;
+            }
+        }
+        if (threadIdx.x < 128) t[m0 + threadIdx.x] = rsum[threadIdx.x];
+    }
+    float* out = partial + (size_t)blockIdx.y * N * L;
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int tt = 0; tt < 4; ++tt)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int n = 32 * nb + ty + 8 * r;
+                if (n < N) out[(size_t)n * L + p0 + 32 * tt + tx] = acc[nb][tt][r];
+            }
+}
+
+// Segments of the batch for the sums of the zero-point gradient, and whether the rows kernel forms them on the way.
+int output_grad_segments(int B, int N, int L, int n_cu, bool* fused) {
+    *fused = (L % 128) == 0 && N <= 128 && B >= 8;
+    if (!*fused) return batch_sum_segments(B, (size_t)N * L, n_cu);
+    const int pos_blocks = L / 128;
+    int segs = (2 * n_cu + pos_blocks - 1) / pos_blocks;
+    if (segs > B / 4) segs = B / 4;
+    if (segs > 128) segs = 128;
+    return segs < 1 ? 1 : segs;
+}
+
+// g_rows, t and (tapmask != nullptr) gz of one layer's output gradient: two launches where the rows kernel can form the
+// batch sums, three otherwise.
+hipError_t launch_output_grad(const float* g, const float* za, const float* sa, const float* sw, const float* tapmask, float* gc, float* t,
+                              float* gz, float* partial, int B, int N, int L, int T, int n_cu, hipStream_t stream) {
+    bool fused = false;
+    const int segs = output_grad_segments(B, N, L, n_cu, &fused);
+    if (!tapmask || !fused) {
+        hipLaunchKernelGGL(dequant_grad_rowsum_kernel, dim3((B * L + 127) / 128), dim3(256), 0, stream, g, sa, sw, gc, t, B * L, N, L);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess || !tapmask) return e;
+        return launch_batch_sum_taps(g, za, sa, sw, tapmask, nullptr, gz, partial, B, N, L, T, n_cu, stream);
+    }
+    const int seg_len = (B + segs - 1) / segs;
+    const int used = (B + seg_len - 1) / seg_len;
+    const dim3 grid(L / 128, used);
+    if (N <= 32) hipLaunchKernelGGL((dequant_grad_rowsum_batch_kernel<1>), grid, dim3(256), 0, stream, g, sa, sw, gc, t, partial, B, N, L, seg_len);
+    else if (N <= 64) hipLaunchKernelGGL((dequant_grad_rowsum_batch_kernel<2>), grid, dim3(256), 0, stream, g, sa, sw, gc, t, partial, B, N, L, seg_len);
+    else hipLaunchKernelGGL((dequant_grad_rowsum_batch_kernel<4>), grid, dim3(256), 0, stream, g, sa, sw, gc, t, partial, B, N, L, seg_len);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(batch_sum_taps_kernel, dim3(N, batch_sum_parts(L)), dim3(256), 0, stream, partial, za, sa, sw, tapmask, (float*)nullptr, gz,
+                       (size_t)N * L, N, L, T, used);
+    return hipGetLastError();
 }
 
 hipError_t launch_dequant_grad_rowsum(const float* g, const float* sa, const float* sw, float* gc, float* t, int M, int N, int L,

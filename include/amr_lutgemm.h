@@ -378,6 +378,18 @@ int amr_conv_weight_grad_f32(const float *gBt, const float *gz, int gz_parts, co
                              int N, int C, int taps, void *stream);
 
 /*
+ * Everything the backward pass of the layer derives from the output gradient g [B][N][L] alone, in one call:
+ * g_c and t of amr_conv_dequant_backward_rowsum_f32 and, with tapmask and gz given, gz of amr_conv_zero_point_grad_f32 (same
+ * values; no g_wr).  Where the geometry allows (L a multiple of 128, N <= 128) the batch sums behind gz are formed by the
+ * kernel that writes g_c, so that g is read once.  workspace: amr_conv_output_grad_workspace_bytes bytes, 16-byte aligned
+ * (only needed with gz).
+ */
+size_t amr_conv_output_grad_workspace_bytes(int batch, int out_channels, int positions);
+int amr_conv_output_grad_f32(const float *g, const float *z_a, const float *s_a, const float *s_w, const float *tapmask, float *g_c,
+                             float *t, float *gz, int batch, int out_channels, int positions, int taps, void *workspace,
+                             size_t workspace_bytes, void *stream);
+
+/*
  * Input gradient of a quantised 3x3 LUT convolution of stride 1 and padding 1 WITHOUT the [M][9C] gradient matrix: gradA of
  * amr_lut_gemm_backward_ex, amr_col2im_f32 and amr_conv_input_grad_f32 as one implicit GEMM over the B*H*W input pixels,
  *   gx[b,c,y,x] = inside[b,c,y,x] ? ((1/16) * sum over taps (ti,tj) and n of gC[(b, y+1-ti, x+1-tj), n] *

@@ -266,7 +266,7 @@ def test_zero_point_gradient_of_a_large_batch_and_ragged_sizes(ops):
         mask = (torch.rand(T, L, device="cuda", generator=g) < 0.8).float()
         gwr = torch.empty(n, L, device="cuda")
         parts = approx_ops.conv_zero_point_grad_parts(L)
-        assert parts == (L + 255) // 256
+        assert parts == (L + 63) // 64
         gz = torch.empty(parts, n, T, device="cuda")
         approx_ops.conv_zero_point_grad(x, one(2.0), one(0.5), one(3.0), mask, gz, gwr)
         want = 3.0 * x.double().sum(dim=0)
@@ -275,6 +275,41 @@ def test_zero_point_gradient_of_a_large_batch_and_ragged_sizes(ops):
         again = torch.empty_like(gz)
         approx_ops.conv_zero_point_grad(x, one(2.0), one(0.5), one(3.0), mask, again)
         assert torch.equal(gz, again)                       # fixed summation order
+
+
+@pytest.mark.parametrize("bn,n,hw,T", [(37, 64, (32, 32), 9), (16, 128, (16, 16), 9), (9, 40, (16, 8), 1), (64, 32, (16, 16), 49),
+                                       (5, 64, (32, 32), 9), (12, 256, (16, 16), 9), (20, 64, (8, 8), 9), (3, 7, (5, 5), 4)])
+def test_output_gradient_side_in_one_call(ops, bn, n, hw, T):
+    """conv_output_grad (rows + row sums + zero-point gradient on the taps; the batch sums come out of the rows kernel where
+    positions are a multiple of 128 and there are at most 128 channels) against the two separate calls: identical rows and
+    row sums, tap sums to summation order and against float64."""
+    import approx_ops
+    print("output gradient side", bn, n, hw, T, flush=True)
+    gen = torch.Generator(device="cuda").manual_seed(bn * 7 + n)
+    L = hw[0] * hw[1]
+    g = torch.randn(bn, n, *hw, device="cuda", generator=gen)
+    mask = (torch.rand(T, L, device="cuda", generator=gen) < 0.8).float()
+    z_a, s_a, s_w = (torch.tensor([v], device="cuda") for v in (-3.0, 0.013, 0.0041))
+    rows0, t0 = torch.empty(bn * L, n, device="cuda"), torch.empty(bn * L, device="cuda")
+    approx_ops.conv_dequant_backward_rowsum(g, s_a, s_w, rows0, t0)
+    parts = approx_ops.conv_zero_point_grad_parts(L)
+    gz0 = torch.empty(parts, n, T, device="cuda")
+    approx_ops.conv_zero_point_grad(g, z_a, s_a, s_w, mask, gz0)
+    rows1, t1 = torch.full_like(rows0, float("nan")), torch.full_like(t0, float("nan"))
+    gz1 = torch.full_like(gz0, float("nan"))
+    approx_ops.conv_output_grad(g, z_a, s_a, s_w, mask, rows1, t1, gz1)
+    assert torch.equal(rows1, rows0) and torch.equal(t1, t0)
+    want = ((z_a * (s_a * s_w)).double() * g.double().sum(dim=0).view(n, L)) @ mask.double().t()
+    bound = 1e-6 * float((g.double().sum(dim=0).abs().view(n, L).sum(dim=1)).max()) * abs(float(z_a * s_a * s_w)) + 1e-12
+    torch.testing.assert_close(gz1.double().sum(dim=0), want, rtol=1e-5, atol=bound)
+    torch.testing.assert_close(gz1.sum(dim=0), gz0.sum(dim=0), rtol=1e-5, atol=bound)
+    again = torch.empty_like(gz1)
+    approx_ops.conv_output_grad(g, z_a, s_a, s_w, mask, torch.empty_like(rows0), torch.empty_like(t0), again)
+    assert torch.equal(again, gz1)                          # fixed summation order
+    # rows and row sums alone
+    rows2, t2 = torch.full_like(rows0, float("nan")), torch.full_like(t0, float("nan"))
+    approx_ops.conv_output_grad(g, None, s_a, s_w, None, rows2, t2, None)
+    assert torch.equal(rows2, rows0) and torch.equal(t2, t0)
 
 
 def test_uint8_layer_path_first_layer_needs_no_input_gradient(ops):

@@ -236,7 +236,15 @@ def test_layer_level_entry_points_check_arguments_without_touching_a_device():
     assert lib.amr_conv_zero_point_grad_f32(*([None] * 7), 0, 4, 10, 9, None, 0, None) == -1
     assert lib.amr_conv_zero_point_grad_f32(*([None] * 7), 4, 4, 10, 65, None, 0, None) == -1                 # more than 64 taps
     assert lib.amr_conv_zero_point_grad_f32(*([None] * 7), 4, 4, 10, 9, None, 0, None) == -1                  # null pointers
-    assert lib.amr_conv_zero_point_grad_parts(1024) == 4 and lib.amr_conv_zero_point_grad_parts(16) == 1 and lib.amr_conv_zero_point_grad_parts(0) == 0
+    assert lib.amr_conv_zero_point_grad_parts(1024) == 16 and lib.amr_conv_zero_point_grad_parts(16) == 1 and lib.amr_conv_zero_point_grad_parts(0) == 0
+    lib.amr_conv_output_grad_workspace_bytes.argtypes = [i, i, i]
+    lib.amr_conv_output_grad_workspace_bytes.restype = sz
+    assert lib.amr_conv_output_grad_workspace_bytes(0, 64, 1024) == 0
+    assert lib.amr_conv_output_grad_workspace_bytes(512, 64, 1024) == 64 * 64 * 1024 * 4          # 64 segments of 8 images
+    assert lib.amr_conv_output_grad_workspace_bytes(512, 512, 16) == lib.amr_conv_zero_point_grad_workspace_bytes(512, 512, 16)
+    lib.amr_conv_output_grad_f32.argtypes = [vp] * 8 + [i, i, i, i, vp, sz, vp]
+    assert lib.amr_conv_output_grad_f32(*([None] * 8), 0, 64, 16, 9, None, 0, None) == -1
+    assert lib.amr_conv_output_grad_f32(*([None] * 8), 4, 64, 16, 9, None, 0, None) == -1                     # null pointers
     lib.amr_conv_weight_grad_f32.argtypes = [vp, vp, i, vp, vp, vp, i, i, i, vp]
     assert lib.amr_conv_weight_grad_f32(None, None, 1, None, None, None, 8, 0, 9, None) == -1
     assert lib.amr_conv_weight_grad_f32(None, None, 0, None, None, None, 8, 4, 9, None) == -1                 # no block of positions
