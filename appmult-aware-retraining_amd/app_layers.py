@@ -76,7 +76,7 @@ def _scale_and_zero_point(observer, quant_max, eps):
     return scale, torch.round(observer.min_val / scale)
 
 
-def _observe(observer, x, quant_max, eps, scale, zp_neg):
+def _observe(observer, x, quant_max, eps, scale, zp_neg, relu=False):
     """One observer step on ``x`` followed by the scale / zero point it implies; returns (scale, zp_neg) as NEW tensors,
     like the reference's ``self.activation_scale = torch.max(...)`` (``app_layers.py:154-160``): an autograd graph built by
     an earlier forward pass keeps the values it saw.  ``scale`` / ``zp_neg`` (the layer's current buffers) only say where the
@@ -88,7 +88,7 @@ def _observe(observer, x, quant_max, eps, scale, zp_neg):
           all(t is not None and t.is_cuda and t.dtype == torch.float32 and t.numel() == 1 and t.is_contiguous()
               for t in (observer.min_val, observer.max_val, scale, zp_neg)))
     if not ok:
-        observer(x)
+        observer(F.relu(x) if relu else x)
         return _scale_and_zero_point(observer, quant_max, eps)
     import approx_ops
     with torch.no_grad():
@@ -106,9 +106,9 @@ def _observe(observer, x, quant_max, eps, scale, zp_neg):
                 state = torch.zeros(approx_ops.MINMAX_STATE_WORDS, dtype=torch.int32, device=x.device)
                 observer.__dict__["_minmax_state"] = state
             approx_ops.observe_minmax(x.detach(), state, observer.min_val, observer.max_val, new_scale, new_zp, mode, momentum,
-                                      float(quant_max), float(eps), inv_qmax)
+                                      float(quant_max), float(eps), inv_qmax, relu=relu)
         else:
-            lo, hi = torch.aminmax(x)
+            lo, hi = torch.aminmax(F.relu(x) if relu else x)
             approx_ops.observer_update(lo.reshape(1), hi.reshape(1), observer.min_val, observer.max_val, new_scale, new_zp, mode,
                                        momentum, float(quant_max), float(eps), inv_qmax)
     return new_scale, new_zp
@@ -217,7 +217,7 @@ class _ApproxConvLayerFn(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, x, w, w_resp, taps, a_scale, a_zp, w_scale, w_zp, bias, a_qmax, stride, padding, dilation, fwd_cache=None,
-                prepared=None, grad_mode=True):
+                prepared=None, grad_mode=True, pre_relu=False):
         import approx_ops
         from self_ops.ops_py import approx_ops as ops
         one = lambda t: t.detach().reshape(1).contiguous()
@@ -232,7 +232,8 @@ class _ApproxConvLayerFn(torch.autograd.Function):
         codes = torch.empty((bn * h * w_in, cin), dtype=torch.uint8, device=dev)
         inside = torch.empty((bn, cin, h, w_in), dtype=torch.uint8, device=dev)
         xs = torch.empty((bn, 1, h, w_in), dtype=torch.float32, device=dev)
-        approx_ops.quantize_codes_nhwc(xc, s_a, z_a, a_qmax, codes, inside, xs)
+        # (pre_relu: the layer's input is max(x, 0); `inside` then carries the ReLU's backward mask as well)
+        approx_ops.quantize_codes_nhwc(xc, s_a, z_a, a_qmax, codes, inside, xs, relu=pre_relu)
         # a 3x3 / stride 1 / padding 1 layer takes its input gradient from one implicit GEMM over the input pixels (no
         # [M][9C] gradient matrix, no col2im) where the library serves the shape and the gradient table fits halves
         same3x3 = (kh, kw, s, p, d) == (3, 3, 1, 1, 1)
@@ -318,7 +319,7 @@ class _ApproxConvLayerFn(torch.autograd.Function):
             g_wr = ((z_a * (s_a * s_w)) * g.sum(dim=0, keepdim=True)).reshape(wr_shape)
         if has_bias and ctx.needs_input_grad[8]:
             g_bias = g.sum(dim=(0, 2, 3))
-        return g_x, g_w, g_wr, None, None, None, None, None, g_bias, None, None, None, None, None, None, None
+        return g_x, g_w, g_wr, None, None, None, None, None, g_bias, None, None, None, None, None, None, None, None
 
 
 # ------------------------------------------------------------------------------------------ quantiser module
@@ -357,11 +358,12 @@ class _QuantParamsMixin:
         self.register_buffer("weight_scale", torch.ones(1, dtype=torch.float32))
         self.register_buffer("weight_zp_neg", torch.zeros(1, dtype=torch.float32))
 
-    def _update_ranges(self, input):
+    def _update_ranges(self, input, relu=False):
         if self.training:
             self.__dict__["_range_epoch"] = self.__dict__.get("_range_epoch", 0) + 1     # (the quantisation parameters may move)
             self.activation_scale, self.activation_zp_neg = _observe(
-                self.activation_observer, input, self.activation_quant_max, self.eps, self.activation_scale, self.activation_zp_neg)
+                self.activation_observer, input, self.activation_quant_max, self.eps, self.activation_scale, self.activation_zp_neg,
+                relu=relu)
             self.weight_scale, self.weight_zp_neg = _observe(
                 self.weight_observer, self.weight, self.weight_quant_max, self.eps, self.weight_scale, self.weight_zp_neg)
 
@@ -423,6 +425,7 @@ class ApproxConv2d(nn.Conv2d, _QuantParamsMixin):
         self.fused_layer = True                     # False: float32 code tensors between quantiser, convolution and dequantisation
         self.keep_expansion_in_eval = True          # evaluation mode: the forward table expanded along the weight codes stays on the device
         self.fused_weight_side = True               # False: weight codes, their all-ones response and their gradients as torch operators
+        self.pre_relu = False                       # True: the layer computes conv(max(input, 0)) -- a ReLU in front folded into its quantiser
 
     def quantize_v2(self, x, s, zpn, qmax):
         return _to_codes(x, s, zpn, qmax)
@@ -516,23 +519,27 @@ class ApproxConv2d(nn.Conv2d, _QuantParamsMixin):
         return prepared, masks[tkey]
 
     def forward(self, input):
-        self._update_ranges(input)
+        uint8_path = self._takes_uint8_path(input)
+        if self.pre_relu and not uint8_path:
+            input = F.relu(input)                    # (the paths on float32 codes take the ReLU as its own operator)
+        relu = self.pre_relu and uint8_path
+        self._update_ranges(input, relu=relu)
         conv_args = dict(bias=None, stride=self.stride, padding=self.padding, dilation=self.dilation, groups=self.groups)
-        if (self.fused_weight_side and self._takes_uint8_path(input) and float(self.weight_quant_max) <= 255
+        if (self.fused_weight_side and uint8_path and float(self.weight_quant_max) <= 255
                 and self.kernel_size[0] * self.kernel_size[1] <= 64):
             frozen = self._frozen_weight_cache()
             prepared, taps = self._prepared_weight_side(input, frozen)
             return _ApproxConvLayerFn.apply(input, self.weight, None, taps, self.activation_scale, self.activation_zp_neg,
                                             self.weight_scale, self.weight_zp_neg, self.bias, float(self.activation_quant_max),
                                             tuple(self.stride), tuple(self.padding), tuple(self.dilation), frozen, prepared,
-                                            torch.is_grad_enabled())
+                                            torch.is_grad_enabled(), relu)
         w_codes = self.quantize_v2(self.weight, self.weight_scale, self.weight_zp_neg, self.weight_quant_max)
-        if self._takes_uint8_path(input):
+        if uint8_path:
             w_resp, taps = self._weight_zero_point_parts(w_codes, input.shape[1:], conv_args, torch.float32, input.device)
             return _ApproxConvLayerFn.apply(input, w_codes, w_resp, taps, self.activation_scale, self.activation_zp_neg,
                                             self.weight_scale, self.weight_zp_neg, self.bias, float(self.activation_quant_max),
                                             tuple(self.stride), tuple(self.padding), tuple(self.dilation), self._frozen_weight_cache(),
-                                            None, torch.is_grad_enabled())
+                                            None, torch.is_grad_enabled(), relu)
         x_codes = self.quantize_v2(input, self.activation_scale, self.activation_zp_neg, self.activation_quant_max)
         total = self.conv2d_op(x_codes, w_codes, **conv_args)       # approximate products of the codes
         if self.reference_zero_point_terms:
@@ -613,6 +620,24 @@ def add_quant_op(module, a_bits=8, w_bits=8, q_type=0, q_level=0, weight_observe
             if child.bias is not None:
                 new.bias.data = child.bias
         module._modules[name] = new
+
+
+def fold_relu(model):
+    """Inside every ``nn.Sequential`` of ``model``: a ReLU directly in front of an ApproxConv2d is replaced by ``nn.Identity``
+    and the layer takes the ReLU into its quantiser (``pre_relu``): the layer observes and quantises max(x, 0) and its in-range
+    mask carries the ReLU's backward mask, so the ReLU costs no pass over the activation in either direction.  Same values
+    and gradients as the two modules (in a Sequential the ReLU's output has no other reader).  Returns the number of ReLUs
+    folded.  An addition to the reference's ``prepare``; call it on a prepared model."""
+    folded = 0
+    for m in model.modules():
+        if isinstance(m, nn.Sequential):
+            names = list(m._modules.keys())
+            for a, b in zip(names, names[1:]):
+                if isinstance(m._modules[a], nn.ReLU) and isinstance(m._modules[b], ApproxConv2d) and not m._modules[b].pre_relu:
+                    m._modules[a] = nn.Identity()
+                    m._modules[b].pre_relu = True
+                    folded += 1
+    return folded
 
 
 def prepare(model, inplace=False, a_bits=8, w_bits=8, q_type=0, q_level=0, weight_observer=0, bn_fuse=False, bn_fuse_calib=False,

@@ -25,11 +25,14 @@ import models  # noqa: E402
 import self_ops  # noqa: E402
 
 
-def build_model(arch, bits, use_ste_gradient, device, num_classes=10, approx_linear=False):
+def build_model(arch, bits, use_ste_gradient, device, num_classes=10, approx_linear=False, fold_relu=True):
     net = models.resnet18(num_classes) if arch == "resnet18" else models.vgg16(num_classes)
     net = net.to(device)
-    return app_layers.prepare(net, inplace=True, a_bits=bits, w_bits=bits, use_ste_gradient=use_ste_gradient,
-                              approx_linear=approx_linear)
+    net = app_layers.prepare(net, inplace=True, a_bits=bits, w_bits=bits, use_ste_gradient=use_ste_gradient,
+                             approx_linear=approx_linear)
+    if fold_relu:
+        app_layers.fold_relu(net)       # (ReLUs whose only reader is a quantised convolution go into that layer's quantiser)
+    return net
 
 
 @torch.no_grad()

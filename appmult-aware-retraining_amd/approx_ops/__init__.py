@@ -79,6 +79,7 @@ _lib.amr_conv_output_grad_workspace_bytes.argtypes = [_i, _i, _i]
 _lib.amr_conv_output_grad_workspace_bytes.restype = _sz
 _lib.amr_conv_output_grad_f32.argtypes = [_vp] * 8 + [_i, _i, _i, _i, _vp, _sz, _vp]
 _lib.amr_conv_weight_grad_f32.argtypes = [_vp, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _vp]
+_lib.amr_quantize_codes_nhwc_relu_u8.argtypes = [_vp, _vp, _vp, ctypes.c_float, _vp, _vp, _vp, _i, _i, _i, _i, _vp]
 _lib.amr_quantize_codes_nhwc_u8.argtypes = [_vp, _vp, _vp, ctypes.c_float, _vp, _vp, _vp, _i, _i, _i, _vp]
 _lib.amr_im2col_nhwc_u8.argtypes = [_vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp]
 _lib.amr_conv_input_grad_f32.argtypes = [_vp] * 6 + [_i] * 9 + [_vp]
@@ -463,9 +464,10 @@ def observer_update(cur_min, cur_max, min_val, max_val, scale, zp_neg, mode, mom
 MINMAX_STATE_WORDS = 4 + 3 * 1024     # AMR_OBSERVE_STATE_WORDS: int32 words of an observer's state, all zero before the first call
 
 
-def observe_minmax(x_tensor, state_tensor, min_val, max_val, scale, zp_neg, mode, momentum, quant_max, eps, inv_quant_max=0.0):
+def observe_minmax(x_tensor, state_tensor, min_val, max_val, scale, zp_neg, mode, momentum, quant_max, eps, inv_quant_max=0.0,
+                   relu=False):
     """observer_update on the extremes of x_tensor, which the same launch finds (x float32, contiguous; state int32
-    [MINMAX_STATE_WORDS] on the device, zeros before the first call)."""
+    [MINMAX_STATE_WORDS] on the device, zeros before the first call).  relu: the extremes of max(x, 0)."""
     _check_input(x_tensor, torch.float32, "x_tensor")
     _check_input(state_tensor, torch.int32, "state_tensor")
     _check(state_tensor.numel() >= MINMAX_STATE_WORDS and x_tensor.numel() > 0, "state too small, or x empty")
@@ -476,7 +478,7 @@ def observe_minmax(x_tensor, state_tensor, min_val, max_val, scale, zp_neg, mode
     _check(all(t.device == dev for t in (state_tensor, min_val, max_val, scale, zp_neg)), "All tensors should be on the same device")
     with torch.cuda.device(dev):
         rc = _lib.amr_observe_minmax_f32(x_tensor.data_ptr(), x_tensor.numel(), state_tensor.data_ptr(), min_val.data_ptr(),
-                                         max_val.data_ptr(), scale.data_ptr(), zp_neg.data_ptr(), int(mode), float(1 - momentum),
+                                         max_val.data_ptr(), scale.data_ptr(), zp_neg.data_ptr(), int(mode) | (4 if relu else 0), float(1 - momentum),
                                          float(momentum), float(quant_max), float(inv_quant_max), float(eps), _stream_ptr(dev))
     _raise_for(rc, "observe_minmax")
 
@@ -519,10 +521,11 @@ def _conv_out_size(H, W, kh, kw, stride, padding, dilation):
     return oh, ow
 
 
-def quantize_codes_nhwc(x_tensor, scale_tensor, zp_neg_tensor, quant_max, codes_tensor, inside_tensor, xsum_tensor):
+def quantize_codes_nhwc(x_tensor, scale_tensor, zp_neg_tensor, quant_max, codes_tensor, inside_tensor, xsum_tensor, relu=False):
     """The quantiser of the reference's quantize_v2 (micronet+/app_layers.py:147-160) writing what the LUT convolution
     consumes: codes uint8 [B*H*W, C] (a pixel's channel codes adjacent), inside uint8 [B,C,H,W] (the mask of the
-    straight-through backward) and xsum float32 [B*H*W] (a pixel's codes summed over the channels), from x float32 [B,C,H,W]."""
+    straight-through backward) and xsum float32 [B*H*W] (a pixel's codes summed over the channels), from x float32 [B,C,H,W].
+    relu: the quantiser of max(x, 0); inside is then also 0 where x <= 0 (the ReLU's own backward mask)."""
     for t, name, dt in ((x_tensor, "x_tensor", torch.float32), (scale_tensor, "scale_tensor", torch.float32),
                         (zp_neg_tensor, "zp_neg_tensor", torch.float32), (codes_tensor, "codes_tensor", torch.uint8),
                         (inside_tensor, "inside_tensor", torch.uint8), (xsum_tensor, "xsum_tensor", torch.float32)):
@@ -537,9 +540,9 @@ def quantize_codes_nhwc(x_tensor, scale_tensor, zp_neg_tensor, quant_max, codes_
     dev = x_tensor.device
     _check(all(t.device == dev for t in (scale_tensor, zp_neg_tensor, codes_tensor, inside_tensor, xsum_tensor)), "All tensors should be on the same device")
     with torch.cuda.device(dev):
-        rc = _lib.amr_quantize_codes_nhwc_u8(x_tensor.data_ptr(), scale_tensor.data_ptr(), zp_neg_tensor.data_ptr(), float(quant_max),
-                                             codes_tensor.data_ptr(), inside_tensor.data_ptr(), xsum_tensor.data_ptr(), Bn, C, H * W,
-                                             _stream_ptr(dev))
+        rc = _lib.amr_quantize_codes_nhwc_relu_u8(x_tensor.data_ptr(), scale_tensor.data_ptr(), zp_neg_tensor.data_ptr(), float(quant_max),
+                                                  codes_tensor.data_ptr(), inside_tensor.data_ptr(), xsum_tensor.data_ptr(), Bn, C, H * W,
+                                                  1 if relu else 0, _stream_ptr(dev))
     _raise_for(rc, "quantize_codes_nhwc")
 
 

@@ -100,7 +100,7 @@ hipError_t launch_gradA_slab_f32tab(const float* gC, const uint8_t* A, const uin
                                     const LutGeom& g, int M, int K, int N, float scale, int n_cu, uint32_t* flags, void* S,
                                     int rows_per_image, hipStream_t stream);
 hipError_t launch_quantize_nhwc(const float* x, const float* scale, const float* zp_neg, float qmax, uint8_t* codes, uint8_t* inside,
-                                float* xs, long B, int C, int L, hipStream_t stream);
+                                float* xs, long B, int C, int L, hipStream_t stream, int relu);
 hipError_t launch_im2col_nhwc(const uint8_t* codes, uint8_t* A, long B, int C, int H, int W, int kh, int kw, int stride, int pad,
                               int dil, int oh, int ow, hipStream_t stream);
 hipError_t launch_conv_input_grad(const float* cols, const float* t, const float* zw, const uint8_t* inside, const float* scale,
@@ -917,7 +917,8 @@ int amr_observer_update_f32(const float* cur_min, const float* cur_max, float* m
 
 int amr_observe_minmax_f32(const float* x, int64_t n, uint32_t* state, float* min_val, float* max_val, float* scale, float* zp_neg,
                            int mode, float keep, float momentum, float quant_max, float inv_quant_max, float eps, void* stream) {
-    if (mode < 0 || mode > 2 || !(quant_max > 0.f) || n <= 0) return fail(AMR_EINVAL, "bad observer mode, code range or element count");
+    if (mode < 0 || (mode & 3) > 2 || mode > 7 || !(quant_max > 0.f) || n <= 0)
+        return fail(AMR_EINVAL, "bad observer mode, code range or element count");
     if (!x || !state || !min_val || !max_val || !scale || !zp_neg) return fail(AMR_EINVAL, "null pointer argument");
     if ((uintptr_t)state & 3) return fail(AMR_EINVAL, "state must be 4-byte aligned");
     const int n_cu = current_device_cus(nullptr);
@@ -956,11 +957,17 @@ static bool conv_geometry(int C, int H, int W, int kh, int kw, int stride, int p
 
 int amr_quantize_codes_nhwc_u8(const float* x, const float* scale, const float* zp_neg, float qmax, uint8_t* codes, uint8_t* inside,
                                float* x_sum, int B, int C, int L, void* stream) {
+    return amr_quantize_codes_nhwc_relu_u8(x, scale, zp_neg, qmax, codes, inside, x_sum, B, C, L, 0, stream);
+}
+
+int amr_quantize_codes_nhwc_relu_u8(const float* x, const float* scale, const float* zp_neg, float qmax, uint8_t* codes, uint8_t* inside,
+                                    float* x_sum, int B, int C, int L, int relu, void* stream) {
     if (B < 0 || C <= 0 || L <= 0 || !(qmax >= 0.f) || qmax > 255.f) return fail(AMR_EINVAL, "bad shape or code range");
     if (B == 0) return AMR_OK;
     if ((long)B * L >= (1L << 31)) return fail(AMR_EUNSUPPORTED, "more than 2^31 pixels");
     if (!x || !scale || !zp_neg || !codes || !inside || !x_sum) return fail(AMR_EINVAL, "null pointer argument");
-    hipError_t e = amr::launch_quantize_nhwc(x, scale, zp_neg, qmax, codes, inside, x_sum, B, C, L, reinterpret_cast<hipStream_t>(stream));
+    hipError_t e = amr::launch_quantize_nhwc(x, scale, zp_neg, qmax, codes, inside, x_sum, B, C, L, reinterpret_cast<hipStream_t>(stream),
+                                             relu ? 1 : 0);
     return e == hipSuccess ? AMR_OK : hip_fail(e, "quantize launch");
 }
 

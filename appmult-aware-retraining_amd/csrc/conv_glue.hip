@@ -41,7 +41,7 @@ constexpr int kQnCB = 512;
 __global__ __launch_bounds__(256) void quantize_nhwc_kernel(const float* __restrict__ x, const float* __restrict__ scale,
                                                             const float* __restrict__ zp_neg, float qmax,
                                                             uint8_t* __restrict__ codes, uint8_t* __restrict__ inside,
-                                                            float* __restrict__ xs, int C, int L, long M) {
+                                                            float* __restrict__ xs, int C, int L, long M, int relu) {
     extern __shared__ __align__(16) unsigned char smem[];
     __shared__ float part[4][64];
     const float s = *scale, zp = *zp_neg;
@@ -67,7 +67,10 @@ __global__ __launch_bounds__(256) void quantize_nhwc_kernel(const float* __restr
                 const int c = c0 + 4 * u;
                 if (c < cn) {
                     uint32_t in;
-                    const uint32_t code = quant_code_u8(v[u], s, zp, qmax, &in);
+                    // relu: the quantiser of max(x, 0); its backward passes a gradient where x > 0 and the code was in range
+                    const float xv = relu ? (v[u] < 0.f ? 0.f : v[u]) : v[u];
+                    const uint32_t code = quant_code_u8(xv, s, zp, qmax, &in);
+                    if (relu && !(v[u] > 0.f)) in = 0u;
                     smem[lane * pitch + c] = (unsigned char)code;
                     if (live) ip[(size_t)(cb + c) * L] = (unsigned char)in;
                     sum += (float)code;
@@ -96,12 +99,12 @@ __global__ __launch_bounds__(256) void quantize_nhwc_kernel(const float* __restr
 }
 
 hipError_t launch_quantize_nhwc(const float* x, const float* scale, const float* zp_neg, float qmax, uint8_t* codes, uint8_t* inside,
-                                float* xs, long B, int C, int L, hipStream_t stream) {
+                                float* xs, long B, int C, int L, hipStream_t stream, int relu) {
     const long M = B * L;
     const int cn = C < kQnCB ? C : kQnCB;
     const size_t lds = 64 * (size_t)(((cn + 15) & ~15) + 16);
     hipLaunchKernelGGL(quantize_nhwc_kernel, dim3((unsigned)((M + 63) / 64)), dim3(256), lds, stream, x, scale, zp_neg, qmax, codes,
-                       inside, xs, C, L, M);
+                       inside, xs, C, L, M, relu);
     return hipGetLastError();
 }
 

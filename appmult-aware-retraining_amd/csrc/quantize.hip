@@ -181,8 +181,10 @@ __global__ __launch_bounds__(256) void observe_minmax_kernel(const float* __rest
     if (threadIdx.x == 0) {
         float t_lo = fminf(fminf(s_lo[0], s_lo[1]), fminf(s_lo[2], s_lo[3]));
         float t_hi = fmaxf(fmaxf(s_hi[0], s_hi[1]), fmaxf(s_hi[2], s_hi[3]));
+        // (mode bit 2: the extremes of max(x, 0) -- the maximum with zero is monotone, so it is taken on the two results)
+        if (mode & 4) { t_lo = fmaxf(t_lo, 0.f); t_hi = fmaxf(t_hi, 0.f); }
         if (s_nan[0] | s_nan[1] | s_nan[2] | s_nan[3]) t_lo = t_hi = __builtin_nanf("");
-        observer_update_scalars(t_lo, t_hi, min_val, max_val, scale, zp_neg, mode, keep, momentum, qmax, inv_qmax, eps);
+        observer_update_scalars(t_lo, t_hi, min_val, max_val, scale, zp_neg, mode & 3, keep, momentum, qmax, inv_qmax, eps);
         atomicExch(&state[0], 0u);
     }
 }

@@ -300,6 +300,7 @@ int amr_observer_update_f32(const float *cur_min, const float *cur_max, float *m
  * state: AMR_OBSERVE_STATE_WORDS 32-bit words of device memory owned by the caller, one set per observer, all zero before the
  * first call (word 0 counts the workgroups that have finished and is back at zero when the call ends; the others hold their
  * partial results).  Calls that share a state must not overlap in time.
+ * mode | 4: the extremes of max(x, 0) instead of x (an observer behind a ReLU that the caller does not materialise).
  */
 #define AMR_OBSERVE_STATE_WORDS (4 + 3 * 1024)
 int amr_observe_minmax_f32(const float *x, int64_t n, uint32_t *state, float *min_val, float *max_val, float *scale,
@@ -330,6 +331,11 @@ int amr_quantize_codes_backward_f32(const float *g, const float *x, const float 
  */
 int amr_quantize_codes_nhwc_u8(const float *x, const float *scale, const float *zp_neg, float qmax, uint8_t *codes,
                                uint8_t *inside, float *x_sum, int B, int C, int L, void *stream);
+/* relu != 0: the quantiser of max(x, 0) -- a ReLU in front of the layer (as in the reference's networks, micronet+/models.py:103)
+ * without its own pass: codes and x_sum of max(x, 0); inside = 1 where x > 0 AND the rounded value lay in [0, qmax], i.e. the
+ * product of the two backward masks, so that the backward pass of the layer yields the gradient in front of the ReLU. */
+int amr_quantize_codes_nhwc_relu_u8(const float *x, const float *scale, const float *zp_neg, float qmax, uint8_t *codes,
+                                    uint8_t *inside, float *x_sum, int B, int C, int L, int relu, void *stream);
 
 /*
  * im2col of pixel-major codes: A [B*oh*ow, kh*kw*C] uint8, row (b,oy,ox), column (i*kw + j)*C + c ("tap-major": the

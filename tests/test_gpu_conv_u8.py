@@ -312,6 +312,54 @@ def test_output_gradient_side_in_one_call(ops, bn, n, hw, T):
     assert torch.equal(rows2, rows0) and torch.equal(t2, t0)
 
 
+@pytest.mark.parametrize("cin,cout,k,stride,padding,hw,bn", [(16, 24, 3, 1, 1, 12, 4), (64, 64, 3, 1, 1, 16, 16), (5, 7, 3, 2, 1, 9, 3), (32, 40, 1, 1, 0, 8, 4)])
+def test_relu_folded_into_the_layers_quantiser(ops, cin, cout, k, stride, padding, hw, bn):
+    """ApproxConv2d with pre_relu on x against the same layer on relu(x): identical observer state, quantisation parameters
+    and outputs; identical input gradients (the in-range mask carries the ReLU's mask) and weight gradients -- on the uint8
+    path in training and evaluation mode, and on the float-code path (where the layer applies the ReLU as an operator)."""
+    import copy
+    import approx_ops
+    import app_layers as L
+    print("relu fold", cin, cout, k, stride, padding, hw, bn, flush=True)
+    torch.manual_seed(11)
+    plain = L.ApproxConv2d(cin, cout, k, stride=stride, padding=padding, bias=False, a_bits=7, w_bits=7).cuda().train()
+    fold = copy.deepcopy(plain)
+    fold.pre_relu = True
+    x = torch.randn(bn, cin, hw, hw, device="cuda") * 2 - 0.2
+    x.view(-1)[::7] = 0.0                                           # exact zeros: the ReLU passes no gradient there
+    gy = None
+    for mode in ("train", "train", "eval", "float"):
+        if mode == "eval":
+            plain.eval(); fold.eval()
+        if mode == "float":
+            plain.fused_layer = fold.fused_layer = False
+        xa, xb = x.clone().requires_grad_(), x.clone().requires_grad_()
+        plain.zero_grad(); fold.zero_grad()
+        ya = plain(F.relu(xa))
+        yb = fold(xb)
+        if gy is None:
+            gy = torch.randn_like(ya)
+        ya.backward(gy); yb.backward(gy)
+        for name in ("activation_scale", "activation_zp_neg", "weight_scale", "weight_zp_neg"):
+            assert torch.equal(getattr(plain, name), getattr(fold, name)), (mode, name)
+        assert torch.equal(plain.activation_observer.min_val, fold.activation_observer.min_val)
+        assert torch.equal(plain.activation_observer.max_val, fold.activation_observer.max_val)
+        assert float(fold.activation_observer.min_val) >= 0.0
+        assert torch.equal(ya, yb), mode
+        assert torch.equal(xa.grad, xb.grad), mode
+        assert (xb.grad[x <= 0] == 0).all()
+        torch.testing.assert_close(fold.weight.grad, plain.weight.grad, rtol=0, atol=0)
+    # the observer and quantiser entry points by themselves
+    big = torch.randn(3, 8, 33, 31, device="cuda") - 0.5
+    state = torch.zeros(approx_ops.MINMAX_STATE_WORDS, dtype=torch.int32, device="cuda")
+    lo, hi, sc, zp = (torch.zeros(1, device="cuda") for _ in range(4))
+    approx_ops.observe_minmax(big, state, lo, hi, sc, zp, 0, 0.1, 127.0, 1e-7, relu=True)
+    assert float(lo) == 0.0 and float(hi) == float(big.max())
+    neg = -torch.rand(1000, device="cuda") - 1.0
+    approx_ops.observe_minmax(neg, state, lo, hi, sc, zp, 0, 0.1, 127.0, 1e-7, relu=True)
+    assert float(lo) == 0.0 and float(hi) == 0.0
+
+
 def test_uint8_layer_path_first_layer_needs_no_input_gradient(ops):
     import app_layers as L
     torch.manual_seed(1)

@@ -180,6 +180,9 @@ def test_layer_level_entry_points_check_arguments_without_touching_a_device():
     assert lib.amr_quantize_codes_nhwc_u8(None, None, None, 300.0, None, None, None, 2, 3, 4, None) == -1      # codes must fit a byte
     assert lib.amr_quantize_codes_nhwc_u8(None, None, None, 127.0, None, None, None, 0, 3, 4, None) == 0       # empty batch
     assert lib.amr_quantize_codes_nhwc_u8(None, None, None, 127.0, None, None, None, 2, 3, 4, None) == -1      # null pointers
+    lib.amr_quantize_codes_nhwc_relu_u8.argtypes = [vp, vp, vp, f, vp, vp, vp, i, i, i, i, vp]
+    assert lib.amr_quantize_codes_nhwc_relu_u8(None, None, None, 127.0, None, None, None, 2, 3, 4, 1, None) == -1  # null pointers
+    assert lib.amr_quantize_codes_nhwc_relu_u8(None, None, None, 127.0, None, None, None, 0, 3, 4, 1, None) == 0   # empty batch
     lib.amr_im2col_nhwc_u8.argtypes = [vp, vp, i, i, i, i, i, i, i, i, i, vp]
     assert lib.amr_im2col_nhwc_u8(None, None, 2, 3, 4, 4, 5, 5, 1, 0, 1, None) == -1                            # window larger than the image
     assert lib.amr_im2col_nhwc_u8(None, None, 2, 3, 4, 4, 3, 3, 1, 1, 1, None) == -1                            # null pointers
@@ -204,6 +207,8 @@ def test_layer_level_entry_points_check_arguments_without_touching_a_device():
     assert lib.amr_lut_conv_input_grad_f32(*([None] * 4), 17408, *([None] * 5), 512, 64, 32, 32, 64, None, None, None, 0, None) == -1
     lib.amr_observe_minmax_f32.argtypes = [vp, i64, vp, vp, vp, vp, vp, i] + [f] * 5 + [vp]
     assert lib.amr_observe_minmax_f32(None, 10, None, None, None, None, None, 3, 0.9, 0.1, 127.0, 0.0, 1e-7, None) == -1   # mode
+    assert lib.amr_observe_minmax_f32(None, 10, None, None, None, None, None, 7, 0.9, 0.1, 127.0, 0.0, 1e-7, None) == -1   # mode 3 with the ReLU bit
+    assert lib.amr_observe_minmax_f32(None, 10, None, None, None, None, None, 8, 0.9, 0.1, 127.0, 0.0, 1e-7, None) == -1   # unknown bit
     assert lib.amr_observe_minmax_f32(None, 10, None, None, None, None, None, 2, 0.9, 0.1, 127.0, 0.0, 1e-7, None) == -1   # null pointers
     lib.amr_lut_conv_forward_implicit_supported.argtypes = [i64, i, i, i, i, i]
     lib.amr_lut_conv_forward_implicit_workspace_bytes.argtypes = [i64, i, i, i, i, i, i, i]

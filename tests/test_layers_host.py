@@ -104,3 +104,23 @@ def test_benchmark_network_shapes():
     assert sorted(set(convs)) == sorted({(27, 64), (576, 64), (576, 128), (1152, 128), (64, 128), (1152, 256), (2304, 256),
                                          (128, 256), (2304, 512), (4608, 512), (256, 512)})
     assert sum(isinstance(m, nn.Conv2d) for m in models.vgg16().modules()) == 13
+
+
+def test_fold_relu_rewrites_only_relus_whose_reader_is_a_quantised_convolution():
+    """app_layers.fold_relu on the package's networks (structure only: no kernel runs on the CPU)."""
+    import app_layers as L
+    import models
+    net = L.prepare(models.resnet18(10), inplace=True, a_bits=7, w_bits=7)
+    n_relu = sum(isinstance(m, nn.ReLU) for m in net.modules())
+    assert L.fold_relu(net) == 8                                 # the ReLU between the two convolutions of each of the 8 blocks
+    assert sum(isinstance(m, nn.ReLU) for m in net.modules()) == n_relu - 8
+    flagged = [m for m in net.modules() if isinstance(m, L.ApproxConv2d) and m.pre_relu]
+    assert len(flagged) == 8 and all(m.kernel_size == (3, 3) and m.stride == (1, 1) for m in flagged)
+    for blk in (m for m in net.modules() if isinstance(m, models.BasicBlock)):
+        mods = list(blk.residual_function)
+        assert isinstance(mods[2], nn.Identity) and mods[3].pre_relu and not mods[0].pre_relu
+    assert L.fold_relu(net) == 0                                 # nothing left to fold
+    # the ReLU in front of a pooling layer stays
+    seq = nn.Sequential(nn.Conv2d(3, 8, 3), nn.ReLU(), nn.MaxPool2d(2), nn.ReLU(), nn.Conv2d(8, 8, 3))
+    q = L.prepare(seq, inplace=True, a_bits=7, w_bits=7)
+    assert L.fold_relu(q) == 1 and isinstance(q[1], nn.ReLU) and isinstance(q[3], nn.Identity) and q[4].pre_relu
