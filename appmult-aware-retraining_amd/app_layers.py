@@ -208,6 +208,10 @@ class _ApproxConvLayerFn(torch.autograd.Function):
     uint8 im2col; LUT GEMM; zero-point terms, scaling and bias from the GEMM's rows to the NCHW activation.  Backward: the
     output gradient to GEMM rows (with its row sums) in one pass, the two LUT gradient GEMMs, then col2im + gradient of the
     zero-point term + straight-through backward of the quantiser in one pass.  No float32 code tensor exists on this path.
+    A 3x3 / stride 1 / padding 1 layer takes its input gradient from an implicit GEMM over the input pixels and, where no
+    weight gradient will need the window matrix (``grad_mode`` off, frozen weights), its forward pass reads the pixel-major
+    codes itself.  ``pre_relu``: the layer computes the convolution of max(x, 0); the quantiser's mask byte then also holds
+    the ReLU's backward mask, so the gradient returned for ``x`` is the one in front of the ReLU.
 
     The weight side comes in one of two forms.  ``prepared`` = (b_mat uint8 [kh*kw*C, N], inside_w uint8 [N,C,kh,kw],
     w_resp float32 [N, L], tapmask float32 [kh*kw, L]) from ``approx_ops.conv_weight_prepare``: then ``w`` is the layer's real
