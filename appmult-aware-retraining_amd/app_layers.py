@@ -275,6 +275,7 @@ class _ApproxConvLayerFn(torch.autograd.Function):
         ctx.save_for_backward(a_mat, b_mat, inside, s_a, z_a, s_w, z_w, codes if conv_shaped else None, inside_w, tapmask)
         ctx.geo = (bn, cin, h, w_in, cout, kh, kw, s, p, d, oh, ow)
         ctx.aux = (w_resp.shape, bias is not None, x.dtype)
+        ctx.bwd_cache = (fwd_cache[2], fwd_cache[1]) if fwd_cache and len(fwd_cache) > 2 else None
         return out
 
     @staticmethod
@@ -309,7 +310,9 @@ class _ApproxConvLayerFn(torch.autograd.Function):
             if need_x:
                 g_x = torch.empty((bn, cin, h, w), dtype=torch.float32, device=dev)
                 if conv_shaped:
-                    approx_ops.approx_conv_input_grad(g_rows, codes, b_mat, ops.lut_grad_a, t, z_w, inside, s_a, g_x)
+                    bc = ctx.bwd_cache
+                    approx_ops.approx_conv_input_grad(g_rows, codes, b_mat, ops.lut_grad_a, t, z_w, inside, s_a, g_x,
+                                                      cache=bc[0] if bc else None, b_version=bc[1] if bc else 0)
                 else:
                     approx_ops.conv_input_grad(g_a, t, z_w, inside, s_a, g_x, (kh, kw), s, p, d)
                 g_x = g_x.to(x_dtype)
@@ -428,6 +431,8 @@ class ApproxConv2d(nn.Conv2d, _QuantParamsMixin):
         self.fused_dequant = True                   # False: zero-point terms and scaling as torch operators
         self.fused_layer = True                     # False: float32 code tensors between quantiser, convolution and dequantisation
         self.keep_expansion_in_eval = True          # evaluation mode: the forward table expanded along the weight codes stays on the device
+        self.keep_expansions_in_training = False    # True: the expanded forward and input-gradient tables stay on the device in training
+                                                    # mode too (frozen layers, gradient accumulation: weights that outlive a step)
         self.fused_weight_side = True               # False: weight codes, their all-ones response and their gradients as torch operators
         self.pre_relu = False                       # True: the layer computes conv(max(input, 0)) -- a ReLU in front folded into its quantiser
 
@@ -472,16 +477,26 @@ class ApproxConv2d(nn.Conv2d, _QuantParamsMixin):
         """In evaluation mode the weight codes only change when the weights, their quantisation parameters or the tables do:
         the expansion of the forward table along them is then kept on the device between calls (approx_ops.ForwardCache) under a
         number made of everything that could change them.  Training mode: None (the weights move every step)."""
-        if self.training or not self.keep_expansion_in_eval:
+        if not (self.keep_expansions_in_training if self.training else self.keep_expansion_in_eval):
             return None
         import approx_ops
         from self_ops.ops_py import approx_ops as ops
         cache = self.__dict__.get("_fwd_cache")
         if cache is None:
             cache = self.__dict__["_fwd_cache"] = approx_ops.ForwardCache()
-        token = hash((self.weight._version, self.weight.data_ptr(), self.weight_scale._version, self.weight_scale.data_ptr(),
-                      self.weight_zp_neg._version, self.weight_zp_neg.data_ptr(), self.__dict__.get("_range_epoch", 0), ops.table_generation))
-        return cache, token & 0xFFFFFFFFFFFFFFFF
+            self.__dict__["_bwd_cache"] = approx_ops.ForwardCache()      # (the input-gradient table expanded along the same codes)
+        if self.training:
+            # Every training pass leaves NEW scale / zero-point tensors, so their identity says nothing.  The weight observer keeps
+            # running extremes: weights it has already seen (same tensor, same version) give the same parameters again, and with
+            # them the same codes -- the weight alone identifies them.  (Any other kind of weight observer: no caching.)
+            if type(self.weight_observer) is not MinMaxObserver:
+                return None
+            token = hash(("training", self.weight._version, self.weight.data_ptr(), float(self.weight_quant_max), ops.table_generation))
+        else:
+            token = hash((self.weight._version, self.weight.data_ptr(), self.weight_scale._version, self.weight_scale.data_ptr(),
+                          self.weight_zp_neg._version, self.weight_zp_neg.data_ptr(), self.__dict__.get("_range_epoch", 0),
+                          ops.table_generation))
+        return cache, token & 0xFFFFFFFFFFFFFFFF, self.__dict__["_bwd_cache"]
 
     def _takes_uint8_path(self, input):
         """The one-operator path on uint8 codes serves the LUT-gradient convolution of float32 CUDA tensors with square

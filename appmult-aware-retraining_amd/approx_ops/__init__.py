@@ -60,6 +60,9 @@ _lib.amr_lut_conv_input_grad_workspace_bytes.argtypes = [_i64, _i, _i, _i, _i, _
 _lib.amr_lut_conv_input_grad_workspace_bytes.restype = _sz
 _lib.amr_grad_table_fits_halves.argtypes = [_vp, _i64]
 _lib.amr_lut_conv_input_grad_f32.argtypes = [_vp] * 4 + [_i64] + [_vp] * 5 + [_i] * 5 + [_vp, _vp, _vp, _sz, _vp]
+_lib.amr_lut_conv_input_grad_cached_workspace_bytes.argtypes = [_i64, _i, _i, _i, _i, _i]
+_lib.amr_lut_conv_input_grad_cached_workspace_bytes.restype = _sz
+_lib.amr_lut_conv_input_grad_cached_f32.argtypes = [_vp, ctypes.c_uint64] + [_vp] * 4 + [_i64] + [_vp] * 5 + [_i] * 5 + [_vp, _vp, _vp, _sz, _vp]
 _u64 = ctypes.c_uint64
 _lib.amr_fwd_cache_create.argtypes = [ctypes.POINTER(_vp)]
 _lib.amr_fwd_cache_destroy.argtypes = [_vp]
@@ -684,11 +687,12 @@ def conv_input_grad_supported(lut_grad_a_tensor, image_shape, out_channels):
 
 
 def approx_conv_input_grad(gc_rows, codes_tensor, bt_tensor, lut_grad_a_tensor, t_tensor, z_w, inside_tensor, scale_tensor, gx_tensor,
-                           a_fallback=None):
+                           a_fallback=None, cache=None, b_version=0):
     """Input gradient of the quantised 3x3 / stride 1 / padding 1 LUT convolution as one implicit GEMM over the input pixels
     (amr_lut_conv_input_grad_f32): gc_rows float32 [B*H*W, N], codes uint8 [B*H*W, C], bt uint8 [9*C, N] tap-major, gx float32
     [B,C,H,W].  a_fallback: the window matrix uint8 [B*H*W, 9*C]; given, tables that do not fit halves and masked codes are
-    served too (through a scratch of 9*C*B*H*W floats), else such a call yields NaN."""
+    served too (through a scratch of 9*C*B*H*W floats), else such a call yields NaN.  cache (a ForwardCache of its own) and
+    b_version: the gradient table expanded along bt stays on the device between calls, as in approx_gemm_forward."""
     _check_input(gc_rows, torch.float32, "gc_rows")
     _check_input(codes_tensor, torch.uint8, "codes_tensor")
     _check_input(bt_tensor, torch.uint8, "bt_tensor")
@@ -713,9 +717,11 @@ def approx_conv_input_grad(gc_rows, codes_tensor, bt_tensor, lut_grad_a_tensor, 
     with torch.cuda.device(dev):
         if a_fallback is not None:
             cols = torch.empty((Bn, 9 * C, H * W), dtype=torch.float32, device=dev)
-        need = _lib.amr_lut_conv_input_grad_workspace_bytes(lut_grad_a_tensor.numel(), Bn, C, H, W, N)
+        query = _lib.amr_lut_conv_input_grad_cached_workspace_bytes if cache is not None else _lib.amr_lut_conv_input_grad_workspace_bytes
+        need = query(lut_grad_a_tensor.numel(), Bn, C, H, W, N)
         ws = torch.empty(max(need, 256), dtype=torch.uint8, device=dev)
-        rc = _lib.amr_lut_conv_input_grad_f32(gc_rows.data_ptr(), codes_tensor.data_ptr(), bt_tensor.data_ptr(), lut_grad_a_tensor.data_ptr(),
+        rc = _lib.amr_lut_conv_input_grad_cached_f32(cache._h if cache is not None else None, int(b_version) & 0xFFFFFFFFFFFFFFFF,
+                                              gc_rows.data_ptr(), codes_tensor.data_ptr(), bt_tensor.data_ptr(), lut_grad_a_tensor.data_ptr(),
                                               lut_grad_a_tensor.numel(), t_tensor.data_ptr(), z_w.data_ptr(), inside_tensor.data_ptr(),
                                               scale_tensor.data_ptr(), gx_tensor.data_ptr(), Bn, C, H, W, N,
                                               a_fallback.data_ptr() if a_fallback is not None else None,

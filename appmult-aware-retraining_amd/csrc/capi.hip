@@ -111,7 +111,7 @@ size_t gradA_slab_conv_workspace_bytes(int C, int N);
 hipError_t launch_gradA_slab_conv(const float* gC, const uint8_t* codes, const uint8_t* Bt, float* g_in, const int16_t* lut,
                                   const LutGeom& g, int Bn, int C, int H, int W, int N, float scale, int n_cu, uint32_t* flags,
                                   void* S, const float* zero_line, hipStream_t stream, const float* zt, const float* zw,
-                                  const float* qscale, const uint8_t* inside);
+                                  const float* qscale, const uint8_t* inside, int expanded);
 bool gradA_slab_conv_can_finish(int Bn, int H, int W, const float* g_in);
 hipError_t launch_conv_weight_prepare(const float* w, const float* scale, const float* zp_neg, float qmax, const float* tapmask,
                                       uint8_t* Bt, uint8_t* inside, float* w_resp, int N, int C, int T, int L, hipStream_t stream);
@@ -1010,6 +1010,11 @@ size_t amr_lut_conv_input_grad_workspace_bytes(int64_t lut_elems, int B, int C, 
     return 256 + conv_grad_zt_bytes(B, H, W) + amr::gradA_slab_conv_workspace_bytes(C, N);
 }
 
+size_t amr_lut_conv_input_grad_cached_workspace_bytes(int64_t lut_elems, int B, int C, int H, int W, int N) {
+    if (!amr_lut_conv_input_grad_supported(lut_elems, B, C, H, W, N)) return 0;
+    return 256 + conv_grad_zt_bytes(B, H, W);
+}
+
 // The decision bwd_header_kernel takes on the device (lutgemm_bwd_slab.hip), for a table in host memory.
 int amr_grad_table_fits_halves(const int16_t* host_table, int64_t lut_elems) {
     amr::LutGeom g;
@@ -1036,6 +1041,15 @@ int amr_lut_conv_input_grad_f32(const float* gC, const uint8_t* codes, const uin
                                 const float* t, const float* z_w, const uint8_t* inside, const float* scale, float* gx, int B, int C,
                                 int H, int W, int N, const uint8_t* A_fallback, float* cols_fallback, void* workspace,
                                 size_t workspace_bytes, void* stream) {
+    return amr_lut_conv_input_grad_cached_f32(nullptr, 0, gC, codes, Bt, lut_grad_a, lut_elems, t, z_w, inside, scale, gx, B, C, H, W, N,
+                                              A_fallback, cols_fallback, workspace, workspace_bytes, stream);
+}
+
+int amr_lut_conv_input_grad_cached_f32(amr_fwd_cache* cache, uint64_t b_version, const float* gC, const uint8_t* codes, const uint8_t* Bt,
+                                       const int16_t* lut_grad_a, int64_t lut_elems, const float* t, const float* z_w,
+                                       const uint8_t* inside, const float* scale, float* gx, int B, int C, int H, int W, int N,
+                                       const uint8_t* A_fallback, float* cols_fallback, void* workspace, size_t workspace_bytes,
+                                       void* stream) {
     amr::LutGeom g;
     if (!amr::lut_geom_from_elems(lut_elems, &g))
         return fail(AMR_ELUTLEN, "lut size should be one of 1024/5120/17408/66306, got %lld", (long long)lut_elems);
@@ -1048,7 +1062,8 @@ int amr_lut_conv_input_grad_f32(const float* gC, const uint8_t* codes, const uin
     if (!mode || !amr::gradA_slab_conv_applies(g, M, C, N, gC, mode == 2))
         return fail(AMR_EUNSUPPORTED, "shape, alignment or mode not served by the convolution-shaped gradA (ask amr_lut_conv_input_grad_supported)");
     const size_t zt_bytes = conv_grad_zt_bytes(B, H, W);
-    const size_t need = 256 + zt_bytes + amr::gradA_slab_conv_workspace_bytes(C, N);
+    const size_t s_bytes = amr::gradA_slab_conv_workspace_bytes(C, N);
+    const size_t need = 256 + zt_bytes + (cache ? 0 : s_bytes);      // (with a cache the expanded table lives there)
     if (!workspace || workspace_bytes < need)
         return fail(AMR_EWORKSPACE, "workspace of %zu bytes is smaller than the %zu required", workspace ? workspace_bytes : (size_t)0, need);
     if ((uintptr_t)workspace & 255) return fail(AMR_EINVAL, "workspace must be 256-byte aligned");
@@ -1065,10 +1080,19 @@ int amr_lut_conv_input_grad_f32(const float* gC, const uint8_t* codes, const uin
     const bool finish = amr::gradA_slab_conv_can_finish(B, H, W, gx);
     float* zt = reinterpret_cast<float*>(reinterpret_cast<unsigned char*>(workspace) + 256);
     if (finish && (e = amr::launch_window_sums_3x3(t, zt, B, H, W, s)) != hipSuccess) return hip_fail(e, "window sums launch");
-    e = amr::launch_gradA_slab_conv(gC, codes, Bt, gx, lut_grad_a, g, B, C, H, W, N, factor, n_cu, flags,
-                                    reinterpret_cast<unsigned char*>(workspace) + 256 + zt_bytes, reinterpret_cast<const float*>(flags + 32), s,
-                                    finish ? zt : nullptr, z_w, scale, inside);
-    if (e != hipSuccess) return hip_fail(e, "gradA launch");
+    void* s_buf = reinterpret_cast<unsigned char*>(workspace) + 256 + zt_bytes;
+    bool hit = false;
+    if (cache) {
+        hipError_t ec;
+        s_buf = fwd_cache_lookup(cache, dev, s_bytes, b_version, lut_grad_a, lut_elems, 9 * C, N, &hit, &ec);
+        if (!s_buf) return hip_fail(ec, "cache hipMalloc");
+    }
+    e = amr::launch_gradA_slab_conv(gC, codes, Bt, gx, lut_grad_a, g, B, C, H, W, N, factor, n_cu, flags, s_buf,
+                                    reinterpret_cast<const float*>(flags + 32), s, finish ? zt : nullptr, z_w, scale, inside, hit ? 1 : 0);
+    if (e != hipSuccess) {
+        if (cache) fwd_cache_forget(cache);      // (whether the expansion got there is unknown)
+        return hip_fail(e, "gradA launch");
+    }
     // flags[2]: a masked code, an entry a half cannot hold, or a table that cannot be held as halves at all
     const bool fallback = A_fallback != nullptr;
     if (!finish)

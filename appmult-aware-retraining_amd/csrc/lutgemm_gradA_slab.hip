@@ -994,14 +994,17 @@ bool gradA_slab_conv_can_finish(int Bn, int H, int W, const float* g_in) {
 hipError_t launch_gradA_slab_conv(const float* gC, const uint8_t* codes, const uint8_t* Bt, float* g_in, const int16_t* lut,
                                   const LutGeom& g, int Bn, int C, int H, int W, int N, float scale, int n_cu, uint32_t* flags,
                                   void* S, const float* zero_line, hipStream_t stream, const float* zt, const float* zw,
-                                  const float* qscale, const uint8_t* inside) {
+                                  const float* qscale, const uint8_t* inside, int expanded) {
     const GaFinish fin{zt, zw, qscale, inside};
     const int lut_dwords = g.rows * g.cols / 2;
     const int K = 9 * C, M = Bn * H * W;
     const int qpw = (long)(N / kGaCols) * ((K / 4 + 3) / 4) >= n_cu ? 4 : 1;
-    hipLaunchKernelGGL(expand_gradA_kernel, dim3(N / kGaCols, (K / 4 + qpw - 1) / qpw), dim3(256), (size_t)lut_dwords * 4, stream, Bt,
-                       reinterpret_cast<const uint32_t*>(lut), lut_dwords, g.cols, 1 << g.bits, reinterpret_cast<uint32_t*>(S),
-                       flags, K, N, qpw);
+    // (expanded: S already holds the expansion of this Bt and table -- a caller's cache; the offset in flags[3] is a function of
+    // the table alone, so the header of this call agrees with what the cached entries were built with)
+    if (!expanded)
+        hipLaunchKernelGGL(expand_gradA_kernel, dim3(N / kGaCols, (K / 4 + qpw - 1) / qpw), dim3(256), (size_t)lut_dwords * 4, stream, Bt,
+                           reinterpret_cast<const uint32_t*>(lut), lut_dwords, g.cols, 1 << g.bits, reinterpret_cast<uint32_t*>(S),
+                           flags, K, N, qpw);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     const u32x4* S4 = reinterpret_cast<const u32x4*>(S);

@@ -419,6 +419,16 @@ int amr_lut_conv_input_grad_f32(const float *gC, const uint8_t *codes, const uin
                                 int64_t lut_elems, const float *t, const float *z_w, const uint8_t *inside, const float *scale,
                                 float *gx, int B, int C, int H, int W, int N, const uint8_t *A_fallback, float *cols_fallback,
                                 void *workspace, size_t workspace_bytes, void *stream);
+/* The same with the gradient table expanded along Bt kept in an amr_fwd_cache of its own between calls (weights that do not
+ * change between backward passes: frozen layers that still hand a gradient to their input, gradient accumulation over
+ * micro-batches); b_version as in amr_lut_gemm_forward_cached.  cache = NULL: as above.  With a cache the workspace needs
+ * amr_lut_conv_input_grad_cached_workspace_bytes bytes only. */
+size_t amr_lut_conv_input_grad_cached_workspace_bytes(int64_t lut_elems, int B, int C, int H, int W, int N);
+int amr_lut_conv_input_grad_cached_f32(amr_fwd_cache *cache, uint64_t b_version, const float *gC, const uint8_t *codes,
+                                       const uint8_t *Bt, const int16_t *lut_grad_a, int64_t lut_elems, const float *t,
+                                       const float *z_w, const uint8_t *inside, const float *scale, float *gx, int B, int C, int H,
+                                       int W, int N, const uint8_t *A_fallback, float *cols_fallback, void *workspace,
+                                       size_t workspace_bytes, void *stream);
 
 /* amr_conv_dequant_backward_f32 that also leaves t[m] = sum over n of g_c[m, n] (ascending n), in the same pass. */
 int amr_conv_dequant_backward_rowsum_f32(const float *g, const float *s_a, const float *s_w, float *g_c, float *t, int batch,

@@ -522,6 +522,61 @@ def test_layer_reads_the_codes_itself_where_no_window_matrix_is_needed(ops):
         approx_ops.im2col_nhwc = native
 
 
+def test_expansions_kept_in_training_mode_for_weights_that_outlive_a_step(ops):
+    """keep_expansions_in_training: a frozen 3x3 layer in training mode expands its forward and input-gradient tables once;
+    later passes hit both caches (and the prepared weight operand) with identical results; an in-place weight update
+    invalidates them.  The convolution-shaped input gradient with a cache of its own: miss, hit, stale on purpose, new number."""
+    import copy
+    import approx_ops
+    import app_layers as L
+    from self_ops.ops_py import approx_ops as P
+    torch.manual_seed(5)
+    layer = L.ApproxConv2d(64, 64, 3, padding=1, bias=False, a_bits=7, w_bits=7).cuda().train()
+    layer.weight.requires_grad_(False)
+    plain = copy.deepcopy(layer)
+    layer.keep_expansions_in_training = True
+    x = torch.randn(16, 64, 32, 32, device="cuda") * 2 + 0.3
+    gy = None
+    for it in range(3):
+        if it == 2:
+            with torch.no_grad():
+                layer.weight.add_(0.01); plain.weight.add_(0.01)
+        xa, xb = x.clone().requires_grad_(), x.clone().requires_grad_()
+        ya, yb = layer(xa), plain(xb)
+        if gy is None:
+            gy = torch.randn_like(ya)
+        ya.backward(gy); yb.backward(gy)
+        assert torch.equal(ya, yb) and torch.equal(xa.grad, xb.grad), it
+    assert layer._fwd_cache.stats()[:2] == (1, 2)         # hit on the second pass, miss again after the weight update
+    assert layer._bwd_cache.stats()[:2] == (1, 2)
+    assert plain.__dict__.get("_fwd_cache") is None
+    # the entry point by itself
+    bn, c, h, w, n = 8, 32, 16, 16, 64
+    g = torch.Generator(device="cuda").manual_seed(8)
+    M = bn * h * w
+    codes = torch.randint(0, 128, (M, c), device="cuda", generator=g, dtype=torch.int32).to(torch.uint8)
+    bt = torch.randint(0, 128, (9 * c, n), device="cuda", generator=g, dtype=torch.int32).to(torch.uint8)
+    rows = torch.randn(M, n, device="cuda", generator=g)
+    t = rows.sum(dim=1).contiguous()
+    inside = (torch.rand(bn, c, h, w, device="cuda", generator=g) < 0.9).to(torch.uint8)
+    zw, sc = torch.tensor([-61.0], device="cuda"), torch.tensor([0.037], device="cuda")
+    old = approx_ops._lib.amr_set_expanded_table_kernels(2)
+    try:
+        def run(b, cache=None, version=0):
+            gx = torch.full((bn, c, h, w), float("nan"), device="cuda")
+            approx_ops.approx_conv_input_grad(rows, codes, b, P.lut_grad_a, t, zw, inside, sc, gx, cache=cache, b_version=version)
+            return gx
+        want = run(bt)
+        cache = approx_ops.ForwardCache()
+        assert torch.equal(run(bt, cache, 1), want) and torch.equal(run(bt, cache, 1), want)
+        bt2 = bt.clone(); bt2[5, 7] ^= 1
+        assert torch.equal(run(bt2, cache, 1), want)                 # same number: the old expansion, on purpose
+        assert torch.equal(run(bt2, cache, 2), run(bt2))
+        assert cache.stats()[:2] == (2, 2)
+    finally:
+        approx_ops._lib.amr_set_expanded_table_kernels(old)
+
+
 def _conv_grad_case(oracle, seed, bn, c, h, w, n, lo=-1024, hi=3073, masked=False):
     """Operands of one input-gradient problem of a 3x3 / stride 1 / padding 1 convolution and its float64 answer."""
     rng = np.random.default_rng(seed)

@@ -205,6 +205,12 @@ def test_layer_level_entry_points_check_arguments_without_touching_a_device():
     assert lib.amr_lut_conv_input_grad_workspace_bytes(17408, 512, 64, 32, 32, 64) == 256 + 512 * 1024 * 4 + 9 * 64 * 64 * 256
     lib.amr_lut_conv_input_grad_f32.argtypes = [vp] * 4 + [i64] + [vp] * 5 + [i] * 5 + [vp, vp, vp, sz, vp]
     assert lib.amr_lut_conv_input_grad_f32(*([None] * 4), 17408, *([None] * 5), 512, 64, 32, 32, 64, None, None, None, 0, None) == -1
+    lib.amr_lut_conv_input_grad_cached_workspace_bytes.argtypes = [i64, i, i, i, i, i]
+    lib.amr_lut_conv_input_grad_cached_workspace_bytes.restype = sz
+    assert lib.amr_lut_conv_input_grad_cached_workspace_bytes(17408, 512, 64, 32, 32, 64) == 256 + 512 * 1024 * 4
+    assert lib.amr_lut_conv_input_grad_cached_workspace_bytes(17408, 512, 24, 32, 32, 64) == 0
+    lib.amr_lut_conv_input_grad_cached_f32.argtypes = [vp, ctypes.c_uint64] + [vp] * 4 + [i64] + [vp] * 5 + [i] * 5 + [vp, vp, vp, sz, vp]
+    assert lib.amr_lut_conv_input_grad_cached_f32(None, 0, *([None] * 4), 17408, *([None] * 5), 512, 64, 32, 32, 64, None, None, None, 0, None) == -1
     lib.amr_observe_minmax_f32.argtypes = [vp, i64, vp, vp, vp, vp, vp, i] + [f] * 5 + [vp]
     assert lib.amr_observe_minmax_f32(None, 10, None, None, None, None, None, 3, 0.9, 0.1, 127.0, 0.0, 1e-7, None) == -1   # mode
     assert lib.amr_observe_minmax_f32(None, 10, None, None, None, None, None, 7, 0.9, 0.1, 127.0, 0.0, 1e-7, None) == -1   # mode 3 with the ReLU bit
