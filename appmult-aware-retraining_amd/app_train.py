@@ -77,6 +77,8 @@ def main(argv=None):
     ap.add_argument("--float-grad-window", type=int, default=0, metavar="W",
                     help="replace the file's int16 gradient tables by the float32 difference slopes of its forward table, "
                          "half window W (the float-table backward pass; no counterpart in the reference)")
+    ap.add_argument("--eval-batches", type=int, default=0, metavar="N",
+                    help="afterwards time N evaluation-mode forward passes of one batch (frozen ranges and weights, no graph)")
     args = ap.parse_args(argv)
     assert torch.cuda.is_available(), "a GPU is required"
     device = torch.device("cuda")
@@ -108,6 +110,19 @@ def main(argv=None):
     dt = time.perf_counter() - t0
     print(f"{args.arch} batch {args.batch}: {args.steps * args.batch / dt:.1f} img/s, {dt / args.steps * 1e3:.1f} ms/step, "
           f"loss {float(losses[0]):.4f} -> {float(losses[-1]):.4f}")
+    if args.eval_batches > 0:
+        model.eval()
+        with torch.no_grad():
+            for _ in range(2):
+                model(xs[0])                            # (the first pass expands the tables of the frozen weights)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(args.eval_batches):
+                model(xs[0])
+            torch.cuda.synchronize()
+            dt = time.perf_counter() - t0
+        print(f"{args.arch} batch {args.batch}, evaluation mode: {args.eval_batches * args.batch / dt:.1f} img/s, "
+              f"{dt / args.eval_batches * 1e3:.2f} ms per batch")
 
 
 if __name__ == "__main__":
